@@ -1,0 +1,335 @@
+/*
+ * TEST INFRASTRUCTURE ONLY -- driver that runs the *reference's own* compiled
+ * hot-path functions on inputs supplied by the test harness, so the oracle
+ * (ace_oracle.c) can be compared with the real thing limb by limb.
+ *
+ * It is linked against the reference sources where they lie (see Makefile);
+ * the context is created with the reference's Prepare_context_for_cmplr
+ * (context/src/cmplr_context.c:22-45), so every getter the poly layer calls is
+ * the reference's own.  No reference code is copied here: this file only
+ * calls public functions declared in the reference headers.
+ *
+ * usage: ref_driver <request.bin> <response.bin>
+ * request  (int64 words): N num_q q0_bits sf_bits parts n_ops, then per op
+ *          opcode a1 a2 a3 a4 n_in  in[n_in]
+ * response (int64 words): L K part_size  prime[L+K] root[L+K]
+ *          modulus[5*(L+K)], then per op  n_out out[n_out]
+ */
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "common/cmplr_api.h"
+#include "common/rt_config.h"
+#include "context/ckks_context.h"
+#include "crt_impl.h"
+#include "hal/hal.h"
+#include "ntt_impl.h"
+#include "number_theory_impl.h"
+#include "poly/rns_poly.h"
+#include "rns_poly_impl.h"
+#include "type_impl.h"
+#include "util/crt.h"
+#include "util/ntt.h"
+#include "util/number_theory.h"
+
+enum {
+  OP_NTT = 1, OP_INTT, OP_HW, OP_DECOMP_MODUP, OP_PRECOMP, OP_MOD_DOWN,
+  OP_RESCALE, OP_DOT_PROD, OP_AUTO_ORDER, OP_AUTO_INDEX, OP_AUTOMORPHISM,
+  OP_EXTEND, OP_TBL_MODUP, OP_TBL_MODDOWN, OP_TBL_RESCALE, OP_POLY, OP_TWIDDLES,
+  OP_MOD_UP
+};
+
+static int64_t* in_buf;
+static size_t   in_pos;
+static FILE*    out_f;
+
+static int64_t rd(void) { return in_buf[in_pos++]; }
+static void wr(const int64_t* p, size_t n) { fwrite(p, sizeof(int64_t), n, out_f); }
+static void wr1(int64_t v) { wr(&v, 1); }
+
+static size_t L, K, N;
+
+static CRT_PRIME* prime_at(size_t idx) {
+  CRT_CONTEXT* crt = Get_crt_context();
+  return idx < L ? Get_prime_at(Get_q(crt), idx) : Get_prime_at(Get_p(crt), idx - L);
+}
+
+/* wrap caller memory as a POLYNOMIAL with num_q + num_p limbs allocated */
+static void wrap_poly(POLYNOMIAL* p, int64_t* data, size_t num_q, size_t num_p, bool ntt) {
+  memset(p, 0, sizeof(*p));
+  p->_num_alloc_primes = num_q + num_p;
+  Init_poly_data(p, (uint32_t)N, num_q, num_p, data);
+  Set_is_ntt(p, ntt);
+}
+
+int main(int argc, char** argv) {
+  if (argc != 3) { fprintf(stderr, "usage: %s req resp\n", argv[0]); return 2; }
+  FILE* f = fopen(argv[1], "rb");
+  if (!f) { perror("request"); return 2; }
+  fseek(f, 0, SEEK_END);
+  long sz = ftell(f);
+  fseek(f, 0, SEEK_SET);
+  in_buf = (int64_t*)malloc((size_t)sz + 8);
+  if (fread(in_buf, 1, (size_t)sz, f) != (size_t)sz) { perror("read"); return 2; }
+  fclose(f);
+  out_f = fopen(argv[2], "wb");
+  if (!out_f) { perror("response"); return 2; }
+
+  N = (size_t)rd();
+  size_t num_q = (size_t)rd(), q0 = (size_t)rd(), sf = (size_t)rd(), parts = (size_t)rd();
+  size_t n_ops = (size_t)rd();
+  Prepare_context_for_cmplr((uint32_t)N, 0, (uint32_t)(num_q - 1), (uint32_t)num_q,
+                            (uint32_t)q0, (uint32_t)sf, (uint32_t)parts, 0);
+  CRT_CONTEXT* crt = Get_crt_context();
+  L = Get_q_cnt();
+  K = Get_p_cnt();
+  wr1((int64_t)L);
+  wr1((int64_t)K);
+  wr1((int64_t)Get_per_part_size(Get_qpart(crt)));
+  for (size_t i = 0; i < L + K; i++) wr1(Get_modulus_val(prime_at(i)));
+  for (size_t i = 0; i < L + K; i++)
+    wr1(Get_i64_value_at(Get_ntt(prime_at(i))->_rou, N / 2)); /* rou[bitrev(1)] = psi */
+  for (size_t i = 0; i < L + K; i++) {
+    MODULUS* m = Get_modulus(prime_at(i));
+    wr1(m->_val); wr1(m->_br_k); wr1(m->_br_m);
+    wr1((int64_t)(uint64_t)m->_prec128);
+    wr1((int64_t)(uint64_t)(m->_prec128 >> 64));
+  }
+
+  for (size_t op = 0; op < n_ops; op++) {
+    int64_t code = rd(), a1 = rd(), a2 = rd(), a3 = rd(), a4 = rd();
+    size_t  n_in = (size_t)rd();
+    int64_t* in = in_buf + in_pos;
+    in_pos += n_in;
+    (void)a4;
+    switch (code) {
+      case OP_NTT:
+      case OP_INTT: { /* a1 = n_limbs; in = prime_idx[n_limbs] data[n_limbs*N] */
+        size_t nl = (size_t)a1;
+        int64_t* data = in + nl;
+        for (size_t t = 0; t < nl; t++) {
+          VALUE_LIST vl;
+          Init_i64_value_list_no_copy(&vl, N, data + t * N);
+          NTT_CONTEXT* ntt = Get_ntt(prime_at((size_t)in[t]));
+          if (code == OP_NTT) Ftt_fwd(&vl, ntt, &vl);
+          else                Ftt_inv(&vl, ntt, &vl);
+        }
+        wr1((int64_t)(nl * N));
+        wr(data, nl * N);
+        break;
+      }
+      case OP_HW: { /* a1 = which, a2 = prime idx, a3 = n; in = r[n] a[n] b[n] */
+        size_t n = (size_t)a3;
+        int64_t *r = in, *a = in + n, *b = in + 2 * n;
+        MODULUS* m = Get_modulus(prime_at((size_t)a2));
+        switch (a1) {
+          case 0: Hw_modadd(r, a, b, m, n); break;
+          case 1: Hw_modsub(r, a, b, m, n); break;
+          case 2: Hw_modmul(r, a, b, m, n); break;
+          case 3: Hw_modmuladd(r, a, b, m, n); break;
+          case 4: Hw_modadd_scalar(r, a, b[0], m, n); break;
+          case 5: Hw_modsub_scalar(r, a, b[0], m, n); break;
+          case 6: Hw_modmul_scalar(r, a, b[0], m, n); break;
+          case 7: Hw_modmuladd_scalar(r, a, b[0], m, n); break;
+          case 8: Hw_rotate(r, a, b, m, n); break;
+          default: fprintf(stderr, "bad hw op\n"); return 2;
+        }
+        wr1((int64_t)n);
+        wr(r, n);
+        break;
+      }
+      case OP_DECOMP_MODUP: { /* a1 level, a2 part, a3 is_ntt; in = level*N */
+        size_t lv = (size_t)a1;
+        POLYNOMIAL src, res;
+        wrap_poly(&src, in, lv, 0, a3 != 0);
+        int64_t* out = (int64_t*)calloc((lv + K) * N, sizeof(int64_t));
+        wrap_poly(&res, out, lv, K, a3 != 0);
+        Decomp_modup(&res, &src, (uint32_t)a2);
+        wr1((int64_t)((lv + K) * N));
+        wr(out, (lv + K) * N);
+        free(out);
+        break;
+      }
+      case OP_MOD_UP: { /* a1 level, a2 part, a3 is_ntt, in = level*N (Decomp then Mod_up) */
+        size_t lv = (size_t)a1;
+        POLYNOMIAL src, res, dig;
+        wrap_poly(&src, in, lv, 0, a3 != 0);
+        int64_t* out = (int64_t*)calloc((lv + K) * N, sizeof(int64_t));
+        wrap_poly(&res, out, lv, K, a3 != 0);
+        memset(&dig, 0, sizeof(dig));
+        Alloc_poly_data(&dig, (uint32_t)N, lv + K, 0);
+        Decomp(&dig, &src, (uint32_t)a2);
+        Mod_up(&res, &dig, (uint32_t)a2);
+        wr1((int64_t)((lv + K) * N));
+        wr(out, (lv + K) * N);
+        free(out);
+        Free_poly_data(&dig);
+        break;
+      }
+      case OP_PRECOMP: { /* a1 level, a2 is_ntt, a3 fused */
+        size_t lv = (size_t)a1;
+        POLYNOMIAL src;
+        wrap_poly(&src, in, lv, 0, a2 != 0);
+        Set_rtlib_config(CONF_OP_FUSION_DECOMP_MODUP, a3 ? 1 : 0);
+        VALUE_LIST* pl = Alloc_precomp(&src);
+        size_t nd = LIST_LEN(pl);
+        wr1((int64_t)(nd * (lv + K) * N));
+        for (size_t d = 0; d < nd; d++) {
+          POLYNOMIAL* p = (POLYNOMIAL*)Get_ptr_value_at(pl, d);
+          wr(Get_poly_coeffs(p), (lv + K) * N);
+        }
+        Free_precomp(pl);
+        break;
+      }
+      case OP_MOD_DOWN: { /* a1 level, a2 is_ntt; in = (level+K)*N */
+        size_t lv = (size_t)a1;
+        POLYNOMIAL src, res;
+        wrap_poly(&src, in, lv, K, a2 != 0);
+        int64_t* out = (int64_t*)calloc(lv * N, sizeof(int64_t));
+        wrap_poly(&res, out, lv, 0, a2 != 0);
+        Mod_down(&res, &src);
+        wr1((int64_t)(lv * N));
+        wr(out, lv * N);
+        free(out);
+        break;
+      }
+      case OP_RESCALE: { /* a1 level, a2 is_ntt; in = level*N */
+        size_t lv = (size_t)a1;
+        POLYNOMIAL src, res;
+        wrap_poly(&src, in, lv, 0, a2 != 0);
+        int64_t* out = (int64_t*)calloc(lv * N, sizeof(int64_t));
+        wrap_poly(&res, out, lv, 0, a2 != 0);
+        Rescale(&res, &src);
+        wr1((int64_t)((lv - 1) * N));
+        wr(out, (lv - 1) * N);
+        free(out);
+        break;
+      }
+      case OP_DOT_PROD: { /* a1 level, a2 n_parts, a3 fast; in = digits, keys */
+        size_t lv = (size_t)a1, np = (size_t)a2;
+        POLYNOMIAL dg[16], ky[16], res;
+        int64_t* digits = in;
+        int64_t* keys   = in + np * (lv + K) * N;
+        for (size_t d = 0; d < np; d++) {
+          wrap_poly(&dg[d], digits + d * (lv + K) * N, lv, K, true);
+          wrap_poly(&ky[d], keys + d * (L + K) * N, L, K, true);
+        }
+        Set_rtlib_config(CONF_FAST_DOT_PROD, a3 ? 1 : 0);
+        memset(&res, 0, sizeof(res));
+        Dot_prod(&res, dg, ky, (uint32_t)np);
+        wr1((int64_t)((lv + K) * N));
+        wr(Get_poly_coeffs(&res), (lv + K) * N);
+        Free_poly_data(&res);
+        break;
+      }
+      case OP_AUTO_ORDER: { /* a1 k, a2 is_ntt */
+        VALUE_LIST* vl = Alloc_value_list(I64_TYPE, N);
+        Precompute_automorphism_order(vl, (uint32_t)a1, (uint32_t)N, a2 != 0);
+        wr1((int64_t)N);
+        wr(Get_i64_values(vl), N);
+        Free_value_list(vl);
+        break;
+      }
+      case OP_AUTO_INDEX: { /* a1 rot_idx */
+        MODULUS m;
+        Init_modulus(&m, 2 * (int64_t)N);
+        wr1(1);
+        wr1((int64_t)Find_automorphism_index((int32_t)a1, &m));
+        break;
+      }
+      case OP_AUTOMORPHISM: { /* a1 level, a2 with_p, a3 is_ntt; in = poly, order[N] */
+        size_t lv = (size_t)a1, T = lv + (a2 ? K : 0);
+        POLYNOMIAL src, res;
+        wrap_poly(&src, in, lv, a2 ? K : 0, a3 != 0);
+        int64_t* out = (int64_t*)calloc(T * N, sizeof(int64_t));
+        wrap_poly(&res, out, lv, a2 ? K : 0, a3 != 0);
+        VALUE_LIST ord;
+        Init_i64_value_list_no_copy(&ord, N, in + T * N);
+        Automorphism_transform(&res, &src, &ord);
+        wr1((int64_t)(T * N));
+        wr(out, T * N);
+        free(out);
+        break;
+      }
+      case OP_EXTEND: { /* a1 level */
+        size_t lv = (size_t)a1;
+        POLYNOMIAL src, res;
+        wrap_poly(&src, in, lv, 0, true);
+        int64_t* out = (int64_t*)calloc((lv + K) * N, sizeof(int64_t));
+        wrap_poly(&res, out, lv, K, true);
+        Extend(&res, &src);
+        wr1((int64_t)((lv + K) * N));
+        wr(out, (lv + K) * N);
+        free(out);
+        break;
+      }
+      case OP_TBL_MODUP: { /* a1 level, a2 part: hat_inv[nd], hat[nd][nc], compl primes[nc] */
+        size_t lv = (size_t)a1, part = (size_t)a2;
+        CRT_PRIMES* qp = Get_qpart(crt);
+        size_t ps = Get_per_part_size(qp), ndec = Get_num_decomp(crt, lv);
+        size_t nd = (part == ndec - 1) ? lv - ps * part
+                                       : LIST_LEN(Get_qpart_prime_at_l1(qp, part));
+        VALUE_LIST* hinv = VL_L2_VALUE_AT(Get_qlhatinvmodq(qp), part, nd - 1);
+        VL_VL_I64*  hat  = VL_L2_VALUE_AT(Get_qlhatmodp(qp), lv - 1, part);
+        VL_CRTPRIME* cp  = Get_qpart_compl_at(Get_qpart_compl(crt), lv - 1, part);
+        size_t nc = LIST_LEN(cp);
+        wr1((int64_t)(2 + nd + nd * nc + nc));
+        wr1((int64_t)nd);
+        wr1((int64_t)nc);
+        wr(Get_i64_values(hinv), nd);
+        for (size_t i = 0; i < nd; i++) wr(Get_i64_values(VL_VALUE_AT(hat, i)), nc);
+        for (size_t j = 0; j < nc; j++) wr1(Get_modulus_val(Get_vlprime_at(cp, j)));
+        break;
+      }
+      case OP_TBL_MODDOWN: { /* phat_inv[K], phat_modq[L][K], pinv_modq[L], pmodq[L] */
+        CRT_PRIMES* p = Get_p(crt);
+        wr1((int64_t)(K + L * K + 2 * L));
+        wr(Get_i64_values(Get_phatinvmodp(p)), K);
+        for (size_t i = 0; i < L; i++) wr(Get_i64_values(Get_phatmodq_at(p, i)), K);
+        wr(Get_i64_values(Get_pinvmodq(p)), L);
+        wr(Get_i64_values(Get_pmodq(p)), L);
+        break;
+      }
+      case OP_TBL_RESCALE: { /* a1 level: ql_inv[level-1], qlql[level-1] */
+        size_t lv = (size_t)a1;
+        CRT_PRIMES* q = Get_q(crt);
+        wr1((int64_t)(2 * (lv - 1)));
+        wr(Get_i64_values(Get_ql_inv_mod_qi_at(q, lv - 2)), lv - 1);
+        wr(Get_i64_values(Get_ql_ql_inv_mod_ql_div_ql_mod_qi_at(q, lv - 2)), lv - 1);
+        break;
+      }
+      case OP_POLY: { /* a1 which (0 add 1 sub 2 mul), a2 level, a3 with_p; in = a, b */
+        size_t lv = (size_t)a2, T = lv + (a3 ? K : 0);
+        POLYNOMIAL pa, pb, res;
+        wrap_poly(&pa, in, lv, a3 ? K : 0, true);
+        wrap_poly(&pb, in + T * N, lv, a3 ? K : 0, true);
+        int64_t* out = (int64_t*)calloc(T * N, sizeof(int64_t));
+        wrap_poly(&res, out, lv, a3 ? K : 0, true);
+        if (a1 == 0) Add_poly(&res, &pa, &pb);
+        else if (a1 == 1) Sub_poly(&res, &pa, &pb);
+        else Mul_poly(&res, &pa, &pb);
+        wr1((int64_t)(T * N));
+        wr(out, T * N);
+        free(out);
+        break;
+      }
+      case OP_TWIDDLES: { /* a1 prime idx: rou, rou_prec, rou_inv, rou_inv_prec, ninv, ninv_prec */
+        NTT_CONTEXT* ntt = Get_ntt(prime_at((size_t)a1));
+        wr1((int64_t)(4 * N + 2));
+        wr(Get_i64_values(ntt->_rou), N);
+        wr((int64_t*)Get_ui64_values(ntt->_rou_prec), N);
+        wr(Get_i64_values(ntt->_rou_inv), N);
+        wr((int64_t*)Get_ui64_values(ntt->_rou_inv_prec), N);
+        wr1((int64_t)ntt->_degree_inv);
+        wr1((int64_t)ntt->_degree_inv_prec);
+        break;
+      }
+      default:
+        fprintf(stderr, "unknown opcode %ld\n", (long)code);
+        return 2;
+    }
+  }
+  fclose(out_f);
+  return 0;
+}
