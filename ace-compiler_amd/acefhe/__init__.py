@@ -1,0 +1,317 @@
+"""ctypes binding of libace_hip.so, the MI355X CKKS polynomial runtime.
+
+The binding is a thin veneer over the C-ABI declared in include/ace_hip.h:
+device buffers are raw HBM pointers wrapped in `DevBuf`, every method maps to
+one C entry point, and a non-zero return raises `AceError` with the library's
+message.  There is no CPU fallback: if the shared library is missing, import
+fails; if no GPU is present, every compute call raises.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(os.path.dirname(_HERE), "libace_hip.so")
+
+_i64p = C.POINTER(C.c_int64)
+_i32p = C.POINTER(C.c_int32)
+_u64p = C.POINTER(C.c_uint64)
+_vp = C.c_void_p
+_sz = C.c_size_t
+
+
+class AceError(RuntimeError):
+    pass
+
+
+def _sig(lib):
+    def f(name, res, *args):
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = list(args)
+
+    f("ace_ctx_create", _vp, C.c_uint32, _sz, _sz, _sz, _sz)
+    f("ace_ctx_create_with_primes", _vp, C.c_uint32, _sz, _i64p, _sz)
+    f("ace_ctx_destroy", None, _vp)
+    f("ace_has_device", C.c_int, _vp)
+    f("ace_last_error", C.c_char_p)
+    f("ace_degree", C.c_uint32, _vp)
+    for n in ("ace_num_q", "ace_num_p", "ace_num_parts", "ace_part_size"):
+        f(n, _sz, _vp)
+    f("ace_num_decomp", _sz, _vp, _sz)
+    f("ace_prime", C.c_int64, _vp, _sz)
+    f("ace_root", C.c_int64, _vp, _sz)
+    f("ace_modulus", None, _vp, _sz, _u64p)
+    f("ace_host_twiddles", C.c_int, _vp, _sz, C.c_int, _u64p)
+    f("ace_host_tbl_modup", C.c_int, _vp, _sz, _sz, _i64p, _i64p, _i32p, C.POINTER(_sz), C.POINTER(_sz))
+    f("ace_host_tbl_moddown", C.c_int, _vp, _i64p, _i64p, _i64p, _i64p)
+    f("ace_host_tbl_rescale", C.c_int, _vp, _sz, _i64p, _i64p)
+    f("ace_host_automorphism_order", C.c_int, _vp, _i64p, C.c_uint32, C.c_int)
+    f("ace_alloc", _vp, _vp, _sz)
+    f("ace_free", None, _vp, _vp)
+    f("ace_upload", C.c_int, _vp, _vp, _i64p, _sz)
+    f("ace_download", C.c_int, _vp, _i64p, _vp, _sz)
+    f("ace_copy", C.c_int, _vp, _vp, _vp, _sz)
+    f("ace_zero", C.c_int, _vp, _vp, _sz)
+    f("ace_sync", C.c_int, _vp)
+    f("ace_timer_start", C.c_int, _vp)
+    f("ace_timer_stop_ms", C.c_float, _vp)
+    f("ace_ntt", C.c_int, _vp, _vp, _vp, _i32p, _sz, _sz, _sz)
+    f("ace_intt", C.c_int, _vp, _vp, _vp, _i32p, _sz, _sz, _sz)
+    for n in ("modadd", "modsub", "modmul", "modmuladd"):
+        f("ace_hw_" + n, C.c_int, _vp, _vp, _vp, _vp, _sz, _sz)
+        f("ace_hw_" + n + "_scalar", C.c_int, _vp, _vp, _vp, C.c_int64, _sz, _sz)
+    f("ace_hw_rotate", C.c_int, _vp, _vp, _vp, _vp, _sz, _sz)
+    f("ace_find_automorphism_index", C.c_uint32, _vp, C.c_int32)
+    f("ace_automorphism_order", C.c_int, _vp, _vp, C.c_uint32, C.c_int)
+    for n in ("add", "sub", "mul"):
+        f("ace_poly_" + n, C.c_int, _vp, _vp, _vp, _vp, _sz, C.c_int)
+    f("ace_poly_automorphism", C.c_int, _vp, _vp, _vp, _vp, _sz, C.c_int)
+    f("ace_decomp_modup", C.c_int, _vp, _vp, _vp, _sz, _sz, C.c_int)
+    f("ace_precomp", C.c_int, _vp, _vp, _vp, _sz, C.c_int)
+    f("ace_mod_down", C.c_int, _vp, _vp, _vp, _sz, C.c_int)
+    f("ace_rescale", C.c_int, _vp, _vp, _vp, _sz, C.c_int)
+    f("ace_extend", C.c_int, _vp, _vp, _vp, _sz)
+    f("ace_dot_prod", C.c_int, _vp, _vp, _vp, _vp, _sz, _sz, _sz)
+    f("ace_mul_ciph3", C.c_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz)
+    f("ace_fast_switch_key", C.c_int, _vp, _vp, _vp, _vp, _vp, _sz)
+    f("ace_relin", C.c_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz)
+    f("ace_rescale_ciph", C.c_int, _vp, _vp, _vp, _vp, _vp, _sz)
+    f("ace_mul_relin_rescale", C.c_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz)
+    f("ace_fast_rotate", C.c_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz)
+    f("ace_rotate_batch", C.c_int, _vp, _vp, _vp, _vp, _vp, C.POINTER(_vp), C.POINTER(_vp), _sz, _sz)
+
+
+# every symbol include/ace_hip.h declares
+EXPORTS = [
+    "ace_ctx_create", "ace_ctx_create_with_primes", "ace_ctx_destroy", "ace_has_device", "ace_last_error",
+    "ace_degree", "ace_num_q", "ace_num_p", "ace_num_parts", "ace_part_size", "ace_num_decomp", "ace_prime",
+    "ace_root", "ace_modulus", "ace_host_twiddles", "ace_host_tbl_modup", "ace_host_tbl_moddown",
+    "ace_host_tbl_rescale", "ace_host_automorphism_order", "ace_alloc", "ace_free", "ace_upload", "ace_download",
+    "ace_copy", "ace_zero", "ace_sync", "ace_timer_start", "ace_timer_stop_ms", "ace_ntt", "ace_intt",
+    "ace_hw_modadd", "ace_hw_modsub", "ace_hw_modmul", "ace_hw_modmuladd", "ace_hw_modadd_scalar",
+    "ace_hw_modsub_scalar", "ace_hw_modmul_scalar", "ace_hw_modmuladd_scalar", "ace_hw_rotate",
+    "ace_find_automorphism_index", "ace_automorphism_order", "ace_poly_add", "ace_poly_sub", "ace_poly_mul",
+    "ace_poly_automorphism", "ace_decomp_modup", "ace_precomp", "ace_mod_down", "ace_rescale", "ace_extend",
+    "ace_dot_prod", "ace_mul_ciph3", "ace_fast_switch_key", "ace_relin", "ace_rescale_ciph",
+    "ace_mul_relin_rescale", "ace_fast_rotate", "ace_rotate_batch",
+]
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError("libace_hip.so is not built: run `python -c 'import __graft_entry__ as g; g.build()'`")
+        _lib = C.CDLL(LIB_PATH)
+        _sig(_lib)
+    return _lib
+
+
+class DevBuf:
+    """n int64 words of HBM owned by a context."""
+
+    def __init__(self, ctx, n_words, ptr=None):
+        self.ctx, self.n = ctx, int(n_words)
+        self.own = ptr is None
+        self.ptr = ctx.lib.ace_alloc(ctx.h, self.n) if ptr is None else ptr
+        if not self.ptr:
+            raise AceError(ctx.err())
+
+    def get(self):
+        out = np.empty(self.n, np.int64)
+        self.ctx._chk(self.ctx.lib.ace_download(self.ctx.h, out.ctypes.data_as(_i64p), self.ptr, self.n))
+        return out
+
+    def set(self, arr):
+        arr = np.ascontiguousarray(arr, dtype=np.int64).ravel()
+        assert arr.size == self.n
+        self.ctx._chk(self.ctx.lib.ace_upload(self.ctx.h, self.ptr, arr.ctypes.data_as(_i64p), self.n))
+        return self
+
+    def view(self, off_words, n_words):
+        assert off_words + n_words <= self.n
+        return DevBuf(self.ctx, n_words, ptr=self.ptr + 8 * off_words)
+
+    def free(self):
+        if self.own and self.ptr:
+            self.ctx.lib.ace_free(self.ctx.h, self.ptr)
+            self.ptr = None
+
+
+class Context:
+    """One CRT context (primes, tables in HBM, one HIP stream)."""
+
+    def __init__(self, degree, num_q, q0_bits=0, sf_bits=0, parts=1, primes=None):
+        self.lib = lib()
+        if primes is None:
+            h = self.lib.ace_ctx_create(degree, num_q, q0_bits, sf_bits, parts)
+        else:
+            p = np.ascontiguousarray(primes, dtype=np.int64)
+            h = self.lib.ace_ctx_create_with_primes(degree, len(p), p.ctypes.data_as(_i64p), parts)
+        if not h:
+            raise AceError(self.err())
+        self.h = _vp(h)
+        self.N = self.lib.ace_degree(self.h)
+        self.L = self.lib.ace_num_q(self.h)
+        self.K = self.lib.ace_num_p(self.h)
+        self.parts = self.lib.ace_num_parts(self.h)
+        self.part_size = self.lib.ace_part_size(self.h)
+        self.primes = [self.lib.ace_prime(self.h, i) for i in range(self.L + self.K)]
+        self.roots = [self.lib.ace_root(self.h, i) for i in range(self.L + self.K)]
+        self.has_device = bool(self.lib.ace_has_device(self.h))
+
+    def err(self):
+        return (self.lib.ace_last_error() or b"").decode()
+
+    def _chk(self, rc):
+        if rc != 0:
+            raise AceError(self.err())
+
+    def close(self):
+        if self.h:
+            self.lib.ace_ctx_destroy(self.h)
+            self.h = None
+
+    # ---- getters / host tables
+    def num_decomp(self, level):
+        return self.lib.ace_num_decomp(self.h, level)
+
+    def modulus(self, i):
+        out = (C.c_uint64 * 5)()
+        self.lib.ace_modulus(self.h, i, out)
+        return list(out)
+
+    def limb_primes(self, level, with_p=True):
+        return list(range(level)) + ([self.L + j for j in range(self.K)] if with_p else [])
+
+    def twiddles(self, i, which):
+        out = np.empty(self.N, np.uint64)
+        self._chk(self.lib.ace_host_twiddles(self.h, i, which, out.ctypes.data_as(_u64p)))
+        return out
+
+    def tbl_modup(self, level, part):
+        hat_inv = np.zeros(96, np.int64)
+        hat = np.zeros(96 * 96, np.int64)
+        cidx = np.zeros(96, np.int32)
+        nd, nc = _sz(), _sz()
+        self._chk(self.lib.ace_host_tbl_modup(self.h, level, part, hat_inv.ctypes.data_as(_i64p),
+                                              hat.ctypes.data_as(_i64p), cidx.ctypes.data_as(_i32p),
+                                              C.byref(nd), C.byref(nc)))
+        nd, nc = nd.value, nc.value
+        return hat_inv[:nd].copy(), hat[:nd * nc].reshape(nd, nc).copy(), cidx[:nc].copy()
+
+    def tbl_moddown(self):
+        a = np.zeros(self.K, np.int64)
+        b = np.zeros(self.L * self.K, np.int64)
+        c = np.zeros(self.L, np.int64)
+        d = np.zeros(self.L, np.int64)
+        self._chk(self.lib.ace_host_tbl_moddown(self.h, *[x.ctypes.data_as(_i64p) for x in (a, b, c, d)]))
+        return a, b.reshape(self.L, self.K), c, d
+
+    def tbl_rescale(self, level):
+        a = np.zeros(level - 1, np.int64)
+        b = np.zeros(level - 1, np.int64)
+        self._chk(self.lib.ace_host_tbl_rescale(self.h, level, a.ctypes.data_as(_i64p), b.ctypes.data_as(_i64p)))
+        return a, b
+
+    def find_automorphism_index(self, rot):
+        return self.lib.ace_find_automorphism_index(self.h, rot)
+
+    def host_automorphism_order(self, k, is_ntt=True):
+        out = np.zeros(self.N, np.int64)
+        self._chk(self.lib.ace_host_automorphism_order(self.h, out.ctypes.data_as(_i64p), k, int(is_ntt)))
+        return out
+
+    # ---- memory
+    def alloc(self, n_words):
+        return DevBuf(self, n_words)
+
+    def upload(self, arr):
+        arr = np.ascontiguousarray(arr, dtype=np.int64).ravel()
+        return DevBuf(self, arr.size).set(arr)
+
+    def sync(self):
+        self._chk(self.lib.ace_sync(self.h))
+
+    def timer_start(self):
+        self._chk(self.lib.ace_timer_start(self.h))
+
+    def timer_stop_ms(self):
+        ms = self.lib.ace_timer_stop_ms(self.h)
+        if ms < 0:
+            raise AceError(self.err())
+        return ms
+
+    # ---- NTT
+    def ntt(self, dst, src, prime_idx, n_polys=1, poly_stride_limbs=0, inverse=False):
+        idx = np.ascontiguousarray(prime_idx, dtype=np.int32)
+        f = self.lib.ace_intt if inverse else self.lib.ace_ntt
+        self._chk(f(self.h, dst.ptr, src.ptr, idx.ctypes.data_as(_i32p), len(idx), n_polys, poly_stride_limbs))
+
+    def intt(self, dst, src, prime_idx, n_polys=1, poly_stride_limbs=0):
+        self.ntt(dst, src, prime_idx, n_polys, poly_stride_limbs, inverse=True)
+
+    # ---- Hw_*
+    def hw(self, name, r, a, b, prime_idx, n=None):
+        n = a.n if n is None else n
+        f = getattr(self.lib, "ace_hw_" + name)
+        if name.endswith("_scalar"):
+            self._chk(f(self.h, r.ptr, a.ptr, int(b), prime_idx, n))
+        else:
+            self._chk(f(self.h, r.ptr, a.ptr, b.ptr, prime_idx, n))
+
+    def automorphism_order(self, k, is_ntt=True):
+        buf = self.alloc(self.N)
+        self._chk(self.lib.ace_automorphism_order(self.h, buf.ptr, k, int(is_ntt)))
+        return buf
+
+    # ---- polynomial ops
+    def poly(self, name, r, a, b, level, with_p=False):
+        self._chk(getattr(self.lib, "ace_poly_" + name)(self.h, r.ptr, a.ptr, b.ptr, level, int(with_p)))
+
+    def decomp_modup(self, res, src, level, part, is_ntt=True):
+        self._chk(self.lib.ace_decomp_modup(self.h, res.ptr, src.ptr, level, part, int(is_ntt)))
+
+    def precomp(self, res, src, level, is_ntt=True):
+        self._chk(self.lib.ace_precomp(self.h, res.ptr, src.ptr, level, int(is_ntt)))
+
+    def mod_down(self, res, src, level, is_ntt=True):
+        self._chk(self.lib.ace_mod_down(self.h, res.ptr, src.ptr, level, int(is_ntt)))
+
+    def rescale(self, res, src, level, is_ntt=True):
+        self._chk(self.lib.ace_rescale(self.h, res.ptr, src.ptr, level, int(is_ntt)))
+
+    def extend(self, res, src, level):
+        self._chk(self.lib.ace_extend(self.h, res.ptr, src.ptr, level))
+
+    def dot_prod(self, res, digits, key, key_stride, n_parts, level):
+        self._chk(self.lib.ace_dot_prod(self.h, res.ptr, digits.ptr, key.ptr, key_stride, n_parts, level))
+
+    # ---- ciphertext level
+    def mul_ciph3(self, d0, d1, d2, a0, a1, b0, b1, level):
+        self._chk(self.lib.ace_mul_ciph3(self.h, d0.ptr, d1.ptr, d2.ptr, a0.ptr, a1.ptr, b0.ptr, b1.ptr, level))
+
+    def fast_switch_key(self, o0, o1, digits, swk, level):
+        self._chk(self.lib.ace_fast_switch_key(self.h, o0.ptr, o1.ptr, digits.ptr, swk.ptr, level))
+
+    def relin(self, r0, r1, d0, d1, d2, swk, level):
+        self._chk(self.lib.ace_relin(self.h, r0.ptr, r1.ptr, d0.ptr, d1.ptr, d2.ptr, swk.ptr, level))
+
+    def rescale_ciph(self, r0, r1, c0, c1, level):
+        self._chk(self.lib.ace_rescale_ciph(self.h, r0.ptr, r1.ptr, c0.ptr, c1.ptr, level))
+
+    def mul_relin_rescale(self, r0, r1, a0, a1, b0, b1, swk, level):
+        self._chk(self.lib.ace_mul_relin_rescale(self.h, r0.ptr, r1.ptr, a0.ptr, a1.ptr, b0.ptr, b1.ptr, swk.ptr, level))
+
+    def fast_rotate(self, r0, r1, c0, digits, swk, order, level):
+        self._chk(self.lib.ace_fast_rotate(self.h, r0.ptr, r1.ptr, c0.ptr, digits.ptr, swk.ptr, order.ptr, level))
+
+    def rotate_batch(self, r0s, r1s, c0, c1, swks, orders, level):
+        n = len(swks)
+        ks = (_vp * n)(*[k.ptr for k in swks])
+        os_ = (_vp * n)(*[o.ptr for o in orders])
+        self._chk(self.lib.ace_rotate_batch(self.h, r0s.ptr, r1s.ptr, c0.ptr, c1.ptr, ks, os_, n, level))

@@ -1,0 +1,102 @@
+// Device-side data structures and 64-bit modular arithmetic for gfx950.
+//
+// All residues are 64-bit words in [0, q), q < 2^62.  There is no 64x64->128
+// VALU multiply on CDNA4; __umul64hi and `*` lower to v_mad_u64_u32 chains.
+// Three reductions are used, each value-identical to the reference's because
+// the canonical residue of an integer is unique:
+//   shoup_*    multiply by a constant w with precomputed floor(w*2^64/q)
+//              (Fast_mul_const_with_mod, include/util/modular.h:249-256)
+//   mulmod     product of two residues, shifted Barrett with a 64-bit mu
+//              (same result as Mul_int64_mod_barret, modular.h:231-241)
+//   barrett128 any 128-bit value, mu = floor(2^128/q)
+//              (Mod_barrett_128, modular.h:185-224)
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ace {
+
+typedef uint64_t u64;
+typedef int64_t  i64;
+typedef uint32_t u32;
+
+constexpr int kMaxPrimes = 96;
+
+struct DevPrime {
+  u64 q;
+  u64 mu_lo, mu_hi;  // floor(2^128/q)
+  u64 mu_sh;         // floor(2^(shift+64)/q)
+  u32 shift;         // bitlen(q)-1
+  u32 pad;
+  u64 ninv, ninv_p;  // N^-1 mod q and its Shoup companion
+};
+
+// What every kernel needs to find primes and twiddles.
+struct DevCtx {
+  const DevPrime* primes;
+  const u64 *rou, *rou_p, *irou, *irou_p;  // [num primes][N]
+  u32 N, logN;
+};
+
+// limb t of a launch -> prime index
+struct LimbMap {
+  uint8_t prime[kMaxPrimes];
+};
+
+// base conversion: target j -> prime index and limb position in the output
+struct ConvMap {
+  uint8_t prime[kMaxPrimes];
+  uint8_t out_limb[kMaxPrimes];
+};
+
+__device__ __forceinline__ u64 csub(u64 a, u64 q) { return a >= q ? a - q : a; }
+
+// a*w mod q up to one extra q: result in [0, 2q) for any a < 2^64
+__device__ __forceinline__ u64 shoup_lazy(u64 a, u64 w, u64 wp, u64 q) {
+  return a * w - __umul64hi(a, wp) * q;
+}
+__device__ __forceinline__ u64 shoup_mul(u64 a, u64 w, u64 wp, u64 q) {
+  return csub(shoup_lazy(a, w, wp, q), q);
+}
+
+// a*b mod q for a*b < 2^(2*(shift+1))
+__device__ __forceinline__ u64 mulmod(u64 a, u64 b, const DevPrime& p) {
+  u64 lo = a * b, hi = __umul64hi(a, b);
+  u64 x1 = (hi << (64 - p.shift)) | (lo >> p.shift);
+  u64 r  = lo - __umul64hi(x1, p.mu_sh) * p.q;  // < 3q
+  return csub(csub(r, p.q), p.q);
+}
+
+// (hi:lo) mod q for any 128-bit value
+__device__ __forceinline__ u64 barrett128(u64 hi, u64 lo, const DevPrime& p) {
+  u64 ll_hi = __umul64hi(lo, p.mu_lo);
+  u64 lh_lo = lo * p.mu_hi, lh_hi = __umul64hi(lo, p.mu_hi);
+  u64 hl_lo = hi * p.mu_lo, hl_hi = __umul64hi(hi, p.mu_lo);
+  u64 s1 = ll_hi + lh_lo;
+  u64 c1 = s1 < ll_hi;
+  u64 s2 = s1 + hl_lo;
+  u64 c2 = s2 < s1;
+  u64 qhat = lh_hi + hl_hi + c1 + c2 + hi * p.mu_hi;
+  u64 r = lo - qhat * p.q;  // < 2q
+  return csub(csub(r, p.q), p.q);
+}
+
+// acc += a*b over 128 bits
+__device__ __forceinline__ void mac128(u64& hi, u64& lo, u64 a, u64 b) {
+  u64 pl = a * b, ph = __umul64hi(a, b);
+  lo += pl;
+  hi += ph + (lo < pl);
+}
+
+// Add_int64_with_mod / Sub_int64_with_mod (modular.h:139-160), literally
+__device__ __forceinline__ u64 add_mod(u64 a, u64 b, u64 q) {
+  i64 s = (i64)(a + b);
+  return (u64)(s >= (i64)q ? s - (i64)q : s);
+}
+__device__ __forceinline__ u64 sub_mod(u64 a, u64 b, u64 q) {
+  i64 r = (i64)(a - b);
+  if (r > (i64)a || r < 0) r += (i64)q;
+  return (u64)r;
+}
+
+}  // namespace ace

@@ -1,0 +1,325 @@
+// Streaming RNS-polynomial kernels for gfx950: per-limb modular vector ops,
+// automorphism gather, ciphertext tensor product, fast base conversion,
+// switch-key inner product, Mod_down and Rescale tails.
+//
+// All are HBM-streaming except the base conversion, which is VALU-bound
+// (nd 128-bit multiply-accumulates plus one Barrett-128 per output word).
+// Grids are (ceil(n / (256*kUnroll)), n_limbs): blockIdx.y picks the limb and
+// with it the modulus, so modulus constants are wave-uniform (scalar loads).
+#include "ace_kernels.h"
+
+namespace ace {
+
+constexpr int kThreads = 256;
+constexpr int kUnroll = 4;
+
+static inline dim3 ew_grid(u64 n, u32 n_limbs, u32 z = 1) {
+  u64 per_block = (u64)kThreads * kUnroll;
+  return dim3((unsigned)((n + per_block - 1) / per_block), n_limbs, z);
+}
+
+#define ACE_EW_LOOP(i, n)                                                      \
+  for (u64 i = (u64)blockIdx.x * (kThreads * kUnroll) + threadIdx.x, _k = 0;   \
+       _k < kUnroll && i < (n); ++_k, i += kThreads)
+
+// ---- Hw_modadd ... Hw_modmuladd_scalar (hal/src/hal.c:15-121) -------------
+template <int OP>
+__global__ __launch_bounds__(kThreads) void ew_kernel(DevCtx c, u64* __restrict__ r, const u64* __restrict__ a,
+                                                      const u64* __restrict__ b, u64 scalar, LimbMap lm, u64 n) {
+  const u32 limb = blockIdx.y;
+  const DevPrime P = c.primes[lm.prime[limb]];
+  const u64 base = (u64)limb * n;
+#pragma unroll
+  ACE_EW_LOOP(i, n) {
+    u64 x = a[base + i];
+    u64 y = (OP >= EW_ADD_S) ? scalar : b[base + i];
+    u64 v;
+    if (OP == EW_ADD || OP == EW_ADD_S) v = add_mod(x, y, P.q);
+    else if (OP == EW_SUB || OP == EW_SUB_S) v = sub_mod(x, y, P.q);
+    else if (OP == EW_MUL || OP == EW_MUL_S) v = mulmod(x, y, P);
+    else v = add_mod(r[base + i], mulmod(x, y, P), P.q);
+    r[base + i] = v;
+  }
+}
+
+void launch_ew(hipStream_t st, const DevCtx& c, EwOp op, u64* r, const u64* a, const u64* b, u64 scalar,
+               const LimbMap& lm, u32 n_limbs, u64 n) {
+  if (!n || !n_limbs) return;
+  dim3 g = ew_grid(n, n_limbs);
+#define ACE_EW_CASE(OP) \
+  case OP: hipLaunchKernelGGL(ew_kernel<OP>, g, dim3(kThreads), 0, st, c, r, a, b, scalar, lm, n); break;
+  switch (op) {
+    ACE_EW_CASE(EW_ADD) ACE_EW_CASE(EW_SUB) ACE_EW_CASE(EW_MUL) ACE_EW_CASE(EW_MULADD)
+    ACE_EW_CASE(EW_ADD_S) ACE_EW_CASE(EW_SUB_S) ACE_EW_CASE(EW_MUL_S) ACE_EW_CASE(EW_MULADD_S)
+  }
+#undef ACE_EW_CASE
+}
+
+// ---- Hw_rotate / Automorphism_transform (hal.c:123-138, rns_poly.c:1056-1099)
+__global__ __launch_bounds__(kThreads) void gather_kernel(DevCtx c, u64* __restrict__ r0, u64* __restrict__ r1,
+                                                          const u64* __restrict__ a0, const u64* __restrict__ a1,
+                                                          const i64* __restrict__ order, LimbMap lm, u64 n) {
+  const u32 limb = blockIdx.y;
+  const u64 q = c.primes[lm.prime[limb]].q;
+  const u64 base = (u64)limb * n;
+#pragma unroll
+  ACE_EW_LOOP(i, n) {
+    i64 k = order[i];
+    if (k >= 0) {
+      r0[base + i] = a0[base + k];
+      if (r1) r1[base + i] = a1[base + k];
+    } else {
+      r0[base + i] = q - a0[base - k];
+      if (r1) r1[base + i] = q - a1[base - k];
+    }
+  }
+}
+
+void launch_gather(hipStream_t st, const DevCtx& c, u64* r, const u64* a, const i64* order, const LimbMap& lm,
+                   u32 n_limbs, u64 n) {
+  if (!n || !n_limbs) return;
+  hipLaunchKernelGGL(gather_kernel, ew_grid(n, n_limbs), dim3(kThreads), 0, st, c, r, (u64*)nullptr, a,
+                     (const u64*)nullptr, order, lm, n);
+}
+void launch_gather2(hipStream_t st, const DevCtx& c, u64* r0, u64* r1, const u64* a0, const u64* a1,
+                    const i64* order, const LimbMap& lm, u32 n_limbs, u64 n) {
+  if (!n || !n_limbs) return;
+  hipLaunchKernelGGL(gather_kernel, ew_grid(n, n_limbs), dim3(kThreads), 0, st, c, r0, r1, a0, a1, order, lm, n);
+}
+
+// ---- Mul_ciphertext3 (evaluator.c:142-175) in one pass -------------------
+__global__ __launch_bounds__(kThreads) void tensor_kernel(DevCtx c, u64* __restrict__ d0, u64* __restrict__ d1,
+                                                          u64* __restrict__ d2, const u64* __restrict__ a0,
+                                                          const u64* __restrict__ a1, const u64* __restrict__ b0,
+                                                          const u64* __restrict__ b1, LimbMap lm) {
+  const u32 limb = blockIdx.y;
+  const DevPrime P = c.primes[lm.prime[limb]];
+  const u64 n = c.N, base = (u64)limb * n;
+#pragma unroll
+  ACE_EW_LOOP(i, n) {
+    u64 x0 = a0[base + i], x1 = a1[base + i], y0 = b0[base + i], y1 = b1[base + i];
+    d0[base + i] = mulmod(x0, y0, P);
+    d1[base + i] = add_mod(mulmod(x0, y1, P), mulmod(x1, y0, P), P.q);
+    d2[base + i] = mulmod(x1, y1, P);
+  }
+}
+
+void launch_tensor(hipStream_t st, const DevCtx& c, u64* d0, u64* d1, u64* d2, const u64* a0, const u64* a1,
+                   const u64* b0, const u64* b1, const LimbMap& lm, u32 n_limbs) {
+  if (!n_limbs) return;
+  hipLaunchKernelGGL(tensor_kernel, ew_grid(c.N, n_limbs), dim3(kThreads), 0, st, c, d0, d1, d2, a0, a1, b0, b1, lm);
+}
+
+// ---- fast base conversion (rns_poly.c:218-242, rns_poly_impl.c:324-336) ----
+// One thread per coefficient and kConvTargets targets; the nd source words
+// stay in registers, the cofactor table is read through wave-uniform loads.
+constexpr int kConvTargets = 4;
+constexpr int kConvMaxSrc = 16;
+
+__global__ __launch_bounds__(kThreads) void baseconv_kernel(DevCtx c, u64* __restrict__ out,
+                                                            const u64* __restrict__ t, const u64* __restrict__ hat,
+                                                            u32 hat_stride, u32 nd, u32 nc, ConvMap map) {
+  const u64 n = c.N;
+  const u64 i = (u64)blockIdx.x * kThreads + threadIdx.x;
+  if (i >= n) return;
+  const u32 j0 = blockIdx.y * kConvTargets;
+  if (nd <= kConvMaxSrc) {
+    u64 x[kConvMaxSrc];
+#pragma unroll
+    for (int k = 0; k < kConvMaxSrc; ++k) x[k] = (u32)k < nd ? t[(u64)k * n + i] : 0;
+#pragma unroll
+    for (int jj = 0; jj < kConvTargets; ++jj) {
+      u32 j = j0 + jj;
+      if (j >= nc) break;
+      u64 hi = 0, lo = 0;
+#pragma unroll
+      for (int k = 0; k < kConvMaxSrc; ++k)
+        if ((u32)k < nd) mac128(hi, lo, x[k], hat[(u64)k * hat_stride + j]);
+      out[(u64)map.out_limb[j] * n + i] = barrett128(hi, lo, c.primes[map.prime[j]]);
+    }
+  } else {
+    for (int jj = 0; jj < kConvTargets; ++jj) {
+      u32 j = j0 + jj;
+      if (j >= nc) break;
+      const DevPrime P = c.primes[map.prime[j]];
+      u64 hi = 0, lo = 0;
+      for (u32 k = 0; k < nd; ++k) {
+        mac128(hi, lo, t[(u64)k * n + i], hat[(u64)k * hat_stride + j]);
+        if ((k & 7) == 7) { lo = barrett128(hi, lo, P); hi = 0; }  // keep the sum below 2^128
+      }
+      out[(u64)map.out_limb[j] * n + i] = barrett128(hi, lo, P);
+    }
+  }
+}
+
+void launch_baseconv(hipStream_t st, const DevCtx& c, u64* out, const u64* t, const u64* hat, u32 hat_stride,
+                     u32 nd, u32 nc, const ConvMap& map) {
+  if (!nd || !nc) return;
+  dim3 g((c.N + kThreads - 1) / kThreads, (nc + kConvTargets - 1) / kConvTargets);
+  hipLaunchKernelGGL(baseconv_kernel, g, dim3(kThreads), 0, st, c, out, t, hat, hat_stride, nd, nc, map);
+}
+
+// ---- Dot_prod (rns_poly.c:502-529, rns_poly_impl.c:102-162) ----------------
+// Both key halves in one pass so the digits are read once.  Up to 8 products
+// are accumulated in 128 bits before one Barrett-128 (the reference's
+// Fast_dotprod_poly); the result equals the reference's default
+// multiply-reduce-add chain because canonical residues are unique.
+template <bool TWO>
+__global__ __launch_bounds__(kThreads) void dotprod_kernel(DevCtx c, u64* __restrict__ out0, u64* __restrict__ out1,
+                                                           const u64* __restrict__ digits, u64 digit_stride,
+                                                           const u64* __restrict__ key0, const u64* __restrict__ key1,
+                                                           u64 key_stride, u32 n_parts, LimbMap lm, LimbMap key_limb) {
+  const u32 limb = blockIdx.y;
+  const DevPrime P = c.primes[lm.prime[limb]];
+  const u64 n = c.N, dbase = (u64)limb * n, kbase = (u64)key_limb.prime[limb] * n;
+#pragma unroll
+  ACE_EW_LOOP(i, n) {
+    u64 h0 = 0, l0 = 0, h1 = 0, l1 = 0;
+    for (u32 d = 0; d < n_parts; ++d) {
+      u64 x = digits[d * digit_stride + dbase + i];
+      mac128(h0, l0, x, key0[d * key_stride + kbase + i]);
+      if (TWO) mac128(h1, l1, x, key1[d * key_stride + kbase + i]);
+      if ((d & 7) == 7 && d + 1 < n_parts) {
+        l0 = barrett128(h0, l0, P); h0 = 0;
+        if (TWO) { l1 = barrett128(h1, l1, P); h1 = 0; }
+      }
+    }
+    out0[dbase + i] = barrett128(h0, l0, P);
+    if (TWO) out1[dbase + i] = barrett128(h1, l1, P);
+  }
+}
+
+void launch_dotprod(hipStream_t st, const DevCtx& c, u64* out0, u64* out1, const u64* digits, u64 digit_stride,
+                    const u64* key0, const u64* key1, u64 key_stride, u32 n_parts, const LimbMap& lm,
+                    const LimbMap& key_limb, u32 n_limbs) {
+  if (!n_limbs) return;
+  dim3 g = ew_grid(c.N, n_limbs);
+  if (out1)
+    hipLaunchKernelGGL(dotprod_kernel<true>, g, dim3(kThreads), 0, st, c, out0, out1, digits, digit_stride, key0,
+                       key1, key_stride, n_parts, lm, key_limb);
+  else
+    hipLaunchKernelGGL(dotprod_kernel<false>, g, dim3(kThreads), 0, st, c, out0, out1, digits, digit_stride, key0,
+                       key1, key_stride, n_parts, lm, key_limb);
+}
+
+// ---- Mod_down tail (rns_poly.c:292-303): (src - y) * P^-1 [+ addend] --------
+__global__ __launch_bounds__(kThreads) void moddown_tail_kernel(DevCtx c, u64* __restrict__ out,
+                                                                const u64* __restrict__ src,
+                                                                const u64* __restrict__ y,
+                                                                const u64* __restrict__ addend,
+                                                                const u64* __restrict__ cst, LimbMap lm) {
+  const u32 limb = blockIdx.y;
+  const u64 q = c.primes[lm.prime[limb]].q;
+  const u64 w = cst[2 * limb], wp = cst[2 * limb + 1];
+  const u64 n = c.N, base = (u64)limb * n;
+#pragma unroll
+  ACE_EW_LOOP(i, n) {
+    u64 v = shoup_mul(sub_mod(src[base + i], y[base + i], q), w, wp, q);
+    if (addend) v = add_mod(v, addend[base + i], q);
+    out[base + i] = v;
+  }
+}
+
+void launch_moddown_tail(hipStream_t st, const DevCtx& c, u64* out, const u64* src, const u64* y,
+                         const u64* addend, const u64* cst, const LimbMap& lm, u32 n_limbs) {
+  if (!n_limbs) return;
+  hipLaunchKernelGGL(moddown_tail_kernel, ew_grid(c.N, n_limbs), dim3(kThreads), 0, st, c, out, src, y, addend, cst,
+                     lm);
+}
+
+// ---- Rescale (rns_poly.c:310-404) ------------------------------------------
+// Switch_modulus (include/util/modular.h:296-322): centred lift q_l -> q_t.
+// cst per limb: K, K' (Shoup), diff = q_t - (q_l mod q_t)
+__global__ __launch_bounds__(kThreads) void rescale_switch_kernel(DevCtx c, u64* __restrict__ u,
+                                                                  const u64* __restrict__ last, u32 last_prime,
+                                                                  const u64* __restrict__ cst, LimbMap lm) {
+  const u32 limb = blockIdx.y;
+  const DevPrime P = c.primes[lm.prime[limb]];
+  const u64 ql = c.primes[last_prime].q, half = ql >> 1;
+  const u64 K = cst[3 * limb], Kp = cst[3 * limb + 1], diff = cst[3 * limb + 2];
+  const u64 n = c.N, base = (u64)limb * n;
+#pragma unroll
+  ACE_EW_LOOP(i, n) {
+    u64 v = last[i];
+    if (P.q > ql) {
+      if (v > half) v += P.q - ql;
+    } else {
+      if (v > half) v += diff;
+      if (v >= P.q) v = barrett128(0, v, P);
+    }
+    u[base + i] = shoup_mul(v, K, Kp, P.q);
+  }
+}
+void launch_rescale_switch(hipStream_t st, const DevCtx& c, u64* u, const u64* last, u32 last_prime,
+                           const u64* cst, const LimbMap& lm, u32 n_limbs) {
+  if (!n_limbs) return;
+  hipLaunchKernelGGL(rescale_switch_kernel, ew_grid(c.N, n_limbs), dim3(kThreads), 0, st, c, u, last, last_prime,
+                     cst, lm);
+}
+
+__global__ __launch_bounds__(kThreads) void rescale_tail_kernel(DevCtx c, u64* __restrict__ out,
+                                                                const u64* __restrict__ src,
+                                                                const u64* __restrict__ u,
+                                                                const u64* __restrict__ cst, LimbMap lm) {
+  const u32 limb = blockIdx.y;
+  const u64 q = c.primes[lm.prime[limb]].q;
+  const u64 w = cst[2 * limb], wp = cst[2 * limb + 1];
+  const u64 n = c.N, base = (u64)limb * n;
+#pragma unroll
+  ACE_EW_LOOP(i, n) out[base + i] = add_mod(shoup_mul(src[base + i], w, wp, q), u[base + i], q);
+}
+void launch_rescale_tail(hipStream_t st, const DevCtx& c, u64* out, const u64* src, const u64* u, const u64* cst,
+                         const LimbMap& lm, u32 n_limbs) {
+  if (!n_limbs) return;
+  hipLaunchKernelGGL(rescale_tail_kernel, ew_grid(c.N, n_limbs), dim3(kThreads), 0, st, c, out, src, u, cst, lm);
+}
+
+// coefficient form (rns_poly.c:380-400): plain residue of the last limb
+__global__ __launch_bounds__(kThreads) void rescale_coef_kernel(DevCtx c, u64* __restrict__ out,
+                                                                const u64* __restrict__ src,
+                                                                const u64* __restrict__ last,
+                                                                const u64* __restrict__ cst, LimbMap lm) {
+  const u32 limb = blockIdx.y;
+  const DevPrime P = c.primes[lm.prime[limb]];
+  const u64 w = cst[2 * limb], wp = cst[2 * limb + 1];
+  const u64 n = c.N, base = (u64)limb * n;
+#pragma unroll
+  ACE_EW_LOOP(i, n) {
+    u64 lc = barrett128(0, last[i], P);
+    out[base + i] = shoup_mul(sub_mod(src[base + i], lc, P.q), w, wp, P.q);
+  }
+}
+void launch_rescale_coef(hipStream_t st, const DevCtx& c, u64* out, const u64* src, const u64* last,
+                         const u64* cst, const LimbMap& lm, u32 n_limbs) {
+  if (!n_limbs) return;
+  hipLaunchKernelGGL(rescale_coef_kernel, ew_grid(c.N, n_limbs), dim3(kThreads), 0, st, c, out, src, last, cst, lm);
+}
+
+// ---- multiply every limb by its own constant (Extend, rns_poly.c:483-500) ---
+__global__ __launch_bounds__(kThreads) void mul_const_kernel(DevCtx c, u64* __restrict__ out,
+                                                             const u64* __restrict__ src,
+                                                             const u64* __restrict__ cst, LimbMap lm) {
+  const u32 limb = blockIdx.y;
+  const u64 q = c.primes[lm.prime[limb]].q;
+  const u64 w = cst[2 * limb], wp = cst[2 * limb + 1];
+  const u64 n = c.N, base = (u64)limb * n;
+#pragma unroll
+  ACE_EW_LOOP(i, n) out[base + i] = shoup_mul(src[base + i], w, wp, q);
+}
+void launch_mul_const(hipStream_t st, const DevCtx& c, u64* out, const u64* src, const u64* cst, const LimbMap& lm,
+                      u32 n_limbs) {
+  if (!n_limbs) return;
+  hipLaunchKernelGGL(mul_const_kernel, ew_grid(c.N, n_limbs), dim3(kThreads), 0, st, c, out, src, cst, lm);
+}
+
+__global__ __launch_bounds__(kThreads) void fill_zero_kernel(u64* __restrict__ p, u64 n) {
+  for (u64 i = (u64)blockIdx.x * kThreads + threadIdx.x; i < n; i += (u64)gridDim.x * kThreads) p[i] = 0;
+}
+void launch_fill_zero(hipStream_t st, u64* p, u64 n) {
+  if (!n) return;
+  u64 blocks = (n + kThreads - 1) / kThreads;
+  if (blocks > 65536) blocks = 65536;
+  hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, st, p, n);
+}
+
+}  // namespace ace

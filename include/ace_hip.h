@@ -1,0 +1,176 @@
+/*
+ * MI355X (gfx950) CKKS polynomial runtime -- device C-ABI.
+ *
+ * Plain C: opaque context handle, raw device pointers, sizes, prime indices.
+ * Every polynomial is int64 limb-major (`data[limb * degree + i]`, values in
+ * [0, q_limb)), exactly the reference's POLYNOMIAL::_data layout
+ * (fhe-cmplr/rtlib/ant/include/poly/rns_poly.h:23-32,253-256), but resident in
+ * HBM.  All calls are asynchronous on the context's HIP stream unless stated;
+ * results are visible to the host after ace_sync() or a download.
+ *
+ * Each entry point names the reference function it replaces (paths relative
+ * to fhe-cmplr/rtlib/ant).  Prime index convention: 0..num_q-1 are the Q
+ * primes, num_q..num_q+num_p-1 the P (special) primes.
+ *
+ * Return convention: functions returning int give 0 on success, non-zero on a
+ * rejected call (message via ace_last_error()); nothing is launched then.
+ */
+#ifndef ACE_HIP_H
+#define ACE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ace_ctx ace_ctx;
+
+/* ---- context -------------------------------------------------------------
+ * Replaces Init_crtcontext_with_prime_size (util/src/crt.c:607-618): same
+ * prime sequence, same 2N-th roots, same number of special primes, all NTT and
+ * base-conversion tables built on the host and uploaded once. */
+ace_ctx* ace_ctx_create(uint32_t degree, size_t num_q, size_t q0_bits,
+                        size_t sf_bits, size_t num_parts);
+/* Replaces Init_crtcontext (util/src/crt.c:596-605) with the Q primes given. */
+ace_ctx* ace_ctx_create_with_primes(uint32_t degree, size_t num_q,
+                                    const int64_t* q_primes, size_t num_parts);
+/* Both return NULL on invalid parameters.  On a machine without a HIP device
+ * the context still holds every host-side table (primes, roots, cofactors) and
+ * answers the getters below, but each call that would touch the GPU is
+ * rejected with an error: there is no CPU fallback. */
+void        ace_ctx_destroy(ace_ctx* ctx);
+int         ace_has_device(const ace_ctx* ctx);
+const char* ace_last_error(void);
+/* Degree / Get_q_cnt / Get_p_cnt / Get_q_parts (context/src/ckks_context.c:213-237) */
+uint32_t ace_degree(const ace_ctx* ctx);
+size_t   ace_num_q(const ace_ctx* ctx);
+size_t   ace_num_p(const ace_ctx* ctx);
+size_t   ace_num_parts(const ace_ctx* ctx);
+size_t   ace_part_size(const ace_ctx* ctx);
+/* Get_num_decomp (util/src/crt.c:1135-1144) */
+size_t   ace_num_decomp(const ace_ctx* ctx, size_t level);
+int64_t  ace_prime(const ace_ctx* ctx, size_t prime_idx);
+int64_t  ace_root(const ace_ctx* ctx, size_t prime_idx);
+/* MODULUS fields (include/util/modular.h:21-26): val, br_k, br_m, prec128 lo, hi */
+void     ace_modulus(const ace_ctx* ctx, size_t prime_idx, uint64_t out[5]);
+
+/* Host copies of the precomputed tables (what the kernels read from HBM), for
+ * inspection and table-level parity checks.
+ * ace_host_twiddles: which = 0 rou, 1 rou Shoup, 2 rou_inv, 3 rou_inv Shoup
+ *   (Precompute_ntt, util/src/ntt.c:91-138), `degree` words.
+ * ace_host_tbl_modup: _l_hat_inv_modq / _l_hat_modp of digit `part` at `level`
+ *   (util/src/crt.c:459-566): hat_inv[n_digit], hat[n_digit][n_compl], and the
+ *   prime index of each target limb in the reference's complement order.
+ * ace_host_tbl_moddown: (P/p_j)^-1 mod p_j [num_p], (P/p_j) mod q_i [num_q][num_p],
+ *   P^-1 mod q_i [num_q], P mod q_i [num_q] (crt.c:264-291,354-420).
+ * ace_host_tbl_rescale: q_l^-1 mod q_i and the reference's second rescale
+ *   constant (== -q_l^-1 mod q_i), i < level-1 (crt.c:299-349). */
+int ace_host_twiddles(const ace_ctx* ctx, size_t prime_idx, int which, uint64_t* out);
+int ace_host_tbl_modup(const ace_ctx* ctx, size_t level, size_t part, int64_t* hat_inv, int64_t* hat,
+                       int32_t* compl_idx, size_t* n_digit, size_t* n_compl);
+int ace_host_tbl_moddown(const ace_ctx* ctx, int64_t* phat_inv, int64_t* phat_modq, int64_t* pinv_modq, int64_t* pmodq);
+int ace_host_tbl_rescale(const ace_ctx* ctx, size_t level, int64_t* ql_inv, int64_t* neg_ql_inv);
+/* Precompute_automorphism_order into host memory (`degree` words) */
+int ace_host_automorphism_order(const ace_ctx* ctx, int64_t* host_order, uint32_t k, int is_ntt);
+
+/* ---- device memory -------------------------------------------------------
+ * Replaces the malloc+memset of Alloc_poly_data (include/poly/rns_poly.h:109-119):
+ * zero-filled HBM, n int64 words. */
+int64_t* ace_alloc(ace_ctx* ctx, size_t n_words);
+void     ace_free(ace_ctx* ctx, int64_t* dev_ptr);
+int      ace_upload(ace_ctx* ctx, int64_t* dev_dst, const int64_t* host_src, size_t n_words);
+int      ace_download(ace_ctx* ctx, int64_t* host_dst, const int64_t* dev_src, size_t n_words); /* synchronises */
+int      ace_copy(ace_ctx* ctx, int64_t* dev_dst, const int64_t* dev_src, size_t n_words);
+int      ace_zero(ace_ctx* ctx, int64_t* dev_dst, size_t n_words);
+int      ace_sync(ace_ctx* ctx);
+/* HIP-event stopwatch on the context's stream (for benchmarks) */
+int      ace_timer_start(ace_ctx* ctx);
+float    ace_timer_stop_ms(ace_ctx* ctx); /* synchronises; <0 on error */
+
+/* ---- NTT -----------------------------------------------------------------
+ * Replaces Ftt_fwd / Ftt_inv (util/src/ntt.c:140-164) as driven by
+ * Conv_poly2ntt(_inplace)(_with_primes), Conv_ntt2poly* (poly/src/rns_poly.c:
+ * 608-699, rns_poly_impl.c:164-285) and Hw_ntt / Hw_intt (hal/src/hal.c:140-153).
+ * Polynomial p (0..n_polys-1) limb t (0..n_limbs-1) lives at
+ * base + (p*poly_stride_limbs + t)*degree and uses prime prime_idx[t].
+ * Forward: natural order in, bit-reversed out.  Inverse: the opposite, 1/N
+ * included.  dst may equal src. */
+int ace_ntt(ace_ctx* ctx, int64_t* dst, const int64_t* src, const int32_t* prime_idx,
+            size_t n_limbs, size_t n_polys, size_t poly_stride_limbs);
+int ace_intt(ace_ctx* ctx, int64_t* dst, const int64_t* src, const int32_t* prime_idx,
+             size_t n_limbs, size_t n_polys, size_t poly_stride_limbs);
+
+/* ---- per-limb vector ops: Hw_* (hal/src/hal.c:15-138) ----------------------
+ * n coefficients with the modulus of prime_idx. */
+int ace_hw_modadd(ace_ctx* ctx, int64_t* res, const int64_t* a, const int64_t* b, size_t prime_idx, size_t n);
+int ace_hw_modsub(ace_ctx* ctx, int64_t* res, const int64_t* a, const int64_t* b, size_t prime_idx, size_t n);
+int ace_hw_modmul(ace_ctx* ctx, int64_t* res, const int64_t* a, const int64_t* b, size_t prime_idx, size_t n);
+int ace_hw_modmuladd(ace_ctx* ctx, int64_t* res, const int64_t* a, const int64_t* b, size_t prime_idx, size_t n);
+int ace_hw_modadd_scalar(ace_ctx* ctx, int64_t* res, const int64_t* a, int64_t s, size_t prime_idx, size_t n);
+int ace_hw_modsub_scalar(ace_ctx* ctx, int64_t* res, const int64_t* a, int64_t s, size_t prime_idx, size_t n);
+int ace_hw_modmul_scalar(ace_ctx* ctx, int64_t* res, const int64_t* a, int64_t s, size_t prime_idx, size_t n);
+int ace_hw_modmuladd_scalar(ace_ctx* ctx, int64_t* res, const int64_t* a, int64_t s, size_t prime_idx, size_t n);
+/* Hw_rotate: res[i] = order[i] >= 0 ? a[order[i]] : q - a[-order[i]]; order is a device table */
+int ace_hw_rotate(ace_ctx* ctx, int64_t* res, const int64_t* a, const int64_t* order, size_t prime_idx, size_t n);
+
+/* ---- automorphism tables (util/src/number_theory.c:192-231) ---------------- */
+uint32_t ace_find_automorphism_index(const ace_ctx* ctx, int32_t rot_idx);
+/* Precompute_automorphism_order into a device table of `degree` words */
+int ace_automorphism_order(ace_ctx* ctx, int64_t* dev_order, uint32_t k, int is_ntt);
+
+/* ---- RNS polynomial ops (poly/src/rns_poly.c) -------------------------------
+ * A polynomial "at level l" is l Q limbs; "extended" adds the num_p P limbs
+ * right after them (l + num_p contiguous limbs). */
+/* Add_poly / Sub_poly / Mul_poly (:852-1010), Automorphism_transform (:1056-1099) */
+int ace_poly_add(ace_ctx* ctx, int64_t* res, const int64_t* a, const int64_t* b, size_t level, int with_p);
+int ace_poly_sub(ace_ctx* ctx, int64_t* res, const int64_t* a, const int64_t* b, size_t level, int with_p);
+int ace_poly_mul(ace_ctx* ctx, int64_t* res, const int64_t* a, const int64_t* b, size_t level, int with_p);
+int ace_poly_automorphism(ace_ctx* ctx, int64_t* res, const int64_t* a, const int64_t* order, size_t level, int with_p);
+/* Decomp_modup (:160-258) (== Decomp :74-105 + Mod_up :107-158): digit `part`
+ * of src (level limbs) raised to level+num_p limbs. */
+int ace_decomp_modup(ace_ctx* ctx, int64_t* res, const int64_t* src, size_t level, size_t part, int is_ntt);
+/* Precomp / Alloc_precomp (:416-481): all digits, res = num_decomp x (level+num_p) limbs */
+int ace_precomp(ace_ctx* ctx, int64_t* res, const int64_t* src, size_t level, int is_ntt);
+/* Mod_down (:260-308): src level+num_p limbs -> res level limbs */
+int ace_mod_down(ace_ctx* ctx, int64_t* res, const int64_t* src, size_t level, int is_ntt);
+/* Rescale (:310-404): src level limbs -> res level-1 limbs */
+int ace_rescale(ace_ctx* ctx, int64_t* res, const int64_t* src, size_t level, int is_ntt);
+/* Extend (:483-500): src level limbs -> res level+num_p limbs (P limbs zero) */
+int ace_extend(ace_ctx* ctx, int64_t* res, const int64_t* src, size_t level);
+/* Dot_prod / Fast_dot_prod (:502-529): digits = n_parts x (level+num_p) limbs;
+ * key = n_parts polynomials, key_stride words apart, each laid out as all num_q
+ * Q limbs followed by num_p P limbs and viewed at `level` (Derive_poly :701-707). */
+int ace_dot_prod(ace_ctx* ctx, int64_t* res, const int64_t* digits, const int64_t* key,
+                 size_t key_stride, size_t n_parts, size_t level);
+
+/* ---- ciphertext level (ckks/src/evaluator.c, ckks/src/cipher.c) ------------
+ * A ciphertext at level l is two polynomials (c0, c1) of l limbs.  A switch
+ * key is [num_parts][2][(num_q+num_p) limbs]: per digit the b polynomial then
+ * the a polynomial (include/ckks/switch_key.h:27-29, public_key.h:24-27). */
+/* Mul_ciphertext3 (evaluator.c:142-175) */
+int ace_mul_ciph3(ace_ctx* ctx, int64_t* d0, int64_t* d1, int64_t* d2, const int64_t* a0, const int64_t* a1,
+                  const int64_t* b0, const int64_t* b1, size_t level);
+/* Fast_switch_key (evaluator.c:411-462) on hoisted digits: out0/out1 level limbs */
+int ace_fast_switch_key(ace_ctx* ctx, int64_t* out0, int64_t* out1, const int64_t* digits, const int64_t* swk, size_t level);
+/* Relinearize_ciph3 (evaluator.c:288-306) */
+int ace_relin(ace_ctx* ctx, int64_t* r0, int64_t* r1, const int64_t* d0, const int64_t* d1, const int64_t* d2,
+              const int64_t* swk, size_t level);
+/* Rescale_ciphertext (evaluator.c:342-362): level -> level-1 limbs */
+int ace_rescale_ciph(ace_ctx* ctx, int64_t* r0, int64_t* r1, const int64_t* c0, const int64_t* c1, size_t level);
+/* Mul_ciphertext + Rescale_ciphertext (evaluator.c:177-190, 342-362): r0/r1 level-1 limbs */
+int ace_mul_relin_rescale(ace_ctx* ctx, int64_t* r0, int64_t* r1, const int64_t* a0, const int64_t* a1,
+                          const int64_t* b0, const int64_t* b1, const int64_t* swk, size_t level);
+/* Fast_rotate (evaluator.c:503-522) with the digits of c1 hoisted (Alloc_precomp) */
+int ace_fast_rotate(ace_ctx* ctx, int64_t* r0, int64_t* r1, const int64_t* c0, const int64_t* digits,
+                    const int64_t* swk, const int64_t* order, size_t level);
+/* Rotate_batch_ciph (cipher.c:459-479): one ModUp of c1, then `count` rotations.
+ * r0s/r1s: count x level limbs; swks/orders: host arrays of `count` device pointers. */
+int ace_rotate_batch(ace_ctx* ctx, int64_t* r0s, int64_t* r1s, const int64_t* c0, const int64_t* c1,
+                     const int64_t* const* swks, const int64_t* const* orders, size_t count, size_t level);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ACE_HIP_H */
