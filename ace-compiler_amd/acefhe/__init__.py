@@ -59,6 +59,7 @@ def _sig(lib):
     f("ace_timer_stop_ms", C.c_float, _vp)
     f("ace_ntt", C.c_int, _vp, _vp, _vp, _i32p, _sz, _sz, _sz)
     f("ace_intt", C.c_int, _vp, _vp, _vp, _i32p, _sz, _sz, _sz)
+    f("ace_ntt_pass", C.c_int, _vp, _vp, _vp, _i32p, _sz, _sz, _sz, C.c_int, C.c_int)
     for n in ("modadd", "modsub", "modmul", "modmuladd"):
         f("ace_hw_" + n, C.c_int, _vp, _vp, _vp, _vp, _sz, _sz)
         f("ace_hw_" + n + "_scalar", C.c_int, _vp, _vp, _vp, C.c_int64, _sz, _sz)
@@ -89,7 +90,7 @@ EXPORTS = [
     "ace_degree", "ace_num_q", "ace_num_p", "ace_num_parts", "ace_part_size", "ace_num_decomp", "ace_prime",
     "ace_root", "ace_modulus", "ace_host_twiddles", "ace_host_tbl_modup", "ace_host_tbl_moddown",
     "ace_host_tbl_rescale", "ace_host_automorphism_order", "ace_alloc", "ace_free", "ace_upload", "ace_download",
-    "ace_copy", "ace_zero", "ace_sync", "ace_timer_start", "ace_timer_stop_ms", "ace_ntt", "ace_intt",
+    "ace_copy", "ace_zero", "ace_sync", "ace_timer_start", "ace_timer_stop_ms", "ace_ntt", "ace_intt", "ace_ntt_pass",
     "ace_hw_modadd", "ace_hw_modsub", "ace_hw_modmul", "ace_hw_modmuladd", "ace_hw_modadd_scalar",
     "ace_hw_modsub_scalar", "ace_hw_modmul_scalar", "ace_hw_modmuladd_scalar", "ace_hw_rotate",
     "ace_find_automorphism_index", "ace_automorphism_order", "ace_poly_add", "ace_poly_sub", "ace_poly_mul",
@@ -254,6 +255,11 @@ class Context:
 
     def intt(self, dst, src, prime_idx, n_polys=1, poly_stride_limbs=0):
         self.ntt(dst, src, prime_idx, n_polys, poly_stride_limbs, inverse=True)
+
+    def ntt_pass(self, dst, src, prime_idx, n_polys, poly_stride_limbs, inverse, which):
+        idx = np.ascontiguousarray(prime_idx, dtype=np.int32)
+        self._chk(self.lib.ace_ntt_pass(self.h, dst.ptr, src.ptr, idx.ctypes.data_as(_i32p), len(idx), n_polys,
+                                        poly_stride_limbs, int(inverse), which))
 
     # ---- Hw_*
     def hw(self, name, r, a, b, prime_idx, n=None):

@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <memory>
@@ -162,6 +163,25 @@ struct ace_ctx {
     d.irou_p = upload_vec(h.irou_p);
     d.N = h.N;
     d.logN = h.logN;
+    {
+      // FP64 twiddles for the primes the FP64 NTT back end can take
+      const char* force_int = std::getenv("ACE_NTT_FORCE_INT");
+      bool use_fp = !(force_int && force_int[0] == '1') && h.logN > 12;
+      std::vector<double> w(T * h.N, 0.0), iw(T * h.N, 0.0);
+      for (size_t i = 0; i < T; ++i) {
+        d.fp_ok[i] = (use_fp && h.primes[i].q < kFpPrimeLimit) ? 1 : 0;
+        if (!d.fp_ok[i]) continue;
+        for (size_t k = 0; k < h.N; ++k) {
+          size_t o = i * h.N + k;
+          w[o] = (double)h.rou[o];
+          iw[o] = (double)h.irou[o];
+        }
+      }
+      if (use_fp) {
+        d.roud = upload_vec(w);
+        d.iroud = upload_vec(iw);
+      }
+    }
     for (size_t i = 0; i < h.L && i < (size_t)kMaxPrimes; ++i) q_lm.prime[i] = (uint8_t)i;
     for (size_t j = 0; j < h.K; ++j) p_lm.prime[j] = (uint8_t)(h.L + j);
     // P -> Q tables, transposed to [K][L] so that targets are contiguous
@@ -430,7 +450,7 @@ float ace_timer_stop_ms(ace_ctx* c) {
 
 // ---- NTT ---------------------------------------------------------------------
 static int ntt_common(ace_ctx* c, int64_t* dst, const int64_t* src, const int32_t* prime_idx, size_t n_limbs,
-                      size_t n_polys, size_t stride_limbs, bool inverse) {
+                      size_t n_polys, size_t stride_limbs, bool inverse, int passes = 3) {
   ACE_TRY
   if (n_limbs == 0 || n_polys == 0) return 0;
   if (!dst || !src || !prime_idx) return fail("ace_ntt: null argument");
@@ -443,7 +463,7 @@ static int ntt_common(ace_ctx* c, int64_t* dst, const int64_t* src, const int32_
     lm.prime[t] = (uint8_t)prime_idx[t];
   }
   if (!launch_ntt(c->stream, c->d, U(dst), U(src), lm, nullptr, (u32)n_limbs, (u32)n_polys,
-                  (u64)stride_limbs * c->h.N, inverse, nullptr))
+                  (u64)stride_limbs * c->h.N, inverse, nullptr, passes))
     return fail("ace_ntt: ring degree not supported");
   ACE_CATCH_INT
 }
@@ -454,6 +474,13 @@ int ace_ntt(ace_ctx* c, int64_t* dst, const int64_t* src, const int32_t* prime_i
 int ace_intt(ace_ctx* c, int64_t* dst, const int64_t* src, const int32_t* prime_idx, size_t n_limbs, size_t n_polys,
              size_t stride) {
   return ntt_common(c, dst, src, prime_idx, n_limbs, n_polys, stride, true);
+}
+
+int ace_ntt_pass(ace_ctx* c, int64_t* dst, const int64_t* src, const int32_t* prime_idx, size_t n_limbs,
+                 size_t n_polys, size_t stride, int inverse, int pass) {
+  if (pass != 1 && pass != 2) return fail("ace_ntt_pass: pass must be 1 or 2");
+  if (c && c->h.logN <= 12) return fail("ace_ntt_pass: ring degrees up to 4096 are a single kernel");
+  return ntt_common(c, dst, src, prime_idx, n_limbs, n_polys, stride, inverse != 0, pass);
 }
 
 // ---- Hw_* ---------------------------------------------------------------------

@@ -35,8 +35,15 @@ struct DevPrime {
 struct DevCtx {
   const DevPrime* primes;
   const u64 *rou, *rou_p, *irou, *irou_p;  // [num primes][N]
+  // FP64 copies of rou / irou for the primes flagged in fp_ok
+  const double *roud, *iroud;
   u32 N, logN;
+  uint8_t fp_ok[kMaxPrimes];  // prime is small enough for the FP64 NTT back end
 };
+
+// largest prime the FP64 back end accepts: below 2^50.2, so that eight stages'
+// worth of lazily accumulated magnitude stays under 2^53 (see ace_ntt.hip)
+constexpr u64 kFpPrimeLimit = 1290000000000000ull;
 
 // limb t of a launch -> prime index
 struct LimbMap {

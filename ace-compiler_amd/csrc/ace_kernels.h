@@ -11,8 +11,10 @@ enum EwOp { EW_ADD, EW_SUB, EW_MUL, EW_MULADD, EW_ADD_S, EW_SUB_S, EW_MUL_S, EW_
 // base + p*poly_stride + t*N words).  scale: optional device array of
 // 2*n_limbs words (constant, Shoup companion) replacing 1/N in the inverse.
 // pos: optional limb positions (limb t at pos->prime[t]*N instead of t*N).
+// passes: for N > 4096 the transform is two kernels; bit 0 / bit 1 select them
+// (both by default; single passes exist so a benchmark can time each kernel).
 bool launch_ntt(hipStream_t st, const DevCtx& c, u64* dst, const u64* src, const LimbMap& lm, const LimbMap* pos,
-                u32 n_limbs, u32 n_polys, u64 poly_stride, bool inverse, const u64* scale);
+                u32 n_limbs, u32 n_polys, u64 poly_stride, bool inverse, const u64* scale, int passes = 3);
 
 // elementwise over n_limbs limbs of n words each (limb t uses lm.prime[t]);
 // scalar ops take the same scalar for every limb.

@@ -15,10 +15,28 @@
 //            the 16-word-strided accesses are conflict-free), and a last
 //            transpose so the global store is coalesced.
 //   inverse  the same two kernels mirrored (chunk first, strided last).
-// Inside a kernel values are kept lazily reduced (forward < 4q, inverse < 2q,
-// Harvey butterflies); the last kernel of a transform stores canonical
-// residues.  N <= 4096 uses one workgroup per limb with the limb in LDS.
+// N <= 4096 uses one workgroup per limb with the limb in LDS.
+//
+// Two arithmetic back ends share the index logic:
+//   ArithInt  64-bit integers, Harvey lazy butterflies (forward < 4q, inverse
+//             < 2q) with Shoup twiddles; any prime below 2^62.  About 30 VALU
+//             instructions per butterfly, which makes the chunk pass
+//             instruction-bound.
+//   ArithFp   for primes below 2^50.2: residues are carried as exact integers
+//             in FP64 (|x| < 2^53).  A twiddle product is y*w - rint(y*(w/q))*q
+//             evaluated exactly with one FMA for the low half of y*w and one
+//             for the subtraction (6 full-rate FP64 ops); sums are brought
+//             back to |x| <= q/2 every few stages with x - rint(x/q)*q.  All
+//             intermediate values are integers below 2^53, so no rounding
+//             ever happens and the final canonical residue is exact.
+// Between the two passes the buffer holds back-end specific words (lazily
+// reduced integers, or raw FP64 bits); the second pass stores canonical
+// residues.
+#include <vector>
+
 #include "ace_kernels.h"
+
+#pragma clang fp contract(off)
 
 namespace ace {
 
@@ -27,25 +45,188 @@ constexpr int kLogChunk = 12;
 
 __device__ __forceinline__ int lds_pos(int e) { return e + (e >> 4); }
 
-// forward butterfly, Harvey: x,y < 4q -> x' , y' < 4q
-__device__ __forceinline__ void ct_bfly(u64& x, u64& y, u64 w, u64 wp, u64 q, u64 q2) {
-  u64 a = csub(x, q2);
-  u64 t = shoup_lazy(y, w, wp, q);
-  x = a + t;
-  y = a - t + q2;
-}
-// inverse butterfly: x,y < 2q -> x', y' < 2q
-__device__ __forceinline__ void gs_bfly(u64& x, u64& y, u64 w, u64 wp, u64 q, u64 q2) {
-  u64 s = csub(x + y, q2);
-  u64 d = x - y + q2;
-  x = s;
-  y = shoup_lazy(d, w, wp, q);
-}
+// ---------------------------------------------------------------------------
+struct ArithInt {
+  typedef u64 T;
+  u64 q, q2;
+  const u64 *w, *wp;  // twiddle, Shoup companion
+  u64 sc, scp;        // inverse: final scale constant
+  __device__ __forceinline__ void init(const DevCtx& c, u32 pi, bool inverse, const u64* scale, u32 sidx) {
+    const DevPrime& P = c.primes[pi];
+    q = P.q;
+    q2 = q << 1;
+    w = (inverse ? c.irou : c.rou) + (u64)pi * c.N;
+    wp = (inverse ? c.irou_p : c.rou_p) + (u64)pi * c.N;
+    sc = P.ninv;
+    scp = P.ninv_p;
+    if (scale) { sc = scale[2 * sidx]; scp = scale[2 * sidx + 1]; }
+  }
+  struct TW { u64 w, wp; };
+  // NG consecutive twiddles starting at index ti0 (a multiple of NG): 16-byte loads
+  template <int NG>
+  __device__ __forceinline__ void load_tw(u32 ti0, TW* tw) const {
+    if (NG == 1) {
+      tw[0].w = w[ti0];
+      tw[0].wp = wp[ti0];
+    } else {
+      const ulonglong2* a = reinterpret_cast<const ulonglong2*>(w + ti0);
+      const ulonglong2* b = reinterpret_cast<const ulonglong2*>(wp + ti0);
+#pragma unroll
+      for (int k = 0; k < NG / 2; ++k) {
+        ulonglong2 x = a[k], y = b[k];
+        tw[2 * k].w = x.x; tw[2 * k + 1].w = x.y;
+        tw[2 * k].wp = y.x; tw[2 * k + 1].wp = y.y;
+      }
+    }
+  }
+  __device__ __forceinline__ T in_canon(u64 v) const { return v; }
+  __device__ __forceinline__ T in_mid(u64 v) const { return v; }
+  __device__ __forceinline__ u64 out_mid(T v) const { return v; }
+  __device__ __forceinline__ void reduce(T&) const {}
+  // forward, Harvey: x,y < 4q -> < 4q
+  __device__ __forceinline__ void ct(T& x, T& y, const TW& tw) const {
+    u64 a = csub(x, q2);
+    u64 t = shoup_lazy(y, tw.w, tw.wp, q);
+    x = a + t;
+    y = a - t + q2;
+  }
+  // inverse: x,y < 2q -> < 2q
+  __device__ __forceinline__ void gs(T& x, T& y, const TW& tw) const {
+    u64 s = csub(x + y, q2);
+    u64 d = x - y + q2;
+    x = s;
+    y = shoup_lazy(d, tw.w, tw.wp, q);
+  }
+  __device__ __forceinline__ u64 out_canon(T v) const { return csub(csub(v, q2), q); }
+  __device__ __forceinline__ u64 out_scaled(T v) const { return shoup_mul(v, sc, scp, q); }
+};
+
+struct ArithFp {
+  typedef double T;
+  double q, qinv;
+  const double* w;  // twiddles as exact FP64 integers
+  double sc, sci;
+  static constexpr double kMagic = 4503599627370496.0;  // 2^52
+  __device__ __forceinline__ void init(const DevCtx& c, u32 pi, bool inverse, const u64* scale, u32 sidx) {
+    const DevPrime& P = c.primes[pi];
+    q = (double)P.q;
+    qinv = 1.0 / q;
+    w = (inverse ? c.iroud : c.roud) + (u64)pi * c.N;
+    u64 s = scale ? scale[2 * sidx] : P.ninv;
+    sc = (double)s;
+    sci = sc / q;
+  }
+  struct TW { double w, wi; };
+  // NG consecutive twiddles from index ti0 (a multiple of NG); w/q is formed as
+  // w * (1/q): two roundings, relative error 2^-52, which only widens the
+  // quotient estimate (|product| <= (1/2 + 0.43 |y|/q) q), never the exactness
+  template <int NG>
+  __device__ __forceinline__ void load_tw(u32 ti0, TW* tw) const {
+    if (NG == 1) {
+      tw[0].w = w[ti0];
+    } else {
+      const double2* a = reinterpret_cast<const double2*>(w + ti0);
+#pragma unroll
+      for (int k = 0; k < NG / 2; ++k) {
+        double2 x = a[k];
+        tw[2 * k].w = x.x; tw[2 * k + 1].w = x.y;
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < NG; ++k) tw[k].wi = tw[k].w * qinv;
+  }
+  __device__ __forceinline__ T in_canon(u64 v) const {  // v < 2^52
+    return __longlong_as_double((long long)(v | 0x4330000000000000ull)) - kMagic;
+  }
+  __device__ __forceinline__ T in_mid(u64 v) const { return __longlong_as_double((long long)v); }
+  __device__ __forceinline__ u64 out_mid(T v) const { return (u64)__double_as_longlong(v); }
+  // x - rint(x/q)*q: |result| <= (1/2 + 2^-49) q, exact
+  __device__ __forceinline__ void reduce(T& x) const { x = __builtin_fma(-__builtin_rint(x * qinv), q, x); }
+  // y*w mod q as a signed integer of magnitude <= (1/2 + 0.43 |y|/q) q, exact
+  __device__ __forceinline__ double mulmod(double y, double ww, double wwi) const {
+    double c = __builtin_rint(y * wwi);
+    double h = y * ww;
+    double l = __builtin_fma(y, ww, -h);
+    double d = __builtin_fma(-c, q, h);
+    return d + l;
+  }
+  __device__ __forceinline__ void ct(T& x, T& y, const TW& tw) const {
+    double t = mulmod(y, tw.w, tw.wi);
+    y = x - t;
+    x = x + t;
+  }
+  __device__ __forceinline__ void gs(T& x, T& y, const TW& tw) const {
+    double d = x - y;
+    x = x + y;
+    y = mulmod(d, tw.w, tw.wi);
+  }
+  __device__ __forceinline__ u64 to_u64(double r) const {  // |r| <= q/2 (+)
+    r = r < 0.0 ? r + q : r;
+    return (u64)__double_as_longlong(r + kMagic) & 0x000FFFFFFFFFFFFFull;
+  }
+  __device__ __forceinline__ u64 out_canon(T v) const {
+    reduce(v);
+    return to_u64(v);
+  }
+  __device__ __forceinline__ u64 out_scaled(T v) const {
+    reduce(v);
+    double t = mulmod(v, sc, sci);
+    reduce(t);
+    return to_u64(t);
+  }
+};
 
 // ---------------------------------------------------------------------------
-// forward, strided pass: stages 0..LOGR-1
-// grid = (N/R/256, n_limbs, n_polys)
-template <int LOGR>
+// One radix-2 stage over a register file of R values.
+// forward stage K (0 = widest span): groups = 2^K, pairs (i, i + R/2^(K+1))
+template <class A, int R, int K>
+__device__ __forceinline__ void ct_stage(const A& ar, typename A::T* v, u32 ti0) {
+  constexpr int G = 1 << K, half = R >> (K + 1);
+  typename A::TW tw[G];
+  ar.template load_tw<G>(ti0, tw);
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+#pragma unroll
+    for (int j = 0; j < half; ++j) ar.ct(v[g * 2 * half + j], v[g * 2 * half + j + half], tw[g]);
+  }
+}
+// inverse stage K (0 = narrowest span): span = 2^K, groups = R/2^(K+1)
+template <class A, int R, int K>
+__device__ __forceinline__ void gs_stage(const A& ar, typename A::T* v, u32 ti0) {
+  constexpr int G = R >> (K + 1), span = 1 << K;
+  typename A::TW tw[G];
+  ar.template load_tw<G>(ti0, tw);
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+#pragma unroll
+    for (int j = 0; j < span; ++j) ar.gs(v[g * 2 * span + j], v[g * 2 * span + j + span], tw[g]);
+  }
+}
+template <class A, int R>
+__device__ __forceinline__ void reduce_all(const A& ar, typename A::T* v) {
+#pragma unroll
+  for (int r = 0; r < R; ++r) ar.reduce(v[r]);
+}
+
+// all LOGR stages of the strided passes (twiddle indices are wave-uniform)
+template <class A, int LOGR, int K = 0>
+__device__ __forceinline__ void fwd_strided_stages(const A& ar, typename A::T* v) {
+  if constexpr (K < LOGR) {
+    ct_stage<A, (1 << LOGR), K>(ar, v, 1u << K);
+    fwd_strided_stages<A, LOGR, K + 1>(ar, v);
+  }
+}
+template <class A, int LOGR, int K = 0>
+__device__ __forceinline__ void inv_strided_stages(const A& ar, typename A::T* v) {
+  if constexpr (K < LOGR) {
+    if ((K & 1) == 0) reduce_all<A, (1 << LOGR)>(ar, v);
+    gs_stage<A, (1 << LOGR), K>(ar, v, (1u << LOGR) >> (K + 1));
+    inv_strided_stages<A, LOGR, K + 1>(ar, v);
+  }
+}
+
+// forward, strided pass: stages 0..LOGR-1.  grid = (N/R/256, n_limbs, n_polys)
+template <class A, int LOGR>
 __global__ __launch_bounds__(256) void ntt_fwd_strided(DevCtx c, u64* __restrict__ dst, const u64* __restrict__ src,
                                                        LimbMap lm, LimbMap pos, u64 poly_stride) {
   constexpr int R = 1 << LOGR;
@@ -53,131 +234,100 @@ __global__ __launch_bounds__(256) void ntt_fwd_strided(DevCtx c, u64* __restrict
   const u32 limb = blockIdx.y, pi = lm.prime[limb];
   const u64 rs = c.N >> LOGR;  // row stride
   const u64 off = blockIdx.z * poly_stride + (u64)pos.prime[limb] * c.N + col;
-  const u64 q = c.primes[pi].q, q2 = q << 1;
-  const u64* w = c.rou + (u64)pi * c.N;
-  const u64* wp = c.rou_p + (u64)pi * c.N;
-  u64 v[R];
+  A ar;
+  ar.init(c, pi, false, nullptr, 0);
+  typename A::T v[R];
 #pragma unroll
-  for (int r = 0; r < R; ++r) v[r] = src[off + r * rs];
+  for (int r = 0; r < R; ++r) v[r] = ar.in_canon(src[off + r * rs]);
+  if (LOGR > 4) reduce_all<A, R>(ar, v);
+  fwd_strided_stages<A, LOGR>(ar, v);
 #pragma unroll
-  for (int ls = 0; ls < LOGR; ++ls) {
-    const int half = R >> (ls + 1);
-#pragma unroll
-    for (int g = 0; g < (1 << ls); ++g) {
-      u64 W = w[(1 << ls) + g], Wp = wp[(1 << ls) + g];
-#pragma unroll
-      for (int j = 0; j < half; ++j) ct_bfly(v[g * 2 * half + j], v[g * 2 * half + j + half], W, Wp, q, q2);
-    }
-  }
-#pragma unroll
-  for (int r = 0; r < R; ++r) dst[off + r * rs] = v[r];
+  for (int r = 0; r < R; ++r) dst[off + r * rs] = ar.out_mid(v[r]);
 }
 
-// forward, chunk pass: stages logr..logN-1 on 4096 contiguous words.
-// grid = (N/4096, n_limbs, n_polys); in place on `data`, or src -> data when
-// logr == 0 is impossible here (N > 4096 always has a strided pass first).
-__global__ __launch_bounds__(256) void ntt_fwd_chunk(DevCtx c, u64* __restrict__ data, LimbMap lm, LimbMap pos, u64 poly_stride,
-                                                     u32 logr) {
-  __shared__ u64 lds[kChunk + kChunk / 16];
+// forward, chunk pass: stages logr..logN-1 on 4096 contiguous words, in place.
+// grid = (N/4096, n_limbs, n_polys)
+template <class A>
+__global__ __launch_bounds__(256) void ntt_fwd_chunk(DevCtx c, u64* __restrict__ data, LimbMap lm, LimbMap pos,
+                                                     u64 poly_stride, u32 logr) {
+  typedef typename A::T T;
+  __shared__ T lds[kChunk + kChunk / 16];
   const int t = threadIdx.x;
   const u32 chunk = blockIdx.x, limb = blockIdx.y, pi = lm.prime[limb];
   u64* base = data + blockIdx.z * poly_stride + (u64)pos.prime[limb] * c.N + (u64)chunk * kChunk;
-  const u64 q = c.primes[pi].q, q2 = q << 1;
-  const u64* w = c.rou + (u64)pi * c.N;
-  const u64* wp = c.rou_p + (u64)pi * c.N;
-  u64 v[16];
-  // round A: element e = t + 256 r, local stages 0..3; twiddles are uniform
+  A ar;
+  ar.init(c, pi, false, nullptr, 0);
+  T v[16];
+  // twiddle index of local stage ls, local group 0 of this chunk: m + (chunk << ls)
+  const u32 m0 = 1u << logr;
+  // round A: element e = t + 256 r, local stages 0..3; twiddles are wave-uniform
 #pragma unroll
-  for (int r = 0; r < 16; ++r) v[r] = base[t + 256 * r];
-#pragma unroll
-  for (int ls = 0; ls < 4; ++ls) {
-    const int half = 8 >> ls;
-    const u32 m = 1u << (logr + ls);
-#pragma unroll
-    for (int g = 0; g < (1 << ls); ++g) {
-      u32 ti = m + (chunk << ls) + g;
-      u64 W = w[ti], Wp = wp[ti];
-#pragma unroll
-      for (int j = 0; j < half; ++j) ct_bfly(v[g * 2 * half + j], v[g * 2 * half + j + half], W, Wp, q, q2);
-    }
-  }
+  for (int r = 0; r < 16; ++r) v[r] = ar.in_mid(base[t + 256 * r]);
+  reduce_all<A, 16>(ar, v);
+  ct_stage<A, 16, 0>(ar, v, (m0 << 0) + (chunk << 0));
+  ct_stage<A, 16, 1>(ar, v, (m0 << 1) + (chunk << 1));
+  ct_stage<A, 16, 2>(ar, v, (m0 << 2) + (chunk << 2));
+  ct_stage<A, 16, 3>(ar, v, (m0 << 3) + (chunk << 3));
 #pragma unroll
   for (int r = 0; r < 16; ++r) lds[lds_pos(t + 256 * r)] = v[r];
   __syncthreads();
-  // round B: e = hi*256 + r*16 + lo, local stages 4..7
+  // round B: e = hi*256 + r*16 + lo, local stages 4..7: local group = (hi << (ls-4)) + g
   const int hi = t >> 4, lo = t & 15;
 #pragma unroll
   for (int r = 0; r < 16; ++r) v[r] = lds[lds_pos(hi * 256 + r * 16 + lo)];
-#pragma unroll
-  for (int ls = 4; ls < 8; ++ls) {
-    const int half = 8 >> (ls - 4);
-    const u32 m = 1u << (logr + ls);
-#pragma unroll
-    for (int g = 0; g < (1 << (ls - 4)); ++g) {
-      u32 ti = m + (chunk << ls) + (hi << (ls - 4)) + g;
-      u64 W = w[ti], Wp = wp[ti];
-#pragma unroll
-      for (int j = 0; j < half; ++j) ct_bfly(v[g * 2 * half + j], v[g * 2 * half + j + half], W, Wp, q, q2);
-    }
-  }
+  reduce_all<A, 16>(ar, v);
+  ct_stage<A, 16, 0>(ar, v, (m0 << 4) + (chunk << 4) + (hi << 0));
+  ct_stage<A, 16, 1>(ar, v, (m0 << 5) + (chunk << 5) + (hi << 1));
+  ct_stage<A, 16, 2>(ar, v, (m0 << 6) + (chunk << 6) + (hi << 2));
+  ct_stage<A, 16, 3>(ar, v, (m0 << 7) + (chunk << 7) + (hi << 3));
 #pragma unroll
   for (int r = 0; r < 16; ++r) lds[lds_pos(hi * 256 + r * 16 + lo)] = v[r];
   __syncthreads();
-  // round C: e = t*16 + r, local stages 8..11
+  // round C: e = t*16 + r, local stages 8..11: local group = (t << (ls-8)) + g
 #pragma unroll
   for (int r = 0; r < 16; ++r) v[r] = lds[lds_pos(t * 16 + r)];
+  reduce_all<A, 16>(ar, v);
+  ct_stage<A, 16, 0>(ar, v, (m0 << 8) + (chunk << 8) + (t << 0));
+  ct_stage<A, 16, 1>(ar, v, (m0 << 9) + (chunk << 9) + (t << 1));
+  ct_stage<A, 16, 2>(ar, v, (m0 << 10) + (chunk << 10) + (t << 2));
+  ct_stage<A, 16, 3>(ar, v, (m0 << 11) + (chunk << 11) + (t << 3));
+  u64* ldsu = reinterpret_cast<u64*>(lds);
 #pragma unroll
-  for (int ls = 8; ls < 12; ++ls) {
-    const int half = 8 >> (ls - 8);
-    const u32 m = 1u << (logr + ls);
-#pragma unroll
-    for (int g = 0; g < (1 << (ls - 8)); ++g) {
-      u32 ti = m + (chunk << ls) + (t << (ls - 8)) + g;
-      u64 W = w[ti], Wp = wp[ti];
-#pragma unroll
-      for (int j = 0; j < half; ++j) ct_bfly(v[g * 2 * half + j], v[g * 2 * half + j + half], W, Wp, q, q2);
-    }
-  }
-#pragma unroll
-  for (int r = 0; r < 16; ++r) lds[lds_pos(t * 16 + r)] = csub(csub(v[r], q2), q);
+  for (int r = 0; r < 16; ++r) ldsu[lds_pos(t * 16 + r)] = ar.out_canon(v[r]);
   __syncthreads();
 #pragma unroll
-  for (int r = 0; r < 16; ++r) base[t + 256 * r] = lds[lds_pos(t + 256 * r)];
+  for (int r = 0; r < 16; ++r) base[t + 256 * r] = ldsu[lds_pos(t + 256 * r)];
 }
 
 // ---------------------------------------------------------------------------
 // inverse, chunk pass: spans 1..2048 on 4096 contiguous words; src -> dst.
 // Nothing is scaled here: 1/N (times an optional per-limb constant) is applied
-// by the strided pass that always follows.
+// by the strided pass that always follows.  At span 2^u the stage has
+// m = N >> (u+1) groups and element j belongs to group j >> (u+1).
+template <class A>
 __global__ __launch_bounds__(256) void ntt_inv_chunk(DevCtx c, u64* __restrict__ dst, const u64* __restrict__ src,
                                                      LimbMap lm, LimbMap pos, u64 poly_stride) {
-  __shared__ u64 lds[kChunk + kChunk / 16];
+  typedef typename A::T T;
+  __shared__ T lds[kChunk + kChunk / 16];
   const int t = threadIdx.x;
   const u32 chunk = blockIdx.x, limb = blockIdx.y, pi = lm.prime[limb];
   const u64 off = blockIdx.z * poly_stride + (u64)pos.prime[limb] * c.N + (u64)chunk * kChunk;
-  const u64 q = c.primes[pi].q, q2 = q << 1;
-  const u64* w = c.irou + (u64)pi * c.N;
-  const u64* wp = c.irou_p + (u64)pi * c.N;
-  const u32 logN = c.logN;
-  u64 v[16];
+  A ar;
+  ar.init(c, pi, true, nullptr, 0);
+  const u32 mh = c.N >> 1;  // groups at span 1
+  T v[16];
 #pragma unroll
-  for (int r = 0; r < 16; ++r) lds[lds_pos(t + 256 * r)] = src[off + t + 256 * r];
+  for (int r = 0; r < 16; ++r) lds[lds_pos(t + 256 * r)] = ar.in_canon(src[off + t + 256 * r]);
   __syncthreads();
-  // round C': e = t*16 + r, spans 2^u, u = 0..3
+  // round C': e = t*16 + r, u = 0..3
 #pragma unroll
   for (int r = 0; r < 16; ++r) v[r] = lds[lds_pos(t * 16 + r)];
-#pragma unroll
-  for (int u = 0; u < 4; ++u) {
-    const int span = 1 << u;
-    const u32 m = 1u << (logN - u - 1);
-#pragma unroll
-    for (int g = 0; g < (8 >> u); ++g) {
-      u32 ti = m + (chunk << (11 - u)) + (t << (3 - u)) + g;
-      u64 W = w[ti], Wp = wp[ti];
-#pragma unroll
-      for (int j = 0; j < span; ++j) gs_bfly(v[g * 2 * span + j], v[g * 2 * span + j + span], W, Wp, q, q2);
-    }
-  }
+  reduce_all<A, 16>(ar, v);
+  gs_stage<A, 16, 0>(ar, v, (mh >> 0) + (chunk << 11) + (t << 3));
+  gs_stage<A, 16, 1>(ar, v, (mh >> 1) + (chunk << 10) + (t << 2));
+  reduce_all<A, 16>(ar, v);
+  gs_stage<A, 16, 2>(ar, v, (mh >> 2) + (chunk << 9) + (t << 1));
+  gs_stage<A, 16, 3>(ar, v, (mh >> 3) + (chunk << 8) + (t << 0));
 #pragma unroll
   for (int r = 0; r < 16; ++r) lds[lds_pos(t * 16 + r)] = v[r];
   __syncthreads();
@@ -185,149 +335,116 @@ __global__ __launch_bounds__(256) void ntt_inv_chunk(DevCtx c, u64* __restrict__
   const int hi = t >> 4, lo = t & 15;
 #pragma unroll
   for (int r = 0; r < 16; ++r) v[r] = lds[lds_pos(hi * 256 + r * 16 + lo)];
-#pragma unroll
-  for (int u = 4; u < 8; ++u) {
-    const int span = 1 << (u - 4);
-    const u32 m = 1u << (logN - u - 1);
-#pragma unroll
-    for (int g = 0; g < (8 >> (u - 4)); ++g) {
-      u32 ti = m + (chunk << (11 - u)) + (hi << (7 - u)) + g;
-      u64 W = w[ti], Wp = wp[ti];
-#pragma unroll
-      for (int j = 0; j < span; ++j) gs_bfly(v[g * 2 * span + j], v[g * 2 * span + j + span], W, Wp, q, q2);
-    }
-  }
+  reduce_all<A, 16>(ar, v);
+  gs_stage<A, 16, 0>(ar, v, (mh >> 4) + (chunk << 7) + (hi << 3));
+  gs_stage<A, 16, 1>(ar, v, (mh >> 5) + (chunk << 6) + (hi << 2));
+  reduce_all<A, 16>(ar, v);
+  gs_stage<A, 16, 2>(ar, v, (mh >> 6) + (chunk << 5) + (hi << 1));
+  gs_stage<A, 16, 3>(ar, v, (mh >> 7) + (chunk << 4) + (hi << 0));
 #pragma unroll
   for (int r = 0; r < 16; ++r) lds[lds_pos(hi * 256 + r * 16 + lo)] = v[r];
   __syncthreads();
-  // round A': e = t + 256 r, u = 8..11; twiddles uniform
+  // round A': e = t + 256 r, u = 8..11; twiddles wave-uniform
 #pragma unroll
   for (int r = 0; r < 16; ++r) v[r] = lds[lds_pos(t + 256 * r)];
+  reduce_all<A, 16>(ar, v);
+  gs_stage<A, 16, 0>(ar, v, (mh >> 8) + (chunk << 3));
+  gs_stage<A, 16, 1>(ar, v, (mh >> 9) + (chunk << 2));
+  reduce_all<A, 16>(ar, v);
+  gs_stage<A, 16, 2>(ar, v, (mh >> 10) + (chunk << 1));
+  gs_stage<A, 16, 3>(ar, v, (mh >> 11) + (chunk << 0));
 #pragma unroll
-  for (int u = 8; u < 12; ++u) {
-    const int span = 1 << (u - 8);
-    const u32 m = 1u << (logN - u - 1);
-#pragma unroll
-    for (int g = 0; g < (8 >> (u - 8)); ++g) {
-      u32 ti = m + (chunk << (11 - u)) + g;
-      u64 W = w[ti], Wp = wp[ti];
-#pragma unroll
-      for (int j = 0; j < span; ++j) gs_bfly(v[g * 2 * span + j], v[g * 2 * span + j + span], W, Wp, q, q2);
-    }
-  }
-#pragma unroll
-  for (int r = 0; r < 16; ++r) dst[off + t + 256 * r] = v[r];
+  for (int r = 0; r < 16; ++r) dst[off + t + 256 * r] = ar.out_mid(v[r]);
 }
 
-// inverse, strided pass: spans 4096..N/2, then scale every word by
-// scale[limb] (default 1/N) and store canonical residues.  In place.
-// scale: nullptr or 2*n_limbs words (constant, Shoup companion) per limb.
-template <int LOGR>
-__global__ __launch_bounds__(256) void ntt_inv_strided(DevCtx c, u64* __restrict__ data, LimbMap lm, LimbMap pos, u64 poly_stride,
+// inverse, strided pass: spans 4096..N/2, then scale every word by the limb's
+// constant (default 1/N) and store canonical residues.  In place.
+// scale: nullptr, or (constant, Shoup companion) pairs indexed by sidx.prime[limb].
+template <class A, int LOGR>
+__global__ __launch_bounds__(256) void ntt_inv_strided(DevCtx c, u64* __restrict__ data, LimbMap lm, LimbMap pos,
+                                                       LimbMap sidx, u64 poly_stride,
                                                        const u64* __restrict__ scale) {
   constexpr int R = 1 << LOGR;
   const u32 col = blockIdx.x * 256 + threadIdx.x;
   const u32 limb = blockIdx.y, pi = lm.prime[limb];
   const u64 rs = c.N >> LOGR;
   const u64 off = blockIdx.z * poly_stride + (u64)pos.prime[limb] * c.N + col;
-  const DevPrime P = c.primes[pi];
-  const u64 q = P.q, q2 = q << 1;
-  const u64* w = c.irou + (u64)pi * c.N;
-  const u64* wp = c.irou_p + (u64)pi * c.N;
-  u64 v[R];
+  A ar;
+  ar.init(c, pi, true, scale, sidx.prime[limb]);
+  typename A::T v[R];
 #pragma unroll
-  for (int r = 0; r < R; ++r) v[r] = data[off + r * rs];
+  for (int r = 0; r < R; ++r) v[r] = ar.in_mid(data[off + r * rs]);
+  inv_strided_stages<A, LOGR>(ar, v);
 #pragma unroll
-  for (int u = 0; u < LOGR; ++u) {  // span 2^u rows, m = R >> (u+1) groups
-    const int span = 1 << u;
-#pragma unroll
-    for (int g = 0; g < (R >> (u + 1)); ++g) {
-      u64 W = w[(R >> (u + 1)) + g], Wp = wp[(R >> (u + 1)) + g];
-#pragma unroll
-      for (int j = 0; j < span; ++j) gs_bfly(v[g * 2 * span + j], v[g * 2 * span + j + span], W, Wp, q, q2);
-    }
-  }
-  u64 s = P.ninv, sp = P.ninv_p;
-  if (scale) { s = scale[2 * limb]; sp = scale[2 * limb + 1]; }
-#pragma unroll
-  for (int r = 0; r < R; ++r) data[off + r * rs] = shoup_mul(v[r], s, sp, q);
+  for (int r = 0; r < R; ++r) data[off + r * rs] = ar.out_scaled(v[r]);
 }
 
 // ---------------------------------------------------------------------------
 // N <= 4096: one workgroup per limb, the limb in LDS, one butterfly per
-// thread per step.  grid = (1, n_limbs, n_polys)
+// thread per step (integer back end).  grid = (1, n_limbs, n_polys)
 __global__ __launch_bounds__(256) void ntt_small(DevCtx c, u64* __restrict__ dst, const u64* __restrict__ src,
                                                  LimbMap lm, LimbMap pos, u64 poly_stride, int inverse,
                                                  const u64* __restrict__ scale) {
   __shared__ u64 a[kChunk];
   const u32 N = c.N, logN = c.logN, limb = blockIdx.y, pi = lm.prime[limb];
   const u64 off = blockIdx.z * poly_stride + (u64)pos.prime[limb] * N;
-  const DevPrime P = c.primes[pi];
-  const u64 q = P.q, q2 = q << 1;
+  ArithInt ar;
+  ar.init(c, pi, inverse != 0, scale, limb);
   for (u32 i = threadIdx.x; i < N; i += 256) a[i] = src[off + i];
   __syncthreads();
   if (!inverse) {
-    const u64* w = c.rou + (u64)pi * N;
-    const u64* wp = c.rou_p + (u64)pi * N;
     for (u32 s = 0; s < logN; ++s) {
       const u32 tspan = N >> (s + 1);
       for (u32 b = threadIdx.x; b < (N >> 1); b += 256) {
         u32 g = b / tspan, j = b - g * tspan, i0 = g * 2 * tspan + j;
-        ct_bfly(a[i0], a[i0 + tspan], w[(1u << s) + g], wp[(1u << s) + g], q, q2);
+        ArithInt::TW tw;
+        ar.load_tw<1>((1u << s) + g, &tw);
+        ar.ct(a[i0], a[i0 + tspan], tw);
       }
       __syncthreads();
     }
-    for (u32 i = threadIdx.x; i < N; i += 256) dst[off + i] = csub(csub(a[i], q2), q);
+    for (u32 i = threadIdx.x; i < N; i += 256) dst[off + i] = ar.out_canon(a[i]);
   } else {
-    const u64* w = c.irou + (u64)pi * N;
-    const u64* wp = c.irou_p + (u64)pi * N;
     for (u32 u = 0; u < logN; ++u) {
       const u32 span = 1u << u, m = N >> (u + 1);
       for (u32 b = threadIdx.x; b < (N >> 1); b += 256) {
         u32 g = b >> u, j = b & (span - 1), i0 = g * 2 * span + j;
-        gs_bfly(a[i0], a[i0 + span], w[m + g], wp[m + g], q, q2);
+        ArithInt::TW tw;
+        ar.load_tw<1>(m + g, &tw);
+        ar.gs(a[i0], a[i0 + span], tw);
       }
       __syncthreads();
     }
-    u64 s = P.ninv, sp = P.ninv_p;
-    if (scale) { s = scale[2 * limb]; sp = scale[2 * limb + 1]; }
-    for (u32 i = threadIdx.x; i < N; i += 256) dst[off + i] = shoup_mul(a[i], s, sp, q);
+    for (u32 i = threadIdx.x; i < N; i += 256) dst[off + i] = ar.out_scaled(a[i]);
   }
 }
 
 // ---------------------------------------------------------------------------
-template <int LOGR>
-static void fwd_large(hipStream_t st, const DevCtx& c, u64* dst, const u64* src, const LimbMap& lm, const LimbMap& pos,
-                      u32 n_limbs, u32 n_polys, u64 poly_stride) {
-  dim3 g1((c.N >> LOGR) / 256, n_limbs, n_polys), g2(c.N / kChunk, n_limbs, n_polys);
-  hipLaunchKernelGGL(ntt_fwd_strided<LOGR>, g1, dim3(256), 0, st, c, dst, src, lm, pos, poly_stride);
-  hipLaunchKernelGGL(ntt_fwd_chunk, g2, dim3(256), 0, st, c, dst, lm, pos, poly_stride, (u32)LOGR);
-}
-template <int LOGR>
-static void inv_large(hipStream_t st, const DevCtx& c, u64* dst, const u64* src, const LimbMap& lm, const LimbMap& pos,
-                      u32 n_limbs, u32 n_polys, u64 poly_stride, const u64* scale) {
-  dim3 g1(c.N / kChunk, n_limbs, n_polys), g2((c.N >> LOGR) / 256, n_limbs, n_polys);
-  hipLaunchKernelGGL(ntt_inv_chunk, g1, dim3(256), 0, st, c, dst, src, lm, pos, poly_stride);
-  hipLaunchKernelGGL(ntt_inv_strided<LOGR>, g2, dim3(256), 0, st, c, dst, lm, pos, poly_stride, scale);
+template <class A, int LOGR>
+static void run_large(hipStream_t st, const DevCtx& c, u64* dst, const u64* src, const LimbMap& lm, const LimbMap& pos,
+                      const LimbMap& sidx, u32 n_limbs, u32 n_polys, u64 poly_stride, bool inverse,
+                      const u64* scale, int passes) {
+  dim3 gs((c.N >> LOGR) / 256, n_limbs, n_polys), gc(c.N / kChunk, n_limbs, n_polys);
+  if (!inverse) {
+    if (passes & 1)
+      hipLaunchKernelGGL((ntt_fwd_strided<A, LOGR>), gs, dim3(256), 0, st, c, dst, src, lm, pos, poly_stride);
+    if (passes & 2)
+      hipLaunchKernelGGL((ntt_fwd_chunk<A>), gc, dim3(256), 0, st, c, dst, lm, pos, poly_stride, (u32)LOGR);
+  } else {
+    if (passes & 1) hipLaunchKernelGGL((ntt_inv_chunk<A>), gc, dim3(256), 0, st, c, dst, src, lm, pos, poly_stride);
+    if (passes & 2)
+      hipLaunchKernelGGL((ntt_inv_strided<A, LOGR>), gs, dim3(256), 0, st, c, dst, lm, pos, sidx, poly_stride, scale);
+  }
 }
 
-bool launch_ntt(hipStream_t st, const DevCtx& c, u64* dst, const u64* src, const LimbMap& lm, const LimbMap* pos_in,
-                u32 n_limbs, u32 n_polys, u64 poly_stride, bool inverse, const u64* scale) {
-  if (n_limbs == 0 || n_polys == 0) return true;
-  LimbMap pos{};
-  if (pos_in) pos = *pos_in;
-  else
-    for (u32 t = 0; t < n_limbs; ++t) pos.prime[t] = (uint8_t)t;
-  if (c.logN <= kLogChunk) {
-    hipLaunchKernelGGL(ntt_small, dim3(1, n_limbs, n_polys), dim3(256), 0, st, c, dst, src, lm, pos,
-                       poly_stride, inverse ? 1 : 0, scale);
-    return true;
-  }
+template <class A>
+static bool run_large_dispatch(hipStream_t st, const DevCtx& c, u64* dst, const u64* src, const LimbMap& lm,
+                               const LimbMap& pos, const LimbMap& sidx, u32 n_limbs, u32 n_polys, u64 poly_stride,
+                               bool inverse, const u64* scale, int passes) {
   switch (c.logN - kLogChunk) {
-#define ACE_NTT_CASE(LR)                                                                  \
-  case LR:                                                                                \
-    if (inverse) inv_large<LR>(st, c, dst, src, lm, pos, n_limbs, n_polys, poly_stride, scale); \
-    else         fwd_large<LR>(st, c, dst, src, lm, pos, n_limbs, n_polys, poly_stride);        \
+#define ACE_NTT_CASE(LR)                                                                                         \
+  case LR:                                                                                                       \
+    run_large<A, LR>(st, c, dst, src, lm, pos, sidx, n_limbs, n_polys, poly_stride, inverse, scale, passes);      \
     return true;
     ACE_NTT_CASE(1)
     ACE_NTT_CASE(2)
@@ -338,6 +455,39 @@ bool launch_ntt(hipStream_t st, const DevCtx& c, u64* dst, const u64* src, const
     default:
       return false;  // ring degree above 2^17 not supported
   }
+}
+
+bool launch_ntt(hipStream_t st, const DevCtx& c, u64* dst, const u64* src, const LimbMap& lm, const LimbMap* pos_in,
+                u32 n_limbs, u32 n_polys, u64 poly_stride, bool inverse, const u64* scale, int passes) {
+  if (n_limbs == 0 || n_polys == 0) return true;
+  LimbMap pos{};
+  if (pos_in) pos = *pos_in;
+  else
+    for (u32 t = 0; t < n_limbs; ++t) pos.prime[t] = (uint8_t)t;
+  if (c.logN <= kLogChunk) {
+    hipLaunchKernelGGL(ntt_small, dim3(1, n_limbs, n_polys), dim3(256), 0, st, c, dst, src, lm, pos, poly_stride,
+                       inverse ? 1 : 0, scale);
+    return true;
+  }
+  if (c.logN - kLogChunk > 5) return false;
+  // split the limbs by arithmetic back end: one launch per pass and group
+  LimbMap lm_g[2]{}, pos_g[2]{}, sidx_g[2]{};
+  u32 cnt[2] = {0, 0};
+  for (u32 t = 0; t < n_limbs; ++t) {
+    int gsel = c.fp_ok[lm.prime[t]] ? 1 : 0;
+    lm_g[gsel].prime[cnt[gsel]] = lm.prime[t];
+    pos_g[gsel].prime[cnt[gsel]] = pos.prime[t];
+    sidx_g[gsel].prime[cnt[gsel]] = (uint8_t)t;
+    ++cnt[gsel];
+  }
+  bool ok = true;
+  if (cnt[0])
+    ok &= run_large_dispatch<ArithInt>(st, c, dst, src, lm_g[0], pos_g[0], sidx_g[0], cnt[0], n_polys, poly_stride,
+                                       inverse, scale, passes);
+  if (cnt[1])
+    ok &= run_large_dispatch<ArithFp>(st, c, dst, src, lm_g[1], pos_g[1], sidx_g[1], cnt[1], n_polys, poly_stride,
+                                      inverse, scale, passes);
+  return ok;
 }
 
 }  // namespace ace

@@ -1,0 +1,191 @@
+#!/usr/bin/env python3
+"""Benchmark of the CKKS polynomial hot path on one MI355X.
+
+Headline workload (the batched RNS NTT configuration): 32 polynomials x 24
+limbs of 50-bit primes at N = 2^16, uint64 coefficients uniform mod q_i from a
+seeded generator, already resident in HBM; one step = forward NTT of the whole
+batch followed by the inverse NTT (a round trip).  `value` is algorithmic
+GB/s: 16 bytes per coefficient per transform (one read + one write of every
+limb) x 2 transforms / step time.
+
+The same line also reports, as extra fields, HMult+relinearise+rescale pairs/s
+(L=24, k=7 special primes, dnum=3) and hoisted rotations/s, the per-kernel
+roofline of the dominant NTT kernel measured with HIP events on the library's
+stream, and the CPU oracle timed on this host for the same workload.
+
+Prints exactly one JSON line on stdout.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "ace-compiler_amd"))
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
+N, LIMBS, POLYS = 65536, 24, 32
+CFG = (N, LIMBS, 50, 50, 3)
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def time_region(g, fn, reps):
+    """Average milliseconds per call of fn over reps calls, by HIP events on the library's stream."""
+    g.sync()
+    g.timer_start()
+    for _ in range(reps):
+        fn()
+    return g.timer_stop_ms() / reps
+
+
+def cpu_baseline(x_host, idx, budget_s):
+    """The oracle's NTT round trip on a bounded sample of the same batch (one thread)."""
+    from oracle_lib import Oracle
+
+    o = Oracle(*CFG)
+    per_poly = LIMBS * N
+    done, t0 = 0, time.perf_counter()
+    while done < POLYS:
+        s = slice(done * per_poly, (done + 1) * per_poly)
+        y = o.ntt(x_host[s], idx)
+        z = o.intt(y, idx)
+        assert (z == x_host[s]).all()
+        done += 1
+        if time.perf_counter() - t0 > budget_s:
+            break
+    dt = time.perf_counter() - t0
+    o.close()
+    gbs = done * per_poly * 16 * 2 / dt / 1e9
+    return {"value": round(gbs, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": "%d of %d polynomials (x%d limbs, forward+inverse), %.1f s, single thread, gcc -O3" % (
+                done, POLYS, LIMBS, dt)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="time budget of the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the key-switch / rotation measurements")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU; this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+
+    import acefhe
+    import seeded
+
+    g = acefhe.Context(*CFG)
+    if not g.has_device:
+        log("no GPU visible: " + g.err())
+        sys.exit(1)
+    assert (g.L, g.K, g.part_size) == (24, 7, 8)
+    idx = list(range(LIMBS))
+    per_poly = LIMBS * N
+    log("generating %d x %d limbs of seeded input" % (POLYS, LIMBS))
+    x_host = np.concatenate([seeded.uniform_poly(1000 + p, g.primes[:LIMBS], N) for p in range(POLYS)])
+    x = g.upload(x_host)
+
+    def step():
+        g.ntt(x, x, idx, n_polys=POLYS, poly_stride_limbs=LIMBS)
+        g.intt(x, x, idx, n_polys=POLYS, poly_stride_limbs=LIMBS)
+
+    for _ in range(args.warmup):
+        step()
+    g.sync()
+    t0 = time.perf_counter()
+    g.timer_start()
+    for _ in range(args.steps):
+        step()
+    ev_ms = g.timer_stop_ms()
+    g.sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ms_per_step = wall_ms / args.steps
+    assert (x.get() == x_host).all(), "round trip did not return the input"
+    step_bytes = POLYS * per_poly * 16 * 2
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+
+    # per-kernel timing of the four NTT kernels (each reads and writes every coefficient once)
+    kern = {}
+    scratch = g.alloc(POLYS * per_poly)
+    pass_bytes = POLYS * per_poly * 16
+    for name, inv, which in (("ntt_fwd_strided", 0, 1), ("ntt_fwd_chunk", 0, 2), ("ntt_inv_chunk", 1, 1),
+                             ("ntt_inv_strided", 1, 2)):
+        src = x if which == 1 else scratch
+        f = lambda: g.ntt_pass(scratch, src, idx, POLYS, LIMBS, inv, which)
+        f()
+        ms = time_region(g, f, 10)
+        kern[name] = {"ms": round(ms, 4), "GB/s": round(pass_bytes / (ms * 1e-3) / 1e9, 1)}
+    dom = max(kern, key=lambda k: kern[k]["ms"])
+    roofline = {"bound": "hbm", "kernel": dom, "achieved": kern[dom]["GB/s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(kern[dom]["GB/s"] / HBM_PEAK_GBS, 4), "traffic": None,
+                "bytes_per_launch": pass_bytes, "all_ntt_kernels": kern}
+    scratch.free()
+
+    extra = {}
+    if not args.no_extra:
+        level, T = g.L, g.L + g.K
+        kwords = 2 * g.parts * T * N
+        log("key-switch leg: 16 ciphertext pairs, one relinearisation key")
+        swk = g.upload(np.concatenate([seeded.uniform_poly(2000 + i, g.primes, N) for i in range(2 * g.parts)]))
+        cts = [g.upload(seeded.uniform_poly(3000 + i, g.primes[:level], N)) for i in range(4)]
+        r0, r1 = g.alloc((level - 1) * N), g.alloc((level - 1) * N)
+        pairs = 16
+
+        def hmult_batch():
+            for p in range(pairs):
+                g.mul_relin_rescale(r0, r1, cts[0], cts[1], cts[2], cts[3], swk, level)
+
+        hmult_batch()
+        ms = time_region(g, hmult_batch, 3)
+        extra["keyswitch_ops_per_s"] = round(pairs / (ms * 1e-3), 1)
+        extra["hmult_relin_rescale_ms"] = round(ms / pairs, 4)
+        # 172 MB compulsory traffic per op (96 input + 186 key + 46 output limbs of 512 KiB)
+        extra["keyswitch_hbm_frac"] = round(328 * N * 8 * pairs / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+
+        nrot = 32
+        log("rotation leg: %d rotations of one ciphertext, hoisted ModUp" % nrot)
+        rots = [1 << i for i in range(15)] + [-1] + [int(v) for v in 1 + seeded.splitmix64(7, 16) % np.uint64(N // 2 - 1)]
+        keys, orders = [], []
+        for i, r in enumerate(rots):
+            kbuf = g.alloc(kwords)
+            # distinct keys derived on the device from the seeded one: key_i = key_0 + (i+1) per limb
+            for d in range(2 * g.parts):
+                for t in range(T):
+                    off = (d * T + t) * N
+                    g.hw("modadd_scalar", kbuf.view(off, N), swk.view(off, N), i + 1, t)
+            keys.append(kbuf)
+            orders.append(g.automorphism_order(g.find_automorphism_index(r), True))
+        s0, s1 = g.alloc(nrot * level * N), g.alloc(nrot * level * N)
+        f = lambda: g.rotate_batch(s0, s1, cts[0], cts[1], keys, orders, level)
+        f()
+        ms = time_region(g, f, 3)
+        extra["rotations_per_s"] = round(nrot / (ms * 1e-3), 1)
+        extra["rotate_batch_ms"] = round(ms, 3)
+        extra["rotation_hbm_frac"] = round(327 * N * 8 * nrot / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+
+    cpu = cpu_baseline(x_host, idx, args.cpu_seconds)
+
+    out = {
+        "metric": "ntt_roundtrip_algorithmic_bandwidth", "value": round(value, 2), "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u64", "data": "synthetic",
+        "config": {"workload": "batched RNS NTT+INTT round trip, 32 polys x 24 limbs (50-bit primes), N=65536",
+                   "bytes_per_step": step_bytes, "hbm_frac": round(value / HBM_PEAK_GBS, 4),
+                   "event_ms_per_step": round(ev_ms / args.steps, 4)},
+        "roofline": roofline, "cpu_baseline": cpu, "extra": extra,
+    }
+    print(json.dumps(out))
+    g.close()
+
+
+if __name__ == "__main__":
+    main()

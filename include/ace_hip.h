@@ -102,6 +102,12 @@ int ace_ntt(ace_ctx* ctx, int64_t* dst, const int64_t* src, const int32_t* prime
 int ace_intt(ace_ctx* ctx, int64_t* dst, const int64_t* src, const int32_t* prime_idx,
              size_t n_limbs, size_t n_polys, size_t poly_stride_limbs);
 
+/* One of the two kernels a transform consists of when degree > 4096 (pass 1 then
+ * pass 2 equals ace_ntt / ace_intt).  For profiling each kernel on its own; the
+ * intermediate buffer holds lazily reduced values. */
+int ace_ntt_pass(ace_ctx* ctx, int64_t* dst, const int64_t* src, const int32_t* prime_idx,
+                 size_t n_limbs, size_t n_polys, size_t poly_stride_limbs, int inverse, int pass);
+
 /* ---- per-limb vector ops: Hw_* (hal/src/hal.c:15-138) ----------------------
  * n coefficients with the modulus of prime_idx. */
 int ace_hw_modadd(ace_ctx* ctx, int64_t* res, const int64_t* a, const int64_t* b, size_t prime_idx, size_t n);
