@@ -235,6 +235,9 @@ class Context:
         arr = np.ascontiguousarray(arr, dtype=np.int64).ravel()
         return DevBuf(self, arr.size).set(arr)
 
+    def copy(self, dst, src, n_words=None):
+        self._chk(self.lib.ace_copy(self.h, dst.ptr, src.ptr, src.n if n_words is None else n_words))
+
     def sync(self):
         self._chk(self.lib.ace_sync(self.h))
 

@@ -62,9 +62,11 @@ struct ArithInt {
     if (scale) { sc = scale[2 * sidx]; scp = scale[2 * sidx + 1]; }
   }
   struct TW { u64 w, wp; };
+  typedef TW TWL;  // as loaded == as used
+  __device__ __forceinline__ TW prep(const TWL& t) const { return t; }
   // NG consecutive twiddles starting at index ti0 (a multiple of NG): 16-byte loads
   template <int NG>
-  __device__ __forceinline__ void load_tw(u32 ti0, TW* tw) const {
+  __device__ __forceinline__ void load_tw(u32 ti0, TWL* tw) const {
     if (NG == 1) {
       tw[0].w = w[ti0];
       tw[0].wp = wp[ti0];
@@ -117,23 +119,24 @@ struct ArithFp {
     sci = sc / q;
   }
   struct TW { double w, wi; };
-  // NG consecutive twiddles from index ti0 (a multiple of NG); w/q is formed as
-  // w * (1/q): two roundings, relative error 2^-52, which only widens the
-  // quotient estimate (|product| <= (1/2 + 0.43 |y|/q) q), never the exactness
+  typedef double TWL;  // only w is loaded
+  // w/q is formed at use as w * (1/q): two roundings, relative error 2^-52,
+  // which only widens the quotient estimate (|product| <= (1/2 + 0.43 |y|/q) q),
+  // never the exactness
+  __device__ __forceinline__ TW prep(const TWL& t) const { return TW{t, t * qinv}; }
+  // NG consecutive twiddles from index ti0 (a multiple of NG), 16-byte loads
   template <int NG>
-  __device__ __forceinline__ void load_tw(u32 ti0, TW* tw) const {
+  __device__ __forceinline__ void load_tw(u32 ti0, TWL* tw) const {
     if (NG == 1) {
-      tw[0].w = w[ti0];
+      tw[0] = w[ti0];
     } else {
       const double2* a = reinterpret_cast<const double2*>(w + ti0);
 #pragma unroll
       for (int k = 0; k < NG / 2; ++k) {
         double2 x = a[k];
-        tw[2 * k].w = x.x; tw[2 * k + 1].w = x.y;
+        tw[2 * k] = x.x; tw[2 * k + 1] = x.y;
       }
     }
-#pragma unroll
-    for (int k = 0; k < NG; ++k) tw[k].wi = tw[k].w * qinv;
   }
   __device__ __forceinline__ T in_canon(u64 v) const {  // v < 2^52
     return __longlong_as_double((long long)(v | 0x4330000000000000ull)) - kMagic;
@@ -180,27 +183,37 @@ struct ArithFp {
 // One radix-2 stage over a register file of R values.
 // forward stage K (0 = widest span): groups = 2^K, pairs (i, i + R/2^(K+1))
 template <class A, int R, int K>
-__device__ __forceinline__ void ct_stage(const A& ar, typename A::T* v, u32 ti0) {
+__device__ __forceinline__ void ct_stage_pre(const A& ar, typename A::T* v, const typename A::TWL* tw) {
   constexpr int G = 1 << K, half = R >> (K + 1);
-  typename A::TW tw[G];
-  ar.template load_tw<G>(ti0, tw);
 #pragma unroll
   for (int g = 0; g < G; ++g) {
+    const typename A::TW w = ar.prep(tw[g]);
 #pragma unroll
-    for (int j = 0; j < half; ++j) ar.ct(v[g * 2 * half + j], v[g * 2 * half + j + half], tw[g]);
+    for (int j = 0; j < half; ++j) ar.ct(v[g * 2 * half + j], v[g * 2 * half + j + half], w);
   }
+}
+template <class A, int R, int K>
+__device__ __forceinline__ void ct_stage(const A& ar, typename A::T* v, u32 ti0) {
+  typename A::TWL tw[1 << K];
+  ar.template load_tw<(1 << K)>(ti0, tw);
+  ct_stage_pre<A, R, K>(ar, v, tw);
 }
 // inverse stage K (0 = narrowest span): span = 2^K, groups = R/2^(K+1)
 template <class A, int R, int K>
-__device__ __forceinline__ void gs_stage(const A& ar, typename A::T* v, u32 ti0) {
+__device__ __forceinline__ void gs_stage_pre(const A& ar, typename A::T* v, const typename A::TWL* tw) {
   constexpr int G = R >> (K + 1), span = 1 << K;
-  typename A::TW tw[G];
-  ar.template load_tw<G>(ti0, tw);
 #pragma unroll
   for (int g = 0; g < G; ++g) {
+    const typename A::TW w = ar.prep(tw[g]);
 #pragma unroll
-    for (int j = 0; j < span; ++j) ar.gs(v[g * 2 * span + j], v[g * 2 * span + j + span], tw[g]);
+    for (int j = 0; j < span; ++j) ar.gs(v[g * 2 * span + j], v[g * 2 * span + j + span], w);
   }
+}
+template <class A, int R, int K>
+__device__ __forceinline__ void gs_stage(const A& ar, typename A::T* v, u32 ti0) {
+  typename A::TWL tw[R >> (K + 1)];
+  ar.template load_tw<(R >> (K + 1))>(ti0, tw);
+  gs_stage_pre<A, R, K>(ar, v, tw);
 }
 template <class A, int R>
 __device__ __forceinline__ void reduce_all(const A& ar, typename A::T* v) {
@@ -245,58 +258,143 @@ __global__ __launch_bounds__(256) void ntt_fwd_strided(DevCtx c, u64* __restrict
   for (int r = 0; r < R; ++r) dst[off + r * rs] = ar.out_mid(v[r]);
 }
 
+// Work-group -> (chunk, limb, polynomial) for the chunk passes.  The grid is
+// one-dimensional.  Hardware hands consecutive work-groups to the 8 XCDs in
+// turn, and each XCD has its own L2; the map below gives every XCD whole
+// (limb, chunk) groups and runs the polynomials of a group back to back on
+// that XCD, so the group's 32 KiB of twiddles is fetched from HBM once per
+// group instead of once per polynomial.
+__device__ __forceinline__ bool chunk_block(const DevCtx& c, u32 n_limbs, u32 slots_per_group, u32& chunk,
+                                            u32& limb, u32& slot_in_group) {
+  const u32 n_chunks = c.N >> kLogChunk, n_groups = n_limbs * n_chunks;
+#if ACE_NTT_XCD
+  const u32 id = blockIdx.x, xcd = id & 7, slot = id >> 3;
+  const u32 grp = (slot / slots_per_group) * 8 + xcd;
+  slot_in_group = slot % slots_per_group;
+#else
+  const u32 grp = blockIdx.x % (((n_groups + 7) / 8) * 8);
+  slot_in_group = blockIdx.x / (((n_groups + 7) / 8) * 8);
+#endif
+  if (grp >= n_groups) return false;
+  chunk = grp % n_chunks;
+  limb = grp / n_chunks;
+  return true;
+}
+static inline unsigned chunk_grid(const DevCtx& c, u32 n_limbs, u32 slots_per_group) {
+  u32 n_groups = n_limbs * (c.N >> kLogChunk);
+  return ((n_groups + 7) / 8) * 8 * slots_per_group;
+}
+
+// Polynomials handled by one work-group of a chunk pass.  They share the
+// (limb, chunk) pair and therefore every twiddle, which is loaded once; the
+// next polynomial's words are requested before the current one is transformed.
+#ifndef ACE_NTT_PB
+#define ACE_NTT_PB 1
+#endif
+#ifndef ACE_NTT_PREFETCH
+#define ACE_NTT_PREFETCH 0
+#endif
+#ifndef ACE_NTT_XCD
+#define ACE_NTT_XCD 1
+#endif
+constexpr int kPolysPerBlock = ACE_NTT_PB;
+constexpr bool kPrefetchTw = ACE_NTT_PREFETCH != 0;
+
 // forward, chunk pass: stages logr..logN-1 on 4096 contiguous words, in place.
-// grid = (N/4096, n_limbs, n_polys)
+// grid = chunk_grid(n_limbs, ceil(n_polys / kPolysPerBlock))
 template <class A>
 __global__ __launch_bounds__(256) void ntt_fwd_chunk(DevCtx c, u64* __restrict__ data, LimbMap lm, LimbMap pos,
-                                                     u64 poly_stride, u32 logr) {
+                                                     u64 poly_stride, u32 logr, u32 n_limbs, u32 n_polys) {
   typedef typename A::T T;
   __shared__ T lds[kChunk + kChunk / 16];
   const int t = threadIdx.x;
-  const u32 chunk = blockIdx.x, limb = blockIdx.y, pi = lm.prime[limb];
-  u64* base = data + blockIdx.z * poly_stride + (u64)pos.prime[limb] * c.N + (u64)chunk * kChunk;
+  u32 chunk, limb, pblk;
+  if (!chunk_block(c, n_limbs, (n_polys + kPolysPerBlock - 1) / kPolysPerBlock, chunk, limb, pblk)) return;
+  const u32 poly0 = pblk * kPolysPerBlock;
+  const u32 cnt = min((u32)kPolysPerBlock, n_polys - poly0);
+  const u32 pi = lm.prime[limb];
+  u64* base = data + poly0 * poly_stride + (u64)pos.prime[limb] * c.N + (u64)chunk * kChunk;
   A ar;
   ar.init(c, pi, false, nullptr, 0);
-  T v[16];
   // twiddle index of local stage ls, local group 0 of this chunk: m + (chunk << ls)
   const u32 m0 = 1u << logr;
-  // round A: element e = t + 256 r, local stages 0..3; twiddles are wave-uniform
-#pragma unroll
-  for (int r = 0; r < 16; ++r) v[r] = ar.in_mid(base[t + 256 * r]);
-  reduce_all<A, 16>(ar, v);
-  ct_stage<A, 16, 0>(ar, v, (m0 << 0) + (chunk << 0));
-  ct_stage<A, 16, 1>(ar, v, (m0 << 1) + (chunk << 1));
-  ct_stage<A, 16, 2>(ar, v, (m0 << 2) + (chunk << 2));
-  ct_stage<A, 16, 3>(ar, v, (m0 << 3) + (chunk << 3));
-#pragma unroll
-  for (int r = 0; r < 16; ++r) lds[lds_pos(t + 256 * r)] = v[r];
-  __syncthreads();
-  // round B: e = hi*256 + r*16 + lo, local stages 4..7: local group = (hi << (ls-4)) + g
   const int hi = t >> 4, lo = t & 15;
+  u64 raw[16], nxt[16];
 #pragma unroll
-  for (int r = 0; r < 16; ++r) v[r] = lds[lds_pos(hi * 256 + r * 16 + lo)];
-  reduce_all<A, 16>(ar, v);
-  ct_stage<A, 16, 0>(ar, v, (m0 << 4) + (chunk << 4) + (hi << 0));
-  ct_stage<A, 16, 1>(ar, v, (m0 << 5) + (chunk << 5) + (hi << 1));
-  ct_stage<A, 16, 2>(ar, v, (m0 << 6) + (chunk << 6) + (hi << 2));
-  ct_stage<A, 16, 3>(ar, v, (m0 << 7) + (chunk << 7) + (hi << 3));
+  for (int r = 0; r < 16; ++r) raw[r] = base[t + 256 * r];
+  // the per-thread twiddles of rounds B and C (round A's are wave-uniform)
+  typename A::TWL twB0[1], twB1[2], twB2[4], twB3[8], twC0[1], twC1[2], twC2[4], twC3[8];
+  if (kPrefetchTw) {
+    ar.template load_tw<1>((m0 << 4) + (chunk << 4) + (hi << 0), twB0);
+    ar.template load_tw<2>((m0 << 5) + (chunk << 5) + (hi << 1), twB1);
+    ar.template load_tw<4>((m0 << 6) + (chunk << 6) + (hi << 2), twB2);
+    ar.template load_tw<8>((m0 << 7) + (chunk << 7) + (hi << 3), twB3);
+    ar.template load_tw<1>((m0 << 8) + (chunk << 8) + (t << 0), twC0);
+    ar.template load_tw<2>((m0 << 9) + (chunk << 9) + (t << 1), twC1);
+    ar.template load_tw<4>((m0 << 10) + (chunk << 10) + (t << 2), twC2);
+    ar.template load_tw<8>((m0 << 11) + (chunk << 11) + (t << 3), twC3);
+  }
+  for (u32 it = 0; it < cnt; ++it, base += poly_stride) {
+    if (it + 1 < cnt) {
 #pragma unroll
-  for (int r = 0; r < 16; ++r) lds[lds_pos(hi * 256 + r * 16 + lo)] = v[r];
-  __syncthreads();
-  // round C: e = t*16 + r, local stages 8..11: local group = (t << (ls-8)) + g
+      for (int r = 0; r < 16; ++r) nxt[r] = base[poly_stride + t + 256 * r];
+    }
+    T v[16];
+    // round A: element e = t + 256 r, local stages 0..3
 #pragma unroll
-  for (int r = 0; r < 16; ++r) v[r] = lds[lds_pos(t * 16 + r)];
-  reduce_all<A, 16>(ar, v);
-  ct_stage<A, 16, 0>(ar, v, (m0 << 8) + (chunk << 8) + (t << 0));
-  ct_stage<A, 16, 1>(ar, v, (m0 << 9) + (chunk << 9) + (t << 1));
-  ct_stage<A, 16, 2>(ar, v, (m0 << 10) + (chunk << 10) + (t << 2));
-  ct_stage<A, 16, 3>(ar, v, (m0 << 11) + (chunk << 11) + (t << 3));
-  u64* ldsu = reinterpret_cast<u64*>(lds);
+    for (int r = 0; r < 16; ++r) v[r] = ar.in_mid(raw[r]);
+    reduce_all<A, 16>(ar, v);
+    ct_stage<A, 16, 0>(ar, v, (m0 << 0) + (chunk << 0));
+    ct_stage<A, 16, 1>(ar, v, (m0 << 1) + (chunk << 1));
+    ct_stage<A, 16, 2>(ar, v, (m0 << 2) + (chunk << 2));
+    ct_stage<A, 16, 3>(ar, v, (m0 << 3) + (chunk << 3));
 #pragma unroll
-  for (int r = 0; r < 16; ++r) ldsu[lds_pos(t * 16 + r)] = ar.out_canon(v[r]);
-  __syncthreads();
+    for (int r = 0; r < 16; ++r) lds[lds_pos(t + 256 * r)] = v[r];
+    __syncthreads();
+    // round B: e = hi*256 + r*16 + lo, local stages 4..7: local group = (hi << (ls-4)) + g
 #pragma unroll
-  for (int r = 0; r < 16; ++r) base[t + 256 * r] = ldsu[lds_pos(t + 256 * r)];
+    for (int r = 0; r < 16; ++r) v[r] = lds[lds_pos(hi * 256 + r * 16 + lo)];
+    reduce_all<A, 16>(ar, v);
+    if (kPrefetchTw) {
+      ct_stage_pre<A, 16, 0>(ar, v, twB0);
+      ct_stage_pre<A, 16, 1>(ar, v, twB1);
+      ct_stage_pre<A, 16, 2>(ar, v, twB2);
+      ct_stage_pre<A, 16, 3>(ar, v, twB3);
+    } else {
+      ct_stage<A, 16, 0>(ar, v, (m0 << 4) + (chunk << 4) + (hi << 0));
+      ct_stage<A, 16, 1>(ar, v, (m0 << 5) + (chunk << 5) + (hi << 1));
+      ct_stage<A, 16, 2>(ar, v, (m0 << 6) + (chunk << 6) + (hi << 2));
+      ct_stage<A, 16, 3>(ar, v, (m0 << 7) + (chunk << 7) + (hi << 3));
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) lds[lds_pos(hi * 256 + r * 16 + lo)] = v[r];
+    __syncthreads();
+    // round C: e = t*16 + r, local stages 8..11: local group = (t << (ls-8)) + g
+#pragma unroll
+    for (int r = 0; r < 16; ++r) v[r] = lds[lds_pos(t * 16 + r)];
+    reduce_all<A, 16>(ar, v);
+    if (kPrefetchTw) {
+      ct_stage_pre<A, 16, 0>(ar, v, twC0);
+      ct_stage_pre<A, 16, 1>(ar, v, twC1);
+      ct_stage_pre<A, 16, 2>(ar, v, twC2);
+      ct_stage_pre<A, 16, 3>(ar, v, twC3);
+    } else {
+      ct_stage<A, 16, 0>(ar, v, (m0 << 8) + (chunk << 8) + (t << 0));
+      ct_stage<A, 16, 1>(ar, v, (m0 << 9) + (chunk << 9) + (t << 1));
+      ct_stage<A, 16, 2>(ar, v, (m0 << 10) + (chunk << 10) + (t << 2));
+      ct_stage<A, 16, 3>(ar, v, (m0 << 11) + (chunk << 11) + (t << 3));
+    }
+    u64* ldsu = reinterpret_cast<u64*>(lds);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) ldsu[lds_pos(t * 16 + r)] = ar.out_canon(v[r]);
+    __syncthreads();
+    // each thread reads back the words it will overwrite first in the next
+    // iteration, so no further barrier is needed
+#pragma unroll
+    for (int r = 0; r < 16; ++r) base[t + 256 * r] = ldsu[lds_pos(t + 256 * r)];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) raw[r] = nxt[r];
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -306,55 +404,100 @@ __global__ __launch_bounds__(256) void ntt_fwd_chunk(DevCtx c, u64* __restrict__
 // m = N >> (u+1) groups and element j belongs to group j >> (u+1).
 template <class A>
 __global__ __launch_bounds__(256) void ntt_inv_chunk(DevCtx c, u64* __restrict__ dst, const u64* __restrict__ src,
-                                                     LimbMap lm, LimbMap pos, u64 poly_stride) {
+                                                     LimbMap lm, LimbMap pos, u64 poly_stride, u32 n_limbs,
+                                                     u32 n_polys) {
   typedef typename A::T T;
   __shared__ T lds[kChunk + kChunk / 16];
   const int t = threadIdx.x;
-  const u32 chunk = blockIdx.x, limb = blockIdx.y, pi = lm.prime[limb];
-  const u64 off = blockIdx.z * poly_stride + (u64)pos.prime[limb] * c.N + (u64)chunk * kChunk;
+  u32 chunk, limb, pblk;
+  if (!chunk_block(c, n_limbs, (n_polys + kPolysPerBlock - 1) / kPolysPerBlock, chunk, limb, pblk)) return;
+  const u32 poly0 = pblk * kPolysPerBlock;
+  const u32 cnt = min((u32)kPolysPerBlock, n_polys - poly0);
+  const u32 pi = lm.prime[limb];
+  u64 off = poly0 * poly_stride + (u64)pos.prime[limb] * c.N + (u64)chunk * kChunk;
   A ar;
   ar.init(c, pi, true, nullptr, 0);
   const u32 mh = c.N >> 1;  // groups at span 1
-  T v[16];
-#pragma unroll
-  for (int r = 0; r < 16; ++r) lds[lds_pos(t + 256 * r)] = ar.in_canon(src[off + t + 256 * r]);
-  __syncthreads();
-  // round C': e = t*16 + r, u = 0..3
-#pragma unroll
-  for (int r = 0; r < 16; ++r) v[r] = lds[lds_pos(t * 16 + r)];
-  reduce_all<A, 16>(ar, v);
-  gs_stage<A, 16, 0>(ar, v, (mh >> 0) + (chunk << 11) + (t << 3));
-  gs_stage<A, 16, 1>(ar, v, (mh >> 1) + (chunk << 10) + (t << 2));
-  reduce_all<A, 16>(ar, v);
-  gs_stage<A, 16, 2>(ar, v, (mh >> 2) + (chunk << 9) + (t << 1));
-  gs_stage<A, 16, 3>(ar, v, (mh >> 3) + (chunk << 8) + (t << 0));
-#pragma unroll
-  for (int r = 0; r < 16; ++r) lds[lds_pos(t * 16 + r)] = v[r];
-  __syncthreads();
-  // round B': e = hi*256 + r*16 + lo, u = 4..7
   const int hi = t >> 4, lo = t & 15;
+  u64 raw[16], nxt[16];
 #pragma unroll
-  for (int r = 0; r < 16; ++r) v[r] = lds[lds_pos(hi * 256 + r * 16 + lo)];
-  reduce_all<A, 16>(ar, v);
-  gs_stage<A, 16, 0>(ar, v, (mh >> 4) + (chunk << 7) + (hi << 3));
-  gs_stage<A, 16, 1>(ar, v, (mh >> 5) + (chunk << 6) + (hi << 2));
-  reduce_all<A, 16>(ar, v);
-  gs_stage<A, 16, 2>(ar, v, (mh >> 6) + (chunk << 5) + (hi << 1));
-  gs_stage<A, 16, 3>(ar, v, (mh >> 7) + (chunk << 4) + (hi << 0));
+  for (int r = 0; r < 16; ++r) raw[r] = src[off + t + 256 * r];
+  // per-thread twiddles of rounds C' and B' (round A' has wave-uniform ones)
+  typename A::TWL twC0[8], twC1[4], twC2[2], twC3[1], twB0[8], twB1[4], twB2[2], twB3[1];
+  if (kPrefetchTw) {
+    ar.template load_tw<8>((mh >> 0) + (chunk << 11) + (t << 3), twC0);
+    ar.template load_tw<4>((mh >> 1) + (chunk << 10) + (t << 2), twC1);
+    ar.template load_tw<2>((mh >> 2) + (chunk << 9) + (t << 1), twC2);
+    ar.template load_tw<1>((mh >> 3) + (chunk << 8) + (t << 0), twC3);
+    ar.template load_tw<8>((mh >> 4) + (chunk << 7) + (hi << 3), twB0);
+    ar.template load_tw<4>((mh >> 5) + (chunk << 6) + (hi << 2), twB1);
+    ar.template load_tw<2>((mh >> 6) + (chunk << 5) + (hi << 1), twB2);
+    ar.template load_tw<1>((mh >> 7) + (chunk << 4) + (hi << 0), twB3);
+  }
+  for (u32 it = 0; it < cnt; ++it, off += poly_stride) {
+    if (it + 1 < cnt) {
 #pragma unroll
-  for (int r = 0; r < 16; ++r) lds[lds_pos(hi * 256 + r * 16 + lo)] = v[r];
-  __syncthreads();
-  // round A': e = t + 256 r, u = 8..11; twiddles wave-uniform
+      for (int r = 0; r < 16; ++r) nxt[r] = src[off + poly_stride + t + 256 * r];
+    }
+    T v[16];
 #pragma unroll
-  for (int r = 0; r < 16; ++r) v[r] = lds[lds_pos(t + 256 * r)];
-  reduce_all<A, 16>(ar, v);
-  gs_stage<A, 16, 0>(ar, v, (mh >> 8) + (chunk << 3));
-  gs_stage<A, 16, 1>(ar, v, (mh >> 9) + (chunk << 2));
-  reduce_all<A, 16>(ar, v);
-  gs_stage<A, 16, 2>(ar, v, (mh >> 10) + (chunk << 1));
-  gs_stage<A, 16, 3>(ar, v, (mh >> 11) + (chunk << 0));
+    for (int r = 0; r < 16; ++r) lds[lds_pos(t + 256 * r)] = ar.in_canon(raw[r]);
+    __syncthreads();
+    // round C': e = t*16 + r, u = 0..3
 #pragma unroll
-  for (int r = 0; r < 16; ++r) dst[off + t + 256 * r] = ar.out_mid(v[r]);
+    for (int r = 0; r < 16; ++r) v[r] = lds[lds_pos(t * 16 + r)];
+    reduce_all<A, 16>(ar, v);
+    if (kPrefetchTw) {
+      gs_stage_pre<A, 16, 0>(ar, v, twC0);
+      gs_stage_pre<A, 16, 1>(ar, v, twC1);
+      reduce_all<A, 16>(ar, v);
+      gs_stage_pre<A, 16, 2>(ar, v, twC2);
+      gs_stage_pre<A, 16, 3>(ar, v, twC3);
+    } else {
+      gs_stage<A, 16, 0>(ar, v, (mh >> 0) + (chunk << 11) + (t << 3));
+      gs_stage<A, 16, 1>(ar, v, (mh >> 1) + (chunk << 10) + (t << 2));
+      reduce_all<A, 16>(ar, v);
+      gs_stage<A, 16, 2>(ar, v, (mh >> 2) + (chunk << 9) + (t << 1));
+      gs_stage<A, 16, 3>(ar, v, (mh >> 3) + (chunk << 8) + (t << 0));
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) lds[lds_pos(t * 16 + r)] = v[r];
+    __syncthreads();
+    // round B': e = hi*256 + r*16 + lo, u = 4..7
+#pragma unroll
+    for (int r = 0; r < 16; ++r) v[r] = lds[lds_pos(hi * 256 + r * 16 + lo)];
+    reduce_all<A, 16>(ar, v);
+    if (kPrefetchTw) {
+      gs_stage_pre<A, 16, 0>(ar, v, twB0);
+      gs_stage_pre<A, 16, 1>(ar, v, twB1);
+      reduce_all<A, 16>(ar, v);
+      gs_stage_pre<A, 16, 2>(ar, v, twB2);
+      gs_stage_pre<A, 16, 3>(ar, v, twB3);
+    } else {
+      gs_stage<A, 16, 0>(ar, v, (mh >> 4) + (chunk << 7) + (hi << 3));
+      gs_stage<A, 16, 1>(ar, v, (mh >> 5) + (chunk << 6) + (hi << 2));
+      reduce_all<A, 16>(ar, v);
+      gs_stage<A, 16, 2>(ar, v, (mh >> 6) + (chunk << 5) + (hi << 1));
+      gs_stage<A, 16, 3>(ar, v, (mh >> 7) + (chunk << 4) + (hi << 0));
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) lds[lds_pos(hi * 256 + r * 16 + lo)] = v[r];
+    __syncthreads();
+    // round A': e = t + 256 r, u = 8..11; twiddles wave-uniform.  The words read
+    // here are the ones this thread overwrites first in the next iteration.
+#pragma unroll
+    for (int r = 0; r < 16; ++r) v[r] = lds[lds_pos(t + 256 * r)];
+    reduce_all<A, 16>(ar, v);
+    gs_stage<A, 16, 0>(ar, v, (mh >> 8) + (chunk << 3));
+    gs_stage<A, 16, 1>(ar, v, (mh >> 9) + (chunk << 2));
+    reduce_all<A, 16>(ar, v);
+    gs_stage<A, 16, 2>(ar, v, (mh >> 10) + (chunk << 1));
+    gs_stage<A, 16, 3>(ar, v, (mh >> 11) + (chunk << 0));
+#pragma unroll
+    for (int r = 0; r < 16; ++r) dst[off + t + 256 * r] = ar.out_mid(v[r]);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) raw[r] = nxt[r];
+  }
 }
 
 // inverse, strided pass: spans 4096..N/2, then scale every word by the limb's
@@ -424,14 +567,17 @@ template <class A, int LOGR>
 static void run_large(hipStream_t st, const DevCtx& c, u64* dst, const u64* src, const LimbMap& lm, const LimbMap& pos,
                       const LimbMap& sidx, u32 n_limbs, u32 n_polys, u64 poly_stride, bool inverse,
                       const u64* scale, int passes) {
-  dim3 gs((c.N >> LOGR) / 256, n_limbs, n_polys), gc(c.N / kChunk, n_limbs, n_polys);
+  dim3 gs((c.N >> LOGR) / 256, n_limbs, n_polys), gc(chunk_grid(c, n_limbs, (n_polys + kPolysPerBlock - 1) / kPolysPerBlock));
   if (!inverse) {
     if (passes & 1)
       hipLaunchKernelGGL((ntt_fwd_strided<A, LOGR>), gs, dim3(256), 0, st, c, dst, src, lm, pos, poly_stride);
     if (passes & 2)
-      hipLaunchKernelGGL((ntt_fwd_chunk<A>), gc, dim3(256), 0, st, c, dst, lm, pos, poly_stride, (u32)LOGR);
+      hipLaunchKernelGGL((ntt_fwd_chunk<A>), gc, dim3(256), 0, st, c, dst, lm, pos, poly_stride, (u32)LOGR, n_limbs,
+                         n_polys);
   } else {
-    if (passes & 1) hipLaunchKernelGGL((ntt_inv_chunk<A>), gc, dim3(256), 0, st, c, dst, src, lm, pos, poly_stride);
+    if (passes & 1)
+      hipLaunchKernelGGL((ntt_inv_chunk<A>), gc, dim3(256), 0, st, c, dst, src, lm, pos, poly_stride, n_limbs,
+                         n_polys);
     if (passes & 2)
       hipLaunchKernelGGL((ntt_inv_strided<A, LOGR>), gs, dim3(256), 0, st, c, dst, lm, pos, sidx, poly_stride, scale);
   }
