@@ -43,6 +43,16 @@ struct ModUpDev {
   ConvMap conv{};
 };
 
+// all digits of a level at once (Precomp)
+struct PrecompDev {
+  u64* scale_ntt = nullptr;   // [level][2]: 1/N * hat_inv of the limb's own digit
+  u64* scale_coef = nullptr;  // [level][2]
+  std::vector<ConvJob> jobs;  // one per digit; t_off / out_off filled for one operand
+  LimbMap tgt_lm{}, tgt_pos{};  // every converted limb of every digit: prime, position in the digits block
+  u32 n_tgt = 0;
+  bool one_ntt_launch = false;  // positions fit a byte and n_tgt <= kMaxPrimes
+};
+
 struct RescaleDev {
   u64* sw = nullptr;    // [level-1][3]: K, K', diff
   u64* tail = nullptr;  // [level-1][2]: q_l^-1, Shoup
@@ -59,6 +69,7 @@ struct ace_ctx {
   std::vector<void*> owned;  // device allocations freed with the context
   std::map<std::pair<size_t, size_t>, ModUpDev> modup;
   std::map<size_t, RescaleDev> rescale;
+  std::map<size_t, PrecompDev> precomp;
   // Mod_down / Extend constants
   u64* phat = nullptr;        // [K][L]
   u64* pscale_ntt = nullptr;  // [K][2]
@@ -126,6 +137,46 @@ struct ace_ctx {
       m.conv.out_limb[j] = (uint8_t)pos;
     }
     return modup.emplace(key, std::move(m)).first->second;
+  }
+
+  const PrecompDev& precomp_at(size_t level) {
+    auto it = precomp.find(level);
+    if (it != precomp.end()) return it->second;
+    PrecompDev pd;
+    const size_t nd = h.num_decomp(level), T = level + h.K, N = h.N;
+    std::vector<u64> sn(2 * level), scf(2 * level);
+    pd.one_ntt_launch = nd * T <= 256;
+    for (size_t d = 0; d < nd; ++d) {
+      const ModUpDev& m = modup_at(level, d);
+      const size_t start = h.part_size * d, len = m.t.digit.size(), nc = m.t.compl_idx.size();
+      for (size_t i = 0; i < len; ++i) {
+        size_t pi = m.t.digit[i];
+        u64 q = h.primes[pi].q;
+        u64 a = mul_mod(h.primes[pi].ninv, m.t.hat_inv[i], q);
+        sn[2 * pi] = a;                 sn[2 * pi + 1] = shoup(a, q);
+        scf[2 * pi] = m.t.hat_inv[i];   scf[2 * pi + 1] = shoup(m.t.hat_inv[i], q);
+      }
+      ConvJob j{};
+      j.hat = m.hat;
+      j.hat_stride = (u32)nc;
+      j.nd = (u32)len;
+      j.nc = (u32)nc;
+      j.t_off = start * N;
+      j.out_off = d * T * N;
+      j.map = m.conv;
+      pd.jobs.push_back(j);
+      for (size_t k = 0; k < nc; ++k) {
+        if (pd.n_tgt < (u32)kMaxPrimes) {
+          pd.tgt_lm.prime[pd.n_tgt] = m.compl_lm.prime[k];
+          pd.tgt_pos.prime[pd.n_tgt] = (uint8_t)(d * T + m.compl_pos.prime[k]);
+        }
+        ++pd.n_tgt;
+      }
+    }
+    if (pd.n_tgt > (u32)kMaxPrimes) pd.one_ntt_launch = false;
+    pd.scale_ntt = upload_vec(sn);
+    pd.scale_coef = upload_vec(scf);
+    return precomp.emplace(level, std::move(pd)).first->second;
   }
 
   const RescaleDev& rescale_at(size_t level) {
@@ -232,9 +283,18 @@ LimbMap poly_lm(const ace_ctx* c, size_t level, bool with_p) {
 bool level_ok(const ace_ctx* c, size_t level) { return level >= 1 && level <= c->h.L; }
 
 // ---- internal sequencers: scratch comes from the arena, already sized ------
+// Every sequencer works on a batch: n polynomials (or operands) per launch.
 
-// Decomp_modup (rns_poly.c:160-258): copy the digit, INTT it scaled by the
-// inverse cofactors, convert to the complement basis, NTT the new limbs.
+PolySeq shifted(const PolySeq& s, u64 words) {
+  PolySeq r = s;
+  r.b[0] += words;
+  r.b[1] += words;
+  return r;
+}
+
+// Decomp_modup (rns_poly.c:160-258), one digit of one polynomial: copy the
+// digit, INTT it scaled by the inverse cofactors, convert to the complement
+// basis, NTT the new limbs.
 void do_decomp_modup(ace_ctx* c, u64* res, const u64* src, size_t level, size_t part, bool is_ntt) {
   const ModUpDev& m = c->modup_at(level, part);
   const size_t N = c->h.N, nd = m.t.digit.size(), nc = m.t.compl_idx.size(), start = c->h.part_size * part;
@@ -242,52 +302,126 @@ void do_decomp_modup(ace_ctx* c, u64* res, const u64* src, size_t level, size_t 
     HIP_OK(hipMemcpyAsync(res + start * N, src + start * N, nd * N * sizeof(u64), hipMemcpyDeviceToDevice, c->stream));
   size_t mark = c->ws_used;
   u64* t = c->take(nd * N);
-  if (is_ntt) launch_ntt(c->stream, c->d, t, src + start * N, m.digit_lm, nullptr, (u32)nd, 1, 0, true, m.scale_ntt);
-  else        launch_mul_const(c->stream, c->d, t, src + start * N, m.scale_coef, m.digit_lm, (u32)nd);
-  launch_baseconv(c->stream, c->d, res, t, m.hat, (u32)nc, (u32)nd, (u32)nc, m.conv);
-  if (is_ntt) launch_ntt(c->stream, c->d, res, res, m.compl_lm, &m.compl_pos, (u32)nc, 1, 0, false, nullptr);
+  if (is_ntt)
+    launch_ntt(c->stream, c->d, seq_strided(t, 0), seq_strided(src + start * N, 0), m.digit_lm, nullptr, (u32)nd, 1,
+               true, m.scale_ntt);
+  else
+    launch_mul_const(c->stream, c->d, t, src + start * N, m.scale_coef, m.digit_lm, (u32)nd);
+  ConvBatch b{};
+  b.n_jobs = 1;
+  b.job[0].hat = m.hat;
+  b.job[0].hat_stride = (u32)nc;
+  b.job[0].nd = (u32)nd;
+  b.job[0].nc = (u32)nc;
+  b.job[0].map = m.conv;
+  launch_baseconv(c->stream, c->d, res, t, b, 1);
+  if (is_ntt)
+    launch_ntt(c->stream, c->d, seq_strided(res, 0), seq_strided(res, 0), m.compl_lm, &m.compl_pos, (u32)nc, 1, false,
+               nullptr);
   c->ws_used = mark;
 }
 
-// Mod_down (rns_poly.c:260-308); addend (optional) is added to the result
-void do_mod_down(ace_ctx* c, u64* res, const u64* src, size_t level, bool is_ntt, const u64* addend) {
+// Precomp (rns_poly.c:416-481) for nb polynomials: operand o reads
+// src + o*src_stride (level limbs) and writes res + o*res_stride
+// (num_decomp x (level+K) limbs).  One INTT over all limbs (each scaled by its
+// own digit's inverse cofactor), one base-conversion launch per 4 digits, one
+// NTT over every converted limb.
+void do_precomp(ace_ctx* c, u64* res, u64 res_stride, const u64* src, u64 src_stride, size_t nb, size_t level,
+                bool is_ntt) {
+  const PrecompDev& pd = c->precomp_at(level);
+  const size_t N = c->h.N, nd = c->h.num_decomp(level), T = level + c->h.K;
+  size_t mark = c->ws_used;
+  u64* t = c->take(nb * level * N);
+  if (is_ntt) {
+    launch_ntt(c->stream, c->d, seq_strided(t, level * N), seq_strided(src, src_stride), c->q_lm, nullptr, (u32)level,
+               (u32)nb, true, pd.scale_ntt);
+  } else {
+    for (size_t o = 0; o < nb; ++o)
+      launch_mul_const(c->stream, c->d, t + o * level * N, src + o * src_stride, pd.scale_coef, c->q_lm, (u32)level);
+  }
+  launch_digit_copy(c->stream, c->d, res, src, (u32)level, (u32)c->h.part_size, (u32)nd, T * N, res_stride, src_stride,
+                    (u32)nb);
+  for (size_t j0 = 0; j0 < nd; j0 += kMaxConvJobs) {
+    ConvBatch b{};
+    b.n_jobs = (u32)std::min<size_t>(kMaxConvJobs, nd - j0);
+    for (u32 k = 0; k < b.n_jobs; ++k) b.job[k] = pd.jobs[j0 + k];
+    b.t_stride = level * N;
+    b.out_stride = res_stride;
+    launch_baseconv(c->stream, c->d, res, t, b, (u32)nb);
+  }
+  if (is_ntt) {
+    PolySeq rs = seq_strided(res, res_stride);
+    if (pd.one_ntt_launch) {
+      launch_ntt(c->stream, c->d, rs, rs, pd.tgt_lm, &pd.tgt_pos, pd.n_tgt, (u32)nb, false, nullptr);
+    } else {
+      for (size_t d = 0; d < nd; ++d) {
+        const ModUpDev& m = c->modup_at(level, d);
+        PolySeq ds = shifted(rs, d * T * N);
+        launch_ntt(c->stream, c->d, ds, ds, m.compl_lm, &m.compl_pos, (u32)m.t.compl_idx.size(), (u32)nb, false,
+                   nullptr);
+      }
+    }
+  }
+  c->ws_used = mark;
+}
+
+// Mod_down (rns_poly.c:260-308) of np polynomials; addend_mode: 0 none,
+// 1 add addend.at(p) to every polynomial, 2 only to even p
+void do_mod_down(ace_ctx* c, const PolySeq& res, const PolySeq& src, size_t np, size_t level, bool is_ntt,
+                 const PolySeq* addend, int addend_mode) {
   const size_t N = c->h.N, K = c->h.K, L = c->h.L;
   size_t mark = c->ws_used;
-  u64* t = c->take(K * N);
-  u64* y = c->take(level * N);
-  if (is_ntt) launch_ntt(c->stream, c->d, t, src + level * N, c->p_lm, nullptr, (u32)K, 1, 0, true, c->pscale_ntt);
-  else        launch_mul_const(c->stream, c->d, t, src + level * N, c->pscale_coef, c->p_lm, (u32)K);
-  ConvMap cm{};
-  for (size_t i = 0; i < level; ++i) { cm.prime[i] = (uint8_t)i; cm.out_limb[i] = (uint8_t)i; }
-  launch_baseconv(c->stream, c->d, y, t, c->phat, (u32)L, (u32)K, (u32)level, cm);
-  if (is_ntt) launch_ntt(c->stream, c->d, y, y, c->q_lm, nullptr, (u32)level, 1, 0, false, nullptr);
-  launch_moddown_tail(c->stream, c->d, res, src, y, addend, c->pinv, c->q_lm, (u32)level);
+  u64* t = c->take(np * K * N);
+  u64* y = c->take(np * level * N);
+  if (is_ntt) {
+    launch_ntt(c->stream, c->d, seq_strided(t, K * N), shifted(src, level * N), c->p_lm, nullptr, (u32)K, (u32)np, true,
+               c->pscale_ntt);
+  } else {
+    for (size_t p = 0; p < np; ++p)
+      launch_mul_const(c->stream, c->d, t + p * K * N, src.at((u32)p) + level * N, c->pscale_coef, c->p_lm, (u32)K);
+  }
+  ConvBatch b{};
+  b.n_jobs = 1;
+  b.job[0].hat = c->phat;
+  b.job[0].hat_stride = (u32)L;
+  b.job[0].nd = (u32)K;
+  b.job[0].nc = (u32)level;
+  for (size_t i = 0; i < level; ++i) { b.job[0].map.prime[i] = (uint8_t)i; b.job[0].map.out_limb[i] = (uint8_t)i; }
+  b.t_stride = K * N;
+  b.out_stride = level * N;
+  launch_baseconv(c->stream, c->d, y, t, b, (u32)np);
+  if (is_ntt) {
+    PolySeq ys = seq_strided(y, level * N);
+    launch_ntt(c->stream, c->d, ys, ys, c->q_lm, nullptr, (u32)level, (u32)np, false, nullptr);
+  }
+  launch_moddown_tail(c->stream, c->d, res, src, y, level * N, addend_mode ? addend : nullptr, addend_mode, c->pinv,
+                      c->q_lm, (u32)level, (u32)np);
   c->ws_used = mark;
 }
 
-// Rescale (rns_poly.c:310-404)
-void do_rescale(ace_ctx* c, u64* res, const u64* src, size_t level, bool is_ntt) {
+// Rescale (rns_poly.c:310-404) of np polynomials
+void do_rescale(ace_ctx* c, const PolySeq& res, const PolySeq& src, size_t np, size_t level, bool is_ntt) {
   const size_t N = c->h.N;
   const RescaleDev& r = c->rescale_at(level);
   if (!is_ntt) {
-    launch_rescale_coef(c->stream, c->d, res, src, src + (level - 1) * N, r.tail, c->q_lm, (u32)(level - 1));
+    for (size_t p = 0; p < np; ++p)
+      launch_rescale_coef(c->stream, c->d, res.at((u32)p), src.at((u32)p), src.at((u32)p) + (level - 1) * N, r.tail,
+                          c->q_lm, (u32)(level - 1));
     return;
   }
   size_t mark = c->ws_used;
-  u64* last = c->take(N);
-  u64* u = c->take((level - 1) * N);
+  u64* last = c->take(np * N);
+  u64* u = c->take(np * (level - 1) * N);
+  launch_pick_limb(c->stream, c->d, last, src, (u32)(level - 1), (u32)np);
   LimbMap one{};
   one.prime[0] = (uint8_t)(level - 1);
-  launch_ntt(c->stream, c->d, last, src + (level - 1) * N, one, nullptr, 1, 1, 0, true, nullptr);
-  launch_rescale_switch(c->stream, c->d, u, last, (u32)(level - 1), r.sw, c->q_lm, (u32)(level - 1));
-  launch_ntt(c->stream, c->d, u, u, c->q_lm, nullptr, (u32)(level - 1), 1, 0, false, nullptr);
-  launch_rescale_tail(c->stream, c->d, res, src, u, r.tail, c->q_lm, (u32)(level - 1));
+  PolySeq ls = seq_strided(last, N), us = seq_strided(u, (level - 1) * N);
+  launch_ntt(c->stream, c->d, ls, ls, one, nullptr, 1, (u32)np, true, nullptr);
+  launch_rescale_switch(c->stream, c->d, u, (level - 1) * N, last, N, (u32)(level - 1), r.sw, c->q_lm,
+                        (u32)(level - 1), (u32)np);
+  launch_ntt(c->stream, c->d, us, us, c->q_lm, nullptr, (u32)(level - 1), (u32)np, false, nullptr);
+  launch_rescale_tail(c->stream, c->d, res, src, u, (level - 1) * N, r.tail, c->q_lm, (u32)(level - 1), (u32)np);
   c->ws_used = mark;
-}
-
-void do_precomp(ace_ctx* c, u64* res, const u64* src, size_t level, bool is_ntt) {
-  size_t nd = c->h.num_decomp(level), stride = (level + c->h.K) * (size_t)c->h.N;
-  for (size_t part = 0; part < nd; ++part) do_decomp_modup(c, res + part * stride, src, level, part, is_ntt);
 }
 
 // key limb positions of a polynomial viewed at `level` (Derive_poly, rns_poly.c:701-707)
@@ -298,18 +432,42 @@ LimbMap key_pos(const ace_ctx* c, size_t level) {
   return kp;
 }
 
-// Fast_switch_key (evaluator.c:411-462); add0/add1 are fused into the Mod_down tails
-void do_switch_key(ace_ctx* c, u64* out0, u64* out1, const u64* digits, const u64* swk, size_t level,
-                   const u64* add0, const u64* add1) {
+// Fast_switch_key (evaluator.c:411-462) for nb operands.  Operand o reads the
+// digits at digits + o*digits_op_stride (0: all share one set) and key
+// keys.p[o] (or keys.p[0] when keys.n == 1); its two results are polynomials
+// 2o and 2o+1 of `out`.  The addend is fused into the Mod_down tail.
+void do_switch_key(ace_ctx* c, const PolySeq& out, const u64* digits, u64 digits_op_stride, const KeySet& keys,
+                   size_t nb, size_t level, const PolySeq* addend, int addend_mode) {
   const size_t N = c->h.N, T = level + c->h.K, kpoly = (c->h.L + c->h.K) * N, nd = c->h.num_decomp(level);
   size_t mark = c->ws_used;
-  u64* e0 = c->take(T * N);
-  u64* e1 = c->take(T * N);
+  u64* e = c->take(nb * 2 * T * N);  // [operand][b|a][T limbs]
   LimbMap lm = poly_lm(c, level, true), kp = key_pos(c, level);
-  launch_dotprod(c->stream, c->d, e0, e1, digits, T * N, swk, swk + kpoly, 2 * kpoly, (u32)nd, lm, kp, (u32)T);
-  do_mod_down(c, out0, e0, level, true, add0);
-  do_mod_down(c, out1, e1, level, true, add1);
+  launch_dotprod(c->stream, c->d, e, e + T * N, 2 * T * N, digits, T * N, digits_op_stride, keys, kpoly, 2 * kpoly,
+                 (u32)nd, lm, kp, (u32)T, (u32)nb);
+  do_mod_down(c, out, seq_strided(e, T * N), 2 * nb, level, true, addend, addend_mode);
   c->ws_used = mark;
+}
+
+KeySet one_key(const u64* swk) {
+  KeySet k{};
+  k.n = 1;
+  k.p[0] = swk;
+  return k;
+}
+
+// Mul_ciphertext + Rescale_ciphertext for nb ciphertext pairs (evaluator.c:142-190, 342-362)
+void do_mul_relin_rescale(ace_ctx* c, u64* r0, u64* r1, u64 out_stride, const u64* a0, const u64* a1, const u64* b0,
+                          const u64* b1, u64 in_stride, const u64* swk, size_t nb, size_t level) {
+  const size_t N = c->h.N, nd = c->h.num_decomp(level), T = level + c->h.K;
+  u64* d01 = c->take(nb * 2 * level * N);  // [operand][c0|c1][level limbs]
+  u64* d2 = c->take(nb * level * N);
+  u64* digits = c->take(nb * nd * T * N);
+  launch_tensor(c->stream, c->d, d01, d01 + level * N, d2, a0, a1, b0, b1, c->q_lm, (u32)level, (u32)nb,
+                2 * level * N, level * N, in_stride);
+  do_precomp(c, digits, nd * T * N, d2, level * N, nb, level, true);
+  PolySeq ds = seq_strided(d01, level * N);
+  do_switch_key(c, ds, digits, nd * T * N, one_key(swk), nb, level, &ds, 1);  // relinearised ct replaces d0, d1
+  do_rescale(c, seq_pair(r0, r1, out_stride), ds, 2 * nb, level, true);
 }
 
 }  // namespace
@@ -462,8 +620,9 @@ static int ntt_common(ace_ctx* c, int64_t* dst, const int64_t* src, const int32_
     if (prime_idx[t] < 0 || (size_t)prime_idx[t] >= c->h.L + c->h.K) return fail("ace_ntt: prime index out of range");
     lm.prime[t] = (uint8_t)prime_idx[t];
   }
-  if (!launch_ntt(c->stream, c->d, U(dst), U(src), lm, nullptr, (u32)n_limbs, (u32)n_polys,
-                  (u64)stride_limbs * c->h.N, inverse, nullptr, passes))
+  const u64 stride = (u64)stride_limbs * c->h.N;
+  if (!launch_ntt(c->stream, c->d, seq_strided(U(dst), stride), seq_strided(U(src), stride), lm, nullptr,
+                  (u32)n_limbs, (u32)n_polys, inverse, nullptr, passes))
     return fail("ace_ntt: ring degree not supported");
   ACE_CATCH_INT
 }
@@ -621,7 +780,7 @@ int ace_precomp(ace_ctx* c, int64_t* res, const int64_t* src, size_t level, int 
   if (!level_ok(c, level)) return fail("ace_precomp: level out of range");
   c->ensure_ws(c->std_ws(level));
   c->ws_used = 0;
-  do_precomp(c, U(res), U(src), level, is_ntt != 0);
+  do_precomp(c, U(res), 0, U(src), 0, 1, level, is_ntt != 0);
   ACE_CATCH_INT
 }
 
@@ -631,7 +790,7 @@ int ace_mod_down(ace_ctx* c, int64_t* res, const int64_t* src, size_t level, int
   if (!level_ok(c, level)) return fail("ace_mod_down: level out of range");
   c->ensure_ws(c->std_ws(level));
   c->ws_used = 0;
-  do_mod_down(c, U(res), U(src), level, is_ntt != 0, nullptr);
+  do_mod_down(c, seq_strided(U(res), 0), seq_strided(U(src), 0), 1, level, is_ntt != 0, nullptr, 0);
   ACE_CATCH_INT
 }
 
@@ -641,7 +800,7 @@ int ace_rescale(ace_ctx* c, int64_t* res, const int64_t* src, size_t level, int 
   if (level < 2 || level > c->h.L) return fail("Level of rescale opnd is too small");
   c->ensure_ws(c->std_ws(level));
   c->ws_used = 0;
-  do_rescale(c, U(res), U(src), level, is_ntt != 0);
+  do_rescale(c, seq_strided(U(res), 0), seq_strided(U(src), 0), 1, level, is_ntt != 0);
   ACE_CATCH_INT
 }
 
@@ -662,8 +821,8 @@ int ace_dot_prod(ace_ctx* c, int64_t* res, const int64_t* digits, const int64_t*
   if (n_parts == 0 || n_parts > c->h.parts) return fail("ace_dot_prod: number of digits out of range");
   size_t T = level + c->h.K;
   LimbMap lm = poly_lm(c, level, true), kp = key_pos(c, level);
-  launch_dotprod(c->stream, c->d, U(res), nullptr, U(digits), T * (size_t)c->h.N, U(key), nullptr, key_stride,
-                 (u32)n_parts, lm, kp, (u32)T);
+  launch_dotprod(c->stream, c->d, U(res), nullptr, 0, U(digits), T * (size_t)c->h.N, 0, one_key(U(key)), 0,
+                 key_stride, (u32)n_parts, lm, kp, (u32)T, 1);
   ACE_CATCH_INT
 }
 
@@ -673,7 +832,7 @@ int ace_mul_ciph3(ace_ctx* c, int64_t* d0, int64_t* d1, int64_t* d2, const int64
   ACE_TRY
   if (!d0 || !d1 || !d2 || !a0 || !a1 || !b0 || !b1) return fail("ace_mul_ciph3: null argument");
   if (!level_ok(c, level)) return fail("ace_mul_ciph3: level out of range");
-  launch_tensor(c->stream, c->d, U(d0), U(d1), U(d2), U(a0), U(a1), U(b0), U(b1), c->q_lm, (u32)level);
+  launch_tensor(c->stream, c->d, U(d0), U(d1), U(d2), U(a0), U(a1), U(b0), U(b1), c->q_lm, (u32)level, 1, 0, 0, 0);
   ACE_CATCH_INT
 }
 
@@ -684,7 +843,7 @@ int ace_fast_switch_key(ace_ctx* c, int64_t* out0, int64_t* out1, const int64_t*
   if (!level_ok(c, level)) return fail("ace_fast_switch_key: level out of range");
   c->ensure_ws(c->std_ws(level));
   c->ws_used = 0;
-  do_switch_key(c, U(out0), U(out1), U(digits), U(swk), level, nullptr, nullptr);
+  do_switch_key(c, seq_pair(U(out0), U(out1), 0), U(digits), 0, one_key(U(swk)), 1, level, nullptr, 0);
   ACE_CATCH_INT
 }
 
@@ -697,8 +856,9 @@ int ace_relin(ace_ctx* c, int64_t* r0, int64_t* r1, const int64_t* d0, const int
   c->ws_used = 0;
   size_t nd = c->h.num_decomp(level), T = level + c->h.K;
   u64* digits = c->take(nd * T * c->h.N);
-  do_precomp(c, digits, U(d2), level, true);
-  do_switch_key(c, U(r0), U(r1), digits, U(swk), level, U(d0), U(d1));
+  do_precomp(c, digits, 0, U(d2), 0, 1, level, true);
+  PolySeq add = seq_pair(U(d0), U(d1), 0);
+  do_switch_key(c, seq_pair(U(r0), U(r1), 0), digits, 0, one_key(U(swk)), 1, level, &add, 1);
   ACE_CATCH_INT
 }
 
@@ -708,8 +868,7 @@ int ace_rescale_ciph(ace_ctx* c, int64_t* r0, int64_t* r1, const int64_t* c0, co
   if (level < 2 || level > c->h.L) return fail("Level of rescale opnd is too small");
   c->ensure_ws(c->std_ws(level));
   c->ws_used = 0;
-  do_rescale(c, U(r0), U(c0), level, true);
-  do_rescale(c, U(r1), U(c1), level, true);
+  do_rescale(c, seq_pair(U(r0), U(r1), 0), seq_pair(U(c0), U(c1), 0), 2, level, true);
   ACE_CATCH_INT
 }
 
@@ -720,27 +879,41 @@ int ace_mul_relin_rescale(ace_ctx* c, int64_t* r0, int64_t* r1, const int64_t* a
   if (level < 2 || level > c->h.L) return fail("ace_mul_relin_rescale: level out of range");
   c->ensure_ws(c->std_ws(level));
   c->ws_used = 0;
-  const size_t N = c->h.N, nd = c->h.num_decomp(level), T = level + c->h.K;
-  u64* d0 = c->take(level * N);
-  u64* d1 = c->take(level * N);
-  u64* d2 = c->take(level * N);
-  u64* digits = c->take(nd * T * N);
-  launch_tensor(c->stream, c->d, d0, d1, d2, U(a0), U(a1), U(b0), U(b1), c->q_lm, (u32)level);
-  do_precomp(c, digits, d2, level, true);
-  do_switch_key(c, d0, d1, digits, U(swk), level, d0, d1);  // relinearised ciphertext replaces d0, d1
-  do_rescale(c, U(r0), d0, level, true);
-  do_rescale(c, U(r1), d1, level, true);
+  do_mul_relin_rescale(c, U(r0), U(r1), 0, U(a0), U(a1), U(b0), U(b1), 0, U(swk), 1, level);
   ACE_CATCH_INT
 }
 
-static void do_fast_rotate(ace_ctx* c, u64* r0, u64* r1, const u64* c0, const u64* digits, const u64* swk,
-                           const i64* order, size_t level) {
+int ace_mul_relin_rescale_batch(ace_ctx* c, int64_t* r0, int64_t* r1, size_t out_stride, const int64_t* a0,
+                                const int64_t* a1, const int64_t* b0, const int64_t* b1, size_t in_stride,
+                                const int64_t* swk, size_t level, size_t count) {
+  ACE_TRY
+  if (count == 0) return 0;
+  if (!r0 || !r1 || !a0 || !a1 || !b0 || !b1 || !swk) return fail("ace_mul_relin_rescale_batch: null argument");
+  if (level < 2 || level > c->h.L) return fail("ace_mul_relin_rescale_batch: level out of range");
+  if (count > 1 && (in_stride < level * (size_t)c->h.N || out_stride < (level - 1) * (size_t)c->h.N))
+    return fail("ace_mul_relin_rescale_batch: stride smaller than one polynomial");
+  const size_t chunk = 16;  // operands per pass: bounds the scratch arena at 16x the single-operand size
+  c->ensure_ws(std::min(count, chunk) * c->std_ws(level));
+  for (size_t o = 0; o < count; o += chunk) {
+    size_t nb = std::min(chunk, count - o);
+    c->ws_used = 0;
+    do_mul_relin_rescale(c, U(r0) + o * out_stride, U(r1) + o * out_stride, out_stride, U(a0) + o * in_stride,
+                         U(a1) + o * in_stride, U(b0) + o * in_stride, U(b1) + o * in_stride, in_stride, U(swk), nb,
+                         level);
+  }
+  ACE_CATCH_INT
+}
+
+// Fast_rotate for nr <= kMaxBatchPtrs rotations of one ciphertext sharing the digits
+static void do_fast_rotate(ace_ctx* c, u64* r0, u64* r1, u64 r_stride, const u64* c0, const u64* digits,
+                           const KeySet& keys, const OrderSet& orders, size_t nr, size_t level) {
   const size_t N = c->h.N;
   size_t mark = c->ws_used;
-  u64* t0 = c->take(level * N);
-  u64* t1 = c->take(level * N);
-  do_switch_key(c, t0, t1, digits, swk, level, c0, nullptr);
-  launch_gather2(c->stream, c->d, r0, r1, t0, t1, order, c->q_lm, (u32)level, N);
+  u64* t01 = c->take(nr * 2 * level * N);  // [rotation][c0|c1][level limbs]
+  PolySeq add = seq_pair(c0, c0, 0);       // c0 is added to the first polynomial of every rotation
+  do_switch_key(c, seq_strided(t01, level * N), digits, 0, keys, nr, level, &add, 2);
+  launch_gather2(c->stream, c->d, r0, r1, r_stride, t01, t01 + level * N, 2 * level * N, orders, c->q_lm, (u32)level,
+                 (u32)nr);
   c->ws_used = mark;
 }
 
@@ -751,7 +924,10 @@ int ace_fast_rotate(ace_ctx* c, int64_t* r0, int64_t* r1, const int64_t* c0, con
   if (!level_ok(c, level)) return fail("ace_fast_rotate: level out of range");
   c->ensure_ws(c->std_ws(level));
   c->ws_used = 0;
-  do_fast_rotate(c, U(r0), U(r1), U(c0), U(digits), U(swk), order, level);
+  OrderSet os{};
+  os.n = 1;
+  os.p[0] = order;
+  do_fast_rotate(c, U(r0), U(r1), 0, U(c0), U(digits), one_key(U(swk)), os, 1, level);
   ACE_CATCH_INT
 }
 
@@ -763,13 +939,21 @@ int ace_rotate_batch(ace_ctx* c, int64_t* r0s, int64_t* r1s, const int64_t* c0, 
   if (!level_ok(c, level)) return fail("ace_rotate_batch: level out of range");
   for (size_t i = 0; i < count; ++i)
     if (!swks[i] || !orders[i]) return fail("ace_rotate_batch: null key or order table");
-  c->ensure_ws(c->std_ws(level));
-  c->ws_used = 0;
   const size_t N = c->h.N, nd = c->h.num_decomp(level), T = level + c->h.K;
+  const size_t chunk = kMaxBatchPtrs;
+  c->ensure_ws((std::min(count, chunk) + 1) * c->std_ws(level));
+  c->ws_used = 0;
   u64* digits = c->take(nd * T * N);
-  do_precomp(c, digits, U(c1), level, true);
-  for (size_t i = 0; i < count; ++i)
-    do_fast_rotate(c, U(r0s) + i * level * N, U(r1s) + i * level * N, U(c0), digits, U(swks[i]), orders[i], level);
+  do_precomp(c, digits, 0, U(c1), 0, 1, level, true);
+  for (size_t i0 = 0; i0 < count; i0 += chunk) {
+    size_t nr = std::min(chunk, count - i0);
+    KeySet ks{};
+    OrderSet os{};
+    ks.n = os.n = (u32)nr;
+    for (size_t i = 0; i < nr; ++i) { ks.p[i] = U(swks[i0 + i]); os.p[i] = orders[i0 + i]; }
+    if (nr == 1) { ks.n = os.n = 1; }
+    do_fast_rotate(c, U(r0s) + i0 * level * N, U(r1s) + i0 * level * N, level * N, U(c0), digits, ks, os, nr, level);
+  }
   ACE_CATCH_INT
 }
 

@@ -50,6 +50,30 @@ struct LimbMap {
   uint8_t prime[kMaxPrimes];
 };
 
+// A sequence of polynomials addressed as pairs: polynomial p lives at
+// b[p & 1] + (p >> 1) * pair_stride words.  Covers a plain strided batch
+// (b[1] = b[0] + stride, pair_stride = 2*stride) as well as the two halves
+// (c0, c1) of a batch of ciphertexts held in separate buffers.
+struct PolySeq {
+  u64* b[2];
+  u64 pair_stride;
+  __host__ __device__ __forceinline__ u64* at(u32 p) const { return b[p & 1] + (u64)(p >> 1) * pair_stride; }
+};
+inline PolySeq seq_strided(const u64* base, u64 stride) {
+  PolySeq s;
+  s.b[0] = const_cast<u64*>(base);
+  s.b[1] = const_cast<u64*>(base) + stride;
+  s.pair_stride = 2 * stride;
+  return s;
+}
+inline PolySeq seq_pair(const u64* c0, const u64* c1, u64 op_stride) {
+  PolySeq s;
+  s.b[0] = const_cast<u64*>(c0);
+  s.b[1] = const_cast<u64*>(c1);
+  s.pair_stride = op_stride;
+  return s;
+}
+
 // base conversion: target j -> prime index and limb position in the output
 struct ConvMap {
   uint8_t prime[kMaxPrimes];

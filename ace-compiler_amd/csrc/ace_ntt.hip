@@ -240,13 +240,15 @@ __device__ __forceinline__ void inv_strided_stages(const A& ar, typename A::T* v
 
 // forward, strided pass: stages 0..LOGR-1.  grid = (N/R/256, n_limbs, n_polys)
 template <class A, int LOGR>
-__global__ __launch_bounds__(256) void ntt_fwd_strided(DevCtx c, u64* __restrict__ dst, const u64* __restrict__ src,
-                                                       LimbMap lm, LimbMap pos, u64 poly_stride) {
+__global__ __launch_bounds__(256) void ntt_fwd_strided(DevCtx c, PolySeq dsts, PolySeq srcs, LimbMap lm,
+                                                       LimbMap pos) {
   constexpr int R = 1 << LOGR;
   const u32 col = blockIdx.x * 256 + threadIdx.x;
   const u32 limb = blockIdx.y, pi = lm.prime[limb];
   const u64 rs = c.N >> LOGR;  // row stride
-  const u64 off = blockIdx.z * poly_stride + (u64)pos.prime[limb] * c.N + col;
+  const u64 off = (u64)pos.prime[limb] * c.N + col;
+  u64* __restrict__ dst = dsts.at(blockIdx.z);
+  const u64* __restrict__ src = srcs.at(blockIdx.z);
   A ar;
   ar.init(c, pi, false, nullptr, 0);
   typename A::T v[R];
@@ -298,8 +300,8 @@ constexpr bool kPrefetchTw = ACE_NTT_PREFETCH != 0;
 // forward, chunk pass: stages logr..logN-1 on 4096 contiguous words, in place.
 // grid = chunk_grid(n_limbs, ceil(n_polys / kPolysPerBlock))
 template <class A>
-__global__ __launch_bounds__(256) void ntt_fwd_chunk(DevCtx c, u64* __restrict__ data, LimbMap lm, LimbMap pos,
-                                                     u64 poly_stride, u32 logr, u32 n_limbs, u32 n_polys) {
+__global__ __launch_bounds__(256) void ntt_fwd_chunk(DevCtx c, PolySeq datas, LimbMap lm, LimbMap pos, u32 logr,
+                                                     u32 n_limbs, u32 n_polys) {
   typedef typename A::T T;
   __shared__ T lds[kChunk + kChunk / 16];
   const int t = threadIdx.x;
@@ -308,7 +310,8 @@ __global__ __launch_bounds__(256) void ntt_fwd_chunk(DevCtx c, u64* __restrict__
   const u32 poly0 = pblk * kPolysPerBlock;
   const u32 cnt = min((u32)kPolysPerBlock, n_polys - poly0);
   const u32 pi = lm.prime[limb];
-  u64* base = data + poly0 * poly_stride + (u64)pos.prime[limb] * c.N + (u64)chunk * kChunk;
+  const u64 loff = (u64)pos.prime[limb] * c.N + (u64)chunk * kChunk;
+  u64* base = datas.at(poly0) + loff;
   A ar;
   ar.init(c, pi, false, nullptr, 0);
   // twiddle index of local stage ls, local group 0 of this chunk: m + (chunk << ls)
@@ -329,10 +332,12 @@ __global__ __launch_bounds__(256) void ntt_fwd_chunk(DevCtx c, u64* __restrict__
     ar.template load_tw<4>((m0 << 10) + (chunk << 10) + (t << 2), twC2);
     ar.template load_tw<8>((m0 << 11) + (chunk << 11) + (t << 3), twC3);
   }
-  for (u32 it = 0; it < cnt; ++it, base += poly_stride) {
+  for (u32 it = 0; it < cnt; ++it) {
+    base = datas.at(poly0 + it) + loff;
     if (it + 1 < cnt) {
+      const u64* nb = datas.at(poly0 + it + 1) + loff;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) nxt[r] = base[poly_stride + t + 256 * r];
+      for (int r = 0; r < 16; ++r) nxt[r] = nb[t + 256 * r];
     }
     T v[16];
     // round A: element e = t + 256 r, local stages 0..3
@@ -398,9 +403,8 @@ __global__ __launch_bounds__(256) void ntt_fwd_chunk(DevCtx c, u64* __restrict__
 // by the strided pass that always follows.  At span 2^u the stage has
 // m = N >> (u+1) groups and element j belongs to group j >> (u+1).
 template <class A>
-__global__ __launch_bounds__(256) void ntt_inv_chunk(DevCtx c, u64* __restrict__ dst, const u64* __restrict__ src,
-                                                     LimbMap lm, LimbMap pos, u64 poly_stride, u32 n_limbs,
-                                                     u32 n_polys) {
+__global__ __launch_bounds__(256) void ntt_inv_chunk(DevCtx c, PolySeq dsts, PolySeq srcs, LimbMap lm, LimbMap pos,
+                                                     u32 n_limbs, u32 n_polys) {
   typedef typename A::T T;
   __shared__ T lds[kChunk + kChunk / 16];
   const int t = threadIdx.x;
@@ -409,14 +413,17 @@ __global__ __launch_bounds__(256) void ntt_inv_chunk(DevCtx c, u64* __restrict__
   const u32 poly0 = pblk * kPolysPerBlock;
   const u32 cnt = min((u32)kPolysPerBlock, n_polys - poly0);
   const u32 pi = lm.prime[limb];
-  u64 off = poly0 * poly_stride + (u64)pos.prime[limb] * c.N + (u64)chunk * kChunk;
+  const u64 off = (u64)pos.prime[limb] * c.N + (u64)chunk * kChunk;
   A ar;
   ar.init(c, pi, true, nullptr, 0);
   const u32 mh = c.N >> 1;  // groups at span 1
   const int hi = t >> 4, lo = t & 15;
   u64 raw[16], nxt[16];
+  {
+    const u64* src = srcs.at(poly0);
 #pragma unroll
-  for (int r = 0; r < 16; ++r) raw[r] = src[off + t + 256 * r];
+    for (int r = 0; r < 16; ++r) raw[r] = src[off + t + 256 * r];
+  }
   // per-thread twiddles of rounds C' and B' (round A' has wave-uniform ones)
   typename A::TWL twC0[8], twC1[4], twC2[2], twC3[1], twB0[8], twB1[4], twB2[2], twB3[1];
   if (kPrefetchTw) {
@@ -429,10 +436,12 @@ __global__ __launch_bounds__(256) void ntt_inv_chunk(DevCtx c, u64* __restrict__
     ar.template load_tw<2>((mh >> 6) + (chunk << 5) + (hi << 1), twB2);
     ar.template load_tw<1>((mh >> 7) + (chunk << 4) + (hi << 0), twB3);
   }
-  for (u32 it = 0; it < cnt; ++it, off += poly_stride) {
+  for (u32 it = 0; it < cnt; ++it) {
+    u64* dst = dsts.at(poly0 + it);
     if (it + 1 < cnt) {
+      const u64* src = srcs.at(poly0 + it + 1);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) nxt[r] = src[off + poly_stride + t + 256 * r];
+      for (int r = 0; r < 16; ++r) nxt[r] = src[off + t + 256 * r];
     }
     T v[16];
 #pragma unroll
@@ -499,14 +508,14 @@ __global__ __launch_bounds__(256) void ntt_inv_chunk(DevCtx c, u64* __restrict__
 // constant (default 1/N) and store canonical residues.  In place.
 // scale: nullptr, or (constant, Shoup companion) pairs indexed by sidx.prime[limb].
 template <class A, int LOGR>
-__global__ __launch_bounds__(256) void ntt_inv_strided(DevCtx c, u64* __restrict__ data, LimbMap lm, LimbMap pos,
-                                                       LimbMap sidx, u64 poly_stride,
-                                                       const u64* __restrict__ scale) {
+__global__ __launch_bounds__(256) void ntt_inv_strided(DevCtx c, PolySeq datas, LimbMap lm, LimbMap pos,
+                                                       LimbMap sidx, const u64* __restrict__ scale) {
   constexpr int R = 1 << LOGR;
   const u32 col = blockIdx.x * 256 + threadIdx.x;
   const u32 limb = blockIdx.y, pi = lm.prime[limb];
   const u64 rs = c.N >> LOGR;
-  const u64 off = blockIdx.z * poly_stride + (u64)pos.prime[limb] * c.N + col;
+  const u64 off = (u64)pos.prime[limb] * c.N + col;
+  u64* __restrict__ data = datas.at(blockIdx.z);
   A ar;
   ar.init(c, pi, true, scale, sidx.prime[limb]);
   typename A::T v[R];
@@ -520,12 +529,13 @@ __global__ __launch_bounds__(256) void ntt_inv_strided(DevCtx c, u64* __restrict
 // ---------------------------------------------------------------------------
 // N <= 4096: one workgroup per limb, the limb in LDS, one butterfly per
 // thread per step (integer back end).  grid = (1, n_limbs, n_polys)
-__global__ __launch_bounds__(256) void ntt_small(DevCtx c, u64* __restrict__ dst, const u64* __restrict__ src,
-                                                 LimbMap lm, LimbMap pos, u64 poly_stride, int inverse,
-                                                 const u64* __restrict__ scale) {
+__global__ __launch_bounds__(256) void ntt_small(DevCtx c, PolySeq dsts, PolySeq srcs, LimbMap lm, LimbMap pos,
+                                                 int inverse, const u64* __restrict__ scale) {
   __shared__ u64 a[kChunk];
   const u32 N = c.N, logN = c.logN, limb = blockIdx.y, pi = lm.prime[limb];
-  const u64 off = blockIdx.z * poly_stride + (u64)pos.prime[limb] * N;
+  const u64 off = (u64)pos.prime[limb] * N;
+  u64* __restrict__ dst = dsts.at(blockIdx.z);
+  const u64* __restrict__ src = srcs.at(blockIdx.z);
   ArithInt ar;
   ar.init(c, pi, inverse != 0, scale, limb);
   for (u32 i = threadIdx.x; i < N; i += 256) a[i] = src[off + i];
@@ -559,33 +569,31 @@ __global__ __launch_bounds__(256) void ntt_small(DevCtx c, u64* __restrict__ dst
 
 // ---------------------------------------------------------------------------
 template <class A, int LOGR>
-static void run_large(hipStream_t st, const DevCtx& c, u64* dst, const u64* src, const LimbMap& lm, const LimbMap& pos,
-                      const LimbMap& sidx, u32 n_limbs, u32 n_polys, u64 poly_stride, bool inverse,
+static void run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolySeq& src, const LimbMap& lm,
+                      const LimbMap& pos, const LimbMap& sidx, u32 n_limbs, u32 n_polys, bool inverse,
                       const u64* scale, int passes) {
   dim3 gs((c.N >> LOGR) / 256, n_limbs, n_polys), gc(chunk_grid(c, n_limbs, (n_polys + kPolysPerBlock - 1) / kPolysPerBlock));
   if (!inverse) {
     if (passes & 1)
-      hipLaunchKernelGGL((ntt_fwd_strided<A, LOGR>), gs, dim3(256), 0, st, c, dst, src, lm, pos, poly_stride);
+      hipLaunchKernelGGL((ntt_fwd_strided<A, LOGR>), gs, dim3(256), 0, st, c, dst, src, lm, pos);
     if (passes & 2)
-      hipLaunchKernelGGL((ntt_fwd_chunk<A>), gc, dim3(256), 0, st, c, dst, lm, pos, poly_stride, (u32)LOGR, n_limbs,
-                         n_polys);
+      hipLaunchKernelGGL((ntt_fwd_chunk<A>), gc, dim3(256), 0, st, c, dst, lm, pos, (u32)LOGR, n_limbs, n_polys);
   } else {
     if (passes & 1)
-      hipLaunchKernelGGL((ntt_inv_chunk<A>), gc, dim3(256), 0, st, c, dst, src, lm, pos, poly_stride, n_limbs,
-                         n_polys);
+      hipLaunchKernelGGL((ntt_inv_chunk<A>), gc, dim3(256), 0, st, c, dst, src, lm, pos, n_limbs, n_polys);
     if (passes & 2)
-      hipLaunchKernelGGL((ntt_inv_strided<A, LOGR>), gs, dim3(256), 0, st, c, dst, lm, pos, sidx, poly_stride, scale);
+      hipLaunchKernelGGL((ntt_inv_strided<A, LOGR>), gs, dim3(256), 0, st, c, dst, lm, pos, sidx, scale);
   }
 }
 
 template <class A>
-static bool run_large_dispatch(hipStream_t st, const DevCtx& c, u64* dst, const u64* src, const LimbMap& lm,
-                               const LimbMap& pos, const LimbMap& sidx, u32 n_limbs, u32 n_polys, u64 poly_stride,
+static bool run_large_dispatch(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolySeq& src,
+                               const LimbMap& lm, const LimbMap& pos, const LimbMap& sidx, u32 n_limbs, u32 n_polys,
                                bool inverse, const u64* scale, int passes) {
   switch (c.logN - kLogChunk) {
 #define ACE_NTT_CASE(LR)                                                                                         \
   case LR:                                                                                                       \
-    run_large<A, LR>(st, c, dst, src, lm, pos, sidx, n_limbs, n_polys, poly_stride, inverse, scale, passes);      \
+    run_large<A, LR>(st, c, dst, src, lm, pos, sidx, n_limbs, n_polys, inverse, scale, passes);                   \
     return true;
     ACE_NTT_CASE(1)
     ACE_NTT_CASE(2)
@@ -598,16 +606,16 @@ static bool run_large_dispatch(hipStream_t st, const DevCtx& c, u64* dst, const 
   }
 }
 
-bool launch_ntt(hipStream_t st, const DevCtx& c, u64* dst, const u64* src, const LimbMap& lm, const LimbMap* pos_in,
-                u32 n_limbs, u32 n_polys, u64 poly_stride, bool inverse, const u64* scale, int passes) {
+bool launch_ntt(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolySeq& src, const LimbMap& lm,
+                const LimbMap* pos_in, u32 n_limbs, u32 n_polys, bool inverse, const u64* scale, int passes) {
   if (n_limbs == 0 || n_polys == 0) return true;
   LimbMap pos{};
   if (pos_in) pos = *pos_in;
   else
     for (u32 t = 0; t < n_limbs; ++t) pos.prime[t] = (uint8_t)t;
   if (c.logN <= kLogChunk) {
-    hipLaunchKernelGGL(ntt_small, dim3(1, n_limbs, n_polys), dim3(256), 0, st, c, dst, src, lm, pos, poly_stride,
-                       inverse ? 1 : 0, scale);
+    hipLaunchKernelGGL(ntt_small, dim3(1, n_limbs, n_polys), dim3(256), 0, st, c, dst, src, lm, pos, inverse ? 1 : 0,
+                       scale);
     return true;
   }
   if (c.logN - kLogChunk > 5) return false;
@@ -623,11 +631,11 @@ bool launch_ntt(hipStream_t st, const DevCtx& c, u64* dst, const u64* src, const
   }
   bool ok = true;
   if (cnt[0])
-    ok &= run_large_dispatch<ArithInt>(st, c, dst, src, lm_g[0], pos_g[0], sidx_g[0], cnt[0], n_polys, poly_stride,
-                                       inverse, scale, passes);
+    ok &= run_large_dispatch<ArithInt>(st, c, dst, src, lm_g[0], pos_g[0], sidx_g[0], cnt[0], n_polys, inverse,
+                                       scale, passes);
   if (cnt[1])
-    ok &= run_large_dispatch<ArithFp>(st, c, dst, src, lm_g[1], pos_g[1], sidx_g[1], cnt[1], n_polys, poly_stride,
-                                      inverse, scale, passes);
+    ok &= run_large_dispatch<ArithFp>(st, c, dst, src, lm_g[1], pos_g[1], sidx_g[1], cnt[1], n_polys, inverse,
+                                      scale, passes);
   return ok;
 }
 

@@ -56,12 +56,18 @@ void launch_ew(hipStream_t st, const DevCtx& c, EwOp op, u64* r, const u64* a, c
 }
 
 // ---- Hw_rotate / Automorphism_transform (hal.c:123-138, rns_poly.c:1056-1099)
+// blockIdx.z = rotation: its own index table, input pair and output pair.
 __global__ __launch_bounds__(kThreads) void gather_kernel(DevCtx c, u64* __restrict__ r0, u64* __restrict__ r1,
-                                                          const u64* __restrict__ a0, const u64* __restrict__ a1,
-                                                          const i64* __restrict__ order, LimbMap lm, u64 n) {
-  const u32 limb = blockIdx.y;
+                                                          u64 r_stride, const u64* __restrict__ a0,
+                                                          const u64* __restrict__ a1, u64 a_stride, OrderSet orders,
+                                                          LimbMap lm, u64 n) {
+  const u32 limb = blockIdx.y, z = blockIdx.z;
   const u64 q = c.primes[lm.prime[limb]].q;
   const u64 base = (u64)limb * n;
+  const i64* __restrict__ order = orders.p[orders.n == 1 ? 0 : z];
+  r0 += z * r_stride;
+  a0 += z * a_stride;
+  if (r1) { r1 += z * r_stride; a1 += z * a_stride; }
 #pragma unroll
   ACE_EW_LOOP(i, n) {
     i64 k = order[i];
@@ -78,23 +84,31 @@ __global__ __launch_bounds__(kThreads) void gather_kernel(DevCtx c, u64* __restr
 void launch_gather(hipStream_t st, const DevCtx& c, u64* r, const u64* a, const i64* order, const LimbMap& lm,
                    u32 n_limbs, u64 n) {
   if (!n || !n_limbs) return;
-  hipLaunchKernelGGL(gather_kernel, ew_grid(n, n_limbs), dim3(kThreads), 0, st, c, r, (u64*)nullptr, a,
-                     (const u64*)nullptr, order, lm, n);
+  OrderSet os{};
+  os.n = 1;
+  os.p[0] = order;
+  hipLaunchKernelGGL(gather_kernel, ew_grid(n, n_limbs), dim3(kThreads), 0, st, c, r, (u64*)nullptr, (u64)0, a,
+                     (const u64*)nullptr, (u64)0, os, lm, n);
 }
-void launch_gather2(hipStream_t st, const DevCtx& c, u64* r0, u64* r1, const u64* a0, const u64* a1,
-                    const i64* order, const LimbMap& lm, u32 n_limbs, u64 n) {
-  if (!n || !n_limbs) return;
-  hipLaunchKernelGGL(gather_kernel, ew_grid(n, n_limbs), dim3(kThreads), 0, st, c, r0, r1, a0, a1, order, lm, n);
+void launch_gather2(hipStream_t st, const DevCtx& c, u64* r0, u64* r1, u64 r_stride, const u64* a0, const u64* a1,
+                    u64 a_stride, const OrderSet& orders, const LimbMap& lm, u32 n_limbs, u32 n_rot) {
+  if (!n_limbs || !n_rot) return;
+  hipLaunchKernelGGL(gather_kernel, ew_grid(c.N, n_limbs, n_rot), dim3(kThreads), 0, st, c, r0, r1, r_stride, a0, a1,
+                     a_stride, orders, lm, (u64)c.N);
 }
 
 // ---- Mul_ciphertext3 (evaluator.c:142-175) in one pass -------------------
 __global__ __launch_bounds__(kThreads) void tensor_kernel(DevCtx c, u64* __restrict__ d0, u64* __restrict__ d1,
                                                           u64* __restrict__ d2, const u64* __restrict__ a0,
                                                           const u64* __restrict__ a1, const u64* __restrict__ b0,
-                                                          const u64* __restrict__ b1, LimbMap lm) {
+                                                          const u64* __restrict__ b1, LimbMap lm, u64 d01_stride,
+                                                          u64 d2_stride, u64 in_stride) {
   const u32 limb = blockIdx.y;
   const DevPrime P = c.primes[lm.prime[limb]];
   const u64 n = c.N, base = (u64)limb * n;
+  d0 += blockIdx.z * d01_stride; d1 += blockIdx.z * d01_stride; d2 += blockIdx.z * d2_stride;
+  a0 += blockIdx.z * in_stride; a1 += blockIdx.z * in_stride;
+  b0 += blockIdx.z * in_stride; b1 += blockIdx.z * in_stride;
 #pragma unroll
   ACE_EW_LOOP(i, n) {
     u64 x0 = a0[base + i], x1 = a1[base + i], y0 = b0[base + i], y1 = b1[base + i];
@@ -105,24 +119,34 @@ __global__ __launch_bounds__(kThreads) void tensor_kernel(DevCtx c, u64* __restr
 }
 
 void launch_tensor(hipStream_t st, const DevCtx& c, u64* d0, u64* d1, u64* d2, const u64* a0, const u64* a1,
-                   const u64* b0, const u64* b1, const LimbMap& lm, u32 n_limbs) {
-  if (!n_limbs) return;
-  hipLaunchKernelGGL(tensor_kernel, ew_grid(c.N, n_limbs), dim3(kThreads), 0, st, c, d0, d1, d2, a0, a1, b0, b1, lm);
+                   const u64* b0, const u64* b1, const LimbMap& lm, u32 n_limbs, u32 n_ops, u64 d01_stride,
+                   u64 d2_stride, u64 in_stride) {
+  if (!n_limbs || !n_ops) return;
+  hipLaunchKernelGGL(tensor_kernel, ew_grid(c.N, n_limbs, n_ops), dim3(kThreads), 0, st, c, d0, d1, d2, a0, a1, b0,
+                     b1, lm, d01_stride, d2_stride, in_stride);
 }
 
 // ---- fast base conversion (rns_poly.c:218-242, rns_poly_impl.c:324-336) ----
 // One thread per coefficient and kConvTargets targets; the nd source words
 // stay in registers, the cofactor table is read through wave-uniform loads.
+// blockIdx.z enumerates (operand, job): a job is one digit's conversion, all
+// jobs of a launch share the operand strides.
 constexpr int kConvTargets = 4;
 constexpr int kConvMaxSrc = 16;
 
-__global__ __launch_bounds__(kThreads) void baseconv_kernel(DevCtx c, u64* __restrict__ out,
-                                                            const u64* __restrict__ t, const u64* __restrict__ hat,
-                                                            u32 hat_stride, u32 nd, u32 nc, ConvMap map) {
+__global__ __launch_bounds__(kThreads) void baseconv_kernel(DevCtx c, u64* __restrict__ out_base,
+                                                            const u64* __restrict__ t_base, ConvBatch b) {
   const u64 n = c.N;
   const u64 i = (u64)blockIdx.x * kThreads + threadIdx.x;
   if (i >= n) return;
+  const u32 jobi = blockIdx.z % b.n_jobs, op = blockIdx.z / b.n_jobs;
+  const ConvJob& J = b.job[jobi];
+  const u32 nd = J.nd, nc = J.nc, hat_stride = J.hat_stride;
+  const u64* __restrict__ hat = J.hat;
+  const u64* __restrict__ t = t_base + op * b.t_stride + J.t_off;
+  u64* __restrict__ out = out_base + op * b.out_stride + J.out_off;
   const u32 j0 = blockIdx.y * kConvTargets;
+  if (j0 >= nc) return;
   if (nd <= kConvMaxSrc) {
     u64 x[kConvMaxSrc];
 #pragma unroll
@@ -135,28 +159,51 @@ __global__ __launch_bounds__(kThreads) void baseconv_kernel(DevCtx c, u64* __res
 #pragma unroll
       for (int k = 0; k < kConvMaxSrc; ++k)
         if ((u32)k < nd) mac128(hi, lo, x[k], hat[(u64)k * hat_stride + j]);
-      out[(u64)map.out_limb[j] * n + i] = barrett128(hi, lo, c.primes[map.prime[j]]);
+      out[(u64)J.map.out_limb[j] * n + i] = barrett128(hi, lo, c.primes[J.map.prime[j]]);
     }
   } else {
     for (int jj = 0; jj < kConvTargets; ++jj) {
       u32 j = j0 + jj;
       if (j >= nc) break;
-      const DevPrime P = c.primes[map.prime[j]];
+      const DevPrime P = c.primes[J.map.prime[j]];
       u64 hi = 0, lo = 0;
       for (u32 k = 0; k < nd; ++k) {
         mac128(hi, lo, t[(u64)k * n + i], hat[(u64)k * hat_stride + j]);
         if ((k & 7) == 7) { lo = barrett128(hi, lo, P); hi = 0; }  // keep the sum below 2^128
       }
-      out[(u64)map.out_limb[j] * n + i] = barrett128(hi, lo, P);
+      out[(u64)J.map.out_limb[j] * n + i] = barrett128(hi, lo, P);
     }
   }
 }
 
-void launch_baseconv(hipStream_t st, const DevCtx& c, u64* out, const u64* t, const u64* hat, u32 hat_stride,
-                     u32 nd, u32 nc, const ConvMap& map) {
-  if (!nd || !nc) return;
-  dim3 g((c.N + kThreads - 1) / kThreads, (nc + kConvTargets - 1) / kConvTargets);
-  hipLaunchKernelGGL(baseconv_kernel, g, dim3(kThreads), 0, st, c, out, t, hat, hat_stride, nd, nc, map);
+void launch_baseconv(hipStream_t st, const DevCtx& c, u64* out, const u64* t, const ConvBatch& b, u32 n_ops) {
+  if (!b.n_jobs || !n_ops) return;
+  u32 max_nc = 0;
+  for (u32 k = 0; k < b.n_jobs; ++k) max_nc = b.job[k].nc > max_nc ? b.job[k].nc : max_nc;
+  if (!max_nc) return;
+  dim3 g((c.N + kThreads - 1) / kThreads, (max_nc + kConvTargets - 1) / kConvTargets, b.n_jobs * n_ops);
+  hipLaunchKernelGGL(baseconv_kernel, g, dim3(kThreads), 0, st, c, out, t, b);
+}
+
+// copies the digit limbs of `src` (level limbs per operand) into their places
+// in the raised polynomials: limb t of digit d = t / part_size goes to
+// res + op*res_stride + d*digit_stride + t*N  (Decomp, rns_poly.c:74-105)
+__global__ __launch_bounds__(kThreads) void digit_copy_kernel(u64* __restrict__ res, const u64* __restrict__ src,
+                                                              u64 n, u32 part_size, u32 n_digits, u64 digit_stride,
+                                                              u64 res_stride, u64 src_stride) {
+  const u32 limb = blockIdx.y, op = blockIdx.z;
+  u32 d = limb / part_size;
+  if (d >= n_digits) d = n_digits - 1;
+  const u64* __restrict__ s = src + op * src_stride + (u64)limb * n;
+  u64* __restrict__ r = res + op * res_stride + d * digit_stride + (u64)limb * n;
+#pragma unroll
+  ACE_EW_LOOP(i, n) r[i] = s[i];
+}
+void launch_digit_copy(hipStream_t st, const DevCtx& c, u64* res, const u64* src, u32 level, u32 part_size,
+                       u32 n_digits, u64 digit_stride, u64 res_stride, u64 src_stride, u32 n_ops) {
+  if (!level || !n_ops) return;
+  hipLaunchKernelGGL(digit_copy_kernel, ew_grid(c.N, level, n_ops), dim3(kThreads), 0, st, res, src, (u64)c.N,
+                     part_size, n_digits, digit_stride, res_stride, src_stride);
 }
 
 // ---- Dot_prod (rns_poly.c:502-529, rns_poly_impl.c:102-162) ----------------
@@ -166,12 +213,18 @@ void launch_baseconv(hipStream_t st, const DevCtx& c, u64* out, const u64* t, co
 // multiply-reduce-add chain because canonical residues are unique.
 template <bool TWO>
 __global__ __launch_bounds__(kThreads) void dotprod_kernel(DevCtx c, u64* __restrict__ out0, u64* __restrict__ out1,
-                                                           const u64* __restrict__ digits, u64 digit_stride,
-                                                           const u64* __restrict__ key0, const u64* __restrict__ key1,
-                                                           u64 key_stride, u32 n_parts, LimbMap lm, LimbMap key_limb) {
-  const u32 limb = blockIdx.y;
+                                                           u64 out_stride, const u64* __restrict__ digits,
+                                                           u64 digit_stride, u64 digits_op_stride, KeySet keys,
+                                                           u64 key1_off, u64 key_stride, u32 n_parts, LimbMap lm,
+                                                           LimbMap key_limb) {
+  const u32 limb = blockIdx.y, op = blockIdx.z;
   const DevPrime P = c.primes[lm.prime[limb]];
   const u64 n = c.N, dbase = (u64)limb * n, kbase = (u64)key_limb.prime[limb] * n;
+  const u64* __restrict__ key0 = keys.p[keys.n == 1 ? 0 : op];
+  const u64* __restrict__ key1 = key0 + key1_off;
+  digits += op * digits_op_stride;
+  out0 += op * out_stride;
+  if (TWO) out1 += op * out_stride;
 #pragma unroll
   ACE_EW_LOOP(i, n) {
     u64 h0 = 0, l0 = 0, h1 = 0, l1 = 0;
@@ -189,29 +242,34 @@ __global__ __launch_bounds__(kThreads) void dotprod_kernel(DevCtx c, u64* __rest
   }
 }
 
-void launch_dotprod(hipStream_t st, const DevCtx& c, u64* out0, u64* out1, const u64* digits, u64 digit_stride,
-                    const u64* key0, const u64* key1, u64 key_stride, u32 n_parts, const LimbMap& lm,
-                    const LimbMap& key_limb, u32 n_limbs) {
-  if (!n_limbs) return;
-  dim3 g = ew_grid(c.N, n_limbs);
+void launch_dotprod(hipStream_t st, const DevCtx& c, u64* out0, u64* out1, u64 out_stride, const u64* digits,
+                    u64 digit_stride, u64 digits_op_stride, const KeySet& keys, u64 key1_off, u64 key_stride,
+                    u32 n_parts, const LimbMap& lm, const LimbMap& key_limb, u32 n_limbs, u32 n_ops) {
+  if (!n_limbs || !n_ops) return;
+  dim3 g = ew_grid(c.N, n_limbs, n_ops);
   if (out1)
-    hipLaunchKernelGGL(dotprod_kernel<true>, g, dim3(kThreads), 0, st, c, out0, out1, digits, digit_stride, key0,
-                       key1, key_stride, n_parts, lm, key_limb);
+    hipLaunchKernelGGL(dotprod_kernel<true>, g, dim3(kThreads), 0, st, c, out0, out1, out_stride, digits,
+                       digit_stride, digits_op_stride, keys, key1_off, key_stride, n_parts, lm, key_limb);
   else
-    hipLaunchKernelGGL(dotprod_kernel<false>, g, dim3(kThreads), 0, st, c, out0, out1, digits, digit_stride, key0,
-                       key1, key_stride, n_parts, lm, key_limb);
+    hipLaunchKernelGGL(dotprod_kernel<false>, g, dim3(kThreads), 0, st, c, out0, out1, out_stride, digits,
+                       digit_stride, digits_op_stride, keys, key1_off, key_stride, n_parts, lm, key_limb);
 }
 
 // ---- Mod_down tail (rns_poly.c:292-303): (src - y) * P^-1 [+ addend] --------
-__global__ __launch_bounds__(kThreads) void moddown_tail_kernel(DevCtx c, u64* __restrict__ out,
-                                                                const u64* __restrict__ src,
-                                                                const u64* __restrict__ y,
-                                                                const u64* __restrict__ addend,
+// blockIdx.z = polynomial; src/out/addend are addressed as PolySeq.
+__global__ __launch_bounds__(kThreads) void moddown_tail_kernel(DevCtx c, PolySeq outs, PolySeq srcs,
+                                                                const u64* __restrict__ y_base, u64 y_stride,
+                                                                PolySeq addends, int addend_mode,
                                                                 const u64* __restrict__ cst, LimbMap lm) {
-  const u32 limb = blockIdx.y;
+  const u32 limb = blockIdx.y, p = blockIdx.z;
   const u64 q = c.primes[lm.prime[limb]].q;
   const u64 w = cst[2 * limb], wp = cst[2 * limb + 1];
   const u64 n = c.N, base = (u64)limb * n;
+  u64* out = outs.at(p);  // may be the addend itself (in-place relinearisation): no restrict
+  const u64* __restrict__ src = srcs.at(p);
+  const u64* __restrict__ y = y_base + p * y_stride;
+  // addend_mode: 0 none, 1 every polynomial, 2 even polynomials only
+  const u64* addend = (addend_mode == 1 || (addend_mode == 2 && !(p & 1))) ? addends.at(p) : nullptr;
 #pragma unroll
   ACE_EW_LOOP(i, n) {
     u64 v = shoup_mul(sub_mod(src[base + i], y[base + i], q), w, wp, q);
@@ -220,24 +278,29 @@ __global__ __launch_bounds__(kThreads) void moddown_tail_kernel(DevCtx c, u64* _
   }
 }
 
-void launch_moddown_tail(hipStream_t st, const DevCtx& c, u64* out, const u64* src, const u64* y,
-                         const u64* addend, const u64* cst, const LimbMap& lm, u32 n_limbs) {
-  if (!n_limbs) return;
-  hipLaunchKernelGGL(moddown_tail_kernel, ew_grid(c.N, n_limbs), dim3(kThreads), 0, st, c, out, src, y, addend, cst,
-                     lm);
+void launch_moddown_tail(hipStream_t st, const DevCtx& c, const PolySeq& out, const PolySeq& src, const u64* y,
+                         u64 y_stride, const PolySeq* addend, int addend_mode, const u64* cst, const LimbMap& lm,
+                         u32 n_limbs, u32 n_polys) {
+  if (!n_limbs || !n_polys) return;
+  PolySeq ad = addend ? *addend : out;
+  hipLaunchKernelGGL(moddown_tail_kernel, ew_grid(c.N, n_limbs, n_polys), dim3(kThreads), 0, st, c, out, src, y,
+                     y_stride, ad, addend ? addend_mode : 0, cst, lm);
 }
 
 // ---- Rescale (rns_poly.c:310-404) ------------------------------------------
 // Switch_modulus (include/util/modular.h:296-322): centred lift q_l -> q_t.
 // cst per limb: K, K' (Shoup), diff = q_t - (q_l mod q_t)
-__global__ __launch_bounds__(kThreads) void rescale_switch_kernel(DevCtx c, u64* __restrict__ u,
-                                                                  const u64* __restrict__ last, u32 last_prime,
-                                                                  const u64* __restrict__ cst, LimbMap lm) {
-  const u32 limb = blockIdx.y;
+__global__ __launch_bounds__(kThreads) void rescale_switch_kernel(DevCtx c, u64* __restrict__ u_base, u64 u_stride,
+                                                                  const u64* __restrict__ last_base, u64 last_stride,
+                                                                  u32 last_prime, const u64* __restrict__ cst,
+                                                                  LimbMap lm) {
+  const u32 limb = blockIdx.y, p = blockIdx.z;
   const DevPrime P = c.primes[lm.prime[limb]];
   const u64 ql = c.primes[last_prime].q, half = ql >> 1;
   const u64 K = cst[3 * limb], Kp = cst[3 * limb + 1], diff = cst[3 * limb + 2];
   const u64 n = c.N, base = (u64)limb * n;
+  u64* __restrict__ u = u_base + p * u_stride;
+  const u64* __restrict__ last = last_base + p * last_stride;
 #pragma unroll
   ACE_EW_LOOP(i, n) {
     u64 v = last[i];
@@ -250,28 +313,31 @@ __global__ __launch_bounds__(kThreads) void rescale_switch_kernel(DevCtx c, u64*
     u[base + i] = shoup_mul(v, K, Kp, P.q);
   }
 }
-void launch_rescale_switch(hipStream_t st, const DevCtx& c, u64* u, const u64* last, u32 last_prime,
-                           const u64* cst, const LimbMap& lm, u32 n_limbs) {
-  if (!n_limbs) return;
-  hipLaunchKernelGGL(rescale_switch_kernel, ew_grid(c.N, n_limbs), dim3(kThreads), 0, st, c, u, last, last_prime,
-                     cst, lm);
+void launch_rescale_switch(hipStream_t st, const DevCtx& c, u64* u, u64 u_stride, const u64* last, u64 last_stride,
+                           u32 last_prime, const u64* cst, const LimbMap& lm, u32 n_limbs, u32 n_polys) {
+  if (!n_limbs || !n_polys) return;
+  hipLaunchKernelGGL(rescale_switch_kernel, ew_grid(c.N, n_limbs, n_polys), dim3(kThreads), 0, st, c, u, u_stride,
+                     last, last_stride, last_prime, cst, lm);
 }
 
-__global__ __launch_bounds__(kThreads) void rescale_tail_kernel(DevCtx c, u64* __restrict__ out,
-                                                                const u64* __restrict__ src,
-                                                                const u64* __restrict__ u,
+__global__ __launch_bounds__(kThreads) void rescale_tail_kernel(DevCtx c, PolySeq outs, PolySeq srcs,
+                                                                const u64* __restrict__ u_base, u64 u_stride,
                                                                 const u64* __restrict__ cst, LimbMap lm) {
-  const u32 limb = blockIdx.y;
+  const u32 limb = blockIdx.y, p = blockIdx.z;
   const u64 q = c.primes[lm.prime[limb]].q;
   const u64 w = cst[2 * limb], wp = cst[2 * limb + 1];
   const u64 n = c.N, base = (u64)limb * n;
+  u64* __restrict__ out = outs.at(p);
+  const u64* __restrict__ src = srcs.at(p);
+  const u64* __restrict__ u = u_base + p * u_stride;
 #pragma unroll
   ACE_EW_LOOP(i, n) out[base + i] = add_mod(shoup_mul(src[base + i], w, wp, q), u[base + i], q);
 }
-void launch_rescale_tail(hipStream_t st, const DevCtx& c, u64* out, const u64* src, const u64* u, const u64* cst,
-                         const LimbMap& lm, u32 n_limbs) {
-  if (!n_limbs) return;
-  hipLaunchKernelGGL(rescale_tail_kernel, ew_grid(c.N, n_limbs), dim3(kThreads), 0, st, c, out, src, u, cst, lm);
+void launch_rescale_tail(hipStream_t st, const DevCtx& c, const PolySeq& out, const PolySeq& src, const u64* u,
+                         u64 u_stride, const u64* cst, const LimbMap& lm, u32 n_limbs, u32 n_polys) {
+  if (!n_limbs || !n_polys) return;
+  hipLaunchKernelGGL(rescale_tail_kernel, ew_grid(c.N, n_limbs, n_polys), dim3(kThreads), 0, st, c, out, src, u,
+                     u_stride, cst, lm);
 }
 
 // coefficient form (rns_poly.c:380-400): plain residue of the last limb
@@ -293,6 +359,19 @@ void launch_rescale_coef(hipStream_t st, const DevCtx& c, u64* out, const u64* s
                          const u64* cst, const LimbMap& lm, u32 n_limbs) {
   if (!n_limbs) return;
   hipLaunchKernelGGL(rescale_coef_kernel, ew_grid(c.N, n_limbs), dim3(kThreads), 0, st, c, out, src, last, cst, lm);
+}
+
+// gathers limb `limb` of every polynomial of a sequence into a dense buffer
+__global__ __launch_bounds__(kThreads) void pick_limb_kernel(u64* __restrict__ dst, PolySeq srcs, u64 n, u32 limb) {
+  const u32 p = blockIdx.z;
+  const u64* __restrict__ s = srcs.at(p) + (u64)limb * n;
+  u64* __restrict__ d = dst + (u64)p * n;
+#pragma unroll
+  ACE_EW_LOOP(i, n) d[i] = s[i];
+}
+void launch_pick_limb(hipStream_t st, const DevCtx& c, u64* dst, const PolySeq& src, u32 limb, u32 n_polys) {
+  if (!n_polys) return;
+  hipLaunchKernelGGL(pick_limb_kernel, ew_grid(c.N, 1, n_polys), dim3(kThreads), 0, st, dst, src, (u64)c.N, limb);
 }
 
 // ---- multiply every limb by its own constant (Extend, rns_poly.c:483-500) ---

@@ -69,6 +69,66 @@ def cpu_baseline(x_host, idx, budget_s):
                       "%.1f s, single thread, gcc -O3" % (done, LIMBS, POLYS, dt)}
 
 
+def extra_legs(g, np, seeded):
+    """HMult+relinearise+rescale pairs/s and hoisted rotations/s at l=24, k=7, dnum=3."""
+    extra = {}
+    level, T = g.L, g.L + g.K
+    kwords = 2 * g.parts * T * N
+    log("key-switch leg: 16 ciphertext pairs, one relinearisation key")
+    swk = g.upload(np.concatenate([seeded.uniform_poly(2000 + i, g.primes, N) for i in range(2 * g.parts)]))
+    cts = [g.upload(seeded.uniform_poly(3000 + i, g.primes[:level], N)) for i in range(4)]
+    pairs = 16
+    # 16 distinct ciphertext pairs derived on the device from the seeded one: operand p = operand 0 + p per limb
+    stride = level * N
+    ops = [g.alloc(pairs * stride) for _ in range(4)]
+    for k in range(4):
+        for p in range(pairs):
+            for t in range(level):
+                g.hw("modadd_scalar", ops[k].view(p * stride + t * N, N), cts[k].view(t * N, N), p, t)
+    ostride = (level - 1) * N
+    r0, r1 = g.alloc(pairs * ostride), g.alloc(pairs * ostride)
+
+    def hmult_batch():
+        g.mul_relin_rescale_batch(r0, r1, ostride, ops[0], ops[1], ops[2], ops[3], stride, swk, level, pairs)
+
+    hmult_batch()
+    ms = time_region(g, hmult_batch, 5)
+    extra["keyswitch_ops_per_s"] = round(pairs / (ms * 1e-3), 1)
+    extra["hmult_relin_rescale_ms"] = round(ms / pairs, 4)
+    # 172 MB compulsory traffic per op (96 input + 186 key + 46 output limbs of 512 KiB)
+    extra["keyswitch_hbm_frac"] = round(328 * N * 8 * pairs / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+
+    def hmult_single():
+        g.mul_relin_rescale(r0, r1, cts[0], cts[1], cts[2], cts[3], swk, level)
+
+    hmult_single()
+    extra["hmult_relin_rescale_single_ms"] = round(time_region(g, hmult_single, 10), 4)
+    for b in ops:
+        b.free()
+
+    nrot = 32
+    log("rotation leg: %d rotations of one ciphertext, hoisted ModUp" % nrot)
+    rots = [1 << i for i in range(15)] + [-1] + [int(v) for v in 1 + seeded.splitmix64(7, 16) % np.uint64(N // 2 - 1)]
+    keys, orders = [], []
+    for i, r in enumerate(rots):
+        kbuf = g.alloc(kwords)
+        # distinct keys derived on the device from the seeded one: key_i = key_0 + (i+1) per limb
+        for d in range(2 * g.parts):
+            for t in range(T):
+                off = (d * T + t) * N
+                g.hw("modadd_scalar", kbuf.view(off, N), swk.view(off, N), i + 1, t)
+        keys.append(kbuf)
+        orders.append(g.automorphism_order(g.find_automorphism_index(r), True))
+    s0, s1 = g.alloc(nrot * level * N), g.alloc(nrot * level * N)
+    f = lambda: g.rotate_batch(s0, s1, cts[0], cts[1], keys, orders, level)
+    f()
+    ms = time_region(g, f, 5)
+    extra["rotations_per_s"] = round(nrot / (ms * 1e-3), 1)
+    extra["rotate_batch_ms"] = round(ms, 3)
+    extra["rotation_hbm_frac"] = round(327 * N * 8 * nrot / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+    return extra
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -76,6 +136,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="time budget of the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the key-switch / rotation measurements")
+    ap.add_argument("--only-extra", action="store_true",
+                    help="profiling aid: run only the key-switch and rotation legs (prints their fields alone)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU; this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
@@ -101,6 +163,8 @@ def main():
         g.ntt(x, x, idx, n_polys=POLYS, poly_stride_limbs=LIMBS)
         g.intt(x, x, idx, n_polys=POLYS, poly_stride_limbs=LIMBS)
 
+    if args.only_extra:
+        args.warmup, args.steps = 0, 1
     for _ in range(args.warmup):
         step()
     g.sync()
@@ -118,6 +182,9 @@ def main():
 
     # per-kernel timing of the four NTT kernels (each reads and writes every coefficient once)
     kern = {}
+    if args.only_extra:
+        print(json.dumps(extra_legs(g, np, seeded)))
+        return
     scratch = g.alloc(POLYS * per_poly)
     pass_bytes = POLYS * per_poly * 16
     # a plain device copy of the whole batch: the known-size kernel against which the
@@ -137,47 +204,7 @@ def main():
                 "bytes_per_launch": pass_bytes, "all_ntt_kernels": kern}
     scratch.free()
 
-    extra = {}
-    if not args.no_extra:
-        level, T = g.L, g.L + g.K
-        kwords = 2 * g.parts * T * N
-        log("key-switch leg: 16 ciphertext pairs, one relinearisation key")
-        swk = g.upload(np.concatenate([seeded.uniform_poly(2000 + i, g.primes, N) for i in range(2 * g.parts)]))
-        cts = [g.upload(seeded.uniform_poly(3000 + i, g.primes[:level], N)) for i in range(4)]
-        r0, r1 = g.alloc((level - 1) * N), g.alloc((level - 1) * N)
-        pairs = 16
-
-        def hmult_batch():
-            for p in range(pairs):
-                g.mul_relin_rescale(r0, r1, cts[0], cts[1], cts[2], cts[3], swk, level)
-
-        hmult_batch()
-        ms = time_region(g, hmult_batch, 3)
-        extra["keyswitch_ops_per_s"] = round(pairs / (ms * 1e-3), 1)
-        extra["hmult_relin_rescale_ms"] = round(ms / pairs, 4)
-        # 172 MB compulsory traffic per op (96 input + 186 key + 46 output limbs of 512 KiB)
-        extra["keyswitch_hbm_frac"] = round(328 * N * 8 * pairs / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
-
-        nrot = 32
-        log("rotation leg: %d rotations of one ciphertext, hoisted ModUp" % nrot)
-        rots = [1 << i for i in range(15)] + [-1] + [int(v) for v in 1 + seeded.splitmix64(7, 16) % np.uint64(N // 2 - 1)]
-        keys, orders = [], []
-        for i, r in enumerate(rots):
-            kbuf = g.alloc(kwords)
-            # distinct keys derived on the device from the seeded one: key_i = key_0 + (i+1) per limb
-            for d in range(2 * g.parts):
-                for t in range(T):
-                    off = (d * T + t) * N
-                    g.hw("modadd_scalar", kbuf.view(off, N), swk.view(off, N), i + 1, t)
-            keys.append(kbuf)
-            orders.append(g.automorphism_order(g.find_automorphism_index(r), True))
-        s0, s1 = g.alloc(nrot * level * N), g.alloc(nrot * level * N)
-        f = lambda: g.rotate_batch(s0, s1, cts[0], cts[1], keys, orders, level)
-        f()
-        ms = time_region(g, f, 3)
-        extra["rotations_per_s"] = round(nrot / (ms * 1e-3), 1)
-        extra["rotate_batch_ms"] = round(ms, 3)
-        extra["rotation_hbm_frac"] = round(327 * N * 8 * nrot / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+    extra = {} if args.no_extra else extra_legs(g, np, seeded)
 
     cpu = cpu_baseline(x_host, idx, args.cpu_seconds) if args.cpu_seconds > 0 else None
 

@@ -168,6 +168,12 @@ int ace_rescale_ciph(ace_ctx* ctx, int64_t* r0, int64_t* r1, const int64_t* c0, 
 /* Mul_ciphertext + Rescale_ciphertext (evaluator.c:177-190, 342-362): r0/r1 level-1 limbs */
 int ace_mul_relin_rescale(ace_ctx* ctx, int64_t* r0, int64_t* r1, const int64_t* a0, const int64_t* a1,
                           const int64_t* b0, const int64_t* b1, const int64_t* swk, size_t level);
+/* The same for `count` independent ciphertext pairs that share the relinearisation key: pair i reads
+ * a0 + i*in_stride (likewise a1, b0, b1) and writes r0 + i*out_stride, r1 + i*out_stride (strides in
+ * words).  Equivalent to `count` calls of ace_mul_relin_rescale; every kernel launch covers the batch. */
+int ace_mul_relin_rescale_batch(ace_ctx* ctx, int64_t* r0, int64_t* r1, size_t out_stride, const int64_t* a0,
+                                const int64_t* a1, const int64_t* b0, const int64_t* b1, size_t in_stride,
+                                const int64_t* swk, size_t level, size_t count);
 /* Fast_rotate (evaluator.c:503-522) with the digits of c1 hoisted (Alloc_precomp) */
 int ace_fast_rotate(ace_ctx* ctx, int64_t* r0, int64_t* r1, const int64_t* c0, const int64_t* digits,
                     const int64_t* swk, const int64_t* order, size_t level);

@@ -257,6 +257,66 @@ def test_ciphertext_ops(pair):
         eq(s0, m0, "composite == pieces")
 
 
+def test_mul_relin_rescale_batch(pair):
+    """Three ciphertext pairs in one call, operands padded apart; every pair equals the oracle's single op."""
+    g, o = pair.g, pair.o
+    N = g.N
+    if g.L < 2:
+        pytest.skip("needs two levels")
+    swk = make_swk(g, 900)
+    dk = g.upload(swk)
+    level, nb = g.L, 3
+    pr = g.primes[:level]
+    in_stride, out_stride = (level + 1) * N, level * N  # one limb of padding between operands
+    host = [np.zeros(nb * in_stride, np.int64) for _ in range(4)]
+    ops = []
+    for b in range(nb):
+        polys = [seeded.uniform_poly(910 + 4 * b + i, pr, N) for i in range(4)]
+        ops.append(polys)
+        for i in range(4):
+            host[i][b * in_stride:b * in_stride + level * N] = polys[i]
+    dev = [g.upload(h) for h in host]
+    r0, r1 = g.alloc(nb * out_stride), g.alloc(nb * out_stride)
+    g.mul_relin_rescale_batch(r0, r1, out_stride, dev[0], dev[1], dev[2], dev[3], in_stride, dk, level, nb)
+    got0, got1 = r0.get(), r1.get()
+    n = (level - 1) * N
+    for b in range(nb):
+        m0, m1 = o.mul_relin_rescale(*ops[b], swk, level)
+        eq(got0[b * out_stride:b * out_stride + n], m0, "batch[%d] c0" % b)
+        eq(got1[b * out_stride:b * out_stride + n], m1, "batch[%d] c1" % b)
+        assert not got0[b * out_stride + n:(b + 1) * out_stride].any(), "padding written"
+    g.mul_relin_rescale_batch(r0, r1, 0, dev[0], dev[1], dev[2], dev[3], 0, dk, level, 0)  # empty batch: no-op
+    with pytest.raises(acefhe.AceError):
+        g.mul_relin_rescale_batch(r0, r1, n - 1, dev[0], dev[1], dev[2], dev[3], in_stride, dk, level, 2)  # overlap
+
+
+def test_rotation_many(pair):
+    """More rotations than one batched launch holds (small rings only: the oracle does each one)."""
+    g, o = pair.g, pair.o
+    N = g.N
+    if N < 16 or N > 2048:
+        pytest.skip("covered at one size class")
+    level = g.L
+    pr = g.primes[:level]
+    c0, c1 = seeded.uniform_poly(750, pr, N), seeded.uniform_poly(751, pr, N)
+    dc0, dc1 = g.upload(c0), g.upload(c1)
+    rots = [int(r) for r in 1 + seeded.splitmix64(77, 35) % np.uint64(N // 2 - 1)]
+    base = make_swk(g, 850)
+    swks = [(base + i) % np.tile(np.repeat(np.array(g.primes, np.int64), N), 2 * g.parts) for i in range(len(rots))]
+    orders = [o.automorphism_order(o.find_automorphism_index(r), True) for r in rots]
+    digits = o.precomp(c1, level, True)
+    dswk = [g.upload(s) for s in swks]
+    dord = [g.automorphism_order(g.find_automorphism_index(r), True) for r in rots]
+    n = level * N
+    r0s, r1s = g.alloc(len(rots) * n), g.alloc(len(rots) * n)
+    g.rotate_batch(r0s, r1s, dc0, dc1, dswk, dord, level)
+    got0, got1 = r0s.get(), r1s.get()
+    for i in range(len(rots)):
+        w0, w1 = o.fast_rotate(c0, digits, swks[i], orders[i], level)
+        eq(got0[i * n:(i + 1) * n], w0, "rotate_batch[%d] c0" % i)
+        eq(got1[i * n:(i + 1) * n], w1, "rotate_batch[%d] c1" % i)
+
+
 def test_rotation(pair):
     g, o = pair.g, pair.o
     N = g.N
