@@ -70,6 +70,7 @@ def _sig(lib):
         f("ace_poly_" + n, C.c_int, _vp, _vp, _vp, _vp, _sz, C.c_int)
     f("ace_poly_automorphism", C.c_int, _vp, _vp, _vp, _vp, _sz, C.c_int)
     f("ace_decomp_modup", C.c_int, _vp, _vp, _vp, _sz, _sz, C.c_int)
+    f("ace_mod_up", C.c_int, _vp, _vp, _vp, _sz, _sz, C.c_int)
     f("ace_precomp", C.c_int, _vp, _vp, _vp, _sz, C.c_int)
     f("ace_mod_down", C.c_int, _vp, _vp, _vp, _sz, C.c_int)
     f("ace_rescale", C.c_int, _vp, _vp, _vp, _sz, C.c_int)
@@ -95,7 +96,7 @@ EXPORTS = [
     "ace_hw_modadd", "ace_hw_modsub", "ace_hw_modmul", "ace_hw_modmuladd", "ace_hw_modadd_scalar",
     "ace_hw_modsub_scalar", "ace_hw_modmul_scalar", "ace_hw_modmuladd_scalar", "ace_hw_rotate",
     "ace_find_automorphism_index", "ace_automorphism_order", "ace_poly_add", "ace_poly_sub", "ace_poly_mul",
-    "ace_poly_automorphism", "ace_decomp_modup", "ace_precomp", "ace_mod_down", "ace_rescale", "ace_extend",
+    "ace_poly_automorphism", "ace_decomp_modup", "ace_mod_up", "ace_precomp", "ace_mod_down", "ace_rescale", "ace_extend",
     "ace_dot_prod", "ace_mul_ciph3", "ace_fast_switch_key", "ace_relin", "ace_rescale_ciph",
     "ace_mul_relin_rescale", "ace_mul_relin_rescale_batch", "ace_fast_rotate", "ace_rotate_batch",
 ]
@@ -285,6 +286,9 @@ class Context:
 
     def decomp_modup(self, res, src, level, part, is_ntt=True):
         self._chk(self.lib.ace_decomp_modup(self.h, res.ptr, src.ptr, level, part, int(is_ntt)))
+
+    def mod_up(self, res, digit, level, part, is_ntt=True):
+        self._chk(self.lib.ace_mod_up(self.h, res.ptr, digit.ptr, level, part, int(is_ntt)))
 
     def precomp(self, res, src, level, is_ntt=True):
         self._chk(self.lib.ace_precomp(self.h, res.ptr, src.ptr, level, int(is_ntt)))

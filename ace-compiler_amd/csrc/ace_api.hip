@@ -10,6 +10,7 @@
 #include <memory>
 #include <stdexcept>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 #include "../../include/ace_hip.h"
@@ -77,6 +78,17 @@ struct ace_ctx {
   u64* pinv = nullptr;        // [L][2]
   u64* pmodq = nullptr;       // [L][2]
   LimbMap q_lm{}, p_lm{};     // identity maps: limb t -> prime t / prime L+t
+  // ace_alloc / ace_free: sizes of the buffers handed out, and freed buffers kept for reuse
+  static constexpr size_t kPoolLimitWords = (size_t)4 << 30;  // 32 GiB
+  std::unordered_map<void*, size_t> live;
+  std::multimap<size_t, void*> pool;
+  size_t pooled_words = 0;
+  void drop_pool() {
+    if (stream) (void)hipStreamSynchronize(stream);
+    for (auto& kv : pool) (void)hipFree(kv.second);
+    pool.clear();
+    pooled_words = 0;
+  }
   // scratch arena
   u64* ws = nullptr;
   size_t ws_words = 0, ws_used = 0;
@@ -259,6 +271,7 @@ struct ace_ctx {
   ~ace_ctx() {
     if (stream) (void)hipStreamSynchronize(stream);
     for (void* p : owned) (void)hipFree(p);
+    drop_pool();
     if (ws) (void)hipFree(ws);
     if (ev0) (void)hipEventDestroy(ev0);
     if (ev1) (void)hipEventDestroy(ev1);
@@ -294,19 +307,20 @@ PolySeq shifted(const PolySeq& s, u64 words) {
 
 // Decomp_modup (rns_poly.c:160-258), one digit of one polynomial: copy the
 // digit, INTT it scaled by the inverse cofactors, convert to the complement
-// basis, NTT the new limbs.
-void do_decomp_modup(ace_ctx* c, u64* res, const u64* src, size_t level, size_t part, bool is_ntt) {
+// basis, NTT the new limbs.  `digit` points at the digit's first limb (inside
+// the source polynomial for the fused call, a compact copy for Mod_up).
+void do_decomp_modup(ace_ctx* c, u64* res, const u64* digit, size_t level, size_t part, bool is_ntt) {
   const ModUpDev& m = c->modup_at(level, part);
   const size_t N = c->h.N, nd = m.t.digit.size(), nc = m.t.compl_idx.size(), start = c->h.part_size * part;
-  if (res + start * N != src + start * N)
-    HIP_OK(hipMemcpyAsync(res + start * N, src + start * N, nd * N * sizeof(u64), hipMemcpyDeviceToDevice, c->stream));
+  if (res + start * N != digit)
+    HIP_OK(hipMemcpyAsync(res + start * N, digit, nd * N * sizeof(u64), hipMemcpyDeviceToDevice, c->stream));
   size_t mark = c->ws_used;
   u64* t = c->take(nd * N);
   if (is_ntt)
-    launch_ntt(c->stream, c->d, seq_strided(t, 0), seq_strided(src + start * N, 0), m.digit_lm, nullptr, (u32)nd, 1,
-               true, m.scale_ntt);
+    launch_ntt(c->stream, c->d, seq_strided(t, 0), seq_strided(digit, 0), m.digit_lm, nullptr, (u32)nd, 1, true,
+               m.scale_ntt);
   else
-    launch_mul_const(c->stream, c->d, t, src + start * N, m.scale_coef, m.digit_lm, (u32)nd);
+    launch_mul_const(c->stream, c->d, t, digit, m.scale_coef, m.digit_lm, (u32)nd);
   ConvBatch b{};
   b.n_jobs = 1;
   b.job[0].hat = m.hat;
@@ -543,11 +557,31 @@ void ace_modulus(const ace_ctx* c, size_t i, uint64_t out[5]) {
 }
 
 // ---- memory -----------------------------------------------------------------
+// Buffers handed back by ace_free are kept, by size, for the next ace_alloc of
+// that size: programs allocate and free the same few polynomial shapes in a
+// loop, and hipMalloc / hipFree cost far more than the kernels between them.
+// Reuse is safe without a wait because every use of a buffer is ordered on
+// the context's one stream.
 int64_t* ace_alloc(ace_ctx* c, size_t n_words) {
   try {
     if (!c || !c->device_ok) throw std::runtime_error("no HIP device: this context holds host tables only");
+    const size_t words = std::max<size_t>(n_words, 1);
     u64* p = nullptr;
-    HIP_OK(hipMalloc((void**)&p, std::max<size_t>(n_words, 1) * sizeof(u64)));
+    auto it = c->pool.find(words);
+    if (it != c->pool.end()) {
+      p = static_cast<u64*>(it->second);
+      c->pool.erase(it);
+      c->pooled_words -= words;
+    } else {
+      hipError_t e = hipMalloc((void**)&p, words * sizeof(u64));
+      if (e != hipSuccess && c->pooled_words) {  // give the cached buffers back and try once more
+        (void)hipGetLastError();
+        c->drop_pool();
+        e = hipMalloc((void**)&p, words * sizeof(u64));
+      }
+      HIP_OK(e);
+    }
+    c->live[p] = words;
     launch_fill_zero(c->stream, p, n_words);
     return reinterpret_cast<int64_t*>(p);
   } catch (const std::exception& e) {
@@ -557,6 +591,15 @@ int64_t* ace_alloc(ace_ctx* c, size_t n_words) {
 }
 void ace_free(ace_ctx* c, int64_t* p) {
   if (!p || !c || !c->device_ok) return;
+  auto it = c->live.find(p);
+  if (it == c->live.end()) return;  // not from ace_alloc of this context (a view, or freed twice)
+  const size_t words = it->second;
+  c->live.erase(it);
+  if (c->pooled_words + words <= ace_ctx::kPoolLimitWords) {
+    c->pool.emplace(words, p);
+    c->pooled_words += words;
+    return;
+  }
   (void)hipStreamSynchronize(c->stream);
   (void)hipFree(p);
 }
@@ -770,7 +813,18 @@ int ace_decomp_modup(ace_ctx* c, int64_t* res, const int64_t* src, size_t level,
   if (part >= c->h.num_decomp(level)) return fail("ace_decomp_modup: digit index out of range");
   c->ensure_ws(c->std_ws(level));
   c->ws_used = 0;
-  do_decomp_modup(c, U(res), U(src), level, part, is_ntt != 0);
+  do_decomp_modup(c, U(res), U(src) + c->h.part_size * part * (size_t)c->h.N, level, part, is_ntt != 0);
+  ACE_CATCH_INT
+}
+
+int ace_mod_up(ace_ctx* c, int64_t* res, const int64_t* digit, size_t level, size_t part, int is_ntt) {
+  ACE_TRY
+  if (!res || !digit) return fail("ace_mod_up: null argument");
+  if (!level_ok(c, level)) return fail("ace_mod_up: level out of range");
+  if (part >= c->h.num_decomp(level)) return fail("ace_mod_up: digit index out of range");
+  c->ensure_ws(c->std_ws(level));
+  c->ws_used = 0;
+  do_decomp_modup(c, U(res), U(digit), level, part, is_ntt != 0);
   ACE_CATCH_INT
 }
 

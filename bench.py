@@ -69,16 +69,13 @@ def cpu_baseline(x_host, idx, budget_s):
                       "%.1f s, single thread, gcc -O3" % (done, LIMBS, POLYS, dt)}
 
 
-def extra_legs(g, np, seeded):
-    """HMult+relinearise+rescale pairs/s and hoisted rotations/s at l=24, k=7, dnum=3."""
+def keyswitch_leg(g, np, seeded, swk, cts):
+    """16 independent HMult + relinearise + rescale at l=24, k=7, dnum=3, one batched call."""
     extra = {}
-    level, T = g.L, g.L + g.K
-    kwords = 2 * g.parts * T * N
-    log("key-switch leg: 16 ciphertext pairs, one relinearisation key")
-    swk = g.upload(np.concatenate([seeded.uniform_poly(2000 + i, g.primes, N) for i in range(2 * g.parts)]))
-    cts = [g.upload(seeded.uniform_poly(3000 + i, g.primes[:level], N)) for i in range(4)]
+    level = g.L
     pairs = 16
-    # 16 distinct ciphertext pairs derived on the device from the seeded one: operand p = operand 0 + p per limb
+    log("key-switch leg: %d ciphertext pairs, one relinearisation key" % pairs)
+    # distinct ciphertext pairs derived on the device from the seeded one: operand p = operand 0 + p per limb
     stride = level * N
     ops = [g.alloc(pairs * stride) for _ in range(4)]
     for k in range(4):
@@ -95,17 +92,24 @@ def extra_legs(g, np, seeded):
     ms = time_region(g, hmult_batch, 5)
     extra["keyswitch_ops_per_s"] = round(pairs / (ms * 1e-3), 1)
     extra["hmult_relin_rescale_ms"] = round(ms / pairs, 4)
-    # 172 MB compulsory traffic per op (96 input + 186 key + 46 output limbs of 512 KiB)
-    extra["keyswitch_hbm_frac"] = round(328 * N * 8 * pairs / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+    # compulsory traffic per op: 96 input + 46 output limbs of 512 KiB (the key's 186 limbs are shared by the batch)
+    extra["keyswitch_hbm_frac"] = round((142 * pairs + 186) * N * 8 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
 
     def hmult_single():
         g.mul_relin_rescale(r0, r1, cts[0], cts[1], cts[2], cts[3], swk, level)
 
     hmult_single()
     extra["hmult_relin_rescale_single_ms"] = round(time_region(g, hmult_single, 10), 4)
-    for b in ops:
+    for b in ops + [r0, r1]:
         b.free()
+    return extra
 
+
+def rotation_leg(g, np, seeded, swk, cts):
+    """32 rotations of one ciphertext with the raised digits of c1 shared (hoisting), one batched call."""
+    extra = {}
+    level, T = g.L, g.L + g.K
+    kwords = 2 * g.parts * T * N
     nrot = 32
     log("rotation leg: %d rotations of one ciphertext, hoisted ModUp" % nrot)
     rots = [1 << i for i in range(15)] + [-1] + [int(v) for v in 1 + seeded.splitmix64(7, 16) % np.uint64(N // 2 - 1)]
@@ -125,7 +129,20 @@ def extra_legs(g, np, seeded):
     ms = time_region(g, f, 5)
     extra["rotations_per_s"] = round(nrot / (ms * 1e-3), 1)
     extra["rotate_batch_ms"] = round(ms, 3)
-    extra["rotation_hbm_frac"] = round(327 * N * 8 * nrot / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+    # compulsory traffic: 186 key limbs in + 48 result limbs out per rotation, 48 input limbs once
+    extra["rotation_hbm_frac"] = round((234 * nrot + 48) * N * 8 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+    return extra
+
+
+def extra_legs(g, np, seeded, which="all"):
+    level = g.L
+    swk = g.upload(np.concatenate([seeded.uniform_poly(2000 + i, g.primes, N) for i in range(2 * g.parts)]))
+    cts = [g.upload(seeded.uniform_poly(3000 + i, g.primes[:level], N)) for i in range(4)]
+    extra = {}
+    if which in ("all", "keyswitch"):
+        extra.update(keyswitch_leg(g, np, seeded, swk, cts))
+    if which in ("all", "rotation"):
+        extra.update(rotation_leg(g, np, seeded, swk, cts))
     return extra
 
 
@@ -136,8 +153,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="time budget of the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the key-switch / rotation measurements")
-    ap.add_argument("--only-extra", action="store_true",
-                    help="profiling aid: run only the key-switch and rotation legs (prints their fields alone)")
+    ap.add_argument("--only-extra", choices=("all", "keyswitch", "rotation"), default=None,
+                    help="profiling aid: run only the key-switch and/or rotation legs (prints their fields alone)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU; this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
@@ -183,7 +200,7 @@ def main():
     # per-kernel timing of the four NTT kernels (each reads and writes every coefficient once)
     kern = {}
     if args.only_extra:
-        print(json.dumps(extra_legs(g, np, seeded)))
+        print(json.dumps(extra_legs(g, np, seeded, args.only_extra)))
         return
     scratch = g.alloc(POLYS * per_poly)
     pass_bytes = POLYS * per_poly * 16

@@ -77,7 +77,9 @@ int ace_host_automorphism_order(const ace_ctx* ctx, int64_t* host_order, uint32_
 
 /* ---- device memory -------------------------------------------------------
  * Replaces the malloc+memset of Alloc_poly_data (include/poly/rns_poly.h:109-119):
- * zero-filled HBM, n int64 words. */
+ * zero-filled HBM, n int64 words.  ace_free keeps the buffer (up to 32 GiB in
+ * total) for the next ace_alloc of the same size, so alloc/free pairs inside a
+ * program's loops cost a fill kernel, not a hipMalloc. */
 int64_t* ace_alloc(ace_ctx* ctx, size_t n_words);
 void     ace_free(ace_ctx* ctx, int64_t* dev_ptr);
 int      ace_upload(ace_ctx* ctx, int64_t* dev_dst, const int64_t* host_src, size_t n_words);
@@ -137,6 +139,9 @@ int ace_poly_automorphism(ace_ctx* ctx, int64_t* res, const int64_t* a, const in
 /* Decomp_modup (:160-258) (== Decomp :74-105 + Mod_up :107-158): digit `part`
  * of src (level limbs) raised to level+num_p limbs. */
 int ace_decomp_modup(ace_ctx* ctx, int64_t* res, const int64_t* src, size_t level, size_t part, int is_ntt);
+/* Mod_up (:107-158) alone: `digit` holds only the limbs of digit `part` (what
+ * Decomp :74-105 produced), res as for ace_decomp_modup. */
+int ace_mod_up(ace_ctx* ctx, int64_t* res, const int64_t* digit, size_t level, size_t part, int is_ntt);
 /* Precomp / Alloc_precomp (:416-481): all digits, res = num_decomp x (level+num_p) limbs */
 int ace_precomp(ace_ctx* ctx, int64_t* res, const int64_t* src, size_t level, int is_ntt);
 /* Mod_down (:260-308): src level+num_p limbs -> res level limbs */

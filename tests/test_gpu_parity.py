@@ -162,7 +162,15 @@ def test_decomp_modup_and_precomp(pair):
             for part in range(nd):
                 dr = g.alloc(T * N)
                 g.decomp_modup(dr, dc, level, part, is_ntt)
-                eq(dr, o.decomp_modup(c, level, part, is_ntt), "decomp_modup l=%d part=%d ntt=%d" % (level, part, is_ntt))
+                want = o.decomp_modup(c, level, part, is_ntt)
+                eq(dr, want, "decomp_modup l=%d part=%d ntt=%d" % (level, part, is_ntt))
+                # Decomp then Mod_up: the digit handed over as a compact copy
+                start = g.part_size * part
+                length = min(g.part_size, level - start)
+                dd = g.upload(c[start * N:(start + length) * N])
+                dr2 = g.alloc(T * N)
+                g.mod_up(dr2, dd, level, part, is_ntt)
+                eq(dr2, want, "mod_up l=%d part=%d ntt=%d" % (level, part, is_ntt))
             dr = g.alloc(nd * T * N)
             g.precomp(dr, dc, level, is_ntt)
             eq(dr, o.precomp(c, level, is_ntt), "precomp l=%d ntt=%d" % (level, is_ntt))

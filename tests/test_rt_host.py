@@ -1,0 +1,75 @@
+"""The program-facing C runtime (rt_hip.h) without a GPU: it builds, keeps the reference's struct layouts,
+takes the reference's own generated fixtures unchanged, and refuses to run without a HIP device."""
+import ctypes
+import os
+import subprocess
+
+import pytest
+
+import rt_program
+from oracle_lib import Oracle
+
+ROOT = rt_program.ROOT
+INC = ["-I" + os.path.join(ROOT, "ace-compiler_amd", "rt_hip", "include"), "-I" + os.path.join(ROOT, "include")]
+REF_EXAMPLES = "/root/reference/fhe-cmplr/rtlib/ant/example"
+
+
+def test_library_exports():
+    lib = ctypes.CDLL(os.path.join(ROOT, "ace-compiler_amd", "librt_hip.so"))
+    for name in ("Prepare_context Finalize_context Run_main_graph Degree Get_q_cnt Get_p_cnt Get_q_parts Q_modulus "
+                 "P_modulus Free_poly_data Alloc_polys Init_poly Copy_poly Decomp Mod_up Decomp_modup Mod_down Rescale "
+                 "Modswitch Precomp Dot_prod Extend Conv_poly2ntt_inplace Conv_ntt2poly_inplace Add_poly Sub_poly "
+                 "Mul_poly Hw_modadd Hw_modsub Hw_modmul Hw_modmuladd Hw_modadd_scalar Hw_modsub_scalar "
+                 "Hw_modmul_scalar Hw_modmuladd_scalar Hw_rotate Hw_ntt Hw_intt Auto_idx Auto_order Swk Get_swk_at "
+                 "Swk_c0 Swk_c1 Level Sc_degree Init_ciph_same_scale Init_ciph_up_scale Init_ciph_down_scale "
+                 "Init_ciph_same_scale_ciph3 Init_ciph3_up_scale Copy_ciph Free_ciph_poly Zero_ciph Add_ciph Sub_ciph "
+                 "Mul_ciph3 Relin Mul_ciph Rescale_ciph Modswitch_ciph Rotate_ciph Rotate_batch_ciph Conjugate_ciph "
+                 "Get_input_data Set_output_data Tm_start Tm_taken Rt_load_switch_key Rt_set_input "
+                 "Rt_get_output").split():
+        assert hasattr(lib, name), name
+
+
+def test_struct_layouts(tmp_path):
+    """Sizes and offsets the reference's headers give on x86-64 (generated code keeps these structs on its stack)."""
+    src = tmp_path / "layout.c"
+    src.write_text('#include <stddef.h>\n#include "rt_ant/rt_ant.h"\nint main(void){printf("%zu %zu %zu %zu %zu %zu %zu %zu %zu\\n",'
+                   "sizeof(MODULUS),offsetof(MODULUS,_prec128),sizeof(POLYNOMIAL),offsetof(POLYNOMIAL,_is_ntt),"
+                   "offsetof(POLYNOMIAL,_data),sizeof(CIPHERTEXT),sizeof(CIPHERTEXT3),sizeof(PUBLIC_KEY),"
+                   "sizeof(SWITCH_KEY));return 0;}\n")
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-std=gnu11"] + INC + [str(src), "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], capture_output=True, text=True, check=True).stdout.split()
+    assert [int(v) for v in out] == [48, 32, 48, 32, 40, 120, 168, 96, 8]
+
+
+@pytest.mark.skipif(not os.path.isdir(REF_EXAMPLES), reason="reference checkout not present")
+@pytest.mark.parametrize("fixture", ["eg_fhertlib_add.inc", "eg_fhertlib_relin.inc", "eg_fhertlib_relin_02.inc",
+                                     "eg_fhertlib_rotate.inc", "eg_fhertlib_rotate_02.inc"])
+def test_reference_generated_programs_compile_unchanged(fixture, tmp_path):
+    """The compiler's own output for the ANT runtime builds and links against this runtime as it is."""
+    obj = tmp_path / "prog.o"
+    r = subprocess.run(["gcc", "-std=gnu11", "-Werror=implicit-function-declaration"] + INC +
+                       ["-x", "c", "-c", os.path.join(REF_EXAMPLES, fixture), "-o", str(obj)],
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    main = tmp_path / "main.c"
+    main.write_text('#include "common/rtlib.h"\nint main(void){Prepare_context();Run_main_graph();Finalize_context();return 0;}\n')
+    pkg = os.path.join(ROOT, "ace-compiler_amd")
+    r = subprocess.run(["gcc", "-std=gnu11"] + INC + [str(main), str(obj), "-o", str(tmp_path / "prog"), "-L" + pkg,
+                        "-lrt_hip", "-lace_hip", "-Wl,-rpath," + pkg], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+
+
+def test_program_refuses_to_run_without_gpu(tmp_path):
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    cfg = (64, 3, 45, 40, 2)
+    o = Oracle(*cfg)
+    blob, _ = rt_program.make_inputs(o, cfg, [1], seed=1)
+    o.close()
+    p = tmp_path / "in.bin"
+    p.write_bytes(blob)
+    res = rt_program.run_program(str(p), str(tmp_path / "out.bin"))
+    assert res.returncode != 0
+    assert "no HIP device" in res.stderr
