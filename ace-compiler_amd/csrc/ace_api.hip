@@ -382,7 +382,7 @@ void do_precomp(ace_ctx* c, u64* res, u64 res_stride, const u64* src, u64 src_st
 // Mod_down (rns_poly.c:260-308) of np polynomials; addend_mode: 0 none,
 // 1 add addend.at(p) to every polynomial, 2 only to even p
 void do_mod_down(ace_ctx* c, const PolySeq& res, const PolySeq& src, size_t np, size_t level, bool is_ntt,
-                 const PolySeq* addend, int addend_mode) {
+                 const PolySeq* addend, int addend_mode, const OrderSet* orders = nullptr) {
   const size_t N = c->h.N, K = c->h.K, L = c->h.L;
   size_t mark = c->ws_used;
   u64* t = c->take(np * K * N);
@@ -409,7 +409,7 @@ void do_mod_down(ace_ctx* c, const PolySeq& res, const PolySeq& src, size_t np, 
     launch_ntt(c->stream, c->d, ys, ys, c->q_lm, nullptr, (u32)level, (u32)np, false, nullptr);
   }
   launch_moddown_tail(c->stream, c->d, res, src, y, level * N, addend_mode ? addend : nullptr, addend_mode, c->pinv,
-                      c->q_lm, (u32)level, (u32)np);
+                      c->q_lm, (u32)level, (u32)np, orders);
   c->ws_used = mark;
 }
 
@@ -449,16 +449,17 @@ LimbMap key_pos(const ace_ctx* c, size_t level) {
 // Fast_switch_key (evaluator.c:411-462) for nb operands.  Operand o reads the
 // digits at digits + o*digits_op_stride (0: all share one set) and key
 // keys.p[o] (or keys.p[0] when keys.n == 1); its two results are polynomials
-// 2o and 2o+1 of `out`.  The addend is fused into the Mod_down tail.
+// 2o and 2o+1 of `out`.  The addend, and with `orders` the automorphism of
+// operand o (table o), are fused into the Mod_down tail.
 void do_switch_key(ace_ctx* c, const PolySeq& out, const u64* digits, u64 digits_op_stride, const KeySet& keys,
-                   size_t nb, size_t level, const PolySeq* addend, int addend_mode) {
+                   size_t nb, size_t level, const PolySeq* addend, int addend_mode, const OrderSet* orders = nullptr) {
   const size_t N = c->h.N, T = level + c->h.K, kpoly = (c->h.L + c->h.K) * N, nd = c->h.num_decomp(level);
   size_t mark = c->ws_used;
   u64* e = c->take(nb * 2 * T * N);  // [operand][b|a][T limbs]
   LimbMap lm = poly_lm(c, level, true), kp = key_pos(c, level);
   launch_dotprod(c->stream, c->d, e, e + T * N, 2 * T * N, digits, T * N, digits_op_stride, keys, kpoly, 2 * kpoly,
                  (u32)nd, lm, kp, (u32)T, (u32)nb);
-  do_mod_down(c, out, seq_strided(e, T * N), 2 * nb, level, true, addend, addend_mode);
+  do_mod_down(c, out, seq_strided(e, T * N), 2 * nb, level, true, addend, addend_mode, orders);
   c->ws_used = mark;
 }
 
@@ -958,17 +959,12 @@ int ace_mul_relin_rescale_batch(ace_ctx* c, int64_t* r0, int64_t* r1, size_t out
   ACE_CATCH_INT
 }
 
-// Fast_rotate for nr <= kMaxBatchPtrs rotations of one ciphertext sharing the digits
+// Fast_rotate for nr <= kMaxBatchPtrs rotations of one ciphertext sharing the digits:
+// switch key, add c0 to the first polynomial, permute -- the last two inside the Mod_down tail
 static void do_fast_rotate(ace_ctx* c, u64* r0, u64* r1, u64 r_stride, const u64* c0, const u64* digits,
                            const KeySet& keys, const OrderSet& orders, size_t nr, size_t level) {
-  const size_t N = c->h.N;
-  size_t mark = c->ws_used;
-  u64* t01 = c->take(nr * 2 * level * N);  // [rotation][c0|c1][level limbs]
-  PolySeq add = seq_pair(c0, c0, 0);       // c0 is added to the first polynomial of every rotation
-  do_switch_key(c, seq_strided(t01, level * N), digits, 0, keys, nr, level, &add, 2);
-  launch_gather2(c->stream, c->d, r0, r1, r_stride, t01, t01 + level * N, 2 * level * N, orders, c->q_lm, (u32)level,
-                 (u32)nr);
-  c->ws_used = mark;
+  PolySeq add = seq_pair(c0, c0, 0);  // c0 is added to the first polynomial of every rotation
+  do_switch_key(c, seq_pair(r0, r1, r_stride), digits, 0, keys, nr, level, &add, 2, &orders);
 }
 
 int ace_fast_rotate(ace_ctx* c, int64_t* r0, int64_t* r1, const int64_t* c0, const int64_t* digits,
@@ -976,6 +972,7 @@ int ace_fast_rotate(ace_ctx* c, int64_t* r0, int64_t* r1, const int64_t* c0, con
   ACE_TRY
   if (!r0 || !r1 || !c0 || !digits || !swk || !order) return fail("ace_fast_rotate: null argument");
   if (!level_ok(c, level)) return fail("ace_fast_rotate: level out of range");
+  if (r0 == c0 || r1 == c0) return fail("ace_fast_rotate: the result must not overwrite c0 (it is permuted on the way out)");
   c->ensure_ws(c->std_ws(level));
   c->ws_used = 0;
   OrderSet os{};
@@ -991,6 +988,7 @@ int ace_rotate_batch(ace_ctx* c, int64_t* r0s, int64_t* r1s, const int64_t* c0, 
   if (count == 0) return 0;
   if (!r0s || !r1s || !c0 || !c1 || !swks || !orders) return fail("ace_rotate_batch: null argument");
   if (!level_ok(c, level)) return fail("ace_rotate_batch: level out of range");
+  if (r0s == c0 || r1s == c0) return fail("ace_rotate_batch: the results must not overwrite c0 (it is permuted on the way out)");
   for (size_t i = 0; i < count; ++i)
     if (!swks[i] || !orders[i]) return fail("ace_rotate_batch: null key or order table");
   const size_t N = c->h.N, nd = c->h.num_decomp(level), T = level + c->h.K;

@@ -65,10 +65,11 @@ void launch_dotprod(hipStream_t st, const DevCtx& c, u64* out0, u64* out1, u64 o
                     u64 digit_stride, u64 digits_op_stride, const KeySet& keys, u64 key1_off, u64 key_stride,
                     u32 n_parts, const LimbMap& lm, const LimbMap& key_limb, u32 n_limbs, u32 n_ops);
 // Mod_down tail for n_polys polynomials: out = (src - y) * pinv (+ addend), per limb constants cst[2t], cst[2t+1];
-// addend_mode 0 none, 1 every polynomial, 2 even polynomials only
+// addend_mode 0 none, 1 every polynomial, 2 even polynomials only.  With `orders` the result is permuted on the
+// way out: out[i] = value at orders[p / 2][i] (the automorphism closing a rotation; out must not alias an input).
 void launch_moddown_tail(hipStream_t st, const DevCtx& c, const PolySeq& out, const PolySeq& src, const u64* y,
                          u64 y_stride, const PolySeq* addend, int addend_mode, const u64* cst, const LimbMap& lm,
-                         u32 n_limbs, u32 n_polys);
+                         u32 n_limbs, u32 n_polys, const OrderSet* orders = nullptr);
 // Rescale: u[p][t][i] = switch_modulus(last[p][i], q_l -> q_t) * K_t ;  cst per limb: K, K', diff
 void launch_rescale_switch(hipStream_t st, const DevCtx& c, u64* u, u64 u_stride, const u64* last, u64 last_stride,
                            u32 last_prime, const u64* cst, const LimbMap& lm, u32 n_limbs, u32 n_polys);

@@ -242,10 +242,102 @@ __global__ __launch_bounds__(kThreads) void dotprod_kernel(DevCtx c, u64* __rest
   }
 }
 
+// The same for operands that share one key: each thread keeps its 2*NP key
+// words in registers and walks the operands blockIdx.z, blockIdx.z + gridDim.z, ...
+// so the key, the largest stream of a key switch, is fetched gridDim.z times
+// instead of once per operand.
+template <int NP>
+__global__ __launch_bounds__(kThreads) void dotprod_shared_key_kernel(
+    DevCtx c, u64* __restrict__ out0, u64* __restrict__ out1, u64 out_stride, const u64* __restrict__ digits,
+    u64 digit_stride, u64 digits_op_stride, const u64* __restrict__ key0, u64 key1_off, u64 key_stride, LimbMap lm,
+    LimbMap key_limb, u32 n_ops) {
+  const u32 limb = blockIdx.y;
+  const DevPrime P = c.primes[lm.prime[limb]];
+  const u64 n = c.N, dbase = (u64)limb * n, kbase = (u64)key_limb.prime[limb] * n;
+  const u64* __restrict__ key1 = key0 + key1_off;
+#pragma unroll 1
+  ACE_EW_LOOP(i, n) {
+    u64 k0[NP], k1[NP];
+#pragma unroll
+    for (int d = 0; d < NP; ++d) {
+      k0[d] = key0[d * key_stride + kbase + i];
+      k1[d] = key1[d * key_stride + kbase + i];
+    }
+    for (u32 op = blockIdx.z; op < n_ops; op += gridDim.z) {
+      const u64* __restrict__ dg = digits + op * digits_op_stride + dbase + i;
+      u64 h0 = 0, l0 = 0, h1 = 0, l1 = 0;
+#pragma unroll
+      for (int d = 0; d < NP; ++d) {
+        u64 x = dg[d * digit_stride];
+        mac128(h0, l0, x, k0[d]);
+        mac128(h1, l1, x, k1[d]);
+      }
+      out0[op * out_stride + dbase + i] = barrett128(h0, l0, P);
+      out1[op * out_stride + dbase + i] = barrett128(h1, l1, P);
+    }
+  }
+}
+
+// The mirror case, rotations of one ciphertext: every operand multiplies the
+// same digits by its own key.  The NP digit words stay in registers while the
+// thread walks the operands, so the digits are fetched gridDim.z times instead
+// of once per rotation (they do not survive in L2 between rotations: each
+// rotation streams a whole key through it).
+template <int NP>
+__global__ __launch_bounds__(kThreads) void dotprod_shared_digits_kernel(
+    DevCtx c, u64* __restrict__ out0, u64* __restrict__ out1, u64 out_stride, const u64* __restrict__ digits,
+    u64 digit_stride, KeySet keys, u64 key1_off, u64 key_stride, LimbMap lm, LimbMap key_limb, u32 n_ops) {
+  const u32 limb = blockIdx.y;
+  const DevPrime P = c.primes[lm.prime[limb]];
+  const u64 n = c.N, dbase = (u64)limb * n, kbase = (u64)key_limb.prime[limb] * n;
+#pragma unroll 1
+  ACE_EW_LOOP(i, n) {
+    u64 x[NP];
+#pragma unroll
+    for (int d = 0; d < NP; ++d) x[d] = digits[d * digit_stride + dbase + i];
+    for (u32 op = blockIdx.z; op < n_ops; op += gridDim.z) {
+      const u64* __restrict__ key0 = keys.p[op] + kbase + i;
+      const u64* __restrict__ key1 = key0 + key1_off;
+      u64 h0 = 0, l0 = 0, h1 = 0, l1 = 0;
+#pragma unroll
+      for (int d = 0; d < NP; ++d) {
+        mac128(h0, l0, x[d], key0[d * key_stride]);
+        mac128(h1, l1, x[d], key1[d * key_stride]);
+      }
+      out0[op * out_stride + dbase + i] = barrett128(h0, l0, P);
+      out1[op * out_stride + dbase + i] = barrett128(h1, l1, P);
+    }
+  }
+}
+
 void launch_dotprod(hipStream_t st, const DevCtx& c, u64* out0, u64* out1, u64 out_stride, const u64* digits,
                     u64 digit_stride, u64 digits_op_stride, const KeySet& keys, u64 key1_off, u64 key_stride,
                     u32 n_parts, const LimbMap& lm, const LimbMap& key_limb, u32 n_limbs, u32 n_ops) {
   if (!n_limbs || !n_ops) return;
+  if (keys.n == 1 && n_ops > 1 && out1 && n_parts >= 1 && n_parts <= 4) {
+    // NP <= 4 products of residues below 2^61 fit 128 bits without an intermediate reduction
+    dim3 g = ew_grid(c.N, n_limbs, n_ops < 4 ? n_ops : 4);
+#define ACE_DP_CASE(NP)                                                                                          \
+  case NP:                                                                                                       \
+    hipLaunchKernelGGL(dotprod_shared_key_kernel<NP>, g, dim3(kThreads), 0, st, c, out0, out1, out_stride,       \
+                       digits, digit_stride, digits_op_stride, keys.p[0], key1_off, key_stride, lm, key_limb,    \
+                       n_ops);                                                                                   \
+    break;
+    switch (n_parts) { ACE_DP_CASE(1) ACE_DP_CASE(2) ACE_DP_CASE(3) ACE_DP_CASE(4) }
+#undef ACE_DP_CASE
+    return;
+  }
+  if (keys.n == n_ops && n_ops > 1 && digits_op_stride == 0 && out1 && n_parts >= 1 && n_parts <= 4) {
+    dim3 g = ew_grid(c.N, n_limbs, n_ops < 4 ? n_ops : 4);
+#define ACE_DP_CASE(NP)                                                                                          \
+  case NP:                                                                                                       \
+    hipLaunchKernelGGL(dotprod_shared_digits_kernel<NP>, g, dim3(kThreads), 0, st, c, out0, out1, out_stride,    \
+                       digits, digit_stride, keys, key1_off, key_stride, lm, key_limb, n_ops);                   \
+    break;
+    switch (n_parts) { ACE_DP_CASE(1) ACE_DP_CASE(2) ACE_DP_CASE(3) ACE_DP_CASE(4) }
+#undef ACE_DP_CASE
+    return;
+  }
   dim3 g = ew_grid(c.N, n_limbs, n_ops);
   if (out1)
     hipLaunchKernelGGL(dotprod_kernel<true>, g, dim3(kThreads), 0, st, c, out0, out1, out_stride, digits,
@@ -256,11 +348,15 @@ void launch_dotprod(hipStream_t st, const DevCtx& c, u64* out0, u64* out1, u64 o
 }
 
 // ---- Mod_down tail (rns_poly.c:292-303): (src - y) * P^-1 [+ addend] --------
-// blockIdx.z = polynomial; src/out/addend are addressed as PolySeq.
+// blockIdx.z = polynomial; src/out/addend are addressed as PolySeq.  With index
+// tables (orders.n != 0) the automorphism that ends a rotation is applied on the
+// way out: out[i] = value at order[i] (polynomials 2r and 2r+1 use table r),
+// negative entries as in gather_kernel.
 __global__ __launch_bounds__(kThreads) void moddown_tail_kernel(DevCtx c, PolySeq outs, PolySeq srcs,
                                                                 const u64* __restrict__ y_base, u64 y_stride,
                                                                 PolySeq addends, int addend_mode,
-                                                                const u64* __restrict__ cst, LimbMap lm) {
+                                                                const u64* __restrict__ cst, LimbMap lm,
+                                                                OrderSet orders) {
   const u32 limb = blockIdx.y, p = blockIdx.z;
   const u64 q = c.primes[lm.prime[limb]].q;
   const u64 w = cst[2 * limb], wp = cst[2 * limb + 1];
@@ -270,21 +366,26 @@ __global__ __launch_bounds__(kThreads) void moddown_tail_kernel(DevCtx c, PolySe
   const u64* __restrict__ y = y_base + p * y_stride;
   // addend_mode: 0 none, 1 every polynomial, 2 even polynomials only
   const u64* addend = (addend_mode == 1 || (addend_mode == 2 && !(p & 1))) ? addends.at(p) : nullptr;
+  const i64* __restrict__ order = orders.n ? orders.p[orders.n == 1 ? 0 : (p >> 1)] : nullptr;
 #pragma unroll
   ACE_EW_LOOP(i, n) {
-    u64 v = shoup_mul(sub_mod(src[base + i], y[base + i], q), w, wp, q);
-    if (addend) v = add_mod(v, addend[base + i], q);
-    out[base + i] = v;
+    i64 k = order ? order[i] : (i64)i;
+    u64 j = base + (u64)(k < 0 ? -k : k);
+    u64 v = shoup_mul(sub_mod(src[j], y[j], q), w, wp, q);
+    if (addend) v = add_mod(v, addend[j], q);
+    out[base + i] = k < 0 ? q - v : v;
   }
 }
 
 void launch_moddown_tail(hipStream_t st, const DevCtx& c, const PolySeq& out, const PolySeq& src, const u64* y,
                          u64 y_stride, const PolySeq* addend, int addend_mode, const u64* cst, const LimbMap& lm,
-                         u32 n_limbs, u32 n_polys) {
+                         u32 n_limbs, u32 n_polys, const OrderSet* orders) {
   if (!n_limbs || !n_polys) return;
   PolySeq ad = addend ? *addend : out;
+  OrderSet os{};
+  if (orders) os = *orders;
   hipLaunchKernelGGL(moddown_tail_kernel, ew_grid(c.N, n_limbs, n_polys), dim3(kThreads), 0, st, c, out, src, y,
-                     y_stride, ad, addend ? addend_mode : 0, cst, lm);
+                     y_stride, ad, addend ? addend_mode : 0, cst, lm, os);
 }
 
 // ---- Rescale (rns_poly.c:310-404) ------------------------------------------
