@@ -255,25 +255,41 @@ __global__ __launch_bounds__(kThreads) void dotprod_shared_key_kernel(
   const DevPrime P = c.primes[lm.prime[limb]];
   const u64 n = c.N, dbase = (u64)limb * n, kbase = (u64)key_limb.prime[limb] * n;
   const u64* __restrict__ key1 = key0 + key1_off;
-#pragma unroll 1
-  ACE_EW_LOOP(i, n) {
-    u64 k0[NP], k1[NP];
+  // the thread's kUnroll coefficients are handled together so that every operand has
+  // kUnroll * NP independent loads in flight
+  const u64 i0 = (u64)blockIdx.x * (kThreads * kUnroll) + threadIdx.x;
+  u64 k0[kUnroll][NP], k1[kUnroll][NP];
+#pragma unroll
+  for (int u = 0; u < kUnroll; ++u) {
+    const u64 i = i0 + u * kThreads;
 #pragma unroll
     for (int d = 0; d < NP; ++d) {
-      k0[d] = key0[d * key_stride + kbase + i];
-      k1[d] = key1[d * key_stride + kbase + i];
+      k0[u][d] = i < n ? key0[d * key_stride + kbase + i] : 0;
+      k1[u][d] = i < n ? key1[d * key_stride + kbase + i] : 0;
     }
-    for (u32 op = blockIdx.z; op < n_ops; op += gridDim.z) {
-      const u64* __restrict__ dg = digits + op * digits_op_stride + dbase + i;
+  }
+  for (u32 op = blockIdx.z; op < n_ops; op += gridDim.z) {
+    const u64* __restrict__ dg = digits + op * digits_op_stride + dbase;
+    u64 x[kUnroll][NP];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const u64 i = i0 + u * kThreads;
+#pragma unroll
+      for (int d = 0; d < NP; ++d) x[u][d] = i < n ? dg[d * digit_stride + i] : 0;
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const u64 i = i0 + u * kThreads;
       u64 h0 = 0, l0 = 0, h1 = 0, l1 = 0;
 #pragma unroll
       for (int d = 0; d < NP; ++d) {
-        u64 x = dg[d * digit_stride];
-        mac128(h0, l0, x, k0[d]);
-        mac128(h1, l1, x, k1[d]);
+        mac128(h0, l0, x[u][d], k0[u][d]);
+        mac128(h1, l1, x[u][d], k1[u][d]);
       }
-      out0[op * out_stride + dbase + i] = barrett128(h0, l0, P);
-      out1[op * out_stride + dbase + i] = barrett128(h1, l1, P);
+      if (i < n) {
+        out0[op * out_stride + dbase + i] = barrett128(h0, l0, P);
+        out1[op * out_stride + dbase + i] = barrett128(h1, l1, P);
+      }
     }
   }
 }
@@ -290,22 +306,40 @@ __global__ __launch_bounds__(kThreads) void dotprod_shared_digits_kernel(
   const u32 limb = blockIdx.y;
   const DevPrime P = c.primes[lm.prime[limb]];
   const u64 n = c.N, dbase = (u64)limb * n, kbase = (u64)key_limb.prime[limb] * n;
-#pragma unroll 1
-  ACE_EW_LOOP(i, n) {
-    u64 x[NP];
+  const u64 i0 = (u64)blockIdx.x * (kThreads * kUnroll) + threadIdx.x;
+  u64 x[kUnroll][NP];
 #pragma unroll
-    for (int d = 0; d < NP; ++d) x[d] = digits[d * digit_stride + dbase + i];
-    for (u32 op = blockIdx.z; op < n_ops; op += gridDim.z) {
-      const u64* __restrict__ key0 = keys.p[op] + kbase + i;
-      const u64* __restrict__ key1 = key0 + key1_off;
+  for (int u = 0; u < kUnroll; ++u) {
+    const u64 i = i0 + u * kThreads;
+#pragma unroll
+    for (int d = 0; d < NP; ++d) x[u][d] = i < n ? digits[d * digit_stride + dbase + i] : 0;
+  }
+  for (u32 op = blockIdx.z; op < n_ops; op += gridDim.z) {
+    const u64* __restrict__ key0 = keys.p[op] + kbase;
+    const u64* __restrict__ key1 = key0 + key1_off;
+    u64 k0[kUnroll][NP], k1[kUnroll][NP];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const u64 i = i0 + u * kThreads;
+#pragma unroll
+      for (int d = 0; d < NP; ++d) {
+        k0[u][d] = i < n ? key0[d * key_stride + i] : 0;
+        k1[u][d] = i < n ? key1[d * key_stride + i] : 0;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const u64 i = i0 + u * kThreads;
       u64 h0 = 0, l0 = 0, h1 = 0, l1 = 0;
 #pragma unroll
       for (int d = 0; d < NP; ++d) {
-        mac128(h0, l0, x[d], key0[d * key_stride]);
-        mac128(h1, l1, x[d], key1[d * key_stride]);
+        mac128(h0, l0, x[u][d], k0[u][d]);
+        mac128(h1, l1, x[u][d], k1[u][d]);
       }
-      out0[op * out_stride + dbase + i] = barrett128(h0, l0, P);
-      out1[op * out_stride + dbase + i] = barrett128(h1, l1, P);
+      if (i < n) {
+        out0[op * out_stride + dbase + i] = barrett128(h0, l0, P);
+        out1[op * out_stride + dbase + i] = barrett128(h1, l1, P);
+      }
     }
   }
 }
