@@ -71,6 +71,9 @@ def _sig(lib):
     f("ace_poly_automorphism", C.c_int, _vp, _vp, _vp, _vp, _sz, C.c_int)
     f("ace_decomp_modup", C.c_int, _vp, _vp, _vp, _sz, _sz, C.c_int)
     f("ace_mod_up", C.c_int, _vp, _vp, _vp, _sz, _sz, C.c_int)
+    f("ace_mod_down_rescale", C.c_int, _vp, _vp, _vp, _sz, C.c_int)
+    f("ace_reduce_rescale_modup", C.c_int, _vp, _vp, _vp, _vp, _sz, C.c_int)
+    f("ace_transform_from_level0", C.c_int, _vp, _vp, _vp, _sz)
     f("ace_precomp", C.c_int, _vp, _vp, _vp, _sz, C.c_int)
     f("ace_mod_down", C.c_int, _vp, _vp, _vp, _sz, C.c_int)
     f("ace_rescale", C.c_int, _vp, _vp, _vp, _sz, C.c_int)
@@ -96,7 +99,8 @@ EXPORTS = [
     "ace_hw_modadd", "ace_hw_modsub", "ace_hw_modmul", "ace_hw_modmuladd", "ace_hw_modadd_scalar",
     "ace_hw_modsub_scalar", "ace_hw_modmul_scalar", "ace_hw_modmuladd_scalar", "ace_hw_rotate",
     "ace_find_automorphism_index", "ace_automorphism_order", "ace_poly_add", "ace_poly_sub", "ace_poly_mul",
-    "ace_poly_automorphism", "ace_decomp_modup", "ace_mod_up", "ace_precomp", "ace_mod_down", "ace_rescale", "ace_extend",
+    "ace_poly_automorphism", "ace_decomp_modup", "ace_mod_up", "ace_mod_down_rescale",
+    "ace_reduce_rescale_modup", "ace_transform_from_level0", "ace_precomp", "ace_mod_down", "ace_rescale", "ace_extend",
     "ace_dot_prod", "ace_mul_ciph3", "ace_fast_switch_key", "ace_relin", "ace_rescale_ciph",
     "ace_mul_relin_rescale", "ace_mul_relin_rescale_batch", "ace_fast_rotate", "ace_rotate_batch",
 ]
@@ -286,6 +290,15 @@ class Context:
 
     def decomp_modup(self, res, src, level, part, is_ntt=True):
         self._chk(self.lib.ace_decomp_modup(self.h, res.ptr, src.ptr, level, part, int(is_ntt)))
+
+    def mod_down_rescale(self, res, poly, level, is_ntt=True):
+        self._chk(self.lib.ace_mod_down_rescale(self.h, res.ptr, poly.ptr, level, int(is_ntt)))
+
+    def reduce_rescale_modup(self, res, raised, poly, level, is_ntt=True):
+        self._chk(self.lib.ace_reduce_rescale_modup(self.h, res.ptr, raised.ptr, poly.ptr, level, int(is_ntt)))
+
+    def transform_from_level0(self, res, src, level):
+        self._chk(self.lib.ace_transform_from_level0(self.h, res.ptr, src.ptr, level))
 
     def mod_up(self, res, digit, level, part, is_ntt=True):
         self._chk(self.lib.ace_mod_up(self.h, res.ptr, digit.ptr, level, part, int(is_ntt)))

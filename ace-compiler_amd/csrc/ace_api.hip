@@ -438,6 +438,33 @@ void do_rescale(ace_ctx* c, const PolySeq& res, const PolySeq& src, size_t np, s
   c->ws_used = mark;
 }
 
+// Shared front of Mod_down_rescale and Reduce_and_rescale_modup: poly (level+K
+// limbs) goes to coefficient form in place, y = its P part in the Q basis
+// (level limbs), x = the fused Mod_down + rescale value (level-1 limbs,
+// coefficient form); last_out, when given, receives the reduced last limb.
+void do_moddown_rescale_core(ace_ctx* c, u64* x, u64* y, u64* last_out, u64* poly, size_t level, bool is_ntt) {
+  const size_t N = c->h.N, K = c->h.K;
+  if (is_ntt) {
+    LimbMap lm = poly_lm(c, level, true);
+    PolySeq ps = seq_strided(poly, 0);
+    launch_ntt(c->stream, c->d, ps, ps, lm, nullptr, (u32)(level + K), 1, true, nullptr);
+  }
+  size_t mark = c->ws_used;
+  u64* t = c->take(K * N);
+  launch_mul_const(c->stream, c->d, t, poly + level * N, c->pscale_coef, c->p_lm, (u32)K);
+  ConvBatch b{};
+  b.n_jobs = 1;
+  b.job[0].hat = c->phat;
+  b.job[0].hat_stride = (u32)c->h.L;
+  b.job[0].nd = (u32)K;
+  b.job[0].nc = (u32)level;
+  for (size_t i = 0; i < level; ++i) { b.job[0].map.prime[i] = (uint8_t)i; b.job[0].map.out_limb[i] = (uint8_t)i; }
+  launch_baseconv(c->stream, c->d, y, t, b, 1);
+  const RescaleDev& r = c->rescale_at(level);
+  launch_moddown_rescale(c->stream, c->d, x, poly, y, last_out, c->pinv, r.tail, (u32)level);
+  c->ws_used = mark;
+}
+
 // key limb positions of a polynomial viewed at `level` (Derive_poly, rns_poly.c:701-707)
 LimbMap key_pos(const ace_ctx* c, size_t level) {
   LimbMap kp{};
@@ -856,6 +883,48 @@ int ace_rescale(ace_ctx* c, int64_t* res, const int64_t* src, size_t level, int 
   c->ensure_ws(c->std_ws(level));
   c->ws_used = 0;
   do_rescale(c, seq_strided(U(res), 0), seq_strided(U(src), 0), 1, level, is_ntt != 0);
+  ACE_CATCH_INT
+}
+
+int ace_mod_down_rescale(ace_ctx* c, int64_t* res, int64_t* poly, size_t level, int is_ntt) {
+  ACE_TRY
+  if (!res || !poly) return fail("ace_mod_down_rescale: null argument");
+  if (level < 2 || level > c->h.L) return fail("ace_mod_down_rescale: level out of range");
+  if (res == poly) return fail("ace_mod_down_rescale: the result must not overwrite the operand");
+  c->ensure_ws(c->std_ws(level));
+  c->ws_used = 0;
+  u64* y = c->take(level * (size_t)c->h.N);
+  do_moddown_rescale_core(c, U(res), y, nullptr, U(poly), level, is_ntt != 0);
+  PolySeq rs = seq_strided(U(res), 0);
+  launch_ntt(c->stream, c->d, rs, rs, c->q_lm, nullptr, (u32)(level - 1), 1, false, nullptr);
+  ACE_CATCH_INT
+}
+
+int ace_reduce_rescale_modup(ace_ctx* c, int64_t* res, int64_t* raised, int64_t* poly, size_t level, int is_ntt) {
+  ACE_TRY
+  if (!res || !raised || !poly) return fail("ace_reduce_rescale_modup: null argument");
+  if (level < 2 || level > c->h.L) return fail("ace_reduce_rescale_modup: level out of range");
+  if (res == poly || raised == poly || raised == res) return fail("ace_reduce_rescale_modup: buffers must be distinct");
+  c->ensure_ws(c->std_ws(level));
+  c->ws_used = 0;
+  const size_t N = c->h.N, nl = level - 1;
+  u64* x = c->take(nl * N);
+  u64* last = c->take(N);
+  // the reference leaves the converted P part in res and the reduced last limb in its limb level-1;
+  // the kernel reads that limb of y from every block, so the reduced value goes to scratch first
+  do_moddown_rescale_core(c, x, U(res), last, U(poly), level, is_ntt != 0);
+  HIP_OK(hipMemcpyAsync(U(res) + nl * N, last, N * sizeof(u64), hipMemcpyDeviceToDevice, c->stream));
+  do_precomp(c, U(raised), 0, x, 0, 1, nl, false);
+  ACE_CATCH_INT
+}
+
+int ace_transform_from_level0(ace_ctx* c, int64_t* res, const int64_t* src, size_t level) {
+  ACE_TRY
+  if (!res || !src) return fail("ace_transform_from_level0: null argument");
+  if (!level_ok(c, level)) return fail("ace_transform_from_level0: level out of range");
+  if (res != src && res < src + c->h.N && src < res + level * (size_t)c->h.N)
+    return fail("ace_transform_from_level0: buffers overlap");
+  launch_from_level0(c->stream, c->d, U(res), U(src), (u32)level);
   ACE_CATCH_INT
 }
 

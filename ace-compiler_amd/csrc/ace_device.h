@@ -112,6 +112,19 @@ __device__ __forceinline__ u64 barrett128(u64 hi, u64 lo, const DevPrime& p) {
   return csub(csub(r, p.q), p.q);
 }
 
+// Sub_mul_const_mod (modular.h:262-276), literally: ((v1 - v2) * w) mod q with the
+// Shoup companion wp.  One +q after the subtraction; if the difference is still
+// negative (v2 a residue of a larger prime) the reference's casts decide the
+// value: the 128-bit product sees the sign-extended difference, i.e. the high
+// word of s*wp taken as unsigned minus wp.
+__device__ __forceinline__ u64 sub_mul_const(u64 v1, u64 v2, u64 w, u64 wp, u64 q) {
+  i64 s = (i64)v1 - (i64)v2;
+  if (s < 0) s += (i64)q;
+  u64 qq = __umul64hi((u64)s, wp) - (s < 0 ? wp : 0);
+  u64 y = (u64)s * w - qq * q;
+  return y >= q ? y - q : y;
+}
+
 // acc += a*b over 128 bits
 __device__ __forceinline__ void mac128(u64& hi, u64& lo, u64 a, u64 b) {
   u64 pl = a * b, ph = __umul64hi(a, b);

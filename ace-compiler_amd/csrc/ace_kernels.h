@@ -79,6 +79,11 @@ void launch_rescale_tail(hipStream_t st, const DevCtx& c, const PolySeq& out, co
 // coefficient-form rescale: out = (src - (last mod q_t)) * qlinv
 void launch_rescale_coef(hipStream_t st, const DevCtx& c, u64* out, const u64* src, const u64* last,
                          const u64* cst, const LimbMap& lm, u32 n_limbs);
+// fused Mod_down + rescale tail in coefficient form (see moddown_rescale_kernel); out: level-1 limbs
+void launch_moddown_rescale(hipStream_t st, const DevCtx& c, u64* out, const u64* poly, const u64* y, u64* last_out,
+                            const u64* pinv, const u64* qlinv, u32 level);
+// out[0] = src, out[i] = Switch_modulus(src, q_0 -> q_i) for i < level
+void launch_from_level0(hipStream_t st, const DevCtx& c, u64* out, const u64* src, u32 level);
 // dst[p][i] = limb `limb` of polynomial p of src
 void launch_pick_limb(hipStream_t st, const DevCtx& c, u64* dst, const PolySeq& src, u32 limb, u32 n_polys);
 // out[t] = src[t] * cst[2t] (Shoup constant per limb)

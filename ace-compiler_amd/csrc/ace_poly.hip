@@ -496,6 +496,67 @@ void launch_rescale_coef(hipStream_t st, const DevCtx& c, u64* out, const u64* s
   hipLaunchKernelGGL(rescale_coef_kernel, ew_grid(c.N, n_limbs), dim3(kThreads), 0, st, c, out, src, last, cst, lm);
 }
 
+// ---- Mod_down_rescale / Reduce_and_rescale_modup tail (rns_poly.c:555-590,
+// rns_poly_impl.c:549-607), coefficient form ---------------------------------
+// y holds the P part converted to the Q basis (level limbs).  For limb i < level-1:
+//   last = (poly_last - y_last) * P^-1 mod q_last
+//   out_i = (((poly_i - y_i) * P^-1 mod q_i) - last) * q_last^-1 mod q_i
+// with Sub_mul_const_mod's exact semantics.  When last_out is given, the blocks of
+// limb 0 also store `last` there; it must not alias y (every block reads y_last).
+// pinv / qlinv: (constant, Shoup) pairs per limb.
+__global__ __launch_bounds__(kThreads) void moddown_rescale_kernel(DevCtx c, u64* __restrict__ out,
+                                                                   const u64* __restrict__ poly,
+                                                                   const u64* __restrict__ y,
+                                                                   u64* __restrict__ last_out,
+                                                                   const u64* __restrict__ pinv,
+                                                                   const u64* __restrict__ qlinv, u32 level) {
+  const u32 limb = blockIdx.y, last = level - 1;
+  const u64 q = c.primes[limb].q, ql = c.primes[last].q;
+  const u64 w = pinv[2 * limb], wp = pinv[2 * limb + 1], wl = pinv[2 * last], wlp = pinv[2 * last + 1];
+  const u64 v = qlinv[2 * limb], vp = qlinv[2 * limb + 1];
+  const u64 n = c.N, base = (u64)limb * n, lbase = (u64)last * n;
+#pragma unroll
+  ACE_EW_LOOP(i, n) {
+    u64 lastv = sub_mul_const(poly[lbase + i], y[lbase + i], wl, wlp, ql);
+    u64 t = sub_mul_const(poly[base + i], y[base + i], w, wp, q);
+    out[base + i] = sub_mul_const(t, lastv, v, vp, q);
+    if (last_out && limb == 0) last_out[i] = lastv;
+  }
+}
+void launch_moddown_rescale(hipStream_t st, const DevCtx& c, u64* out, const u64* poly, const u64* y, u64* last_out,
+                            const u64* pinv, const u64* qlinv, u32 level) {
+  if (level < 2) return;
+  hipLaunchKernelGGL(moddown_rescale_kernel, ew_grid(c.N, level - 1), dim3(kThreads), 0, st, c, out, poly, y,
+                     last_out, pinv, qlinv, level);
+}
+
+// ---- Transform_values_from_level0 (rns_poly.c:1101-1125) ---------------------
+// out limb 0 = src; out limb i = Switch_modulus(src, q_0 -> q_i) (modular.h:296-322)
+__global__ __launch_bounds__(kThreads) void from_level0_kernel(DevCtx c, u64* __restrict__ out,
+                                                               const u64* __restrict__ src) {
+  const u32 limb = blockIdx.y;
+  const DevPrime P = c.primes[limb];
+  const u64 q0 = c.primes[0].q, half = q0 >> 1;
+  const u64 n = c.N, base = (u64)limb * n;
+#pragma unroll
+  ACE_EW_LOOP(i, n) {
+    u64 v = src[i];
+    if (limb != 0) {
+      if (P.q > q0) {
+        if (v > half) v += P.q - q0;
+      } else {
+        if (v > half) v += P.q - (q0 % P.q);
+        if (v >= P.q) v = barrett128(0, v, P);
+      }
+    }
+    out[base + i] = v;
+  }
+}
+void launch_from_level0(hipStream_t st, const DevCtx& c, u64* out, const u64* src, u32 level) {
+  if (!level) return;
+  hipLaunchKernelGGL(from_level0_kernel, ew_grid(c.N, level), dim3(kThreads), 0, st, c, out, src);
+}
+
 // gathers limb `limb` of every polynomial of a sequence into a dense buffer
 __global__ __launch_bounds__(kThreads) void pick_limb_kernel(u64* __restrict__ dst, PolySeq srcs, u64 n, u32 limb) {
   const u32 p = blockIdx.z;

@@ -223,6 +223,8 @@ POLY     Decomp_modup(POLY res, POLY poly, uint32_t q_part_idx);
 POLY     Mod_down(POLY res, POLY poly);
 POLY     Rescale(POLY res, POLY poly);
 POLY     Modswitch(POLY res, POLY poly);
+POLY     Mod_down_rescale(POLY res, POLY poly); /* poly is left in coefficient form, as in the reference */
+void     Transform_values_from_level0(POLY res, POLY poly);
 POLY_ARR Precomp(POLY_ARR res, size_t size, POLY input);
 POLY_ARR Rt_alloc_precomp(POLY input, size_t* size); /* Alloc_precomp (rns_poly.c:471-481) without the VALUE_LIST box */
 void     Rt_free_precomp(POLY_ARR digits);

@@ -320,6 +320,24 @@ POLY Rescale(POLY res, POLY poly) {
   return res;
 }
 
+POLY Mod_down_rescale(POLY res, POLY poly) {
+  need_packed_ext(poly, "Mod_down_rescale");
+  size_t level = poly->_num_primes;
+  FMT_ASSERT(res->_ring_degree == poly->_ring_degree && res->_num_primes == level && level > 1 && res->_num_primes_p == 0,
+             "Reduce_and_rescale_rns: size not match");
+  ACE_OK(ace_mod_down_rescale(G.ctx, res->_data, poly->_data, level, poly->_is_ntt));
+  poly->_is_ntt = false;
+  Set_poly_level(res, level - 1);
+  res->_is_ntt = true;
+  return res;
+}
+
+void Transform_values_from_level0(POLY res, POLY poly) {
+  FMT_ASSERT(res->_ring_degree == poly->_ring_degree, "unmatched ring degree");
+  FMT_ASSERT(Get_poly_alloc_len(res) >= Get_poly_len(poly) && res->_num_alloc_primes <= G.L, "not enough memory");
+  ACE_OK(ace_transform_from_level0(G.ctx, res->_data, poly->_data, res->_num_primes));
+}
+
 POLY_ARR Precomp(POLY_ARR res, size_t size, POLY input) {
   size_t level = input->_num_primes, T = level + G.K;
   FMT_ASSERT(size == ace_num_decomp(G.ctx, level), "length of precompute not match");

@@ -148,6 +148,19 @@ int ace_precomp(ace_ctx* ctx, int64_t* res, const int64_t* src, size_t level, in
 int ace_mod_down(ace_ctx* ctx, int64_t* res, const int64_t* src, size_t level, int is_ntt);
 /* Rescale (:310-404): src level limbs -> res level-1 limbs */
 int ace_rescale(ace_ctx* ctx, int64_t* res, const int64_t* src, size_t level, int is_ntt);
+/* Mod_down_rescale (:531-597): Mod_down and rescale in one pass over the coefficient
+ * form.  `poly` (level + num_p limbs) is converted to coefficient form IN PLACE, as the
+ * reference does to its argument; res receives level-1 limbs in NTT form. */
+int ace_mod_down_rescale(ace_ctx* ctx, int64_t* res, int64_t* poly, size_t level, int is_ntt);
+/* Reduce_and_rescale_modup (poly/src/rns_poly_impl.c:521-620): the same value, left in
+ * coefficient form and raised digit by digit: `raised` = num_decomp(level-1) polynomials of
+ * (level-1 + num_p) limbs, coefficient form.  `res` (level limbs) is left as the reference
+ * leaves it: the converted P part in limbs 0..level-2, the reduced last limb in limb level-1.
+ * `poly` is converted to coefficient form in place. */
+int ace_reduce_rescale_modup(ace_ctx* ctx, int64_t* res, int64_t* raised, int64_t* poly, size_t level, int is_ntt);
+/* Transform_values_from_level0 (:1101-1125): limb 0 of src copied, limb i of res =
+ * Switch_modulus(limb 0, q_0 -> q_i), i < level. */
+int ace_transform_from_level0(ace_ctx* ctx, int64_t* res, const int64_t* src, size_t level);
 /* Extend (:483-500): src level limbs -> res level+num_p limbs (P limbs zero) */
 int ace_extend(ace_ctx* ctx, int64_t* res, const int64_t* src, size_t level);
 /* Dot_prod / Fast_dot_prod (:502-529): digits = n_parts x (level+num_p) limbs;

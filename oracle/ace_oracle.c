@@ -936,6 +936,105 @@ void orc_rescale(const orc_ctx* c, int64_t* out, const int64_t* in, size_t level
   }
 }
 
+/* modular.h:262-276 Sub_mul_const_mod, literally: ((v1 - v2) * w) mod q with a
+ * Shoup constant, one conditional +q after the subtraction.  When v2 exceeds
+ * v1 + q (possible where v2 is a residue of a LARGER prime, as in
+ * Mod_down_rescale) the difference stays negative and the reference's casts
+ * decide the value; they are reproduced here: (UINT128_T)int64 sign-extends,
+ * int64 * uint64 wraps modulo 2^64. */
+static inline i64 sub_mul_const(u64 v1, u64 v2, u64 w, u64 wp, u64 q) {
+  i64 s = (i64)v1 - (i64)v2;
+  if (s < 0) s += (i64)q;
+  u64 qq = (u64)(((u128)(i128)s * wp) >> 64);
+  u64 y  = ((u64)s * w) - qq * q;
+  return (i64)(y >= q ? y - q : y);
+}
+int64_t orc_sub_mul_const(uint64_t v1, uint64_t v2, uint64_t w, uint64_t wp, uint64_t q) {
+  return sub_mul_const(v1, v2, w, wp, q);
+}
+
+/* shared front of Mod_down_rescale (rns_poly.c:531-597) and
+ * Reduce_and_rescale_modup (rns_poly_impl.c:521-620): the input is brought to
+ * coefficient form IN PLACE (all level+K limbs), its P part is converted to the
+ * Q basis into y, and limb level-1 of y becomes (old - y) * P^-1 mod q_last. */
+static void moddown_rescale_front(const orc_ctx* c, i64* y, i64* poly, size_t level, int is_ntt) {
+  size_t N = c->N, K = c->K;
+  int32_t idx[128];
+  if (is_ntt) {
+    for (size_t i = 0; i < level; i++) idx[i] = (int32_t)i;
+    for (size_t j = 0; j < K; j++) idx[level + j] = (int32_t)(c->L + j);
+    orc_intt(c, poly, poly, idx, level + K);
+  }
+  base_conv_p2q(c, y, poly + level * N, level);
+  i64* phat_inv = (i64*)malloc(sizeof(i64) * K);
+  i64* phat     = (i64*)malloc(sizeof(i64) * c->L * K);
+  i64* pinv     = (i64*)malloc(sizeof(i64) * c->L);
+  i64* pmod     = (i64*)malloc(sizeof(i64) * c->L);
+  orc_tbl_moddown(c, phat_inv, phat, pinv, pmod);
+  size_t last = level - 1;
+  u64 ql = (u64)c->mod[last].val, w = (u64)pinv[last], wp = orc_precompute_const(w, ql);
+  for (size_t n = 0; n < N; n++)
+    y[last * N + n] = sub_mul_const((u64)poly[last * N + n], (u64)y[last * N + n], w, wp, ql);
+  free(phat_inv); free(phat); free(pinv); free(pmod);
+}
+
+/* value of limb i < level-1 after the fused Mod_down and rescale */
+static void moddown_rescale_limb(const orc_ctx* c, i64* dst, const i64* poly, const i64* y, size_t level, size_t i) {
+  size_t N = c->N, last = level - 1;
+  i64 ql_inv[64], qlql[64];
+  orc_tbl_rescale(c, level, ql_inv, qlql);
+  i64* phat_inv = (i64*)malloc(sizeof(i64) * c->K);
+  i64* phat     = (i64*)malloc(sizeof(i64) * c->L * c->K);
+  i64* pinv     = (i64*)malloc(sizeof(i64) * c->L);
+  i64* pmod     = (i64*)malloc(sizeof(i64) * c->L);
+  orc_tbl_moddown(c, phat_inv, phat, pinv, pmod);
+  u64 q = (u64)c->mod[i].val;
+  u64 w = (u64)pinv[i], wp = orc_precompute_const(w, q);
+  u64 v = (u64)ql_inv[i], vp = orc_precompute_const(v, q);
+  for (size_t n = 0; n < N; n++) {
+    i64 t = sub_mul_const((u64)poly[i * N + n], (u64)y[i * N + n], w, wp, q);
+    dst[n] = sub_mul_const((u64)t, (u64)y[last * N + n], v, vp, q);
+  }
+  free(phat_inv); free(phat); free(pinv); free(pmod);
+}
+
+/* rns_poly.c:531-597.  poly: (level+K) limbs, converted to coefficient form in
+ * place (the reference does the same to its argument); out: level-1 limbs, NTT form. */
+void orc_mod_down_rescale(const orc_ctx* c, int64_t* out, int64_t* poly, size_t level, int is_ntt) {
+  ORC_ASSERT(level >= 2, "Mod_down_rescale: level too small");
+  size_t N = c->N;
+  i64* y = (i64*)malloc(sizeof(i64) * level * N);
+  moddown_rescale_front(c, y, poly, level, is_ntt);
+  for (size_t i = 0; i + 1 < level; i++) moddown_rescale_limb(c, out + i * N, poly, y, level, i);
+  int32_t idx[128];
+  for (size_t i = 0; i + 1 < level; i++) idx[i] = (int32_t)i;
+  orc_ntt(c, out, out, idx, level - 1);
+  free(y);
+}
+
+/* rns_poly_impl.c:521-620.  res: level limbs as the reference leaves them (the
+ * converted P part in limbs 0..level-2, the reduced last limb in limb level-1;
+ * its level is then lowered by one).  raised: num_decomp(level-1) polynomials
+ * of (level-1+K) limbs, coefficient form: the rescaled value in each digit's
+ * own limbs, its base conversion (Modup_inplace, rns_poly_impl.c:380-434) elsewhere. */
+void orc_reduce_rescale_modup(const orc_ctx* c, int64_t* res, int64_t* raised, int64_t* poly, size_t level, int is_ntt) {
+  ORC_ASSERT(level >= 2, "Reduce_and_rescale_modup: level too small");
+  size_t N = c->N, nl = level - 1;
+  moddown_rescale_front(c, res, poly, level, is_ntt);
+  i64* x = (i64*)malloc(sizeof(i64) * nl * N);
+  for (size_t i = 0; i < nl; i++) moddown_rescale_limb(c, x + i * N, poly, res, level, i);
+  orc_precomp(c, raised, x, nl, 0, 1);
+  free(x);
+}
+
+/* rns_poly.c:1101-1125: limb 0 copied, limb i = Switch_modulus(limb 0, q_0 -> q_i) */
+void orc_transform_from_level0(const orc_ctx* c, int64_t* out, const int64_t* in, size_t level) {
+  size_t N = c->N;
+  memcpy(out, in, sizeof(i64) * N);
+  for (size_t i = 1; i < level; i++)
+    for (size_t n = 0; n < N; n++) out[i * N + n] = orc_switch_modulus(in[n], c->mod[0].val, c->mod[i].val);
+}
+
 /* rns_poly.c:483-500 */
 void orc_extend(const orc_ctx* c, int64_t* out, const int64_t* in, size_t level) {
   size_t N = c->N, K = c->K;

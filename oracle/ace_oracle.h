@@ -126,6 +126,14 @@ void orc_mod_down(const orc_ctx* c, int64_t* out, const int64_t* in, size_t leve
 void orc_rescale(const orc_ctx* c, int64_t* out, const int64_t* in, size_t level, int is_ntt);
 /* :483-500 Extend: in level limbs -> out level+num_p limbs (P part zero) */
 void orc_extend(const orc_ctx* c, int64_t* out, const int64_t* in, size_t level);
+/* Sub_mul_const_mod (include/util/modular.h:262-276) */
+int64_t orc_sub_mul_const(uint64_t v1, uint64_t v2, uint64_t w, uint64_t wp, uint64_t q);
+/* Mod_down_rescale (rns_poly.c:531-597): poly (level+K limbs) is converted to coefficient form in place */
+void orc_mod_down_rescale(const orc_ctx* c, int64_t* out, int64_t* poly, size_t level, int is_ntt);
+/* Reduce_and_rescale_modup (rns_poly_impl.c:521-620) */
+void orc_reduce_rescale_modup(const orc_ctx* c, int64_t* res, int64_t* raised, int64_t* poly, size_t level, int is_ntt);
+/* Transform_values_from_level0 (rns_poly.c:1101-1125) */
+void orc_transform_from_level0(const orc_ctx* c, int64_t* out, const int64_t* in, size_t level);
 /* :502-529 Dot_prod / Fast_dot_prod.  digits: n_parts x (level+num_p) limbs.
  * key: n_parts polynomials of key_stride int64 each, laid out with all num_q
  * Q limbs followed by num_p P limbs; viewed at `level`. */

@@ -37,7 +37,7 @@ enum {
   OP_NTT = 1, OP_INTT, OP_HW, OP_DECOMP_MODUP, OP_PRECOMP, OP_MOD_DOWN,
   OP_RESCALE, OP_DOT_PROD, OP_AUTO_ORDER, OP_AUTO_INDEX, OP_AUTOMORPHISM,
   OP_EXTEND, OP_TBL_MODUP, OP_TBL_MODDOWN, OP_TBL_RESCALE, OP_POLY, OP_TWIDDLES,
-  OP_MOD_UP
+  OP_MOD_UP, OP_MOD_DOWN_RESCALE, OP_REDUCE_RESCALE_MODUP, OP_FROM_LEVEL0
 };
 
 static int64_t* in_buf;
@@ -189,6 +189,48 @@ int main(int argc, char** argv) {
         int64_t* out = (int64_t*)calloc(lv * N, sizeof(int64_t));
         wrap_poly(&res, out, lv, 0, a2 != 0);
         Mod_down(&res, &src);
+        wr1((int64_t)(lv * N));
+        wr(out, lv * N);
+        free(out);
+        break;
+      }
+      case OP_MOD_DOWN_RESCALE: { /* a1 level, a2 is_ntt; in = (level+K)*N; out = result, input as left */
+        size_t lv = (size_t)a1;
+        POLYNOMIAL src, res;
+        wrap_poly(&src, in, lv, K, a2 != 0);
+        int64_t* out = (int64_t*)calloc(lv * N, sizeof(int64_t));
+        wrap_poly(&res, out, lv, 0, a2 != 0);
+        Mod_down_rescale(&res, &src);
+        wr1((int64_t)((lv - 1) * N + (lv + K) * N + 1));
+        wr(out, (lv - 1) * N);
+        wr(in, (lv + K) * N);
+        wr1((int64_t)Is_ntt(&res));
+        free(out);
+        break;
+      }
+      case OP_REDUCE_RESCALE_MODUP: { /* a1 level, a2 is_ntt; in = (level+K)*N; out = res[level], raised, input */
+        size_t lv = (size_t)a1;
+        POLYNOMIAL src, res;
+        wrap_poly(&src, in, lv, K, a2 != 0);
+        int64_t* out = (int64_t*)calloc(lv * N, sizeof(int64_t));
+        wrap_poly(&res, out, lv, 0, a2 != 0);
+        VALUE_LIST* raised = Reduce_and_rescale_modup(&res, &src);
+        size_t nd = LIST_LEN(raised), each = (lv - 1 + K) * N;
+        wr1((int64_t)(lv * N + nd * each + (lv + K) * N));
+        wr(out, lv * N);
+        for (size_t d = 0; d < nd; d++) wr(Get_poly_coeffs((POLYNOMIAL*)Get_ptr_value_at(raised, d)), each);
+        wr(in, (lv + K) * N);
+        Free_precomp(raised);
+        free(out);
+        break;
+      }
+      case OP_FROM_LEVEL0: { /* a1 level; in = N words (limb 0) */
+        size_t lv = (size_t)a1;
+        POLYNOMIAL src, res;
+        wrap_poly(&src, in, 1, 0, false);
+        int64_t* out = (int64_t*)calloc(lv * N, sizeof(int64_t));
+        wrap_poly(&res, out, lv, 0, false);
+        Transform_values_from_level0(&res, &src);
         wr1((int64_t)(lv * N));
         wr(out, lv * N);
         free(out);

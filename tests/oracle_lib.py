@@ -69,6 +69,8 @@ def lib():
         L.orc_precompute_const.argtypes = [C.c_uint64, C.c_uint64]
         L.orc_fast_mul_const.restype = C.c_int64
         L.orc_fast_mul_const.argtypes = [C.c_uint64] * 4
+        L.orc_sub_mul_const.restype = C.c_int64
+        L.orc_sub_mul_const.argtypes = [C.c_uint64] * 5
         L.orc_mod_inv.restype = C.c_int64
         L.orc_mod_inv.argtypes = [C.c_int64, C.c_int64]
         L.orc_is_prime.restype = C.c_int
@@ -211,6 +213,28 @@ class Oracle:
         src = np.ascontiguousarray(src, dtype=np.int64)
         out = np.zeros((level + self.K) * self.N, np.int64)
         self.L_.orc_extend(self.h, _ptr(out), _ptr(src), C.c_size_t(level))
+        return out
+
+    def mod_down_rescale(self, src, level, is_ntt=True):
+        """Returns (result at level-1 in NTT form, the input as the call leaves it: coefficient form)."""
+        poly = np.array(src, dtype=np.int64, copy=True)
+        out = np.zeros((level - 1) * self.N, np.int64)
+        self.L_.orc_mod_down_rescale(self.h, _ptr(out), _ptr(poly), C.c_size_t(level), C.c_int(int(is_ntt)))
+        return out, poly
+
+    def reduce_rescale_modup(self, src, level, is_ntt=True):
+        """Returns (res as left by the call: level limbs, raised digits, the input in coefficient form)."""
+        poly = np.array(src, dtype=np.int64, copy=True)
+        res = np.zeros(level * self.N, np.int64)
+        raised = np.zeros(self.num_decomp(level - 1) * (level - 1 + self.K) * self.N, np.int64)
+        self.L_.orc_reduce_rescale_modup(self.h, _ptr(res), _ptr(raised), _ptr(poly), C.c_size_t(level),
+                                         C.c_int(int(is_ntt)))
+        return res, raised, poly
+
+    def transform_from_level0(self, src, level):
+        src = np.ascontiguousarray(src, dtype=np.int64)
+        out = np.zeros(level * self.N, np.int64)
+        self.L_.orc_transform_from_level0(self.h, _ptr(out), _ptr(src), C.c_size_t(level))
         return out
 
     def dot_prod(self, digits, key, n_parts, level, fast=False):

@@ -205,6 +205,38 @@ def test_mod_down_rescale_extend(pair):
             g.rescale(g.alloc(N), g.alloc(N), 1, True)
 
 
+def test_mod_down_rescale_family(pair):
+    """Mod_down_rescale, Reduce_and_rescale_modup (both mutate their operand) and Transform_values_from_level0."""
+    g, o = pair.g, pair.o
+    N = g.N
+    for level in [l for l in levels_of(g) if l >= 2]:
+        pr = [g.primes[i] for i in g.limb_primes(level)]
+        e = seeded.uniform_poly(250 + level, pr, N)
+        for is_ntt in (True, False):
+            want, left = o.mod_down_rescale(e, level, is_ntt)
+            de = g.upload(e)
+            dr = g.alloc((level - 1) * N)
+            g.mod_down_rescale(dr, de, level, is_ntt)
+            eq(dr, want, "mod_down_rescale l=%d ntt=%d" % (level, is_ntt))
+            eq(de, left, "mod_down_rescale operand afterwards l=%d ntt=%d" % (level, is_ntt))
+            wres, wraised, left = o.reduce_rescale_modup(e, level, is_ntt)
+            de = g.upload(e)
+            dres, draised = g.alloc(level * N), g.alloc(wraised.size)
+            g.reduce_rescale_modup(dres, draised, de, level, is_ntt)
+            eq(dres, wres, "reduce_rescale_modup res l=%d ntt=%d" % (level, is_ntt))
+            eq(draised, wraised, "reduce_rescale_modup raised l=%d ntt=%d" % (level, is_ntt))
+            eq(de, left, "reduce_rescale_modup operand afterwards l=%d ntt=%d" % (level, is_ntt))
+    for level in levels_of(g):
+        x = seeded.uniform_limb(260 + level, g.primes[0], N)
+        x[:3] = [0, g.primes[0] - 1, g.primes[0] // 2 + 1][:min(3, N)]
+        dx = g.upload(x)
+        dr = g.alloc(level * N)
+        g.transform_from_level0(dr, dx, level)
+        eq(dr, o.transform_from_level0(x, level), "transform_from_level0 l=%d" % level)
+    with pytest.raises(acefhe.AceError):
+        g.mod_down_rescale(g.alloc(N), g.alloc(N), 1, True)
+
+
 def make_swk(g, seed):
     return np.concatenate([seeded.uniform_poly(seed + i, g.primes, g.N) for i in range(2 * g.parts)])
 

@@ -359,3 +359,24 @@ def test_keyswitch_decrypts(ctx):
         v %= Q
         v = v - Q if v > Q // 2 else v
         assert abs(v) < 2 ** 30, "key-switch noise too large: wrong digit/key/limb pairing"
+
+
+def test_sub_mul_const_matches_its_c_semantics():
+    """(v1 - v2) * w mod q where it is a plain modular product, and the wrapped value where v2 > v1 + q."""
+    import ctypes as C
+    from oracle_lib import lib
+    L_ = lib()
+    q = (1 << 40) + 15 * 128 + 1
+    rng = np.random.default_rng(5)
+    for _ in range(200):
+        w = int(rng.integers(1, q))
+        wp = (w << 64) // q
+        v1, v2 = int(rng.integers(0, q)), int(rng.integers(0, q))
+        assert L_.orc_sub_mul_const(v1, v2, w, wp, q) == (v1 - v2) * w % q
+        big = int(rng.integers(2 * q, 1 << 50))  # a residue of a larger prime
+        s_ = v1 - big + q
+        assert s_ < 0
+        m64 = (1 << 64) - 1
+        qq = ((s_ % (1 << 128)) * wp >> 64) & m64
+        y = ((s_ & m64) * w - qq * q) & m64
+        assert L_.orc_sub_mul_const(v1, big, w, wp, q) == C.c_int64(y - q if y >= q else y).value

@@ -86,6 +86,11 @@ def run_config(cfg, levels, heavy=True):
             q(refdrv.OP_MOD_DOWN, o.mod_down(e, level, is_ntt), level, is_ntt, 0, 0, e)
             if level >= 2:
                 q(refdrv.OP_RESCALE, o.rescale(c, level, is_ntt), level, is_ntt, 0, 0, c)
+                out, left = o.mod_down_rescale(e, level, is_ntt)
+                q(refdrv.OP_MOD_DOWN_RESCALE, np.concatenate([out, left, [1]]), level, is_ntt, 0, 0, e)
+                res_, raised, left = o.reduce_rescale_modup(e, level, is_ntt)
+                q(refdrv.OP_REDUCE_RESCALE_MODUP, np.concatenate([res_, raised, left]), level, is_ntt, 0, 0, e)
+        q(refdrv.OP_FROM_LEVEL0, o.transform_from_level0(c[:N], level), level, 0, 0, 0, c[:N])
         q(refdrv.OP_EXTEND, o.extend(c, level), level, 0, 0, 0, c)
         digits = np.concatenate([seeded.uniform_poly(300 + d, pr_qp, N) for d in range(nd)])
         key = np.concatenate([seeded.uniform_poly(400 + d, o.primes, N) for d in range(nd)])
@@ -140,4 +145,27 @@ def test_headline_config_tables_and_one_keyswitch():
     assert (res[0] == o.decomp_modup(c, level, 2, True)).all()
     assert (res[1] == o.mod_down(e, level, True)).all()
     assert (res[2] == o.rescale(c, level, True)).all()
+    o.close()
+
+
+def test_mod_down_rescale_with_a_small_first_prime():
+    """q_0 of 40 bits under 50-bit scaling primes: the last-limb value exceeds q_0, so Sub_mul_const_mod's
+    difference stays negative after its single +q and the reference's casts decide the result."""
+    cfg = (64, 4, 40, 50, 2)
+    N = cfg[0]
+    o = Oracle(*cfg)
+    s = RefSession(*cfg)
+    want = []
+    for level in (4, 3, 2):
+        e = seeded.uniform_poly(7 + level, [o.primes[i] for i in o.limb_primes(level)], N)
+        for is_ntt in (1, 0):
+            out, left = o.mod_down_rescale(e, level, is_ntt)
+            s.add(refdrv.OP_MOD_DOWN_RESCALE, level, is_ntt, 0, 0, e)
+            want.append(np.concatenate([out, left, [1]]))
+            res_, raised, left = o.reduce_rescale_modup(e, level, is_ntt)
+            s.add(refdrv.OP_REDUCE_RESCALE_MODUP, level, is_ntt, 0, 0, e)
+            want.append(np.concatenate([res_, raised, left]))
+    _, res = s.run()
+    for got, w in zip(res, want):
+        assert np.array_equal(got, w)
     o.close()

@@ -18,7 +18,7 @@ def test_library_exports():
     lib = ctypes.CDLL(os.path.join(ROOT, "ace-compiler_amd", "librt_hip.so"))
     for name in ("Prepare_context Finalize_context Run_main_graph Degree Get_q_cnt Get_p_cnt Get_q_parts Q_modulus "
                  "P_modulus Free_poly_data Alloc_polys Init_poly Copy_poly Decomp Mod_up Decomp_modup Mod_down Rescale "
-                 "Modswitch Precomp Dot_prod Extend Conv_poly2ntt_inplace Conv_ntt2poly_inplace Add_poly Sub_poly "
+                 "Modswitch Mod_down_rescale Transform_values_from_level0 Precomp Dot_prod Extend Conv_poly2ntt_inplace Conv_ntt2poly_inplace Add_poly Sub_poly "
                  "Mul_poly Hw_modadd Hw_modsub Hw_modmul Hw_modmuladd Hw_modadd_scalar Hw_modsub_scalar "
                  "Hw_modmul_scalar Hw_modmuladd_scalar Hw_rotate Hw_ntt Hw_intt Auto_idx Auto_order Swk Get_swk_at "
                  "Swk_c0 Swk_c1 Level Sc_degree Init_ciph_same_scale Init_ciph_up_scale Init_ciph_down_scale "
