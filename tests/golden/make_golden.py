@@ -48,6 +48,12 @@ def plan(cfg, info):
         ops.append(("mod_down_coef_l%d" % level, refdrv.OP_MOD_DOWN, (level, 0, 0, 0), [e]))
         ops.append(("rescale_l%d" % level, refdrv.OP_RESCALE, (level, 1, 0, 0), [c]))
         ops.append(("rescale_coef_l%d" % level, refdrv.OP_RESCALE, (level, 0, 0, 0), [c]))
+        # output, then the operand as the call leaves it (coefficient form), then the result's NTT flag
+        ops.append(("mod_down_rescale_l%d" % level, refdrv.OP_MOD_DOWN_RESCALE, (level, 1, 0, 0), [e]))
+        ops.append(("mod_down_rescale_coef_l%d" % level, refdrv.OP_MOD_DOWN_RESCALE, (level, 0, 0, 0), [e]))
+        # res as left by the call, the raised digits, the operand afterwards
+        ops.append(("reduce_rescale_modup_l%d" % level, refdrv.OP_REDUCE_RESCALE_MODUP, (level, 1, 0, 0), [e]))
+        ops.append(("from_level0_l%d" % level, refdrv.OP_FROM_LEVEL0, (level, 0, 0, 0), [c[:N]]))
         digits = np.concatenate([seeded.uniform_poly(300 + d, qp, N) for d in range(nd)])
         key = np.concatenate([seeded.uniform_poly(400 + d, primes, N) for d in range(nd)])
         ops.append(("dot_prod_l%d" % level, refdrv.OP_DOT_PROD, (level, nd, 0, 0), [digits, key]))

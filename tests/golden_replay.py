@@ -32,6 +32,13 @@ def run_op(impl, code, args, arrays):
         return impl.mod_down(arrays[0], args[0], bool(args[1]))
     if code == refdrv.OP_RESCALE:
         return impl.rescale(arrays[0], args[0], bool(args[1]))
+    if code == refdrv.OP_MOD_DOWN_RESCALE:
+        out, left = impl.mod_down_rescale(arrays[0], args[0], bool(args[1]))
+        return np.concatenate([out, left, [1]])
+    if code == refdrv.OP_REDUCE_RESCALE_MODUP:
+        return np.concatenate(impl.reduce_rescale_modup(arrays[0], args[0], bool(args[1])))
+    if code == refdrv.OP_FROM_LEVEL0:
+        return impl.transform_from_level0(arrays[0], args[0])
     if code == refdrv.OP_DOT_PROD:
         return impl.dot_prod(arrays[0], arrays[1], args[1], args[0])
     if code == refdrv.OP_AUTO_INDEX:
@@ -94,6 +101,26 @@ class GpuImpl:
 
     def rescale(self, x, level, is_ntt):
         return self._unary(self.g.rescale, x, (level - 1) * self.N, level, is_ntt)
+
+    def mod_down_rescale(self, x, level, is_ntt):
+        d, r = self.g.upload(x), self.g.alloc((level - 1) * self.N)
+        self.g.mod_down_rescale(r, d, level, is_ntt)
+        out = r.get(), d.get()
+        d.free()
+        r.free()
+        return out
+
+    def reduce_rescale_modup(self, x, level, is_ntt):
+        nd = self.g.num_decomp(level - 1)
+        d, r, up = self.g.upload(x), self.g.alloc(level * self.N), self.g.alloc(nd * (level - 1 + self.K) * self.N)
+        self.g.reduce_rescale_modup(r, up, d, level, is_ntt)
+        out = r.get(), up.get(), d.get()
+        for b in (d, r, up):
+            b.free()
+        return out
+
+    def transform_from_level0(self, x, level):
+        return self._unary(self.g.transform_from_level0, x, level * self.N, level)
 
     def dot_prod(self, digits, key, n_parts, level):
         dd, dk, r = self.g.upload(digits), self.g.upload(key), self.g.alloc((level + self.K) * self.N)
