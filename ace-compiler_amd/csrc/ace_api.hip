@@ -406,6 +406,19 @@ void do_mod_down(ace_ctx* c, const PolySeq& res, const PolySeq& src, size_t np, 
   launch_baseconv(c->stream, c->d, y, t, b, (u32)np);
   if (is_ntt) {
     PolySeq ys = seq_strided(y, level * N);
+    if (c->d.logN > 12 && !orders) {  // the tail rides on the transform's last kernel
+      FwdFuse f{};
+      f.epi = 1;
+      f.out = res;
+      f.src = src;
+      f.addend = addend_mode ? *addend : res;
+      f.addend_mode = addend_mode;
+      f.cst = c->pinv;
+      if (!launch_ntt(c->stream, c->d, ys, ys, c->q_lm, nullptr, (u32)level, (u32)np, false, nullptr, 3, &f))
+        throw std::runtime_error("internal: fused Mod_down transform rejected");
+      c->ws_used = mark;
+      return;
+    }
     launch_ntt(c->stream, c->d, ys, ys, c->q_lm, nullptr, (u32)level, (u32)np, false, nullptr);
   }
   launch_moddown_tail(c->stream, c->d, res, src, y, level * N, addend_mode ? addend : nullptr, addend_mode, c->pinv,
@@ -431,6 +444,23 @@ void do_rescale(ace_ctx* c, const PolySeq& res, const PolySeq& src, size_t np, s
   one.prime[0] = (uint8_t)(level - 1);
   PolySeq ls = seq_strided(last, N), us = seq_strided(u, (level - 1) * N);
   launch_ntt(c->stream, c->d, ls, ls, one, nullptr, 1, (u32)np, true, nullptr);
+  if (c->d.logN > 12) {  // modulus switch and tail ride on the transform's first and last kernels
+    FwdFuse f{};
+    f.pro = 1;
+    f.last = last;
+    f.last_stride = N;
+    f.last_prime = (u32)(level - 1);
+    f.sw = r.sw;
+    f.epi = 2;
+    f.out = res;
+    f.src = src;
+    f.addend = res;
+    f.cst = r.tail;
+    if (!launch_ntt(c->stream, c->d, us, us, c->q_lm, nullptr, (u32)(level - 1), (u32)np, false, nullptr, 3, &f))
+      throw std::runtime_error("internal: fused Rescale transform rejected");
+    c->ws_used = mark;
+    return;
+  }
   launch_rescale_switch(c->stream, c->d, u, (level - 1) * N, last, N, (u32)(level - 1), r.sw, c->q_lm,
                         (u32)(level - 1), (u32)np);
   launch_ntt(c->stream, c->d, us, us, c->q_lm, nullptr, (u32)(level - 1), (u32)np, false, nullptr);

@@ -143,4 +143,24 @@ __device__ __forceinline__ u64 sub_mod(u64 a, u64 b, u64 q) {
   return (u64)r;
 }
 
+
+// Work folded into a forward NTT of N > 4096 (launch_ntt): a prologue that forms
+// the transform's input on the fly, and an epilogue that consumes its output
+// instead of storing it.  Limb t of polynomial p is word offset pos[t]*N.
+//   pro 1  Rescale's modulus switch (rns_poly.c:340-360): input word i of limb t =
+//          Switch_modulus(last[p*last_stride + i], q_last -> q_t) * sw[3t] (Shoup sw[3t+1], sw[3t+2] = q_t - q_last mod q_t)
+//   epi 1  Mod_down tail (rns_poly.c:292-303): out = (src - ntt) * cst[2t] (+ addend)
+//   epi 2  Rescale tail (rns_poly.c:362-372):  out = src * cst[2t] + ntt
+// addend_mode: 0 none, 1 every polynomial, 2 even polynomials only.
+struct FwdFuse {
+  int pro, epi;
+  const u64* last;
+  u64 last_stride;
+  u32 last_prime;
+  const u64* sw;
+  PolySeq out, src, addend;
+  int addend_mode;
+  const u64* cst;
+};
+
 }  // namespace ace

@@ -37,8 +37,11 @@ struct OrderSet { // one automorphism table per rotation, or one shared (n == 1)
 // replacing 1/N in the inverse.
 // passes: for N > 4096 the transform is two kernels; bit 0 / bit 1 select them
 // (both by default; single passes exist so a benchmark can time each kernel).
+// fuse: optional prologue / epilogue of a whole forward transform of N > 4096 (FwdFuse); with an epilogue dst
+// only holds the intermediate between the two kernels.  Returns false when the request cannot be served.
 bool launch_ntt(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolySeq& src, const LimbMap& lm,
-                const LimbMap* pos, u32 n_limbs, u32 n_polys, bool inverse, const u64* scale, int passes = 3);
+                const LimbMap* pos, u32 n_limbs, u32 n_polys, bool inverse, const u64* scale, int passes = 3,
+                const FwdFuse* fuse = nullptr);
 
 // elementwise over n_limbs limbs of n words each (limb t uses lm.prime[t]);
 // scalar ops take the same scalar for every limb.

@@ -239,21 +239,42 @@ __device__ __forceinline__ void inv_strided_stages(const A& ar, typename A::T* v
 }
 
 // forward, strided pass: stages 0..LOGR-1.  grid = (N/R/256, n_limbs, n_polys)
-template <class A, int LOGR>
+// PRO = 1: the input is not read from src but formed from the last limb of a
+// rescale (FwdFuse::pro).
+template <class A, int LOGR, int PRO>
 __global__ __launch_bounds__(256) void ntt_fwd_strided(DevCtx c, PolySeq dsts, PolySeq srcs, LimbMap lm,
-                                                       LimbMap pos) {
+                                                       LimbMap pos, FwdFuse f) {
   constexpr int R = 1 << LOGR;
   const u32 col = blockIdx.x * 256 + threadIdx.x;
   const u32 limb = blockIdx.y, pi = lm.prime[limb];
   const u64 rs = c.N >> LOGR;  // row stride
   const u64 off = (u64)pos.prime[limb] * c.N + col;
   u64* __restrict__ dst = dsts.at(blockIdx.z);
-  const u64* __restrict__ src = srcs.at(blockIdx.z);
   A ar;
   ar.init(c, pi, false, nullptr, 0);
   typename A::T v[R];
+  if (PRO == 0) {
+    const u64* __restrict__ src = srcs.at(blockIdx.z);
 #pragma unroll
-  for (int r = 0; r < R; ++r) v[r] = ar.in_canon(src[off + r * rs]);
+    for (int r = 0; r < R; ++r) v[r] = ar.in_canon(src[off + r * rs]);
+  } else {
+    const DevPrime P = c.primes[pi];
+    const u32 lt = pos.prime[limb];
+    const u64 ql = c.primes[f.last_prime].q, half = ql >> 1;
+    const u64 K = f.sw[3 * lt], Kp = f.sw[3 * lt + 1], diff = f.sw[3 * lt + 2];
+    const u64* __restrict__ last = f.last + blockIdx.z * f.last_stride + col;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      u64 x = last[r * rs];
+      if (P.q > ql) {
+        if (x > half) x += P.q - ql;
+      } else {
+        if (x > half) x += diff;
+        if (x >= P.q) x = barrett128(0, x, P);
+      }
+      v[r] = ar.in_canon(shoup_mul(x, K, Kp, P.q));
+    }
+  }
   if (LOGR > 4) reduce_all<A, R>(ar, v);
   fwd_strided_stages<A, LOGR>(ar, v);
 #pragma unroll
@@ -299,9 +320,10 @@ constexpr bool kPrefetchTw = ACE_NTT_PREFETCH != 0;
 
 // forward, chunk pass: stages logr..logN-1 on 4096 contiguous words, in place.
 // grid = chunk_grid(n_limbs, ceil(n_polys / kPolysPerBlock))
-template <class A>
+// EPI != 0: the result is not stored back but consumed by FwdFuse::epi.
+template <class A, int EPI>
 __global__ __launch_bounds__(256) void ntt_fwd_chunk(DevCtx c, PolySeq datas, LimbMap lm, LimbMap pos, u32 logr,
-                                                     u32 n_limbs, u32 n_polys) {
+                                                     u32 n_limbs, u32 n_polys, FwdFuse f) {
   typedef typename A::T T;
   __shared__ T lds[kChunk + kChunk / 16];
   const int t = threadIdx.x;
@@ -390,8 +412,37 @@ __global__ __launch_bounds__(256) void ntt_fwd_chunk(DevCtx c, PolySeq datas, Li
     __syncthreads();
     // each thread reads back the words it will overwrite first in the next
     // iteration, so no further barrier is needed
+    if (EPI == 0) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) base[t + 256 * r] = ldsu[lds_pos(t + 256 * r)];
+      for (int r = 0; r < 16; ++r) base[t + 256 * r] = ldsu[lds_pos(t + 256 * r)];
+    } else {
+      const u32 p = poly0 + it, lt = pos.prime[limb];
+      const u64 q = c.primes[pi].q, w = f.cst[2 * lt], wp = f.cst[2 * lt + 1];
+      const u64 o = (u64)lt * c.N + (u64)chunk * kChunk + t;
+      u64* out = f.out.at(p) + o;  // may alias the addend (in-place relinearisation)
+      const u64* __restrict__ src = f.src.at(p) + o;
+      const u64* addend =
+          (EPI == 1 && (f.addend_mode == 1 || (f.addend_mode == 2 && !(p & 1)))) ? f.addend.at(p) + o : nullptr;
+      u64 sv[16], av[16];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sv[r] = src[256 * r];
+      if (addend) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) av[r] = addend[256 * r];
+      }
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const u64 y = ldsu[lds_pos(t + 256 * r)];
+        u64 v;
+        if (EPI == 1) {
+          v = shoup_mul(sub_mod(sv[r], y, q), w, wp, q);
+          if (addend) v = add_mod(v, av[r], q);
+        } else {
+          v = add_mod(shoup_mul(sv[r], w, wp, q), y, q);
+        }
+        out[256 * r] = v;
+      }
+    }
 #pragma unroll
     for (int r = 0; r < 16; ++r) raw[r] = nxt[r];
   }
@@ -571,13 +622,24 @@ __global__ __launch_bounds__(256) void ntt_small(DevCtx c, PolySeq dsts, PolySeq
 template <class A, int LOGR>
 static void run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolySeq& src, const LimbMap& lm,
                       const LimbMap& pos, const LimbMap& sidx, u32 n_limbs, u32 n_polys, bool inverse,
-                      const u64* scale, int passes) {
+                      const u64* scale, int passes, const FwdFuse& f) {
   dim3 gs((c.N >> LOGR) / 256, n_limbs, n_polys), gc(chunk_grid(c, n_limbs, (n_polys + kPolysPerBlock - 1) / kPolysPerBlock));
   if (!inverse) {
-    if (passes & 1)
-      hipLaunchKernelGGL((ntt_fwd_strided<A, LOGR>), gs, dim3(256), 0, st, c, dst, src, lm, pos);
-    if (passes & 2)
-      hipLaunchKernelGGL((ntt_fwd_chunk<A>), gc, dim3(256), 0, st, c, dst, lm, pos, (u32)LOGR, n_limbs, n_polys);
+    if (passes & 1) {
+      if (f.pro == 0)
+        hipLaunchKernelGGL((ntt_fwd_strided<A, LOGR, 0>), gs, dim3(256), 0, st, c, dst, src, lm, pos, f);
+      else
+        hipLaunchKernelGGL((ntt_fwd_strided<A, LOGR, 1>), gs, dim3(256), 0, st, c, dst, src, lm, pos, f);
+    }
+    if (passes & 2) {
+      const u32 lr = LOGR;
+      if (f.epi == 0)
+        hipLaunchKernelGGL((ntt_fwd_chunk<A, 0>), gc, dim3(256), 0, st, c, dst, lm, pos, lr, n_limbs, n_polys, f);
+      else if (f.epi == 1)
+        hipLaunchKernelGGL((ntt_fwd_chunk<A, 1>), gc, dim3(256), 0, st, c, dst, lm, pos, lr, n_limbs, n_polys, f);
+      else
+        hipLaunchKernelGGL((ntt_fwd_chunk<A, 2>), gc, dim3(256), 0, st, c, dst, lm, pos, lr, n_limbs, n_polys, f);
+    }
   } else {
     if (passes & 1)
       hipLaunchKernelGGL((ntt_inv_chunk<A>), gc, dim3(256), 0, st, c, dst, src, lm, pos, n_limbs, n_polys);
@@ -589,11 +651,11 @@ static void run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst, const
 template <class A>
 static bool run_large_dispatch(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolySeq& src,
                                const LimbMap& lm, const LimbMap& pos, const LimbMap& sidx, u32 n_limbs, u32 n_polys,
-                               bool inverse, const u64* scale, int passes) {
+                               bool inverse, const u64* scale, int passes, const FwdFuse& f) {
   switch (c.logN - kLogChunk) {
 #define ACE_NTT_CASE(LR)                                                                                         \
   case LR:                                                                                                       \
-    run_large<A, LR>(st, c, dst, src, lm, pos, sidx, n_limbs, n_polys, inverse, scale, passes);                   \
+    run_large<A, LR>(st, c, dst, src, lm, pos, sidx, n_limbs, n_polys, inverse, scale, passes, f);                \
     return true;
     ACE_NTT_CASE(1)
     ACE_NTT_CASE(2)
@@ -607,8 +669,14 @@ static bool run_large_dispatch(hipStream_t st, const DevCtx& c, const PolySeq& d
 }
 
 bool launch_ntt(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolySeq& src, const LimbMap& lm,
-                const LimbMap* pos_in, u32 n_limbs, u32 n_polys, bool inverse, const u64* scale, int passes) {
+                const LimbMap* pos_in, u32 n_limbs, u32 n_polys, bool inverse, const u64* scale, int passes,
+                const FwdFuse* fuse) {
   if (n_limbs == 0 || n_polys == 0) return true;
+  FwdFuse f{};
+  if (fuse) {
+    if (inverse || c.logN <= kLogChunk || passes != 3) return false;  // only whole forward transforms of N > 4096
+    f = *fuse;
+  }
   LimbMap pos{};
   if (pos_in) pos = *pos_in;
   else
@@ -632,10 +700,10 @@ bool launch_ntt(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolyS
   bool ok = true;
   if (cnt[0])
     ok &= run_large_dispatch<ArithInt>(st, c, dst, src, lm_g[0], pos_g[0], sidx_g[0], cnt[0], n_polys, inverse,
-                                       scale, passes);
+                                       scale, passes, f);
   if (cnt[1])
     ok &= run_large_dispatch<ArithFp>(st, c, dst, src, lm_g[1], pos_g[1], sidx_g[1], cnt[1], n_polys, inverse,
-                                      scale, passes);
+                                      scale, passes, f);
   return ok;
 }
 
