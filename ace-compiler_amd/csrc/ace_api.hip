@@ -42,6 +42,7 @@ struct ModUpDev {
   u64* scale_coef = nullptr;  // [nd][2]: (hat_inv, Shoup)
   LimbMap digit_lm{}, compl_lm{}, compl_pos{};
   ConvMap conv{};
+  ConvJob job{};  // the digit's conversion, offsets zero
 };
 
 // all digits of a level at once (Precomp)
@@ -77,6 +78,7 @@ struct ace_ctx {
   u64* pscale_coef = nullptr; // [K][2]
   u64* pinv = nullptr;        // [L][2]
   u64* pmodq = nullptr;       // [L][2]
+  ConvJob p2q_job{};          // P -> Q conversion onto all L limbs (callers lower nc to their level)
   LimbMap q_lm{}, p_lm{};     // identity maps: limb t -> prime t / prime L+t
   // ace_alloc / ace_free: sizes of the buffers handed out, and freed buffers kept for reuse
   static constexpr size_t kPoolLimitWords = (size_t)4 << 30;  // 32 GiB
@@ -102,6 +104,55 @@ struct ace_ctx {
     return p;
   }
   ShoupConst sc(u64 w, size_t prime) const { return {w, shoup(w, h.primes[prime].q)}; }
+
+  // FP64 tables of a base conversion (ConvJob::fw / fq): targets below the FP64 limit convert in
+  // exact double arithmetic; sources above it are split into two 30-bit-and-rest halves
+  bool conv_fp = true;
+  void conv_fp_tables(ConvJob& j, const std::vector<size_t>& src, const std::vector<size_t>& tgt, const u64* hat,
+                      size_t hat_stride) {
+    j.fw = j.fq = nullptr;
+    j.fp_mode = j.fw_stride = 0;
+    std::memset(j.fp_target, 0, sizeof(j.fp_target));
+    if (!conv_fp) return;
+    bool any = false, narrow = true, fits = true;
+    for (size_t jj = 0; jj < tgt.size(); ++jj) {
+      j.fp_target[jj] = h.primes[tgt[jj]].q < kFpPrimeLimit ? 1 : 0;
+      any |= j.fp_target[jj] != 0;
+    }
+    for (size_t s : src) {
+      narrow &= h.primes[s].q < kFpPrimeLimit;
+      fits &= h.primes[s].q < ((u64)1 << 62);
+    }
+    if (!any || !fits) {
+      std::memset(j.fp_target, 0, sizeof(j.fp_target));
+      return;
+    }
+    const size_t nd = src.size(), nc = tgt.size(), terms = narrow ? nd : 2 * nd;
+    std::vector<double> fw(terms * nc * 2, 0.0), fq(nc * 2, 0.0);
+    auto put = [&](size_t term, size_t jj, u64 w, u64 q) {
+      fw[2 * (term * nc + jj)] = (double)w;
+      fw[2 * (term * nc + jj) + 1] = (double)((long double)w / (long double)q);
+    };
+    for (size_t jj = 0; jj < nc; ++jj) {
+      const u64 q = h.primes[tgt[jj]].q;
+      fq[2 * jj] = (double)q;
+      fq[2 * jj + 1] = (double)(1.0L / (long double)q);
+      if (!j.fp_target[jj]) continue;
+      for (size_t k = 0; k < nd; ++k) {
+        const u64 w = hat[k * hat_stride + jj];
+        if (narrow) {
+          put(k, jj, w, q);
+        } else {
+          put(2 * k, jj, w, q);
+          put(2 * k + 1, jj, mul_mod(w, ((u64)1 << 30) % q, q), q);
+        }
+      }
+    }
+    j.fw = upload_vec(fw);
+    j.fq = upload_vec(fq);
+    j.fp_mode = narrow ? 1 : 2;
+    j.fw_stride = (u32)nc;
+  }
 
   void ensure_ws(size_t words) {
     if (words <= ws_words) return;
@@ -148,6 +199,13 @@ struct ace_ctx {
       m.conv.prime[j] = (uint8_t)m.t.compl_idx[j];
       m.conv.out_limb[j] = (uint8_t)pos;
     }
+    m.job.hat = m.hat;
+    m.job.hat_stride = (u32)nc;
+    m.job.nd = (u32)nd;
+    m.job.nc = (u32)nc;
+    m.job.map = m.conv;
+    conv_fp_tables(m.job, std::vector<size_t>(m.t.digit.begin(), m.t.digit.end()),
+                   std::vector<size_t>(m.t.compl_idx.begin(), m.t.compl_idx.end()), m.t.hat.data(), nc);
     return modup.emplace(key, std::move(m)).first->second;
   }
 
@@ -168,14 +226,9 @@ struct ace_ctx {
         sn[2 * pi] = a;                 sn[2 * pi + 1] = shoup(a, q);
         scf[2 * pi] = m.t.hat_inv[i];   scf[2 * pi + 1] = shoup(m.t.hat_inv[i], q);
       }
-      ConvJob j{};
-      j.hat = m.hat;
-      j.hat_stride = (u32)nc;
-      j.nd = (u32)len;
-      j.nc = (u32)nc;
+      ConvJob j = m.job;
       j.t_off = start * N;
       j.out_off = d * T * N;
-      j.map = m.conv;
       pd.jobs.push_back(j);
       for (size_t k = 0; k < nc; ++k) {
         if (pd.n_tgt < (u32)kMaxPrimes) {
@@ -229,7 +282,8 @@ struct ace_ctx {
     {
       // FP64 twiddles for the primes the FP64 NTT back end can take
       const char* force_int = std::getenv("ACE_NTT_FORCE_INT");
-      bool use_fp = !(force_int && force_int[0] == '1') && h.logN > 12;
+      conv_fp = !(force_int && force_int[0] == '1');
+      bool use_fp = conv_fp && h.logN > 12;
       std::vector<double> w(T * h.N, 0.0), iw(T * h.N, 0.0);
       for (size_t i = 0; i < T; ++i) {
         d.fp_ok[i] = (use_fp && h.primes[i].q < kFpPrimeLimit) ? 1 : 0;
@@ -262,6 +316,20 @@ struct ace_ctx {
       pm[2 * i] = h.pmodq[i];     pm[2 * i + 1] = shoup(h.pmodq[i], q);
     }
     phat = upload_vec(ph);
+    {
+      std::vector<size_t> src, tgt;
+      for (size_t j = 0; j < h.K; ++j) src.push_back(h.L + j);
+      for (size_t i = 0; i < h.L && i < (size_t)kMaxPrimes; ++i) {
+        tgt.push_back(i);
+        p2q_job.map.prime[i] = (uint8_t)i;
+        p2q_job.map.out_limb[i] = (uint8_t)i;
+      }
+      p2q_job.hat = phat;
+      p2q_job.hat_stride = (u32)h.L;
+      p2q_job.nd = (u32)h.K;
+      p2q_job.nc = (u32)h.L;
+      conv_fp_tables(p2q_job, src, tgt, ph.data(), h.L);
+    }
     pscale_ntt = upload_vec(sn);
     pscale_coef = upload_vec(scf);
     pinv = upload_vec(pi);
@@ -323,11 +391,7 @@ void do_decomp_modup(ace_ctx* c, u64* res, const u64* digit, size_t level, size_
     launch_mul_const(c->stream, c->d, t, digit, m.scale_coef, m.digit_lm, (u32)nd);
   ConvBatch b{};
   b.n_jobs = 1;
-  b.job[0].hat = m.hat;
-  b.job[0].hat_stride = (u32)nc;
-  b.job[0].nd = (u32)nd;
-  b.job[0].nc = (u32)nc;
-  b.job[0].map = m.conv;
+  b.job[0] = m.job;
   launch_baseconv(c->stream, c->d, res, t, b, 1);
   if (is_ntt)
     launch_ntt(c->stream, c->d, seq_strided(res, 0), seq_strided(res, 0), m.compl_lm, &m.compl_pos, (u32)nc, 1, false,
@@ -396,11 +460,8 @@ void do_mod_down(ace_ctx* c, const PolySeq& res, const PolySeq& src, size_t np, 
   }
   ConvBatch b{};
   b.n_jobs = 1;
-  b.job[0].hat = c->phat;
-  b.job[0].hat_stride = (u32)L;
-  b.job[0].nd = (u32)K;
+  b.job[0] = c->p2q_job;
   b.job[0].nc = (u32)level;
-  for (size_t i = 0; i < level; ++i) { b.job[0].map.prime[i] = (uint8_t)i; b.job[0].map.out_limb[i] = (uint8_t)i; }
   b.t_stride = K * N;
   b.out_stride = level * N;
   launch_baseconv(c->stream, c->d, y, t, b, (u32)np);
@@ -484,11 +545,8 @@ void do_moddown_rescale_core(ace_ctx* c, u64* x, u64* y, u64* last_out, u64* pol
   launch_mul_const(c->stream, c->d, t, poly + level * N, c->pscale_coef, c->p_lm, (u32)K);
   ConvBatch b{};
   b.n_jobs = 1;
-  b.job[0].hat = c->phat;
-  b.job[0].hat_stride = (u32)c->h.L;
-  b.job[0].nd = (u32)K;
+  b.job[0] = c->p2q_job;
   b.job[0].nc = (u32)level;
-  for (size_t i = 0; i < level; ++i) { b.job[0].map.prime[i] = (uint8_t)i; b.job[0].map.out_limb[i] = (uint8_t)i; }
   launch_baseconv(c->stream, c->d, y, t, b, 1);
   const RescaleDev& r = c->rescale_at(level);
   launch_moddown_rescale(c->stream, c->d, x, poly, y, last_out, c->pinv, r.tail, (u32)level);

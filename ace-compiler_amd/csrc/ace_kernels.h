@@ -11,11 +11,22 @@ constexpr int kMaxConvJobs = 4;   // digits converted per base-conversion launch
 constexpr int kMaxBatchPtrs = 32; // keys / index tables per batched launch
 
 // one digit's base conversion: out[map.out_limb[j]][i] = (sum_k t[k][i] * hat[k*hat_stride + j]) mod prime map.prime[j]
+// Targets below the FP64 limit can take the conversion in exact double arithmetic (fp_mode != 0):
+//   fp_mode 1: every source prime is below the limit too; term k is t_k with cofactor fw[k][j]
+//   fp_mode 2: sources may be up to 2^62: t_k is split into its low 30 bits and the rest,
+//              term 2k is the low part with fw[2k][j] = hat, term 2k+1 the high part with
+//              fw[2k+1][j] = hat * 2^30 mod m_j
+// fw: [terms][fw_stride][2] = (cofactor, cofactor / m_j) as doubles; fq: [nc][2] = (m_j, 1 / m_j);
+// fp_target[j] says whether target j uses them.
 struct ConvJob {
   const u64* hat;
   u32 hat_stride, nd, nc;
   u64 t_off, out_off;  // word offsets of this job's source limbs / output polynomial inside one operand
   ConvMap map;
+  const double* fw;
+  const double* fq;
+  u32 fp_mode, fw_stride;
+  uint8_t fp_target[kMaxPrimes];
 };
 struct ConvBatch {
   ConvJob job[kMaxConvJobs];

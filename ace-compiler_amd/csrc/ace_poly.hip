@@ -132,8 +132,39 @@ void launch_tensor(hipStream_t st, const DevCtx& c, u64* d0, u64* d1, u64* d2, c
 // blockIdx.z enumerates (operand, job): a job is one digit's conversion, all
 // jobs of a launch share the operand strides.
 constexpr int kConvTargets = 4;
-constexpr int kConvMaxSrc = 16;
 
+// exact x*w mod q in doubles: |result| <= (1/2 + |x| 2^-52) q; w, wi = w/q, q as doubles
+__device__ __forceinline__ double conv_fp_term(double x, double w, double wi, double q) {
+#pragma clang fp contract(off)
+  double c = __builtin_rint(x * wi);
+  double h = x * w;
+  double l = __builtin_fma(x, w, -h);
+  double d = __builtin_fma(-c, q, h);
+  return d + l;
+}
+
+// one target in FP64: TERMS exact products accumulated as integers below 2^53
+// (re-centred every 4 terms), result canonical
+template <int MAXT>
+__device__ __forceinline__ u64 conv_fp_target(const double* xd, u32 terms, const double* __restrict__ fw, u32 nc,
+                                              u32 j, double q, double qinv) {
+#pragma clang fp contract(off)
+  double acc = 0.0;
+#pragma unroll
+  for (int k = 0; k < MAXT; ++k) {
+    if ((u32)k < terms) {
+      const double2 ww = *reinterpret_cast<const double2*>(fw + 2 * ((u64)k * nc + j));
+      acc += conv_fp_term(xd[k], ww.x, ww.y, q);
+      if ((k & 3) == 3) acc = __builtin_fma(-__builtin_rint(acc * qinv), q, acc);
+    }
+  }
+  acc = __builtin_fma(-__builtin_rint(acc * qinv), q, acc);
+  acc = acc < 0.0 ? acc + q : acc;
+  return (u64)__double_as_longlong(acc + 4503599627370496.0) & 0x000FFFFFFFFFFFFFull;
+}
+
+// MAXS: compile-time bound on the number of source limbs (register arrays); 0 = any number, looped
+template <int MAXS>
 __global__ __launch_bounds__(kThreads) void baseconv_kernel(DevCtx c, u64* __restrict__ out_base,
                                                             const u64* __restrict__ t_base, ConvBatch b) {
   const u64 n = c.N;
@@ -147,14 +178,42 @@ __global__ __launch_bounds__(kThreads) void baseconv_kernel(DevCtx c, u64* __res
   u64* __restrict__ out = out_base + op * b.out_stride + J.out_off;
   const u32 j0 = blockIdx.y * kConvTargets;
   if (j0 >= nc) return;
-  if (nd <= kConvMaxSrc) {
+  if constexpr (MAXS > 0) {
+    constexpr int kConvMaxSrc = MAXS;
     u64 x[kConvMaxSrc];
 #pragma unroll
     for (int k = 0; k < kConvMaxSrc; ++k) x[k] = (u32)k < nd ? t[(u64)k * n + i] : 0;
+    // sources as doubles for the targets that convert in FP64 (wave-uniform choice per target)
+    bool any_fp = false;
+    for (int jj = 0; jj < kConvTargets; ++jj) any_fp |= J.fp_mode && j0 + jj < nc && J.fp_target[j0 + jj];
+    double xd[2 * kConvMaxSrc];
+    u32 terms = 0;
+    if (any_fp) {
+      if (J.fp_mode == 1) {
+        terms = nd;
+#pragma unroll
+        for (int k = 0; k < kConvMaxSrc; ++k)
+          xd[k] = __longlong_as_double((long long)(x[k] | 0x4330000000000000ull)) - 4503599627370496.0;
+      } else {
+        terms = 2 * nd;
+#pragma unroll
+        for (int k = 0; k < kConvMaxSrc; ++k) {
+          xd[2 * k] = (double)(u32)(x[k] & 0x3FFFFFFFu);
+          xd[2 * k + 1] = (double)(u32)(x[k] >> 30);
+        }
+      }
+    }
 #pragma unroll
     for (int jj = 0; jj < kConvTargets; ++jj) {
       u32 j = j0 + jj;
       if (j >= nc) break;
+      if (any_fp && J.fp_target[j]) {
+        const double q = J.fq[2 * j], qinv = J.fq[2 * j + 1];
+        u64 r = J.fp_mode == 1 ? conv_fp_target<kConvMaxSrc>(xd, terms, J.fw, J.fw_stride, j, q, qinv)
+                               : conv_fp_target<2 * kConvMaxSrc>(xd, terms, J.fw, J.fw_stride, j, q, qinv);
+        out[(u64)J.map.out_limb[j] * n + i] = r;
+        continue;
+      }
       u64 hi = 0, lo = 0;
 #pragma unroll
       for (int k = 0; k < kConvMaxSrc; ++k)
@@ -178,11 +237,21 @@ __global__ __launch_bounds__(kThreads) void baseconv_kernel(DevCtx c, u64* __res
 
 void launch_baseconv(hipStream_t st, const DevCtx& c, u64* out, const u64* t, const ConvBatch& b, u32 n_ops) {
   if (!b.n_jobs || !n_ops) return;
-  u32 max_nc = 0;
-  for (u32 k = 0; k < b.n_jobs; ++k) max_nc = b.job[k].nc > max_nc ? b.job[k].nc : max_nc;
+  u32 max_nc = 0, max_nd = 0;
+  for (u32 k = 0; k < b.n_jobs; ++k) {
+    max_nc = b.job[k].nc > max_nc ? b.job[k].nc : max_nc;
+    max_nd = b.job[k].nd > max_nd ? b.job[k].nd : max_nd;
+  }
   if (!max_nc) return;
   dim3 g((c.N + kThreads - 1) / kThreads, (max_nc + kConvTargets - 1) / kConvTargets, b.n_jobs * n_ops);
-  hipLaunchKernelGGL(baseconv_kernel, g, dim3(kThreads), 0, st, c, out, t, b);
+  if (max_nd <= 4)
+    hipLaunchKernelGGL(baseconv_kernel<4>, g, dim3(kThreads), 0, st, c, out, t, b);
+  else if (max_nd <= 8)
+    hipLaunchKernelGGL(baseconv_kernel<8>, g, dim3(kThreads), 0, st, c, out, t, b);
+  else if (max_nd <= 16)
+    hipLaunchKernelGGL(baseconv_kernel<16>, g, dim3(kThreads), 0, st, c, out, t, b);
+  else
+    hipLaunchKernelGGL(baseconv_kernel<0>, g, dim3(kThreads), 0, st, c, out, t, b);
 }
 
 // copies the digit limbs of `src` (level limbs per operand) into their places
