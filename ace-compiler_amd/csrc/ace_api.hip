@@ -108,13 +108,14 @@ struct ace_ctx {
   // FP64 tables of a base conversion (ConvJob::fw / fq): targets below the FP64 limit convert in
   // exact double arithmetic; sources above it are split into two 30-bit-and-rest halves
   bool conv_fp = true;
+  bool digits_narrow = true;  // every Q prime is below the FP64 limit: digit conversions need no splitting
   void conv_fp_tables(ConvJob& j, const std::vector<size_t>& src, const std::vector<size_t>& tgt, const u64* hat,
-                      size_t hat_stride) {
+                      size_t hat_stride, bool force_split, size_t pad_sources) {
     j.fw = j.fq = nullptr;
-    j.fp_mode = j.fw_stride = 0;
+    j.fp_mode = j.fw_stride = j.fp_pad = 0;
     std::memset(j.fp_target, 0, sizeof(j.fp_target));
     if (!conv_fp) return;
-    bool any = false, narrow = true, fits = true;
+    bool any = false, narrow = !force_split, fits = pad_sources != 0 && src.size() <= pad_sources;
     for (size_t jj = 0; jj < tgt.size(); ++jj) {
       j.fp_target[jj] = h.primes[tgt[jj]].q < kFpPrimeLimit ? 1 : 0;
       any |= j.fp_target[jj] != 0;
@@ -127,7 +128,8 @@ struct ace_ctx {
       std::memset(j.fp_target, 0, sizeof(j.fp_target));
       return;
     }
-    const size_t nd = src.size(), nc = tgt.size(), terms = narrow ? nd : 2 * nd;
+    const size_t nd = src.size(), nc = tgt.size();
+    const size_t terms = pad_sources * (narrow ? 1 : 2);  // zero rows past the real sources
     std::vector<double> fw(terms * nc * 2, 0.0), fq(nc * 2, 0.0);
     auto put = [&](size_t term, size_t jj, u64 w, u64 q) {
       fw[2 * (term * nc + jj)] = (double)w;
@@ -152,6 +154,7 @@ struct ace_ctx {
     j.fq = upload_vec(fq);
     j.fp_mode = narrow ? 1 : 2;
     j.fw_stride = (u32)nc;
+    j.fp_pad = (u32)pad_sources;
   }
 
   void ensure_ws(size_t words) {
@@ -205,7 +208,8 @@ struct ace_ctx {
     m.job.nc = (u32)nc;
     m.job.map = m.conv;
     conv_fp_tables(m.job, std::vector<size_t>(m.t.digit.begin(), m.t.digit.end()),
-                   std::vector<size_t>(m.t.compl_idx.begin(), m.t.compl_idx.end()), m.t.hat.data(), nc);
+                   std::vector<size_t>(m.t.compl_idx.begin(), m.t.compl_idx.end()), m.t.hat.data(), nc,
+                   !digits_narrow, (size_t)conv_padded_sources((u32)h.part_size));
     return modup.emplace(key, std::move(m)).first->second;
   }
 
@@ -283,6 +287,7 @@ struct ace_ctx {
       // FP64 twiddles for the primes the FP64 NTT back end can take
       const char* force_int = std::getenv("ACE_NTT_FORCE_INT");
       conv_fp = !(force_int && force_int[0] == '1');
+      for (size_t i = 0; i < h.L; ++i) digits_narrow &= h.primes[i].q < kFpPrimeLimit;
       bool use_fp = conv_fp && h.logN > 12;
       std::vector<double> w(T * h.N, 0.0), iw(T * h.N, 0.0);
       for (size_t i = 0; i < T; ++i) {
@@ -328,7 +333,7 @@ struct ace_ctx {
       p2q_job.hat_stride = (u32)h.L;
       p2q_job.nd = (u32)h.K;
       p2q_job.nc = (u32)h.L;
-      conv_fp_tables(p2q_job, src, tgt, ph.data(), h.L);
+      conv_fp_tables(p2q_job, src, tgt, ph.data(), h.L, true, (size_t)conv_padded_sources((u32)h.K));
     }
     pscale_ntt = upload_vec(sn);
     pscale_coef = upload_vec(scf);

@@ -16,7 +16,8 @@ constexpr int kMaxBatchPtrs = 32; // keys / index tables per batched launch
 //   fp_mode 2: sources may be up to 2^62: t_k is split into its low 30 bits and the rest,
 //              term 2k is the low part with fw[2k][j] = hat, term 2k+1 the high part with
 //              fw[2k+1][j] = hat * 2^30 mod m_j
-// fw: [terms][fw_stride][2] = (cofactor, cofactor / m_j) as doubles; fq: [nc][2] = (m_j, 1 / m_j);
+// fw: [terms][fw_stride][2] = (cofactor, cofactor / m_j) as doubles, the terms padded with zero rows to
+//     fp_pad sources; fq: [nc][2] = (m_j, 1 / m_j);
 // fp_target[j] says whether target j uses them.
 struct ConvJob {
   const u64* hat;
@@ -25,7 +26,7 @@ struct ConvJob {
   ConvMap map;
   const double* fw;
   const double* fq;
-  u32 fp_mode, fw_stride;
+  u32 fp_mode, fw_stride, fp_pad;  // fp_pad: sources the tables are padded to (4, 8, 12 or 16)
   uint8_t fp_target[kMaxPrimes];
 };
 struct ConvBatch {
@@ -69,6 +70,7 @@ void launch_tensor(hipStream_t st, const DevCtx& c, u64* d0, u64* d1, u64* d2, c
                    const u64* b0, const u64* b1, const LimbMap& lm, u32 n_limbs, u32 n_ops, u64 d01_stride,
                    u64 d2_stride, u64 in_stride);
 // fast base conversion of b.n_jobs digits for each of n_ops operands
+int conv_padded_sources(u32 nd);
 void launch_baseconv(hipStream_t st, const DevCtx& c, u64* out, const u64* t, const ConvBatch& b, u32 n_ops);
 // digit limbs of src copied into the raised polynomials (see digit_copy_kernel)
 void launch_digit_copy(hipStream_t st, const DevCtx& c, u64* res, const u64* src, u32 level, u32 part_size,

@@ -144,27 +144,27 @@ __device__ __forceinline__ double conv_fp_term(double x, double w, double wi, do
 }
 
 // one target in FP64: TERMS exact products accumulated as integers below 2^53
-// (re-centred every 4 terms), result canonical
-template <int MAXT>
-__device__ __forceinline__ u64 conv_fp_target(const double* xd, u32 terms, const double* __restrict__ fw, u32 nc,
-                                              u32 j, double q, double qinv) {
+// (re-centred every 4 terms), result canonical.  The table holds TERMS rows
+// (rows past the real sources are zero), so the loop has no guards.
+template <int TERMS>
+__device__ __forceinline__ u64 conv_fp_target(const double* xd, const double* __restrict__ fw, u32 stride, u32 j,
+                                              double q, double qinv) {
 #pragma clang fp contract(off)
   double acc = 0.0;
 #pragma unroll
-  for (int k = 0; k < MAXT; ++k) {
-    if ((u32)k < terms) {
-      const double2 ww = *reinterpret_cast<const double2*>(fw + 2 * ((u64)k * nc + j));
-      acc += conv_fp_term(xd[k], ww.x, ww.y, q);
-      if ((k & 3) == 3) acc = __builtin_fma(-__builtin_rint(acc * qinv), q, acc);
-    }
+  for (int k = 0; k < TERMS; ++k) {
+    const double2 ww = *reinterpret_cast<const double2*>(fw + 2 * ((u64)k * stride + j));
+    acc += conv_fp_term(xd[k], ww.x, ww.y, q);
+    if ((k & 3) == 3 && k + 1 < TERMS) acc = __builtin_fma(-__builtin_rint(acc * qinv), q, acc);
   }
   acc = __builtin_fma(-__builtin_rint(acc * qinv), q, acc);
   acc = acc < 0.0 ? acc + q : acc;
   return (u64)__double_as_longlong(acc + 4503599627370496.0) & 0x000FFFFFFFFFFFFFull;
 }
 
-// MAXS: compile-time bound on the number of source limbs (register arrays); 0 = any number, looped
-template <int MAXS>
+// MAXS: compile-time bound on the number of source limbs (register arrays); 0 = any number, looped.
+// MODE: ConvJob::fp_mode of every job of the launch (0: integer arithmetic only).
+template <int MAXS, int MODE>
 __global__ __launch_bounds__(kThreads) void baseconv_kernel(DevCtx c, u64* __restrict__ out_base,
                                                             const u64* __restrict__ t_base, ConvBatch b) {
   const u64 n = c.N;
@@ -179,44 +179,34 @@ __global__ __launch_bounds__(kThreads) void baseconv_kernel(DevCtx c, u64* __res
   const u32 j0 = blockIdx.y * kConvTargets;
   if (j0 >= nc) return;
   if constexpr (MAXS > 0) {
-    constexpr int kConvMaxSrc = MAXS;
-    u64 x[kConvMaxSrc];
+    u64 x[MAXS];
 #pragma unroll
-    for (int k = 0; k < kConvMaxSrc; ++k) x[k] = (u32)k < nd ? t[(u64)k * n + i] : 0;
-    // sources as doubles for the targets that convert in FP64 (wave-uniform choice per target)
-    bool any_fp = false;
-    for (int jj = 0; jj < kConvTargets; ++jj) any_fp |= J.fp_mode && j0 + jj < nc && J.fp_target[j0 + jj];
-    double xd[2 * kConvMaxSrc];
-    u32 terms = 0;
-    if (any_fp) {
-      if (J.fp_mode == 1) {
-        terms = nd;
+    for (int k = 0; k < MAXS; ++k) x[k] = (u32)k < nd ? t[(u64)k * n + i] : 0;
+    constexpr int TERMS = MODE == 1 ? MAXS : (MODE == 2 ? 2 * MAXS : 1);
+    double xd[TERMS];
+    if constexpr (MODE == 1) {
 #pragma unroll
-        for (int k = 0; k < kConvMaxSrc; ++k)
-          xd[k] = __longlong_as_double((long long)(x[k] | 0x4330000000000000ull)) - 4503599627370496.0;
-      } else {
-        terms = 2 * nd;
+      for (int k = 0; k < MAXS; ++k)
+        xd[k] = __longlong_as_double((long long)(x[k] | 0x4330000000000000ull)) - 4503599627370496.0;
+    } else if constexpr (MODE == 2) {
 #pragma unroll
-        for (int k = 0; k < kConvMaxSrc; ++k) {
-          xd[2 * k] = (double)(u32)(x[k] & 0x3FFFFFFFu);
-          xd[2 * k + 1] = (double)(u32)(x[k] >> 30);
-        }
+      for (int k = 0; k < MAXS; ++k) {
+        xd[2 * k] = (double)(u32)(x[k] & 0x3FFFFFFFu);
+        xd[2 * k + 1] = (double)(u32)(x[k] >> 30);
       }
     }
 #pragma unroll
     for (int jj = 0; jj < kConvTargets; ++jj) {
       u32 j = j0 + jj;
       if (j >= nc) break;
-      if (any_fp && J.fp_target[j]) {
-        const double q = J.fq[2 * j], qinv = J.fq[2 * j + 1];
-        u64 r = J.fp_mode == 1 ? conv_fp_target<kConvMaxSrc>(xd, terms, J.fw, J.fw_stride, j, q, qinv)
-                               : conv_fp_target<2 * kConvMaxSrc>(xd, terms, J.fw, J.fw_stride, j, q, qinv);
-        out[(u64)J.map.out_limb[j] * n + i] = r;
+      if (MODE != 0 && J.fp_target[j]) {  // wave-uniform
+        out[(u64)J.map.out_limb[j] * n + i] =
+            conv_fp_target<TERMS>(xd, J.fw, J.fw_stride, j, J.fq[2 * j], J.fq[2 * j + 1]);
         continue;
       }
       u64 hi = 0, lo = 0;
 #pragma unroll
-      for (int k = 0; k < kConvMaxSrc; ++k)
+      for (int k = 0; k < MAXS; ++k)
         if ((u32)k < nd) mac128(hi, lo, x[k], hat[(u64)k * hat_stride + j]);
       out[(u64)J.map.out_limb[j] * n + i] = barrett128(hi, lo, c.primes[J.map.prime[j]]);
     }
@@ -235,23 +225,33 @@ __global__ __launch_bounds__(kThreads) void baseconv_kernel(DevCtx c, u64* __res
   }
 }
 
+// register-array size used for nd source limbs (0: the looped kernel); the FP64 tables are padded to it
+int conv_padded_sources(u32 nd) { return nd <= 4 ? 4 : nd <= 8 ? 8 : nd <= 12 ? 12 : nd <= 16 ? 16 : 0; }
+
 void launch_baseconv(hipStream_t st, const DevCtx& c, u64* out, const u64* t, const ConvBatch& b, u32 n_ops) {
   if (!b.n_jobs || !n_ops) return;
-  u32 max_nc = 0, max_nd = 0;
+  u32 max_nc = 0, max_nd = 0, mode = b.job[0].fp_mode, pad = b.job[0].fp_pad;
   for (u32 k = 0; k < b.n_jobs; ++k) {
     max_nc = b.job[k].nc > max_nc ? b.job[k].nc : max_nc;
     max_nd = b.job[k].nd > max_nd ? b.job[k].nd : max_nd;
+    if (b.job[k].fp_mode != mode || b.job[k].fp_pad != pad) mode = 0;  // mixed launches keep to integer arithmetic
   }
   if (!max_nc) return;
+  if (mode != 0 && max_nd > pad) mode = 0;
+  const int maxs = mode != 0 ? (int)pad : conv_padded_sources(max_nd);
   dim3 g((c.N + kThreads - 1) / kThreads, (max_nc + kConvTargets - 1) / kConvTargets, b.n_jobs * n_ops);
-  if (max_nd <= 4)
-    hipLaunchKernelGGL(baseconv_kernel<4>, g, dim3(kThreads), 0, st, c, out, t, b);
-  else if (max_nd <= 8)
-    hipLaunchKernelGGL(baseconv_kernel<8>, g, dim3(kThreads), 0, st, c, out, t, b);
-  else if (max_nd <= 16)
-    hipLaunchKernelGGL(baseconv_kernel<16>, g, dim3(kThreads), 0, st, c, out, t, b);
-  else
-    hipLaunchKernelGGL(baseconv_kernel<0>, g, dim3(kThreads), 0, st, c, out, t, b);
+#define ACE_BC(S, M) hipLaunchKernelGGL((baseconv_kernel<S, M>), g, dim3(kThreads), 0, st, c, out, t, b)
+#define ACE_BC_MODES(S) \
+  do { if (mode == 1) ACE_BC(S, 1); else if (mode == 2) ACE_BC(S, 2); else ACE_BC(S, 0); } while (0)
+  switch (maxs) {
+    case 4: ACE_BC_MODES(4); break;
+    case 8: ACE_BC_MODES(8); break;
+    case 12: ACE_BC_MODES(12); break;
+    case 16: ACE_BC_MODES(16); break;
+    default: ACE_BC(0, 0); break;
+  }
+#undef ACE_BC_MODES
+#undef ACE_BC
 }
 
 // copies the digit limbs of `src` (level limbs per operand) into their places
