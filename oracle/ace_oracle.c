@@ -39,6 +39,9 @@ struct orc_ctx {
   i64*       root; /* [L+K] */
   u64 *      rou, *rou_prec, *rou_inv, *rou_inv_prec; /* [(L+K)*N] */
   u64 *      ninv, *ninv_prec;                        /* [L+K] */
+  size_t     q0_bits, sf_bits;                        /* 0 when the primes were given explicitly */
+  double*    fft_rou;   /* [2N][2]: cos, sin of 2 pi i / 2N (util/src/ntt.c:561-570) */
+  i64*       rot_group; /* [N/2]: 5^i mod 2N           (util/src/ntt.c:580-586) */
 };
 
 /* ---------------------------------------------------------------------- */
@@ -413,6 +416,18 @@ static orc_ctx* ctx_finish(uint32_t N, size_t L, i64* q, size_t parts) {
     build_ntt_tables(c, i);
   }
   free(all);
+  /* Precompute_fft (util/src/ntt.c:559-587) for fft_length = 2N */
+  size_t M = 2 * (size_t)N;
+  c->fft_rou = (double*)malloc(sizeof(double) * 2 * M);
+  for (size_t i = 0; i < M; i++) {
+    double angle = 2 * M_PI * i / M;
+    c->fft_rou[2 * i] = cos(angle);
+    c->fft_rou[2 * i + 1] = sin(angle);
+  }
+  size_t ns = M / 4;
+  c->rot_group = (i64*)malloc(sizeof(i64) * (ns ? ns : 1));
+  c->rot_group[0] = 1;
+  for (size_t i = 1; i < ns; i++) c->rot_group[i] = (5 * c->rot_group[i - 1]) % (i64)M;
   return c;
 }
 
@@ -421,6 +436,8 @@ orc_ctx* orc_ctx_create(uint32_t degree, size_t num_q, size_t q0_bits,
   i64* q = (i64*)malloc(sizeof(i64) * num_q);
   generate_q_primes(q, num_q, q0_bits, sf_bits, degree);
   orc_ctx* c = ctx_finish(degree, num_q, q, num_parts);
+  c->q0_bits = q0_bits;
+  c->sf_bits = sf_bits;
   free(q);
   return c;
 }
@@ -438,6 +455,7 @@ void orc_ctx_destroy(orc_ctx* c) {
   if (!c) return;
   free(c->mod); free(c->root); free(c->rou); free(c->rou_prec);
   free(c->rou_inv); free(c->rou_inv_prec); free(c->ninv); free(c->ninv_prec);
+  free(c->fft_rou); free(c->rot_group);
   free(c);
 }
 
@@ -1164,4 +1182,236 @@ void orc_mul_relin_rescale(const orc_ctx* c, int64_t* r0, int64_t* r1, const int
   orc_relin(c, d + 3 * n, d + 4 * n, d, d + n, d + 2 * n, swk, level);
   orc_rescale_ciph(c, r0, r1, d + 3 * n, d + 4 * n, level);
   free(d);
+}
+
+/* ---------------------------------------------------------------------- */
+/* encoder: ckks/src/encoder.c, util/src/ntt.c:598-675                     */
+/* ---------------------------------------------------------------------- */
+
+#include <complex.h>
+typedef double complex dcmplx;
+
+static dcmplx fft_rou_at(const orc_ctx* c, size_t i) { return c->fft_rou[2 * i] + c->fft_rou[2 * i + 1] * I; }
+
+/* Embedding_inv (ntt.c:631-675): the special inverse FFT over `len` slots */
+static void embedding_inv(const orc_ctx* c, dcmplx* res, const dcmplx* coeffs, size_t len) {
+  size_t M = 2 * (size_t)c->N;
+  dcmplx* r = (dcmplx*)malloc(sizeof(dcmplx) * len);
+  memcpy(r, coeffs, sizeof(dcmplx) * len);
+  size_t logn = 0;
+  while (((size_t)1 << logn) < len) logn++;
+  for (size_t logm = logn; logm > 0; logm--) {
+    size_t idx_mod = (size_t)1 << (logm + 2), gap = M / idx_mod, num1 = (size_t)1 << logm, num2 = num1 >> 1;
+    for (size_t j = 0; j < len; j += num1) {
+      for (size_t i = 0; i < num2; i++) {
+        size_t ie = j + i, io = j + i + num2;
+        size_t rou_idx = (idx_mod - ((size_t)c->rot_group[i] % idx_mod)) * gap;
+        dcmplx plus = r[ie] + r[io], minus = r[ie] - r[io];
+        minus *= fft_rou_at(c, rou_idx);
+        r[ie] = plus;
+        r[io] = minus;
+      }
+    }
+  }
+  for (size_t i = 0; i < len; i++) res[i] = r[reverse_bits(i, (unsigned)logn)];
+  free(r);
+  for (size_t i = 0; i < len; i++) res[i] /= len;
+}
+
+/* Embedding (ntt.c:598-629) */
+static void embedding(const orc_ctx* c, dcmplx* res, const dcmplx* coeffs, size_t len) {
+  size_t M = 2 * (size_t)c->N;
+  size_t logn = 0;
+  while (((size_t)1 << logn) < len) logn++;
+  for (size_t i = 0; i < len; i++) res[i] = coeffs[reverse_bits(i, (unsigned)logn)];
+  for (size_t logm = 1; logm < logn + 1; logm++) {
+    size_t idx_mod = (size_t)1 << (logm + 2), gap = M / idx_mod, num = (size_t)1 << (logm - 1);
+    for (size_t j = 0; j < len; j += (size_t)1 << logm) {
+      for (size_t i = 0; i < num; i++) {
+        size_t ie = j + i, io = j + i + num;
+        size_t rou_idx = ((size_t)c->rot_group[i] % idx_mod) * gap;
+        dcmplx om = fft_rou_at(c, rou_idx) * res[io];
+        dcmplx plus = res[ie] + om, minus = res[ie] - om;
+        res[ie] = plus;
+        res[io] = minus;
+      }
+    }
+  }
+}
+
+void orc_embedding(const orc_ctx* c, double* res, const double* coeffs, size_t len, int inverse) {
+  if (inverse) embedding_inv(c, (dcmplx*)res, (const dcmplx*)coeffs, len);
+  else embedding(c, (dcmplx*)res, (const dcmplx*)coeffs, len);
+}
+
+static i64 max_64bit_value(void) { return (i64)(((u64)1 << 63) - ((u64)1 << 9)) - 1; } /* modular.h:279-281 */
+static i64 mod_int64(i64 v, i64 m) { i64 r = v % m; return r < 0 ? r + m : r; }        /* modular.h:85-92 */
+
+/* Encode_impl (encoder.c:234-326), 64-bit build.  values: n_values complex numbers
+ * (re, im interleaved); out: level Q limbs followed by p_cnt P limbs, NTT form.
+ * Returns 1, or 0 where the reference asserts (vector out of range / overflow). */
+int orc_encode(const orc_ctx* c, int64_t* out, const double* values, size_t n_values, uint32_t slots, size_t level,
+               uint32_t sf_degree, size_t p_cnt) {
+  ORC_ASSERT(c->sf_bits, "context has no scaling factor");
+  size_t N = c->N;
+  double scaling_factor = (double)((u64)1 << c->sf_bits); /* param.c:68 */
+  if (!slots) slots = (uint32_t)(N / 2);
+  if (!level) level = c->L;
+  ORC_ASSERT(level <= c->L && n_values <= slots && slots <= N / 2, "encode: bad sizes");
+  uint32_t sf_bits = (uint32_t)log2(scaling_factor);
+  size_t coeff_bits = c->q0_bits + (level - 1) * c->sf_bits; /* Get_coeff_bit_count */
+  ORC_ASSERT(sf_degree >= 1 && (size_t)sf_bits * sf_degree < coeff_bits, "invalid scaling factor for encode");
+  double scale = pow(scaling_factor, sf_degree);
+  /* Transform_msg_within_range (encoder.c:198-231) */
+  dcmplx* in = (dcmplx*)calloc(slots, sizeof(dcmplx));
+  dcmplx* ts = (dcmplx*)calloc(slots, sizeof(dcmplx));
+  for (size_t i = 0; i < n_values; i++) in[i] = values[2 * i] + values[2 * i + 1] * I;
+  embedding_inv(c, ts, in, slots);
+  double max_coeff = 0.0;
+  for (uint32_t i = 0; i < slots; i++) {
+    double a = fabs(creal(ts[i]) * scale), b = fabs(cimag(ts[i]) * scale);
+    if (a > max_coeff) max_coeff = a;
+    if (b > max_coeff) max_coeff = b;
+  }
+  int32_t bits = (int32_t)(log2(fmax(max_coeff, __DBL_MIN__))) + 1;
+  int32_t valid = (int32_t)c->q0_bits + (int32_t)(level - 1) * (int32_t)sf_bits; /* Check_msg_range (:48-59) */
+  int ok = bits < valid;
+  i64* message = (i64*)calloc(N, sizeof(i64));
+  uint32_t gap = (uint32_t)(N / (slots * 2));
+  for (uint32_t i = 0; ok && i < slots; i++) {
+    double re = creal(ts[i]) * scaling_factor + 0.5, im = cimag(ts[i]) * scaling_factor + 0.5;
+    if (!(re <= (double)INT64_MAX && re >= -(double)INT64_MAX && im <= (double)INT64_MAX && im >= -(double)INT64_MAX)) {
+      ok = 0;
+      break;
+    }
+    i64 r = llround(re), m = llround(im);
+    message[(size_t)i * gap] = r < 0 ? max_64bit_value() + r : r;
+    message[((size_t)i + slots) * gap] = m < 0 ? max_64bit_value() + m : m;
+  }
+  if (ok) {
+    /* Transform_values_to_dcrt (crt.c:1153-1184), I64 values, with modulus */
+    i64 big_bound = max_64bit_value(), big_half = big_bound >> 1;
+    for (size_t t = 0; t < level + p_cnt; t++) {
+      size_t pi = t < level ? t : c->L + (t - level);
+      i64 q = c->mod[pi].val, diff = big_bound - q;
+      for (size_t n = 0; n < N; n++) {
+        i64 v = message[n];
+        out[t * N + n] = v > big_half ? mod_int64(v - diff, q) : mod_int64(v, q);
+      }
+    }
+    if (sf_degree > 1) { /* encoder.c:297-312: only the Q limbs */
+      for (size_t t = 0; t < level; t++) {
+        i64 q = c->mod[t].val, powp = (i64)scaling_factor;
+        for (uint32_t d = 2; d < sf_degree; d++) powp = mul_mod_exact(powp, (i64)scaling_factor, q);
+        for (size_t n = 0; n < N; n++) out[t * N + n] = mul_mod_exact(out[t * N + n], powp, q);
+      }
+    }
+    int32_t idx[128];
+    for (size_t t = 0; t < level + p_cnt; t++) idx[t] = (int32_t)(t < level ? t : c->L + (t - level));
+    orc_ntt(c, out, out, idx, level + p_cnt);
+  }
+  free(in); free(ts); free(message);
+  return ok;
+}
+
+/* Reconstruct (crt.c:1247-1275) + mpz_get_d: the centred integer with residues
+ * v[0..level) as a double, truncated towards zero like mpz_get_d.  Garner's
+ * mixed-radix digits, then exact evaluation in a little-endian multi-word integer. */
+static double crt_to_double(const orc_ctx* c, const i64* v, size_t level) {
+  i64 d[64];
+  /* mixed radix: x = d0 + d1 q0 + d2 q0 q1 + ... */
+  for (size_t i = 0; i < level; i++) {
+    i64 q = c->mod[i].val, t = v[i] % q, prod = 1;
+    /* t = (v_i - (d0 + d1 q0 + ...)) / (q0..q_{i-1}) mod q_i */
+    i64 acc = 0;
+    for (size_t j = 0; j < i; j++) {
+      acc = orc_add_mod(acc, mul_mod_exact(d[j] % q, prod, q), q);
+      prod = mul_mod_exact(prod, c->mod[j].val % q, q);
+    }
+    t = orc_sub_mod(t, acc, q);
+    d[i] = i ? mul_mod_exact(t, inv_prime(prod, q), q) : t;
+  }
+  /* exact value and Q as multi-word integers */
+  u64 x[66] = {0}, Q[66] = {0};
+  size_t nx = 1, nQ = 1;
+  Q[0] = 1;
+  for (size_t i = level; i-- > 0;) { /* Horner from the top digit */
+    u128 carry = 0;
+    for (size_t k = 0; k < nx; k++) { u128 p = (u128)x[k] * (u64)c->mod[i].val + carry; x[k] = (u64)p; carry = p >> 64; }
+    if (carry) x[nx++] = (u64)carry;
+    u128 a = (u128)x[0] + (u64)d[i];
+    x[0] = (u64)a;
+    for (size_t k = 1; (a >> 64) && k <= nx; k++) { a = (u128)x[k] + 1; x[k] = (u64)a; if (k == nx) nx++; }
+  }
+  for (size_t i = 0; i < level; i++) {
+    u128 carry = 0;
+    for (size_t k = 0; k < nQ; k++) { u128 p = (u128)Q[k] * (u64)c->mod[i].val + carry; Q[k] = (u64)p; carry = p >> 64; }
+    if (carry) Q[nQ++] = (u64)carry;
+  }
+  size_t n = nQ > nx ? nQ : nx;
+  /* negative when x > floor(Q/2), i.e. 2x > Q (Q is odd) */
+  u64 x2[67] = {0};
+  for (size_t k = 0; k < n; k++) x2[k] = (x[k] << 1) | (k ? x[k - 1] >> 63 : 0);
+  x2[n] = x[n - 1] >> 63;
+  int neg = 0;
+  if (x2[n]) neg = 1;
+  else
+    for (size_t k = n; k-- > 0;) {
+      if (x2[k] != Q[k]) { neg = x2[k] > Q[k]; break; }
+    }
+  if (neg) { /* x = Q - x */
+    u64 borrow = 0;
+    for (size_t k = 0; k < n; k++) {
+      u128 t = (u128)Q[k] - x[k] - borrow;
+      x[k] = (u64)t;
+      borrow = (u64)(t >> 64) & 1;
+    }
+  }
+  /* truncate to 53 significant bits */
+  size_t top = n;
+  while (top > 0 && x[top - 1] == 0) top--;
+  if (!top) return 0.0;
+  int hb = 63 - __builtin_clzll(x[top - 1]);
+  size_t bitlen = (top - 1) * 64 + (size_t)hb + 1;
+  double r;
+  if (bitlen <= 53) {
+    r = (double)x[0];
+  } else {
+    size_t sh = bitlen - 53, w = sh / 64, b = sh % 64;
+    u64 m = x[w] >> b;
+    if (b && w + 1 < top) m |= x[w + 1] << (64 - b);
+    m &= ((u64)1 << 53) - 1;
+    r = ldexp((double)m, (int)sh);
+  }
+  return neg ? -r : r;
+}
+
+/* Decode (encoder.c:657-704).  poly: level limbs in NTT or coefficient form (a copy is
+ * transformed); res: slots complex numbers (re, im interleaved). */
+void orc_decode(const orc_ctx* c, double* res, const int64_t* poly, size_t level, uint32_t slots, double factor,
+                int is_ntt) {
+  size_t N = c->N, half = N / 2;
+  if (!slots) slots = (uint32_t)half;
+  uint32_t gap = (uint32_t)(half / slots);
+  i64* p = (i64*)malloc(sizeof(i64) * level * N);
+  memcpy(p, poly, sizeof(i64) * level * N);
+  if (is_ntt) {
+    int32_t idx[128];
+    for (size_t t = 0; t < level; t++) idx[t] = (int32_t)t;
+    orc_intt(c, p, p, idx, level);
+  }
+  dcmplx* msg = (dcmplx*)malloc(sizeof(dcmplx) * slots);
+  i64 v[64];
+  for (uint32_t i = 0; i < slots; i++) {
+    for (size_t t = 0; t < level; t++) v[t] = p[t * N + (size_t)i * gap];
+    double re = crt_to_double(c, v, level);
+    for (size_t t = 0; t < level; t++) v[t] = p[t * N + (size_t)i * gap + half];
+    double im = crt_to_double(c, v, level);
+    re /= factor;
+    im /= factor;
+    msg[i] = re + im * I;
+  }
+  embedding(c, (dcmplx*)res, msg, slots);
+  free(p);
+  free(msg);
 }

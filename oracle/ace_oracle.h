@@ -161,6 +161,16 @@ void orc_fast_rotate(const orc_ctx* c, int64_t* r0, int64_t* r1, const int64_t* 
 /* Mul_ciphertext + Rescale_ciphertext (:177-190, :342-362) */
 void orc_mul_relin_rescale(const orc_ctx* c, int64_t* r0, int64_t* r1, const int64_t* a0, const int64_t* a1, const int64_t* b0, const int64_t* b1, const int64_t* swk, size_t level);
 
+/* ---- encoder (ckks/src/encoder.c, util/src/ntt.c:598-675) ---- */
+/* Embedding / Embedding_inv over `len` complex slots (re, im interleaved) */
+void orc_embedding(const orc_ctx* c, double* res, const double* coeffs, size_t len, int inverse);
+/* Encode_impl (encoder.c:234-326): 1 on success, 0 where the reference asserts on range */
+int orc_encode(const orc_ctx* c, int64_t* out, const double* values, size_t n_values, uint32_t slots, size_t level,
+               uint32_t sf_degree, size_t p_cnt);
+/* Decode (encoder.c:657-704) */
+void orc_decode(const orc_ctx* c, double* res, const int64_t* poly, size_t level, uint32_t slots, double factor,
+                int is_ntt);
+
 #ifdef __cplusplus
 }
 #endif

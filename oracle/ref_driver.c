@@ -27,6 +27,9 @@
 #include "ntt_impl.h"
 #include "number_theory_impl.h"
 #include "poly/rns_poly.h"
+#include "ckks/encoder.h"
+#include "ckks/plaintext.h"
+#include "context/ckks_context.h"
 #include "rns_poly_impl.h"
 #include "type_impl.h"
 #include "util/crt.h"
@@ -37,7 +40,7 @@ enum {
   OP_NTT = 1, OP_INTT, OP_HW, OP_DECOMP_MODUP, OP_PRECOMP, OP_MOD_DOWN,
   OP_RESCALE, OP_DOT_PROD, OP_AUTO_ORDER, OP_AUTO_INDEX, OP_AUTOMORPHISM,
   OP_EXTEND, OP_TBL_MODUP, OP_TBL_MODDOWN, OP_TBL_RESCALE, OP_POLY, OP_TWIDDLES,
-  OP_MOD_UP, OP_MOD_DOWN_RESCALE, OP_REDUCE_RESCALE_MODUP, OP_FROM_LEVEL0
+  OP_MOD_UP, OP_MOD_DOWN_RESCALE, OP_REDUCE_RESCALE_MODUP, OP_FROM_LEVEL0, OP_ENCODE, OP_DECODE, OP_EMBEDDING
 };
 
 static int64_t* in_buf;
@@ -234,6 +237,57 @@ int main(int argc, char** argv) {
         wr1((int64_t)(lv * N));
         wr(out, lv * N);
         free(out);
+        break;
+      }
+      case OP_ENCODE: { /* a1 level, a2 slots, a3 sf_degree, a4 p_cnt; in = n_values complex doubles (raw bits) */
+        size_t lv = (size_t)a1, pc = (size_t)a4, nv = n_in / 2;
+        CKKS_ENCODER* enc = (CKKS_ENCODER*)Context->_encoder;
+        VALUE_LIST* vals = Alloc_value_list(DCMPLX_TYPE, nv);
+        memcpy(DCMPLX_VALUES(vals), in, nv * sizeof(DCMPLX));
+        PLAINTEXT pt;
+        memset(&pt, 0, sizeof(pt));
+        if (pc) Encode_ext_at_level(&pt, enc, vals, (uint32_t)lv, (uint32_t)a2, (uint32_t)pc);
+        else Encode_at_level_with_sf(&pt, enc, vals, (uint32_t)lv, (uint32_t)a2, (uint32_t)a3);
+        POLYNOMIAL* poly = Get_plain_poly(&pt);
+        size_t n = (Poly_level(poly) + Num_p(poly)) * N;
+        wr1((int64_t)(n + 3));
+        wr(Get_poly_coeffs(poly), Poly_level(poly) * N);
+        if (Num_p(poly)) wr(Get_p_coeffs(poly), Num_p(poly) * N);
+        wr1((int64_t)pt._slots);
+        wr1((int64_t)pt._sf_degree);
+        { double sf = pt._scaling_factor; int64_t bits; memcpy(&bits, &sf, 8); wr1(bits); }
+        Free_poly_data(poly);
+        Free_value_list(vals);
+        break;
+      }
+      case OP_DECODE: { /* a1 level, a2 slots, a3 is_ntt, a4 raw bits of the scaling factor; in = level*N */
+        size_t lv = (size_t)a1;
+        CKKS_ENCODER* enc = (CKKS_ENCODER*)Context->_encoder;
+        PLAINTEXT pt;
+        memset(&pt, 0, sizeof(pt));
+        wrap_poly(Get_plain_poly(&pt), in, lv, 0, a3 != 0);
+        pt._slots = (uint32_t)a2;
+        memcpy(&pt._scaling_factor, &a4, 8);
+        pt._sf_degree = 1;
+        VALUE_LIST* res = Alloc_value_list(DCMPLX_TYPE, (size_t)a2);
+        Decode(res, enc, &pt);
+        wr1((int64_t)(2 * a2));
+        wr((int64_t*)DCMPLX_VALUES(res), 2 * (size_t)a2);
+        Free_value_list(res);
+        break;
+      }
+      case OP_EMBEDDING: { /* a1 inverse; in = len complex doubles */
+        size_t len = n_in / 2;
+        CKKS_ENCODER* enc = (CKKS_ENCODER*)Context->_encoder;
+        VALUE_LIST* vals = Alloc_value_list(DCMPLX_TYPE, len);
+        VALUE_LIST* res  = Alloc_value_list(DCMPLX_TYPE, len);
+        memcpy(DCMPLX_VALUES(vals), in, len * sizeof(DCMPLX));
+        if (a1) Embedding_inv(res, enc->_fft, vals);
+        else Embedding(res, enc->_fft, vals);
+        wr1((int64_t)(2 * len));
+        wr((int64_t*)DCMPLX_VALUES(res), 2 * len);
+        Free_value_list(vals);
+        Free_value_list(res);
         break;
       }
       case OP_RESCALE: { /* a1 level, a2 is_ntt; in = level*N */

@@ -237,6 +237,31 @@ class Oracle:
         self.L_.orc_transform_from_level0(self.h, _ptr(out), _ptr(src), C.c_size_t(level))
         return out
 
+    # --- encoder
+    def embedding(self, values, inverse=False):
+        v = np.ascontiguousarray(values, dtype=np.complex128)
+        out = np.zeros_like(v)
+        self.L_.orc_embedding(self.h, out.ctypes.data_as(C.c_void_p), v.ctypes.data_as(C.c_void_p),
+                              C.c_size_t(v.size), C.c_int(int(inverse)))
+        return out
+
+    def encode(self, values, slots=0, level=0, sf_degree=1, p_cnt=0):
+        """Plaintext polynomial (level Q limbs + p_cnt P limbs, NTT form), or None where the reference asserts."""
+        v = np.ascontiguousarray(values, dtype=np.complex128)
+        lv = level or self.L
+        out = np.zeros((lv + p_cnt) * self.N, np.int64)
+        self.L_.orc_encode.restype = C.c_int
+        ok = self.L_.orc_encode(self.h, _ptr(out), v.ctypes.data_as(C.c_void_p), C.c_size_t(v.size), C.c_uint32(slots),
+                                C.c_size_t(level), C.c_uint32(sf_degree), C.c_size_t(p_cnt))
+        return out if ok else None
+
+    def decode(self, poly, level, slots, factor, is_ntt=True):
+        poly = np.ascontiguousarray(poly, dtype=np.int64)
+        out = np.zeros(slots, np.complex128)
+        self.L_.orc_decode(self.h, out.ctypes.data_as(C.c_void_p), _ptr(poly), C.c_size_t(level), C.c_uint32(slots),
+                           C.c_double(factor), C.c_int(int(is_ntt)))
+        return out
+
     def dot_prod(self, digits, key, n_parts, level, fast=False):
         digits = np.ascontiguousarray(digits, dtype=np.int64)
         key = np.ascontiguousarray(key, dtype=np.int64)
