@@ -71,6 +71,9 @@ def _sig(lib):
     f("ace_poly_automorphism", C.c_int, _vp, _vp, _vp, _vp, _sz, C.c_int)
     f("ace_decomp_modup", C.c_int, _vp, _vp, _vp, _sz, _sz, C.c_int)
     f("ace_mod_up", C.c_int, _vp, _vp, _vp, _sz, _sz, C.c_int)
+    f("ace_host_fft_tables", C.c_int, _vp, _vp, _vp)
+    f("ace_embedding_inv", C.c_int, _vp, _vp, _vp, _sz)
+    f("ace_encode", C.c_int, _vp, _vp, _vp, _sz, C.c_uint32, _sz, C.c_uint32, _sz)
     f("ace_mod_down_rescale", C.c_int, _vp, _vp, _vp, _sz, C.c_int)
     f("ace_reduce_rescale_modup", C.c_int, _vp, _vp, _vp, _vp, _sz, C.c_int)
     f("ace_transform_from_level0", C.c_int, _vp, _vp, _vp, _sz)
@@ -100,7 +103,7 @@ EXPORTS = [
     "ace_hw_modsub_scalar", "ace_hw_modmul_scalar", "ace_hw_modmuladd_scalar", "ace_hw_rotate",
     "ace_find_automorphism_index", "ace_automorphism_order", "ace_poly_add", "ace_poly_sub", "ace_poly_mul",
     "ace_poly_automorphism", "ace_decomp_modup", "ace_mod_up", "ace_mod_down_rescale",
-    "ace_reduce_rescale_modup", "ace_transform_from_level0", "ace_precomp", "ace_mod_down", "ace_rescale", "ace_extend",
+    "ace_reduce_rescale_modup", "ace_transform_from_level0", "ace_host_fft_tables", "ace_embedding_inv", "ace_encode", "ace_precomp", "ace_mod_down", "ace_rescale", "ace_extend",
     "ace_dot_prod", "ace_mul_ciph3", "ace_fast_switch_key", "ace_relin", "ace_rescale_ciph",
     "ace_mul_relin_rescale", "ace_mul_relin_rescale_batch", "ace_fast_rotate", "ace_rotate_batch",
 ]
@@ -299,6 +302,23 @@ class Context:
 
     def transform_from_level0(self, res, src, level):
         self._chk(self.lib.ace_transform_from_level0(self.h, res.ptr, src.ptr, level))
+
+    def host_fft_tables(self):
+        rou = np.zeros(4 * self.N, np.float64)
+        rot = np.zeros(max(1, self.N // 2), np.uint32)
+        self._chk(self.lib.ace_host_fft_tables(self.h, rou.ctypes.data_as(C.c_void_p), rot.ctypes.data_as(C.c_void_p)))
+        return rou, rot
+
+    def embedding_inv(self, values):
+        v = np.ascontiguousarray(values, dtype=np.complex128)
+        out = np.zeros_like(v)
+        self._chk(self.lib.ace_embedding_inv(self.h, out.ctypes.data_as(C.c_void_p), v.ctypes.data_as(C.c_void_p), v.size))
+        return out
+
+    def encode(self, res, values, slots=0, level=0, sf_degree=1, p_cnt=0):
+        v = np.ascontiguousarray(values, dtype=np.complex128)
+        self._chk(self.lib.ace_encode(self.h, res.ptr, v.ctypes.data_as(C.c_void_p), v.size, slots, level, sf_degree,
+                                      p_cnt))
 
     def mod_up(self, res, digit, level, part, is_ntt=True):
         self._chk(self.lib.ace_mod_up(self.h, res.ptr, digit.ptr, level, part, int(is_ntt)))

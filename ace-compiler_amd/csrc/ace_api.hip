@@ -3,6 +3,7 @@
 // reference operation.  One HIP stream per context; every call only enqueues.
 #include <hip/hip_runtime.h>
 
+#include <cmath>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -79,6 +80,22 @@ struct ace_ctx {
   u64* pinv = nullptr;        // [L][2]
   u64* pmodq = nullptr;       // [L][2]
   ConvJob p2q_job{};          // P -> Q conversion onto all L limbs (callers lower nc to their level)
+  // encoder
+  size_t q0_bits = 0, sf_bits = 0;  // 0: the primes were given explicitly, no scaling factor is known
+  double2* fft_rou = nullptr;       // [2N] exp(2 pi i k / 2N)
+  u32* rot_group = nullptr;         // [N/2] 5^k mod 2N
+  int* d_err = nullptr;             // sticky device flag of checks that run inside kernels
+  void check_deferred() {
+    int e = 0;
+    HIP_OK(hipMemcpyAsync(&e, d_err, sizeof(int), hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    if (e) {
+      HIP_OK(hipMemsetAsync(d_err, 0, sizeof(int), stream));
+      throw std::runtime_error(
+          "encode vector out of range, please increase encoding level or increase first_mod_size & "
+          "scale_mod_size or decrease scale of msg");
+    }
+  }
   LimbMap q_lm{}, p_lm{};     // identity maps: limb t -> prime t / prime L+t
   // ace_alloc / ace_free: sizes of the buffers handed out, and freed buffers kept for reuse
   static constexpr size_t kPoolLimitWords = (size_t)4 << 30;  // 32 GiB
@@ -319,6 +336,17 @@ struct ace_ctx {
       u64 q = h.primes[i].q;
       pi[2 * i] = h.pinv_modq[i]; pi[2 * i + 1] = shoup(h.pinv_modq[i], q);
       pm[2 * i] = h.pmodq[i];     pm[2 * i + 1] = shoup(h.pmodq[i], q);
+    }
+    {
+      std::vector<double> rou_d;
+      std::vector<u32> rot;
+      fft_tables(h.N, rou_d, rot);
+      std::vector<double2> rou(rou_d.size() / 2);
+      for (size_t i = 0; i < rou.size(); ++i) rou[i] = make_double2(rou_d[2 * i], rou_d[2 * i + 1]);
+      fft_rou = upload_vec(rou);
+      rot_group = upload_vec(rot);
+      std::vector<int> z(1, 0);
+      d_err = upload_vec(z);
     }
     phat = upload_vec(ph);
     {
@@ -651,7 +679,12 @@ ace_ctx* ace_ctx_create(uint32_t degree, size_t num_q, size_t q0_bits, size_t sf
     g_err = e.what();
     return nullptr;
   }
-  return make_ctx(degree, q, num_parts);
+  ace_ctx* c = make_ctx(degree, q, num_parts);
+  if (c) {
+    c->q0_bits = q0_bits;
+    c->sf_bits = sf_bits;
+  }
+  return c;
 }
 
 ace_ctx* ace_ctx_create_with_primes(uint32_t degree, size_t num_q, const int64_t* q_primes, size_t num_parts) {
@@ -733,7 +766,7 @@ int ace_upload(ace_ctx* c, int64_t* dst, const int64_t* src, size_t n) {
 int ace_download(ace_ctx* c, int64_t* dst, const int64_t* src, size_t n) {
   ACE_TRY
   HIP_OK(hipMemcpyAsync(dst, src, n * sizeof(u64), hipMemcpyDeviceToHost, c->stream));
-  HIP_OK(hipStreamSynchronize(c->stream));
+  c->check_deferred();
   ACE_CATCH_INT
 }
 int ace_copy(ace_ctx* c, int64_t* dst, const int64_t* src, size_t n) {
@@ -748,7 +781,7 @@ int ace_zero(ace_ctx* c, int64_t* dst, size_t n) {
 }
 int ace_sync(ace_ctx* c) {
   ACE_TRY
-  HIP_OK(hipStreamSynchronize(c->stream));
+  c->check_deferred();
   ACE_CATCH_INT
 }
 int ace_timer_start(ace_ctx* c) {
@@ -861,6 +894,16 @@ int ace_host_twiddles(const ace_ctx* c, size_t prime_idx, int which, uint64_t* o
   std::memcpy(out, t[which]->data() + prime_idx * c->h.N, c->h.N * sizeof(u64));
   return 0;
 }
+int ace_host_fft_tables(const ace_ctx* c, double* rou, uint32_t* rot) {
+  if (!c || !rou || !rot) return fail("ace_host_fft_tables: null argument");
+  std::vector<double> r;
+  std::vector<u32> g;
+  fft_tables(c->h.N, r, g);
+  std::memcpy(rou, r.data(), r.size() * sizeof(double));
+  std::memcpy(rot, g.data(), (c->h.N / 2 ? c->h.N / 2 : 1) * sizeof(u32));
+  return 0;
+}
+
 int ace_host_tbl_modup(const ace_ctx* c, size_t level, size_t part, int64_t* hat_inv, int64_t* hat,
                        int32_t* compl_idx, size_t* n_digit, size_t* n_compl) {
   try {
@@ -1018,6 +1061,68 @@ int ace_transform_from_level0(ace_ctx* c, int64_t* res, const int64_t* src, size
   if (res != src && res < src + c->h.N && src < res + level * (size_t)c->h.N)
     return fail("ace_transform_from_level0: buffers overlap");
   launch_from_level0(c->stream, c->d, U(res), U(src), (u32)level);
+  ACE_CATCH_INT
+}
+
+int ace_embedding_inv(ace_ctx* c, double* host_out, const double* host_in, size_t len) {
+  ACE_TRY
+  if (!host_out || !host_in) return fail("ace_embedding_inv: null argument");
+  if (len == 0 || len > c->h.N / 2 || (len & (len - 1))) return fail("ace_embedding_inv: length must be a power of two of at most N/2");
+  c->ensure_ws(4 * len + 16);
+  c->ws_used = 0;
+  double2* r = reinterpret_cast<double2*>(c->take(2 * len));
+  double2* o = reinterpret_cast<double2*>(c->take(2 * len));
+  HIP_OK(hipMemcpyAsync(r, host_in, len * sizeof(double2), hipMemcpyHostToDevice, c->stream));
+  launch_embedding_inv(c->stream, c->d, o, r, c->fft_rou, c->rot_group, (u32)len);
+  HIP_OK(hipMemcpyAsync(host_out, o, len * sizeof(double2), hipMemcpyDeviceToHost, c->stream));
+  HIP_OK(hipStreamSynchronize(c->stream));
+  ACE_CATCH_INT
+}
+
+int ace_encode(ace_ctx* c, int64_t* res, const double* values, size_t n_values, uint32_t slots, size_t level,
+               uint32_t sf_degree, size_t p_cnt) {
+  ACE_TRY
+  if (!res || (!values && n_values)) return fail("ace_encode: null argument");
+  if (!c->sf_bits) return fail("ace_encode: the context was created from explicit primes and has no scaling factor");
+  const size_t N = c->h.N, K = c->h.K;
+  if (!slots) slots = (uint32_t)(N / 2);
+  if (!level) level = c->h.L;
+  if (level > c->h.L) return fail("level should not be larger than mul_depth + 1");
+  if (n_values > slots) return fail("slot size is too small");
+  if (slots > N / 2 || (slots & (slots - 1))) return fail("slot size must be a power of two of at most N/2");
+  if (p_cnt != 0 && p_cnt != K) return fail("ace_encode: p_cnt must be 0 or the number of special primes");
+  if (sf_degree < 1 || c->sf_bits * sf_degree >= c->q0_bits + (level - 1) * c->sf_bits)
+    return fail("invalid scaling factor for encode");
+  const double scaling_factor = std::ldexp(1.0, (int)c->sf_bits);
+  const double scale = std::pow(scaling_factor, (double)sf_degree);
+  // Check_msg_range (encoder.c:48-59): the largest scaled coefficient must stay below 2^(valid bits - 1)
+  const int valid = (int)c->q0_bits + (int)(level - 1) * (int)c->sf_bits;
+  const double range_bound = std::ldexp(1.0, valid - 1);
+  c->ensure_ws(c->std_ws(level));
+  c->ws_used = 0;
+  double2* z = reinterpret_cast<double2*>(c->take(2 * (size_t)slots));
+  launch_fill_zero(c->stream, reinterpret_cast<u64*>(z), 2 * (size_t)slots);
+  if (n_values)
+    HIP_OK(hipMemcpyAsync(z, values, n_values * sizeof(double2), hipMemcpyHostToDevice, c->stream));
+  LimbMap lm = poly_lm(c, level, p_cnt != 0);
+  const u32 n_limbs = (u32)(level + p_cnt);
+  launch_encode(c->stream, c->d, U(res), z, c->fft_rou, c->rot_group, slots, scaling_factor, scale, range_bound, lm,
+                n_limbs, c->d_err);
+  if (sf_degree > 1) {  // encoder.c:297-312: the Q limbs are multiplied by scaling_factor^(sf_degree-1)
+    std::vector<u64> cst(2 * level);
+    for (size_t t = 0; t < level; ++t) {
+      u64 q = c->h.primes[t].q, base = (u64)scaling_factor % q, powp = base;
+      for (uint32_t d = 2; d < sf_degree; ++d) powp = mul_mod(powp, base, q);
+      cst[2 * t] = powp;
+      cst[2 * t + 1] = shoup(powp, q);
+    }
+    u64* dc = c->take(2 * level);
+    HIP_OK(hipMemcpyAsync(dc, cst.data(), cst.size() * sizeof(u64), hipMemcpyHostToDevice, c->stream));
+    HIP_OK(hipStreamSynchronize(c->stream));  // cst is a local
+    launch_mul_const(c->stream, c->d, U(res), U(res), dc, c->q_lm, (u32)level);
+  }
+  PolySeq rs = seq_strided(U(res), 0);
+  launch_ntt(c->stream, c->d, rs, rs, lm, nullptr, n_limbs, 1, false, nullptr);
   ACE_CATCH_INT
 }
 

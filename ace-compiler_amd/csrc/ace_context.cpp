@@ -303,4 +303,16 @@ void automorphism_order(i64* order, uint32_t k, uint32_t n, bool is_ntt) {
   }
 }
 
+void fft_tables(uint32_t degree, std::vector<double>& rou, std::vector<uint32_t>& rot) {
+  const size_t M = 2 * (size_t)degree, ns = M / 4;
+  rou.resize(2 * M);
+  for (size_t i = 0; i < M; ++i) {
+    double angle = 2 * M_PI * i / M;
+    rou[2 * i] = cos(angle);
+    rou[2 * i + 1] = sin(angle);
+  }
+  rot.assign(ns ? ns : 1, 1);
+  for (size_t i = 1; i < ns; ++i) rot[i] = (uint32_t)((5ull * rot[i - 1]) % M);
+}
+
 }  // namespace ace

@@ -65,6 +65,11 @@ u64 pow_mod(u64 a, u64 e, u64 q);
 u64 inv_mod_prime(u64 a, u64 q);
 u64 shoup(u64 w, u64 q);
 uint32_t find_automorphism_index(int32_t rot_idx, uint32_t degree);
+// Precompute_fft (util/src/ntt.c:559-587) for fft_length = 2*degree: rou[2i], rou[2i+1] = cos, sin of
+// 2 pi i / (2*degree) for i < 2*degree; rot[i] = 5^i mod 2*degree for i < degree/2.
+// This file is built with the host C++ compiler, not hipcc, so that cos and sin are the C library's,
+// as in the reference: the encoder's results depend on the last bit of these tables.
+void fft_tables(uint32_t degree, std::vector<double>& rou, std::vector<uint32_t>& rot);
 void automorphism_order(i64* order, uint32_t k, uint32_t degree, bool is_ntt);
 
 }  // namespace ace

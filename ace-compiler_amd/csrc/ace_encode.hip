@@ -1,0 +1,111 @@
+// CKKS encoder on the device (Encode_impl, ckks/src/encoder.c:234-326): inverse
+// canonical embedding (Embedding_inv, util/src/ntt.c:631-675) in FP64, scaling,
+// rounding, and the split into RNS residues.  Every floating-point step is the
+// reference's operation in the reference's order with contraction off, so the
+// rounded integers -- and with them every residue -- are the same bits.
+#include "ace_kernels.h"
+
+namespace ace {
+
+constexpr int kEncThreads = 256;
+
+// one stage of Embedding_inv over `len` complex slots, in place: butterfly b
+// works on elements (j+i, j+i+num2) of block j
+__global__ __launch_bounds__(kEncThreads) void embed_inv_stage_kernel(double2* __restrict__ r,
+                                                                      const double2* __restrict__ rou,
+                                                                      const u32* __restrict__ rot, u32 M, u32 logm,
+                                                                      u32 len) {
+#pragma clang fp contract(off)
+  const u32 b = blockIdx.x * kEncThreads + threadIdx.x;
+  if (b >= (len >> 1)) return;
+  const u32 num2 = 1u << (logm - 1);
+  const u32 i = b & (num2 - 1), ie = ((b >> (logm - 1)) << logm) + i, io = ie + num2;
+  const u32 idx_mod = 1u << (logm + 2), gap = M / idx_mod;
+  const u32 rou_idx = (idx_mod - (rot[i] & (idx_mod - 1))) * gap;
+  const double2 x = r[ie], y = r[io], w = rou[rou_idx];
+  const double pr = x.x + y.x, pi = x.y + y.y, mr = x.x - y.x, mi = x.y - y.y;
+  // (mr + mi i) * (w.x + w.y i)
+  const double qr = mr * w.x - mi * w.y, qi = mr * w.y + mi * w.x;
+  r[ie] = make_double2(pr, pi);
+  r[io] = make_double2(qr, qi);
+}
+
+// Max_64bit_value (include/util/modular.h:279-281)
+__device__ __forceinline__ i64 max_64bit_value() { return (i64)(((u64)1 << 63) - ((u64)1 << 9)) - 1; }
+__device__ __forceinline__ i64 mod_int64(i64 v, i64 m) {
+  i64 r = v % m;
+  return r < 0 ? r + m : r;
+}
+
+// bit reversal and 1/len of Embedding_inv, then encoder.c:268-291 and
+// Transform_values_to_dcrt (util/src/crt.c:1153-1184): coefficient n of limb t.
+// Slot i lands its real part at coefficient i*gap and its imaginary part at
+// (i+slots)*gap; all other coefficients are zero.  err: set to 1 where the
+// reference asserts (value out of range for the level, or not an int64).
+__global__ __launch_bounds__(kEncThreads) void encode_round_kernel(DevCtx c, u64* __restrict__ out,
+                                                                   const double2* __restrict__ r, u32 slots,
+                                                                   u32 logslots, double scaling_factor, double scale,
+                                                                   double range_bound, LimbMap lm, int* err) {
+#pragma clang fp contract(off)
+  const u32 n = blockIdx.x * kEncThreads + threadIdx.x;
+  if (n >= c.N) return;
+  const u32 limb = blockIdx.y;
+  const i64 q = (i64)c.primes[lm.prime[limb]].q;
+  const u32 gap = c.N / (slots * 2);
+  i64 res = 0;
+  if (n % gap == 0) {
+    u32 i = n / gap;
+    const bool imag = i >= slots;
+    if (imag) i -= slots;
+    const u32 src = logslots ? (__brev(i) >> (32 - logslots)) : 0;
+    const double2 z = r[src];
+    const double v = (imag ? z.y : z.x) * (1.0 / (double)slots);  // slots is a power of two: exact, as the division is
+    if (fabs(v * scale) >= range_bound) *err = 1;
+    const double up = v * scaling_factor + 0.5;
+    if (!(up <= 9223372036854775807.0 && up >= -9223372036854775807.0)) {
+      *err = 1;
+    } else {
+      const i64 m = llround(up);
+      const i64 big = max_64bit_value();
+      const i64 msg = m < 0 ? big + m : m;
+      res = msg > (big >> 1) ? mod_int64(msg - (big - q), q) : mod_int64(msg, q);
+    }
+  }
+  out[(u64)limb * c.N + n] = (u64)res;
+}
+
+// the inverse embedding alone: r (len complex values, overwritten) -> out[i] = r[bitrev(i)] / len
+__global__ __launch_bounds__(kEncThreads) void embed_inv_finish_kernel(double2* __restrict__ out,
+                                                                       const double2* __restrict__ r, u32 len,
+                                                                       u32 loglen) {
+  const u32 i = blockIdx.x * kEncThreads + threadIdx.x;
+  if (i >= len) return;
+  const double2 z = r[loglen ? (__brev(i) >> (32 - loglen)) : 0];
+  const double inv = 1.0 / (double)len;
+  out[i] = make_double2(z.x * inv, z.y * inv);
+}
+void launch_embedding_inv(hipStream_t st, const DevCtx& c, double2* out, double2* r, const double2* rou,
+                          const u32* rot, u32 len) {
+  u32 loglen = 0;
+  while ((1u << loglen) < len) ++loglen;
+  for (u32 logm = loglen; logm > 0; --logm)
+    hipLaunchKernelGGL(embed_inv_stage_kernel, dim3(((len >> 1) + kEncThreads - 1) / kEncThreads), dim3(kEncThreads), 0,
+                       st, r, rou, rot, 2 * c.N, logm, len);
+  hipLaunchKernelGGL(embed_inv_finish_kernel, dim3((len + kEncThreads - 1) / kEncThreads), dim3(kEncThreads), 0, st,
+                     out, r, len, loglen);
+}
+
+void launch_encode(hipStream_t st, const DevCtx& c, u64* out, double2* r, const double2* rou, const u32* rot,
+                   u32 slots, double scaling_factor, double scale, double range_bound, const LimbMap& lm,
+                   u32 n_limbs, int* err) {
+  u32 logslots = 0;
+  while ((1u << logslots) < slots) ++logslots;
+  const u32 M = 2 * c.N;
+  for (u32 logm = logslots; logm > 0; --logm)
+    hipLaunchKernelGGL(embed_inv_stage_kernel, dim3(((slots >> 1) + kEncThreads - 1) / kEncThreads), dim3(kEncThreads),
+                       0, st, r, rou, rot, M, logm, slots);
+  hipLaunchKernelGGL(encode_round_kernel, dim3((c.N + kEncThreads - 1) / kEncThreads, n_limbs), dim3(kEncThreads), 0,
+                     st, c, out, r, slots, logslots, scaling_factor, scale, range_bound, lm, err);
+}
+
+}  // namespace ace

@@ -106,5 +106,14 @@ void launch_pick_limb(hipStream_t st, const DevCtx& c, u64* dst, const PolySeq& 
 void launch_mul_const(hipStream_t st, const DevCtx& c, u64* out, const u64* src, const u64* cst, const LimbMap& lm,
                       u32 n_limbs);
 void launch_fill_zero(hipStream_t st, u64* p, u64 n);
+// Embedding_inv (util/src/ntt.c:631-675) over len complex values: out = result, r = input (overwritten)
+void launch_embedding_inv(hipStream_t st, const DevCtx& c, double2* out, double2* r, const double2* rou,
+                          const u32* rot, u32 len);
+// Encode_impl up to the residues (coefficient form): r holds `slots` complex values on entry (zero-padded
+// message) and is used as scratch; rou = exp(2 pi i k / 2N), k < 2N; rot = 5^k mod 2N, k < N/2.
+// out: n_limbs limbs of N words (limb t uses lm.prime[t]).  *err is set to 1 where the reference asserts.
+void launch_encode(hipStream_t st, const DevCtx& c, u64* out, double2* r, const double2* rou, const u32* rot,
+                   u32 slots, double scaling_factor, double scale, double range_bound, const LimbMap& lm,
+                   u32 n_limbs, int* err);
 
 }  // namespace ace

@@ -68,6 +68,8 @@ void     ace_modulus(const ace_ctx* ctx, size_t prime_idx, uint64_t out[5]);
  * ace_host_tbl_rescale: q_l^-1 mod q_i and the reference's second rescale
  *   constant (== -q_l^-1 mod q_i), i < level-1 (crt.c:299-349). */
 int ace_host_twiddles(const ace_ctx* ctx, size_t prime_idx, int which, uint64_t* out);
+/* Precompute_fft (util/src/ntt.c:559-587), fft_length 2N: rou = 2N (cos, sin) pairs, rot = N/2 powers of 5 */
+int ace_host_fft_tables(const ace_ctx* ctx, double* rou, uint32_t* rot);
 int ace_host_tbl_modup(const ace_ctx* ctx, size_t level, size_t part, int64_t* hat_inv, int64_t* hat,
                        int32_t* compl_idx, size_t* n_digit, size_t* n_compl);
 int ace_host_tbl_moddown(const ace_ctx* ctx, int64_t* phat_inv, int64_t* phat_modq, int64_t* pinv_modq, int64_t* pmodq);
@@ -161,6 +163,17 @@ int ace_reduce_rescale_modup(ace_ctx* ctx, int64_t* res, int64_t* raised, int64_
 /* Transform_values_from_level0 (:1101-1125): limb 0 of src copied, limb i of res =
  * Switch_modulus(limb 0, q_0 -> q_i), i < level. */
 int ace_transform_from_level0(ace_ctx* ctx, int64_t* res, const int64_t* src, size_t level);
+/* Embedding_inv (util/src/ntt.c:631-675) on `len` complex numbers, host to host through the device */
+int ace_embedding_inv(ace_ctx* ctx, double* host_out, const double* host_in, size_t len);
+/* Encode_impl (ckks/src/encoder.c:234-326; Encode_at_level_with_sf, Encode_ext_at_level): `values` is a
+ * HOST array of n_values complex numbers (re, im interleaved), zero-padded to `slots` (0: N/2); the
+ * plaintext polynomial lands in res: level (0: all) Q limbs followed by p_cnt (0 or num_p) P limbs, NTT
+ * form, scale 2^(sf_bits * sf_degree).  The inverse embedding, rounding and residues are computed on the
+ * device with the reference's floating-point operations in the reference's order.  Where the
+ * reference asserts on a value out of range for the level, a flag is raised inside the kernel and
+ * reported by the next ace_sync / ace_download. */
+int ace_encode(ace_ctx* ctx, int64_t* res, const double* values, size_t n_values, uint32_t slots, size_t level,
+               uint32_t sf_degree, size_t p_cnt);
 /* Extend (:483-500): src level limbs -> res level+num_p limbs (P limbs zero) */
 int ace_extend(ace_ctx* ctx, int64_t* res, const int64_t* src, size_t level);
 /* Dot_prod / Fast_dot_prod (:502-529): digits = n_parts x (level+num_p) limbs;

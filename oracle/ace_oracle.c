@@ -1239,6 +1239,8 @@ static void embedding(const orc_ctx* c, dcmplx* res, const dcmplx* coeffs, size_
   }
 }
 
+const double* orc_fft_rou(const orc_ctx* c) { return c->fft_rou; }
+
 void orc_embedding(const orc_ctx* c, double* res, const double* coeffs, size_t len, int inverse) {
   if (inverse) embedding_inv(c, (dcmplx*)res, (const dcmplx*)coeffs, len);
   else embedding(c, (dcmplx*)res, (const dcmplx*)coeffs, len);

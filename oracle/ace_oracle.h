@@ -163,6 +163,8 @@ void orc_mul_relin_rescale(const orc_ctx* c, int64_t* r0, int64_t* r1, const int
 
 /* ---- encoder (ckks/src/encoder.c, util/src/ntt.c:598-675) ---- */
 /* Embedding / Embedding_inv over `len` complex slots (re, im interleaved) */
+/* the 2N (cos, sin) pairs of Precompute_fft */
+const double* orc_fft_rou(const orc_ctx* c);
 void orc_embedding(const orc_ctx* c, double* res, const double* coeffs, size_t len, int inverse);
 /* Encode_impl (encoder.c:234-326): 1 on success, 0 where the reference asserts on range */
 int orc_encode(const orc_ctx* c, int64_t* out, const double* values, size_t n_values, uint32_t slots, size_t level,

@@ -237,6 +237,35 @@ def test_mod_down_rescale_family(pair):
         g.mod_down_rescale(g.alloc(N), g.alloc(N), 1, True)
 
 
+def test_encode(pair):
+    """Device encoder vs the oracle's (itself matched against the reference's compiled encoder): same residues."""
+    g, o = pair.g, pair.o
+    N, (q0_bits, sf_bits) = g.N, pair.cfg[2:4]
+    rng = np.random.default_rng(N)
+    for slots in sorted({N // 2, max(1, N // 8), min(4, N // 2), 1}):
+        z = rng.uniform(-1, 1, slots) + 1j * rng.uniform(-1, 1, slots)
+        for level, deg, pc in ((g.L, 1, 0), (min(2, g.L), 1, 0), (g.L, 2, 0), (g.L, 3, 0), (max(1, g.L - 1), 1, g.K)):
+            if deg * sf_bits >= q0_bits + (level - 1) * sf_bits:
+                with pytest.raises(acefhe.AceError):
+                    g.encode(g.alloc((level + pc) * N), z, slots, level, deg, pc)
+                continue
+            vals = z[:max(1, slots - 1)] * 3.0
+            want = o.encode(vals, slots, level, deg, pc)
+            assert want is not None
+            dr = g.alloc((level + pc) * N)
+            g.encode(dr, vals, slots, level, deg, pc)
+            eq(dr, want, "encode slots=%d level=%d sf_degree=%d p=%d" % (slots, level, deg, pc))
+    # a value too large for the level: the reference asserts, the library reports it at the next synchronisation
+    if q0_bits + (g.L - 1) * sf_bits - sf_bits < 62:
+        big = np.array([2.0 ** (q0_bits + (g.L - 1) * sf_bits - sf_bits)])
+        assert o.encode(big, 1, g.L, 1, 0) is None
+        dr = g.alloc(g.L * N)
+        g.encode(dr, big, 1, g.L, 1, 0)
+        with pytest.raises(acefhe.AceError):
+            g.sync()
+        g.sync()  # the flag is cleared once reported
+
+
 def make_swk(g, seed):
     return np.concatenate([seeded.uniform_poly(seed + i, g.primes, g.N) for i in range(2 * g.parts)])
 

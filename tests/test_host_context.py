@@ -89,3 +89,29 @@ def test_no_gpu_means_no_compute():
     assert b"no HIP device" in lib.ace_last_error()
     assert lib.ace_mul_relin_rescale(c.h, *([dummy] * 7), 2) != 0
     c.close()
+
+
+def test_fft_tables_match_the_oracle_bit_for_bit():
+    """The encoder's root table must carry the very doubles the reference computes (gcc's cos / sin of the C
+    library; the oracle's table, whose encoder is matched against the reference's): at a 50-bit scaling factor
+    one unit in the last place of a twiddle changes rounded coefficients.  A build of the host tables with
+    another compiler's math calls differs in about one entry in a thousand."""
+    import ctypes as C
+    import numpy as np
+    import acefhe
+    from oracle_lib import Oracle
+    cfg = (16384, 4, 60, 50, 2)
+    g = acefhe.Context(*cfg)
+    rou, rot = g.host_fft_tables()
+    g.close()
+    M = 2 * cfg[0]
+    o = Oracle(*cfg)
+    o.L_.orc_fft_rou.restype = C.POINTER(C.c_double)
+    o.L_.orc_fft_rou.argtypes = [C.c_void_p]
+    want = np.ctypeslib.as_array(o.L_.orc_fft_rou(o.h), shape=(2 * M,)).copy()
+    assert np.array_equal(rou.view(np.int64), want.view(np.int64))
+    pw = [1]
+    for _ in range(cfg[0] // 2 - 1):
+        pw.append(pw[-1] * 5 % M)
+    assert rot.tolist() == pw
+    o.close()

@@ -10,7 +10,7 @@ from refdrv import RefSession
 
 pytestmark = pytest.mark.skipif(not refdrv.available(), reason="compiled reference not built")
 
-CONFIGS = [(64, 4, 50, 40, 2), (1024, 5, 45, 40, 3), (8192, 5, 40, 40, 3)]
+CONFIGS = [(64, 4, 50, 40, 2), (1024, 5, 45, 40, 3), (8192, 5, 40, 40, 3), (16384, 4, 60, 50, 2)]
 
 
 def bits(a):
