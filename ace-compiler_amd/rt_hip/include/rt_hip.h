@@ -68,7 +68,7 @@ typedef struct {
   size_t   _input_level;
   size_t   _first_mod_size;   /* bits of q_0 */
   size_t   _scaling_mod_size; /* bits of the other Q primes */
-  size_t   _num_q_parts;      /* 0: default (3) */
+  size_t   _num_q_parts;      /* 0: by depth (1, 2 up to depth 3, else 3) */
   size_t   _hamming_weight;
   size_t   _num_rot_idx;
   int32_t  _rot_idxs[];
@@ -122,6 +122,31 @@ typedef struct {
 } CIPHERTEXT3;
 typedef CIPHERTEXT*  CIPHER;
 typedef CIPHERTEXT3* CIPHER3;
+
+/* ---- plaintext (include/ckks/plaintext.h:23-28) ---- */
+typedef struct {
+  POLYNOMIAL _poly;
+  uint32_t   _slots;
+  double     _scaling_factor;
+  uint32_t   _sf_degree;
+} PLAINTEXT;
+typedef PLAINTEXT* PLAIN;
+typedef double _Complex DCMPLX;
+
+/* ---- tensors handed to Prepare_input (include/common/tensor.h:20-63) ---- */
+typedef struct {
+  SHAPE  _shape;
+  double _vals[];
+} TENSOR;
+#define TENSOR_N(T) (T)->_shape._n
+#define TENSOR_C(T) (T)->_shape._c
+#define TENSOR_H(T) (T)->_shape._h
+#define TENSOR_W(T) (T)->_shape._w
+#define TENSOR_SIZE(T) TENSOR_N(T) * TENSOR_C(T) * TENSOR_H(T) * TENSOR_W(T)
+static inline float* Slice(float* vec, size_t row_idx, size_t col) { return vec + row_idx * col; }
+TENSOR* Alloc_tensor(size_t n, size_t c, size_t h, size_t w, const double* val);
+void    Free_tensor(TENSOR* tensor);
+void    Print_tensor(FILE* fp, TENSOR* tensor);
 
 /* ---- keys (include/ckks/public_key.h:24-27, switch_key.h:27-29) ---- */
 typedef struct {
@@ -198,10 +223,14 @@ static inline void Alloc_poly_data(POLY p, uint32_t degree, size_t num_q, size_t
   p->_data             = Rt_dev_alloc((num_q + num_p) * (size_t)degree);
 }
 void Free_poly_data(POLY p);
+/* Generated code passes the third argument as a flag (1 for an extended polynomial) whatever the
+ * number of P primes is.  A polynomial with some but not all P limbs means nothing to hybrid key
+ * switching (Mod_up, Mod_down assume the full P base), so any non-zero count allocates all of them. */
+size_t Get_p_cnt(void);
 static inline POLY Alloc_poly(uint32_t degree, size_t num_q, size_t num_p) {
   FMT_ASSERT(num_q > 0, "Alloc_poly: q primes should not be NULL");
   POLY p = (POLY)calloc(1, sizeof(POLYNOMIAL));
-  Alloc_poly_data(p, degree, num_q, num_p);
+  Alloc_poly_data(p, degree, num_q, num_p ? Get_p_cnt() : 0);
   p->_is_ntt = true;
   return p;
 }
@@ -293,6 +322,39 @@ CIPHER   Modswitch_ciph(CIPHER res, CIPHER c);
 CIPHER   Rotate_ciph(CIPHER res, CIPHER c, int32_t rot_idx);
 void     Rotate_batch_ciph(CIPHER res_arr, CIPHER c, const int32_t* rot_idx, uint32_t cnt);
 CIPHER   Conjugate_ciph(CIPHER res, CIPHER c);
+
+/* ---- plaintexts (include/ckks/plain.h:24-117, ckks/src/plain.c, cipher.c:58-84,373-396) ----
+ * Vectors are encoded on the device (ace_encode); a single value (len == 1) becomes the constant
+ * residues of Encode_val_at_level (ckks/src/encoder.c:473-575). */
+static inline POLY Get_plain_poly(PLAIN p) { return &p->_poly; }
+void   Encode_float(PLAIN plain, float* input, size_t len, uint32_t sc_degree, uint32_t level);
+void   Encode_double(PLAIN plain, double* input, size_t len, uint32_t sc_degree, uint32_t level);
+void   Encode_dcmplx(PLAIN plain, DCMPLX* input, size_t len, uint32_t sc_degree, uint32_t level);
+void   Encode_float_mask(PLAIN plain, float cst, size_t len, uint32_t sc_degree, uint32_t level);
+void   Encode_double_mask(PLAIN plain, double cst, size_t len, uint32_t sc_degree, uint32_t level);
+void   Encode_dcmplx_ext(PLAIN plain, DCMPLX* input, size_t len, uint32_t level, uint32_t p_cnt);
+void   Encode_single_float(int64_t* res, float input, uint32_t sc_degree, uint32_t level);   /* host words */
+void   Encode_single_double(int64_t* res, double input, uint32_t sc_degree, uint32_t level); /* host words */
+double* Get_msg_from_plain(PLAIN plain);        /* decoded real parts, _slots values; caller frees */
+DCMPLX* Get_dcmplx_msg_from_plain(PLAIN plain); /* decoded slots; caller frees */
+void   Free_plain_poly(PLAIN plain);
+void   Init_ciph_same_scale_plain(CIPHER res, CIPHER c, PLAIN plain);
+void   Init_ciph_up_scale_plain(CIPHER res, CIPHER c, PLAIN plain);
+CIPHER Add_plain(CIPHER res, CIPHER c, PLAIN plain);
+CIPHER Mul_plain(CIPHER res, CIPHER c, PLAIN plain);
+
+/* ---- keys, encryption, decryption (ckks/src/key_gen.c:127-262, encryptor.c:19-75, decryptor.c, rtlib.c:164-229) ----
+ * Rt_generate_keys: secret (ternary with the context's Hamming weight; uniform ternary when that is 0), public key,
+ * relinearisation key and one "fast" rotation key per index of Get_context_params()->_rot_idxs, from a
+ * generator seeded with `seed` (0: the environment's RT_HIP_SEED, else the clock).  Prepare_input and
+ * Handle_output need it; programs that load their own keys (Rt_load_switch_key) do not. */
+void    Rt_generate_keys(uint64_t seed);
+void    Rt_generate_rotation_key(int32_t rot_idx);
+CIPHER  Encrypt(CIPHER res, PLAIN plain);
+void    Rt_decrypt(PLAIN res, CIPHER c);
+void    Rt_decode(DCMPLX* res, PLAIN plain); /* plain->_slots values */
+void    Prepare_input(TENSOR* input, const char* name);
+double* Handle_output(const char* name); /* caller frees */
 
 /* ---- program inputs / outputs (ckks/src/rtlib.c:231-244) ---- */
 CIPHERTEXT Get_input_data(const char* name, size_t idx); /* by value; the program owns the polys */

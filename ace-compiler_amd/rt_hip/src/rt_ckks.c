@@ -1,0 +1,671 @@
+/* rt_ckks.c -- the scheme-level part of the host runtime: key generation, plaintext
+ * encoding entry points, encryption, decryption and decoding, program inputs and
+ * outputs.  Polynomial arithmetic runs on the device through ace_hip.h; what stays
+ * on the host is sampling, the few-word constants of single-value plaintexts and the
+ * multi-precision reconstruction of decoded coefficients.
+ */
+#include <complex.h>
+#include <math.h>
+
+#include "rt_internal.h"
+
+/* ---- random numbers: xoshiro256** seeded through splitmix64 --------------------------------- */
+static uint64_t Rng[4];
+static uint64_t splitmix(uint64_t* s) {
+  uint64_t z = (*s += 0x9E3779B97F4A7C15ull);
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+static void rng_seed(uint64_t seed) {
+  for (int i = 0; i < 4; ++i) Rng[i] = splitmix(&seed);
+}
+static inline uint64_t rotl(uint64_t x, int k) { return (x << k) | (x >> (64 - k)); }
+static uint64_t rng_next(void) {
+  uint64_t r = rotl(Rng[1] * 5, 7) * 9, t = Rng[1] << 17;
+  Rng[2] ^= Rng[0];
+  Rng[3] ^= Rng[1];
+  Rng[1] ^= Rng[2];
+  Rng[0] ^= Rng[3];
+  Rng[2] ^= t;
+  Rng[3] = rotl(Rng[3], 45);
+  return r;
+}
+static uint64_t rng_below(uint64_t bound) { /* unbiased, by rejection */
+  uint64_t lim = UINT64_MAX - UINT64_MAX % bound;
+  for (;;) {
+    uint64_t v = rng_next();
+    if (v < lim) return v % bound;
+  }
+}
+
+/* Sample_triangle (util/src/random_sample.c:80-99): -1, 1 with probability 1/4 each, else 0 */
+static void sample_triangle(int64_t* v, size_t n) {
+  for (size_t i = 0; i < n; ++i) {
+    uint64_t r = rng_next() & 3;
+    v[i] = r == 0 ? -1 : r == 1 ? 1 : 0;
+  }
+}
+/* Sample_ternary (random_sample.c:101-156): weight 0 draws every coefficient uniformly from
+ * {-1, 0, 1}; otherwise exactly `weight` coefficients are +-1, redrawn until the +1s number
+ * weight/2 to within one */
+static void sample_ternary(int64_t* v, size_t n, size_t weight) {
+  if (weight == 0) {
+    for (size_t i = 0; i < n; ++i) v[i] = (int64_t)rng_below(3) - 1;
+    return;
+  }
+  if (weight > n) weight = n;
+  for (;;) {
+    size_t ones = 0;
+    memset(v, 0, n * sizeof(int64_t));
+    for (size_t done = 0; done < weight;) {
+      size_t i = (size_t)rng_below(n);
+      if (v[i]) continue;
+      v[i] = (rng_next() & 1) ? 1 : -1;
+      ones += v[i] == 1;
+      ++done;
+    }
+    if (ones + 1 >= weight / 2 && ones <= weight / 2 + 1) return;
+  }
+}
+
+/* ---- small helpers over the device ------------------------------------------------------------ */
+static size_t prime_of_limb(size_t t, size_t level) { return t < level ? t : G.L + (t - level); }
+
+/* signed small coefficients -> residues of `level` Q limbs (+ the P limbs), NTT form, in dev */
+static void small_to_dev(int64_t* dev, const int64_t* v, size_t level, bool with_p) {
+  size_t   n = G.N, T = level + (with_p ? G.K : 0);
+  int64_t* host = (int64_t*)malloc(T * n * sizeof(int64_t));
+  int32_t  idx[128];
+  for (size_t t = 0; t < T; ++t) {
+    int64_t q = G.q[prime_of_limb(t, level)]._val;
+    idx[t]    = (int32_t)prime_of_limb(t, level);
+    for (size_t i = 0; i < n; ++i) host[t * n + i] = v[i] < 0 ? v[i] + q : v[i];
+  }
+  ACE_OK(ace_upload(G.ctx, dev, host, T * n));
+  ACE_OK(ace_ntt(G.ctx, dev, dev, idx, T, 1, 0));
+  free(host);
+}
+/* uniform residues: a uniform polynomial is uniform in NTT form too */
+static void uniform_to_dev(int64_t* dev, size_t level, bool with_p) {
+  size_t   n = G.N, T = level + (with_p ? G.K : 0);
+  int64_t* host = (int64_t*)malloc(T * n * sizeof(int64_t));
+  for (size_t t = 0; t < T; ++t) {
+    uint64_t q = (uint64_t)G.q[prime_of_limb(t, level)]._val;
+    for (size_t i = 0; i < n; ++i) host[t * n + i] = (int64_t)rng_below(q);
+  }
+  ACE_OK(ace_upload(G.ctx, dev, host, T * n));
+  free(host);
+}
+
+/* ---- keys (ckks/src/key_gen.c:127-262) ----------------------------------------------------------- */
+/* host words of a switch key taking a polynomial that multiplies s_src to a pair that decrypts under
+ * s_res (both: device, L+k limbs, NTT): per digit b = -a*s_res + e + P*s_src on the digit's limbs */
+static int64_t* make_switch_key(const int64_t* s_res, const int64_t* s_src) {
+  size_t   n = G.N, T = G.L + G.K, ps = ace_part_size(G.ctx);
+  int64_t* key = (int64_t*)malloc(2 * G.parts * T * n * sizeof(int64_t));
+  int64_t *a = Rt_dev_alloc(T * n), *b = Rt_dev_alloc(T * n), *e = Rt_dev_alloc(T * n), *t = Rt_dev_alloc(n);
+  int64_t* small = (int64_t*)malloc(n * sizeof(int64_t));
+  unsigned __int128 P = 1; /* only P mod q_i is needed */
+  for (size_t d = 0; d < G.parts; ++d) {
+    uniform_to_dev(a, G.L, true);
+    sample_triangle(small, n);
+    small_to_dev(e, small, G.L, true);
+    ACE_OK(ace_poly_mul(G.ctx, b, a, s_res, G.L, 1));
+    ACE_OK(ace_poly_sub(G.ctx, b, e, b, G.L, 1));
+    for (size_t i = d * ps; i < (d + 1) * ps && i < G.L; ++i) {
+      uint64_t q = (uint64_t)G.q[i]._val, pm = 1;
+      for (size_t j = 0; j < G.K; ++j) pm = (uint64_t)((unsigned __int128)pm * ((uint64_t)G.p[j]._val % q) % q);
+      ACE_OK(ace_hw_modmul_scalar(G.ctx, t, s_src + i * n, (int64_t)pm, i, n));
+      ACE_OK(ace_hw_modadd(G.ctx, b + i * n, b + i * n, t, i, n));
+    }
+    ACE_OK(ace_download(G.ctx, key + (2 * d) * T * n, b, T * n));
+    ACE_OK(ace_download(G.ctx, key + (2 * d + 1) * T * n, a, T * n));
+  }
+  (void)P;
+  free(small);
+  Rt_dev_free(a);
+  Rt_dev_free(b);
+  Rt_dev_free(e);
+  Rt_dev_free(t);
+  return key;
+}
+
+/* sigma_k on signed coefficients: X^i -> X^(i k mod 2N), negated past N */
+static void automorphism_small(int64_t* out, const int64_t* v, uint64_t k) {
+  size_t n = G.N;
+  for (size_t i = 0; i < n; ++i) {
+    uint64_t j = (uint64_t)i * k % (2 * n);
+    out[j % n] = j >= n ? -v[i] : v[i];
+  }
+}
+static uint64_t inv_mod_pow2(uint64_t k, uint64_t m) { /* k odd, m a power of two */
+  uint64_t x = k;                                        /* Newton: doubles the correct bits */
+  for (int i = 0; i < 6; ++i) x *= 2 - k * x;
+  return x & (m - 1);
+}
+
+void Rt_generate_rotation_key(int32_t rot_idx) {
+  FMT_ASSERT(G.secret_ntt, "Rt_generate_keys() has not run");
+  size_t   n = G.N, T = G.L + G.K;
+  uint32_t k = (uint32_t)rot_idx == 2 * G.N - 1 ? 2 * G.N - 1 : ace_find_automorphism_index(G.ctx, rot_idx);
+  /* "fast" key: the evaluator switches the un-rotated c1 and applies the automorphism last, so the
+   * key leads from s to sigma_k^-1(s) (key_gen.c:216-262) */
+  int64_t* rs = (int64_t*)malloc(n * sizeof(int64_t));
+  automorphism_small(rs, G.secret_small, inv_mod_pow2(k, 2 * n));
+  int64_t* s_res = Rt_dev_alloc(T * n);
+  small_to_dev(s_res, rs, G.L, true);
+  int64_t* key = make_switch_key(s_res, G.secret_ntt);
+  Rt_load_switch_key(true, rot_idx, key);
+  free(key);
+  free(rs);
+  Rt_dev_free(s_res);
+}
+
+void Rt_generate_keys(uint64_t seed) {
+  NEED_CTX();
+  if (!seed) {
+    const char* env = getenv("RT_HIP_SEED");
+    seed = env ? strtoull(env, NULL, 0) : 0;
+    if (!seed) seed = (uint64_t)time(NULL) ^ ((uint64_t)clock() << 32) ^ 0x5DEECE66Dull;
+  }
+  rng_seed(seed);
+  Rt_ckks_finalize(); /* a second call replaces the keys */
+  CKKS_PARAMS* prm = Get_context_params();
+  size_t       n = G.N, T = G.L + G.K, hw = prm->_hamming_weight;
+  G.secret_small = (int64_t*)malloc(n * sizeof(int64_t));
+  sample_ternary(G.secret_small, n, hw);
+  G.secret_ntt = Rt_dev_alloc(T * n);
+  small_to_dev(G.secret_ntt, G.secret_small, G.L, true);
+  /* public key: pk1 = a, pk0 = -a s + e  (L limbs) */
+  G.pk0 = Rt_dev_alloc(G.L * n);
+  G.pk1 = Rt_dev_alloc(G.L * n);
+  int64_t* small = (int64_t*)malloc(n * sizeof(int64_t));
+  int64_t* e     = Rt_dev_alloc(G.L * n);
+  uniform_to_dev(G.pk1, G.L, false);
+  sample_triangle(small, n);
+  small_to_dev(e, small, G.L, false);
+  ACE_OK(ace_poly_mul(G.ctx, G.pk0, G.pk1, G.secret_ntt, G.L, 0));
+  ACE_OK(ace_poly_sub(G.ctx, G.pk0, e, G.pk0, G.L, 0));
+  Rt_dev_free(e);
+  free(small);
+  /* relinearisation key: from s^2 to s */
+  int64_t* s2 = Rt_dev_alloc(T * n);
+  ACE_OK(ace_poly_mul(G.ctx, s2, G.secret_ntt, G.secret_ntt, G.L, 1));
+  int64_t* key = make_switch_key(G.secret_ntt, s2);
+  Rt_load_switch_key(false, 0, key);
+  free(key);
+  Rt_dev_free(s2);
+  for (size_t i = 0; i < prm->_num_rot_idx; ++i)
+    if (!Rt_find_rot(prm->_rot_idxs[i])) Rt_generate_rotation_key(prm->_rot_idxs[i]); /* index 0 included: generated code asks for it */
+}
+
+void Rt_ckks_finalize(void) {
+  free(G.secret_small);
+  if (G.secret_ntt) Rt_dev_free(G.secret_ntt);
+  if (G.pk0) Rt_dev_free(G.pk0);
+  if (G.pk1) Rt_dev_free(G.pk1);
+  free(G.fft_rou);
+  free(G.rot_group);
+  G.secret_small = NULL;
+  G.secret_ntt = G.pk0 = G.pk1 = NULL;
+  G.fft_rou   = NULL;
+  G.rot_group = NULL;
+}
+
+/* ---- plaintexts ------------------------------------------------------------------------------------- */
+static void init_plain(PLAIN plain, size_t level, double scale, uint32_t sf_degree, uint32_t slots) {
+  POLY p = &plain->_poly;
+  if (p->_data && (p->_num_primes != level || p->_num_primes_p != 0)) Free_poly_data(p);
+  if (!p->_data) Alloc_poly_data(p, G.N, level, 0);
+  plain->_scaling_factor = scale;
+  plain->_sf_degree      = sf_degree;
+  plain->_slots          = slots;
+  p->_is_ntt             = true;
+}
+
+static void check_sf(uint32_t sf_degree, size_t level) {
+  CKKS_PARAMS* prm = Get_context_params();
+  FMT_ASSERT(sf_degree >= 1 && prm->_scaling_mod_size * sf_degree <
+                                   prm->_first_mod_size + (level - 1) * prm->_scaling_mod_size,
+             "invalid scaling factor for encode");
+}
+
+/* Encode_val_at_level (ckks/src/encoder.c:473-575): the same residue in every coefficient */
+static void encode_value(PLAIN plain, double value, uint32_t sc_degree, uint32_t level) {
+  CKKS_PARAMS* prm = Get_context_params();
+  if (level == 0) level = (uint32_t)G.L;
+  FMT_ASSERT(level <= G.L, "level should not be larger than mul_depth + 1");
+  check_sf(sc_degree, level);
+  double scale = pow(G.sc, sc_degree);
+  init_plain(plain, level, scale, sc_degree, G.N / 2);
+  int32_t log_scale = (int32_t)(log2(fabs(value * scale)));
+  FMT_ASSERT(log_scale <= 61, "encode %f: values that need the approximation factor are not supported", value);
+  double scaled = value * scale; /* approximation factor 2^0 */
+  FMT_ASSERT(scaled <= 9223372036854775807.0 && scaled >= -9223372036854775807.0,
+             "encode %f with scale %f overflow, please choose a smaller scale", value, scale);
+  FMT_ASSERT(log_scale + 1 < (int32_t)prm->_first_mod_size + (int32_t)(level - 1) * (int32_t)prm->_scaling_mod_size,
+             "encode value out of range, please increase encoding level or increase first_mod_size & "
+             "scale_mod_size or decrease scale of msg");
+  int64_t v = (int64_t)scaled;
+  int64_t zero_one[2];
+  for (uint32_t t = 0; t < level; ++t) {
+    int64_t q = G.q[t]._val, r = v % q;
+    if (r < 0) r += q;
+    /* limb t = the constant r: zero it, then add r to every word */
+    zero_one[0] = r;
+    ACE_OK(ace_zero(G.ctx, plain->_poly._data + (size_t)t * G.N, G.N));
+    ACE_OK(ace_hw_modadd_scalar(G.ctx, plain->_poly._data + (size_t)t * G.N, plain->_poly._data + (size_t)t * G.N,
+                                zero_one[0], t, G.N));
+  }
+}
+
+static void encode_vector(PLAIN plain, const double* re_im, size_t len, uint32_t sc_degree, uint32_t level) {
+  if (level == 0) level = (uint32_t)G.L;
+  FMT_ASSERT(level <= G.L, "level should not be larger than mul_depth + 1");
+  init_plain(plain, level, pow(G.sc, sc_degree), sc_degree, G.N / 2);
+  ACE_OK(ace_encode(G.ctx, plain->_poly._data, re_im, len, 0, level, sc_degree, 0));
+}
+
+void Encode_double(PLAIN plain, double* input, size_t len, uint32_t sc_degree, uint32_t level) {
+  if (len == 1) {
+    encode_value(plain, *input, sc_degree, level);
+    return;
+  }
+  double* v = (double*)calloc(2 * len, sizeof(double));
+  for (size_t i = 0; i < len; ++i) v[2 * i] = input[i];
+  encode_vector(plain, v, len, sc_degree, level);
+  free(v);
+}
+void Encode_float(PLAIN plain, float* input, size_t len, uint32_t sc_degree, uint32_t level) {
+  if (len == 1) {
+    encode_value(plain, (double)*input, sc_degree, level);
+    return;
+  }
+  double* v = (double*)calloc(2 * len, sizeof(double));
+  for (size_t i = 0; i < len; ++i) v[2 * i] = (double)input[i];
+  encode_vector(plain, v, len, sc_degree, level);
+  free(v);
+}
+void Encode_dcmplx(PLAIN plain, DCMPLX* input, size_t len, uint32_t sc_degree, uint32_t level) {
+  encode_vector(plain, (const double*)input, len, sc_degree, level);
+}
+void Encode_double_mask(PLAIN plain, double cst, size_t len, uint32_t sc_degree, uint32_t level) {
+  double* v = (double*)calloc(2 * len, sizeof(double));
+  for (size_t i = 0; i < len; ++i) v[2 * i] = cst;
+  encode_vector(plain, v, len, sc_degree, level);
+  free(v);
+}
+void Encode_float_mask(PLAIN plain, float cst, size_t len, uint32_t sc_degree, uint32_t level) {
+  Encode_double_mask(plain, (double)cst, len, sc_degree, level);
+}
+void Encode_dcmplx_ext(PLAIN plain, DCMPLX* input, size_t len, uint32_t level, uint32_t p_cnt) {
+  if (level == 0) level = (uint32_t)G.L;
+  FMT_ASSERT(level <= G.L, "level should not be larger than mul_depth + 1");
+  FMT_ASSERT(p_cnt == 0 || p_cnt == G.K, "extended plaintexts carry all P limbs");
+  POLY p = &plain->_poly;
+  if (p->_data && (p->_num_primes != level || p->_num_primes_p != p_cnt)) Free_poly_data(p);
+  if (!p->_data) Alloc_poly_data(p, G.N, level, p_cnt);
+  plain->_scaling_factor = G.sc;
+  plain->_sf_degree      = 1;
+  plain->_slots          = G.N / 2;
+  p->_is_ntt             = true;
+  ACE_OK(ace_encode(G.ctx, p->_data, (const double*)input, len, 0, level, 1, p_cnt));
+}
+/* Encode_val (ckks/src/encoder.c:473-530) into `level` host words: the residues of the scaled value */
+void Encode_single_double(int64_t* res, double input, uint32_t sc_degree, uint32_t level) {
+  NEED_CTX();
+  double scaled = input * pow(G.sc, sc_degree);
+  FMT_ASSERT(scaled <= 9223372036854775807.0 && scaled >= -9223372036854775807.0,
+             "encode %f overflow, please choose a smaller scale", input);
+  int64_t v = (int64_t)scaled;
+  for (uint32_t t = 0; t < level; ++t) {
+    int64_t q = G.q[t]._val, r = v % q;
+    res[t]    = r < 0 ? r + q : r;
+  }
+}
+void Encode_single_float(int64_t* res, float input, uint32_t sc_degree, uint32_t level) {
+  Encode_single_double(res, (double)input, sc_degree, level);
+}
+void Free_plain_poly(PLAIN plain) { Free_poly_data(&plain->_poly); }
+
+/* result shaped like c at the lower of the two levels (ckks/src/cipher.c:58-84) */
+static void shape_like(CIPHER res, CIPHER c, PLAIN plain, double sf, uint32_t deg) {
+  size_t level = Level(c), pl = plain->_poly._num_primes;
+  if (res != c) {
+    Init_poly(&res->_c0_poly, &c->_c0_poly);
+    Init_poly(&res->_c1_poly, &c->_c1_poly);
+  }
+  res->_scaling_factor  = sf;
+  res->_sf_degree       = deg;
+  res->_slots           = c->_slots;
+  res->_c0_poly._is_ntt = res->_c1_poly._is_ntt = true;
+  if (level > pl) level = pl;
+  Set_poly_level(&res->_c0_poly, level);
+  Set_poly_level(&res->_c1_poly, level);
+}
+void Init_ciph_same_scale_plain(CIPHER res, CIPHER c, PLAIN plain) {
+  shape_like(res, c, plain, c->_scaling_factor, c->_sf_degree);
+}
+void Init_ciph_up_scale_plain(CIPHER res, CIPHER c, PLAIN plain) {
+  shape_like(res, c, plain, c->_scaling_factor * plain->_scaling_factor, c->_sf_degree + plain->_sf_degree);
+}
+
+CIPHER Add_plain(CIPHER res, CIPHER c, PLAIN plain) {
+  FMT_ASSERT(c->_scaling_factor == plain->_scaling_factor, "Scaling factors are not equal.");
+  Init_ciph_same_scale_plain(res, c, plain);
+  size_t level = Level(res), n = G.N;
+  ACE_OK(ace_poly_add(G.ctx, res->_c0_poly._data, c->_c0_poly._data, plain->_poly._data, level, 0));
+  Rt_dev_copy(res->_c1_poly._data, c->_c1_poly._data, level * n);
+  return res;
+}
+CIPHER Mul_plain(CIPHER res, CIPHER c, PLAIN plain) {
+  Init_ciph_up_scale_plain(res, c, plain);
+  size_t level = Level(res);
+  ACE_OK(ace_poly_mul(G.ctx, res->_c0_poly._data, c->_c0_poly._data, plain->_poly._data, level, 0));
+  ACE_OK(ace_poly_mul(G.ctx, res->_c1_poly._data, c->_c1_poly._data, plain->_poly._data, level, 0));
+  return res;
+}
+
+/* ---- encryption / decryption (ckks/src/encryptor.c:19-75, decryptor.c) ------------------------------- */
+CIPHER Encrypt(CIPHER res, PLAIN plain) {
+  NEED_CTX();
+  if (!G.pk0) Rt_generate_keys(0);
+  POLY pt = &plain->_poly;
+  FMT_ASSERT(pt->_num_primes_p == 0, "Encrypt_msg: plain should not be extended");
+  size_t level = pt->_num_primes, n = G.N;
+  Init_poly(&res->_c0_poly, pt);
+  Init_poly(&res->_c1_poly, pt);
+  res->_scaling_factor = plain->_scaling_factor;
+  res->_sf_degree      = plain->_sf_degree;
+  res->_slots          = plain->_slots;
+  int64_t* small = (int64_t*)malloc(n * sizeof(int64_t));
+  int64_t *u = Rt_dev_alloc(level * n), *e = Rt_dev_alloc(level * n);
+  sample_triangle(small, n);
+  small_to_dev(u, small, level, false);
+  /* c0 = pk0 u + e1 + m ; c1 = pk1 u + e2 */
+  sample_triangle(small, n);
+  small_to_dev(e, small, level, false);
+  ACE_OK(ace_poly_mul(G.ctx, res->_c0_poly._data, G.pk0, u, level, 0));
+  ACE_OK(ace_poly_add(G.ctx, res->_c0_poly._data, res->_c0_poly._data, e, level, 0));
+  ACE_OK(ace_poly_add(G.ctx, res->_c0_poly._data, res->_c0_poly._data, pt->_data, level, 0));
+  sample_triangle(small, n);
+  small_to_dev(e, small, level, false);
+  ACE_OK(ace_poly_mul(G.ctx, res->_c1_poly._data, G.pk1, u, level, 0));
+  ACE_OK(ace_poly_add(G.ctx, res->_c1_poly._data, res->_c1_poly._data, e, level, 0));
+  res->_c0_poly._is_ntt = res->_c1_poly._is_ntt = true;
+  free(small);
+  Rt_dev_free(u);
+  Rt_dev_free(e);
+  return res;
+}
+
+void Rt_decrypt(PLAIN res, CIPHER c) {
+  FMT_ASSERT(G.secret_ntt, "Rt_generate_keys() has not run");
+  size_t level = Level(c);
+  init_plain(res, level, c->_scaling_factor, c->_sf_degree, c->_slots);
+  ACE_OK(ace_poly_mul(G.ctx, res->_poly._data, c->_c1_poly._data, G.secret_ntt, level, 0));
+  ACE_OK(ace_poly_add(G.ctx, res->_poly._data, res->_poly._data, c->_c0_poly._data, level, 0));
+}
+
+/* ---- decoding (ckks/src/encoder.c:657-704, util/src/crt.c:1247-1275, util/src/ntt.c:598-629) ---------- */
+typedef unsigned __int128 u128;
+static uint64_t mulmod64(uint64_t a, uint64_t b, uint64_t q) { return (uint64_t)((u128)a * b % q); }
+static uint64_t powmod64(uint64_t a, uint64_t e, uint64_t q) {
+  uint64_t r = 1;
+  for (a %= q; e; e >>= 1, a = mulmod64(a, a, q))
+    if (e & 1) r = mulmod64(r, a, q);
+  return r;
+}
+
+/* the centred integer with residues v[0..level) as a double, truncated towards zero like
+ * mpz_get_d: mixed-radix digits, exact multi-word evaluation, comparison with Q/2 */
+static double crt_to_double(const int64_t* v, size_t level, const uint64_t* inv /* [level]: (q_0..q_{i-1})^-1 mod q_i */) {
+  uint64_t d[64];
+  for (size_t i = 0; i < level; ++i) {
+    uint64_t q = (uint64_t)G.q[i]._val, acc = 0, prod = 1;
+    for (size_t j = 0; j < i; ++j) {
+      acc  = (acc + mulmod64(d[j] % q, prod, q)) % q;
+      prod = mulmod64(prod, (uint64_t)G.q[j]._val % q, q);
+    }
+    uint64_t t = ((uint64_t)v[i] % q + q - acc) % q;
+    d[i]       = i ? mulmod64(t, inv[i], q) : t;
+  }
+  uint64_t x[66] = {0}, Q[66] = {0}, x2[67] = {0};
+  size_t   nx = 1, nQ = 1;
+  Q[0]        = 1;
+  for (size_t i = level; i-- > 0;) { /* Horner from the top digit */
+    u128 carry = 0;
+    for (size_t k = 0; k < nx; ++k) {
+      u128 p = (u128)x[k] * (uint64_t)G.q[i]._val + carry;
+      x[k]   = (uint64_t)p;
+      carry  = p >> 64;
+    }
+    if (carry) x[nx++] = (uint64_t)carry;
+    u128 a = (u128)x[0] + d[i];
+    x[0]   = (uint64_t)a;
+    for (size_t k = 1; (a >> 64) && k <= nx; ++k) {
+      a    = (u128)x[k] + 1;
+      x[k] = (uint64_t)a;
+      if (k == nx) nx++;
+    }
+  }
+  for (size_t i = 0; i < level; ++i) {
+    u128 carry = 0;
+    for (size_t k = 0; k < nQ; ++k) {
+      u128 p = (u128)Q[k] * (uint64_t)G.q[i]._val + carry;
+      Q[k]   = (uint64_t)p;
+      carry  = p >> 64;
+    }
+    if (carry) Q[nQ++] = (uint64_t)carry;
+  }
+  size_t n = nQ > nx ? nQ : nx;
+  for (size_t k = 0; k < n; ++k) x2[k] = (x[k] << 1) | (k ? x[k - 1] >> 63 : 0);
+  x2[n]   = x[n - 1] >> 63;
+  int neg = x2[n] != 0;
+  if (!neg)
+    for (size_t k = n; k-- > 0;)
+      if (x2[k] != Q[k]) {
+        neg = x2[k] > Q[k];
+        break;
+      }
+  if (neg) {
+    uint64_t borrow = 0;
+    for (size_t k = 0; k < n; ++k) {
+      u128 t = (u128)Q[k] - x[k] - borrow;
+      x[k]   = (uint64_t)t;
+      borrow = (uint64_t)(t >> 64) & 1;
+    }
+  }
+  size_t top = n;
+  while (top > 0 && x[top - 1] == 0) top--;
+  if (!top) return 0.0;
+  int    hb     = 63 - __builtin_clzll(x[top - 1]);
+  size_t bitlen = (top - 1) * 64 + (size_t)hb + 1;
+  double r;
+  if (bitlen <= 53) {
+    r = (double)x[0];
+  } else {
+    size_t   sh = bitlen - 53, w = sh / 64, b = sh % 64;
+    uint64_t m  = x[w] >> b;
+    if (b && w + 1 < top) m |= x[w + 1] << (64 - b);
+    m &= ((uint64_t)1 << 53) - 1;
+    r = ldexp((double)m, (int)sh);
+  }
+  return neg ? -r : r;
+}
+
+static void need_fft_tables(void) {
+  if (G.fft_rou) return;
+  G.fft_rou   = (double*)malloc(4 * (size_t)G.N * sizeof(double));
+  G.rot_group = (uint32_t*)malloc((G.N / 2 ? G.N / 2 : 1) * sizeof(uint32_t));
+  ACE_OK(ace_host_fft_tables(G.ctx, G.fft_rou, G.rot_group));
+}
+
+/* Embedding (util/src/ntt.c:598-629) on the host */
+static void embedding(DCMPLX* res, const DCMPLX* coeffs, size_t len) {
+  need_fft_tables();
+  size_t M = 2 * (size_t)G.N, logn = 0;
+  while (((size_t)1 << logn) < len) logn++;
+  for (size_t i = 0; i < len; ++i) {
+    size_t r = 0;
+    for (size_t b = 0; b < logn; ++b) r |= ((i >> b) & 1) << (logn - 1 - b);
+    res[i] = coeffs[r];
+  }
+  for (size_t logm = 1; logm < logn + 1; ++logm) {
+    size_t idx_mod = (size_t)1 << (logm + 2), gap = M / idx_mod, num = (size_t)1 << (logm - 1);
+    for (size_t j = 0; j < len; j += (size_t)1 << logm)
+      for (size_t i = 0; i < num; ++i) {
+        size_t ie = j + i, io = ie + num, ri = ((size_t)G.rot_group[i] % idx_mod) * gap;
+        DCMPLX om = (G.fft_rou[2 * ri] + G.fft_rou[2 * ri + 1] * I) * res[io];
+        DCMPLX plus = res[ie] + om, minus = res[ie] - om;
+        res[ie] = plus;
+        res[io] = minus;
+      }
+  }
+}
+
+void Rt_decode(DCMPLX* res, PLAIN plain) {
+  POLY     p = &plain->_poly;
+  size_t   level = p->_num_primes, n = G.N, half = n / 2;
+  uint32_t slots = plain->_slots ? plain->_slots : (uint32_t)half, gap = (uint32_t)(half / slots);
+  int64_t* host = (int64_t*)malloc(level * n * sizeof(int64_t));
+  if (p->_is_ntt) { /* the plaintext itself stays as it is */
+    int32_t idx[128];
+    for (size_t t = 0; t < level; ++t) idx[t] = (int32_t)t;
+    int64_t* tmp = Rt_dev_alloc(level * n);
+    ACE_OK(ace_intt(G.ctx, tmp, p->_data, idx, level, 1, 0));
+    ACE_OK(ace_download(G.ctx, host, tmp, level * n));
+    Rt_dev_free(tmp);
+  } else {
+    ACE_OK(ace_download(G.ctx, host, p->_data, level * n));
+  }
+  uint64_t inv[64];
+  for (size_t i = 1; i < level; ++i) {
+    uint64_t q = (uint64_t)G.q[i]._val, prod = 1;
+    for (size_t j = 0; j < i; ++j) prod = mulmod64(prod, (uint64_t)G.q[j]._val % q, q);
+    inv[i] = powmod64(prod, q - 2, q);
+  }
+  DCMPLX* msg = (DCMPLX*)malloc(slots * sizeof(DCMPLX));
+  int64_t v[64];
+  for (uint32_t i = 0; i < slots; ++i) {
+    for (size_t t = 0; t < level; ++t) v[t] = host[t * n + (size_t)i * gap];
+    double re = crt_to_double(v, level, inv) / plain->_scaling_factor;
+    for (size_t t = 0; t < level; ++t) v[t] = host[t * n + (size_t)i * gap + half];
+    double im = crt_to_double(v, level, inv) / plain->_scaling_factor;
+    msg[i]    = re + im * I;
+  }
+  embedding(res, msg, slots);
+  free(msg);
+  free(host);
+}
+
+DCMPLX* Get_dcmplx_msg_from_plain(PLAIN plain) {
+  uint32_t slots = plain->_slots ? plain->_slots : G.N / 2;
+  DCMPLX*  vec   = (DCMPLX*)malloc(slots * sizeof(DCMPLX));
+  Rt_decode(vec, plain);
+  return vec;
+}
+double* Get_msg_from_plain(PLAIN plain) {
+  uint32_t slots = plain->_slots ? plain->_slots : G.N / 2;
+  DCMPLX*  vec   = Get_dcmplx_msg_from_plain(plain);
+  double*  data  = (double*)malloc(slots * sizeof(double));
+  for (uint32_t i = 0; i < slots; ++i) data[i] = creal(vec[i]);
+  free(vec);
+  return data;
+}
+
+/* ---- tensors, program inputs and outputs (common/tensor.h, ckks/src/rtlib.c:66-229) ---------------- */
+TENSOR* Alloc_tensor(size_t n, size_t c, size_t h, size_t w, const double* val) {
+  size_t  len = n * c * h * w;
+  TENSOR* t   = (TENSOR*)malloc(sizeof(TENSOR) + len * sizeof(double));
+  t->_shape   = (SHAPE){n, c, h, w};
+  if (val) memcpy(t->_vals, val, len * sizeof(double));
+  else memset(t->_vals, 0, len * sizeof(double));
+  return t;
+}
+void Free_tensor(TENSOR* t) { free(t); }
+void Print_tensor(FILE* fp, TENSOR* t) {
+  size_t len = TENSOR_SIZE(t);
+  fprintf(fp, "[%zu %zu %zu %zu] {", TENSOR_N(t), TENSOR_C(t), TENSOR_H(t), TENSOR_W(t));
+  for (size_t i = 0; i < len && i < 16; ++i) fprintf(fp, " %g", t->_vals[i]);
+  fprintf(fp, len > 16 ? " ... }\n" : " }\n");
+}
+
+static DATA_SCHEME* find_scheme(const char* name, bool input) {
+  int cnt = input ? (Get_input_count ? Get_input_count() : 0) : (Get_output_count ? Get_output_count() : 0);
+  for (int i = 0; i < cnt; ++i) {
+    DATA_SCHEME* s = input ? Get_encode_scheme(i) : Get_decode_scheme(i);
+    FMT_ASSERT(s, "invalid encode scheme");
+    if (strcmp(s->_name, name) == 0) return s;
+  }
+  Rt_fatal(__FILE__, __LINE__, "not find the %s \"%s\"", input ? "input" : "output", name);
+}
+
+void Prepare_input(TENSOR* input, const char* name) {
+  NEED_CTX();
+  DATA_SCHEME* sch = find_scheme(name, true);
+  FMT_ASSERT(sch->_count > 0, "no desc found in scheme");
+  size_t total = TENSOR_SIZE(input), hw = TENSOR_H(input) * TENSOR_W(input);
+  size_t level = G.input_level ? G.input_level : G.L;
+  for (int i = 0; i < sch->_count; ++i) {
+    const MAP_DESC* d = &sch->_desc[i];
+    size_t          len;
+    double*         v;
+    if (d->_count == 0) { /* the whole tensor in one ciphertext */
+      len = total;
+      v   = (double*)calloc(2 * len, sizeof(double));
+      for (size_t k = 0; k < len; ++k) v[2 * k] = input->_vals[k];
+    } else { /* a chunk with optional padding from its neighbours (Pre_encode_scheme) */
+      FMT_ASSERT(d->_kind == NORMAL && d->_stride == 1, "TODO: other kind / stride");
+      FMT_ASSERT((size_t)d->_count < total && (size_t)(d->_start + d->_count) <= total, "chunk out of image bound");
+      size_t loc = (size_t)d->_start, pad = (size_t)d->_pad;
+      bool   begin = loc % hw == 0, end = (loc + (size_t)d->_count) % hw == 0;
+      len = (size_t)d->_count + 2 * pad;
+      v   = (double*)calloc(2 * len, sizeof(double));
+      for (size_t k = 0; k < pad; ++k) v[2 * k] = begin ? 0 : input->_vals[loc - (pad - k)];
+      for (size_t k = 0; k < (size_t)d->_count; ++k) v[2 * (k + pad)] = input->_vals[loc + k];
+      for (size_t k = 0; k < pad; ++k) v[2 * (k + pad + (size_t)d->_count)] = end ? 0 : input->_vals[loc + (size_t)d->_count + k];
+    }
+    PLAINTEXT pt;
+    memset(&pt, 0, sizeof(pt));
+    encode_vector(&pt, v, len, 1, (uint32_t)level);
+    IO_SLOT*    s  = Rt_add_slot(&G.in, &G.n_in, name, (size_t)i);
+    CIPHERTEXT* ct = (CIPHERTEXT*)calloc(1, sizeof(CIPHERTEXT));
+    Encrypt(ct, &pt);
+    s->ct = ct;
+    Free_plain_poly(&pt);
+    free(v);
+  }
+}
+
+double* Handle_output(const char* name) {
+  NEED_CTX();
+  DATA_SCHEME* sch = find_scheme(name, false);
+  FMT_ASSERT(sch->_count > 0, "no desc found in scheme");
+  size_t len = sch->_shape._n * sch->_shape._c * sch->_shape._h * sch->_shape._w;
+  if (len == 0) len = G.N / 2;
+  double* ret = (double*)calloc(len, sizeof(double));
+  for (int i = 0; i < sch->_count; ++i) {
+    IO_SLOT* s = Rt_find_slot(G.out, G.n_out, name, (size_t)i);
+    FMT_ASSERT(s && s->ct, "not find data");
+    PLAINTEXT pt;
+    memset(&pt, 0, sizeof(pt));
+    Rt_decrypt(&pt, s->ct);
+    uint32_t slots = pt._slots ? pt._slots : G.N / 2;
+    DCMPLX*  vec   = (DCMPLX*)malloc(slots * sizeof(DCMPLX));
+    Rt_decode(vec, &pt);
+    const MAP_DESC* d = &sch->_desc[i];
+    if (d->_count == 0) {
+      for (size_t k = 0; k < len && k < slots; ++k) ret[k] = creal(vec[k]);
+    } else {
+      FMT_ASSERT(d->_kind == NORMAL && (size_t)d->_count <= len && (size_t)(d->_start + d->_count * d->_stride) <= len,
+                 "chunk out of image bound");
+      for (size_t k = 0, loc = (size_t)d->_start; k < (size_t)d->_count; ++k, loc += (size_t)d->_stride)
+        ret[loc] = creal(vec[k]);
+    }
+    free(vec);
+    Free_plain_poly(&pt);
+  }
+  return ret;
+}

@@ -8,41 +8,10 @@
 #include <stdarg.h>
 #include <time.h>
 
-#include "ace_hip.h"
 
-/* ---- state ------------------------------------------------------------------- */
-struct rt_key_parts {
-  size_t     n;
-  int64_t*   dev; /* [digit][b | a][(L+k) limbs][N] */
-  PUBLIC_KEY pk[];
-};
+#include "rt_internal.h"
 
-typedef struct {
-  int32_t    rot_idx;
-  uint32_t   auto_idx;
-  SWITCH_KEY swk;
-  int64_t*   order; /* device, NTT-form index table */
-} ROT_KEY;
-
-typedef struct {
-  char*       name;
-  size_t      idx;
-  CIPHERTEXT* ct;
-} IO_SLOT;
-
-static struct {
-  ace_ctx* ctx;
-  uint32_t N;
-  size_t   L, K, parts;
-  MODULUS *q, *p;
-  double   sc;
-  SWITCH_KEY relin;
-  ROT_KEY*   rot;
-  size_t     n_rot, cap_rot;
-  IO_SLOT *in, *out;
-  size_t   n_in, n_out;
-  struct timespec t0;
-} G;
+struct rt_state G;
 
 void Rt_fatal(const char* file, int line, const char* fmt, ...) {
   va_list ap;
@@ -55,18 +24,13 @@ void Rt_fatal(const char* file, int line, const char* fmt, ...) {
   abort();
 }
 
-#define ACE_OK(call)                                                       \
-  do {                                                                     \
-    if ((call) != 0) Rt_fatal(__FILE__, __LINE__, "%s", ace_last_error()); \
-  } while (0)
-#define NEED_CTX() FMT_ASSERT(G.ctx, "Prepare_context() has not run")
-
 /* ---- lifecycle ----------------------------------------------------------------- */
 void Prepare_context(void) {
   FMT_ASSERT(!G.ctx, "Prepare_context() called twice");
   FMT_ASSERT(Get_context_params, "the program does not define Get_context_params()");
   CKKS_PARAMS* prm = Get_context_params();
-  size_t parts = prm->_num_q_parts ? prm->_num_q_parts : 3;
+  /* Get_default_num_q_parts (util/src/std_param.c:356-363) */
+  size_t parts = prm->_num_q_parts ? prm->_num_q_parts : prm->_mul_depth > 3 ? 3 : prm->_mul_depth == 0 ? 1 : 2;
   G.ctx = ace_ctx_create(prm->_poly_degree, prm->_mul_depth + 1, prm->_first_mod_size, prm->_scaling_mod_size, parts);
   if (!G.ctx) Rt_fatal(__FILE__, __LINE__, "%s", ace_last_error());
   if (!ace_has_device(G.ctx)) Rt_fatal(__FILE__, __LINE__, "no HIP device: this runtime has no CPU path");
@@ -74,6 +38,7 @@ void Prepare_context(void) {
   G.L     = ace_num_q(G.ctx);
   G.K     = ace_num_p(G.ctx);
   G.parts = ace_num_parts(G.ctx);
+  G.input_level = prm->_input_level;
   G.sc    = ldexp(1.0, (int)prm->_scaling_mod_size);
   G.q     = (MODULUS*)aligned_alloc(16, sizeof(MODULUS) * (G.L + G.K));
   G.p     = G.q + G.L;
@@ -108,6 +73,7 @@ static void free_slots(IO_SLOT* s, size_t n) {
 
 void Finalize_context(void) {
   if (!G.ctx) return;
+  Rt_ckks_finalize();
   free_key(&G.relin);
   for (size_t i = 0; i < G.n_rot; ++i) {
     free_key(&G.rot[i].swk);
@@ -158,19 +124,19 @@ void Rt_dev_free(int64_t* p) {
 }
 void Rt_dev_copy(int64_t* dst, const int64_t* src, size_t n_words) { ACE_OK(ace_copy(G.ctx, dst, src, n_words)); }
 
-static size_t p_offset(POLY p) { return (p->_num_alloc_primes - p->_num_primes_p) * (size_t)p->_ring_degree; }
+size_t Rt_p_offset(POLY p) { return (p->_num_alloc_primes - p->_num_primes_p) * (size_t)p->_ring_degree; }
 
 void Rt_upload_poly(POLY dst, const int64_t* host) {
   size_t n = dst->_ring_degree;
   ACE_OK(ace_upload(G.ctx, dst->_data, host, dst->_num_primes * n));
   if (dst->_num_primes_p)
-    ACE_OK(ace_upload(G.ctx, dst->_data + p_offset(dst), host + dst->_num_primes * n, dst->_num_primes_p * n));
+    ACE_OK(ace_upload(G.ctx, dst->_data + Rt_p_offset(dst), host + dst->_num_primes * n, dst->_num_primes_p * n));
 }
 void Rt_download_poly(int64_t* host, POLY src) {
   size_t n = src->_ring_degree;
   ACE_OK(ace_download(G.ctx, host, src->_data, src->_num_primes * n));
   if (src->_num_primes_p)
-    ACE_OK(ace_download(G.ctx, host + src->_num_primes * n, src->_data + p_offset(src), src->_num_primes_p * n));
+    ACE_OK(ace_download(G.ctx, host + src->_num_primes * n, src->_data + Rt_p_offset(src), src->_num_primes_p * n));
 }
 
 /* ---- polynomial containers --------------------------------------------------------- */
@@ -185,6 +151,7 @@ void Free_poly_data(POLY p) {
 POLY_ARR Alloc_polys(uint32_t cnt, uint32_t degree, size_t num_q, size_t num_p) {
   FMT_ASSERT(cnt > 0, "Alloc_polys: zero array size specified");
   POLY_ARR arr  = (POLY_ARR)calloc(cnt, sizeof(POLYNOMIAL));
+  if (num_p) num_p = G.K; /* a flag in generated code, like Alloc_poly's */
   size_t   each = (num_q + num_p) * (size_t)degree;
   int64_t* slab = Rt_dev_alloc(each * cnt);
   for (uint32_t i = 0; i < cnt; ++i) {
@@ -225,7 +192,7 @@ void Copy_poly(POLY res, POLY poly) {
   FMT_ASSERT(res->_num_primes_p >= poly->_num_primes_p, "unmatched p primes cnt");
   size_t n = res->_ring_degree;
   Rt_dev_copy(res->_data, poly->_data, res->_num_primes * n);
-  if (poly->_num_primes_p) Rt_dev_copy(res->_data + p_offset(res), poly->_data + p_offset(poly), poly->_num_primes_p * n);
+  if (poly->_num_primes_p) Rt_dev_copy(res->_data + Rt_p_offset(res), poly->_data + Rt_p_offset(poly), poly->_num_primes_p * n);
   res->_is_ntt = poly->_is_ntt;
 }
 
@@ -413,7 +380,7 @@ static void transform_inplace(POLY poly, bool inverse) {
     ACE_OK(ace_ntt(G.ctx, poly->_data, poly->_data, idx, l, 1, 0));
   if (k) {
     for (size_t j = 0; j < k; ++j) idx[j] = (int32_t)(G.L + j);
-    int64_t* p = poly->_data + p_offset(poly);
+    int64_t* p = poly->_data + Rt_p_offset(poly);
     if (inverse)
       ACE_OK(ace_intt(G.ctx, p, p, idx, k, 1, 0));
     else
@@ -441,7 +408,7 @@ static POLY poly_ew(poly_ew_fn fn, const char* who, POLY res, POLY a, POLY b) {
   if (k) { /* P limbs of each operand sit at its own offset */
     FMT_ASSERT(k == G.K && res->_num_primes_p == G.K, "%s: p primes not match", who);
     for (size_t j = 0; j < k; ++j) {
-      int64_t *r = res->_data + p_offset(res) + j * n, *x = a->_data + p_offset(a) + j * n, *y = b->_data + p_offset(b) + j * n;
+      int64_t *r = res->_data + Rt_p_offset(res) + j * n, *x = a->_data + Rt_p_offset(a) + j * n, *y = b->_data + Rt_p_offset(b) + j * n;
       if (fn == ace_poly_add) ACE_OK(ace_hw_modadd(G.ctx, r, x, y, G.L + j, n));
       else if (fn == ace_poly_sub) ACE_OK(ace_hw_modsub(G.ctx, r, x, y, G.L + j, n));
       else ACE_OK(ace_hw_modmul(G.ctx, r, x, y, G.L + j, n));
@@ -498,7 +465,7 @@ void Hw_intt(int64_t* res, int64_t* a, size_t prime_idx, uint32_t degree) {
 }
 
 /* ---- keys --------------------------------------------------------------------------------- */
-static void install_key(SWITCH_KEY* k, const int64_t* host) {
+void Rt_install_key(SWITCH_KEY* k, const int64_t* host) {
   size_t T = G.L + G.K, n = G.N, words = 2 * G.parts * T * n;
   free_key(k);
   RT_KEY_PARTS* kp = (RT_KEY_PARTS*)calloc(1, sizeof(RT_KEY_PARTS) + G.parts * sizeof(PUBLIC_KEY));
@@ -514,7 +481,7 @@ static void install_key(SWITCH_KEY* k, const int64_t* host) {
   k->_public_keys = kp;
 }
 
-static ROT_KEY* find_rot(int32_t rot_idx) {
+ROT_KEY* Rt_find_rot(int32_t rot_idx) {
   for (size_t i = 0; i < G.n_rot; ++i)
     if (G.rot[i].rot_idx == rot_idx) return &G.rot[i];
   return NULL;
@@ -523,10 +490,10 @@ static ROT_KEY* find_rot(int32_t rot_idx) {
 void Rt_load_switch_key(bool is_rot, int32_t rot_idx, const int64_t* host_words) {
   NEED_CTX();
   if (!is_rot) {
-    install_key(&G.relin, host_words);
+    Rt_install_key(&G.relin, host_words);
     return;
   }
-  ROT_KEY* r = find_rot(rot_idx);
+  ROT_KEY* r = Rt_find_rot(rot_idx);
   if (!r) {
     if (G.n_rot == G.cap_rot) {
       G.cap_rot = G.cap_rot ? 2 * G.cap_rot : 16;
@@ -539,16 +506,16 @@ void Rt_load_switch_key(bool is_rot, int32_t rot_idx, const int64_t* host_words)
     r->order    = Rt_dev_alloc(G.N);
     ACE_OK(ace_automorphism_order(G.ctx, r->order, r->auto_idx, 1));
   }
-  install_key(&r->swk, host_words);
+  Rt_install_key(&r->swk, host_words);
 }
 
 uint32_t Auto_idx(int32_t rot_idx) {
-  ROT_KEY* r = find_rot(rot_idx);
+  ROT_KEY* r = Rt_find_rot(rot_idx);
   FMT_ASSERT(r, "cannot get precompute automorphism index of rotation %d", rot_idx);
   return r->auto_idx;
 }
 int64_t* Auto_order(int32_t rot_idx) {
-  ROT_KEY* r = find_rot(rot_idx);
+  ROT_KEY* r = Rt_find_rot(rot_idx);
   FMT_ASSERT(r, "cannot find precomputed automorphism order of rotation %d", rot_idx);
   return r->order;
 }
@@ -557,7 +524,7 @@ SW_KEY Swk(bool is_rot, int32_t rot_idx) {
     FMT_ASSERT(G.relin._public_keys, "no relinearisation key loaded");
     return &G.relin;
   }
-  ROT_KEY* r = find_rot(rot_idx);
+  ROT_KEY* r = Rt_find_rot(rot_idx);
   FMT_ASSERT(r, "cannot find auto key of rotation %d", rot_idx);
   return &r->swk;
 }
@@ -766,7 +733,7 @@ void Rotate_batch_ciph(CIPHER res_arr, CIPHER c, const int32_t* rot_idx, uint32_
       Copy_ciph(&res_arr[i], c);
       continue;
     }
-    ROT_KEY* r = find_rot(rot_idx[i]);
+    ROT_KEY* r = Rt_find_rot(rot_idx[i]);
     FMT_ASSERT(r, "cannot find auto key of rotation %d", rot_idx[i]);
     keys[m]   = r->swk._public_keys->dev;
     orders[m] = r->order;
@@ -797,13 +764,13 @@ CIPHER Rotate_ciph(CIPHER res, CIPHER c, int32_t rot_idx) {
 CIPHER Conjugate_ciph(CIPHER res, CIPHER c) { return Rotate_ciph(res, c, (int32_t)(2 * G.N - 1)); }
 
 /* ---- program inputs / outputs -------------------------------------------------------------------- */
-static IO_SLOT* find_slot(IO_SLOT* s, size_t n, const char* name, size_t idx) {
+IO_SLOT* Rt_find_slot(IO_SLOT* s, size_t n, const char* name, size_t idx) {
   for (size_t i = 0; i < n; ++i)
     if (s[i].idx == idx && strcmp(s[i].name, name) == 0) return &s[i];
   return NULL;
 }
-static IO_SLOT* add_slot(IO_SLOT** s, size_t* n, const char* name, size_t idx) {
-  IO_SLOT* f = find_slot(*s, *n, name, idx);
+IO_SLOT* Rt_add_slot(IO_SLOT** s, size_t* n, const char* name, size_t idx) {
+  IO_SLOT* f = Rt_find_slot(*s, *n, name, idx);
   if (f) {
     if (f->ct) {
       Free_ciph_poly(f->ct, 1);
@@ -824,7 +791,7 @@ void Rt_set_input(const char* name, size_t idx, const int64_t* c0, const int64_t
                   uint32_t sf_degree, uint32_t slots) {
   NEED_CTX();
   FMT_ASSERT(level >= 1 && level <= G.L, "Rt_set_input: level out of range");
-  IO_SLOT*    s  = add_slot(&G.in, &G.n_in, name, idx);
+  IO_SLOT*    s  = Rt_add_slot(&G.in, &G.n_in, name, idx);
   CIPHERTEXT* ct = (CIPHERTEXT*)calloc(1, sizeof(CIPHERTEXT));
   Alloc_poly_data(&ct->_c0_poly, G.N, level, 0);
   Alloc_poly_data(&ct->_c1_poly, G.N, level, 0);
@@ -838,7 +805,7 @@ void Rt_set_input(const char* name, size_t idx, const int64_t* c0, const int64_t
 }
 
 CIPHERTEXT Get_input_data(const char* name, size_t idx) {
-  IO_SLOT* s = find_slot(G.in, G.n_in, name, idx);
+  IO_SLOT* s = Rt_find_slot(G.in, G.n_in, name, idx);
   FMT_ASSERT(s && s->ct, "not find data: input \"%s\"[%zu]", name, idx);
   CIPHERTEXT ret = *s->ct; /* ownership of the polynomials moves to the program */
   free(s->ct);
@@ -847,7 +814,7 @@ CIPHERTEXT Get_input_data(const char* name, size_t idx) {
 }
 
 void Set_output_data(const char* name, size_t idx, CIPHER data) {
-  IO_SLOT*    s  = add_slot(&G.out, &G.n_out, name, idx);
+  IO_SLOT*    s  = Rt_add_slot(&G.out, &G.n_out, name, idx);
   CIPHERTEXT* ct = (CIPHERTEXT*)calloc(1, sizeof(CIPHERTEXT));
   Copy_ciph(ct, data);
   Free_ciph_poly(data, 1);
@@ -855,7 +822,7 @@ void Set_output_data(const char* name, size_t idx, CIPHER data) {
 }
 
 size_t Rt_get_output(const char* name, size_t idx, int64_t* c0, int64_t* c1, CIPHERTEXT* meta) {
-  IO_SLOT* s = find_slot(G.out, G.n_out, name, idx);
+  IO_SLOT* s = Rt_find_slot(G.out, G.n_out, name, idx);
   if (!s || !s->ct) return 0;
   if (c0) Rt_download_poly(c0, &s->ct->_c0_poly);
   if (c1) Rt_download_poly(c1, &s->ct->_c1_poly);

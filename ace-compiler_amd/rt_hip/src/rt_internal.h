@@ -1,0 +1,63 @@
+/* rt_internal.h -- state shared by the files of the host-side runtime (not installed) */
+#ifndef RT_INTERNAL_H
+#define RT_INTERNAL_H
+
+#include <time.h>
+
+#include "ace_hip.h"
+#include "rt_hip.h"
+
+struct rt_key_parts {
+  size_t     n;
+  int64_t*   dev; /* [digit][b | a][(L+k) limbs][N] */
+  PUBLIC_KEY pk[];
+};
+
+typedef struct {
+  int32_t    rot_idx;
+  uint32_t   auto_idx;
+  SWITCH_KEY swk;
+  int64_t*   order; /* device, NTT-form index table */
+} ROT_KEY;
+
+typedef struct {
+  char*       name;
+  size_t      idx;
+  CIPHERTEXT* ct;
+} IO_SLOT;
+
+struct rt_state {
+  ace_ctx* ctx;
+  uint32_t N;
+  size_t   L, K, parts, input_level;
+  MODULUS *q, *p;
+  double   sc;
+  SWITCH_KEY relin;
+  ROT_KEY*   rot;
+  size_t     n_rot, cap_rot;
+  IO_SLOT *in, *out;
+  size_t   n_in, n_out;
+  struct timespec t0;
+  /* key material of Rt_generate_keys (rt_ckks.c); absent when the harness loads keys itself */
+  int64_t* secret_small; /* host: N signed coefficients */
+  int64_t* secret_ntt;   /* device: (L+k) limbs */
+  int64_t *pk0, *pk1;    /* device: L limbs each */
+  double*   fft_rou;     /* host: 2N (cos, sin) pairs */
+  uint32_t* rot_group;   /* host: N/2 powers of 5 */
+};
+extern struct rt_state G;
+
+#define ACE_OK(call)                                                       \
+  do {                                                                     \
+    if ((call) != 0) Rt_fatal(__FILE__, __LINE__, "%s", ace_last_error()); \
+  } while (0)
+#define NEED_CTX() FMT_ASSERT(G.ctx, "Prepare_context() has not run")
+
+size_t   Rt_p_offset(POLY p);
+IO_SLOT* Rt_find_slot(IO_SLOT* s, size_t n, const char* name, size_t idx);
+IO_SLOT* Rt_add_slot(IO_SLOT** s, size_t* n, const char* name, size_t idx);
+void     Rt_install_key(SWITCH_KEY* k, const int64_t* host);
+ROT_KEY* Rt_find_rot(int32_t rot_idx);
+void     Rt_ckks_finalize(void);
+
+#endif

@@ -25,7 +25,11 @@ def test_library_exports():
                  "Init_ciph_same_scale_ciph3 Init_ciph3_up_scale Copy_ciph Free_ciph_poly Zero_ciph Add_ciph Sub_ciph "
                  "Mul_ciph3 Relin Mul_ciph Rescale_ciph Modswitch_ciph Rotate_ciph Rotate_batch_ciph Conjugate_ciph "
                  "Get_input_data Set_output_data Tm_start Tm_taken Rt_load_switch_key Rt_set_input "
-                 "Rt_get_output").split():
+                 "Rt_get_output Rt_generate_keys Rt_generate_rotation_key Encrypt Rt_decrypt Rt_decode Prepare_input "
+                 "Handle_output Encode_float Encode_double Encode_dcmplx Encode_dcmplx_ext Encode_float_mask "
+                 "Encode_double_mask Encode_single_float Encode_single_double Get_msg_from_plain "
+                 "Get_dcmplx_msg_from_plain Free_plain_poly Init_ciph_same_scale_plain Init_ciph_up_scale_plain "
+                 "Add_plain Mul_plain Alloc_tensor Free_tensor Print_tensor").split():
         assert hasattr(lib, name), name
 
 
