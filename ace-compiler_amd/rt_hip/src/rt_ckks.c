@@ -231,32 +231,54 @@ static void check_sf(uint32_t sf_degree, size_t level) {
              "invalid scaling factor for encode");
 }
 
-/* Encode_val_at_level (ckks/src/encoder.c:473-575): the same residue in every coefficient */
-static void encode_value(PLAIN plain, double value, uint32_t sc_degree, uint32_t level) {
+/* Encode_val (ckks/src/encoder.c:428-523): the residues of trunc(value * scale).  A product beyond
+ * 61 bits is encoded divided by a power of two, which is multiplied back in modulo each prime. */
+static void encode_val_words(int64_t* res, double value, uint32_t level, double scale) {
   CKKS_PARAMS* prm = Get_context_params();
+  FMT_ASSERT(level > 0 && level <= G.L, "level should not be larger than q_cnt");
+  size_t bits = prm->_first_mod_size + (level - 1) * prm->_scaling_mod_size;
+  FMT_ASSERT(scale > 0 && (uint32_t)log2(scale) < bits, "invalid scale for encode");
+  if (value == 0.0) {
+    memset(res, 0, level * sizeof(int64_t));
+    return;
+  }
+  int32_t log_scale  = (int32_t)(log2(fabs(value * scale)));
+  int32_t log_valid  = log_scale <= 61 ? log_scale : 61;
+  int32_t log_approx = log_scale - log_valid;
+  double  scaled     = value / pow(2, log_approx) * scale;
+  FMT_ASSERT(scaled <= 9223372036854775807.0 && scaled >= -9223372036854775807.0,
+             "encode %f with scale %f overflow, please choose a smaller scale", value, scale);
+  FMT_ASSERT(log_scale + 1 < (int32_t)bits,
+             "encode value out of range, please increase encoding level or increase first_mod_size & "
+             "scale_mod_size or decrease scale of msg");
+  int64_t v = (int64_t)scaled;
+  for (uint32_t t = 0; t < level; ++t) {
+    uint64_t q = (uint64_t)G.q[t]._val;
+    int64_t  r = v % (int64_t)q;
+    if (r < 0) r += (int64_t)q;
+    uint64_t back = 1; /* 2^log_approx mod q, in steps of at most 60 bits */
+    for (int32_t left = log_approx; left > 0;) {
+      int32_t step = left <= 60 ? left : 60;
+      back         = (uint64_t)((unsigned __int128)back * (((uint64_t)1 << step) % q) % q);
+      left -= step;
+    }
+    res[t] = (int64_t)((unsigned __int128)(uint64_t)r * back % q);
+  }
+}
+
+/* Encode_val_at_level (encoder.c:544-575): the same residue in every coefficient */
+static void encode_value(PLAIN plain, double value, uint32_t sc_degree, uint32_t level) {
   if (level == 0) level = (uint32_t)G.L;
   FMT_ASSERT(level <= G.L, "level should not be larger than mul_depth + 1");
   check_sf(sc_degree, level);
   double scale = pow(G.sc, sc_degree);
   init_plain(plain, level, scale, sc_degree, G.N / 2);
-  int32_t log_scale = (int32_t)(log2(fabs(value * scale)));
-  FMT_ASSERT(log_scale <= 61, "encode %f: values that need the approximation factor are not supported", value);
-  double scaled = value * scale; /* approximation factor 2^0 */
-  FMT_ASSERT(scaled <= 9223372036854775807.0 && scaled >= -9223372036854775807.0,
-             "encode %f with scale %f overflow, please choose a smaller scale", value, scale);
-  FMT_ASSERT(log_scale + 1 < (int32_t)prm->_first_mod_size + (int32_t)(level - 1) * (int32_t)prm->_scaling_mod_size,
-             "encode value out of range, please increase encoding level or increase first_mod_size & "
-             "scale_mod_size or decrease scale of msg");
-  int64_t v = (int64_t)scaled;
-  int64_t zero_one[2];
+  int64_t words[128];
+  encode_val_words(words, value, level, scale);
   for (uint32_t t = 0; t < level; ++t) {
-    int64_t q = G.q[t]._val, r = v % q;
-    if (r < 0) r += q;
-    /* limb t = the constant r: zero it, then add r to every word */
-    zero_one[0] = r;
-    ACE_OK(ace_zero(G.ctx, plain->_poly._data + (size_t)t * G.N, G.N));
-    ACE_OK(ace_hw_modadd_scalar(G.ctx, plain->_poly._data + (size_t)t * G.N, plain->_poly._data + (size_t)t * G.N,
-                                zero_one[0], t, G.N));
+    int64_t* limb = plain->_poly._data + (size_t)t * G.N;
+    ACE_OK(ace_zero(G.ctx, limb, G.N));
+    ACE_OK(ace_hw_modadd_scalar(G.ctx, limb, limb, words[t], t, G.N));
   }
 }
 
@@ -312,17 +334,10 @@ void Encode_dcmplx_ext(PLAIN plain, DCMPLX* input, size_t len, uint32_t level, u
   p->_is_ntt             = true;
   ACE_OK(ace_encode(G.ctx, p->_data, (const double*)input, len, 0, level, 1, p_cnt));
 }
-/* Encode_val (ckks/src/encoder.c:473-530) into `level` host words: the residues of the scaled value */
+/* Encode_single_double (ckks/src/plain.c:139-147): `level` host words */
 void Encode_single_double(int64_t* res, double input, uint32_t sc_degree, uint32_t level) {
   NEED_CTX();
-  double scaled = input * pow(G.sc, sc_degree);
-  FMT_ASSERT(scaled <= 9223372036854775807.0 && scaled >= -9223372036854775807.0,
-             "encode %f overflow, please choose a smaller scale", input);
-  int64_t v = (int64_t)scaled;
-  for (uint32_t t = 0; t < level; ++t) {
-    int64_t q = G.q[t]._val, r = v % q;
-    res[t]    = r < 0 ? r + q : r;
-  }
+  encode_val_words(res, input, level, pow(G.sc, sc_degree));
 }
 void Encode_single_float(int64_t* res, float input, uint32_t sc_degree, uint32_t level) {
   Encode_single_double(res, (double)input, sc_degree, level);

@@ -10,6 +10,7 @@ graph, decryption and decoding (needs an MI355X).
 """
 import os
 import subprocess
+from fractions import Fraction
 
 import pytest
 
@@ -44,3 +45,52 @@ def test_reference_example(name):
         pytest.skip("built only where the reference tree is present")
     r = run([exe], 77)
     assert r.returncode == 0 and "SUCESS" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
+
+
+CODEC = os.path.join(rt_program.ROOT, "tests", "programs", "codec_program")
+
+
+@pytest.mark.parametrize("cfg,level,sf_degree,n_values",
+                         [((64, 4, 45, 40, 2), 4, 1, 32), ((4096, 4, 60, 50, 2), 3, 2, 100),
+                          ((65536, 6, 50, 50, 3), 6, 1, 32768)],
+                         ids=["N64", "N4096_sf2", "N65536"])
+def test_plaintext_codec_matches_the_oracle(cfg, level, sf_degree, n_values, tmp_path):
+    """Encode_dcmplx, the one-value form of Encode_double and Get_dcmplx_msg_from_plain, bit for bit."""
+    import numpy as np
+
+    from oracle_lib import Oracle
+
+    assert os.path.exists(CODEC), "tests/programs/codec_program is not built"
+    N, L, q0, sf, parts = cfg
+    rng = np.random.Generator(np.random.PCG64(900 + N))
+    values = (rng.uniform(-1, 1, n_values) + 1j * rng.uniform(-1, 1, n_values)).astype(np.complex128)
+    head = np.array([N, L - 1, q0, sf, parts, level, sf_degree, n_values], np.int64)
+    in_path, out_path = str(tmp_path / "in.bin"), str(tmp_path / "out.bin")
+    with open(in_path, "wb") as f:
+        f.write(head.tobytes() + values.tobytes())
+    r = run([CODEC, in_path, out_path], 0)
+    assert r.returncode == 0, r.stdout + r.stderr
+    raw = open(out_path, "rb").read()
+    words = level * N
+    enc = np.frombuffer(raw, np.int64, words)
+    dec = np.frombuffer(raw, np.complex128, N // 2, offset=8 * words)
+    one = np.frombuffer(raw, np.int64, words, offset=8 * words + 16 * (N // 2))
+    o = Oracle(*cfg)
+    want = o.encode(values, 0, level, sf_degree)
+    assert want is not None and np.array_equal(enc, want)
+    want_dec = o.decode(want, level, N // 2, float(2.0 ** (sf * sf_degree)))
+    assert np.array_equal(dec.view(np.float64), want_dec.view(np.float64))
+    assert np.abs(dec[:n_values] - values).max() < 1e-7
+    # Encode_val_at_level: a constant polynomial (constant in NTT form too) whose residues recombine to the
+    # scaled value, truncated to 61 significant bits when it is larger than that
+    primes = [int(q) for q in o.primes[:level]]
+    o.close()
+    res = one.reshape(level, N)
+    assert (res == res[:, :1]).all()
+    Q = 1
+    for q in primes:
+        Q *= q
+    x = sum(int(res[t, 0]) * (Q // q) * pow(Q // q, -1, q) for t, q in enumerate(primes)) % Q
+    x = x - Q if x > Q // 2 else x
+    exact = Fraction(float(values[0].real)) * 2 ** (sf * sf_degree)
+    assert abs(x - exact) <= max(1, abs(exact) / 2 ** 60)
