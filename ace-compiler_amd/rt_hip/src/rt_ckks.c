@@ -233,7 +233,7 @@ static void check_sf(uint32_t sf_degree, size_t level) {
 
 /* Encode_val (ckks/src/encoder.c:428-523): the residues of trunc(value * scale).  A product beyond
  * 61 bits is encoded divided by a power of two, which is multiplied back in modulo each prime. */
-static void encode_val_words(int64_t* res, double value, uint32_t level, double scale) {
+void Rt_encode_val_words(int64_t* res, double value, uint32_t level, double scale) {
   CKKS_PARAMS* prm = Get_context_params();
   FMT_ASSERT(level > 0 && level <= G.L, "level should not be larger than q_cnt");
   size_t bits = prm->_first_mod_size + (level - 1) * prm->_scaling_mod_size;
@@ -274,7 +274,7 @@ static void encode_value(PLAIN plain, double value, uint32_t sc_degree, uint32_t
   double scale = pow(G.sc, sc_degree);
   init_plain(plain, level, scale, sc_degree, G.N / 2);
   int64_t words[128];
-  encode_val_words(words, value, level, scale);
+  Rt_encode_val_words(words, value, level, scale);
   for (uint32_t t = 0; t < level; ++t) {
     int64_t* limb = plain->_poly._data + (size_t)t * G.N;
     ACE_OK(ace_zero(G.ctx, limb, G.N));
@@ -337,7 +337,7 @@ void Encode_dcmplx_ext(PLAIN plain, DCMPLX* input, size_t len, uint32_t level, u
 /* Encode_single_double (ckks/src/plain.c:139-147): `level` host words */
 void Encode_single_double(int64_t* res, double input, uint32_t sc_degree, uint32_t level) {
   NEED_CTX();
-  encode_val_words(res, input, level, pow(G.sc, sc_degree));
+  Rt_encode_val_words(res, input, level, pow(G.sc, sc_degree));
 }
 void Encode_single_float(int64_t* res, float input, uint32_t sc_degree, uint32_t level) {
   Encode_single_double(res, (double)input, sc_degree, level);

@@ -73,6 +73,7 @@ static void free_slots(IO_SLOT* s, size_t n) {
 
 void Finalize_context(void) {
   if (!G.ctx) return;
+  Rt_bootstrap_finalize();
   Rt_ckks_finalize();
   free_key(&G.relin);
   for (size_t i = 0; i < G.n_rot; ++i) {

@@ -59,5 +59,8 @@ IO_SLOT* Rt_add_slot(IO_SLOT** s, size_t* n, const char* name, size_t idx);
 void     Rt_install_key(SWITCH_KEY* k, const int64_t* host);
 ROT_KEY* Rt_find_rot(int32_t rot_idx);
 void     Rt_ckks_finalize(void);
+void     Rt_bootstrap_finalize(void);
+/* Encode_val: `level` residues of trunc(value * scale), large products through the approximation factor */
+void     Rt_encode_val_words(int64_t* res, double value, uint32_t level, double scale);
 
 #endif

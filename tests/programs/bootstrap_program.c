@@ -1,0 +1,88 @@
+/* Bootstrapping on the HIP-backed runtime: a vector is encrypted at level 1, refreshed with Bootstrap(),
+ * squared once at the refreshed level (so the new levels are really usable), decrypted and compared
+ * (reference flow: rtlib/ant/example/eg_fhertlib_bootstrap.inc, ckks/src/cipher.c:565-583).
+ *
+ * usage: bootstrap_program <poly degree> <mul depth> <q0 bits> <scale bits> <hamming weight> <slots>
+ *                          <level after bootstrap, 0 = highest> <seed>
+ * prints "max_err <e> level <l> ms <t>"; exit status 0 when max_err < 1e-3 and the level is the one asked for.
+ */
+#include <math.h>
+#include <time.h>
+
+#include "rt_ant/rt_ant.h"
+
+static CKKS_PARAMS Params = {._provider = LIB_ANT};
+CKKS_PARAMS*       Get_context_params(void) { return &Params; }
+
+static double Unit(uint64_t* state) { /* in [-1, 1) */
+  *state = *state * 6364136223846793005ull + 1442695040888963407ull;
+  return (double)(int64_t)(*state >> 11) / (double)(1ull << 52) - 1.0;
+}
+static double Now_ms(void) {
+  struct timespec t;
+  clock_gettime(CLOCK_MONOTONIC, &t);
+  return t.tv_sec * 1e3 + t.tv_nsec * 1e-6;
+}
+
+int main(int argc, char** argv) {
+  if (argc != 9) {
+    fprintf(stderr, "usage: %s <degree> <depth> <q0 bits> <scale bits> <hamming weight> <slots> <level after> <seed>\n", argv[0]);
+    return 2;
+  }
+  Params._poly_degree      = (uint32_t)strtoul(argv[1], NULL, 0);
+  Params._mul_depth        = strtoul(argv[2], NULL, 0);
+  Params._first_mod_size   = strtoul(argv[3], NULL, 0);
+  Params._scaling_mod_size = strtoul(argv[4], NULL, 0);
+  Params._hamming_weight   = strtoul(argv[5], NULL, 0);
+  uint32_t slots           = (uint32_t)strtoul(argv[6], NULL, 0);
+  uint32_t level_after     = (uint32_t)strtoul(argv[7], NULL, 0);
+  uint64_t seed            = strtoull(argv[8], NULL, 0);
+
+  Prepare_context();
+  Rt_generate_keys(seed);
+  uint64_t st = seed * 77 + 1;
+  double*  x  = (double*)malloc(slots * sizeof(double));
+  for (uint32_t i = 0; i < slots; ++i) x[i] = Unit(&st);
+
+  PLAINTEXT  pt;
+  CIPHERTEXT ct, fresh, sq;
+  memset(&pt, 0, sizeof(pt));
+  memset(&ct, 0, sizeof(ct));
+  memset(&fresh, 0, sizeof(fresh));
+  memset(&sq, 0, sizeof(sq));
+  /* a sparsely packed message is the same polynomial as its copies filling every slot */
+  uint32_t all   = Degree() / 2;
+  double*  tiled = (double*)malloc(all * sizeof(double));
+  for (uint32_t i = 0; i < all; ++i) tiled[i] = x[i % slots];
+  Encode_double(&pt, tiled, all, 1, 1);
+  free(tiled);
+  Encrypt(&ct, &pt);
+  Set_slots(&ct, slots);
+
+  double t0 = Now_ms();
+  Eval_bootstrap_ciph(&fresh, &ct, level_after, slots);
+  PLAINTEXT back;
+  memset(&back, 0, sizeof(back));
+  Rt_decrypt(&back, &fresh); /* also the synchronisation point of the timing */
+  double   t1    = Now_ms();
+  uint32_t level = Level(&fresh);
+
+  Mul_ciph(&sq, &fresh, &fresh);
+  Rescale_ciph(&sq, &sq);
+  PLAINTEXT back2;
+  memset(&back2, 0, sizeof(back2));
+  Rt_decrypt(&back2, &sq);
+  double* y  = Get_msg_from_plain(&back);
+  double* y2 = Get_msg_from_plain(&back2);
+  double  max_err = 0, max_sq = 0;
+  for (uint32_t i = 0; i < slots; ++i) {
+    max_err = fmax(max_err, fabs(y[i] - x[i]));
+    max_sq  = fmax(max_sq, fabs(y2[i] - x[i] * x[i]));
+  }
+  printf("max_err %.3e square_err %.3e level %u ms %.1f\n", max_err, max_sq, level, t1 - t0);
+  free(y);
+  free(y2);
+  free(x);
+  Finalize_context();
+  return (max_err < 1e-3 && max_sq < 2e-3 && (level_after == 0 || level == level_after)) ? 0 : 1;
+}

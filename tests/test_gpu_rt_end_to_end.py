@@ -20,8 +20,8 @@ pytestmark = pytest.mark.gpu
 
 GEMM = os.path.join(rt_program.ROOT, "tests", "programs", "gemm_program")
 EXAMPLES_DIR = os.path.join(rt_program.ROOT, "oracle", "_ref", "examples")
-EXAMPLES = ["add", "add_const", "avg_pool", "conv2d", "gemm", "gemm_02", "mul_const", "relin", "relin_02", "rotate",
-            "rotate_02"]
+EXAMPLES = ["add", "add_const", "avg_pool", "bootstrap", "bootstrap_02", "conv2d", "gemm", "gemm_02", "mul_const", "relin",
+            "relin_02", "relu", "rotate", "rotate_02"]
 
 
 def run(cmd, seed):
@@ -94,3 +94,24 @@ def test_plaintext_codec_matches_the_oracle(cfg, level, sf_degree, n_values, tmp
     x = x - Q if x > Q // 2 else x
     exact = Fraction(float(values[0].real)) * 2 ** (sf * sf_degree)
     assert abs(x - exact) <= max(1, abs(exact) / 2 ** 60)
+
+
+BOOTSTRAP = os.path.join(rt_program.ROOT, "tests", "programs", "bootstrap_program")
+
+
+@pytest.mark.parametrize("args,env", [
+    ("16 25 60 51 0 8 0 1", {}),               # the reference example's ring, fully packed
+    ("256 25 60 51 0 128 0 2", {}),            # uniform ternary secret: K = 512, six double-angle steps
+    ("256 25 60 51 0 16 5 3", {}),             # sparsely packed, to a requested level
+    ("1024 20 60 51 64 512 0 4", {}),          # Hamming weight <= 192: K = 32, three double-angle steps
+    ("1024 20 60 51 64 512 0 5", {"RTLIB_BTS_EVEN_POLY": "1"}),   # the even series
+    ("256 25 60 51 0 128 0 6", {"RT_BTS_CLEAR_IMAG": "1"}),       # imaginary parts cleared by conjugation
+    ("16384 23 60 56 192 8192 0 7", {}),       # the reference's bootstrap_full parameters
+], ids=["N16", "N256", "N256_sparse", "N1024_hw64", "N1024_even", "N256_clear_imag", "N16384"])
+def test_bootstrap_refreshes_levels(args, env):
+    """Encrypt at level 1, bootstrap, check the message (1e-3), the level, and one multiplication at the new level."""
+    assert os.path.exists(BOOTSTRAP), "tests/programs/bootstrap_program is not built"
+    e = dict(os.environ, **env)
+    print("running bootstrap_program", args, env, flush=True)
+    r = subprocess.run([BOOTSTRAP] + args.split(), capture_output=True, text=True, timeout=110, env=e)
+    assert r.returncode == 0, r.stdout + r.stderr
