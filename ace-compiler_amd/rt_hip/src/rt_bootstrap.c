@@ -30,18 +30,13 @@ typedef struct {
 } SIN_POLY;
 static SIN_POLY Sin_poly;
 
-static const SIN_POLY* sin_poly(void) {
-  if (Sin_poly.n_coeff) return &Sin_poly;
-  CKKS_PARAMS* prm  = Get_context_params();
-  const char*  env  = getenv("RTLIB_BTS_EVEN_POLY");
-  bool         even = env && atoi(env) != 0;
-  bool         low  = prm->_hamming_weight > 0 && prm->_hamming_weight <= 192;
-  SIN_POLY*    p    = &Sin_poly;
-  p->even           = even;
-  p->k_bound        = low ? 32 : 512;
-  p->double_angle   = low ? 3 : (even ? 7 : 6);
-  p->n_coeff        = (low || even) ? 55 : 89;
-  uint32_t nodes    = 4 * p->n_coeff;
+static void fill_sin_poly(SIN_POLY* p, size_t hamming_weight, bool even) {
+  bool low        = hamming_weight > 0 && hamming_weight <= 192;
+  p->even         = even;
+  p->k_bound      = low ? 32 : 512;
+  p->double_angle = low ? 3 : (even ? 7 : 6);
+  p->n_coeff      = (low || even) ? 55 : 89;
+  uint32_t nodes  = 4 * p->n_coeff;
   double   pw = pow(2.0, p->double_angle), amp = pow(2.0 * M_PI, -1.0 / pw), shift = even ? 0.0 : M_PI / 2;
   for (uint32_t k = 0; k < p->n_coeff; ++k) {
     double acc = 0;
@@ -51,7 +46,21 @@ static const SIN_POLY* sin_poly(void) {
     }
     p->coeff[k] = (even && (k & 1)) ? 0.0 : 2.0 * acc / nodes;
   }
-  return p;
+}
+static const SIN_POLY* sin_poly(void) {
+  if (Sin_poly.n_coeff) return &Sin_poly;
+  const char* env = getenv("RTLIB_BTS_EVEN_POLY");
+  fill_sin_poly(&Sin_poly, Get_context_params()->_hamming_weight, env && atoi(env) != 0);
+  return &Sin_poly;
+}
+/* for inspection without a context: the series of a Hamming weight; returns the number of coefficients */
+size_t Rt_sin_series(size_t hamming_weight, int even, double* coeff, uint32_t* k_bound, uint32_t* double_angle) {
+  SIN_POLY p;
+  fill_sin_poly(&p, hamming_weight, even != 0);
+  memcpy(coeff, p.coeff, p.n_coeff * sizeof(double));
+  *k_bound      = p.k_bound;
+  *double_angle = p.double_angle;
+  return p.n_coeff;
 }
 
 /* multiplicative depth of a Chebyshev series by degree (bootstrap.c:64-80), normalised input */
@@ -622,7 +631,7 @@ static void series_divide(SERIES* q, SERIES* r, const SERIES* f, const SERIES* g
   gt[0] /= 2;
   for (;;) {
     uint32_t d = n - k;
-    double   c = (d ? 2.0 : 1.0) * r->v[n] / gt[k];
+    double   c = ((d && k) ? 2.0 : 1.0) * r->v[n] / gt[k];
     q->v[d]    = c;
     for (uint32_t i = 0; i <= k; ++i) {
       if (d == 0) {
@@ -641,6 +650,18 @@ static void series_divide(SERIES* q, SERIES* r, const SERIES* f, const SERIES* g
   q->v[0] *= 2;
   r->v[0] *= 2;
   free(gt);
+}
+
+/* for inspection: f / g with n_f and n_g coefficients; q and r must hold n_f entries; returns the lengths */
+void Rt_series_divide(double* q, size_t* n_q, double* r, size_t* n_r, const double* f, size_t n_f, const double* g, size_t n_g) {
+  SERIES sf = {(double*)f, n_f}, sg = {(double*)g, n_g}, sq, sr;
+  series_divide(&sq, &sr, &sf, &sg);
+  memcpy(q, sq.v, sq.n * sizeof(double));
+  memcpy(r, sr.v, sr.n * sizeof(double));
+  *n_q = sq.n;
+  *n_r = sr.n;
+  free(sq.v);
+  free(sr.v);
 }
 
 /* k and m of the evaluation: degree < k (2^m - 1), depth ceil(log2 k) + m minimal (chebyshev_impl.c:71-141) */

@@ -60,6 +60,8 @@ void     Rt_install_key(SWITCH_KEY* k, const int64_t* host);
 ROT_KEY* Rt_find_rot(int32_t rot_idx);
 void     Rt_ckks_finalize(void);
 void     Rt_bootstrap_finalize(void);
+size_t   Rt_sin_series(size_t hamming_weight, int even, double* coeff, uint32_t* k_bound, uint32_t* double_angle);
+void     Rt_series_divide(double* q, size_t* n_q, double* r, size_t* n_r, const double* f, size_t n_f, const double* g, size_t n_g);
 /* Encode_val: `level` residues of trunc(value * scale), large products through the approximation factor */
 void     Rt_encode_val_words(int64_t* res, double value, uint32_t level, double scale);
 

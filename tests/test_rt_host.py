@@ -29,7 +29,7 @@ def test_library_exports():
                  "Handle_output Encode_float Encode_double Encode_dcmplx Encode_dcmplx_ext Encode_float_mask "
                  "Encode_double_mask Encode_single_float Encode_single_double Get_msg_from_plain "
                  "Get_dcmplx_msg_from_plain Free_plain_poly Init_ciph_same_scale_plain Init_ciph_up_scale_plain "
-                 "Add_plain Mul_plain Alloc_tensor Free_tensor Print_tensor").split():
+                 "Add_plain Mul_plain Alloc_tensor Free_tensor Print_tensor Bootstrap Eval_bootstrap_ciph Mul_mono_ciph").split():
         assert hasattr(lib, name), name
 
 
