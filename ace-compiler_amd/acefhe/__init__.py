@@ -90,11 +90,12 @@ def _sig(lib):
     f("ace_mul_relin_rescale_batch", C.c_int, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _sz, _vp, _sz, _sz)
     f("ace_fast_rotate", C.c_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz)
     f("ace_rotate_batch", C.c_int, _vp, _vp, _vp, _vp, _vp, C.POINTER(_vp), C.POINTER(_vp), _sz, _sz)
+    f("ace_ext_plain_mac", C.c_int, _vp, _vp, _vp, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), _sz, _sz, _sz, C.c_int)
 
 
 # every symbol include/ace_hip.h declares
 EXPORTS = [
-    "ace_ctx_create", "ace_ctx_create_with_primes", "ace_ctx_destroy", "ace_has_device", "ace_last_error",
+    "ace_ext_plain_mac", "ace_ctx_create", "ace_ctx_create_with_primes", "ace_ctx_destroy", "ace_has_device", "ace_last_error",
     "ace_degree", "ace_num_q", "ace_num_p", "ace_num_parts", "ace_part_size", "ace_num_decomp", "ace_prime",
     "ace_root", "ace_modulus", "ace_host_twiddles", "ace_host_tbl_modup", "ace_host_tbl_moddown",
     "ace_host_tbl_rescale", "ace_host_automorphism_order", "ace_alloc", "ace_free", "ace_upload", "ace_download",
@@ -360,6 +361,14 @@ class Context:
 
     def fast_rotate(self, r0, r1, c0, digits, swk, order, level):
         self._chk(self.lib.ace_fast_rotate(self.h, r0.ptr, r1.ptr, c0.ptr, digits.ptr, swk.ptr, order.ptr, level))
+
+    def ext_plain_mac(self, r0, r1, a0s, a1s, plains, level, plain_level, accumulate=False):
+        n = len(plains)
+        p0 = (_vp * n)(*[a.ptr for a in a0s])
+        p1 = (_vp * n)(*[a.ptr for a in a1s])
+        pp = (_vp * n)(*[a.ptr for a in plains])
+        self._chk(self.lib.ace_ext_plain_mac(self.h, r0.ptr, r1.ptr, p0, p1, pp, C.c_size_t(n), C.c_size_t(level),
+                                             C.c_size_t(plain_level), C.c_int(int(accumulate))))
 
     def rotate_batch(self, r0s, r1s, c0, c1, swks, orders, level):
         n = len(swks)

@@ -960,6 +960,32 @@ int ace_poly_add(ace_ctx* c, int64_t* r, const int64_t* a, const int64_t* b, siz
 int ace_poly_sub(ace_ctx* c, int64_t* r, const int64_t* a, const int64_t* b, size_t level, int with_p) { return poly_ew(c, EW_SUB, r, a, b, level, with_p); }
 int ace_poly_mul(ace_ctx* c, int64_t* r, const int64_t* a, const int64_t* b, size_t level, int with_p) { return poly_ew(c, EW_MUL, r, a, b, level, with_p); }
 
+int ace_ext_plain_mac(ace_ctx* c, int64_t* r0, int64_t* r1, const int64_t* const* a0, const int64_t* const* a1,
+                      const int64_t* const* plain, size_t count, size_t level, size_t plain_level, int accumulate) {
+  ACE_TRY
+  if (!r0 || !r1 || !a0 || !a1 || !plain) return fail("ace_ext_plain_mac: null argument");
+  if (!level_ok(c, level) || !level_ok(c, plain_level) || plain_level < level)
+    return fail("ace_ext_plain_mac: levels out of range (the plaintext may not sit below the ciphertext)");
+  if (!count) return fail("ace_ext_plain_mac: no operands");
+  for (size_t j = 0; j < count; ++j) {
+    if (!a0[j] || !a1[j] || !plain[j]) return fail("ace_ext_plain_mac: null operand");
+    if (a0[j] == r0 || a1[j] == r1 || a0[j] == r1 || a1[j] == r0) return fail("ace_ext_plain_mac: an operand aliases the result");
+  }
+  LimbMap lm = poly_lm(c, level, true);
+  for (size_t done = 0; done < count; done += kMaxMacOps) {
+    MacSet ops{};
+    ops.n = (u32)std::min<size_t>(kMaxMacOps, count - done);
+    for (u32 j = 0; j < ops.n; ++j) {
+      ops.a0[j] = U(a0[done + j]);
+      ops.a1[j] = U(a1[done + j]);
+      ops.p[j]  = U(plain[done + j]);
+    }
+    launch_plain_mac(c->stream, c->d, U(r0), U(r1), ops, lm, (u32)(level + c->h.K), (u32)level, (u32)plain_level,
+                     accumulate != 0 || done != 0, c->h.N);
+  }
+  ACE_CATCH_INT
+}
+
 int ace_poly_automorphism(ace_ctx* c, int64_t* r, const int64_t* a, const int64_t* order, size_t level, int with_p) {
   ACE_TRY
   if (!r || !a || !order) return fail("ace_poly_automorphism: null argument");

@@ -55,6 +55,17 @@ bool launch_ntt(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolyS
                 const LimbMap* pos, u32 n_limbs, u32 n_polys, bool inverse, const u64* scale, int passes = 3,
                 const FwdFuse* fuse = nullptr);
 
+constexpr u32 kMaxMacOps = 32;
+struct MacSet { // operands of one multiply-accumulate launch
+  const u64* a0[kMaxMacOps];
+  const u64* a1[kMaxMacOps];
+  const u64* p[kMaxMacOps];
+  u32 n;
+};
+// (r0, r1) (+)= sum_j (a0_j, a1_j) * p_j over n_limbs limbs; limb t of p_j sits at limb t below `level`,
+// at plain_level + (t - level) above it
+void launch_plain_mac(hipStream_t st, const DevCtx& c, u64* r0, u64* r1, const MacSet& ops, const LimbMap& lm,
+                      u32 n_limbs, u32 level, u32 plain_level, bool accumulate, u64 n);
 // elementwise over n_limbs limbs of n words each (limb t uses lm.prime[t]);
 // scalar ops take the same scalar for every limb.
 void launch_ew(hipStream_t st, const DevCtx& c, EwOp op, u64* r, const u64* a, const u64* b, u64 scalar,

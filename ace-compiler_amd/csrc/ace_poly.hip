@@ -55,6 +55,36 @@ void launch_ew(hipStream_t st, const DevCtx& c, EwOp op, u64* r, const u64* a, c
 #undef ACE_EW_CASE
 }
 
+// ---- sum over operands of (a0_j, a1_j) * plain_j: the inner sum of a baby-step group --------------
+// (the Mul_plaintext + Add_ciphertext loop of Rotate_iteration, ckks/src/bootstrap.c:1291-1311).
+// The operands are extended polynomials (level Q limbs, then the P limbs); a plaintext may be kept at a
+// higher level, so its P limbs start plain_level limbs in (Derive_plain, include/ckks/plaintext.h:107-114).
+__global__ __launch_bounds__(kThreads) void plain_mac_kernel(DevCtx c, u64* __restrict__ r0, u64* __restrict__ r1,
+                                                             MacSet ops, LimbMap lm, u32 level, u32 plain_level,
+                                                             int accumulate, u64 n) {
+  const u32 limb = blockIdx.y;
+  const DevPrime P = c.primes[lm.prime[limb]];
+  const u64 base = (u64)limb * n;
+  const u64 pbase = (u64)(limb < level ? limb : plain_level + (limb - level)) * n;
+#pragma unroll
+  ACE_EW_LOOP(i, n) {
+    u64 s0 = accumulate ? r0[base + i] : 0, s1 = accumulate ? r1[base + i] : 0;
+    for (u32 j = 0; j < ops.n; ++j) {
+      u64 w = ops.p[j][pbase + i];
+      s0 = add_mod(s0, mulmod(ops.a0[j][base + i], w, P), P.q);
+      s1 = add_mod(s1, mulmod(ops.a1[j][base + i], w, P), P.q);
+    }
+    r0[base + i] = s0;
+    r1[base + i] = s1;
+  }
+}
+void launch_plain_mac(hipStream_t st, const DevCtx& c, u64* r0, u64* r1, const MacSet& ops, const LimbMap& lm,
+                      u32 n_limbs, u32 level, u32 plain_level, bool accumulate, u64 n) {
+  if (!n || !n_limbs || !ops.n) return;
+  hipLaunchKernelGGL(plain_mac_kernel, ew_grid(n, n_limbs), dim3(kThreads), 0, st, c, r0, r1, ops, lm, level,
+                     plain_level, accumulate ? 1 : 0, n);
+}
+
 // ---- Hw_rotate / Automorphism_transform (hal.c:123-138, rns_poly.c:1056-1099)
 // blockIdx.z = rotation: its own index table, input pair and output pair.
 __global__ __launch_bounds__(kThreads) void gather_kernel(DevCtx c, u64* __restrict__ r0, u64* __restrict__ r1,

@@ -499,21 +499,6 @@ static void ext_rotate(EXT_CT* out, const int64_t* digits, size_t n_digits, cons
   ACE_OK(ace_poly_automorphism(G.ctx, out->c0, tmp->c0, key->order, level, 1));
   ACE_OK(ace_poly_automorphism(G.ctx, out->c1, tmp->c1, key->order, level, 1));
 }
-/* res (+)= a * plain, where the plaintext may sit at a higher level than the ciphertext: its P limbs
- * follow all of ITS Q limbs (Derive_plain, include/ckks/plaintext.h:107-114) */
-static void ext_mul_plain(int64_t* res, const int64_t* a, PLAINTEXT* pt, size_t level, bool accumulate) {
-  size_t n = G.N, pl = pt->_poly._num_primes;
-  FMT_ASSERT(pl >= level && pt->_poly._num_primes_p == G.K, "bootstrap plaintext below the ciphertext level");
-  for (size_t t = 0; t < level + G.K; ++t) {
-    size_t         prime = t < level ? t : G.L + (t - level);
-    const int64_t* p     = pt->_poly._data + (t < level ? t : pl + (t - level)) * n;
-    if (accumulate)
-      ACE_OK(ace_hw_modmuladd(G.ctx, res + t * n, a + t * n, p, prime, n));
-    else
-      ACE_OK(ace_hw_modmul(G.ctx, res + t * n, a + t * n, p, prime, n));
-  }
-}
-
 static void rotate_iteration(CIPHER ct, BTS_PRECOM* pre, bool encoding, int32_t s, bool is_rem, bool first_step) {
   const FFT_PLAN* p      = encoding ? &pre->enc : &pre->dec;
   PLAINTEXT*      plains = (encoding ? pre->enc_plain : pre->dec_plain)[s];
@@ -538,15 +523,19 @@ static void rotate_iteration(CIPHER ct, BTS_PRECOM* pre, bool encoding, int32_t 
   }
   int64_t *first = Rt_dev_alloc(T * n), *moved = Rt_dev_alloc(T * n), *low = Rt_dev_alloc(level * n);
   int64_t* low_digits = Rt_dev_alloc(nd * T * n);
+  const int64_t *in0[64], *in1[64], *inp[64];
   for (int32_t i = 0; i < r.baby; ++i) {
-    bool started = false;
+    size_t count = 0, plain_level = 0;
     for (int32_t j = 0; j < r.giant; ++j) {
       int32_t d = r.giant * i + j;
       if (d == r.num_rot) continue;
-      ext_mul_plain(inner.c0, rots[j].c0, &plains[d], level, started);
-      ext_mul_plain(inner.c1, rots[j].c1, &plains[d], level, started);
-      started = true;
+      FMT_ASSERT(plains[d]._poly._num_primes >= level, "bootstrap plaintext below the ciphertext level");
+      plain_level  = plains[d]._poly._num_primes;
+      in0[count]   = rots[j].c0;
+      in1[count]   = rots[j].c1;
+      inp[count++] = plains[d]._poly._data;
     }
+    ACE_OK(ace_ext_plain_mac(G.ctx, inner.c0, inner.c1, in0, in1, inp, count, level, plain_level, 0));
     if (i == 0) { /* the c0 parts are summed aside and meet the c1 parts at the end */
       Rt_dev_copy(first, inner.c0, T * n);
       ACE_OK(ace_zero(G.ctx, outer.c0, T * n));

@@ -138,6 +138,13 @@ int ace_poly_add(ace_ctx* ctx, int64_t* res, const int64_t* a, const int64_t* b,
 int ace_poly_sub(ace_ctx* ctx, int64_t* res, const int64_t* a, const int64_t* b, size_t level, int with_p);
 int ace_poly_mul(ace_ctx* ctx, int64_t* res, const int64_t* a, const int64_t* b, size_t level, int with_p);
 int ace_poly_automorphism(ace_ctx* ctx, int64_t* res, const int64_t* a, const int64_t* order, size_t level, int with_p);
+/* The inner sum of a baby-step group of the bootstrap's linear transforms (Mul_plaintext + Add_ciphertext,
+ * ckks/src/bootstrap.c:1291-1311): (r0, r1) = sum_j (a0[j], a1[j]) * plain[j], or += when `accumulate`.
+ * Operands and result are extended polynomials at `level`; a plaintext holds plain_level >= level Q limbs
+ * before its P limbs (Derive_plain, include/ckks/plaintext.h:107-114).  a0/a1/plain: host arrays of `count`
+ * device pointers; no operand may alias the result. */
+int ace_ext_plain_mac(ace_ctx* ctx, int64_t* r0, int64_t* r1, const int64_t* const* a0, const int64_t* const* a1,
+                      const int64_t* const* plain, size_t count, size_t level, size_t plain_level, int accumulate);
 /* Decomp_modup (:160-258) (== Decomp :74-105 + Mod_up :107-158): digit `part`
  * of src (level limbs) raised to level+num_p limbs. */
 int ace_decomp_modup(ace_ctx* ctx, int64_t* res, const int64_t* src, size_t level, size_t part, int is_ntt);

@@ -4,7 +4,7 @@
  *
  * usage: bootstrap_program <poly degree> <mul depth> <q0 bits> <scale bits> <hamming weight> <slots>
  *                          <level after bootstrap, 0 = highest> <seed>
- * prints "max_err <e> level <l> ms <t>"; exit status 0 when max_err < 1e-3 and the level is the one asked for.
+ * prints "max_err <e> square_err <e> level <l> first_ms <t> ms <t>" (the first call includes the set-up); exit status 0 when max_err < 1e-3 and the level is the one asked for.
  */
 #include <math.h>
 #include <time.h>
@@ -59,11 +59,18 @@ int main(int argc, char** argv) {
   Encrypt(&ct, &pt);
   Set_slots(&ct, slots);
 
-  double t0 = Now_ms();
-  Eval_bootstrap_ciph(&fresh, &ct, level_after, slots);
+  /* the first call also builds the plaintext diagonals and the rotation keys of this slot count */
+  double    t_first = Now_ms();
   PLAINTEXT back;
   memset(&back, 0, sizeof(back));
-  Rt_decrypt(&back, &fresh); /* also the synchronisation point of the timing */
+  Eval_bootstrap_ciph(&fresh, &ct, level_after, slots);
+  Rt_decrypt(&back, &fresh); /* decryption downloads nothing; Get_msg_from_plain below synchronises */
+  free(Get_msg_from_plain(&back));
+  t_first   = Now_ms() - t_first;
+  double t0 = Now_ms();
+  Eval_bootstrap_ciph(&fresh, &ct, level_after, slots);
+  Rt_decrypt(&back, &fresh);
+  double*  y     = Get_msg_from_plain(&back);
   double   t1    = Now_ms();
   uint32_t level = Level(&fresh);
 
@@ -72,14 +79,13 @@ int main(int argc, char** argv) {
   PLAINTEXT back2;
   memset(&back2, 0, sizeof(back2));
   Rt_decrypt(&back2, &sq);
-  double* y  = Get_msg_from_plain(&back);
   double* y2 = Get_msg_from_plain(&back2);
   double  max_err = 0, max_sq = 0;
   for (uint32_t i = 0; i < slots; ++i) {
     max_err = fmax(max_err, fabs(y[i] - x[i]));
     max_sq  = fmax(max_sq, fabs(y2[i] - x[i] * x[i]));
   }
-  printf("max_err %.3e square_err %.3e level %u ms %.1f\n", max_err, max_sq, level, t1 - t0);
+  printf("max_err %.3e square_err %.3e level %u first_ms %.1f ms %.1f\n", max_err, max_sq, level, t_first, t1 - t0);
   free(y);
   free(y2);
   free(x);

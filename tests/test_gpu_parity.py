@@ -430,3 +430,43 @@ def test_rejected_calls(pair):
         g.hw("modmul_scalar", buf, buf, g.primes[0], 0)
     g.ntt(buf, buf, [], n_polys=0)  # empty input is a no-op
     g.hw("modadd", buf, buf, buf, 0, n=0)
+
+
+def test_ext_plain_mac(pair):
+    """Sum of plaintext products in the extended domain against limb-wise modmul / modadd of the oracle:
+    plaintexts kept at a higher level than the ciphertext, 35 operands (two launches), then accumulation."""
+    g, o = pair.g, pair.o
+    N, L, K = g.N, g.L, g.K
+    if N > 8192:
+        pytest.skip("the oracle works limb by limb; covered at the smaller rings")
+    level = max(1, L - 1)
+    primes_ct = list(g.primes[:level]) + list(g.primes[L:])
+    idx_ct = list(range(level)) + list(range(L, L + K))
+    count = 35
+    a0 = [seeded.uniform_poly(3000 + j, primes_ct, N) for j in range(count)]
+    a1 = [seeded.uniform_poly(3100 + j, primes_ct, N) for j in range(count)]
+    pl = [seeded.uniform_poly(3200 + j, list(g.primes), N) for j in range(count)]  # L Q limbs, then the P limbs
+    pick = np.concatenate([np.arange(level * N), np.arange(L * N, (L + K) * N)])
+
+    def mac(acc, xs):
+        out = acc.copy()
+        for x, p in zip(xs, pl):
+            pv = p[pick]
+            for t, pi in enumerate(idx_ct):
+                sl = slice(t * N, (t + 1) * N)
+                out[sl] = o.hw("modadd", out[sl], o.hw("modmul", x[sl], pv[sl], pi), pi)
+        return out
+    zero = np.zeros((level + K) * N, np.int64)
+    w0, w1 = mac(zero, a0), mac(zero, a1)
+    d0, d1, dp = [g.upload(v) for v in a0], [g.upload(v) for v in a1], [g.upload(v) for v in pl]
+    r0, r1 = g.alloc((level + K) * N), g.alloc((level + K) * N)
+    g.ext_plain_mac(r0, r1, d0, d1, dp, level, L)
+    eq(r0.get(), w0, "ext_plain_mac c0")
+    eq(r1.get(), w1, "ext_plain_mac c1")
+    g.ext_plain_mac(r0, r1, d0[:3], d1[:3], dp[:3], level, L, accumulate=True)
+    eq(r0.get(), mac(w0, a0[:3]), "ext_plain_mac accumulate c0")
+    eq(r1.get(), mac(w1, a1[:3]), "ext_plain_mac accumulate c1")
+    with pytest.raises(RuntimeError):
+        g.ext_plain_mac(r0, r1, [r0], d1[:1], dp[:1], level, L)
+    with pytest.raises(RuntimeError):
+        g.ext_plain_mac(r0, r1, d0[:1], d1[:1], dp[:1], L, level)

@@ -25,6 +25,10 @@ def test_library_exports_every_declared_symbol():
     missing = [s for s in sorted(declared) if not hasattr(lib, s)]
     assert not missing, missing
     assert declared == set(acefhe.EXPORTS)
+    # every binding declares its argument types: an undeclared one would pass 64-bit pointers as C ints
+    bound = acefhe.lib()
+    untyped = [s for s in sorted(declared) if getattr(bound, s).argtypes is None]
+    assert not untyped, untyped
 
 
 @pytest.mark.parametrize("cfg", CONFIGS)
