@@ -90,12 +90,16 @@ def _sig(lib):
     f("ace_mul_relin_rescale_batch", C.c_int, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _sz, _vp, _sz, _sz)
     f("ace_fast_rotate", C.c_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz)
     f("ace_rotate_batch", C.c_int, _vp, _vp, _vp, _vp, _vp, C.POINTER(_vp), C.POINTER(_vp), _sz, _sz)
+    f("ace_poly_add_scalars", C.c_int, _vp, _vp, _vp, _i64p, _sz)
+    f("ace_poly_mul_scalars", C.c_int, _vp, _vp, _vp, _i64p, _sz)
+    f("ace_ciph_wsum", C.c_int, _vp, _vp, _vp, C.POINTER(_vp), C.POINTER(_vp), _i64p, _sz, _sz)
+    f("ace_alloc_uninit", _vp, _vp, _sz)
     f("ace_ext_plain_mac", C.c_int, _vp, _vp, _vp, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), _sz, _sz, _sz, C.c_int)
 
 
 # every symbol include/ace_hip.h declares
 EXPORTS = [
-    "ace_ext_plain_mac", "ace_ctx_create", "ace_ctx_create_with_primes", "ace_ctx_destroy", "ace_has_device", "ace_last_error",
+    "ace_ext_plain_mac", "ace_poly_add_scalars", "ace_poly_mul_scalars", "ace_ciph_wsum", "ace_alloc_uninit", "ace_ctx_create", "ace_ctx_create_with_primes", "ace_ctx_destroy", "ace_has_device", "ace_last_error",
     "ace_degree", "ace_num_q", "ace_num_p", "ace_num_parts", "ace_part_size", "ace_num_decomp", "ace_prime",
     "ace_root", "ace_modulus", "ace_host_twiddles", "ace_host_tbl_modup", "ace_host_tbl_moddown",
     "ace_host_tbl_rescale", "ace_host_automorphism_order", "ace_alloc", "ace_free", "ace_upload", "ace_download",
@@ -361,6 +365,19 @@ class Context:
 
     def fast_rotate(self, r0, r1, c0, digits, swk, order, level):
         self._chk(self.lib.ace_fast_rotate(self.h, r0.ptr, r1.ptr, c0.ptr, digits.ptr, swk.ptr, order.ptr, level))
+
+    def poly_scalars(self, mul, r, a, scalars, level):
+        sc = np.ascontiguousarray(scalars, dtype=np.int64)
+        fn = self.lib.ace_poly_mul_scalars if mul else self.lib.ace_poly_add_scalars
+        self._chk(fn(self.h, r.ptr, a.ptr, sc.ctypes.data_as(_i64p), level))
+
+    def ciph_wsum(self, r0, r1, a0s, a1s, weights, level):
+        n = len(a0s)
+        w = np.ascontiguousarray(weights, dtype=np.int64).ravel()
+        assert w.size == n * level
+        p0 = (_vp * n)(*[a.ptr for a in a0s])
+        p1 = (_vp * n)(*[a.ptr for a in a1s])
+        self._chk(self.lib.ace_ciph_wsum(self.h, r0.ptr, r1.ptr, p0, p1, w.ctypes.data_as(_i64p), n, level))
 
     def ext_plain_mac(self, r0, r1, a0s, a1s, plains, level, plain_level, accumulate=False):
         n = len(plains)

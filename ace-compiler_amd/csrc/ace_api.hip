@@ -716,7 +716,10 @@ void ace_modulus(const ace_ctx* c, size_t i, uint64_t out[5]) {
 // loop, and hipMalloc / hipFree cost far more than the kernels between them.
 // Reuse is safe without a wait because every use of a buffer is ordered on
 // the context's one stream.
-int64_t* ace_alloc(ace_ctx* c, size_t n_words) {
+static int64_t* alloc_words(ace_ctx* c, size_t n_words, bool zero);
+int64_t* ace_alloc(ace_ctx* c, size_t n_words) { return alloc_words(c, n_words, true); }
+int64_t* ace_alloc_uninit(ace_ctx* c, size_t n_words) { return alloc_words(c, n_words, false); }
+static int64_t* alloc_words(ace_ctx* c, size_t n_words, bool zero) {
   try {
     if (!c || !c->device_ok) throw std::runtime_error("no HIP device: this context holds host tables only");
     const size_t words = std::max<size_t>(n_words, 1);
@@ -736,7 +739,7 @@ int64_t* ace_alloc(ace_ctx* c, size_t n_words) {
       HIP_OK(e);
     }
     c->live[p] = words;
-    launch_fill_zero(c->stream, p, n_words);
+    if (zero) launch_fill_zero(c->stream, p, n_words);
     return reinterpret_cast<int64_t*>(p);
   } catch (const std::exception& e) {
     g_err = e.what();
@@ -983,6 +986,45 @@ int ace_ext_plain_mac(ace_ctx* c, int64_t* r0, int64_t* r1, const int64_t* const
     launch_plain_mac(c->stream, c->d, U(r0), U(r1), ops, lm, (u32)(level + c->h.K), (u32)level, (u32)plain_level,
                      accumulate != 0 || done != 0, c->h.N);
   }
+  ACE_CATCH_INT
+}
+
+static int poly_scalars(ace_ctx* c, bool mul, int64_t* r, const int64_t* a, const int64_t* scalars, size_t level) {
+  ACE_TRY
+  if (!r || !a || !scalars) return fail("ace_poly_scalars: null argument");
+  if (!level_ok(c, level)) return fail("ace_poly_scalars: level out of range");
+  LimbScalars s{};
+  for (size_t t = 0; t < level; ++t) {
+    if (scalars[t] < 0 || (u64)scalars[t] >= c->h.primes[t].q) return fail("ace_poly_scalars: scalar is not a residue");
+    s.v[t] = (u64)scalars[t];
+  }
+  launch_limb_scalars(c->stream, c->d, mul, U(r), U(a), s, poly_lm(c, level, false), (u32)level, c->h.N);
+  ACE_CATCH_INT
+}
+int ace_poly_add_scalars(ace_ctx* c, int64_t* r, const int64_t* a, const int64_t* scalars, size_t level) { return poly_scalars(c, false, r, a, scalars, level); }
+int ace_poly_mul_scalars(ace_ctx* c, int64_t* r, const int64_t* a, const int64_t* scalars, size_t level) { return poly_scalars(c, true, r, a, scalars, level); }
+
+int ace_ciph_wsum(ace_ctx* c, int64_t* r0, int64_t* r1, const int64_t* const* a0, const int64_t* const* a1,
+                  const int64_t* weights, size_t count, size_t level) {
+  ACE_TRY
+  if (!r0 || !r1 || !a0 || !a1 || !weights) return fail("ace_ciph_wsum: null argument");
+  if (!level_ok(c, level)) return fail("ace_ciph_wsum: level out of range");
+  if (!count || count > kMaxMacOps) return fail("ace_ciph_wsum: between 1 and 32 terms");
+  MacSet ops{};
+  ops.n = (u32)count;
+  for (size_t j = 0; j < count; ++j) {
+    if (!a0[j] || !a1[j]) return fail("ace_ciph_wsum: null operand");
+    ops.a0[j] = U(a0[j]);
+    ops.a1[j] = U(a1[j]);
+    for (size_t t = 0; t < level; ++t)
+      if (weights[j * level + t] < 0 || (u64)weights[j * level + t] >= c->h.primes[t].q)
+        return fail("ace_ciph_wsum: weight is not a residue");
+  }
+  c->ensure_ws(count * level);
+  c->ws_used = 0;
+  u64* w = c->take(count * level);
+  HIP_OK(hipMemcpyAsync(w, weights, count * level * sizeof(u64), hipMemcpyHostToDevice, c->stream));
+  launch_wsum(c->stream, c->d, U(r0), U(r1), ops, w, poly_lm(c, level, false), (u32)level, c->h.N);
   ACE_CATCH_INT
 }
 

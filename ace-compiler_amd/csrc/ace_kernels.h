@@ -66,6 +66,15 @@ struct MacSet { // operands of one multiply-accumulate launch
 // at plain_level + (t - level) above it
 void launch_plain_mac(hipStream_t st, const DevCtx& c, u64* r0, u64* r1, const MacSet& ops, const LimbMap& lm,
                       u32 n_limbs, u32 level, u32 plain_level, bool accumulate, u64 n);
+struct LimbScalars { // one residue per limb
+  u64 v[kMaxPrimes];
+};
+// r[t] = a[t] + s.v[t] (mul == false) or a[t] * s.v[t] (mul == true) modulo prime lm.prime[t]
+void launch_limb_scalars(hipStream_t st, const DevCtx& c, bool mul, u64* r, const u64* a, const LimbScalars& s,
+                         const LimbMap& lm, u32 n_limbs, u64 n);
+// (r0, r1) = sum_j w[j*n_limbs + t] * (a0_j, a1_j)[t]; w is a device array
+void launch_wsum(hipStream_t st, const DevCtx& c, u64* r0, u64* r1, const MacSet& ops, const u64* w,
+                 const LimbMap& lm, u32 n_limbs, u64 n);
 // elementwise over n_limbs limbs of n words each (limb t uses lm.prime[t]);
 // scalar ops take the same scalar for every limb.
 void launch_ew(hipStream_t st, const DevCtx& c, EwOp op, u64* r, const u64* a, const u64* b, u64 scalar,

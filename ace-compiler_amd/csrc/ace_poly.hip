@@ -85,6 +85,51 @@ void launch_plain_mac(hipStream_t st, const DevCtx& c, u64* r0, u64* r1, const M
                      plain_level, accumulate ? 1 : 0, n);
 }
 
+// ---- per-limb scalars: Scalars_integer_add_poly / Scalars_integer_multiply_poly (poly/src/rns_poly.c) ----
+template <int MUL>
+__global__ __launch_bounds__(kThreads) void limb_scalar_kernel(DevCtx c, u64* __restrict__ r, const u64* __restrict__ a,
+                                                               LimbScalars s, LimbMap lm, u64 n) {
+  const u32 limb = blockIdx.y;
+  const DevPrime P = c.primes[lm.prime[limb]];
+  const u64 base = (u64)limb * n, v = s.v[limb];
+#pragma unroll
+  ACE_EW_LOOP(i, n) r[base + i] = MUL ? mulmod(a[base + i], v, P) : add_mod(a[base + i], v, P.q);
+}
+void launch_limb_scalars(hipStream_t st, const DevCtx& c, bool mul, u64* r, const u64* a, const LimbScalars& s,
+                         const LimbMap& lm, u32 n_limbs, u64 n) {
+  if (!n || !n_limbs) return;
+  if (mul)
+    hipLaunchKernelGGL(limb_scalar_kernel<1>, ew_grid(n, n_limbs), dim3(kThreads), 0, st, c, r, a, s, lm, n);
+  else
+    hipLaunchKernelGGL(limb_scalar_kernel<0>, ew_grid(n, n_limbs), dim3(kThreads), 0, st, c, r, a, s, lm, n);
+}
+
+// ---- weighted sum of ciphertexts: (r0, r1) = sum_j w[j][limb] * (a0_j, a1_j) -------------------------------
+// (Mul_const + Add_ciphertext over the terms of Eval_linear_wsum, ckks/src/chebyshev_impl.c:276-318)
+__global__ __launch_bounds__(kThreads) void wsum_kernel(DevCtx c, u64* __restrict__ r0, u64* __restrict__ r1,
+                                                        MacSet ops, const u64* __restrict__ w, LimbMap lm,
+                                                        u32 n_limbs, u64 n) {
+  const u32 limb = blockIdx.y;
+  const DevPrime P = c.primes[lm.prime[limb]];
+  const u64 base = (u64)limb * n;
+#pragma unroll
+  ACE_EW_LOOP(i, n) {
+    u64 s0 = 0, s1 = 0;
+    for (u32 j = 0; j < ops.n; ++j) {
+      u64 v = w[j * n_limbs + limb];
+      s0 = add_mod(s0, mulmod(ops.a0[j][base + i], v, P), P.q);
+      s1 = add_mod(s1, mulmod(ops.a1[j][base + i], v, P), P.q);
+    }
+    r0[base + i] = s0;
+    r1[base + i] = s1;
+  }
+}
+void launch_wsum(hipStream_t st, const DevCtx& c, u64* r0, u64* r1, const MacSet& ops, const u64* w,
+                 const LimbMap& lm, u32 n_limbs, u64 n) {
+  if (!n || !n_limbs || !ops.n) return;
+  hipLaunchKernelGGL(wsum_kernel, ew_grid(n, n_limbs), dim3(kThreads), 0, st, c, r0, r1, ops, w, lm, n_limbs, n);
+}
+
 // ---- Hw_rotate / Automorphism_transform (hal.c:123-138, rns_poly.c:1056-1099)
 // blockIdx.z = rotation: its own index table, input pair and output pair.
 __global__ __launch_bounds__(kThreads) void gather_kernel(DevCtx c, u64* __restrict__ r0, u64* __restrict__ r1,

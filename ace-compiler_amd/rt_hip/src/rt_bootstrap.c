@@ -407,10 +407,7 @@ static void add_const(CIPHER c, double value) { /* Add_const, in place */
   int64_t w[128];
   size_t  l = Level(c);
   Rt_encode_val_words(w, value, (uint32_t)l, c->_scaling_factor);
-  for (size_t t = 0; t < l; ++t) {
-    int64_t* limb = c->_c0_poly._data + t * G.N;
-    ACE_OK(ace_hw_modadd_scalar(G.ctx, limb, limb, w[t], t, G.N));
-  }
+  ACE_OK(ace_poly_add_scalars(G.ctx, c->_c0_poly._data, c->_c0_poly._data, w, l));
 }
 static void scale_words(CIPHER res, CIPHER c, const int64_t* w, double sf, uint32_t deg) {
   size_t l = Level(c);
@@ -420,10 +417,8 @@ static void scale_words(CIPHER res, CIPHER c, const int64_t* w, double sf, uint3
     res->_slots = c->_slots;
   }
   res->_c0_poly._is_ntt = res->_c1_poly._is_ntt = true;
-  for (size_t t = 0; t < l; ++t) {
-    ACE_OK(ace_hw_modmul_scalar(G.ctx, res->_c0_poly._data + t * G.N, c->_c0_poly._data + t * G.N, w[t], t, G.N));
-    ACE_OK(ace_hw_modmul_scalar(G.ctx, res->_c1_poly._data + t * G.N, c->_c1_poly._data + t * G.N, w[t], t, G.N));
-  }
+  ACE_OK(ace_poly_mul_scalars(G.ctx, res->_c0_poly._data, c->_c0_poly._data, w, l));
+  ACE_OK(ace_poly_mul_scalars(G.ctx, res->_c1_poly._data, c->_c1_poly._data, w, l));
   res->_scaling_factor = sf;
   res->_sf_degree      = deg;
 }
@@ -479,7 +474,7 @@ typedef struct {
   int64_t *c0, *c1; /* level + num_p limbs each */
 } EXT_CT;
 static EXT_CT ext_alloc(size_t level) {
-  EXT_CT e = {Rt_dev_alloc((level + G.K) * G.N), Rt_dev_alloc((level + G.K) * G.N)};
+  EXT_CT e = {Rt_dev_alloc_raw((level + G.K) * G.N), Rt_dev_alloc_raw((level + G.K) * G.N)};
   return e;
 }
 static void ext_free(EXT_CT* e) {
@@ -506,9 +501,9 @@ static void rotate_iteration(CIPHER ct, BTS_PRECOM* pre, bool encoding, int32_t 
   if (!first_step) rescale(ct);
   size_t level = Level(ct), T = level + G.K, n = G.N, nd = ace_num_decomp(G.ctx, level);
 
-  int64_t* digits = Rt_dev_alloc(nd * T * n);
+  int64_t* digits = Rt_dev_alloc_raw(nd * T * n);
   ACE_OK(ace_precomp(G.ctx, digits, ct->_c1_poly._data, level, 1));
-  int64_t* c0_ext = Rt_dev_alloc(T * n);
+  int64_t* c0_ext = Rt_dev_alloc_raw(T * n);
   ACE_OK(ace_extend(G.ctx, c0_ext, ct->_c0_poly._data, level));
   EXT_CT  tmp = ext_alloc(level), inner = ext_alloc(level), outer = ext_alloc(level);
   EXT_CT* rots = (EXT_CT*)calloc((size_t)r.giant, sizeof(EXT_CT));
@@ -521,8 +516,8 @@ static void rotate_iteration(CIPHER ct, BTS_PRECOM* pre, bool encoding, int32_t 
       ACE_OK(ace_extend(G.ctx, rots[j].c1, ct->_c1_poly._data, level));
     }
   }
-  int64_t *first = Rt_dev_alloc(T * n), *moved = Rt_dev_alloc(T * n), *low = Rt_dev_alloc(level * n);
-  int64_t* low_digits = Rt_dev_alloc(nd * T * n);
+  int64_t *first = Rt_dev_alloc_raw(T * n), *moved = Rt_dev_alloc_raw(T * n), *low = Rt_dev_alloc_raw(level * n);
+  int64_t* low_digits = Rt_dev_alloc_raw(nd * T * n);
   const int64_t *in0[64], *in1[64], *inp[64];
   for (int32_t i = 0; i < r.baby; ++i) {
     size_t count = 0, plain_level = 0;
@@ -673,22 +668,31 @@ typedef struct {
 
 /* out = sum w_i T_i (i = 1..count) as one level (Eval_linear_wsum, chebyshev_impl.c:276-318) */
 static void weighted_sum(CIPHER out, CHEB_BASIS* b, const double* w, uint32_t count) {
-  CIPHERTEXT tmp;
-  new_ciph(&tmp);
-  bool first = true;
+  const int64_t *in0[64], *in1[64];
+  size_t         terms = 0, level = Level(&b->t[0]);
+  FMT_ASSERT(count <= 32, "more than 32 terms in one weighted sum");
+  for (uint32_t i = 0; i < count; ++i) /* the T_i share one level (see eval_chebyshev), except unused odd ones */
+    if (w[i] != 0.0 && Level(&b->t[i]) < level) level = Level(&b->t[i]);
+  int64_t* words = (int64_t*)malloc(32 * 128 * sizeof(int64_t));
+  CIPHER   like  = NULL;
   for (uint32_t i = 0; i < count; ++i) {
     if (w[i] == 0.0) continue;
-    if (first) {
-      mul_const(out, &b->t[i], w[i]);
-      first = false;
-    } else {
-      mul_const(&tmp, &b->t[i], w[i]);
-      Add_ciph(out, out, &tmp);
-    }
+    like = &b->t[i];
+    Rt_encode_val_words(words + terms * level, w[i], (uint32_t)level, G.sc);
+    in0[terms]   = b->t[i]._c0_poly._data;
+    in1[terms++] = b->t[i]._c1_poly._data;
   }
-  FMT_ASSERT(!first, "polynomial has no non_zero coefficient");
+  FMT_ASSERT(terms, "polynomial has no non_zero coefficient");
+  Init_poly(&out->_c0_poly, &like->_c0_poly);
+  Init_poly(&out->_c1_poly, &like->_c1_poly);
+  set_level(out, level);
+  out->_c0_poly._is_ntt = out->_c1_poly._is_ntt = true;
+  out->_slots          = like->_slots;
+  out->_scaling_factor = like->_scaling_factor * G.sc;
+  out->_sf_degree      = like->_sf_degree + 1;
+  ACE_OK(ace_ciph_wsum(G.ctx, out->_c0_poly._data, out->_c1_poly._data, in0, in1, words, terms, level));
+  free(words);
   rescale(out);
-  Free_ciph_poly(&tmp, 1);
 }
 /* a series of degree <= k whose T_k coefficient is known to be `lead` (a power of two, or 1):
  * that term is added, never multiplied, to save the level (Eval_quot_or_rem, chebyshev_impl.c:320-384) */

@@ -54,6 +54,7 @@ extern struct rt_state G;
 #define NEED_CTX() FMT_ASSERT(G.ctx, "Prepare_context() has not run")
 
 size_t   Rt_p_offset(POLY p);
+int64_t* Rt_dev_alloc_raw(size_t n_words);
 IO_SLOT* Rt_find_slot(IO_SLOT* s, size_t n, const char* name, size_t idx);
 IO_SLOT* Rt_add_slot(IO_SLOT** s, size_t* n, const char* name, size_t idx);
 void     Rt_install_key(SWITCH_KEY* k, const int64_t* host);

@@ -83,6 +83,8 @@ int ace_host_automorphism_order(const ace_ctx* ctx, int64_t* host_order, uint32_
  * total) for the next ace_alloc of the same size, so alloc/free pairs inside a
  * program's loops cost a fill kernel, not a hipMalloc. */
 int64_t* ace_alloc(ace_ctx* ctx, size_t n_words);
+/* the same without the zero fill, for buffers that are written before they are read */
+int64_t* ace_alloc_uninit(ace_ctx* ctx, size_t n_words);
 void     ace_free(ace_ctx* ctx, int64_t* dev_ptr);
 int      ace_upload(ace_ctx* ctx, int64_t* dev_dst, const int64_t* host_src, size_t n_words);
 int      ace_download(ace_ctx* ctx, int64_t* host_dst, const int64_t* dev_src, size_t n_words); /* synchronises */
@@ -138,6 +140,16 @@ int ace_poly_add(ace_ctx* ctx, int64_t* res, const int64_t* a, const int64_t* b,
 int ace_poly_sub(ace_ctx* ctx, int64_t* res, const int64_t* a, const int64_t* b, size_t level, int with_p);
 int ace_poly_mul(ace_ctx* ctx, int64_t* res, const int64_t* a, const int64_t* b, size_t level, int with_p);
 int ace_poly_automorphism(ace_ctx* ctx, int64_t* res, const int64_t* a, const int64_t* order, size_t level, int with_p);
+/* Scalars_integer_add_poly / Scalars_integer_multiply_poly (poly/src/rns_poly.c; Add_scalars, Mul_scalars,
+ * evaluator.c:113-125,218-235): limb t of res = limb t of a plus / times scalars[t] (a HOST array of `level`
+ * residues).  res may equal a. */
+int ace_poly_add_scalars(ace_ctx* ctx, int64_t* res, const int64_t* a, const int64_t* scalars, size_t level);
+int ace_poly_mul_scalars(ace_ctx* ctx, int64_t* res, const int64_t* a, const int64_t* scalars, size_t level);
+/* Eval_linear_wsum (ckks/src/chebyshev_impl.c:276-318) without its rescale: (r0, r1) = sum_j weights[j] *
+ * (a0[j], a1[j]) at `level`; weights is a HOST array of count x level residues (the encoded constants of
+ * Mul_const), a0/a1 host arrays of `count` (<= 32) device pointers.  The result may alias an operand. */
+int ace_ciph_wsum(ace_ctx* ctx, int64_t* r0, int64_t* r1, const int64_t* const* a0, const int64_t* const* a1,
+                  const int64_t* weights, size_t count, size_t level);
 /* The inner sum of a baby-step group of the bootstrap's linear transforms (Mul_plaintext + Add_ciphertext,
  * ckks/src/bootstrap.c:1291-1311): (r0, r1) = sum_j (a0[j], a1[j]) * plain[j], or += when `accumulate`.
  * Operands and result are extended polynomials at `level`; a plaintext holds plain_level >= level Q limbs

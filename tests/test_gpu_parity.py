@@ -470,3 +470,46 @@ def test_ext_plain_mac(pair):
         g.ext_plain_mac(r0, r1, [r0], d1[:1], dp[:1], level, L)
     with pytest.raises(RuntimeError):
         g.ext_plain_mac(r0, r1, d0[:1], d1[:1], dp[:1], L, level)
+
+
+def test_limb_scalars_and_weighted_sum(pair):
+    """Per-limb scalar add / multiply and the weighted sum of ciphertexts against limb-wise oracle calls."""
+    g, o = pair.g, pair.o
+    N, L = g.N, g.L
+    if N > 8192:
+        pytest.skip("the oracle works limb by limb; covered at the smaller rings")
+    level = L
+    pr = g.primes[:level]
+    a = seeded.uniform_poly(4000, pr, N)
+    sc = np.array([int(seeded.splitmix64(4100 + t, 1)[0] % np.uint64(q)) for t, q in enumerate(pr)], np.int64)
+    da, r = g.upload(a), g.alloc(level * N)
+    for mul, name in ((False, "modadd_scalar"), (True, "modmul_scalar")):
+        g.poly_scalars(mul, r, da, sc, level)
+        want = np.concatenate([o.hw(name, a[t * N:(t + 1) * N], int(sc[t]), t) for t in range(level)])
+        eq(r.get(), want, name + " per limb")
+    g.poly_scalars(True, da, da, sc, level)  # in place
+    eq(da.get(), want, "modmul_scalar per limb, in place")
+    with pytest.raises(RuntimeError):
+        g.poly_scalars(True, r, da, np.array(pr, np.int64), level)  # q itself is not a residue
+
+    count = 7
+    a0 = [seeded.uniform_poly(4200 + j, pr, N) for j in range(count)]
+    a1 = [seeded.uniform_poly(4300 + j, pr, N) for j in range(count)]
+    w = np.array([[int(seeded.splitmix64(4400 + 100 * j + t, 1)[0] % np.uint64(q)) for t, q in enumerate(pr)]
+                  for j in range(count)], np.int64)
+
+    def wsum(xs):
+        out = np.zeros(level * N, np.int64)
+        for j, x in enumerate(xs):
+            for t in range(level):
+                sl = slice(t * N, (t + 1) * N)
+                out[sl] = o.hw("modadd", out[sl], o.hw("modmul_scalar", x[sl], int(w[j, t]), t), t)
+        return out
+    d0, d1 = [g.upload(v) for v in a0], [g.upload(v) for v in a1]
+    r0, r1 = g.alloc(level * N), g.alloc(level * N)
+    g.ciph_wsum(r0, r1, d0, d1, w, level)
+    eq(r0.get(), wsum(a0), "ciph_wsum c0")
+    eq(r1.get(), wsum(a1), "ciph_wsum c1")
+    g.ciph_wsum(d0[0], d1[0], d0, d1, w, level)  # the result over the first operand
+    eq(d0[0].get(), wsum(a0), "ciph_wsum c0 over an operand")
+    eq(d1[0].get(), wsum(a1), "ciph_wsum c1 over an operand")
