@@ -18,6 +18,7 @@ Prints exactly one JSON line on stdout.
 import argparse
 import json
 import os
+import subprocess
 import sys
 import time
 
@@ -134,6 +135,28 @@ def rotation_leg(g, np, seeded, swk, cts):
     return extra
 
 
+def bootstrap_leg():
+    """One CKKS bootstrap on the host runtime (tests/programs/bootstrap_program, a separate process): N=65536,
+    34 limbs (q0 60 bits, scale 56 bits: the parameters of the reference's published ResNet-20 run, whose 19
+    bootstraps take 784.03 s on one CPU thread), fully packed, refreshed to level 15 as that program asks."""
+    exe = os.path.join(ROOT, "tests", "programs", "bootstrap_program")
+    if not os.path.exists(exe):
+        return {"bootstrap": {"error": "tests/programs/bootstrap_program is not built"}}
+    try:
+        r = subprocess.run([exe, "65536", "33", "60", "56", "192", "32768", "15", "1"], capture_output=True, text=True,
+                           timeout=240)
+        f = r.stdout.split()
+        vals = dict(zip(f[0::2], f[1::2]))
+        ms = float(vals["ms"])
+        return {"bootstrap": {"workload": "one bootstrap, N=65536, 34 limbs (60/56 bits), 32768 slots, to level 15",
+                              "ms": ms, "first_call_ms_with_setup_and_keys": float(vals["first_ms"]),
+                              "max_err": float(vals["max_err"]), "exit_status": r.returncode,
+                              "published_cpu_ms": round(784.03e3 / 19, 1),
+                              "vs_published_cpu": round(784.03e3 / 19 / ms, 1)}}
+    except Exception as e:  # the headline line must still be printed
+        return {"bootstrap": {"error": repr(e)[:200]}}
+
+
 def extra_legs(g, np, seeded, which="all"):
     level = g.L
     swk = g.upload(np.concatenate([seeded.uniform_poly(2000 + i, g.primes, N) for i in range(2 * g.parts)]))
@@ -222,6 +245,8 @@ def main():
     scratch.free()
 
     extra = {} if args.no_extra else extra_legs(g, np, seeded)
+    if not args.no_extra:
+        extra.update(bootstrap_leg())
 
     cpu = cpu_baseline(x_host, idx, args.cpu_seconds) if args.cpu_seconds > 0 else None
 
