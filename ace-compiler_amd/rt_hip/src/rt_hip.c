@@ -120,6 +120,10 @@ int64_t* Rt_dev_alloc(size_t n_words) {
   if (!p) Rt_fatal(__FILE__, __LINE__, "device allocation of %zu words failed: %s", n_words, ace_last_error());
   return p;
 }
+void Rt_sync(void) {
+  NEED_CTX();
+  ACE_OK(ace_sync(G.ctx));
+}
 int64_t* Rt_dev_alloc_raw(size_t n_words) { /* not zero-filled: for buffers written before they are read */
   NEED_CTX();
   int64_t* p = ace_alloc_uninit(G.ctx, n_words);

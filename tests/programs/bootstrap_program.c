@@ -67,11 +67,13 @@ int main(int argc, char** argv) {
   Rt_decrypt(&back, &fresh); /* decryption downloads nothing; Get_msg_from_plain below synchronises */
   free(Get_msg_from_plain(&back));
   t_first   = Now_ms() - t_first;
+  Rt_sync();
   double t0 = Now_ms();
   Eval_bootstrap_ciph(&fresh, &ct, level_after, slots);
+  Rt_sync();
+  double t1 = Now_ms();
   Rt_decrypt(&back, &fresh);
-  double*  y     = Get_msg_from_plain(&back);
-  double   t1    = Now_ms();
+  double* y = Get_msg_from_plain(&back);
   uint32_t level = Level(&fresh);
 
   Mul_ciph(&sq, &fresh, &fresh);
