@@ -1,0 +1,141 @@
+/* rt_data.c -- the weight side-file of a compiled model and the plaintexts made from it.
+ *
+ * File layout (fhe-cmplr/include/fhe/core/rt_data_def.h:62-84, rt_data_writer.h:34-107): a 136-byte header
+ * at offset 0, entries from offset 4096 on, each padded to 2^_ent_align bytes, and a lookup table of
+ * 32-byte records at _lut_ofst.  Message files (float or double entries) are read whole at Prepare_context,
+ * as Pt_mgr_init does (rtlib/ant/porting/pt_mgr.c:35-99); Pt_from_msg encodes `len` values of entry `index`
+ * (pt_mgr.c:188-243).  Files of pre-encoded plaintexts hold host-side polynomial images and are refused.
+ *
+ * RT_HIP_DATA_FILE names the file when the path compiled into the program does not exist here.
+ * RT_HIP_SYNTHETIC_WEIGHTS=<amplitude> replaces a missing file by reproducible pseudo-random values in
+ * (-amplitude, amplitude): for timing a model whose weights are not at hand, never for its accuracy.
+ */
+#include <math.h>
+#include <time.h>
+
+#include "rt_internal.h"
+
+#define DATA_PAGE 4096
+typedef struct {
+  char            magic[8];
+  uint32_t        rt_ver;
+  uint16_t        flag;
+  uint8_t         ent_type, ent_align;
+  uint64_t        ent_count, lut_ofst;
+  struct timespec ctime;
+  char            model[48], uuid[40];
+} DATA_HDR;
+typedef struct {
+  char     name[16];
+  uint32_t index, size;
+  uint64_t scale : 8, level : 8, ofst : 48;
+} LUT_ENTRY;
+_Static_assert(sizeof(DATA_HDR) == 136 && sizeof(LUT_ENTRY) == 32, "side-file records");
+
+static struct {
+  bool       open, synthetic;
+  double     amplitude;
+  DATA_HDR   hdr;
+  LUT_ENTRY* lut;
+  char*      buf; /* the bytes between the first page and the lookup table */
+  uint64_t   size;
+} Data;
+
+bool Pt_mgr_init(const char* fname) {
+  const char* over = getenv("RT_HIP_DATA_FILE");
+  const char* syn  = getenv("RT_HIP_SYNTHETIC_WEIGHTS");
+  if (over && *over) fname = over;
+  memset(&Data, 0, sizeof(Data));
+  FILE* f = fname ? fopen(fname, "rb") : NULL;
+  if (!f) {
+    if (syn && atof(syn) > 0) {
+      Data.open = Data.synthetic = true;
+      Data.amplitude             = atof(syn);
+      fprintf(stderr, "rt_hip: %s not found: synthetic weights of amplitude %g\n", fname ? fname : "(no file)", Data.amplitude);
+      return true;
+    }
+    Rt_fatal(__FILE__, __LINE__, "failed to open rt data file %s (RT_HIP_DATA_FILE overrides the compiled-in path)",
+             fname ? fname : "(null)");
+  }
+  FMT_ASSERT(fread(&Data.hdr, sizeof(DATA_HDR), 1, f) == 1, "failed to read rt data file header");
+  FMT_ASSERT(memcmp(Data.hdr.magic, "!ANTFHE\0", 8) == 0, "%s is not an rt data file", fname);
+  FMT_ASSERT(Data.hdr.ent_type == DE_MSG_F32 || Data.hdr.ent_type == DE_MSG_F64,
+             "rt data files of pre-encoded plaintexts are not supported: their polynomials are host images");
+  FMT_ASSERT(Data.hdr.lut_ofst >= DATA_PAGE, "lookup table inside the first page");
+  Data.lut = (LUT_ENTRY*)malloc((Data.hdr.ent_count ? Data.hdr.ent_count : 1) * sizeof(LUT_ENTRY));
+  FMT_ASSERT(fseek(f, (long)Data.hdr.lut_ofst, SEEK_SET) == 0 &&
+                 fread(Data.lut, sizeof(LUT_ENTRY), Data.hdr.ent_count, f) == Data.hdr.ent_count,
+             "failed to read rt data file lookup table");
+  Data.size = Data.hdr.lut_ofst - DATA_PAGE;
+  Data.buf  = (char*)malloc(Data.size ? Data.size : 1);
+  FMT_ASSERT(fseek(f, DATA_PAGE, SEEK_SET) == 0 && fread(Data.buf, 1, Data.size, f) == Data.size,
+             "failed to fill data from file");
+  fclose(f);
+  Data.open = true;
+  return true;
+}
+
+void Pt_mgr_fini(void) {
+  free(Data.lut);
+  free(Data.buf);
+  memset(&Data, 0, sizeof(Data));
+}
+
+/* entry `index` from value `first` on, `len` values, as doubles */
+static double* entry_values(uint32_t index, size_t first, size_t len) {
+  FMT_ASSERT(Data.open, "the program has no rt data file (Get_rt_data_info)");
+  double* v = (double*)malloc((len ? len : 1) * sizeof(double));
+  if (Data.synthetic) {
+    for (size_t i = 0; i < len; ++i) {
+      uint64_t z = ((uint64_t)index << 32 | (uint64_t)(first + i)) + 0x9E3779B97F4A7C15ull;
+      z          = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+      z          = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+      z ^= z >> 31;
+      v[i] = Data.amplitude * ((double)(int64_t)(z >> 11) / (double)(1ull << 52) - 1.0);
+    }
+    return v;
+  }
+  size_t width = Data.hdr.ent_type == DE_MSG_F32 ? sizeof(float) : sizeof(double);
+  FMT_ASSERT(index < Data.hdr.ent_count, "index out of entry range");
+  const LUT_ENTRY* e = &Data.lut[index];
+  FMT_ASSERT(e->size >= (first + len) * width, "entry size too small");
+  FMT_ASSERT(e->ofst >= DATA_PAGE && e->ofst - DATA_PAGE + (first + len) * width <= Data.size, "entry offset too large");
+  const char* p = Data.buf + (e->ofst - DATA_PAGE) + first * width;
+  for (size_t i = 0; i < len; ++i) {
+    if (width == sizeof(float)) {
+      float x;
+      memcpy(&x, p + i * width, width);
+      v[i] = (double)x;
+    } else {
+      memcpy(&v[i], p + i * width, width);
+    }
+  }
+  return v;
+}
+
+void* Pt_from_msg_ofst(void* pt, uint32_t index, size_t ofst, size_t len, uint32_t scale, uint32_t level) {
+  double* v = entry_values(index, ofst, len);
+  Encode_double((PLAIN)pt, v, len, scale, level);
+  free(v);
+  return pt;
+}
+void* Pt_from_msg(void* pt, uint32_t index, size_t len, uint32_t scale, uint32_t level) {
+  return Pt_from_msg_ofst(pt, index, 0, len, scale, level);
+}
+void Pt_from_msg_ofst_validate(void* pt, float* buf, uint32_t index, size_t ofst, size_t len, uint32_t scale, uint32_t level) {
+  double* v = entry_values(index, ofst, len);
+  for (size_t i = 0; i < len; ++i)
+    FMT_ASSERT(fabs((double)buf[i] - v[i]) < 0.000001, "Pt_from_msg_validate failed. index=%u, i=%zu: %f != %f.", index, i,
+               (double)buf[i], v[i]);
+  Encode_double((PLAIN)pt, v, len, scale, level);
+  free(v);
+}
+void Pt_from_msg_validate(void* pt, float* buf, uint32_t index, size_t len, uint32_t scale, uint32_t level) {
+  Pt_from_msg_ofst_validate(pt, buf, index, 0, len, scale, level);
+}
+void* Pt_get(uint32_t index, size_t len, uint32_t scale, uint32_t level) {
+  (void)len, (void)scale, (void)level;
+  Rt_fatal(__FILE__, __LINE__, "Pt_get(%u): pre-encoded plaintext files are not supported; ship messages (f32 / f64)", index);
+}
+/* Free_data (pt_mgr.c:181-185): the polynomial of a plaintext made by Pt_from_msg */
+void Free_data(void* poly) { Free_poly_data((POLY)poly); }

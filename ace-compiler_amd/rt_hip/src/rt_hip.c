@@ -50,6 +50,7 @@ void Prepare_context(void) {
     G.q[i]._br_m    = (int64_t)f[2];
     G.q[i]._prec128 = ((unsigned __int128)f[4] << 64) | f[3];
   }
+  if (Get_rt_data_info && Get_rt_data_info()) Pt_mgr_init(Get_rt_data_info()->_file_name);
   clock_gettime(CLOCK_MONOTONIC, &G.t0);
 }
 
@@ -73,6 +74,7 @@ static void free_slots(IO_SLOT* s, size_t n) {
 
 void Finalize_context(void) {
   if (!G.ctx) return;
+  if (Get_rt_data_info && Get_rt_data_info()) Pt_mgr_fini();
   Rt_bootstrap_finalize();
   Rt_ckks_finalize();
   free_key(&G.relin);

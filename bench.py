@@ -157,6 +157,29 @@ def bootstrap_leg():
         return {"bootstrap": {"error": repr(e)[:200]}}
 
 
+def resnet20_leg():
+    """The reference's generated ResNet-20/CIFAR-10 program (rtlib/ant/dataset/resnet20_cifar10_pre.onnx.inc,
+    N=65536, 34 limbs, 197 rotation keys, 19 bootstraps), built unchanged against the host runtime where the reference
+    tree was present.  Its weight file is not available, so the weights are pseudo-random
+    (RT_HIP_SYNTHETIC_WEIGHTS): the run measures time per image, not accuracy.  The reference's published run takes
+    1453.96 s per image on one CPU thread."""
+    exe = os.path.join(ROOT, "oracle", "_ref", "models", "resnet20_cifar10_pre.onnx")
+    if not os.path.exists(exe):
+        return {"resnet20": {"skipped": "the model binary is built only where the reference tree is present"}}
+    try:
+        env = dict(os.environ, RT_HIP_SYNTHETIC_WEIGHTS="0.05")
+        r = subprocess.run([exe, "3", "32", "32", "10", "1"], capture_output=True, text=True, timeout=400, env=env)
+        line = [l for l in r.stdout.splitlines() if l.startswith("context_s")][0].split()
+        vals = dict(zip(line[0::2], (float(v) for v in line[1::2])))
+        return {"resnet20": {"workload": "ResNet-20 CIFAR-10 inference of one image, the reference's generated program, "
+                                         "synthetic weights and image", "main_graph_s": vals["main_graph_s"],
+                             "keygen_s": vals["keygen_s"], "input_s": vals["input_s"], "output_s": vals["output_s"],
+                             "exit_status": r.returncode, "published_cpu_s": 1453.96,
+                             "vs_published_cpu": round(1453.96 / vals["main_graph_s"], 1)}}
+    except Exception as e:
+        return {"resnet20": {"error": repr(e)[:200]}}
+
+
 def extra_legs(g, np, seeded, which="all"):
     level = g.L
     swk = g.upload(np.concatenate([seeded.uniform_poly(2000 + i, g.primes, N) for i in range(2 * g.parts)]))
@@ -247,6 +270,7 @@ def main():
     extra = {} if args.no_extra else extra_legs(g, np, seeded)
     if not args.no_extra:
         extra.update(bootstrap_leg())
+        extra.update(resnet20_leg())
 
     cpu = cpu_baseline(x_host, idx, args.cpu_seconds) if args.cpu_seconds > 0 else None
 

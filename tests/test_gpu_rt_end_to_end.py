@@ -115,3 +115,21 @@ def test_bootstrap_refreshes_levels(args, env):
     print("running bootstrap_program", args, env, flush=True)
     r = subprocess.run([BOOTSTRAP] + args.split(), capture_output=True, text=True, timeout=110, env=e)
     assert r.returncode == 0, r.stdout + r.stderr
+
+
+RESNET20 = os.path.join(rt_program.ROOT, "oracle", "_ref", "models", "resnet20_cifar10_pre.onnx")
+
+
+def test_reference_resnet20_program_runs():
+    """The compiler's ResNet-20 program (7000 lines of generated C at N=65536, 34 limbs, 197 rotation keys, 19
+    bootstraps, 1038 weight plaintexts encoded on the fly), unchanged, to the end.  The weight file is not part of the
+    reference tree, so the weights are pseudo-random and only completion and finite outputs are checked; the
+    operators it is made of are checked with expected values by the reference's examples above."""
+    if not os.path.exists(RESNET20):
+        pytest.skip("built only where the reference tree is present")
+    env = dict(os.environ, RT_HIP_SYNTHETIC_WEIGHTS="0.05")
+    print("running", RESNET20, flush=True)
+    r = subprocess.run([RESNET20, "3", "32", "32", "10", "1"], capture_output=True, text=True, timeout=230, env=env)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    out = [l for l in r.stdout.splitlines() if l.startswith("output:")][0].split()[1:]
+    assert len(out) == 10 and all(v == v and abs(v) != float("inf") for v in map(float, out))
