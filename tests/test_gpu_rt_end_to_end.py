@@ -133,3 +133,39 @@ def test_reference_resnet20_program_runs():
     assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
     out = [l for l in r.stdout.splitlines() if l.startswith("output:")][0].split()[1:]
     assert len(out) == 10 and all(v == v and abs(v) != float("inf") for v in map(float, out))
+
+
+MSG = os.path.join(rt_program.ROOT, "tests", "programs", "msg_program")
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f64"])
+def test_plaintexts_from_a_weight_file(dtype, tmp_path):
+    """Pt_from_msg / Pt_from_msg_ofst read the right entry of a side-file and encode it like Encode_float."""
+    import numpy as np
+
+    import msgfile
+    from oracle_lib import Oracle
+
+    assert os.path.exists(MSG), "tests/programs/msg_program is not built"
+    cfg, level = (4096, 4, 60, 50, 2), 3
+    N = cfg[0]
+    rng = np.random.Generator(np.random.PCG64(31))
+    np_type = np.float32 if dtype == "f32" else np.float64
+    entries = [("w%d" % i, rng.uniform(-1, 1, n).astype(np_type), 1, level) for i, n in enumerate((5, 2048, 77, 1000))]
+    path, out_path = str(tmp_path / "weights.msg"), str(tmp_path / "out.bin")
+    msgfile.write(path, entries, np_type)
+    picks = [(1, 0, 2048), (3, 0, 900), (2, 10, 60), (0, 0, 5)]
+    args = [MSG, path, str(N), str(cfg[1] - 1), str(cfg[2]), str(cfg[3]), str(cfg[4]), str(level), out_path]
+    for p in picks:
+        args += [str(v) for v in p]
+    r = run(args, 0)
+    assert r.returncode == 0, r.stdout + r.stderr
+    got = np.fromfile(out_path, np.int64).reshape(len(picks), level * N)
+    o = Oracle(*cfg)
+    for row, (index, ofst, n) in zip(got, picks):
+        values = np.asarray(entries[index][1][ofst:ofst + n], np.float64).astype(np.complex128)
+        assert np.array_equal(row, o.encode(values, 0, level, 1)), (index, ofst, n)
+    o.close()
+    if dtype == "f32":  # an index past the table is refused the way the reference refuses it
+        bad = run(args[:9] + ["9", "0", "4"], 0)
+        assert bad.returncode != 0 and "index out of entry range" in bad.stderr

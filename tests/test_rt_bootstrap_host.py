@@ -78,3 +78,25 @@ def test_series_division_is_chebyshev_division(lib, nf, ng, seed):
         assert r.size < ng or ng == 1
     else:
         assert np.array_equal(r, f) and q.size == 1 and q[0] == 0
+
+
+def test_side_file_reader_takes_the_reference_s_own_file(lib):
+    """The one weight side-file in the reference tree (rtlib/ant/dataset/bootstrap_full_data.msg: a header and an
+    empty table, kept under tests/golden) opens; a file written by tests/msgfile.py has the same header layout."""
+    import msgfile
+
+    path = os.path.join(rt_program.ROOT, "tests", "golden", "bootstrap_full_data.msg")
+    raw = open(path, "rb").read()
+    assert len(raw) == 136 and raw[:8] == b"!ANTFHE\0"
+    lib.Pt_mgr_init.restype = C.c_bool
+    assert lib.Pt_mgr_init(path.encode())
+    lib.Pt_mgr_fini()
+    import tempfile
+    with tempfile.TemporaryDirectory() as d:
+        mine = os.path.join(d, "empty.msg")
+        msgfile.write(mine, [])
+        got = open(mine, "rb").read()
+        # identical but for the creation time and the model name
+        assert got[:32] == raw[:32] and got[96:136] == raw[96:136] and len(got) == 4096
+        assert lib.Pt_mgr_init(mine.encode())
+        lib.Pt_mgr_fini()
