@@ -590,6 +590,42 @@ double* Get_msg_from_plain(PLAIN plain) {
   return data;
 }
 
+/* ---- runtime validation aids (ckks/src/cipher.c:188-240, common/src/rt_validate.c:16-55) ------------- */
+DCMPLX* Get_msg_with_imag(CIPHER c) {
+  FMT_ASSERT(c->_c0_poly._num_primes_p == 0, "Get_msg: extended ciphertexts are not supported");
+  PLAINTEXT pt;
+  memset(&pt, 0, sizeof(pt));
+  Rt_decrypt(&pt, c);
+  DCMPLX* v = Get_dcmplx_msg_from_plain(&pt);
+  Free_plain_poly(&pt);
+  return v;
+}
+double* Get_msg(CIPHER c) {
+  uint32_t slots = c->_slots ? c->_slots : G.N / 2;
+  DCMPLX*  v     = Get_msg_with_imag(c);
+  double*  r     = (double*)malloc(slots * sizeof(double));
+  for (uint32_t i = 0; i < slots; ++i) r[i] = creal(v[i]);
+  free(v);
+  return r;
+}
+void Print_cipher_msg(FILE* fp, const char* name, CIPHER c, uint32_t len) {
+  double* m = Get_msg(c);
+  fprintf(fp, "[%s] level %zu, sf_degree %u: {", name, Level(c), c->_sf_degree);
+  for (uint32_t i = 0; i < len; ++i) fprintf(fp, " %g", m[i]);
+  fprintf(fp, " }\n");
+  free(m);
+}
+void Validate_impl(double* res, double* msg, uint32_t len, int32_t epsilon) {
+  double error = pow(10, epsilon);
+  for (uint32_t i = 0; i < len; ++i)
+    if (fabs(res[i] - msg[i]) > error) Rt_fatal(__FILE__, __LINE__, "ERROR: validation failed at %u. %f != %f", i, res[i], msg[i]);
+}
+void Validate(CIPHER c, double* msg, uint32_t len, int32_t epsilon) {
+  double* res = Get_msg(c);
+  Validate_impl(res, msg, len, epsilon);
+  free(res);
+}
+
 /* ---- tensors, program inputs and outputs (common/tensor.h, ckks/src/rtlib.c:66-229) ---------------- */
 TENSOR* Alloc_tensor(size_t n, size_t c, size_t h, size_t w, const double* val) {
   size_t  len = n * c * h * w;

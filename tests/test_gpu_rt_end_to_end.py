@@ -38,6 +38,8 @@ def test_gemm_square_program(degree, dim):
     assert "max_err" in r.stdout
 
 
+# eg_fhertlib_mul_const_rtv builds and links too, but cannot pass anywhere: it multiplies the message 20 at scale 2^30
+# by a plaintext at scale 2^30 under a 63-bit modulus (20 * 2^60 > Q) and validates the wrapped value.
 @pytest.mark.parametrize("name", EXAMPLES)
 def test_reference_example(name):
     exe = os.path.join(EXAMPLES_DIR, "eg_fhertlib_" + name)

@@ -29,7 +29,9 @@ def test_library_exports():
                  "Handle_output Encode_float Encode_double Encode_dcmplx Encode_dcmplx_ext Encode_float_mask "
                  "Encode_double_mask Encode_single_float Encode_single_double Get_msg_from_plain "
                  "Get_dcmplx_msg_from_plain Free_plain_poly Init_ciph_same_scale_plain Init_ciph_up_scale_plain "
-                 "Add_plain Mul_plain Alloc_tensor Free_tensor Print_tensor Bootstrap Eval_bootstrap_ciph Mul_mono_ciph").split():
+                 "Add_plain Mul_plain Alloc_tensor Free_tensor Print_tensor Bootstrap Eval_bootstrap_ciph Mul_mono_ciph "
+                 "Pt_mgr_init Pt_mgr_fini Pt_from_msg Pt_from_msg_ofst Pt_from_msg_validate Pt_from_msg_ofst_validate "
+                 "Free_data Rt_sync").split():
         assert hasattr(lib, name), name
 
 
