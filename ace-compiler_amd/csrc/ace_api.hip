@@ -3,11 +3,14 @@
 // reference operation.  One HIP stream per context; every call only enqueues.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <map>
+#include <set>
+#include <unordered_set>
 #include <memory>
 #include <stdexcept>
 #include <string>
@@ -63,6 +66,15 @@ struct RescaleDev {
 
 }  // namespace
 
+// Hw_* calls recorded for one launch (see flush_pending)
+struct PendingRun {
+  std::vector<BatchOp> ops;
+  u64 n = 0;                                  // words per operand, the same for the whole run
+  std::set<uintptr_t> touched;                // start of every operand and result of the run
+  std::unordered_set<uintptr_t> written;      // starts written by elementwise entries
+  std::unordered_set<uintptr_t> rot_res, rot_src;  // results / sources (and index tables) of rotates
+};
+
 struct ace_ctx {
   HostContext h;
   bool device_ok = false;  // false: host tables only (no GPU present), every compute call is rejected
@@ -70,6 +82,45 @@ struct ace_ctx {
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   DevCtx d{};
   std::vector<void*> owned;  // device allocations freed with the context
+  // host-to-device copies of small host arrays whose lifetime ends with the call: staged through pinned
+  // buffers that are reused only after the copy out of them has finished
+  struct Stage {
+    void* host = nullptr;
+    size_t cap = 0;
+    hipEvent_t done = nullptr;
+    bool pending = false;
+  };
+  static constexpr int kStages = 16;
+  Stage stages[kStages];
+  int next_stage = 0;
+  void h2d(void* dev_dst, const void* src, size_t bytes) {
+    if (!bytes) return;
+    Stage& st = stages[next_stage];
+    next_stage = (next_stage + 1) % kStages;
+    if (st.pending) {
+      HIP_OK(hipEventSynchronize(st.done));
+      st.pending = false;
+    }
+    if (st.cap < bytes) {
+      if (st.host) HIP_OK(hipHostFree(st.host));
+      st.host = nullptr;
+      st.cap = std::max<size_t>(bytes, 64 * 1024);
+      HIP_OK(hipHostMalloc(&st.host, st.cap, hipHostMallocDefault));
+    }
+    if (!st.done) HIP_OK(hipEventCreateWithFlags(&st.done, hipEventDisableTiming));
+    std::memcpy(st.host, src, bytes);
+    HIP_OK(hipMemcpyAsync(dev_dst, st.host, bytes, hipMemcpyHostToDevice, stream));
+    HIP_OK(hipEventRecord(st.done, stream));
+    st.pending = true;
+  }
+  PendingRun run;
+  bool batching = true;      // record Hw_* calls and launch them together
+  BatchOp* run_dev = nullptr;
+  u32* run_chain_dev = nullptr;
+  static constexpr size_t kMaxRun = 2048;
+  void flush_pending();
+  bool run_accepts(const BatchOp& o, u64 n) const;
+  void run_append(const BatchOp& o, u64 n);
   std::map<std::pair<size_t, size_t>, ModUpDev> modup;
   std::map<size_t, RescaleDev> rescale;
   std::map<size_t, PrecompDev> precomp;
@@ -370,7 +421,15 @@ struct ace_ctx {
   }
 
   ~ace_ctx() {
+    try {
+      flush_pending();
+    } catch (...) {
+    }
     if (stream) (void)hipStreamSynchronize(stream);
+    for (Stage& st : stages) {
+      if (st.host) (void)hipHostFree(st.host);
+      if (st.done) (void)hipEventDestroy(st.done);
+    }
     for (void* p : owned) (void)hipFree(p);
     drop_pool();
     if (ws) (void)hipFree(ws);
@@ -379,6 +438,122 @@ struct ace_ctx {
     if (stream) (void)hipStreamDestroy(stream);
   }
 };
+
+// ---- recorded Hw_* calls --------------------------------------------------------------------------
+// A run is launched as one kernel in which the thread of element i carries out its chain's entries in order.
+// That equals issuing the calls one by one as long as (1) ranges that overlap are the same range, so element i
+// of one entry is element i of the other, and (2) a rotate, which reads other elements than its own, neither
+// reads nor overwrites anything else the run touches.  An entry that would break this starts a new run.
+bool ace_ctx::run_accepts(const BatchOp& o, u64 n) const {
+  if (run.ops.empty()) return true;
+  if (n != run.n || run.ops.size() >= kMaxRun) return false;
+  const uintptr_t bytes = (uintptr_t)n * sizeof(u64);
+  auto misaligned = [&](const void* p) {  // overlaps a range of the run without being that range
+    const uintptr_t x = (uintptr_t)p;
+    auto it = run.touched.lower_bound(x);
+    if (it != run.touched.end() && *it != x && *it - x < bytes) return true;
+    if (it != run.touched.begin()) {
+      --it;
+      if (*it != x && x - *it < bytes) return true;
+    }
+    return false;
+  };
+  const bool rotate = o.op == BATCH_ROTATE;
+  const uintptr_t r = (uintptr_t)o.r, a = (uintptr_t)o.a, b = (uintptr_t)o.b;
+  if (misaligned(o.r) || misaligned(o.a) || (o.b && misaligned(o.b))) return false;
+  if (rotate) {
+    if (run.touched.count(r)) return false;                       // its result is anything the run used
+    if (run.written.count(a) || run.rot_res.count(a)) return false;  // its source or table was written by the run
+    if (run.written.count(b) || run.rot_res.count(b)) return false;
+    return true;
+  }
+  // an elementwise entry may not read a rotate's result (other threads wrote it) nor overwrite its sources
+  if (run.rot_res.count(a) || (o.b && run.rot_res.count(b)) || run.rot_res.count(r)) return false;
+  if (run.rot_src.count(r)) return false;
+  return true;
+}
+
+void ace_ctx::run_append(const BatchOp& o, u64 n) {
+  if (!run_accepts(o, n)) flush_pending();
+  run.n = n;
+  run.ops.push_back(o);
+  run.touched.insert((uintptr_t)o.r);
+  run.touched.insert((uintptr_t)o.a);
+  if (o.b) run.touched.insert((uintptr_t)o.b);
+  if (o.op == BATCH_ROTATE) {
+    run.rot_res.insert((uintptr_t)o.r);
+    run.rot_src.insert((uintptr_t)o.a);
+    run.rot_src.insert((uintptr_t)o.b);
+  } else {
+    run.written.insert((uintptr_t)o.r);
+  }
+}
+
+void ace_ctx::flush_pending() {
+  if (run.ops.empty()) return;
+  const size_t count = run.ops.size();
+  // chains: entries joined whenever one writes a range the other reads or writes (union-find over entries)
+  std::vector<u32> parent(count);
+  for (u32 k = 0; k < count; ++k) parent[k] = k;
+  auto find = [&](u32 x) {
+    while (parent[x] != x) x = parent[x] = parent[parent[x]];
+    return x;
+  };
+  auto join = [&](u32 x, u32 y) {
+    x = find(x), y = find(y);
+    if (x != y) parent[std::max(x, y)] = std::min(x, y);
+  };
+  std::unordered_map<uintptr_t, u32> writer;                // last entry that wrote the range
+  std::unordered_map<uintptr_t, std::vector<u32>> readers;  // entries that read it since
+  for (u32 k = 0; k < count; ++k) {
+    const BatchOp& o = run.ops[k];
+    const bool rotate = o.op == BATCH_ROTATE;
+    const uintptr_t reads[3] = {(uintptr_t)o.a, rotate ? 0 : (uintptr_t)o.b,
+                                (o.op == EW_MULADD || o.op == EW_MULADD_S) ? (uintptr_t)o.r : 0};
+    for (uintptr_t x : reads) {
+      if (!x) continue;
+      auto w = writer.find(x);
+      if (w != writer.end()) join(k, w->second);
+      readers[x].push_back(k);
+    }
+    const uintptr_t r = (uintptr_t)o.r;
+    auto w = writer.find(r);
+    if (w != writer.end()) join(k, w->second);
+    auto rd = readers.find(r);
+    if (rd != readers.end()) {
+      for (u32 j : rd->second) join(k, j);
+      rd->second.clear();
+    }
+    writer[r] = k;
+  }
+  // entries sorted by chain, order inside a chain kept
+  std::vector<u32> order(count);
+  for (u32 k = 0; k < count; ++k) order[k] = k;
+  std::stable_sort(order.begin(), order.end(), [&](u32 x, u32 y) { return find(x) < find(y); });
+  std::vector<BatchOp> sorted(count);
+  std::vector<u32> chain_start;
+  for (u32 k = 0; k < count; ++k) {
+    if (k == 0 || find(order[k]) != find(order[k - 1])) chain_start.push_back(k);
+    sorted[k] = run.ops[order[k]];
+  }
+  const u32 n_chains = (u32)chain_start.size();
+  chain_start.push_back((u32)count);
+  const u64 n = run.n;
+  run.ops.clear();
+  run.touched.clear();
+  run.written.clear();
+  run.rot_res.clear();
+  run.rot_src.clear();
+  if (!run_dev) {
+    HIP_OK(hipMalloc((void**)&run_dev, kMaxRun * sizeof(BatchOp)));
+    owned.push_back(run_dev);
+    HIP_OK(hipMalloc((void**)&run_chain_dev, (kMaxRun + 1) * sizeof(u32)));
+    owned.push_back(run_chain_dev);
+  }
+  h2d(run_dev, sorted.data(), count * sizeof(BatchOp));
+  h2d(run_chain_dev, chain_start.data(), chain_start.size() * sizeof(u32));
+  launch_ew_batch(stream, d, run_dev, run_chain_dev, n_chains, n);
+}
 
 namespace {
 
@@ -638,9 +813,10 @@ void do_mul_relin_rescale(ace_ctx* c, u64* r0, u64* r1, u64 out_stride, const u6
 // ===========================================================================
 extern "C" {
 
-#define ACE_TRY try {                                                          \
+#define ACE_TRY_KEEP_RUN try {                                                 \
   if (!c) return fail("null context");                                         \
   if (!c->device_ok) return fail("no HIP device: this context holds host tables only");
+#define ACE_TRY ACE_TRY_KEEP_RUN c->flush_pending();
 #define ACE_CATCH_INT                      \
   }                                        \
   catch (const std::exception& e) {        \
@@ -750,6 +926,11 @@ void ace_free(ace_ctx* c, int64_t* p) {
   if (!p || !c || !c->device_ok) return;
   auto it = c->live.find(p);
   if (it == c->live.end()) return;  // not from ace_alloc of this context (a view, or freed twice)
+  try {
+    c->flush_pending();  // recorded calls may still name this buffer
+  } catch (const std::exception& e) {
+    (void)fail(e.what());
+  }
   const size_t words = it->second;
   c->live.erase(it);
   if (c->pooled_words + words <= ace_ctx::kPoolLimitWords) {
@@ -795,6 +976,7 @@ int ace_timer_start(ace_ctx* c) {
 float ace_timer_stop_ms(ace_ctx* c) {
   try {
     if (!c || !c->device_ok) throw std::runtime_error("no HIP device");
+    c->flush_pending();
     HIP_OK(hipEventRecord(c->ev1, c->stream));
     HIP_OK(hipEventSynchronize(c->ev1));
     float ms = 0;
@@ -845,12 +1027,16 @@ int ace_ntt_pass(ace_ctx* c, int64_t* dst, const int64_t* src, const int32_t* pr
 // ---- Hw_* ---------------------------------------------------------------------
 static int hw_common(ace_ctx* c, EwOp op, int64_t* r, const int64_t* a, const int64_t* b, int64_t s, size_t pi,
                      size_t n) {
-  ACE_TRY
+  ACE_TRY_KEEP_RUN
   if (n == 0) return 0;
   if (!r || !a || (op < EW_ADD_S && !b)) return fail("ace_hw: null argument");
   if (pi >= c->h.L + c->h.K) return fail("ace_hw: prime index out of range");
   if ((op == EW_MUL_S || op == EW_MULADD_S) && (s < 0 || (u64)s >= c->h.primes[pi].q))
     return fail("ace_hw: scalar multiplier must be a residue in [0, q)");
+  if (c->batching) {
+    c->run_append(BatchOp{U(r), U(a), U(b), (u64)s, (u32)op, (u32)pi}, n);
+    return 0;
+  }
   LimbMap lm{};
   lm.prime[0] = (uint8_t)pi;
   launch_ew(c->stream, c->d, op, U(r), U(a), U(b), (u64)s, lm, 1, n);
@@ -866,14 +1052,24 @@ int ace_hw_modmul_scalar(ace_ctx* c, int64_t* r, const int64_t* a, int64_t s, si
 int ace_hw_modmuladd_scalar(ace_ctx* c, int64_t* r, const int64_t* a, int64_t s, size_t pi, size_t n) { return hw_common(c, EW_MULADD_S, r, a, nullptr, s, pi, n); }
 
 int ace_hw_rotate(ace_ctx* c, int64_t* r, const int64_t* a, const int64_t* order, size_t pi, size_t n) {
-  ACE_TRY
+  ACE_TRY_KEEP_RUN
   if (n == 0) return 0;
   if (!r || !a || !order) return fail("ace_hw_rotate: null argument");
   if (r == a) return fail("ace_hw_rotate: in-place gather is not supported");
   if (pi >= c->h.L + c->h.K) return fail("ace_hw_rotate: prime index out of range");
+  if (c->batching) {
+    c->run_append(BatchOp{U(r), U(a), reinterpret_cast<const u64*>(order), 0, (u32)BATCH_ROTATE, (u32)pi}, n);
+    return 0;
+  }
   LimbMap lm{};
   lm.prime[0] = (uint8_t)pi;
   launch_gather(c->stream, c->d, U(r), U(a), order, lm, 1, n);
+  ACE_CATCH_INT
+}
+
+int ace_set_batching(ace_ctx* c, int on) {
+  ACE_TRY
+  c->batching = on != 0;
   ACE_CATCH_INT
 }
 
@@ -945,7 +1141,7 @@ int ace_automorphism_order(ace_ctx* c, int64_t* dev_order, uint32_t k, int is_nt
   if (!(k & 1) || k >= 2 * c->h.N) return fail("ace_automorphism_order: index must be odd and below 2N");
   std::vector<i64> ord(c->h.N);
   automorphism_order(ord.data(), k, c->h.N, is_ntt != 0);
-  HIP_OK(hipMemcpyAsync(dev_order, ord.data(), ord.size() * sizeof(i64), hipMemcpyHostToDevice, c->stream));
+  c->h2d(dev_order, ord.data(), ord.size() * sizeof(i64));
   HIP_OK(hipStreamSynchronize(c->stream));
   ACE_CATCH_INT
 }
@@ -1023,7 +1219,7 @@ int ace_ciph_wsum(ace_ctx* c, int64_t* r0, int64_t* r1, const int64_t* const* a0
   c->ensure_ws(count * level);
   c->ws_used = 0;
   u64* w = c->take(count * level);
-  HIP_OK(hipMemcpyAsync(w, weights, count * level * sizeof(u64), hipMemcpyHostToDevice, c->stream));
+  c->h2d(w, weights, count * level * sizeof(u64));
   launch_wsum(c->stream, c->d, U(r0), U(r1), ops, w, poly_lm(c, level, false), (u32)level, c->h.N);
   ACE_CATCH_INT
 }
@@ -1171,7 +1367,7 @@ int ace_encode(ace_ctx* c, int64_t* res, const double* values, size_t n_values, 
   double2* z = reinterpret_cast<double2*>(c->take(2 * (size_t)slots));
   launch_fill_zero(c->stream, reinterpret_cast<u64*>(z), 2 * (size_t)slots);
   if (n_values)
-    HIP_OK(hipMemcpyAsync(z, values, n_values * sizeof(double2), hipMemcpyHostToDevice, c->stream));
+    c->h2d(z, values, n_values * sizeof(double2));
   LimbMap lm = poly_lm(c, level, p_cnt != 0);
   const u32 n_limbs = (u32)(level + p_cnt);
   launch_encode(c->stream, c->d, U(res), z, c->fft_rou, c->rot_group, slots, scaling_factor, scale, range_bound, lm,
@@ -1185,7 +1381,7 @@ int ace_encode(ace_ctx* c, int64_t* res, const double* values, size_t n_values, 
       cst[2 * t + 1] = shoup(powp, q);
     }
     u64* dc = c->take(2 * level);
-    HIP_OK(hipMemcpyAsync(dc, cst.data(), cst.size() * sizeof(u64), hipMemcpyHostToDevice, c->stream));
+    c->h2d(dc, cst.data(), cst.size() * sizeof(u64));
     HIP_OK(hipStreamSynchronize(c->stream));  // cst is a local
     launch_mul_const(c->stream, c->d, U(res), U(res), dc, c->q_lm, (u32)level);
   }

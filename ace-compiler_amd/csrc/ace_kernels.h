@@ -66,6 +66,18 @@ struct MacSet { // operands of one multiply-accumulate launch
 // at plain_level + (t - level) above it
 void launch_plain_mac(hipStream_t st, const DevCtx& c, u64* r0, u64* r1, const MacSet& ops, const LimbMap& lm,
                       u32 n_limbs, u32 level, u32 plain_level, bool accumulate, u64 n);
+// a run of Hw_* calls executed as one launch: thread i carries out every entry for element i, in order
+enum BatchKind : u32 { BATCH_ROTATE = 100 };
+struct BatchOp {
+  u64* r;
+  const u64* a;
+  const u64* b;  // second operand, or the index table of a rotate
+  u64 scalar;
+  u32 op;        // an EwOp, or BATCH_ROTATE
+  u32 prime;
+};
+// chain y (blockIdx.y) is the entries [chain_start[y], chain_start[y+1]): chains share no written range, so they run side by side
+void launch_ew_batch(hipStream_t st, const DevCtx& c, const BatchOp* dev_ops, const u32* dev_chain_start, u32 n_chains, u64 n);
 struct LimbScalars { // one residue per limb
   u64 v[kMaxPrimes];
 };

@@ -85,6 +85,38 @@ void launch_plain_mac(hipStream_t st, const DevCtx& c, u64* r0, u64* r1, const M
                      plain_level, accumulate ? 1 : 0, n);
 }
 
+// ---- a recorded run of Hw_* calls (hal/src/hal.c:15-138) in one launch --------------------------------
+// The host splits a run into chains that share no written range; a chain's entries are carried out in order by
+// the thread of element i, so an entry may read what an earlier one of its chain wrote (identical ranges only;
+// a rotate never reads or overwrites anything the run touches).
+__global__ __launch_bounds__(kThreads) void ew_batch_kernel(DevCtx c, const BatchOp* ops, const u32* chain_start, u64 n) {
+  const u32 first = chain_start[blockIdx.y], last = chain_start[blockIdx.y + 1];
+  const u64 i = (u64)blockIdx.x * kThreads + threadIdx.x;
+  if (i >= n) return;
+  for (u32 k = first; k < last; ++k) {
+    const BatchOp o = ops[k];
+    const DevPrime P = c.primes[o.prime];
+    u64 v;
+    if (o.op == BATCH_ROTATE) {
+      const i64 src = reinterpret_cast<const i64*>(o.b)[i];
+      v = src >= 0 ? o.a[src] : P.q - o.a[-src];
+    } else {
+      const u64 x = o.a[i];
+      const u64 y = o.op >= EW_ADD_S ? o.scalar : o.b[i];
+      if (o.op == EW_ADD || o.op == EW_ADD_S) v = add_mod(x, y, P.q);
+      else if (o.op == EW_SUB || o.op == EW_SUB_S) v = sub_mod(x, y, P.q);
+      else if (o.op == EW_MUL || o.op == EW_MUL_S) v = mulmod(x, y, P);
+      else v = add_mod(o.r[i], mulmod(x, y, P), P.q);
+    }
+    o.r[i] = v;
+  }
+}
+void launch_ew_batch(hipStream_t st, const DevCtx& c, const BatchOp* dev_ops, const u32* dev_chain_start, u32 n_chains, u64 n) {
+  if (!n || !n_chains) return;
+  dim3 g((unsigned)((n + kThreads - 1) / kThreads), n_chains, 1);
+  hipLaunchKernelGGL(ew_batch_kernel, g, dim3(kThreads), 0, st, c, dev_ops, dev_chain_start, n);
+}
+
 // ---- per-limb scalars: Scalars_integer_add_poly / Scalars_integer_multiply_poly (poly/src/rns_poly.c) ----
 template <int MUL>
 __global__ __launch_bounds__(kThreads) void limb_scalar_kernel(DevCtx c, u64* __restrict__ r, const u64* __restrict__ a,

@@ -124,6 +124,10 @@ int ace_hw_modadd_scalar(ace_ctx* ctx, int64_t* res, const int64_t* a, int64_t s
 int ace_hw_modsub_scalar(ace_ctx* ctx, int64_t* res, const int64_t* a, int64_t s, size_t prime_idx, size_t n);
 int ace_hw_modmul_scalar(ace_ctx* ctx, int64_t* res, const int64_t* a, int64_t s, size_t prime_idx, size_t n);
 int ace_hw_modmuladd_scalar(ace_ctx* ctx, int64_t* res, const int64_t* a, int64_t s, size_t prime_idx, size_t n);
+/* Consecutive ace_hw_* calls are recorded and launched together (one kernel for a run of calls instead of one
+ * each: generated code issues them limb by limb); every other entry point launches what is pending first, so
+ * results are those of issuing the calls one by one.  ace_set_batching(ctx, 0) launches each call on its own. */
+int ace_set_batching(ace_ctx* ctx, int on);
 /* Hw_rotate: res[i] = order[i] >= 0 ? a[order[i]] : q - a[-order[i]]; order is a device table */
 int ace_hw_rotate(ace_ctx* ctx, int64_t* res, const int64_t* a, const int64_t* order, size_t prime_idx, size_t n);
 

@@ -513,3 +513,52 @@ def test_limb_scalars_and_weighted_sum(pair):
     g.ciph_wsum(d0[0], d1[0], d0, d1, w, level)  # the result over the first operand
     eq(d0[0].get(), wsum(a0), "ciph_wsum c0 over an operand")
     eq(d1[0].get(), wsum(a1), "ciph_wsum c1 over an operand")
+
+
+def test_recorded_hw_calls_equal_calls_issued_one_by_one(pair):
+    """Hw_* calls are recorded and launched together; a random program of them (shared temporaries, in-place updates,
+    rotates of freshly written limbs, operands that overlap out of step) must give what one launch per call gives."""
+    g = pair.g
+    N, L = g.N, g.L
+    if N > 8192:
+        pytest.skip("covered at the smaller rings")
+    rng = np.random.Generator(np.random.PCG64(5 + N))
+    n_limbs = 12
+    prime = [int(rng.integers(0, L + g.K)) for _ in range(n_limbs)]
+    host = np.concatenate([seeded.uniform_poly(6000 + t, [g.primes[prime[t]]], N) for t in range(n_limbs)])
+    k = g.find_automorphism_index(1)
+    order = g.automorphism_order(k, True)
+
+    def program(buf):
+        limb = lambda t: buf.view(t * N, N)
+        r = np.random.Generator(np.random.PCG64(99))
+        for step in range(400):
+            kind = int(r.integers(0, 10))
+            t = int(r.integers(0, n_limbs))
+            same = [u for u in range(n_limbs) if prime[u] == prime[t]]
+            a, b, d = (int(r.choice(same)) for _ in range(3))
+            p = prime[t]
+            if kind < 3:
+                g.hw("modmul", limb(d), limb(a), limb(b), p)
+            elif kind < 5:
+                g.hw("modmuladd", limb(d), limb(a), limb(b), p)
+            elif kind < 6:
+                g.hw("modadd", limb(d), limb(d), limb(a), p)
+            elif kind < 7:
+                g.hw("modsub_scalar", limb(d), limb(a), int(r.integers(0, 1 << 30)), p)
+            elif kind < 9:
+                if d != a:
+                    g.hw("rotate", limb(d), limb(a), order, p)
+            elif t + 1 < n_limbs and d not in (t, t + 1):
+                # an operand one word out of step with limbs the run has just written: element i of it is element
+                # i+1 of limb t, which another thread wrote (values need not be reduced for an addition's operand
+                # to be read consistently, only the same words must be seen)
+                g.hw("modadd", limb(d), limb(d), buf.view(t * N + 1, N), prime[d])
+    g.set_batching(False)
+    x = g.upload(host)
+    program(x)
+    want = x.get()
+    g.set_batching(True)
+    y = g.upload(host)
+    program(y)
+    eq(y.get(), want, "recorded run")
