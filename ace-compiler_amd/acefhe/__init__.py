@@ -95,12 +95,14 @@ def _sig(lib):
     f("ace_ciph_wsum", C.c_int, _vp, _vp, _vp, C.POINTER(_vp), C.POINTER(_vp), _i64p, _sz, _sz)
     f("ace_alloc_uninit", _vp, _vp, _sz)
     f("ace_set_batching", C.c_int, _vp, C.c_int)
+    f("ace_sample_uniform", C.c_int, _vp, _vp, _sz, C.c_int, C.c_uint64, C.c_uint64)
+    f("ace_expand_small", C.c_int, _vp, _vp, _i64p, _sz, C.c_int)
     f("ace_ext_plain_mac", C.c_int, _vp, _vp, _vp, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp), _sz, _sz, _sz, C.c_int)
 
 
 # every symbol include/ace_hip.h declares
 EXPORTS = [
-    "ace_set_batching", "ace_ext_plain_mac", "ace_poly_add_scalars", "ace_poly_mul_scalars", "ace_ciph_wsum", "ace_alloc_uninit", "ace_ctx_create", "ace_ctx_create_with_primes", "ace_ctx_destroy", "ace_has_device", "ace_last_error",
+    "ace_sample_uniform", "ace_expand_small", "ace_set_batching", "ace_ext_plain_mac", "ace_poly_add_scalars", "ace_poly_mul_scalars", "ace_ciph_wsum", "ace_alloc_uninit", "ace_ctx_create", "ace_ctx_create_with_primes", "ace_ctx_destroy", "ace_has_device", "ace_last_error",
     "ace_degree", "ace_num_q", "ace_num_p", "ace_num_parts", "ace_part_size", "ace_num_decomp", "ace_prime",
     "ace_root", "ace_modulus", "ace_host_twiddles", "ace_host_tbl_modup", "ace_host_tbl_moddown",
     "ace_host_tbl_rescale", "ace_host_automorphism_order", "ace_alloc", "ace_free", "ace_upload", "ace_download",
@@ -379,6 +381,14 @@ class Context:
         p0 = (_vp * n)(*[a.ptr for a in a0s])
         p1 = (_vp * n)(*[a.ptr for a in a1s])
         self._chk(self.lib.ace_ciph_wsum(self.h, r0.ptr, r1.ptr, p0, p1, w.ctypes.data_as(_i64p), n, level))
+
+    def sample_uniform(self, r, level, with_p, seed, stream):
+        self._chk(self.lib.ace_sample_uniform(self.h, r.ptr, level, int(with_p), seed, stream))
+
+    def expand_small(self, r, small, level, with_p):
+        v = np.ascontiguousarray(small, dtype=np.int64)
+        assert v.size == self.N
+        self._chk(self.lib.ace_expand_small(self.h, r.ptr, v.ctypes.data_as(_i64p), level, int(with_p)))
 
     def set_batching(self, on):
         self._chk(self.lib.ace_set_batching(self.h, int(bool(on))))

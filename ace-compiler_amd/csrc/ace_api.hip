@@ -8,6 +8,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <ctime>
 #include <map>
 #include <set>
 #include <unordered_set>
@@ -460,7 +461,7 @@ bool ace_ctx::run_accepts(const BatchOp& o, u64 n) const {
   };
   const bool rotate = o.op == BATCH_ROTATE;
   const uintptr_t r = (uintptr_t)o.r, a = (uintptr_t)o.a, b = (uintptr_t)o.b;
-  if (misaligned(o.r) || misaligned(o.a) || (o.b && misaligned(o.b))) return false;
+  if (misaligned(o.r) || (o.a && misaligned(o.a)) || (o.b && misaligned(o.b))) return false;
   if (rotate) {
     if (run.touched.count(r)) return false;                       // its result is anything the run used
     if (run.written.count(a) || run.rot_res.count(a)) return false;  // its source or table was written by the run
@@ -468,7 +469,7 @@ bool ace_ctx::run_accepts(const BatchOp& o, u64 n) const {
     return true;
   }
   // an elementwise entry may not read a rotate's result (other threads wrote it) nor overwrite its sources
-  if (run.rot_res.count(a) || (o.b && run.rot_res.count(b)) || run.rot_res.count(r)) return false;
+  if ((o.a && run.rot_res.count(a)) || (o.b && run.rot_res.count(b)) || run.rot_res.count(r)) return false;
   if (run.rot_src.count(r)) return false;
   return true;
 }
@@ -478,7 +479,7 @@ void ace_ctx::run_append(const BatchOp& o, u64 n) {
   run.n = n;
   run.ops.push_back(o);
   run.touched.insert((uintptr_t)o.r);
-  run.touched.insert((uintptr_t)o.a);
+  if (o.a) run.touched.insert((uintptr_t)o.a);
   if (o.b) run.touched.insert((uintptr_t)o.b);
   if (o.op == BATCH_ROTATE) {
     run.rot_res.insert((uintptr_t)o.r);
@@ -811,9 +812,45 @@ void do_mul_relin_rescale(ace_ctx* c, u64* r0, u64* r1, u64 out_stride, const u6
 }  // namespace
 
 // ===========================================================================
+// ACE_HIP_PROFILE=1: host time spent inside each entry point, printed when the process ends
+namespace {
+struct HostProf {
+  bool on = false;
+  std::map<std::string, std::pair<u64, double>> t;
+  HostProf() {
+    const char* e = std::getenv("ACE_HIP_PROFILE");
+    on = e && std::atoi(e) != 0;
+  }
+  ~HostProf() {
+    if (!on) return;
+    std::vector<std::pair<double, std::string>> v;
+    for (auto& kv : t) v.push_back({kv.second.second, kv.first});
+    std::sort(v.rbegin(), v.rend());
+    std::fprintf(stderr, "[ace_hip] host time by entry point\n");
+    for (auto& e : v) std::fprintf(stderr, "  %-28s %9llu calls %9.1f ms\n", e.second.c_str(), (unsigned long long)t[e.second].first, e.first * 1e3);
+  }
+};
+HostProf g_prof;
+struct ScopedProf {
+  const char* name;
+  timespec t0;
+  explicit ScopedProf(const char* n) : name(n) {
+    if (g_prof.on) clock_gettime(CLOCK_MONOTONIC, &t0);
+  }
+  ~ScopedProf() {
+    if (!g_prof.on) return;
+    timespec t1;
+    clock_gettime(CLOCK_MONOTONIC, &t1);
+    auto& e = g_prof.t[name];
+    e.first += 1;
+    e.second += (double)(t1.tv_sec - t0.tv_sec) + 1e-9 * (double)(t1.tv_nsec - t0.tv_nsec);
+  }
+};
+}  // namespace
+
 extern "C" {
 
-#define ACE_TRY_KEEP_RUN try {                                                 \
+#define ACE_TRY_KEEP_RUN ScopedProf prof_scope_(__func__); try {                                                 \
   if (!c) return fail("null context");                                         \
   if (!c->device_ok) return fail("no HIP device: this context holds host tables only");
 #define ACE_TRY ACE_TRY_KEEP_RUN c->flush_pending();
@@ -896,6 +933,7 @@ static int64_t* alloc_words(ace_ctx* c, size_t n_words, bool zero);
 int64_t* ace_alloc(ace_ctx* c, size_t n_words) { return alloc_words(c, n_words, true); }
 int64_t* ace_alloc_uninit(ace_ctx* c, size_t n_words) { return alloc_words(c, n_words, false); }
 static int64_t* alloc_words(ace_ctx* c, size_t n_words, bool zero) {
+  ScopedProf prof_scope_("ace_alloc");
   try {
     if (!c || !c->device_ok) throw std::runtime_error("no HIP device: this context holds host tables only");
     const size_t words = std::max<size_t>(n_words, 1);
@@ -923,6 +961,7 @@ static int64_t* alloc_words(ace_ctx* c, size_t n_words, bool zero) {
   }
 }
 void ace_free(ace_ctx* c, int64_t* p) {
+  ScopedProf prof_scope_("ace_free");
   if (!p || !c || !c->device_ok) return;
   auto it = c->live.find(p);
   if (it == c->live.end()) return;  // not from ace_alloc of this context (a view, or freed twice)
@@ -954,12 +993,24 @@ int ace_download(ace_ctx* c, int64_t* dst, const int64_t* src, size_t n) {
   ACE_CATCH_INT
 }
 int ace_copy(ace_ctx* c, int64_t* dst, const int64_t* src, size_t n) {
-  ACE_TRY
-  if (dst != src) HIP_OK(hipMemcpyAsync(dst, src, n * sizeof(u64), hipMemcpyDeviceToDevice, c->stream));
+  ACE_TRY_KEEP_RUN
+  if (!dst || !src) return fail("ace_copy: null argument");
+  if (dst == src || n == 0) return 0;
+  if (c->batching) {  // a copy is an elementwise entry like any other
+    c->run_append(BatchOp{U(dst), U(src), nullptr, 0, (u32)BATCH_COPY, 0}, n);
+    return 0;
+  }
+  HIP_OK(hipMemcpyAsync(dst, src, n * sizeof(u64), hipMemcpyDeviceToDevice, c->stream));
   ACE_CATCH_INT
 }
 int ace_zero(ace_ctx* c, int64_t* dst, size_t n) {
-  ACE_TRY
+  ACE_TRY_KEEP_RUN
+  if (!dst) return fail("ace_zero: null argument");
+  if (n == 0) return 0;
+  if (c->batching) {
+    c->run_append(BatchOp{U(dst), nullptr, nullptr, 0, (u32)BATCH_ZERO, 0}, n);
+    return 0;
+  }
   launch_fill_zero(c->stream, U(dst), n);
   ACE_CATCH_INT
 }
@@ -1199,6 +1250,29 @@ static int poly_scalars(ace_ctx* c, bool mul, int64_t* r, const int64_t* a, cons
 }
 int ace_poly_add_scalars(ace_ctx* c, int64_t* r, const int64_t* a, const int64_t* scalars, size_t level) { return poly_scalars(c, false, r, a, scalars, level); }
 int ace_poly_mul_scalars(ace_ctx* c, int64_t* r, const int64_t* a, const int64_t* scalars, size_t level) { return poly_scalars(c, true, r, a, scalars, level); }
+
+int ace_sample_uniform(ace_ctx* c, int64_t* res, size_t level, int with_p, uint64_t seed, uint64_t stream) {
+  ACE_TRY
+  if (!res) return fail("ace_sample_uniform: null argument");
+  if (!level_ok(c, level)) return fail("ace_sample_uniform: level out of range");
+  launch_sample_uniform(c->stream, c->d, U(res), seed, stream, poly_lm(c, level, with_p != 0),
+                        (u32)(level + (with_p ? c->h.K : 0)), c->h.N);
+  ACE_CATCH_INT
+}
+int ace_expand_small(ace_ctx* c, int64_t* res, const int64_t* small_host, size_t level, int with_p) {
+  ACE_TRY
+  if (!res || !small_host) return fail("ace_expand_small: null argument");
+  if (!level_ok(c, level)) return fail("ace_expand_small: level out of range");
+  for (size_t i = 0; i < c->h.N; ++i)
+    if (small_host[i] > (1 << 30) || small_host[i] < -(1 << 30)) return fail("ace_expand_small: coefficient is not small");
+  c->ensure_ws(c->h.N);
+  c->ws_used = 0;
+  u64* v = c->take(c->h.N);
+  c->h2d(v, small_host, c->h.N * sizeof(i64));
+  launch_expand_small(c->stream, c->d, U(res), reinterpret_cast<const i64*>(v), poly_lm(c, level, with_p != 0),
+                      (u32)(level + (with_p ? c->h.K : 0)), c->h.N);
+  ACE_CATCH_INT
+}
 
 int ace_ciph_wsum(ace_ctx* c, int64_t* r0, int64_t* r1, const int64_t* const* a0, const int64_t* const* a1,
                   const int64_t* weights, size_t count, size_t level) {

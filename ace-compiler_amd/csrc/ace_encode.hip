@@ -9,25 +9,64 @@ namespace ace {
 
 constexpr int kEncThreads = 256;
 
-// one stage of Embedding_inv over `len` complex slots, in place: butterfly b
-// works on elements (j+i, j+i+num2) of block j
-__global__ __launch_bounds__(kEncThreads) void embed_inv_stage_kernel(double2* __restrict__ r,
-                                                                      const double2* __restrict__ rou,
-                                                                      const u32* __restrict__ rot, u32 M, u32 logm,
-                                                                      u32 len) {
+// stages logm_hi .. logm_lo of Embedding_inv in one launch: a work-group keeps a tile of up to 2048 elements in
+// LDS -- all 2^S values of the S index bits the stages pair up (bits logm_lo-1 .. logm_hi-1), times W consecutive
+// values of the bits below them -- and runs the stages on it with a barrier in between.  Stage logm pairs elements (j+i, j+i+2^(logm-1)) of
+// every block j of 2^logm elements with the twiddle of rot[i]; running the stages in the reference's order on each
+// butterfly keeps the result the same bits however the butterflies are grouped.
+constexpr u32 kTileLog = 11;
+__global__ __launch_bounds__(kEncThreads) void embed_inv_tile_kernel(double2* __restrict__ r,
+                                                                     const double2* __restrict__ rou,
+                                                                     const u32* __restrict__ rot, u32 M, u32 logm_hi,
+                                                                     u32 logm_lo, u32 log_w) {
 #pragma clang fp contract(off)
-  const u32 b = blockIdx.x * kEncThreads + threadIdx.x;
-  if (b >= (len >> 1)) return;
-  const u32 num2 = 1u << (logm - 1);
-  const u32 i = b & (num2 - 1), ie = ((b >> (logm - 1)) << logm) + i, io = ie + num2;
-  const u32 idx_mod = 1u << (logm + 2), gap = M / idx_mod;
-  const u32 rou_idx = (idx_mod - (rot[i] & (idx_mod - 1))) * gap;
-  const double2 x = r[ie], y = r[io], w = rou[rou_idx];
-  const double pr = x.x + y.x, pi = x.y + y.y, mr = x.x - y.x, mi = x.y - y.y;
-  // (mr + mi i) * (w.x + w.y i)
-  const double qr = mr * w.x - mi * w.y, qi = mr * w.y + mi * w.x;
-  r[ie] = make_double2(pr, pi);
-  r[io] = make_double2(qr, qi);
+  __shared__ double2 tile[1u << kTileLog];
+  const u32 S = logm_hi - logm_lo + 1, low_bits = logm_lo - 1;  // low_bits index bits lie below the paired ones
+  const u32 tile_elems = 1u << (S + log_w);
+  // blockIdx.x enumerates (high part, group of W low values)
+  const u32 groups_lo = 1u << (low_bits - log_w);
+  const u32 g_lo0 = (blockIdx.x & (groups_lo - 1)) << log_w, g_hi = blockIdx.x >> (low_bits - log_w);
+  auto global_of = [&](u32 local) {
+    const u32 w = local & ((1u << log_w) - 1), k = local >> log_w;
+    return (g_hi << logm_hi) | (k << low_bits) | (g_lo0 + w);
+  };
+  for (u32 e = threadIdx.x; e < tile_elems; e += kEncThreads) tile[e] = r[global_of(e)];
+  __syncthreads();
+  for (u32 logm = logm_hi; logm >= logm_lo; --logm) {
+    const u32 bitpos = log_w + (logm - logm_lo);
+    const u32 num2 = 1u << (logm - 1), idx_mod = 1u << (logm + 2), gap = M / idx_mod;
+    for (u32 t = threadIdx.x; t < (tile_elems >> 1); t += kEncThreads) {
+      const u32 lo = t & ((1u << bitpos) - 1), le = ((t >> bitpos) << (bitpos + 1)) | lo, lodd = le | (1u << bitpos);
+      const u32 i = global_of(le) & (num2 - 1);
+      const u32 rou_idx = (idx_mod - (rot[i] & (idx_mod - 1))) * gap;
+      const double2 x = tile[le], y = tile[lodd], w = rou[rou_idx];
+      const double pr = x.x + y.x, pi = x.y + y.y, mr = x.x - y.x, mi = x.y - y.y;
+      const double qr = mr * w.x - mi * w.y, qi = mr * w.y + mi * w.x;
+      tile[le] = make_double2(pr, pi);
+      tile[lodd] = make_double2(qr, qi);
+    }
+    __syncthreads();
+    if (logm == logm_lo) break;  // unsigned loop variable
+  }
+  for (u32 e = threadIdx.x; e < tile_elems; e += kEncThreads) r[global_of(e)] = tile[e];
+}
+
+// all stages of Embedding_inv over `len` elements: the top stages in tiles of strided runs, then the rest
+static void launch_embed_inv_stages(hipStream_t st, double2* r, const double2* rou, const u32* rot, u32 M, u32 len) {
+  u32 loglen = 0;
+  while ((1u << loglen) < len) ++loglen;
+  u32 hi = loglen;
+  while (hi > kTileLog) {  // stages hi .. lo on tiles of 2^S x W elements, W >= 16 for coalesced runs
+    const u32 S = (hi - kTileLog) < 7 ? (hi - kTileLog) : 7, lo = hi - S + 1, log_w = kTileLog - S;
+    hipLaunchKernelGGL(embed_inv_tile_kernel, dim3(len >> kTileLog), dim3(kEncThreads), 0, st, r, rou, rot, M, hi, lo,
+                       log_w);
+    hi = lo - 1;
+  }
+  if (hi >= 1) {
+    const u32 tile_log = hi;  // hi <= kTileLog: stages hi .. 1 on tiles of 2^hi consecutive elements
+    hipLaunchKernelGGL(embed_inv_tile_kernel, dim3(len >> tile_log), dim3(kEncThreads), 0, st, r, rou, rot, M, hi, 1u,
+                       0u);
+  }
 }
 
 // Max_64bit_value (include/util/modular.h:279-281)
@@ -88,9 +127,7 @@ void launch_embedding_inv(hipStream_t st, const DevCtx& c, double2* out, double2
                           const u32* rot, u32 len) {
   u32 loglen = 0;
   while ((1u << loglen) < len) ++loglen;
-  for (u32 logm = loglen; logm > 0; --logm)
-    hipLaunchKernelGGL(embed_inv_stage_kernel, dim3(((len >> 1) + kEncThreads - 1) / kEncThreads), dim3(kEncThreads), 0,
-                       st, r, rou, rot, 2 * c.N, logm, len);
+  launch_embed_inv_stages(st, r, rou, rot, 2 * c.N, len);
   hipLaunchKernelGGL(embed_inv_finish_kernel, dim3((len + kEncThreads - 1) / kEncThreads), dim3(kEncThreads), 0, st,
                      out, r, len, loglen);
 }
@@ -100,10 +137,7 @@ void launch_encode(hipStream_t st, const DevCtx& c, u64* out, double2* r, const 
                    u32 n_limbs, int* err) {
   u32 logslots = 0;
   while ((1u << logslots) < slots) ++logslots;
-  const u32 M = 2 * c.N;
-  for (u32 logm = logslots; logm > 0; --logm)
-    hipLaunchKernelGGL(embed_inv_stage_kernel, dim3(((slots >> 1) + kEncThreads - 1) / kEncThreads), dim3(kEncThreads),
-                       0, st, r, rou, rot, M, logm, slots);
+  launch_embed_inv_stages(st, r, rou, rot, 2 * c.N, slots);
   hipLaunchKernelGGL(encode_round_kernel, dim3((c.N + kEncThreads - 1) / kEncThreads, n_limbs), dim3(kEncThreads), 0,
                      st, c, out, r, slots, logslots, scaling_factor, scale, range_bound, lm, err);
 }

@@ -67,7 +67,7 @@ struct MacSet { // operands of one multiply-accumulate launch
 void launch_plain_mac(hipStream_t st, const DevCtx& c, u64* r0, u64* r1, const MacSet& ops, const LimbMap& lm,
                       u32 n_limbs, u32 level, u32 plain_level, bool accumulate, u64 n);
 // a run of Hw_* calls executed as one launch: thread i carries out every entry for element i, in order
-enum BatchKind : u32 { BATCH_ROTATE = 100 };
+enum BatchKind : u32 { BATCH_ROTATE = 100, BATCH_COPY = 101, BATCH_ZERO = 102 };
 struct BatchOp {
   u64* r;
   const u64* a;
@@ -78,6 +78,9 @@ struct BatchOp {
 };
 // chain y (blockIdx.y) is the entries [chain_start[y], chain_start[y+1]): chains share no written range, so they run side by side
 void launch_ew_batch(hipStream_t st, const DevCtx& c, const BatchOp* dev_ops, const u32* dev_chain_start, u32 n_chains, u64 n);
+void launch_sample_uniform(hipStream_t st, const DevCtx& c, u64* r, u64 seed, u64 stream, const LimbMap& lm,
+                           u32 n_limbs, u64 n);
+void launch_expand_small(hipStream_t st, const DevCtx& c, u64* r, const i64* v, const LimbMap& lm, u32 n_limbs, u64 n);
 struct LimbScalars { // one residue per limb
   u64 v[kMaxPrimes];
 };

@@ -100,6 +100,10 @@ __global__ __launch_bounds__(kThreads) void ew_batch_kernel(DevCtx c, const Batc
     if (o.op == BATCH_ROTATE) {
       const i64 src = reinterpret_cast<const i64*>(o.b)[i];
       v = src >= 0 ? o.a[src] : P.q - o.a[-src];
+    } else if (o.op == BATCH_COPY) {
+      v = o.a[i];
+    } else if (o.op == BATCH_ZERO) {
+      v = 0;
     } else {
       const u64 x = o.a[i];
       const u64 y = o.op >= EW_ADD_S ? o.scalar : o.b[i];
@@ -115,6 +119,48 @@ void launch_ew_batch(hipStream_t st, const DevCtx& c, const BatchOp* dev_ops, co
   if (!n || !n_chains) return;
   dim3 g((unsigned)((n + kThreads - 1) / kThreads), n_chains, 1);
   hipLaunchKernelGGL(ew_batch_kernel, g, dim3(kThreads), 0, st, c, dev_ops, dev_chain_start, n);
+}
+
+// ---- key-generation helpers: uniform residues and small signed polynomials spread over limbs ------------
+__device__ __forceinline__ u64 mix64(u64 z) {  // the finaliser of splitmix64
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+// limb t, word i = floor(x q_t / 2^128) for a 128-bit x hashed from (seed, stream, t, i): uniform on [0, q_t) up to
+// a bias below 2^-64
+__global__ __launch_bounds__(kThreads) void sample_uniform_kernel(DevCtx c, u64* __restrict__ r, u64 seed, u64 stream,
+                                                                  LimbMap lm, u64 n) {
+  const u32 limb = blockIdx.y;
+  const u64 q = c.primes[lm.prime[limb]].q;
+#pragma unroll
+  ACE_EW_LOOP(i, n) {
+    const u64 key = mix64(seed + 0x9E3779B97F4A7C15ull * (stream + 1)) ^ ((u64)limb << 40) ^ i;
+    const u64 hi = mix64(key + 0x9E3779B97F4A7C15ull), lo = mix64(key + 2 * 0x9E3779B97F4A7C15ull + 1);
+    const u64 carry = __umul64hi(lo, q);
+    const u64 low = hi * q, sum = low + carry;
+    r[(u64)limb * n + i] = __umul64hi(hi, q) + (sum < low ? 1 : 0);
+  }
+}
+void launch_sample_uniform(hipStream_t st, const DevCtx& c, u64* r, u64 seed, u64 stream, const LimbMap& lm,
+                           u32 n_limbs, u64 n) {
+  if (!n || !n_limbs) return;
+  hipLaunchKernelGGL(sample_uniform_kernel, ew_grid(n, n_limbs), dim3(kThreads), 0, st, c, r, seed, stream, lm, n);
+}
+// limb t, word i = v[i] mod q_t for small signed v (|v| < q_t)
+__global__ __launch_bounds__(kThreads) void expand_small_kernel(DevCtx c, u64* __restrict__ r, const i64* __restrict__ v,
+                                                                LimbMap lm, u64 n) {
+  const u32 limb = blockIdx.y;
+  const u64 q = c.primes[lm.prime[limb]].q;
+#pragma unroll
+  ACE_EW_LOOP(i, n) {
+    const i64 x = v[i];
+    r[(u64)limb * n + i] = x < 0 ? q - (u64)(-x) : (u64)x;
+  }
+}
+void launch_expand_small(hipStream_t st, const DevCtx& c, u64* r, const i64* v, const LimbMap& lm, u32 n_limbs, u64 n) {
+  if (!n || !n_limbs) return;
+  hipLaunchKernelGGL(expand_small_kernel, ew_grid(n, n_limbs), dim3(kThreads), 0, st, c, r, v, lm, n);
 }
 
 // ---- per-limb scalars: Scalars_integer_add_poly / Scalars_integer_multiply_poly (poly/src/rns_poly.c) ----

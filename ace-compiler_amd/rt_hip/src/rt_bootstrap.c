@@ -383,6 +383,16 @@ static void keygen(BTS_PRECOM* pre) {
   pre->keys = true;
 }
 
+/* Bootstrap_precom (context/src/ckks_context.c:239-262): when the chain is deep enough to bootstrap at all, the
+ * plaintext diagonals and the keys of the default slot count are made at key generation, not inside the program */
+void Rt_bootstrap_prepare(void) {
+  uint32_t slots = (uint32_t)(G.N / 2);
+  if (slots < 2) return;
+  uint32_t logs = (uint32_t)log2(slots), budget = logs < 3 ? logs : 3;
+  if (G.L - 1 <= approx_mod_depth() + 2 * budget) return;
+  keygen(setup(slots));
+}
+
 void Rt_bootstrap_finalize(void) {
   while (Precoms) {
     BTS_PRECOM* p = Precoms;

@@ -70,65 +70,47 @@ static void sample_ternary(int64_t* v, size_t n, size_t weight) {
 }
 
 /* ---- small helpers over the device ------------------------------------------------------------ */
-static size_t prime_of_limb(size_t t, size_t level) { return t < level ? t : G.L + (t - level); }
+static uint64_t Seed, Stream; /* of the device-side uniform sampler: one stream per polynomial */
 
 /* signed small coefficients -> residues of `level` Q limbs (+ the P limbs), NTT form, in dev */
 static void small_to_dev(int64_t* dev, const int64_t* v, size_t level, bool with_p) {
-  size_t   n = G.N, T = level + (with_p ? G.K : 0);
-  int64_t* host = (int64_t*)malloc(T * n * sizeof(int64_t));
-  int32_t  idx[128];
-  for (size_t t = 0; t < T; ++t) {
-    int64_t q = G.q[prime_of_limb(t, level)]._val;
-    idx[t]    = (int32_t)prime_of_limb(t, level);
-    for (size_t i = 0; i < n; ++i) host[t * n + i] = v[i] < 0 ? v[i] + q : v[i];
-  }
-  ACE_OK(ace_upload(G.ctx, dev, host, T * n));
+  size_t  T = level + (with_p ? G.K : 0);
+  int32_t idx[128];
+  for (size_t t = 0; t < T; ++t) idx[t] = (int32_t)(t < level ? t : G.L + (t - level));
+  ACE_OK(ace_expand_small(G.ctx, dev, v, level, with_p));
   ACE_OK(ace_ntt(G.ctx, dev, dev, idx, T, 1, 0));
-  free(host);
 }
-/* uniform residues: a uniform polynomial is uniform in NTT form too */
+/* uniform residues, drawn on the device: a uniform polynomial is uniform in NTT form too */
 static void uniform_to_dev(int64_t* dev, size_t level, bool with_p) {
-  size_t   n = G.N, T = level + (with_p ? G.K : 0);
-  int64_t* host = (int64_t*)malloc(T * n * sizeof(int64_t));
-  for (size_t t = 0; t < T; ++t) {
-    uint64_t q = (uint64_t)G.q[prime_of_limb(t, level)]._val;
-    for (size_t i = 0; i < n; ++i) host[t * n + i] = (int64_t)rng_below(q);
-  }
-  ACE_OK(ace_upload(G.ctx, dev, host, T * n));
-  free(host);
+  ACE_OK(ace_sample_uniform(G.ctx, dev, level, with_p, Seed, Stream++));
 }
 
 /* ---- keys (ckks/src/key_gen.c:127-262) ----------------------------------------------------------- */
-/* host words of a switch key taking a polynomial that multiplies s_src to a pair that decrypts under
- * s_res (both: device, L+k limbs, NTT): per digit b = -a*s_res + e + P*s_src on the digit's limbs */
-static int64_t* make_switch_key(const int64_t* s_res, const int64_t* s_src) {
+/* a switch key taking a polynomial that multiplies s_src to a pair that decrypts under s_res (both: device,
+ * L+k limbs, NTT), built in place in HBM: per digit b = -a*s_res + e + P*s_src on the digit's limbs */
+static void make_switch_key(SWITCH_KEY* key, const int64_t* s_res, const int64_t* s_src) {
   size_t   n = G.N, T = G.L + G.K, ps = ace_part_size(G.ctx);
-  int64_t* key = (int64_t*)malloc(2 * G.parts * T * n * sizeof(int64_t));
-  int64_t *a = Rt_dev_alloc(T * n), *b = Rt_dev_alloc(T * n), *e = Rt_dev_alloc(T * n), *t = Rt_dev_alloc(n);
+  int64_t* dev = Rt_dev_alloc_raw(2 * G.parts * T * n);
+  int64_t *e = Rt_dev_alloc_raw(T * n), *t = Rt_dev_alloc_raw(n);
   int64_t* small = (int64_t*)malloc(n * sizeof(int64_t));
-  unsigned __int128 P = 1; /* only P mod q_i is needed */
   for (size_t d = 0; d < G.parts; ++d) {
+    int64_t *b = dev + 2 * d * T * n, *a = b + T * n;
     uniform_to_dev(a, G.L, true);
     sample_triangle(small, n);
     small_to_dev(e, small, G.L, true);
     ACE_OK(ace_poly_mul(G.ctx, b, a, s_res, G.L, 1));
     ACE_OK(ace_poly_sub(G.ctx, b, e, b, G.L, 1));
     for (size_t i = d * ps; i < (d + 1) * ps && i < G.L; ++i) {
-      uint64_t q = (uint64_t)G.q[i]._val, pm = 1;
+      uint64_t q = (uint64_t)G.q[i]._val, pm = 1; /* P mod q_i */
       for (size_t j = 0; j < G.K; ++j) pm = (uint64_t)((unsigned __int128)pm * ((uint64_t)G.p[j]._val % q) % q);
       ACE_OK(ace_hw_modmul_scalar(G.ctx, t, s_src + i * n, (int64_t)pm, i, n));
       ACE_OK(ace_hw_modadd(G.ctx, b + i * n, b + i * n, t, i, n));
     }
-    ACE_OK(ace_download(G.ctx, key + (2 * d) * T * n, b, T * n));
-    ACE_OK(ace_download(G.ctx, key + (2 * d + 1) * T * n, a, T * n));
   }
-  (void)P;
   free(small);
-  Rt_dev_free(a);
-  Rt_dev_free(b);
   Rt_dev_free(e);
   Rt_dev_free(t);
-  return key;
+  Rt_install_key_dev(key, dev);
 }
 
 /* sigma_k on signed coefficients: X^i -> X^(i k mod 2N), negated past N */
@@ -148,16 +130,15 @@ static uint64_t inv_mod_pow2(uint64_t k, uint64_t m) { /* k odd, m a power of tw
 void Rt_generate_rotation_key(int32_t rot_idx) {
   FMT_ASSERT(G.secret_ntt, "Rt_generate_keys() has not run");
   size_t   n = G.N, T = G.L + G.K;
-  uint32_t k = (uint32_t)rot_idx == 2 * G.N - 1 ? 2 * G.N - 1 : ace_find_automorphism_index(G.ctx, rot_idx);
+  ROT_KEY* entry = Rt_rot_entry(rot_idx);
+  uint32_t k = entry->auto_idx;
   /* "fast" key: the evaluator switches the un-rotated c1 and applies the automorphism last, so the
    * key leads from s to sigma_k^-1(s) (key_gen.c:216-262) */
   int64_t* rs = (int64_t*)malloc(n * sizeof(int64_t));
   automorphism_small(rs, G.secret_small, inv_mod_pow2(k, 2 * n));
-  int64_t* s_res = Rt_dev_alloc(T * n);
+  int64_t* s_res = Rt_dev_alloc_raw(T * n);
   small_to_dev(s_res, rs, G.L, true);
-  int64_t* key = make_switch_key(s_res, G.secret_ntt);
-  Rt_load_switch_key(true, rot_idx, key);
-  free(key);
+  make_switch_key(&Rt_find_rot(rot_idx)->swk, s_res, G.secret_ntt);
   free(rs);
   Rt_dev_free(s_res);
 }
@@ -170,18 +151,20 @@ void Rt_generate_keys(uint64_t seed) {
     if (!seed) seed = (uint64_t)time(NULL) ^ ((uint64_t)clock() << 32) ^ 0x5DEECE66Dull;
   }
   rng_seed(seed);
+  Seed   = seed;
+  Stream = 0;
   Rt_ckks_finalize(); /* a second call replaces the keys */
   CKKS_PARAMS* prm = Get_context_params();
   size_t       n = G.N, T = G.L + G.K, hw = prm->_hamming_weight;
   G.secret_small = (int64_t*)malloc(n * sizeof(int64_t));
   sample_ternary(G.secret_small, n, hw);
-  G.secret_ntt = Rt_dev_alloc(T * n);
+  G.secret_ntt = Rt_dev_alloc_raw(T * n);
   small_to_dev(G.secret_ntt, G.secret_small, G.L, true);
   /* public key: pk1 = a, pk0 = -a s + e  (L limbs) */
-  G.pk0 = Rt_dev_alloc(G.L * n);
-  G.pk1 = Rt_dev_alloc(G.L * n);
+  G.pk0 = Rt_dev_alloc_raw(G.L * n);
+  G.pk1 = Rt_dev_alloc_raw(G.L * n);
   int64_t* small = (int64_t*)malloc(n * sizeof(int64_t));
-  int64_t* e     = Rt_dev_alloc(G.L * n);
+  int64_t* e     = Rt_dev_alloc_raw(G.L * n);
   uniform_to_dev(G.pk1, G.L, false);
   sample_triangle(small, n);
   small_to_dev(e, small, G.L, false);
@@ -190,14 +173,13 @@ void Rt_generate_keys(uint64_t seed) {
   Rt_dev_free(e);
   free(small);
   /* relinearisation key: from s^2 to s */
-  int64_t* s2 = Rt_dev_alloc(T * n);
+  int64_t* s2 = Rt_dev_alloc_raw(T * n);
   ACE_OK(ace_poly_mul(G.ctx, s2, G.secret_ntt, G.secret_ntt, G.L, 1));
-  int64_t* key = make_switch_key(G.secret_ntt, s2);
-  Rt_load_switch_key(false, 0, key);
-  free(key);
+  make_switch_key(&G.relin, G.secret_ntt, s2);
   Rt_dev_free(s2);
   for (size_t i = 0; i < prm->_num_rot_idx; ++i)
     if (!Rt_find_rot(prm->_rot_idxs[i])) Rt_generate_rotation_key(prm->_rot_idxs[i]); /* index 0 included: generated code asks for it */
+  Rt_bootstrap_prepare();
 }
 
 void Rt_ckks_finalize(void) {

@@ -478,13 +478,13 @@ void Hw_intt(int64_t* res, int64_t* a, size_t prime_idx, uint32_t degree) {
 }
 
 /* ---- keys --------------------------------------------------------------------------------- */
-void Rt_install_key(SWITCH_KEY* k, const int64_t* host) {
-  size_t T = G.L + G.K, n = G.N, words = 2 * G.parts * T * n;
+/* a switch key over a device buffer [digit][b | a][(L+k) limbs][N] that the key takes ownership of */
+void Rt_install_key_dev(SWITCH_KEY* k, int64_t* dev) {
+  size_t T = G.L + G.K, n = G.N;
   free_key(k);
   RT_KEY_PARTS* kp = (RT_KEY_PARTS*)calloc(1, sizeof(RT_KEY_PARTS) + G.parts * sizeof(PUBLIC_KEY));
   kp->n   = G.parts;
-  kp->dev = Rt_dev_alloc(words);
-  ACE_OK(ace_upload(G.ctx, kp->dev, host, words));
+  kp->dev = dev;
   for (size_t d = 0; d < G.parts; ++d) {
     POLYNOMIAL v = {G.N, T, G.L, G.K, true, kp->dev + 2 * d * T * n};
     kp->pk[d]._p0 = v;
@@ -493,6 +493,12 @@ void Rt_install_key(SWITCH_KEY* k, const int64_t* host) {
   }
   k->_public_keys = kp;
 }
+void Rt_install_key(SWITCH_KEY* k, const int64_t* host) {
+  size_t   words = 2 * G.parts * (G.L + G.K) * G.N;
+  int64_t* dev   = Rt_dev_alloc_raw(words);
+  ACE_OK(ace_upload(G.ctx, dev, host, words));
+  Rt_install_key_dev(k, dev);
+}
 
 ROT_KEY* Rt_find_rot(int32_t rot_idx) {
   for (size_t i = 0; i < G.n_rot; ++i)
@@ -500,26 +506,26 @@ ROT_KEY* Rt_find_rot(int32_t rot_idx) {
   return NULL;
 }
 
+/* the entry of a rotation index, created with its automorphism table when new */
+ROT_KEY* Rt_rot_entry(int32_t rot_idx) {
+  ROT_KEY* r = Rt_find_rot(rot_idx);
+  if (r) return r;
+  if (G.n_rot == G.cap_rot) {
+    G.cap_rot = G.cap_rot ? 2 * G.cap_rot : 16;
+    G.rot     = (ROT_KEY*)realloc(G.rot, G.cap_rot * sizeof(ROT_KEY));
+  }
+  r = &G.rot[G.n_rot++];
+  memset(r, 0, sizeof(*r));
+  r->rot_idx  = rot_idx;
+  r->auto_idx = (uint32_t)rot_idx == 2 * G.N - 1 ? 2 * G.N - 1 : ace_find_automorphism_index(G.ctx, rot_idx);
+  r->order    = Rt_dev_alloc(G.N);
+  ACE_OK(ace_automorphism_order(G.ctx, r->order, r->auto_idx, 1));
+  return r;
+}
+
 void Rt_load_switch_key(bool is_rot, int32_t rot_idx, const int64_t* host_words) {
   NEED_CTX();
-  if (!is_rot) {
-    Rt_install_key(&G.relin, host_words);
-    return;
-  }
-  ROT_KEY* r = Rt_find_rot(rot_idx);
-  if (!r) {
-    if (G.n_rot == G.cap_rot) {
-      G.cap_rot = G.cap_rot ? 2 * G.cap_rot : 16;
-      G.rot     = (ROT_KEY*)realloc(G.rot, G.cap_rot * sizeof(ROT_KEY));
-    }
-    r = &G.rot[G.n_rot++];
-    memset(r, 0, sizeof(*r));
-    r->rot_idx  = rot_idx;
-    r->auto_idx = (uint32_t)rot_idx == 2 * G.N - 1 ? 2 * G.N - 1 : ace_find_automorphism_index(G.ctx, rot_idx);
-    r->order    = Rt_dev_alloc(G.N);
-    ACE_OK(ace_automorphism_order(G.ctx, r->order, r->auto_idx, 1));
-  }
-  Rt_install_key(&r->swk, host_words);
+  Rt_install_key(is_rot ? &Rt_rot_entry(rot_idx)->swk : &G.relin, host_words);
 }
 
 uint32_t Auto_idx(int32_t rot_idx) {

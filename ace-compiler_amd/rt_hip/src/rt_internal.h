@@ -58,9 +58,12 @@ int64_t* Rt_dev_alloc_raw(size_t n_words);
 IO_SLOT* Rt_find_slot(IO_SLOT* s, size_t n, const char* name, size_t idx);
 IO_SLOT* Rt_add_slot(IO_SLOT** s, size_t* n, const char* name, size_t idx);
 void     Rt_install_key(SWITCH_KEY* k, const int64_t* host);
+void     Rt_install_key_dev(SWITCH_KEY* k, int64_t* dev); /* takes ownership of the buffer */
+ROT_KEY* Rt_rot_entry(int32_t rot_idx);
 ROT_KEY* Rt_find_rot(int32_t rot_idx);
 void     Rt_ckks_finalize(void);
 void     Rt_bootstrap_finalize(void);
+void     Rt_bootstrap_prepare(void);
 size_t   Rt_sin_series(size_t hamming_weight, int even, double* coeff, uint32_t* k_bound, uint32_t* double_angle);
 void     Rt_series_divide(double* q, size_t* n_q, double* r, size_t* n_r, const double* f, size_t n_f, const double* g, size_t n_g);
 /* Encode_val: `level` residues of trunc(value * scale), large products through the approximation factor */

@@ -149,7 +149,7 @@ def bootstrap_leg():
         vals = dict(zip(f[0::2], f[1::2]))
         ms = float(vals["ms"])
         return {"bootstrap": {"workload": "one bootstrap, N=65536, 34 limbs (60/56 bits), 32768 slots, to level 15",
-                              "ms": ms, "first_call_ms_with_setup_and_keys": float(vals["first_ms"]),
+                              "ms": ms, "first_call_ms": float(vals["first_ms"]),
                               "max_err": float(vals["max_err"]), "exit_status": r.returncode,
                               "published_cpu_ms": round(784.03e3 / 19, 1),
                               "vs_published_cpu": round(784.03e3 / 19 / ms, 1)}}

@@ -154,6 +154,13 @@ int ace_poly_mul_scalars(ace_ctx* ctx, int64_t* res, const int64_t* a, const int
  * Mul_const), a0/a1 host arrays of `count` (<= 32) device pointers.  The result may alias an operand. */
 int ace_ciph_wsum(ace_ctx* ctx, int64_t* r0, int64_t* r1, const int64_t* const* a0, const int64_t* const* a1,
                   const int64_t* weights, size_t count, size_t level);
+/* Key-generation helpers (the polynomials of ckks/src/key_gen.c:127-200 are drawn limb by limb on the host in the
+ * reference; its generator cannot be reproduced, so these have no bit-level counterpart).
+ * ace_sample_uniform: level Q limbs (+ the P limbs) of residues uniform on [0, q_t), a pure function of
+ *   (seed, stream, limb, position) through a 64-bit mixing hash: reproducible, NOT a cryptographic generator.
+ * ace_expand_small: a HOST array of N small signed coefficients (|v| <= 2^30) as residues of every limb. */
+int ace_sample_uniform(ace_ctx* ctx, int64_t* res, size_t level, int with_p, uint64_t seed, uint64_t stream);
+int ace_expand_small(ace_ctx* ctx, int64_t* res, const int64_t* small_host, size_t level, int with_p);
 /* The inner sum of a baby-step group of the bootstrap's linear transforms (Mul_plaintext + Add_ciphertext,
  * ckks/src/bootstrap.c:1291-1311): (r0, r1) = sum_j (a0[j], a1[j]) * plain[j], or += when `accumulate`.
  * Operands and result are extended polynomials at `level`; a plaintext holds plain_level >= level Q limbs

@@ -533,7 +533,7 @@ def test_recorded_hw_calls_equal_calls_issued_one_by_one(pair):
         limb = lambda t: buf.view(t * N, N)
         r = np.random.Generator(np.random.PCG64(99))
         for step in range(400):
-            kind = int(r.integers(0, 10))
+            kind = int(r.integers(0, 12))
             t = int(r.integers(0, n_limbs))
             same = [u for u in range(n_limbs) if prime[u] == prime[t]]
             a, b, d = (int(r.choice(same)) for _ in range(3))
@@ -549,6 +549,12 @@ def test_recorded_hw_calls_equal_calls_issued_one_by_one(pair):
             elif kind < 9:
                 if d != a:
                     g.hw("rotate", limb(d), limb(a), order, p)
+            elif kind == 10:
+                g.copy(limb(d), limb(a))
+            elif kind == 11:
+                if t + 1 < n_limbs:
+                    g.copy(buf.view(t * N, 2 * N), buf.view(((t + 5) % (n_limbs - 1)) * N, 2 * N)) if abs(((t + 5) % (n_limbs - 1)) - t) >= 2 else None
+                g.lib.ace_zero(g.h, limb(d).ptr, N // 2)
             elif t + 1 < n_limbs and d not in (t, t + 1):
                 # an operand one word out of step with limbs the run has just written: element i of it is element
                 # i+1 of limb t, which another thread wrote (values need not be reduced for an addition's operand
@@ -562,3 +568,42 @@ def test_recorded_hw_calls_equal_calls_issued_one_by_one(pair):
     y = g.upload(host)
     program(y)
     eq(y.get(), want, "recorded run")
+
+
+def test_key_generation_helpers(pair):
+    """ace_expand_small exactly; ace_sample_uniform: in range, reproducible, streams differ, and roughly uniform
+    (mean, and a chi-square over 16 buckets at 6 sigma) -- it has no counterpart to compare bits with."""
+    g = pair.g
+    N, L, K = g.N, g.L, g.K
+    level = L
+    T = level + K
+    primes = list(g.primes[:level]) + list(g.primes[L:])
+    rng = np.random.Generator(np.random.PCG64(8 + N))
+    small = rng.integers(-3, 4, N).astype(np.int64)
+    r = g.alloc(T * N)
+    g.expand_small(r, small, level, True)
+    want = np.concatenate([np.where(small < 0, small + int(q), small) for q in primes])
+    eq(r.get(), want, "expand_small")
+    with pytest.raises(RuntimeError):
+        g.expand_small(r, small * (1 << 40), level, True)
+
+    a, b, c2 = g.alloc(T * N), g.alloc(T * N), g.alloc(T * N)
+    g.sample_uniform(a, level, True, 1234, 7)
+    g.sample_uniform(b, level, True, 1234, 7)
+    g.sample_uniform(c2, level, True, 1234, 8)
+    x, y, z = a.get(), b.get(), c2.get()
+    assert np.array_equal(x, y)
+    if N >= 64:
+        assert not np.array_equal(x, z)
+    for t, q in enumerate(primes):
+        v = x[t * N:(t + 1) * N]
+        assert v.min() >= 0 and v.max() < int(q)
+    if N >= 1024:
+        u = np.concatenate([x[t * N:(t + 1) * N] / float(q) for t, q in enumerate(primes)])
+        assert abs(u.mean() - 0.5) < 6 * (1 / 12) ** 0.5 / u.size ** 0.5
+        counts = np.bincount((u * 16).astype(np.int64), minlength=16).astype(np.float64)
+        expect = u.size / 16
+        chi2 = ((counts - expect) ** 2 / expect).sum()
+        assert chi2 < 15 + 6 * (2 * 15) ** 0.5
+        # limbs are not copies of each other
+        assert np.mean(x[:N] % 1024 == x[N:2 * N] % 1024) < 0.01 if T > 1 else True
