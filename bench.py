@@ -49,11 +49,24 @@ def time_region(g, fn, reps):
 
 
 def cpu_baseline(x_host, idx, budget_s):
-    """The oracle's NTT round trip on a bounded sample of the same batch (one thread)."""
+    """The NTT round trip on the host, one thread, on a bounded sample of the same batch: the reference's own
+    Ftt_fwd / Ftt_inv where the compiled reference (oracle/_ref/ref_driver) is present, else the oracle's port."""
+    import refdrv
+
+    per_poly = LIMBS * N
+    if refdrv.available():
+        s = refdrv.RefSession(*CFG)
+        k = s.add(refdrv.OP_TIME_NTT, LIMBS, int(budget_s * 1000), 0, 0, idx, x_host[:per_poly])
+        _, res = s.run()
+        trips, ns = int(res[k][0]), int(res[k][1])
+        assert (res[k][2:] == x_host[:per_poly]).all()
+        gbs = trips * per_poly * 16 * 2 / (ns * 1e-9) / 1e9
+        return {"value": round(gbs, 4), "unit": "GB/s", "cores": 1, "kind": "reference",
+                "sample": "%d round trips of one polynomial of the batch (%d limbs) through the reference's Ftt_fwd / "
+                          "Ftt_inv, %.1f s, single thread, gcc -O3" % (trips, LIMBS, ns * 1e-9)}
     from oracle_lib import Oracle
 
     o = Oracle(*CFG)
-    per_poly = LIMBS * N
     done, t0 = 0, time.perf_counter()
     while time.perf_counter() - t0 < budget_s:  # walk the batch, again from the start if time is left
         p = done % POLYS

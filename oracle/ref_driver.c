@@ -18,6 +18,7 @@
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <time.h>
 
 #include "common/cmplr_api.h"
 #include "common/rt_config.h"
@@ -40,7 +41,7 @@ enum {
   OP_NTT = 1, OP_INTT, OP_HW, OP_DECOMP_MODUP, OP_PRECOMP, OP_MOD_DOWN,
   OP_RESCALE, OP_DOT_PROD, OP_AUTO_ORDER, OP_AUTO_INDEX, OP_AUTOMORPHISM,
   OP_EXTEND, OP_TBL_MODUP, OP_TBL_MODDOWN, OP_TBL_RESCALE, OP_POLY, OP_TWIDDLES,
-  OP_MOD_UP, OP_MOD_DOWN_RESCALE, OP_REDUCE_RESCALE_MODUP, OP_FROM_LEVEL0, OP_ENCODE, OP_DECODE, OP_EMBEDDING
+  OP_MOD_UP, OP_MOD_DOWN_RESCALE, OP_REDUCE_RESCALE_MODUP, OP_FROM_LEVEL0, OP_ENCODE, OP_DECODE, OP_EMBEDDING, OP_TIME_NTT
 };
 
 static int64_t* in_buf;
@@ -119,6 +120,31 @@ int main(int argc, char** argv) {
           else                Ftt_inv(&vl, ntt, &vl);
         }
         wr1((int64_t)(nl * N));
+        wr(data, nl * N);
+        break;
+      }
+      case OP_TIME_NTT: { /* a1 = n_limbs, a2 = milliseconds; in = prime_idx[n_limbs] data[n_limbs*N];
+                             forward + inverse of every limb, again and again; out = round trips, ns, data */
+        size_t nl = (size_t)a1;
+        int64_t* data = in + nl;
+        struct timespec t0, t1;
+        int64_t trips = 0, ns = 0;
+        clock_gettime(CLOCK_MONOTONIC, &t0);
+        do {
+          for (size_t t = 0; t < nl; t++) {
+            VALUE_LIST vl;
+            Init_i64_value_list_no_copy(&vl, N, data + t * N);
+            NTT_CONTEXT* ntt = Get_ntt(prime_at((size_t)in[t]));
+            Ftt_fwd(&vl, ntt, &vl);
+            Ftt_inv(&vl, ntt, &vl);
+          }
+          trips++;
+          clock_gettime(CLOCK_MONOTONIC, &t1);
+          ns = (int64_t)(t1.tv_sec - t0.tv_sec) * 1000000000 + (t1.tv_nsec - t0.tv_nsec);
+        } while (ns < a2 * 1000000);
+        wr1((int64_t)(2 + nl * N));
+        wr1(trips);
+        wr1(ns);
         wr(data, nl * N);
         break;
       }
