@@ -545,6 +545,13 @@ void ace_ctx::flush_pending() {
   run.written.clear();
   run.rot_res.clear();
   run.rot_src.clear();
+  if (count <= kSmallRun) {
+    SmallRun small{};
+    for (u32 k = 0; k < count; ++k) small.ops[k] = sorted[k];
+    for (size_t k = 0; k < chain_start.size(); ++k) small.chain_start[k] = (uint16_t)chain_start[k];
+    launch_ew_batch_small(stream, d, small, n_chains, n);
+    return;
+  }
   if (!run_dev) {
     HIP_OK(hipMalloc((void**)&run_dev, kMaxRun * sizeof(BatchOp)));
     owned.push_back(run_dev);
@@ -953,7 +960,14 @@ static int64_t* alloc_words(ace_ctx* c, size_t n_words, bool zero) {
       HIP_OK(e);
     }
     c->live[p] = words;
-    if (zero) launch_fill_zero(c->stream, p, n_words);
+    if (zero) {
+      const size_t N = c->h.N;
+      if (c->batching && n_words % N == 0 && n_words / N <= 64) {  // as entries of one limb each, next to the calls that follow
+        for (size_t t = 0; t < n_words / N; ++t) c->run_append(BatchOp{p + t * N, nullptr, nullptr, 0, (u32)BATCH_ZERO, 0}, N);
+      } else {
+        launch_fill_zero(c->stream, p, n_words);
+      }
+    }
     return reinterpret_cast<int64_t*>(p);
   } catch (const std::exception& e) {
     g_err = e.what();

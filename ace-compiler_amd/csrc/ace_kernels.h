@@ -76,6 +76,12 @@ struct BatchOp {
   u32 op;        // an EwOp, or BATCH_ROTATE
   u32 prime;
 };
+constexpr u32 kSmallRun = 64;  // runs up to this many entries travel as kernel arguments, no copy
+struct SmallRun {
+  BatchOp ops[kSmallRun];
+  uint16_t chain_start[kSmallRun + 1];
+};
+void launch_ew_batch_small(hipStream_t st, const DevCtx& c, const SmallRun& run, u32 n_chains, u64 n);
 // chain y (blockIdx.y) is the entries [chain_start[y], chain_start[y+1]): chains share no written range, so they run side by side
 void launch_ew_batch(hipStream_t st, const DevCtx& c, const BatchOp* dev_ops, const u32* dev_chain_start, u32 n_chains, u64 n);
 void launch_sample_uniform(hipStream_t st, const DevCtx& c, u64* r, u64 seed, u64 stream, const LimbMap& lm,

@@ -89,10 +89,18 @@ void launch_plain_mac(hipStream_t st, const DevCtx& c, u64* r0, u64* r1, const M
 // The host splits a run into chains that share no written range; a chain's entries are carried out in order by
 // the thread of element i, so an entry may read what an earlier one of its chain wrote (identical ranges only;
 // a rotate never reads or overwrites anything the run touches).
+__device__ __forceinline__ void run_chain(const DevCtx& c, const BatchOp* ops, u32 first, u32 last, u64 i);
 __global__ __launch_bounds__(kThreads) void ew_batch_kernel(DevCtx c, const BatchOp* ops, const u32* chain_start, u64 n) {
-  const u32 first = chain_start[blockIdx.y], last = chain_start[blockIdx.y + 1];
   const u64 i = (u64)blockIdx.x * kThreads + threadIdx.x;
   if (i >= n) return;
+  run_chain(c, ops, chain_start[blockIdx.y], chain_start[blockIdx.y + 1], i);
+}
+__global__ __launch_bounds__(kThreads) void ew_batch_small_kernel(DevCtx c, SmallRun run, u64 n) {
+  const u64 i = (u64)blockIdx.x * kThreads + threadIdx.x;
+  if (i >= n) return;
+  run_chain(c, run.ops, run.chain_start[blockIdx.y], run.chain_start[blockIdx.y + 1], i);
+}
+__device__ __forceinline__ void run_chain(const DevCtx& c, const BatchOp* ops, u32 first, u32 last, u64 i) {
   for (u32 k = first; k < last; ++k) {
     const BatchOp o = ops[k];
     const DevPrime P = c.primes[o.prime];
@@ -114,6 +122,11 @@ __global__ __launch_bounds__(kThreads) void ew_batch_kernel(DevCtx c, const Batc
     }
     o.r[i] = v;
   }
+}
+void launch_ew_batch_small(hipStream_t st, const DevCtx& c, const SmallRun& run, u32 n_chains, u64 n) {
+  if (!n || !n_chains) return;
+  dim3 g((unsigned)((n + kThreads - 1) / kThreads), n_chains, 1);
+  hipLaunchKernelGGL(ew_batch_small_kernel, g, dim3(kThreads), 0, st, c, run, n);
 }
 void launch_ew_batch(hipStream_t st, const DevCtx& c, const BatchOp* dev_ops, const u32* dev_chain_start, u32 n_chains, u64 n) {
   if (!n || !n_chains) return;
