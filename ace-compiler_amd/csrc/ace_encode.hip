@@ -15,7 +15,8 @@ constexpr int kEncThreads = 256;
 // every block j of 2^logm elements with the twiddle of rot[i]; running the stages in the reference's order on each
 // butterfly keeps the result the same bits however the butterflies are grouped.
 constexpr u32 kTileLog = 11;
-__global__ __launch_bounds__(kEncThreads) void embed_inv_tile_kernel(double2* __restrict__ r,
+constexpr int kTileThreads = 1024;  // one butterfly per thread and stage on a full tile: the stages are latency-bound
+__global__ __launch_bounds__(kTileThreads) void embed_inv_tile_kernel(double2* __restrict__ r,
                                                                      const double2* __restrict__ rou,
                                                                      const u32* __restrict__ rot, u32 M, u32 logm_hi,
                                                                      u32 logm_lo, u32 log_w) {
@@ -30,12 +31,12 @@ __global__ __launch_bounds__(kEncThreads) void embed_inv_tile_kernel(double2* __
     const u32 w = local & ((1u << log_w) - 1), k = local >> log_w;
     return (g_hi << logm_hi) | (k << low_bits) | (g_lo0 + w);
   };
-  for (u32 e = threadIdx.x; e < tile_elems; e += kEncThreads) tile[e] = r[global_of(e)];
+  for (u32 e = threadIdx.x; e < tile_elems; e += blockDim.x) tile[e] = r[global_of(e)];
   __syncthreads();
   for (u32 logm = logm_hi; logm >= logm_lo; --logm) {
     const u32 bitpos = log_w + (logm - logm_lo);
     const u32 num2 = 1u << (logm - 1), idx_mod = 1u << (logm + 2), gap = M / idx_mod;
-    for (u32 t = threadIdx.x; t < (tile_elems >> 1); t += kEncThreads) {
+    for (u32 t = threadIdx.x; t < (tile_elems >> 1); t += blockDim.x) {
       const u32 lo = t & ((1u << bitpos) - 1), le = ((t >> bitpos) << (bitpos + 1)) | lo, lodd = le | (1u << bitpos);
       const u32 i = global_of(le) & (num2 - 1);
       const u32 rou_idx = (idx_mod - (rot[i] & (idx_mod - 1))) * gap;
@@ -48,7 +49,7 @@ __global__ __launch_bounds__(kEncThreads) void embed_inv_tile_kernel(double2* __
     __syncthreads();
     if (logm == logm_lo) break;  // unsigned loop variable
   }
-  for (u32 e = threadIdx.x; e < tile_elems; e += kEncThreads) r[global_of(e)] = tile[e];
+  for (u32 e = threadIdx.x; e < tile_elems; e += blockDim.x) r[global_of(e)] = tile[e];
 }
 
 // all stages of Embedding_inv over `len` elements: the top stages in tiles of strided runs, then the rest
@@ -56,15 +57,17 @@ static void launch_embed_inv_stages(hipStream_t st, double2* r, const double2* r
   u32 loglen = 0;
   while ((1u << loglen) < len) ++loglen;
   u32 hi = loglen;
+  const u32 tile = 1u << (loglen < kTileLog ? loglen : kTileLog), half = tile >> 1;
+  const u32 threads = half >= (u32)kTileThreads ? (u32)kTileThreads : (half < 64 ? 64 : half);
   while (hi > kTileLog) {  // stages hi .. lo on tiles of 2^S x W elements, W >= 16 for coalesced runs
     const u32 S = (hi - kTileLog) < 7 ? (hi - kTileLog) : 7, lo = hi - S + 1, log_w = kTileLog - S;
-    hipLaunchKernelGGL(embed_inv_tile_kernel, dim3(len >> kTileLog), dim3(kEncThreads), 0, st, r, rou, rot, M, hi, lo,
+    hipLaunchKernelGGL(embed_inv_tile_kernel, dim3(len >> kTileLog), dim3(threads), 0, st, r, rou, rot, M, hi, lo,
                        log_w);
     hi = lo - 1;
   }
   if (hi >= 1) {
     const u32 tile_log = hi;  // hi <= kTileLog: stages hi .. 1 on tiles of 2^hi consecutive elements
-    hipLaunchKernelGGL(embed_inv_tile_kernel, dim3(len >> tile_log), dim3(kEncThreads), 0, st, r, rou, rot, M, hi, 1u,
+    hipLaunchKernelGGL(embed_inv_tile_kernel, dim3(len >> tile_log), dim3(threads), 0, st, r, rou, rot, M, hi, 1u,
                        0u);
   }
 }
