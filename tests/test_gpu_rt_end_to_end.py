@@ -49,6 +49,20 @@ def test_reference_example(name):
     assert r.returncode == 0 and "SUCESS" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
 
 
+def test_reference_generated_sine_program():
+    """rtlib/ant/dataset/bootstrap_full.cxx: a C++ program the reference's EDSL generated (N=16384, depth 23, key
+    switches open-coded with Decomp_modup / Set_pk0 / Hw_modmul / Mod_down), built unchanged with g++.  Its harness
+    holds sin(8x) for eight inputs and compares to 1e-2; its side-file is the header-only one the reference ships."""
+    exe = os.path.join(EXAMPLES_DIR, "bootstrap_full")
+    if not os.path.exists(exe):
+        pytest.skip("built only where the reference tree is present")
+    env = dict(os.environ, RT_HIP_SEED="5",
+               RT_HIP_DATA_FILE=os.path.join(rt_program.ROOT, "tests", "golden", "bootstrap_full_data.msg"))
+    print("running", exe, flush=True)
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=110, env=env)
+    assert r.returncode == 0 and "SUCCESS" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
+
+
 CODEC = os.path.join(rt_program.ROOT, "tests", "programs", "codec_program")
 
 
