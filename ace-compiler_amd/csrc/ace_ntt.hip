@@ -10,10 +10,12 @@
 //            (R coefficients 4096 apart) entirely in registers; loads and
 //            stores are 2 KiB-contiguous per wavefront row.  No LDS.
 //            pass 2 "chunk": stages LOGR..logN-1 on one contiguous 4096-word
-//            chunk per workgroup: 256 threads x 16 registers, three rounds of
-//            four stages with two LDS transposes (LDS index padded by e>>4 so
-//            the 16-word-strided accesses are conflict-free), and a last
-//            transpose so the global store is coalesced.
+//            chunk per workgroup: 512 threads x 8 registers, four rounds of
+//            three stages with the chunk passing through LDS between rounds
+//            (LDS index padded by e>>4, which keeps every round's accesses
+//            free of bank conflicts), and once more so that the global
+//            store is coalesced.  Eight registers per thread leave room for
+//            eight waves per SIMD, which is what hides the memory waits.
 //   inverse  the same two kernels mirrored (chunk first, strided last).
 // N <= 4096 uses one workgroup per limb with the limb in LDS.
 //
@@ -26,9 +28,13 @@
 //             in FP64 (|x| < 2^53).  A twiddle product is y*w - rint(y*(w/q))*q
 //             evaluated exactly with one FMA for the low half of y*w and one
 //             for the subtraction (6 full-rate FP64 ops); sums are brought
-//             back to |x| <= q/2 every few stages with x - rint(x/q)*q.  All
-//             intermediate values are integers below 2^53, so no rounding
-//             ever happens and the final canonical residue is exact.
+//             back to |x| <= q/2 with x - rint(x/q)*q before they can pass
+//             2^53: a forward stage takes a bound of B q to at most
+//             (1.43 B + 0.5) q, an inverse stage doubles it, so forward code
+//             reduces at least every four stages (every three in the chunk
+//             pass) and inverse code every two or three.  All intermediate
+//             values are integers below 2^53, so no rounding ever happens
+//             and the final canonical residue is exact.
 // Between the two passes the buffer holds back-end specific words (lazily
 // reduced integers, or raw FP64 bits); the second pass stores canonical
 // residues.
@@ -225,6 +231,9 @@ __device__ __forceinline__ void reduce_all(const A& ar, typename A::T* v) {
 template <class A, int LOGR, int K = 0>
 __device__ __forceinline__ void fwd_strided_stages(const A& ar, typename A::T* v) {
   if constexpr (K < LOGR) {
+    // four stages is the most the FP64 back end may run between reductions; up to three may start from
+    // canonical residues, four need centred ones
+    if ((K == 0 && LOGR >= 4) || K == 4) reduce_all<A, (1 << LOGR)>(ar, v);
     ct_stage<A, (1 << LOGR), K>(ar, v, 1u << K);
     fwd_strided_stages<A, LOGR, K + 1>(ar, v);
   }
@@ -275,7 +284,6 @@ __global__ __launch_bounds__(256) void ntt_fwd_strided(DevCtx c, PolySeq dsts, P
       v[r] = ar.in_canon(shoup_mul(x, K, Kp, P.q));
     }
   }
-  if (LOGR > 4) reduce_all<A, R>(ar, v);
   fwd_strided_stages<A, LOGR>(ar, v);
 #pragma unroll
   for (int r = 0; r < R; ++r) dst[off + r * rs] = ar.out_mid(v[r]);
@@ -307,23 +315,51 @@ static inline unsigned chunk_grid(const DevCtx& c, u32 n_limbs, u32 slots_per_gr
 }
 
 // Polynomials handled by one work-group of a chunk pass.  They share the
-// (limb, chunk) pair and therefore every twiddle, which is loaded once; the
-// next polynomial's words are requested before the current one is transformed.
+// (limb, chunk) pair; the next polynomial's words are requested before the
+// current one is transformed.
 #ifndef ACE_NTT_PB
 #define ACE_NTT_PB 1
 #endif
-#ifndef ACE_NTT_PREFETCH
-#define ACE_NTT_PREFETCH 0
-#endif
 constexpr int kPolysPerBlock = ACE_NTT_PB;
-constexpr bool kPrefetchTw = ACE_NTT_PREFETCH != 0;
+constexpr int kChunkThreads = 512;  // 8 coefficients per thread
+
+// The four thread -> element maps of a chunk pass (r = 0..7).  Each covers the
+// chunk once and keeps the eight elements of three consecutive stages' worth of
+// butterflies in one thread:
+//   wide    t + 512 r                      spans 2048, 1024, 512  (also the coalesced global order)
+//   wave    (t/64)*512 + 64 r + t%64       spans 256, 128, 64     (twiddles are wave-uniform)
+//   octet   h*64 + 8 r + t%8               spans 32, 16, 8        (h = t/8 with its two low bits swapped, which
+//                                                                  puts the two h of a 16-lane group 8 banks apart)
+//   narrow  8 t + r                        spans 4, 2, 1
+struct ChunkMap {
+  int wide, wave, octet, narrow;  // LDS positions of element r = 0; element r is at +off(r)
+  u32 wv, h;
+  __device__ __forceinline__ ChunkMap(int t) {
+    wv = (u32)__builtin_amdgcn_readfirstlane(t >> 6);
+    const u32 a = (u32)t >> 3;
+    h = (a & ~3u) | ((a & 1u) << 1) | ((a >> 1) & 1u);
+    wide = lds_pos(t);
+    wave = lds_pos((int)(wv * 512) + (t & 63));
+    octet = lds_pos((int)(h * 64) + (t & 7));
+    narrow = lds_pos(t * 8);
+  }
+  // lds_pos(e0 + d) == lds_pos(e0) + d + (d >> 4) whenever (e0 & 15) + (d & 15) < 16, which holds for
+  // each map's increments below
+  static __device__ __forceinline__ constexpr int wide_off(int r) { return 512 * r + 32 * r; }
+  static __device__ __forceinline__ constexpr int wave_off(int r) { return 64 * r + 4 * r; }
+  static __device__ __forceinline__ constexpr int octet_off(int r) { return 8 * r + (r >> 1); }
+  static __device__ __forceinline__ constexpr int narrow_off(int r) { return r; }
+};
 
 // forward, chunk pass: stages logr..logN-1 on 4096 contiguous words, in place.
-// grid = chunk_grid(n_limbs, ceil(n_polys / kPolysPerBlock))
+// grid = chunk_grid(n_limbs, ceil(n_polys / kPolysPerBlock)), 512 threads: four
+// rounds of three stages with the chunk passing through LDS between them, and
+// once more so that the global store is coalesced.  A thread writes back the
+// positions it read, so one barrier per round suffices.
 // EPI != 0: the result is not stored back but consumed by FwdFuse::epi.
 template <class A, int EPI>
-__global__ __launch_bounds__(256) void ntt_fwd_chunk(DevCtx c, PolySeq datas, LimbMap lm, LimbMap pos, u32 logr,
-                                                     u32 n_limbs, u32 n_polys, FwdFuse f) {
+__global__ __launch_bounds__(kChunkThreads, 8) void ntt_fwd_chunk(DevCtx c, PolySeq datas, LimbMap lm, LimbMap pos,
+                                                                  u32 logr, u32 n_limbs, u32 n_polys, FwdFuse f) {
   typedef typename A::T T;
   __shared__ T lds[kChunk + kChunk / 16];
   const int t = threadIdx.x;
@@ -336,85 +372,66 @@ __global__ __launch_bounds__(256) void ntt_fwd_chunk(DevCtx c, PolySeq datas, Li
   u64* base = datas.at(poly0) + loff;
   A ar;
   ar.init(c, pi, false, nullptr, 0);
-  // twiddle index of local stage ls, local group 0 of this chunk: m + (chunk << ls)
-  const u32 m0 = 1u << logr;
-  const int hi = t >> 4, lo = t & 15;
-  u64 raw[16], nxt[16];
+  const ChunkMap cm(t);
+  // twiddle index of local stage ls, local group g of this chunk: (m0 << ls) + (chunk << ls) + g
+  const u32 tw0 = (1u << logr) + chunk;
+  u64 raw[8], nxt[8];
 #pragma unroll
-  for (int r = 0; r < 16; ++r) raw[r] = base[t + 256 * r];
-  // the per-thread twiddles of rounds B and C (round A's are wave-uniform)
-  typename A::TWL twB0[1], twB1[2], twB2[4], twB3[8], twC0[1], twC1[2], twC2[4], twC3[8];
-  if (kPrefetchTw) {
-    ar.template load_tw<1>((m0 << 4) + (chunk << 4) + (hi << 0), twB0);
-    ar.template load_tw<2>((m0 << 5) + (chunk << 5) + (hi << 1), twB1);
-    ar.template load_tw<4>((m0 << 6) + (chunk << 6) + (hi << 2), twB2);
-    ar.template load_tw<8>((m0 << 7) + (chunk << 7) + (hi << 3), twB3);
-    ar.template load_tw<1>((m0 << 8) + (chunk << 8) + (t << 0), twC0);
-    ar.template load_tw<2>((m0 << 9) + (chunk << 9) + (t << 1), twC1);
-    ar.template load_tw<4>((m0 << 10) + (chunk << 10) + (t << 2), twC2);
-    ar.template load_tw<8>((m0 << 11) + (chunk << 11) + (t << 3), twC3);
-  }
+  for (int r = 0; r < 8; ++r) raw[r] = base[t + 512 * r];
   for (u32 it = 0; it < cnt; ++it) {
     base = datas.at(poly0 + it) + loff;
     if (it + 1 < cnt) {
       const u64* nb = datas.at(poly0 + it + 1) + loff;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) nxt[r] = nb[t + 256 * r];
+      for (int r = 0; r < 8; ++r) nxt[r] = nb[t + 512 * r];
     }
-    T v[16];
-    // round A: element e = t + 256 r, local stages 0..3
+    T v[8];
+    // local stages 0..2
 #pragma unroll
-    for (int r = 0; r < 16; ++r) v[r] = ar.in_mid(raw[r]);
-    reduce_all<A, 16>(ar, v);
-    ct_stage<A, 16, 0>(ar, v, (m0 << 0) + (chunk << 0));
-    ct_stage<A, 16, 1>(ar, v, (m0 << 1) + (chunk << 1));
-    ct_stage<A, 16, 2>(ar, v, (m0 << 2) + (chunk << 2));
-    ct_stage<A, 16, 3>(ar, v, (m0 << 3) + (chunk << 3));
+    for (int r = 0; r < 8; ++r) v[r] = ar.in_mid(raw[r]);
+    reduce_all<A, 8>(ar, v);
+    ct_stage<A, 8, 0>(ar, v, tw0 << 0);
+    ct_stage<A, 8, 1>(ar, v, tw0 << 1);
+    ct_stage<A, 8, 2>(ar, v, tw0 << 2);
 #pragma unroll
-    for (int r = 0; r < 16; ++r) lds[lds_pos(t + 256 * r)] = v[r];
+    for (int r = 0; r < 8; ++r) lds[cm.wide + ChunkMap::wide_off(r)] = v[r];
     __syncthreads();
-    // round B: e = hi*256 + r*16 + lo, local stages 4..7: local group = (hi << (ls-4)) + g
+    // local stages 3..5: local group = (wv << (ls-3)) + g
 #pragma unroll
-    for (int r = 0; r < 16; ++r) v[r] = lds[lds_pos(hi * 256 + r * 16 + lo)];
-    reduce_all<A, 16>(ar, v);
-    if (kPrefetchTw) {
-      ct_stage_pre<A, 16, 0>(ar, v, twB0);
-      ct_stage_pre<A, 16, 1>(ar, v, twB1);
-      ct_stage_pre<A, 16, 2>(ar, v, twB2);
-      ct_stage_pre<A, 16, 3>(ar, v, twB3);
-    } else {
-      ct_stage<A, 16, 0>(ar, v, (m0 << 4) + (chunk << 4) + (hi << 0));
-      ct_stage<A, 16, 1>(ar, v, (m0 << 5) + (chunk << 5) + (hi << 1));
-      ct_stage<A, 16, 2>(ar, v, (m0 << 6) + (chunk << 6) + (hi << 2));
-      ct_stage<A, 16, 3>(ar, v, (m0 << 7) + (chunk << 7) + (hi << 3));
-    }
+    for (int r = 0; r < 8; ++r) v[r] = lds[cm.wave + ChunkMap::wave_off(r)];
+    reduce_all<A, 8>(ar, v);
+    ct_stage<A, 8, 0>(ar, v, (tw0 << 3) + (cm.wv << 0));
+    ct_stage<A, 8, 1>(ar, v, (tw0 << 4) + (cm.wv << 1));
+    ct_stage<A, 8, 2>(ar, v, (tw0 << 5) + (cm.wv << 2));
 #pragma unroll
-    for (int r = 0; r < 16; ++r) lds[lds_pos(hi * 256 + r * 16 + lo)] = v[r];
+    for (int r = 0; r < 8; ++r) lds[cm.wave + ChunkMap::wave_off(r)] = v[r];
     __syncthreads();
-    // round C: e = t*16 + r, local stages 8..11: local group = (t << (ls-8)) + g
+    // local stages 6..8: local group = (h << (ls-6)) + g
 #pragma unroll
-    for (int r = 0; r < 16; ++r) v[r] = lds[lds_pos(t * 16 + r)];
-    reduce_all<A, 16>(ar, v);
-    if (kPrefetchTw) {
-      ct_stage_pre<A, 16, 0>(ar, v, twC0);
-      ct_stage_pre<A, 16, 1>(ar, v, twC1);
-      ct_stage_pre<A, 16, 2>(ar, v, twC2);
-      ct_stage_pre<A, 16, 3>(ar, v, twC3);
-    } else {
-      ct_stage<A, 16, 0>(ar, v, (m0 << 8) + (chunk << 8) + (t << 0));
-      ct_stage<A, 16, 1>(ar, v, (m0 << 9) + (chunk << 9) + (t << 1));
-      ct_stage<A, 16, 2>(ar, v, (m0 << 10) + (chunk << 10) + (t << 2));
-      ct_stage<A, 16, 3>(ar, v, (m0 << 11) + (chunk << 11) + (t << 3));
-    }
+    for (int r = 0; r < 8; ++r) v[r] = lds[cm.octet + ChunkMap::octet_off(r)];
+    reduce_all<A, 8>(ar, v);
+    ct_stage<A, 8, 0>(ar, v, (tw0 << 6) + (cm.h << 0));
+    ct_stage<A, 8, 1>(ar, v, (tw0 << 7) + (cm.h << 1));
+    ct_stage<A, 8, 2>(ar, v, (tw0 << 8) + (cm.h << 2));
+#pragma unroll
+    for (int r = 0; r < 8; ++r) lds[cm.octet + ChunkMap::octet_off(r)] = v[r];
+    __syncthreads();
+    // local stages 9..11: local group = (t << (ls-9)) + g
+#pragma unroll
+    for (int r = 0; r < 8; ++r) v[r] = lds[cm.narrow + ChunkMap::narrow_off(r)];
+    reduce_all<A, 8>(ar, v);
+    ct_stage<A, 8, 0>(ar, v, (tw0 << 9) + ((u32)t << 0));
+    ct_stage<A, 8, 1>(ar, v, (tw0 << 10) + ((u32)t << 1));
+    ct_stage<A, 8, 2>(ar, v, (tw0 << 11) + ((u32)t << 2));
     u64* ldsu = reinterpret_cast<u64*>(lds);
 #pragma unroll
-    for (int r = 0; r < 16; ++r) ldsu[lds_pos(t * 16 + r)] = ar.out_canon(v[r]);
+    for (int r = 0; r < 8; ++r) ldsu[cm.narrow + ChunkMap::narrow_off(r)] = ar.out_canon(v[r]);
     __syncthreads();
     // each thread reads back the words it will overwrite first in the next
     // iteration, so no further barrier is needed
     if (EPI == 0) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) base[t + 256 * r] = ldsu[lds_pos(t + 256 * r)];
+      for (int r = 0; r < 8; ++r) base[t + 512 * r] = ldsu[cm.wide + ChunkMap::wide_off(r)];
     } else {
       const u32 p = poly0 + it, lt = pos.prime[limb];
       const u64 q = c.primes[pi].q, w = f.cst[2 * lt], wp = f.cst[2 * lt + 1];
@@ -423,16 +440,16 @@ __global__ __launch_bounds__(256) void ntt_fwd_chunk(DevCtx c, PolySeq datas, Li
       const u64* __restrict__ src = f.src.at(p) + o;
       const u64* addend =
           (EPI == 1 && (f.addend_mode == 1 || (f.addend_mode == 2 && !(p & 1)))) ? f.addend.at(p) + o : nullptr;
-      u64 sv[16], av[16];
+      u64 sv[8], av[8];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) sv[r] = src[256 * r];
+      for (int r = 0; r < 8; ++r) sv[r] = src[512 * r];
       if (addend) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) av[r] = addend[256 * r];
+        for (int r = 0; r < 8; ++r) av[r] = addend[512 * r];
       }
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const u64 y = ldsu[lds_pos(t + 256 * r)];
+      for (int r = 0; r < 8; ++r) {
+        const u64 y = ldsu[cm.wide + ChunkMap::wide_off(r)];
         u64 v;
         if (EPI == 1) {
           v = shoup_mul(sub_mod(sv[r], y, q), w, wp, q);
@@ -440,11 +457,11 @@ __global__ __launch_bounds__(256) void ntt_fwd_chunk(DevCtx c, PolySeq datas, Li
         } else {
           v = add_mod(shoup_mul(sv[r], w, wp, q), y, q);
         }
-        out[256 * r] = v;
+        out[512 * r] = v;
       }
     }
 #pragma unroll
-    for (int r = 0; r < 16; ++r) raw[r] = nxt[r];
+    for (int r = 0; r < 8; ++r) raw[r] = nxt[r];
   }
 }
 
@@ -452,10 +469,11 @@ __global__ __launch_bounds__(256) void ntt_fwd_chunk(DevCtx c, PolySeq datas, Li
 // inverse, chunk pass: spans 1..2048 on 4096 contiguous words; src -> dst.
 // Nothing is scaled here: 1/N (times an optional per-limb constant) is applied
 // by the strided pass that always follows.  At span 2^u the stage has
-// m = N >> (u+1) groups and element j belongs to group j >> (u+1).
+// m = N >> (u+1) groups and element j belongs to group j >> (u+1).  The rounds
+// are those of the forward pass in reverse order.
 template <class A>
-__global__ __launch_bounds__(256) void ntt_inv_chunk(DevCtx c, PolySeq dsts, PolySeq srcs, LimbMap lm, LimbMap pos,
-                                                     u32 n_limbs, u32 n_polys) {
+__global__ __launch_bounds__(kChunkThreads, 8) void ntt_inv_chunk(DevCtx c, PolySeq dsts, PolySeq srcs, LimbMap lm,
+                                                                  LimbMap pos, u32 n_limbs, u32 n_polys) {
   typedef typename A::T T;
   __shared__ T lds[kChunk + kChunk / 16];
   const int t = threadIdx.x;
@@ -467,91 +485,67 @@ __global__ __launch_bounds__(256) void ntt_inv_chunk(DevCtx c, PolySeq dsts, Pol
   const u64 off = (u64)pos.prime[limb] * c.N + (u64)chunk * kChunk;
   A ar;
   ar.init(c, pi, true, nullptr, 0);
+  const ChunkMap cm(t);
   const u32 mh = c.N >> 1;  // groups at span 1
-  const int hi = t >> 4, lo = t & 15;
-  u64 raw[16], nxt[16];
+  u64 raw[8], nxt[8];
   {
     const u64* src = srcs.at(poly0);
 #pragma unroll
-    for (int r = 0; r < 16; ++r) raw[r] = src[off + t + 256 * r];
-  }
-  // per-thread twiddles of rounds C' and B' (round A' has wave-uniform ones)
-  typename A::TWL twC0[8], twC1[4], twC2[2], twC3[1], twB0[8], twB1[4], twB2[2], twB3[1];
-  if (kPrefetchTw) {
-    ar.template load_tw<8>((mh >> 0) + (chunk << 11) + (t << 3), twC0);
-    ar.template load_tw<4>((mh >> 1) + (chunk << 10) + (t << 2), twC1);
-    ar.template load_tw<2>((mh >> 2) + (chunk << 9) + (t << 1), twC2);
-    ar.template load_tw<1>((mh >> 3) + (chunk << 8) + (t << 0), twC3);
-    ar.template load_tw<8>((mh >> 4) + (chunk << 7) + (hi << 3), twB0);
-    ar.template load_tw<4>((mh >> 5) + (chunk << 6) + (hi << 2), twB1);
-    ar.template load_tw<2>((mh >> 6) + (chunk << 5) + (hi << 1), twB2);
-    ar.template load_tw<1>((mh >> 7) + (chunk << 4) + (hi << 0), twB3);
+    for (int r = 0; r < 8; ++r) raw[r] = src[off + t + 512 * r];
   }
   for (u32 it = 0; it < cnt; ++it) {
     u64* dst = dsts.at(poly0 + it);
     if (it + 1 < cnt) {
       const u64* src = srcs.at(poly0 + it + 1);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) nxt[r] = src[off + t + 256 * r];
+      for (int r = 0; r < 8; ++r) nxt[r] = src[off + t + 512 * r];
     }
-    T v[16];
+    T v[8];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) lds[lds_pos(t + 256 * r)] = ar.in_canon(raw[r]);
+    for (int r = 0; r < 8; ++r) lds[cm.wide + ChunkMap::wide_off(r)] = ar.in_canon(raw[r]);
     __syncthreads();
-    // round C': e = t*16 + r, u = 0..3
+    // spans 1, 2, 4
 #pragma unroll
-    for (int r = 0; r < 16; ++r) v[r] = lds[lds_pos(t * 16 + r)];
-    reduce_all<A, 16>(ar, v);
-    if (kPrefetchTw) {
-      gs_stage_pre<A, 16, 0>(ar, v, twC0);
-      gs_stage_pre<A, 16, 1>(ar, v, twC1);
-      reduce_all<A, 16>(ar, v);
-      gs_stage_pre<A, 16, 2>(ar, v, twC2);
-      gs_stage_pre<A, 16, 3>(ar, v, twC3);
-    } else {
-      gs_stage<A, 16, 0>(ar, v, (mh >> 0) + (chunk << 11) + (t << 3));
-      gs_stage<A, 16, 1>(ar, v, (mh >> 1) + (chunk << 10) + (t << 2));
-      reduce_all<A, 16>(ar, v);
-      gs_stage<A, 16, 2>(ar, v, (mh >> 2) + (chunk << 9) + (t << 1));
-      gs_stage<A, 16, 3>(ar, v, (mh >> 3) + (chunk << 8) + (t << 0));
-    }
+    for (int r = 0; r < 8; ++r) v[r] = lds[cm.narrow + ChunkMap::narrow_off(r)];
+    reduce_all<A, 8>(ar, v);
+    gs_stage<A, 8, 0>(ar, v, (mh >> 0) + (chunk << 11) + ((u32)t << 2));
+    gs_stage<A, 8, 1>(ar, v, (mh >> 1) + (chunk << 10) + ((u32)t << 1));
+    gs_stage<A, 8, 2>(ar, v, (mh >> 2) + (chunk << 9) + ((u32)t << 0));
 #pragma unroll
-    for (int r = 0; r < 16; ++r) lds[lds_pos(t * 16 + r)] = v[r];
+    for (int r = 0; r < 8; ++r) lds[cm.narrow + ChunkMap::narrow_off(r)] = v[r];
     __syncthreads();
-    // round B': e = hi*256 + r*16 + lo, u = 4..7
+    // spans 8, 16, 32
 #pragma unroll
-    for (int r = 0; r < 16; ++r) v[r] = lds[lds_pos(hi * 256 + r * 16 + lo)];
-    reduce_all<A, 16>(ar, v);
-    if (kPrefetchTw) {
-      gs_stage_pre<A, 16, 0>(ar, v, twB0);
-      gs_stage_pre<A, 16, 1>(ar, v, twB1);
-      reduce_all<A, 16>(ar, v);
-      gs_stage_pre<A, 16, 2>(ar, v, twB2);
-      gs_stage_pre<A, 16, 3>(ar, v, twB3);
-    } else {
-      gs_stage<A, 16, 0>(ar, v, (mh >> 4) + (chunk << 7) + (hi << 3));
-      gs_stage<A, 16, 1>(ar, v, (mh >> 5) + (chunk << 6) + (hi << 2));
-      reduce_all<A, 16>(ar, v);
-      gs_stage<A, 16, 2>(ar, v, (mh >> 6) + (chunk << 5) + (hi << 1));
-      gs_stage<A, 16, 3>(ar, v, (mh >> 7) + (chunk << 4) + (hi << 0));
-    }
+    for (int r = 0; r < 8; ++r) v[r] = lds[cm.octet + ChunkMap::octet_off(r)];
+    reduce_all<A, 8>(ar, v);
+    gs_stage<A, 8, 0>(ar, v, (mh >> 3) + (chunk << 8) + (cm.h << 2));
+    gs_stage<A, 8, 1>(ar, v, (mh >> 4) + (chunk << 7) + (cm.h << 1));
+    gs_stage<A, 8, 2>(ar, v, (mh >> 5) + (chunk << 6) + (cm.h << 0));
 #pragma unroll
-    for (int r = 0; r < 16; ++r) lds[lds_pos(hi * 256 + r * 16 + lo)] = v[r];
+    for (int r = 0; r < 8; ++r) lds[cm.octet + ChunkMap::octet_off(r)] = v[r];
     __syncthreads();
-    // round A': e = t + 256 r, u = 8..11; twiddles wave-uniform.  The words read
-    // here are the ones this thread overwrites first in the next iteration.
+    // spans 64, 128, 256
 #pragma unroll
-    for (int r = 0; r < 16; ++r) v[r] = lds[lds_pos(t + 256 * r)];
-    reduce_all<A, 16>(ar, v);
-    gs_stage<A, 16, 0>(ar, v, (mh >> 8) + (chunk << 3));
-    gs_stage<A, 16, 1>(ar, v, (mh >> 9) + (chunk << 2));
-    reduce_all<A, 16>(ar, v);
-    gs_stage<A, 16, 2>(ar, v, (mh >> 10) + (chunk << 1));
-    gs_stage<A, 16, 3>(ar, v, (mh >> 11) + (chunk << 0));
+    for (int r = 0; r < 8; ++r) v[r] = lds[cm.wave + ChunkMap::wave_off(r)];
+    reduce_all<A, 8>(ar, v);
+    gs_stage<A, 8, 0>(ar, v, (mh >> 6) + (chunk << 5) + (cm.wv << 2));
+    gs_stage<A, 8, 1>(ar, v, (mh >> 7) + (chunk << 4) + (cm.wv << 1));
+    gs_stage<A, 8, 2>(ar, v, (mh >> 8) + (chunk << 3) + (cm.wv << 0));
 #pragma unroll
-    for (int r = 0; r < 16; ++r) dst[off + t + 256 * r] = ar.out_mid(v[r]);
+    for (int r = 0; r < 8; ++r) lds[cm.wave + ChunkMap::wave_off(r)] = v[r];
+    __syncthreads();
+    // spans 512, 1024, 2048; twiddles are uniform over the work-group.  The words read here are the
+    // ones this thread overwrites first in the next iteration.
 #pragma unroll
-    for (int r = 0; r < 16; ++r) raw[r] = nxt[r];
+    for (int r = 0; r < 8; ++r) v[r] = lds[cm.wide + ChunkMap::wide_off(r)];
+    reduce_all<A, 8>(ar, v);
+    gs_stage<A, 8, 0>(ar, v, (mh >> 9) + (chunk << 2));
+    gs_stage<A, 8, 1>(ar, v, (mh >> 10) + (chunk << 1));
+    gs_stage<A, 8, 2>(ar, v, (mh >> 11) + (chunk << 0));
+#pragma unroll
+    for (int r = 0; r < 8; ++r) dst[off + t + 512 * r] = ar.out_mid(v[r]);
+#pragma unroll
+    for (int r = 0; r < 8; ++r) raw[r] = nxt[r];
   }
 }
 
@@ -634,15 +628,15 @@ static void run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst, const
     if (passes & 2) {
       const u32 lr = LOGR;
       if (f.epi == 0)
-        hipLaunchKernelGGL((ntt_fwd_chunk<A, 0>), gc, dim3(256), 0, st, c, dst, lm, pos, lr, n_limbs, n_polys, f);
+        hipLaunchKernelGGL((ntt_fwd_chunk<A, 0>), gc, dim3(kChunkThreads), 0, st, c, dst, lm, pos, lr, n_limbs, n_polys, f);
       else if (f.epi == 1)
-        hipLaunchKernelGGL((ntt_fwd_chunk<A, 1>), gc, dim3(256), 0, st, c, dst, lm, pos, lr, n_limbs, n_polys, f);
+        hipLaunchKernelGGL((ntt_fwd_chunk<A, 1>), gc, dim3(kChunkThreads), 0, st, c, dst, lm, pos, lr, n_limbs, n_polys, f);
       else
-        hipLaunchKernelGGL((ntt_fwd_chunk<A, 2>), gc, dim3(256), 0, st, c, dst, lm, pos, lr, n_limbs, n_polys, f);
+        hipLaunchKernelGGL((ntt_fwd_chunk<A, 2>), gc, dim3(kChunkThreads), 0, st, c, dst, lm, pos, lr, n_limbs, n_polys, f);
     }
   } else {
     if (passes & 1)
-      hipLaunchKernelGGL((ntt_inv_chunk<A>), gc, dim3(256), 0, st, c, dst, src, lm, pos, n_limbs, n_polys);
+      hipLaunchKernelGGL((ntt_inv_chunk<A>), gc, dim3(kChunkThreads), 0, st, c, dst, src, lm, pos, n_limbs, n_polys);
     if (passes & 2)
       hipLaunchKernelGGL((ntt_inv_strided<A, LOGR>), gs, dim3(256), 0, st, c, dst, lm, pos, sidx, scale);
   }

@@ -70,6 +70,40 @@ def test_ntt_all_primes(pair):
     eq(de, e, "edge values round trip")
 
 
+@pytest.mark.parametrize("N,primes", [(8192, [1289999999795201, 1289999999582209]),
+                                      (65536, [1289999997075457, 1289999994191873]),
+                                      (131072, [1289999988293633, 1289999986720769])])
+def test_ntt_largest_primes_of_the_fp64_back_end(N, primes):
+    """Primes just under the bound up to which the transform carries residues in FP64, with inputs made of
+    0, 1, (q-1)/2, (q+1)/2 and q-1: the partial sums between reductions grow fastest for these."""
+    for q in primes:  # the moduli are what they are said to be (Fermat tests to three bases)
+        assert q < 1290000000000000 and q % (2 * N) == 1 and all(pow(a, q - 1, q) == 1 for a in (2, 3, 5))
+    g = acefhe.Context(N, len(primes), primes=primes)
+    o = Oracle(N, len(primes), 0, 0, 1, primes=primes)
+    try:
+        idx = list(range(len(primes)))
+        rng = np.random.Generator(np.random.PCG64(N))
+        for case in range(3):
+            limbs = []
+            for q in primes:
+                pool = np.array([0, 1, (q - 1) // 2, (q + 1) // 2, q - 1], np.int64)
+                pick = rng.integers(0, 5, N) if case < 2 else np.full(N, 4)
+                limbs.append(pool[pick] if case != 1 else np.where(rng.random(N) < 0.5, q - 1, (q + 1) // 2))
+            x = np.concatenate(limbs).astype(np.int64)
+            dx = g.upload(x)
+            g.ntt(dx, dx, idx)
+            eq(dx, o.ntt(x, idx), "forward, case %d" % case)
+            g.intt(dx, dx, idx)
+            eq(dx, x, "round trip, case %d" % case)
+            dx.set(x)
+            g.intt(dx, dx, idx)
+            eq(dx, o.intt(x, idx), "inverse, case %d" % case)
+            dx.free()
+    finally:
+        g.close()
+        o.close()
+
+
 def test_ntt_batched_polys(pair):
     g, o = pair.g, pair.o
     N = g.N
