@@ -38,6 +38,7 @@
 // Between the two passes the buffer holds back-end specific words (lazily
 // reduced integers, or raw FP64 bits); the second pass stores canonical
 // residues.
+#include <algorithm>
 #include <vector>
 
 #include "ace_kernels.h"
@@ -613,32 +614,50 @@ __global__ __launch_bounds__(256) void ntt_small(DevCtx c, PolySeq dsts, PolySeq
 }
 
 // ---------------------------------------------------------------------------
+// A plain two-pass transform of a batch larger than the 256 MiB memory-side cache runs slice by slice, both
+// passes on one slice before the next, so that the second pass finds the first one's output in that cache
+// instead of in HBM (measured on 32 polynomials of 24 limbs at N=2^16: 3 % off the round trip).
+constexpr u64 kSliceBytes = 192ull << 20, kSliceAbove = 256ull << 20;
+
 template <class A, int LOGR>
-static void run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolySeq& src, const LimbMap& lm,
-                      const LimbMap& pos, const LimbMap& sidx, u32 n_limbs, u32 n_polys, bool inverse,
-                      const u64* scale, int passes, const FwdFuse& f) {
-  dim3 gs((c.N >> LOGR) / 256, n_limbs, n_polys), gc(chunk_grid(c, n_limbs, (n_polys + kPolysPerBlock - 1) / kPolysPerBlock));
-  if (!inverse) {
-    if (passes & 1) {
-      if (f.pro == 0)
-        hipLaunchKernelGGL((ntt_fwd_strided<A, LOGR, 0>), gs, dim3(256), 0, st, c, dst, src, lm, pos, f);
-      else
-        hipLaunchKernelGGL((ntt_fwd_strided<A, LOGR, 1>), gs, dim3(256), 0, st, c, dst, src, lm, pos, f);
+static void run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst_all, const PolySeq& src_all,
+                      const LimbMap& lm, const LimbMap& pos, const LimbMap& sidx, u32 n_limbs, u32 n_polys_all,
+                      bool inverse, const u64* scale, int passes, const FwdFuse& f) {
+  const u64 poly_bytes = (u64)n_limbs * c.N * sizeof(u64);
+  u32 slice = n_polys_all;
+  if (passes == 3 && f.epi == 0 && f.pro == 0 && poly_bytes * n_polys_all > kSliceAbove)
+    slice = (u32)std::max<u64>(2, (kSliceBytes / poly_bytes) & ~1ull);
+  for (u32 p0 = 0; p0 < n_polys_all; p0 += slice) {
+    const u32 n_polys = std::min(slice, n_polys_all - p0);
+    const PolySeq dst = dst_all.from(p0), src = src_all.from(p0);
+    dim3 gs((c.N >> LOGR) / 256, n_limbs, n_polys),
+        gc(chunk_grid(c, n_limbs, (n_polys + kPolysPerBlock - 1) / kPolysPerBlock));
+    if (!inverse) {
+      if (passes & 1) {
+        if (f.pro == 0)
+          hipLaunchKernelGGL((ntt_fwd_strided<A, LOGR, 0>), gs, dim3(256), 0, st, c, dst, src, lm, pos, f);
+        else
+          hipLaunchKernelGGL((ntt_fwd_strided<A, LOGR, 1>), gs, dim3(256), 0, st, c, dst, src, lm, pos, f);
+      }
+      if (passes & 2) {
+        const u32 lr = LOGR;
+        if (f.epi == 0)
+          hipLaunchKernelGGL((ntt_fwd_chunk<A, 0>), gc, dim3(kChunkThreads), 0, st, c, dst, lm, pos, lr, n_limbs,
+                             n_polys, f);
+        else if (f.epi == 1)
+          hipLaunchKernelGGL((ntt_fwd_chunk<A, 1>), gc, dim3(kChunkThreads), 0, st, c, dst, lm, pos, lr, n_limbs,
+                             n_polys, f);
+        else
+          hipLaunchKernelGGL((ntt_fwd_chunk<A, 2>), gc, dim3(kChunkThreads), 0, st, c, dst, lm, pos, lr, n_limbs,
+                             n_polys, f);
+      }
+    } else {
+      if (passes & 1)
+        hipLaunchKernelGGL((ntt_inv_chunk<A>), gc, dim3(kChunkThreads), 0, st, c, dst, src, lm, pos, n_limbs,
+                           n_polys);
+      if (passes & 2)
+        hipLaunchKernelGGL((ntt_inv_strided<A, LOGR>), gs, dim3(256), 0, st, c, dst, lm, pos, sidx, scale);
     }
-    if (passes & 2) {
-      const u32 lr = LOGR;
-      if (f.epi == 0)
-        hipLaunchKernelGGL((ntt_fwd_chunk<A, 0>), gc, dim3(kChunkThreads), 0, st, c, dst, lm, pos, lr, n_limbs, n_polys, f);
-      else if (f.epi == 1)
-        hipLaunchKernelGGL((ntt_fwd_chunk<A, 1>), gc, dim3(kChunkThreads), 0, st, c, dst, lm, pos, lr, n_limbs, n_polys, f);
-      else
-        hipLaunchKernelGGL((ntt_fwd_chunk<A, 2>), gc, dim3(kChunkThreads), 0, st, c, dst, lm, pos, lr, n_limbs, n_polys, f);
-    }
-  } else {
-    if (passes & 1)
-      hipLaunchKernelGGL((ntt_inv_chunk<A>), gc, dim3(kChunkThreads), 0, st, c, dst, src, lm, pos, n_limbs, n_polys);
-    if (passes & 2)
-      hipLaunchKernelGGL((ntt_inv_strided<A, LOGR>), gs, dim3(256), 0, st, c, dst, lm, pos, sidx, scale);
   }
 }
 
