@@ -252,11 +252,10 @@ __device__ __forceinline__ void inv_strided_stages(const A& ar, typename A::T* v
 // PRO = 1: the input is not read from src but formed from the last limb of a
 // rescale (FwdFuse::pro).
 template <class A, int LOGR, int PRO>
-__global__ __launch_bounds__(256) void ntt_fwd_strided(DevCtx c, PolySeq dsts, PolySeq srcs, LimbMap lm,
-                                                       LimbMap pos, FwdFuse f) {
+__device__ __forceinline__ void fwd_strided_body(const DevCtx& c, const PolySeq& dsts, const PolySeq& srcs,
+                                                 const LimbMap& pos, const FwdFuse& f, u32 limb, u32 pi) {
   constexpr int R = 1 << LOGR;
   const u32 col = blockIdx.x * 256 + threadIdx.x;
-  const u32 limb = blockIdx.y, pi = lm.prime[limb];
   const u64 rs = c.N >> LOGR;  // row stride
   const u64 off = (u64)pos.prime[limb] * c.N + col;
   u64* __restrict__ dst = dsts.at(blockIdx.z);
@@ -288,6 +287,14 @@ __global__ __launch_bounds__(256) void ntt_fwd_strided(DevCtx c, PolySeq dsts, P
   fwd_strided_stages<A, LOGR>(ar, v);
 #pragma unroll
   for (int r = 0; r < R; ++r) dst[off + r * rs] = ar.out_mid(v[r]);
+}
+// One launch covers limbs of both arithmetic back ends: the choice is uniform over a work-group.
+template <int LOGR, int PRO>
+__global__ __launch_bounds__(256, 4) void ntt_fwd_strided(DevCtx c, PolySeq dsts, PolySeq srcs, LimbMap lm,
+                                                       LimbMap pos, FwdFuse f) {
+  const u32 limb = blockIdx.y, pi = lm.prime[limb];
+  if (c.fp_ok[pi]) fwd_strided_body<ArithFp, LOGR, PRO>(c, dsts, srcs, pos, f, limb, pi);
+  else fwd_strided_body<ArithInt, LOGR, PRO>(c, dsts, srcs, pos, f, limb, pi);
 }
 
 // Work-group -> (chunk, limb, polynomial slot) for the chunk passes.  The grid
@@ -359,16 +366,14 @@ struct ChunkMap {
 // positions it read, so one barrier per round suffices.
 // EPI != 0: the result is not stored back but consumed by FwdFuse::epi.
 template <class A, int EPI>
-__global__ __launch_bounds__(kChunkThreads, 8) void ntt_fwd_chunk(DevCtx c, PolySeq datas, LimbMap lm, LimbMap pos,
-                                                                  u32 logr, u32 n_limbs, u32 n_polys, FwdFuse f) {
+__device__ __forceinline__ void fwd_chunk_body(u64* lds_words, const DevCtx& c, const PolySeq& datas,
+                                               const LimbMap& pos, u32 logr, u32 n_polys, const FwdFuse& f, u32 chunk,
+                                               u32 limb, u32 pblk, u32 pi) {
   typedef typename A::T T;
-  __shared__ T lds[kChunk + kChunk / 16];
+  T* lds = reinterpret_cast<T*>(lds_words);
   const int t = threadIdx.x;
-  u32 chunk, limb, pblk;
-  if (!chunk_block(c, n_limbs, (n_polys + kPolysPerBlock - 1) / kPolysPerBlock, chunk, limb, pblk)) return;
   const u32 poly0 = pblk * kPolysPerBlock;
   const u32 cnt = min((u32)kPolysPerBlock, n_polys - poly0);
-  const u32 pi = lm.prime[limb];
   const u64 loff = (u64)pos.prime[limb] * c.N + (u64)chunk * kChunk;
   u64* base = datas.at(poly0) + loff;
   A ar;
@@ -424,7 +429,7 @@ __global__ __launch_bounds__(kChunkThreads, 8) void ntt_fwd_chunk(DevCtx c, Poly
     ct_stage<A, 8, 0>(ar, v, (tw0 << 9) + ((u32)t << 0));
     ct_stage<A, 8, 1>(ar, v, (tw0 << 10) + ((u32)t << 1));
     ct_stage<A, 8, 2>(ar, v, (tw0 << 11) + ((u32)t << 2));
-    u64* ldsu = reinterpret_cast<u64*>(lds);
+    u64* ldsu = lds_words;
 #pragma unroll
     for (int r = 0; r < 8; ++r) ldsu[cm.narrow + ChunkMap::narrow_off(r)] = ar.out_canon(v[r]);
     __syncthreads();
@@ -441,29 +446,44 @@ __global__ __launch_bounds__(kChunkThreads, 8) void ntt_fwd_chunk(DevCtx c, Poly
       const u64* __restrict__ src = f.src.at(p) + o;
       const u64* addend =
           (EPI == 1 && (f.addend_mode == 1 || (f.addend_mode == 2 && !(p & 1)))) ? f.addend.at(p) + o : nullptr;
-      u64 sv[8], av[8];
+      // four words at a time: the operands of all eight would not fit beside the 64 registers of a thread
 #pragma unroll
-      for (int r = 0; r < 8; ++r) sv[r] = src[512 * r];
-      if (addend) {
+      for (int r0 = 0; r0 < 8; r0 += 4) {
+        u64 sv[4], av[4];
 #pragma unroll
-        for (int r = 0; r < 8; ++r) av[r] = addend[512 * r];
-      }
+        for (int r = 0; r < 4; ++r) sv[r] = src[512 * (r0 + r)];
+        if (addend) {
 #pragma unroll
-      for (int r = 0; r < 8; ++r) {
-        const u64 y = ldsu[cm.wide + ChunkMap::wide_off(r)];
-        u64 v;
-        if (EPI == 1) {
-          v = shoup_mul(sub_mod(sv[r], y, q), w, wp, q);
-          if (addend) v = add_mod(v, av[r], q);
-        } else {
-          v = add_mod(shoup_mul(sv[r], w, wp, q), y, q);
+          for (int r = 0; r < 4; ++r) av[r] = addend[512 * (r0 + r)];
         }
-        out[512 * r] = v;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const u64 y = ldsu[cm.wide + ChunkMap::wide_off(r0 + r)];
+          u64 v;
+          if (EPI == 1) {
+            v = shoup_mul(sub_mod(sv[r], y, q), w, wp, q);
+            if (addend) v = add_mod(v, av[r], q);
+          } else {
+            v = add_mod(shoup_mul(sv[r], w, wp, q), y, q);
+          }
+          out[512 * (r0 + r)] = v;
+        }
       }
     }
 #pragma unroll
     for (int r = 0; r < 8; ++r) raw[r] = nxt[r];
   }
+}
+// (the Mod_down tail keeps three more pointers and constants alive: 80 registers, 6 waves per SIMD)
+template <int EPI>
+__global__ __launch_bounds__(kChunkThreads, EPI == 1 ? 6 : 8) void ntt_fwd_chunk(DevCtx c, PolySeq datas, LimbMap lm, LimbMap pos,
+                                                                  u32 logr, u32 n_limbs, u32 n_polys, FwdFuse f) {
+  __shared__ u64 lds[kChunk + kChunk / 16];
+  u32 chunk, limb, pblk;
+  if (!chunk_block(c, n_limbs, (n_polys + kPolysPerBlock - 1) / kPolysPerBlock, chunk, limb, pblk)) return;
+  const u32 pi = lm.prime[limb];
+  if (c.fp_ok[pi]) fwd_chunk_body<ArithFp, EPI>(lds, c, datas, pos, logr, n_polys, f, chunk, limb, pblk, pi);
+  else fwd_chunk_body<ArithInt, EPI>(lds, c, datas, pos, logr, n_polys, f, chunk, limb, pblk, pi);
 }
 
 // ---------------------------------------------------------------------------
@@ -473,16 +493,14 @@ __global__ __launch_bounds__(kChunkThreads, 8) void ntt_fwd_chunk(DevCtx c, Poly
 // m = N >> (u+1) groups and element j belongs to group j >> (u+1).  The rounds
 // are those of the forward pass in reverse order.
 template <class A>
-__global__ __launch_bounds__(kChunkThreads, 8) void ntt_inv_chunk(DevCtx c, PolySeq dsts, PolySeq srcs, LimbMap lm,
-                                                                  LimbMap pos, u32 n_limbs, u32 n_polys) {
+__device__ __forceinline__ void inv_chunk_body(u64* lds_words, const DevCtx& c, const PolySeq& dsts,
+                                               const PolySeq& srcs, const LimbMap& pos, u32 n_polys, u32 chunk,
+                                               u32 limb, u32 pblk, u32 pi) {
   typedef typename A::T T;
-  __shared__ T lds[kChunk + kChunk / 16];
+  T* lds = reinterpret_cast<T*>(lds_words);
   const int t = threadIdx.x;
-  u32 chunk, limb, pblk;
-  if (!chunk_block(c, n_limbs, (n_polys + kPolysPerBlock - 1) / kPolysPerBlock, chunk, limb, pblk)) return;
   const u32 poly0 = pblk * kPolysPerBlock;
   const u32 cnt = min((u32)kPolysPerBlock, n_polys - poly0);
-  const u32 pi = lm.prime[limb];
   const u64 off = (u64)pos.prime[limb] * c.N + (u64)chunk * kChunk;
   A ar;
   ar.init(c, pi, true, nullptr, 0);
@@ -549,27 +567,42 @@ __global__ __launch_bounds__(kChunkThreads, 8) void ntt_inv_chunk(DevCtx c, Poly
     for (int r = 0; r < 8; ++r) raw[r] = nxt[r];
   }
 }
+__global__ __launch_bounds__(kChunkThreads, 8) void ntt_inv_chunk(DevCtx c, PolySeq dsts, PolySeq srcs, LimbMap lm,
+                                                                  LimbMap pos, u32 n_limbs, u32 n_polys) {
+  __shared__ u64 lds[kChunk + kChunk / 16];
+  u32 chunk, limb, pblk;
+  if (!chunk_block(c, n_limbs, (n_polys + kPolysPerBlock - 1) / kPolysPerBlock, chunk, limb, pblk)) return;
+  const u32 pi = lm.prime[limb];
+  if (c.fp_ok[pi]) inv_chunk_body<ArithFp>(lds, c, dsts, srcs, pos, n_polys, chunk, limb, pblk, pi);
+  else inv_chunk_body<ArithInt>(lds, c, dsts, srcs, pos, n_polys, chunk, limb, pblk, pi);
+}
 
 // inverse, strided pass: spans 4096..N/2, then scale every word by the limb's
 // constant (default 1/N) and store canonical residues.  In place.
-// scale: nullptr, or (constant, Shoup companion) pairs indexed by sidx.prime[limb].
+// scale: nullptr, or (constant, Shoup companion) pairs indexed by the limb's place in the launch.
 template <class A, int LOGR>
-__global__ __launch_bounds__(256) void ntt_inv_strided(DevCtx c, PolySeq datas, LimbMap lm, LimbMap pos,
-                                                       LimbMap sidx, const u64* __restrict__ scale) {
+__device__ __forceinline__ void inv_strided_body(const DevCtx& c, const PolySeq& datas, const LimbMap& pos,
+                                                 const u64* __restrict__ scale, u32 limb, u32 pi) {
   constexpr int R = 1 << LOGR;
   const u32 col = blockIdx.x * 256 + threadIdx.x;
-  const u32 limb = blockIdx.y, pi = lm.prime[limb];
   const u64 rs = c.N >> LOGR;
   const u64 off = (u64)pos.prime[limb] * c.N + col;
   u64* __restrict__ data = datas.at(blockIdx.z);
   A ar;
-  ar.init(c, pi, true, scale, sidx.prime[limb]);
+  ar.init(c, pi, true, scale, limb);
   typename A::T v[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) v[r] = ar.in_mid(data[off + r * rs]);
   inv_strided_stages<A, LOGR>(ar, v);
 #pragma unroll
   for (int r = 0; r < R; ++r) data[off + r * rs] = ar.out_scaled(v[r]);
+}
+template <int LOGR>
+__global__ __launch_bounds__(256) void ntt_inv_strided(DevCtx c, PolySeq datas, LimbMap lm, LimbMap pos,
+                                                       const u64* __restrict__ scale) {
+  const u32 limb = blockIdx.y, pi = lm.prime[limb];
+  if (c.fp_ok[pi]) inv_strided_body<ArithFp, LOGR>(c, datas, pos, scale, limb, pi);
+  else inv_strided_body<ArithInt, LOGR>(c, datas, pos, scale, limb, pi);
 }
 
 // ---------------------------------------------------------------------------
@@ -619,10 +652,10 @@ __global__ __launch_bounds__(256) void ntt_small(DevCtx c, PolySeq dsts, PolySeq
 // instead of in HBM (measured on 32 polynomials of 24 limbs at N=2^16: 3 % off the round trip).
 constexpr u64 kSliceBytes = 192ull << 20, kSliceAbove = 256ull << 20;
 
-template <class A, int LOGR>
+template <int LOGR>
 static void run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst_all, const PolySeq& src_all,
-                      const LimbMap& lm, const LimbMap& pos, const LimbMap& sidx, u32 n_limbs, u32 n_polys_all,
-                      bool inverse, const u64* scale, int passes, const FwdFuse& f) {
+                      const LimbMap& lm, const LimbMap& pos, u32 n_limbs, u32 n_polys_all, bool inverse,
+                      const u64* scale, int passes, const FwdFuse& f) {
   const u64 poly_bytes = (u64)n_limbs * c.N * sizeof(u64);
   u32 slice = n_polys_all;
   if (passes == 3 && f.epi == 0 && f.pro == 0 && poly_bytes * n_polys_all > kSliceAbove)
@@ -635,49 +668,28 @@ static void run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst_all, c
     if (!inverse) {
       if (passes & 1) {
         if (f.pro == 0)
-          hipLaunchKernelGGL((ntt_fwd_strided<A, LOGR, 0>), gs, dim3(256), 0, st, c, dst, src, lm, pos, f);
+          hipLaunchKernelGGL((ntt_fwd_strided<LOGR, 0>), gs, dim3(256), 0, st, c, dst, src, lm, pos, f);
         else
-          hipLaunchKernelGGL((ntt_fwd_strided<A, LOGR, 1>), gs, dim3(256), 0, st, c, dst, src, lm, pos, f);
+          hipLaunchKernelGGL((ntt_fwd_strided<LOGR, 1>), gs, dim3(256), 0, st, c, dst, src, lm, pos, f);
       }
       if (passes & 2) {
         const u32 lr = LOGR;
         if (f.epi == 0)
-          hipLaunchKernelGGL((ntt_fwd_chunk<A, 0>), gc, dim3(kChunkThreads), 0, st, c, dst, lm, pos, lr, n_limbs,
+          hipLaunchKernelGGL((ntt_fwd_chunk<0>), gc, dim3(kChunkThreads), 0, st, c, dst, lm, pos, lr, n_limbs,
                              n_polys, f);
         else if (f.epi == 1)
-          hipLaunchKernelGGL((ntt_fwd_chunk<A, 1>), gc, dim3(kChunkThreads), 0, st, c, dst, lm, pos, lr, n_limbs,
+          hipLaunchKernelGGL((ntt_fwd_chunk<1>), gc, dim3(kChunkThreads), 0, st, c, dst, lm, pos, lr, n_limbs,
                              n_polys, f);
         else
-          hipLaunchKernelGGL((ntt_fwd_chunk<A, 2>), gc, dim3(kChunkThreads), 0, st, c, dst, lm, pos, lr, n_limbs,
+          hipLaunchKernelGGL((ntt_fwd_chunk<2>), gc, dim3(kChunkThreads), 0, st, c, dst, lm, pos, lr, n_limbs,
                              n_polys, f);
       }
     } else {
       if (passes & 1)
-        hipLaunchKernelGGL((ntt_inv_chunk<A>), gc, dim3(kChunkThreads), 0, st, c, dst, src, lm, pos, n_limbs,
-                           n_polys);
+        hipLaunchKernelGGL(ntt_inv_chunk, gc, dim3(kChunkThreads), 0, st, c, dst, src, lm, pos, n_limbs, n_polys);
       if (passes & 2)
-        hipLaunchKernelGGL((ntt_inv_strided<A, LOGR>), gs, dim3(256), 0, st, c, dst, lm, pos, sidx, scale);
+        hipLaunchKernelGGL((ntt_inv_strided<LOGR>), gs, dim3(256), 0, st, c, dst, lm, pos, scale);
     }
-  }
-}
-
-template <class A>
-static bool run_large_dispatch(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolySeq& src,
-                               const LimbMap& lm, const LimbMap& pos, const LimbMap& sidx, u32 n_limbs, u32 n_polys,
-                               bool inverse, const u64* scale, int passes, const FwdFuse& f) {
-  switch (c.logN - kLogChunk) {
-#define ACE_NTT_CASE(LR)                                                                                         \
-  case LR:                                                                                                       \
-    run_large<A, LR>(st, c, dst, src, lm, pos, sidx, n_limbs, n_polys, inverse, scale, passes, f);                \
-    return true;
-    ACE_NTT_CASE(1)
-    ACE_NTT_CASE(2)
-    ACE_NTT_CASE(3)
-    ACE_NTT_CASE(4)
-    ACE_NTT_CASE(5)
-#undef ACE_NTT_CASE
-    default:
-      return false;  // ring degree above 2^17 not supported
   }
 }
 
@@ -699,25 +711,20 @@ bool launch_ntt(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolyS
                        scale);
     return true;
   }
-  if (c.logN - kLogChunk > 5) return false;
-  // split the limbs by arithmetic back end: one launch per pass and group
-  LimbMap lm_g[2]{}, pos_g[2]{}, sidx_g[2]{};
-  u32 cnt[2] = {0, 0};
-  for (u32 t = 0; t < n_limbs; ++t) {
-    int gsel = c.fp_ok[lm.prime[t]] ? 1 : 0;
-    lm_g[gsel].prime[cnt[gsel]] = lm.prime[t];
-    pos_g[gsel].prime[cnt[gsel]] = pos.prime[t];
-    sidx_g[gsel].prime[cnt[gsel]] = (uint8_t)t;
-    ++cnt[gsel];
+  switch (c.logN - kLogChunk) {
+#define ACE_NTT_CASE(LR)                                                                      \
+  case LR:                                                                                    \
+    run_large<LR>(st, c, dst, src, lm, pos, n_limbs, n_polys, inverse, scale, passes, f);     \
+    return true;
+    ACE_NTT_CASE(1)
+    ACE_NTT_CASE(2)
+    ACE_NTT_CASE(3)
+    ACE_NTT_CASE(4)
+    ACE_NTT_CASE(5)
+#undef ACE_NTT_CASE
+    default:
+      return false;  // ring degree above 2^17 not supported
   }
-  bool ok = true;
-  if (cnt[0])
-    ok &= run_large_dispatch<ArithInt>(st, c, dst, src, lm_g[0], pos_g[0], sidx_g[0], cnt[0], n_polys, inverse,
-                                       scale, passes, f);
-  if (cnt[1])
-    ok &= run_large_dispatch<ArithFp>(st, c, dst, src, lm_g[1], pos_g[1], sidx_g[1], cnt[1], n_polys, inverse,
-                                      scale, passes, f);
-  return ok;
 }
 
 }  // namespace ace
