@@ -67,7 +67,7 @@ struct RescaleDev {
 
 }  // namespace
 
-// Hw_* calls recorded for one launch (see flush_pending)
+// Hw_* calls recorded for one launch (see flush_run)
 struct PendingRun {
   std::vector<BatchOp> ops;
   u64 n = 0;                                  // words per operand, the same for the whole run
@@ -119,7 +119,23 @@ struct ace_ctx {
   BatchOp* run_dev = nullptr;
   u32* run_chain_dev = nullptr;
   static constexpr size_t kMaxRun = 2048;
-  void flush_pending();
+  void flush_run();
+  // A Mod_down or Rescale of one polynomial waits for the next call: generated code issues them in pairs (c0, then
+  // c1), and two polynomials through one set of launches take little longer than one, the launches of a single
+  // polynomial being far too small for the machine.  Anything else that arrives first sends it off alone.
+  struct PendingPoly {
+    int kind = 0;  // 0 none, 1 Mod_down, 2 Rescale
+    u64* res = nullptr;
+    const u64* src = nullptr;
+    size_t level = 0;
+    bool is_ntt = false;
+  } ppoly;
+  void flush_poly();
+  void submit_poly(int kind, u64* res, const u64* src, size_t level, bool is_ntt);
+  void flush_pending() {
+    flush_poly();
+    flush_run();
+  }
   bool run_accepts(const BatchOp& o, u64 n) const;
   void run_append(const BatchOp& o, u64 n);
   std::map<std::pair<size_t, size_t>, ModUpDev> modup;
@@ -475,7 +491,7 @@ bool ace_ctx::run_accepts(const BatchOp& o, u64 n) const {
 }
 
 void ace_ctx::run_append(const BatchOp& o, u64 n) {
-  if (!run_accepts(o, n)) flush_pending();
+  if (!run_accepts(o, n)) flush_run();
   run.n = n;
   run.ops.push_back(o);
   run.touched.insert((uintptr_t)o.r);
@@ -490,7 +506,7 @@ void ace_ctx::run_append(const BatchOp& o, u64 n) {
   }
 }
 
-void ace_ctx::flush_pending() {
+void ace_ctx::flush_run() {
   if (run.ops.empty()) return;
   const size_t count = run.ops.size();
   // chains: entries joined whenever one writes a range the other reads or writes (union-find over entries)
@@ -818,6 +834,47 @@ void do_mul_relin_rescale(ace_ctx* c, u64* r0, u64* r1, u64 out_stride, const u6
 
 }  // namespace
 
+static void run_poly_op(ace_ctx* c, int kind, const PolySeq& res, const PolySeq& src, size_t np, size_t level,
+                        bool is_ntt) {
+  c->ensure_ws(c->std_ws(level));
+  c->ws_used = 0;
+  if (kind == 1) do_mod_down(c, res, src, np, level, is_ntt, nullptr, 0);
+  else do_rescale(c, res, src, np, level, is_ntt);
+}
+
+void ace_ctx::flush_poly() {
+  if (!ppoly.kind) return;
+  const PendingPoly o = ppoly;
+  ppoly.kind = 0;
+  run_poly_op(this, o.kind, seq_strided(o.res, 0), seq_strided(const_cast<u64*>(o.src), 0), 1, o.level, o.is_ntt);
+}
+
+void ace_ctx::submit_poly(int kind, u64* res, const u64* src, size_t level, bool is_ntt) {
+  const size_t N = h.N;
+  const size_t res_words = (kind == 1 ? level : level - 1) * N, src_words = (kind == 1 ? level + h.K : level) * N;
+  auto overlap = [](const u64* a, size_t na, const u64* b, size_t nb) { return a < b + nb && b < a + na; };
+  if (ppoly.kind == kind && ppoly.level == level && ppoly.is_ntt == is_ntt &&
+      !overlap(res, res_words, ppoly.res, res_words) && !overlap(res, res_words, ppoly.src, src_words) &&
+      !overlap(src, src_words, ppoly.res, res_words)) {
+    const PendingPoly o = ppoly;
+    ppoly.kind = 0;
+    run_poly_op(this, kind, seq_pair(o.res, res, 0), seq_pair(const_cast<u64*>(o.src), const_cast<u64*>(src), 0), 2,
+                level, is_ntt);
+    return;
+  }
+  flush_poly();
+  if (!batching) {
+    run_poly_op(this, kind, seq_strided(res, 0), seq_strided(const_cast<u64*>(src), 0), 1, level, is_ntt);
+    return;
+  }
+  ppoly.kind = kind;
+  ppoly.res = res;
+  ppoly.src = src;
+  ppoly.level = level;
+  ppoly.is_ntt = is_ntt;
+}
+
+
 // ===========================================================================
 // ACE_HIP_PROFILE=1: host time spent inside each entry point, printed when the process ends
 namespace {
@@ -857,10 +914,11 @@ struct ScopedProf {
 
 extern "C" {
 
-#define ACE_TRY_KEEP_RUN ScopedProf prof_scope_(__func__); try {                                                 \
+#define ACE_TRY_BARE ScopedProf prof_scope_(__func__); try {                                                     \
   if (!c) return fail("null context");                                         \
   if (!c->device_ok) return fail("no HIP device: this context holds host tables only");
-#define ACE_TRY ACE_TRY_KEEP_RUN c->flush_pending();
+#define ACE_TRY_KEEP_RUN ACE_TRY_BARE c->flush_poly();
+#define ACE_TRY ACE_TRY_BARE c->flush_pending();
 #define ACE_CATCH_INT                      \
   }                                        \
   catch (const std::exception& e) {        \
@@ -1355,22 +1413,20 @@ int ace_precomp(ace_ctx* c, int64_t* res, const int64_t* src, size_t level, int 
 }
 
 int ace_mod_down(ace_ctx* c, int64_t* res, const int64_t* src, size_t level, int is_ntt) {
-  ACE_TRY
+  ACE_TRY_BARE
   if (!res || !src) return fail("ace_mod_down: null argument");
   if (!level_ok(c, level)) return fail("ace_mod_down: level out of range");
-  c->ensure_ws(c->std_ws(level));
-  c->ws_used = 0;
-  do_mod_down(c, seq_strided(U(res), 0), seq_strided(U(src), 0), 1, level, is_ntt != 0, nullptr, 0);
+  c->flush_run();
+  c->submit_poly(1, U(res), U(src), level, is_ntt != 0);
   ACE_CATCH_INT
 }
 
 int ace_rescale(ace_ctx* c, int64_t* res, const int64_t* src, size_t level, int is_ntt) {
-  ACE_TRY
+  ACE_TRY_BARE
   if (!res || !src) return fail("ace_rescale: null argument");
   if (level < 2 || level > c->h.L) return fail("Level of rescale opnd is too small");
-  c->ensure_ws(c->std_ws(level));
-  c->ws_used = 0;
-  do_rescale(c, seq_strided(U(res), 0), seq_strided(U(src), 0), 1, level, is_ntt != 0);
+  c->flush_run();
+  c->submit_poly(2, U(res), U(src), level, is_ntt != 0);
   ACE_CATCH_INT
 }
 

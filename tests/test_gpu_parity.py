@@ -239,6 +239,57 @@ def test_mod_down_rescale_extend(pair):
             g.rescale(g.alloc(N), g.alloc(N), 1, True)
 
 
+def test_mod_down_and_rescale_issued_in_pairs(pair):
+    """Two Mod_down (or Rescale) calls in a row go through one set of launches when their buffers allow it; the
+    results are those of the calls made one at a time, also when the second reads what the first wrote, when both
+    read the same operand, when the kinds or levels differ, and with recording switched off."""
+    g, o = pair.g, pair.o
+    N, K = g.N, g.K
+    for level in [l for l in levels_of(g) if l >= 2][-2:]:
+        pr = [g.primes[i] for i in g.limb_primes(level)]
+        e1, e2 = seeded.uniform_poly(300 + level, pr, N), seeded.uniform_poly(310 + level, pr, N)
+        c1, c2 = e1[:level * N].copy(), e2[:level * N].copy()
+        for is_ntt in (True, False):
+            w1, w2 = o.mod_down(e1, level, is_ntt), o.mod_down(e2, level, is_ntt)
+            v1, v2 = o.rescale(c1, level, is_ntt), o.rescale(c2, level, is_ntt)
+            for batching in (True, False):
+                g.set_batching(batching)
+                d1, d2 = g.upload(e1), g.upload(e2)
+                r1, r2, r3 = g.alloc(level * N), g.alloc(level * N), g.alloc(level * N)
+                g.mod_down(r1, d1, level, is_ntt)
+                g.mod_down(r2, d2, level, is_ntt)  # independent: paired
+                g.mod_down(r3, d1, level, is_ntt)  # waits alone; the download sends it off
+                eq(r1, w1, "first of a pair")
+                eq(r2, w2, "second of a pair")
+                eq(r3, w1, "a call left waiting")
+                g.mod_down(r1, d2, level, is_ntt)
+                g.mod_down(r2, d2, level, is_ntt)  # same operand twice
+                eq(r1, w2, "shared operand, first")
+                eq(r2, w2, "shared operand, second")
+                # the second reads what the first writes: d3 = [Mod_down(e1) | P part of e2]
+                d3 = g.upload(e2)
+                g.mod_down(d3.view(0, level * N), d1, level, is_ntt)
+                g.mod_down(r3, d3, level, is_ntt)
+                chained = np.concatenate([w1, e2[level * N:]])
+                eq(r3, o.mod_down(chained, level, is_ntt), "second depends on first")
+                # rescale pairs, and a rescale after a Mod_down
+                dc1, dc2 = g.upload(c1), g.upload(c2)
+                s1, s2 = g.alloc((level - 1) * N), g.alloc((level - 1) * N)
+                g.rescale(s1, dc1, level, is_ntt)
+                g.rescale(s2, dc2, level, is_ntt)
+                eq(s1, v1, "rescale, first of a pair")
+                eq(s2, v2, "rescale, second of a pair")
+                g.mod_down(r1, d1, level, is_ntt)
+                g.rescale(s1, r1, level, is_ntt)  # a different kind, and it reads the pending result
+                eq(s1, o.rescale(w1, level, is_ntt), "rescale of a pending Mod_down")
+                g.rescale(s1, dc1, level, is_ntt)
+                g.rescale(s1, dc2, level, is_ntt)  # same destination: the later call wins
+                eq(s1, v2, "two calls into one buffer")
+                for b in (d1, d2, d3, r1, r2, r3, dc1, dc2, s1, s2):
+                    b.free()
+            g.set_batching(True)
+
+
 def test_mod_down_rescale_family(pair):
     """Mod_down_rescale, Reduce_and_rescale_modup (both mutate their operand) and Transform_values_from_level0."""
     g, o = pair.g, pair.o
