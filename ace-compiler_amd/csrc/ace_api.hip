@@ -1052,6 +1052,9 @@ void ace_free(ace_ctx* c, int64_t* p) {
   (void)hipStreamSynchronize(c->stream);
   (void)hipFree(p);
 }
+// copies and fills longer than this go to the copy engine's / the fill kernel's own launch: a recorded entry moves
+// one word per thread, which is right for a limb and slow for a whole batch
+static constexpr size_t kRecordedWords = (size_t)1 << 20;
 int ace_upload(ace_ctx* c, int64_t* dst, const int64_t* src, size_t n) {
   ACE_TRY
   HIP_OK(hipMemcpyAsync(dst, src, n * sizeof(u64), hipMemcpyHostToDevice, c->stream));
@@ -1068,10 +1071,11 @@ int ace_copy(ace_ctx* c, int64_t* dst, const int64_t* src, size_t n) {
   ACE_TRY_KEEP_RUN
   if (!dst || !src) return fail("ace_copy: null argument");
   if (dst == src || n == 0) return 0;
-  if (c->batching) {  // a copy is an elementwise entry like any other
+  if (c->batching && n <= kRecordedWords) {  // a copy is an elementwise entry like any other
     c->run_append(BatchOp{U(dst), U(src), nullptr, 0, (u32)BATCH_COPY, 0}, n);
     return 0;
   }
+  c->flush_run();
   HIP_OK(hipMemcpyAsync(dst, src, n * sizeof(u64), hipMemcpyDeviceToDevice, c->stream));
   ACE_CATCH_INT
 }
@@ -1079,10 +1083,11 @@ int ace_zero(ace_ctx* c, int64_t* dst, size_t n) {
   ACE_TRY_KEEP_RUN
   if (!dst) return fail("ace_zero: null argument");
   if (n == 0) return 0;
-  if (c->batching) {
+  if (c->batching && n <= kRecordedWords) {
     c->run_append(BatchOp{U(dst), nullptr, nullptr, 0, (u32)BATCH_ZERO, 0}, n);
     return 0;
   }
+  c->flush_run();
   launch_fill_zero(c->stream, U(dst), n);
   ACE_CATCH_INT
 }

@@ -58,8 +58,6 @@ struct PolySeq {
   u64* b[2];
   u64 pair_stride;
   __host__ __device__ __forceinline__ u64* at(u32 p) const { return b[p & 1] + (u64)(p >> 1) * pair_stride; }
-  // the sequence that starts at polynomial p0 (even)
-  __host__ PolySeq from(u32 p0) const { return PolySeq{{at(p0), at(p0 + 1)}, pair_stride}; }
 };
 inline PolySeq seq_strided(const u64* base, u64 stride) {
   PolySeq s;

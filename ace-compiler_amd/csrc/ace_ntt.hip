@@ -38,7 +38,6 @@
 // Between the two passes the buffer holds back-end specific words (lazily
 // reduced integers, or raw FP64 bits); the second pass stores canonical
 // residues.
-#include <algorithm>
 #include <vector>
 
 #include "ace_kernels.h"
@@ -257,15 +256,16 @@ __device__ __forceinline__ void fwd_strided_body(const DevCtx& c, const PolySeq&
   constexpr int R = 1 << LOGR;
   const u32 col = blockIdx.x * 256 + threadIdx.x;
   const u64 rs = c.N >> LOGR;  // row stride
-  const u64 off = (u64)pos.prime[limb] * c.N + col;
-  u64* __restrict__ dst = dsts.at(blockIdx.z);
+  // uniform row base + per-thread 32-bit column: rows are addressed off scalar registers
+  const u64 off = (u64)pos.prime[limb] * c.N;
+  u64* __restrict__ dst = dsts.at(blockIdx.z) + off;
   A ar;
   ar.init(c, pi, false, nullptr, 0);
   typename A::T v[R];
   if (PRO == 0) {
-    const u64* __restrict__ src = srcs.at(blockIdx.z);
+    const u64* __restrict__ src = srcs.at(blockIdx.z) + off;
 #pragma unroll
-    for (int r = 0; r < R; ++r) v[r] = ar.in_canon(src[off + r * rs]);
+    for (int r = 0; r < R; ++r) v[r] = ar.in_canon((src + r * rs)[col]);
   } else {
     const DevPrime P = c.primes[pi];
     const u32 lt = pos.prime[limb];
@@ -286,13 +286,13 @@ __device__ __forceinline__ void fwd_strided_body(const DevCtx& c, const PolySeq&
   }
   fwd_strided_stages<A, LOGR>(ar, v);
 #pragma unroll
-  for (int r = 0; r < R; ++r) dst[off + r * rs] = ar.out_mid(v[r]);
+  for (int r = 0; r < R; ++r) (dst + r * rs)[col] = ar.out_mid(v[r]);
 }
 // One launch covers limbs of both arithmetic back ends: the choice is uniform over a work-group.
 template <int LOGR, int PRO>
 __global__ __launch_bounds__(256, 4) void ntt_fwd_strided(DevCtx c, PolySeq dsts, PolySeq srcs, LimbMap lm,
                                                        LimbMap pos, FwdFuse f) {
-  const u32 limb = blockIdx.y, pi = lm.prime[limb];
+  const u32 limb = gridDim.y - 1 - blockIdx.y, pi = lm.prime[limb];  // last limbs first, as in the chunk passes
   if (c.fp_ok[pi]) fwd_strided_body<ArithFp, LOGR, PRO>(c, dsts, srcs, pos, f, limb, pi);
   else fwd_strided_body<ArithInt, LOGR, PRO>(c, dsts, srcs, pos, f, limb, pi);
 }
@@ -314,7 +314,9 @@ __device__ __forceinline__ bool chunk_block(const DevCtx& c, u32 n_limbs, u32 sl
   slot_in_group = slot % slots_per_group;
   if (grp >= n_groups) return false;
   chunk = grp % n_chunks;
-  limb = grp / n_chunks;
+  // last limbs first: where a launch mixes back ends, the special primes (integer back end, 2.5x the work) sit at
+  // the end of the limb list and should not be the tail of the launch
+  limb = n_limbs - 1 - grp / n_chunks;
   return true;
 }
 static inline unsigned chunk_grid(const DevCtx& c, u32 n_limbs, u32 slots_per_group) {
@@ -586,22 +588,24 @@ __device__ __forceinline__ void inv_strided_body(const DevCtx& c, const PolySeq&
   constexpr int R = 1 << LOGR;
   const u32 col = blockIdx.x * 256 + threadIdx.x;
   const u64 rs = c.N >> LOGR;
-  const u64 off = (u64)pos.prime[limb] * c.N + col;
-  u64* __restrict__ data = datas.at(blockIdx.z);
+  u64* __restrict__ data = datas.at(blockIdx.z) + (u64)pos.prime[limb] * c.N;
   A ar;
   ar.init(c, pi, true, scale, limb);
   typename A::T v[R];
 #pragma unroll
-  for (int r = 0; r < R; ++r) v[r] = ar.in_mid(data[off + r * rs]);
+  for (int r = 0; r < R; ++r) v[r] = ar.in_mid((data + r * rs)[col]);
   inv_strided_stages<A, LOGR>(ar, v);
 #pragma unroll
-  for (int r = 0; r < R; ++r) data[off + r * rs] = ar.out_scaled(v[r]);
+  for (int r = 0; r < R; ++r) (data + r * rs)[col] = ar.out_scaled(v[r]);
 }
-template <int LOGR>
+// ONLY: 0 = limbs of both back ends (the choice is uniform over a work-group), 1 = integer limbs only, 2 = FP64
+// limbs only.  The two bodies in one function need 130 registers at LOGR = 4 where each alone needs 78 / 90, and
+// most launches are of one kind (the special primes of a Mod_down, the digit of a Mod_up).
+template <int LOGR, int ONLY>
 __global__ __launch_bounds__(256) void ntt_inv_strided(DevCtx c, PolySeq datas, LimbMap lm, LimbMap pos,
                                                        const u64* __restrict__ scale) {
-  const u32 limb = blockIdx.y, pi = lm.prime[limb];
-  if (c.fp_ok[pi]) inv_strided_body<ArithFp, LOGR>(c, datas, pos, scale, limb, pi);
+  const u32 limb = gridDim.y - 1 - blockIdx.y, pi = lm.prime[limb];
+  if (ONLY == 2 || (ONLY == 0 && c.fp_ok[pi])) inv_strided_body<ArithFp, LOGR>(c, datas, pos, scale, limb, pi);
   else inv_strided_body<ArithInt, LOGR>(c, datas, pos, scale, limb, pi);
 }
 
@@ -647,48 +651,43 @@ __global__ __launch_bounds__(256) void ntt_small(DevCtx c, PolySeq dsts, PolySeq
 }
 
 // ---------------------------------------------------------------------------
-// A plain two-pass transform of a batch larger than the 256 MiB memory-side cache runs slice by slice, both
-// passes on one slice before the next, so that the second pass finds the first one's output in that cache
-// instead of in HBM (measured on 32 polynomials of 24 limbs at N=2^16: 3 % off the round trip).
-constexpr u64 kSliceBytes = 192ull << 20, kSliceAbove = 256ull << 20;
-
 template <int LOGR>
-static void run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst_all, const PolySeq& src_all,
-                      const LimbMap& lm, const LimbMap& pos, u32 n_limbs, u32 n_polys_all, bool inverse,
-                      const u64* scale, int passes, const FwdFuse& f) {
-  const u64 poly_bytes = (u64)n_limbs * c.N * sizeof(u64);
-  u32 slice = n_polys_all;
-  if (passes == 3 && f.epi == 0 && f.pro == 0 && poly_bytes * n_polys_all > kSliceAbove)
-    slice = (u32)std::max<u64>(2, (kSliceBytes / poly_bytes) & ~1ull);
-  for (u32 p0 = 0; p0 < n_polys_all; p0 += slice) {
-    const u32 n_polys = std::min(slice, n_polys_all - p0);
-    const PolySeq dst = dst_all.from(p0), src = src_all.from(p0);
-    dim3 gs((c.N >> LOGR) / 256, n_limbs, n_polys),
-        gc(chunk_grid(c, n_limbs, (n_polys + kPolysPerBlock - 1) / kPolysPerBlock));
-    if (!inverse) {
-      if (passes & 1) {
-        if (f.pro == 0)
-          hipLaunchKernelGGL((ntt_fwd_strided<LOGR, 0>), gs, dim3(256), 0, st, c, dst, src, lm, pos, f);
-        else
-          hipLaunchKernelGGL((ntt_fwd_strided<LOGR, 1>), gs, dim3(256), 0, st, c, dst, src, lm, pos, f);
-      }
-      if (passes & 2) {
-        const u32 lr = LOGR;
-        if (f.epi == 0)
-          hipLaunchKernelGGL((ntt_fwd_chunk<0>), gc, dim3(kChunkThreads), 0, st, c, dst, lm, pos, lr, n_limbs,
-                             n_polys, f);
-        else if (f.epi == 1)
-          hipLaunchKernelGGL((ntt_fwd_chunk<1>), gc, dim3(kChunkThreads), 0, st, c, dst, lm, pos, lr, n_limbs,
-                             n_polys, f);
-        else
-          hipLaunchKernelGGL((ntt_fwd_chunk<2>), gc, dim3(kChunkThreads), 0, st, c, dst, lm, pos, lr, n_limbs,
-                             n_polys, f);
-      }
-    } else {
-      if (passes & 1)
-        hipLaunchKernelGGL(ntt_inv_chunk, gc, dim3(kChunkThreads), 0, st, c, dst, src, lm, pos, n_limbs, n_polys);
-      if (passes & 2)
-        hipLaunchKernelGGL((ntt_inv_strided<LOGR>), gs, dim3(256), 0, st, c, dst, lm, pos, scale);
+static void run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolySeq& src, const LimbMap& lm,
+                      const LimbMap& pos, u32 n_limbs, u32 n_polys, bool inverse, const u64* scale, int passes,
+                      const FwdFuse& f) {
+  dim3 gs((c.N >> LOGR) / 256, n_limbs, n_polys),
+      gc(chunk_grid(c, n_limbs, (n_polys + kPolysPerBlock - 1) / kPolysPerBlock));
+  if (!inverse) {
+    if (passes & 1) {
+      if (f.pro == 0)
+        hipLaunchKernelGGL((ntt_fwd_strided<LOGR, 0>), gs, dim3(256), 0, st, c, dst, src, lm, pos, f);
+      else
+        hipLaunchKernelGGL((ntt_fwd_strided<LOGR, 1>), gs, dim3(256), 0, st, c, dst, src, lm, pos, f);
+    }
+    if (passes & 2) {
+      const u32 lr = LOGR;
+      if (f.epi == 0)
+        hipLaunchKernelGGL((ntt_fwd_chunk<0>), gc, dim3(kChunkThreads), 0, st, c, dst, lm, pos, lr, n_limbs,
+                           n_polys, f);
+      else if (f.epi == 1)
+        hipLaunchKernelGGL((ntt_fwd_chunk<1>), gc, dim3(kChunkThreads), 0, st, c, dst, lm, pos, lr, n_limbs,
+                           n_polys, f);
+      else
+        hipLaunchKernelGGL((ntt_fwd_chunk<2>), gc, dim3(kChunkThreads), 0, st, c, dst, lm, pos, lr, n_limbs,
+                           n_polys, f);
+    }
+  } else {
+    if (passes & 1)
+      hipLaunchKernelGGL(ntt_inv_chunk, gc, dim3(kChunkThreads), 0, st, c, dst, src, lm, pos, n_limbs, n_polys);
+    if (passes & 2) {
+      u32 n_fp = 0;
+      for (u32 t = 0; t < n_limbs; ++t) n_fp += c.fp_ok[lm.prime[t]] ? 1 : 0;
+      if (n_fp == 0)
+        hipLaunchKernelGGL((ntt_inv_strided<LOGR, 1>), gs, dim3(256), 0, st, c, dst, lm, pos, scale);
+      else if (n_fp == n_limbs)
+        hipLaunchKernelGGL((ntt_inv_strided<LOGR, 2>), gs, dim3(256), 0, st, c, dst, lm, pos, scale);
+      else
+        hipLaunchKernelGGL((ntt_inv_strided<LOGR, 0>), gs, dim3(256), 0, st, c, dst, lm, pos, scale);
     }
   }
 }
