@@ -520,19 +520,59 @@ void ace_ctx::flush_run() {
     x = find(x), y = find(y);
     if (x != y) parent[std::max(x, y)] = std::min(x, y);
   };
+  // Scratch results: entry k's range is read by entry k+1 (which the kernel serves from a register), by nothing
+  // else before a later entry overwrites it.  Such a store is dropped, and the range then ties k to k+1 only:
+  // the limb-by-limb products of an inner product (Hw_modmul into one scratch limb, Hw_modadd from it) become
+  // chains of their own instead of one long chain through the scratch limb.
+  auto reads_of = [](const BatchOp& o, uintptr_t out[3]) {
+    const u32 op = o.op & ~kBatchDeadStore;
+    out[0] = op == BATCH_ZERO ? 0 : (uintptr_t)o.a;
+    out[1] = (op == BATCH_ROTATE || op == BATCH_COPY || op == BATCH_ZERO || (op >= EW_ADD_S && op <= EW_MULADD_S))
+                 ? 0 : (uintptr_t)o.b;
+    out[2] = (op == EW_MULADD || op == EW_MULADD_S) ? (uintptr_t)o.r : 0;
+  };
+  std::vector<uint8_t> scratch_read(count, 0);  // entry reads its predecessor's dropped result
+  for (u32 k = 0; k + 1 < count; ++k) {
+    BatchOp& o = run.ops[k];
+    if (o.op == BATCH_ROTATE || run.ops[k + 1].op == BATCH_ROTATE) continue;
+    const uintptr_t r = (uintptr_t)o.r;
+    uintptr_t rd[3];
+    reads_of(run.ops[k + 1], rd);
+    if (rd[0] != r && rd[1] != r && rd[2] != r) continue;
+    bool dead = false;
+    for (u32 j = k + 1; j < count && j <= k + 16; ++j) {
+      const BatchOp& n = run.ops[j];
+      if (j > k + 1) {
+        reads_of(n, rd);
+        const bool rot_touch = n.op == BATCH_ROTATE && ((uintptr_t)n.a == r || (uintptr_t)n.b == r);
+        if (rd[0] == r || rd[1] == r || rd[2] == r || rot_touch) break;
+      }
+      if ((uintptr_t)n.r == r) {
+        dead = true;
+        break;
+      }
+    }
+    if (dead) {
+      o.op |= kBatchDeadStore;
+      scratch_read[k + 1] = 1;
+    }
+  }
   std::unordered_map<uintptr_t, u32> writer;                // last entry that wrote the range
   std::unordered_map<uintptr_t, std::vector<u32>> readers;  // entries that read it since
   for (u32 k = 0; k < count; ++k) {
     const BatchOp& o = run.ops[k];
-    const bool rotate = o.op == BATCH_ROTATE;
-    const uintptr_t reads[3] = {(uintptr_t)o.a, rotate ? 0 : (uintptr_t)o.b,
-                                (o.op == EW_MULADD || o.op == EW_MULADD_S) ? (uintptr_t)o.r : 0};
+    const bool dead = (o.op & kBatchDeadStore) != 0;
+    uintptr_t reads[3];
+    reads_of(o, reads);
     for (uintptr_t x : reads) {
       if (!x) continue;
+      if (scratch_read[k] && x == (uintptr_t)run.ops[k - 1].r) continue;  // comes in a register
       auto w = writer.find(x);
       if (w != writer.end()) join(k, w->second);
       readers[x].push_back(k);
     }
+    if (scratch_read[k]) join(k, k - 1);
+    if (dead) continue;  // writes nothing
     const uintptr_t r = (uintptr_t)o.r;
     auto w = writer.find(r);
     if (w != writer.end()) join(k, w->second);

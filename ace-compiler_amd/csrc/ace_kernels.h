@@ -68,6 +68,9 @@ void launch_plain_mac(hipStream_t st, const DevCtx& c, u64* r0, u64* r1, const M
                       u32 n_limbs, u32 level, u32 plain_level, bool accumulate, u64 n);
 // a run of Hw_* calls executed as one launch: thread i carries out every entry for element i, in order
 enum BatchKind : u32 { BATCH_ROTATE = 100, BATCH_COPY = 101, BATCH_ZERO = 102 };
+// flag on BatchOp::op: the result is handed to the next entry of the chain in a register and overwritten later in
+// the run, so it need not be stored (the scratch limb between an Hw_modmul and the Hw_modadd that consumes it)
+constexpr u32 kBatchDeadStore = 0x80000000u;
 struct BatchOp {
   u64* r;
   const u64* a;

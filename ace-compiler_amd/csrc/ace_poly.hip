@@ -101,26 +101,33 @@ __global__ __launch_bounds__(kThreads) void ew_batch_small_kernel(DevCtx c, Smal
   run_chain(c, run.ops, run.chain_start[blockIdx.y], run.chain_start[blockIdx.y + 1], i);
 }
 __device__ __forceinline__ void run_chain(const DevCtx& c, const BatchOp* ops, u32 first, u32 last, u64 i) {
+  // what the previous entry produced stays in a register: an operand that names that range is not loaded again
+  const u64* prev_r = nullptr;
+  u64 prev_v = 0;
   for (u32 k = first; k < last; ++k) {
     const BatchOp o = ops[k];
+    const u32 op = o.op & ~kBatchDeadStore;
     const DevPrime P = c.primes[o.prime];
     u64 v;
-    if (o.op == BATCH_ROTATE) {
+    if (op == BATCH_ROTATE) {
       const i64 src = reinterpret_cast<const i64*>(o.b)[i];
       v = src >= 0 ? o.a[src] : P.q - o.a[-src];
-    } else if (o.op == BATCH_COPY) {
-      v = o.a[i];
-    } else if (o.op == BATCH_ZERO) {
+    } else if (op == BATCH_COPY) {
+      v = o.a == prev_r ? prev_v : o.a[i];
+    } else if (op == BATCH_ZERO) {
       v = 0;
     } else {
-      const u64 x = o.a[i];
-      const u64 y = o.op >= EW_ADD_S ? o.scalar : o.b[i];
-      if (o.op == EW_ADD || o.op == EW_ADD_S) v = add_mod(x, y, P.q);
-      else if (o.op == EW_SUB || o.op == EW_SUB_S) v = sub_mod(x, y, P.q);
-      else if (o.op == EW_MUL || o.op == EW_MUL_S) v = mulmod(x, y, P);
-      else v = add_mod(o.r[i], mulmod(x, y, P), P.q);
+      const u64 x = o.a == prev_r ? prev_v : o.a[i];
+      const u64 y = op >= EW_ADD_S ? o.scalar : (o.b == prev_r ? prev_v : o.b[i]);
+      if (op == EW_ADD || op == EW_ADD_S) v = add_mod(x, y, P.q);
+      else if (op == EW_SUB || op == EW_SUB_S) v = sub_mod(x, y, P.q);
+      else if (op == EW_MUL || op == EW_MUL_S) v = mulmod(x, y, P);
+      else v = add_mod(o.r == prev_r ? prev_v : o.r[i], mulmod(x, y, P), P.q);
     }
-    o.r[i] = v;
+    if (!(o.op & kBatchDeadStore)) o.r[i] = v;
+    // a rotate's result is never read inside its run
+    prev_r = op == BATCH_ROTATE ? nullptr : o.r;
+    prev_v = v;
   }
 }
 void launch_ew_batch_small(hipStream_t st, const DevCtx& c, const SmallRun& run, u32 n_chains, u64 n) {

@@ -655,6 +655,52 @@ def test_recorded_hw_calls_equal_calls_issued_one_by_one(pair):
     eq(y.get(), want, "recorded run")
 
 
+def test_recorded_inner_product_through_a_scratch_limb(pair):
+    """The shape generated code gives a key-switch inner product: Hw_modmul into one scratch limb, Hw_modadd from it,
+    limb after limb.  Recorded, the scratch limb travels in a register and its store is dropped where a later entry
+    overwrites it; results, and the scratch limb's final content, are those of one launch per call -- also when the
+    scratch limb is read twice, updated in place by a multiply-add, or copied before it is overwritten."""
+    g = pair.g
+    N, L, K = g.N, g.L, g.K
+    if N > 16384:
+        pytest.skip("covered at the smaller rings")
+    T = min(L + K, 9)
+    primes = list(range(T))
+    mk = lambda seed: np.concatenate([seeded.uniform_poly(seed + t, [g.primes[primes[t]]], N) for t in range(T)])
+    key, ext, acc0, spare0 = mk(7000), mk(7100), mk(7200), mk(7300)
+
+    def program():
+        dk, de, da, ds = g.upload(key), g.upload(ext), g.upload(acc0), g.upload(spare0)
+        tmp, keep = g.alloc(N), g.alloc(N)
+        limb = lambda buf, t: buf.view(t * N, N)
+        for rep in range(2):  # the second pass starts from a scratch limb that holds a value
+            for t in range(T):
+                p = primes[t]
+                g.hw("modmul", tmp, limb(dk, t), limb(de, t), p)
+                g.hw("modadd", limb(da, t), limb(da, t), tmp, p)
+                if t % 4 == 1:  # a second reader: the product has to reach memory
+                    g.hw("modsub", limb(ds, t), limb(ds, t), tmp, p)
+                if t % 4 == 2:  # updated in place before it is consumed
+                    g.hw("modmul", tmp, limb(dk, t), limb(da, t), p)
+                    g.hw("modmuladd", tmp, limb(de, t), limb(ds, t), p)
+                    g.hw("modadd", limb(ds, t), limb(ds, t), tmp, p)
+                if t % 4 == 3:  # copied out between the product and the sum
+                    g.hw("modmul", tmp, limb(de, t), limb(de, t), p)
+                    g.copy(keep, tmp)
+                    g.hw("modadd", limb(da, t), limb(da, t), tmp, p)
+        out = [da.get(), ds.get(), tmp.get(), keep.get()]
+        for b in (dk, de, da, ds, tmp, keep):
+            b.free()
+        return out
+
+    g.set_batching(False)
+    want = program()
+    g.set_batching(True)
+    got = program()
+    for w, x, what in zip(want, got, ("sums", "second readers", "scratch limb afterwards", "copy of the scratch limb")):
+        eq(x, w, what)
+
+
 def test_key_generation_helpers(pair):
     """ace_expand_small exactly; ace_sample_uniform: in range, reproducible, streams differ, and roughly uniform
     (mean, and a chi-square over 16 buckets at 6 sigma) -- it has no counterpart to compare bits with."""
