@@ -74,6 +74,7 @@ def _sig(lib):
     f("ace_host_fft_tables", C.c_int, _vp, _vp, _vp)
     f("ace_embedding_inv", C.c_int, _vp, _vp, _vp, _sz)
     f("ace_encode", C.c_int, _vp, _vp, _vp, _sz, C.c_uint32, _sz, C.c_uint32, _sz)
+    f("ace_encode_real", C.c_int, _vp, _vp, _vp, C.c_int, _sz, C.c_uint32, _sz, C.c_uint32, _sz)
     f("ace_mod_down_rescale", C.c_int, _vp, _vp, _vp, _sz, C.c_int)
     f("ace_reduce_rescale_modup", C.c_int, _vp, _vp, _vp, _vp, _sz, C.c_int)
     f("ace_transform_from_level0", C.c_int, _vp, _vp, _vp, _sz)
@@ -111,7 +112,7 @@ EXPORTS = [
     "ace_hw_modsub_scalar", "ace_hw_modmul_scalar", "ace_hw_modmuladd_scalar", "ace_hw_rotate",
     "ace_find_automorphism_index", "ace_automorphism_order", "ace_poly_add", "ace_poly_sub", "ace_poly_mul",
     "ace_poly_automorphism", "ace_decomp_modup", "ace_mod_up", "ace_mod_down_rescale",
-    "ace_reduce_rescale_modup", "ace_transform_from_level0", "ace_host_fft_tables", "ace_embedding_inv", "ace_encode", "ace_precomp", "ace_mod_down", "ace_rescale", "ace_extend",
+    "ace_reduce_rescale_modup", "ace_transform_from_level0", "ace_host_fft_tables", "ace_embedding_inv", "ace_encode", "ace_encode_real", "ace_precomp", "ace_mod_down", "ace_rescale", "ace_extend",
     "ace_dot_prod", "ace_mul_ciph3", "ace_fast_switch_key", "ace_relin", "ace_rescale_ciph",
     "ace_mul_relin_rescale", "ace_mul_relin_rescale_batch", "ace_fast_rotate", "ace_rotate_batch",
 ]
@@ -327,6 +328,13 @@ class Context:
         v = np.ascontiguousarray(values, dtype=np.complex128)
         self._chk(self.lib.ace_encode(self.h, res.ptr, v.ctypes.data_as(C.c_void_p), v.size, slots, level, sf_degree,
                                       p_cnt))
+
+    def encode_real(self, res, values, slots=0, level=0, sf_degree=1, p_cnt=0):
+        """values: a float32 or float64 array of real numbers."""
+        v = np.ascontiguousarray(values)
+        assert v.dtype in (np.float32, np.float64)
+        self._chk(self.lib.ace_encode_real(self.h, res.ptr, v.ctypes.data_as(C.c_void_p), int(v.dtype == np.float32), v.size,
+                                           slots, level, sf_degree, p_cnt))
 
     def mod_up(self, res, digit, level, part, is_ntt=True):
         self._chk(self.lib.ace_mod_up(self.h, res.ptr, digit.ptr, level, part, int(is_ntt)))

@@ -1532,8 +1532,10 @@ int ace_embedding_inv(ace_ctx* c, double* host_out, const double* host_in, size_
   ACE_CATCH_INT
 }
 
-int ace_encode(ace_ctx* c, int64_t* res, const double* values, size_t n_values, uint32_t slots, size_t level,
-               uint32_t sf_degree, size_t p_cnt) {
+// kind: 0 complex doubles (re, im interleaved), 1 real doubles, 2 real floats.  Real inputs travel as they are and
+// are widened to complex numbers on the device (a float widens exactly, as the host cast would).
+static int encode_impl(ace_ctx* c, int64_t* res, const void* values, int kind, size_t n_values, uint32_t slots,
+                       size_t level, uint32_t sf_degree, size_t p_cnt) {
   ACE_TRY
   if (!res || (!values && n_values)) return fail("ace_encode: null argument");
   if (!c->sf_bits) return fail("ace_encode: the context was created from explicit primes and has no scaling factor");
@@ -1551,14 +1553,23 @@ int ace_encode(ace_ctx* c, int64_t* res, const double* values, size_t n_values, 
   // Check_msg_range (encoder.c:48-59): the largest scaled coefficient must stay below 2^(valid bits - 1)
   const int valid = (int)c->q0_bits + (int)(level - 1) * (int)c->sf_bits;
   const double range_bound = std::ldexp(1.0, valid - 1);
+  LimbMap lm = poly_lm(c, level, p_cnt != 0);
+  const u32 n_limbs = (u32)(level + p_cnt);
+  const size_t value_bytes = kind == 0 ? sizeof(double2) : kind == 1 ? sizeof(double) : sizeof(float);
+  auto stage_values = [&](hipStream_t st, double2* z, void* raw) {  // z = the values, zero-padded to `slots`
+    if (kind == 0) {
+      if (n_values < slots)
+        launch_fill_zero(st, reinterpret_cast<u64*>(z + n_values), 2 * (size_t)(slots - n_values));
+      c->h2d(z, values, n_values * value_bytes);
+    } else {
+      c->h2d(raw, values, n_values * value_bytes);
+      launch_widen_real(st, z, raw, kind == 2, (u32)n_values, slots);
+    }
+  };
   c->ensure_ws(c->std_ws(level));
   c->ws_used = 0;
   double2* z = reinterpret_cast<double2*>(c->take(2 * (size_t)slots));
-  launch_fill_zero(c->stream, reinterpret_cast<u64*>(z), 2 * (size_t)slots);
-  if (n_values)
-    c->h2d(z, values, n_values * sizeof(double2));
-  LimbMap lm = poly_lm(c, level, p_cnt != 0);
-  const u32 n_limbs = (u32)(level + p_cnt);
+  stage_values(c->stream, z, kind == 0 ? nullptr : c->take(slots));
   launch_encode(c->stream, c->d, U(res), z, c->fft_rou, c->rot_group, slots, scaling_factor, scale, range_bound, lm,
                 n_limbs, c->d_err);
   if (sf_degree > 1) {  // encoder.c:297-312: the Q limbs are multiplied by scaling_factor^(sf_degree-1)
@@ -1577,6 +1588,14 @@ int ace_encode(ace_ctx* c, int64_t* res, const double* values, size_t n_values, 
   PolySeq rs = seq_strided(U(res), 0);
   launch_ntt(c->stream, c->d, rs, rs, lm, nullptr, n_limbs, 1, false, nullptr);
   ACE_CATCH_INT
+}
+int ace_encode(ace_ctx* c, int64_t* res, const double* values, size_t n_values, uint32_t slots, size_t level,
+               uint32_t sf_degree, size_t p_cnt) {
+  return encode_impl(c, res, values, 0, n_values, slots, level, sf_degree, p_cnt);
+}
+int ace_encode_real(ace_ctx* c, int64_t* res, const void* values, int is_f32, size_t n_values, uint32_t slots,
+                    size_t level, uint32_t sf_degree, size_t p_cnt) {
+  return encode_impl(c, res, values, is_f32 ? 2 : 1, n_values, slots, level, sf_degree, p_cnt);
 }
 
 int ace_extend(ace_ctx* c, int64_t* res, const int64_t* src, size_t level) {

@@ -135,6 +135,19 @@ void launch_embedding_inv(hipStream_t st, const DevCtx& c, double2* out, double2
                      out, r, len, loglen);
 }
 
+__global__ __launch_bounds__(256) void widen_real_kernel(double2* __restrict__ z, const void* __restrict__ raw,
+                                                         int is_f32, u32 n_values, u32 slots) {
+  const u32 i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= slots) return;
+  double v = 0.0;
+  if (i < n_values) v = is_f32 ? (double)static_cast<const float*>(raw)[i] : static_cast<const double*>(raw)[i];
+  z[i] = make_double2(v, 0.0);
+}
+void launch_widen_real(hipStream_t st, double2* z, const void* raw, bool is_f32, u32 n_values, u32 slots) {
+  hipLaunchKernelGGL(widen_real_kernel, dim3((slots + 255) / 256), dim3(256), 0, st, z, raw, is_f32 ? 1 : 0, n_values,
+                     slots);
+}
+
 void launch_encode(hipStream_t st, const DevCtx& c, u64* out, double2* r, const double2* rou, const u32* rot,
                    u32 slots, double scaling_factor, double scale, double range_bound, const LimbMap& lm,
                    u32 n_limbs, int* err) {

@@ -156,6 +156,8 @@ void launch_embedding_inv(hipStream_t st, const DevCtx& c, double2* out, double2
 // Encode_impl up to the residues (coefficient form): r holds `slots` complex values on entry (zero-padded
 // message) and is used as scratch; rou = exp(2 pi i k / 2N), k < 2N; rot = 5^k mod 2N, k < N/2.
 // out: n_limbs limbs of N words (limb t uses lm.prime[t]).  *err is set to 1 where the reference asserts.
+// z[i] = (raw[i], 0) for i < n_values, (0, 0) up to slots; raw holds doubles or floats
+void launch_widen_real(hipStream_t st, double2* z, const void* raw, bool is_f32, u32 n_values, u32 slots);
 void launch_encode(hipStream_t st, const DevCtx& c, u64* out, double2* r, const double2* rou, const u32* rot,
                    u32 slots, double scaling_factor, double scale, double range_bound, const LimbMap& lm,
                    u32 n_limbs, int* err);

@@ -270,26 +270,27 @@ static void encode_vector(PLAIN plain, const double* re_im, size_t len, uint32_t
   init_plain(plain, level, pow(G.sc, sc_degree), sc_degree, G.N / 2);
   ACE_OK(ace_encode(G.ctx, plain->_poly._data, re_im, len, 0, level, sc_degree, 0));
 }
+/* real-valued messages go to the device as they are (doubles or floats) and are widened there */
+void Rt_encode_real(PLAIN plain, const void* values, int is_f32, size_t len, uint32_t sc_degree, uint32_t level) {
+  if (level == 0) level = (uint32_t)G.L;
+  FMT_ASSERT(level <= G.L, "level should not be larger than mul_depth + 1");
+  init_plain(plain, level, pow(G.sc, sc_degree), sc_degree, G.N / 2);
+  ACE_OK(ace_encode_real(G.ctx, plain->_poly._data, values, is_f32, len, 0, level, sc_degree, 0));
+}
 
 void Encode_double(PLAIN plain, double* input, size_t len, uint32_t sc_degree, uint32_t level) {
   if (len == 1) {
     encode_value(plain, *input, sc_degree, level);
     return;
   }
-  double* v = (double*)calloc(2 * len, sizeof(double));
-  for (size_t i = 0; i < len; ++i) v[2 * i] = input[i];
-  encode_vector(plain, v, len, sc_degree, level);
-  free(v);
+  Rt_encode_real(plain, input, 0, len, sc_degree, level);
 }
 void Encode_float(PLAIN plain, float* input, size_t len, uint32_t sc_degree, uint32_t level) {
   if (len == 1) {
     encode_value(plain, (double)*input, sc_degree, level);
     return;
   }
-  double* v = (double*)calloc(2 * len, sizeof(double));
-  for (size_t i = 0; i < len; ++i) v[2 * i] = (double)input[i];
-  encode_vector(plain, v, len, sc_degree, level);
-  free(v);
+  Rt_encode_real(plain, input, 1, len, sc_degree, level);
 }
 void Encode_dcmplx(PLAIN plain, DCMPLX* input, size_t len, uint32_t sc_degree, uint32_t level) {
   encode_vector(plain, (const double*)input, len, sc_degree, level);

@@ -35,6 +35,10 @@ _Static_assert(sizeof(DATA_HDR) == 136 && sizeof(LUT_ENTRY) == 32, "side-file re
 static struct {
   bool       open, synthetic;
   double     amplitude;
+  /* synthetic entries are made once and kept, as a file's entries are: [index] -> values from 0 on */
+  double** syn;
+  size_t*  syn_len;
+  size_t   syn_count;
   DATA_HDR   hdr;
   LUT_ENTRY* lut;
   char*      buf; /* the bytes between the first page and the lookup table */
@@ -76,23 +80,22 @@ bool Pt_mgr_init(const char* fname) {
 }
 
 void Pt_mgr_fini(void) {
+  for (size_t i = 0; i < Data.syn_count; ++i) free(Data.syn[i]);
+  free(Data.syn);
+  free(Data.syn_len);
   free(Data.lut);
   free(Data.buf);
   memset(&Data, 0, sizeof(Data));
 }
+
+static const double* synthetic_entry(uint32_t index, size_t upto);
 
 /* entry `index` from value `first` on, `len` values, as doubles */
 static double* entry_values(uint32_t index, size_t first, size_t len) {
   FMT_ASSERT(Data.open, "the program has no rt data file (Get_rt_data_info)");
   double* v = (double*)malloc((len ? len : 1) * sizeof(double));
   if (Data.synthetic) {
-    for (size_t i = 0; i < len; ++i) {
-      uint64_t z = ((uint64_t)index << 32 | (uint64_t)(first + i)) + 0x9E3779B97F4A7C15ull;
-      z          = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
-      z          = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
-      z ^= z >> 31;
-      v[i] = Data.amplitude * ((double)(int64_t)(z >> 11) / (double)(1ull << 52) - 1.0);
-    }
+    memcpy(v, synthetic_entry(index, first + len) + first, len * sizeof(double));
     return v;
   }
   size_t width = Data.hdr.ent_type == DE_MSG_F32 ? sizeof(float) : sizeof(double);
@@ -113,7 +116,54 @@ static double* entry_values(uint32_t index, size_t first, size_t len) {
   return v;
 }
 
+/* the entry's values where they lie (floats or doubles of the file, possibly unaligned: only ever copied) */
+static const double* synthetic_entry(uint32_t index, size_t upto) {
+  if (index >= Data.syn_count) {
+    size_t n     = (size_t)index + 64;
+    Data.syn     = (double**)realloc(Data.syn, n * sizeof(double*));
+    Data.syn_len = (size_t*)realloc(Data.syn_len, n * sizeof(size_t));
+    for (size_t i = Data.syn_count; i < n; ++i) {
+      Data.syn[i]     = NULL;
+      Data.syn_len[i] = 0;
+    }
+    Data.syn_count = n;
+  }
+  if (Data.syn_len[index] < upto) {
+    Data.syn[index] = (double*)realloc(Data.syn[index], upto * sizeof(double));
+    for (size_t i = Data.syn_len[index]; i < upto; ++i) {
+      uint64_t z = ((uint64_t)index << 32 | (uint64_t)i) + 0x9E3779B97F4A7C15ull;
+      z          = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+      z          = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+      z ^= z >> 31;
+      Data.syn[index][i] = Data.amplitude * ((double)(int64_t)(z >> 11) / (double)(1ull << 52) - 1.0);
+    }
+    Data.syn_len[index] = upto;
+  }
+  return Data.syn[index];
+}
+
+static const void* entry_bytes(uint32_t index, size_t first, size_t len, int* is_f32) {
+  FMT_ASSERT(Data.open, "the program has no rt data file (Get_rt_data_info)");
+  if (Data.synthetic) {
+    *is_f32 = 0;
+    return synthetic_entry(index, first + len) + first;
+  }
+  size_t width = Data.hdr.ent_type == DE_MSG_F32 ? sizeof(float) : sizeof(double);
+  FMT_ASSERT(index < Data.hdr.ent_count, "index out of entry range");
+  const LUT_ENTRY* e = &Data.lut[index];
+  FMT_ASSERT(e->size >= (first + len) * width, "entry size too small");
+  FMT_ASSERT(e->ofst >= DATA_PAGE && e->ofst - DATA_PAGE + (first + len) * width <= Data.size, "entry offset too large");
+  *is_f32 = width == sizeof(float);
+  return Data.buf + (e->ofst - DATA_PAGE) + first * width;
+}
+
 void* Pt_from_msg_ofst(void* pt, uint32_t index, size_t ofst, size_t len, uint32_t scale, uint32_t level) {
+  int         is_f32 = 0;
+  const void* raw    = len > 1 ? entry_bytes(index, ofst, len, &is_f32) : NULL;
+  if (raw) {
+    Rt_encode_real((PLAIN)pt, raw, is_f32, len, scale, level);
+    return pt;
+  }
   double* v = entry_values(index, ofst, len);
   Encode_double((PLAIN)pt, v, len, scale, level);
   free(v);

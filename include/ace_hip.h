@@ -204,6 +204,11 @@ int ace_embedding_inv(ace_ctx* ctx, double* host_out, const double* host_in, siz
  * reported by the next ace_sync / ace_download. */
 int ace_encode(ace_ctx* ctx, int64_t* res, const double* values, size_t n_values, uint32_t slots, size_t level,
                uint32_t sf_degree, size_t p_cnt);
+/* The same for real-valued messages (Encode_float / Encode_double, ckks/src/plain.c:29-63, and the weight
+ * plaintexts of Pt_from_msg, pt_mgr.c): `values` is a HOST array of n_values doubles (is_f32 = 0) or floats
+ * (is_f32 = 1), widened to complex numbers with zero imaginary part on the device. */
+int ace_encode_real(ace_ctx* ctx, int64_t* res, const void* values, int is_f32, size_t n_values, uint32_t slots,
+                    size_t level, uint32_t sf_degree, size_t p_cnt);
 /* Extend (:483-500): src level limbs -> res level+num_p limbs (P limbs zero) */
 int ace_extend(ace_ctx* ctx, int64_t* res, const int64_t* src, size_t level);
 /* Dot_prod / Fast_dot_prod (:502-529): digits = n_parts x (level+num_p) limbs;

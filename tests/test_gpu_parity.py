@@ -340,6 +340,30 @@ def test_encode(pair):
             dr = g.alloc((level + pc) * N)
             g.encode(dr, vals, slots, level, deg, pc)
             eq(dr, want, "encode slots=%d level=%d sf_degree=%d p=%d" % (slots, level, deg, pc))
+    # real-valued messages (doubles, floats) are widened on the device: same residues as the complex form, with
+    # calls recorded and issued one by one
+    for side in (True, False):
+        g.set_batching(side)
+        for slots, n in ((N // 2, N // 2), (N // 2, max(1, N // 8)), (max(1, N // 4), 1)):
+            for level, deg, pc in ((g.L, 1, 0), (max(1, g.L - 1), 1, g.K)):
+                if deg * sf_bits >= q0_bits + (level - 1) * sf_bits:
+                    continue
+                for dt in (np.float64, np.float32):
+                    x = rng.uniform(-2, 2, n).astype(dt)
+                    want = o.encode(x.astype(np.float64).astype(np.complex128), slots, level, deg, pc)
+                    dr = g.alloc((level + pc) * N)
+                    g.encode_real(dr, x, slots, level, deg, pc)
+                    eq(dr, want, "encode_real %s n=%d slots=%d level=%d p=%d" % (dt.__name__, n, slots, level, pc))
+                    # several in a row into one buffer, consumed between them
+                    acc = g.alloc((level + pc) * N)
+                    for rep in range(10):
+                        y = rng.uniform(-1, 1, n).astype(dt)
+                        g.encode_real(dr, y, slots, level, deg, pc)
+                        g.copy(acc, dr)
+                    eq(acc, o.encode(y.astype(np.float64).astype(np.complex128), slots, level, deg, pc), "tenth in a row")
+                    dr.free()
+                    acc.free()
+    g.set_batching(True)
     # a value too large for the level: the reference asserts, the library reports it at the next synchronisation
     if q0_bits + (g.L - 1) * sf_bits - sf_bits < 62:
         big = np.array([2.0 ** (q0_bits + (g.L - 1) * sf_bits - sf_bits)])
