@@ -270,6 +270,13 @@ static void encode_vector(PLAIN plain, const double* re_im, size_t len, uint32_t
   init_plain(plain, level, pow(G.sc, sc_degree), sc_degree, G.N / 2);
   ACE_OK(ace_encode(G.ctx, plain->_poly._data, re_im, len, 0, level, sc_degree, 0));
 }
+/* a plaintext of `level` limbs at scale degree sc_degree whose polynomial the caller fills in (NTT form) */
+int64_t* Rt_plain_prepare(PLAIN plain, uint32_t sc_degree, uint32_t level) {
+  if (level == 0) level = (uint32_t)G.L;
+  FMT_ASSERT(level <= G.L, "level should not be larger than mul_depth + 1");
+  init_plain(plain, level, pow(G.sc, sc_degree), sc_degree, G.N / 2);
+  return plain->_poly._data;
+}
 /* real-valued messages go to the device as they are (doubles or floats) and are widened there */
 void Rt_encode_real(PLAIN plain, const void* values, int is_f32, size_t len, uint32_t sc_degree, uint32_t level) {
   if (level == 0) level = (uint32_t)G.L;

@@ -45,7 +45,62 @@ static struct {
   uint64_t   size;
 } Data;
 
+/* Encoded weight plaintexts kept in HBM.  A program encodes the same entries for every input it is run on (the
+ * reference avoids that only with files of pre-encoded plaintexts); with a few hundred GB of HBM the encoded
+ * polynomial of each (entry, range, scale degree, level) is kept after its first use and copied from then on.
+ * RT_HIP_PLAINTEXT_CACHE_GB bounds the space (default 48; 0 switches it off). */
+typedef struct {
+  uint64_t k1, k2; /* (index, scale, level), (offset, length); k1 == 0 marks a free cell (level is never 0) */
+  int64_t* dev;
+} PT_CELL;
+static struct {
+  PT_CELL*  cell;
+  size_t    cap, count, words, limit_words;
+  int64_t** slab; /* the polynomials live in 1 GiB slabs: one device allocation per 100-odd plaintexts */
+  size_t    n_slabs, slab_left;
+} Cache;
+#define PT_SLAB_WORDS ((size_t)1 << 27)
+
+static int64_t* cache_room(size_t words) {
+  if (words > PT_SLAB_WORDS) return NULL;
+  if (Cache.slab_left < words) {
+    Cache.slab                  = (int64_t**)realloc(Cache.slab, (Cache.n_slabs + 1) * sizeof(int64_t*));
+    Cache.slab[Cache.n_slabs++] = Rt_dev_alloc_raw(PT_SLAB_WORDS);
+    Cache.slab_left             = PT_SLAB_WORDS;
+  }
+  int64_t* p = Cache.slab[Cache.n_slabs - 1] + (PT_SLAB_WORDS - Cache.slab_left);
+  Cache.slab_left -= words;
+  return p;
+}
+
+static PT_CELL* cache_find(uint64_t k1, uint64_t k2) {
+  if (!Cache.cap) return NULL;
+  uint64_t h = (k1 * 0x9E3779B97F4A7C15ull) ^ (k2 * 0xC2B2AE3D27D4EB4Full);
+  for (size_t i = (size_t)(h >> 20) & (Cache.cap - 1);; i = (i + 1) & (Cache.cap - 1)) {
+    PT_CELL* c = &Cache.cell[i];
+    if (c->k1 == 0 || (c->k1 == k1 && c->k2 == k2)) return c;
+  }
+}
+static void cache_grow(void) {
+  PT_CELL* old     = Cache.cell;
+  size_t   old_cap = Cache.cap;
+  Cache.cap        = old_cap ? 2 * old_cap : 4096;
+  Cache.cell       = (PT_CELL*)calloc(Cache.cap, sizeof(PT_CELL));
+  for (size_t i = 0; i < old_cap; ++i)
+    if (old[i].k1) *cache_find(old[i].k1, old[i].k2) = old[i];
+  free(old);
+}
+static void cache_clear(void) {
+  for (size_t i = 0; i < Cache.n_slabs; ++i) Rt_dev_free(Cache.slab[i]);
+  free(Cache.slab);
+  free(Cache.cell);
+  memset(&Cache, 0, sizeof(Cache));
+}
+
 bool Pt_mgr_init(const char* fname) {
+  const char* gb    = getenv("RT_HIP_PLAINTEXT_CACHE_GB");
+  cache_clear();
+  Cache.limit_words = (size_t)((gb ? atof(gb) : 48.0) * (double)(1ull << 27));
   const char* over = getenv("RT_HIP_DATA_FILE");
   const char* syn  = getenv("RT_HIP_SYNTHETIC_WEIGHTS");
   if (over && *over) fname = over;
@@ -80,6 +135,7 @@ bool Pt_mgr_init(const char* fname) {
 }
 
 void Pt_mgr_fini(void) {
+  cache_clear();
   for (size_t i = 0; i < Data.syn_count; ++i) free(Data.syn[i]);
   free(Data.syn);
   free(Data.syn_len);
@@ -89,6 +145,7 @@ void Pt_mgr_fini(void) {
 }
 
 static const double* synthetic_entry(uint32_t index, size_t upto);
+static void          Pt_encode_entry(void* pt, uint32_t index, size_t ofst, size_t len, uint32_t scale, uint32_t level);
 
 /* entry `index` from value `first` on, `len` values, as doubles */
 static double* entry_values(uint32_t index, size_t first, size_t len) {
@@ -158,16 +215,39 @@ static const void* entry_bytes(uint32_t index, size_t first, size_t len, int* is
 }
 
 void* Pt_from_msg_ofst(void* pt, uint32_t index, size_t ofst, size_t len, uint32_t scale, uint32_t level) {
+  const size_t   words = (size_t)(level ? level : Get_q_cnt()) * Degree();
+  const uint64_t k1    = ((uint64_t)index << 32) | ((uint64_t)(scale & 0xFFFF) << 16) | (level ? level : Get_q_cnt());
+  const uint64_t k2    = ((uint64_t)ofst << 32) | (uint64_t)len;
+  PT_CELL*       cell  = NULL;
+  if (Cache.limit_words && len > 1 && ofst < (1ull << 32) && len < (1ull << 32) && scale < 0x10000) {
+    if (4 * (Cache.count + 1) > 3 * Cache.cap) cache_grow();
+    cell = cache_find(k1, k2);
+    if (cell->k1) { /* encoded before: the polynomial is copied */
+      Rt_copy_words(Rt_plain_prepare((PLAIN)pt, scale, level), cell->dev, words);
+      return pt;
+    }
+    if (Cache.words + words > Cache.limit_words) cell = NULL;
+  }
+  Pt_encode_entry(pt, index, ofst, len, scale, level);
+  if (cell && (cell->dev = cache_room(words)) != NULL) {
+    Rt_copy_words(cell->dev, ((PLAIN)pt)->_poly._data, words);
+    cell->k1 = k1;
+    cell->k2 = k2;
+    ++Cache.count;
+    Cache.words += words;
+  }
+  return pt;
+}
+static void Pt_encode_entry(void* pt, uint32_t index, size_t ofst, size_t len, uint32_t scale, uint32_t level) {
   int         is_f32 = 0;
   const void* raw    = len > 1 ? entry_bytes(index, ofst, len, &is_f32) : NULL;
   if (raw) {
     Rt_encode_real((PLAIN)pt, raw, is_f32, len, scale, level);
-    return pt;
+    return;
   }
   double* v = entry_values(index, ofst, len);
   Encode_double((PLAIN)pt, v, len, scale, level);
   free(v);
-  return pt;
 }
 void* Pt_from_msg(void* pt, uint32_t index, size_t len, uint32_t scale, uint32_t level) {
   return Pt_from_msg_ofst(pt, index, 0, len, scale, level);

@@ -132,6 +132,7 @@ int64_t* Rt_dev_alloc_raw(size_t n_words) { /* not zero-filled: for buffers writ
   if (!p) Rt_fatal(__FILE__, __LINE__, "device allocation of %zu words failed: %s", n_words, ace_last_error());
   return p;
 }
+void Rt_copy_words(int64_t* dst, const int64_t* src, size_t n_words) { ACE_OK(ace_copy(G.ctx, dst, src, n_words)); }
 void Rt_dev_free(int64_t* p) {
   if (p && G.ctx) ace_free(G.ctx, p);
 }

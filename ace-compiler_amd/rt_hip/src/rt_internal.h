@@ -68,6 +68,8 @@ size_t   Rt_sin_series(size_t hamming_weight, int even, double* coeff, uint32_t*
 void     Rt_series_divide(double* q, size_t* n_q, double* r, size_t* n_r, const double* f, size_t n_f, const double* g, size_t n_g);
 /* Encode_val: `level` residues of trunc(value * scale), large products through the approximation factor */
 void     Rt_encode_val_words(int64_t* res, double value, uint32_t level, double scale);
+void     Rt_copy_words(int64_t* dst, const int64_t* src, size_t n_words);
+int64_t* Rt_plain_prepare(PLAIN plain, uint32_t sc_degree, uint32_t level);
 void     Rt_encode_real(PLAIN plain, const void* values, int is_f32, size_t len, uint32_t sc_degree, uint32_t level);
 
 #endif

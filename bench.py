@@ -181,14 +181,20 @@ def resnet20_leg():
         return {"resnet20": {"skipped": "the model binary is built only where the reference tree is present"}}
     try:
         env = dict(os.environ, RT_HIP_SYNTHETIC_WEIGHTS="0.05")
-        r = subprocess.run([exe, "3", "32", "32", "10", "1"], capture_output=True, text=True, timeout=400, env=env)
+        # three images one after another: the first pays for encoding every weight plaintext, the later ones find
+        # the encoded polynomials in HBM
+        r = subprocess.run([exe, "3", "32", "32", "10", "1", "3"], capture_output=True, text=True, timeout=400, env=env)
         line = [l for l in r.stdout.splitlines() if l.startswith("context_s")][0].split()
         vals = dict(zip(line[0::2], (float(v) for v in line[1::2])))
-        return {"resnet20": {"workload": "ResNet-20 CIFAR-10 inference of one image, the reference's generated program, "
-                                         "synthetic weights and image", "main_graph_s": vals["main_graph_s"],
-                             "keygen_s": vals["keygen_s"], "input_s": vals["input_s"], "output_s": vals["output_s"],
-                             "exit_status": r.returncode, "published_cpu_s": 1453.96,
-                             "vs_published_cpu": round(1453.96 / vals["main_graph_s"], 1)}}
+        later = [float(l.split()[5]) for l in r.stdout.splitlines() if l.startswith("image ")]
+        out = {"workload": "ResNet-20 CIFAR-10 inference, the reference's generated program, synthetic weights and "
+                           "images, three images one after another", "main_graph_s": vals["main_graph_s"],
+               "keygen_s": vals["keygen_s"], "input_s": vals["input_s"], "output_s": vals["output_s"],
+               "exit_status": r.returncode, "published_cpu_s": 1453.96,
+               "vs_published_cpu": round(1453.96 / vals["main_graph_s"], 1)}
+        if later:
+            out["main_graph_s_later_images"] = later
+        return {"resnet20": out}
     except Exception as e:
         return {"resnet20": {"error": repr(e)[:200]}}
 

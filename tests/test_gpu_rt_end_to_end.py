@@ -170,13 +170,19 @@ def test_plaintexts_from_a_weight_file(dtype, tmp_path):
     entries = [("w%d" % i, rng.uniform(-1, 1, n).astype(np_type), 1, level) for i, n in enumerate((5, 2048, 77, 1000))]
     path, out_path = str(tmp_path / "weights.msg"), str(tmp_path / "out.bin")
     msgfile.write(path, entries, np_type)
-    picks = [(1, 0, 2048), (3, 0, 900), (2, 10, 60), (0, 0, 5)]
+    # the last three repeat earlier ones: served from the encoded plaintexts kept in HBM
+    picks = [(1, 0, 2048), (3, 0, 900), (2, 10, 60), (0, 0, 5), (3, 0, 900), (1, 0, 2048), (2, 10, 60)]
     args = [MSG, path, str(N), str(cfg[1] - 1), str(cfg[2]), str(cfg[3]), str(cfg[4]), str(level), out_path]
     for p in picks:
         args += [str(v) for v in p]
     r = run(args, 0)
     assert r.returncode == 0, r.stdout + r.stderr
     got = np.fromfile(out_path, np.int64).reshape(len(picks), level * N)
+    if dtype == "f64":  # and with nothing kept
+        env = dict(os.environ, RT_HIP_PLAINTEXT_CACHE_GB="0")
+        r2 = subprocess.run(args, capture_output=True, text=True, timeout=110, env=env)
+        assert r2.returncode == 0, r2.stdout + r2.stderr
+        assert np.array_equal(np.fromfile(out_path, np.int64).reshape(len(picks), level * N), got)
     o = Oracle(*cfg)
     for row, (index, ofst, n) in zip(got, picks):
         values = np.asarray(entries[index][1][ofst:ofst + n], np.float64).astype(np.complex128)
