@@ -74,6 +74,7 @@ def _sig(lib):
     f("ace_host_fft_tables", C.c_int, _vp, _vp, _vp)
     f("ace_embedding_inv", C.c_int, _vp, _vp, _vp, _sz)
     f("ace_encode", C.c_int, _vp, _vp, _vp, _sz, C.c_uint32, _sz, C.c_uint32, _sz)
+    f("ace_ext_rotate", C.c_int, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp, _sz)
     f("ace_encode_real", C.c_int, _vp, _vp, _vp, C.c_int, _sz, C.c_uint32, _sz, C.c_uint32, _sz)
     f("ace_mod_down_rescale", C.c_int, _vp, _vp, _vp, _sz, C.c_int)
     f("ace_reduce_rescale_modup", C.c_int, _vp, _vp, _vp, _vp, _sz, C.c_int)
@@ -112,7 +113,7 @@ EXPORTS = [
     "ace_hw_modsub_scalar", "ace_hw_modmul_scalar", "ace_hw_modmuladd_scalar", "ace_hw_rotate",
     "ace_find_automorphism_index", "ace_automorphism_order", "ace_poly_add", "ace_poly_sub", "ace_poly_mul",
     "ace_poly_automorphism", "ace_decomp_modup", "ace_mod_up", "ace_mod_down_rescale",
-    "ace_reduce_rescale_modup", "ace_transform_from_level0", "ace_host_fft_tables", "ace_embedding_inv", "ace_encode", "ace_encode_real", "ace_precomp", "ace_mod_down", "ace_rescale", "ace_extend",
+    "ace_reduce_rescale_modup", "ace_transform_from_level0", "ace_host_fft_tables", "ace_embedding_inv", "ace_encode", "ace_encode_real", "ace_ext_rotate", "ace_precomp", "ace_mod_down", "ace_rescale", "ace_extend",
     "ace_dot_prod", "ace_mul_ciph3", "ace_fast_switch_key", "ace_relin", "ace_rescale_ciph",
     "ace_mul_relin_rescale", "ace_mul_relin_rescale_batch", "ace_fast_rotate", "ace_rotate_batch",
 ]
@@ -350,6 +351,10 @@ class Context:
 
     def extend(self, res, src, level):
         self._chk(self.lib.ace_extend(self.h, res.ptr, src.ptr, level))
+
+    def ext_rotate(self, out0, out1, digits, key, key_half_words, key_stride, n_parts, addend0, order, level):
+        self._chk(self.lib.ace_ext_rotate(self.h, out0.ptr, out1.ptr, digits.ptr, key.ptr, key_half_words, key_stride,
+                                          n_parts, addend0.ptr if addend0 is not None else None, order.ptr, level))
 
     def dot_prod(self, res, digits, key, key_stride, n_parts, level):
         self._chk(self.lib.ace_dot_prod(self.h, res.ptr, digits.ptr, key.ptr, key_stride, n_parts, level))

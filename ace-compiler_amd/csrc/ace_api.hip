@@ -1620,6 +1620,24 @@ int ace_dot_prod(ace_ctx* c, int64_t* res, const int64_t* digits, const int64_t*
   ACE_CATCH_INT
 }
 
+int ace_ext_rotate(ace_ctx* c, int64_t* out0, int64_t* out1, const int64_t* digits, const int64_t* key,
+                   size_t key_half_words, size_t key_stride, size_t n_parts, const int64_t* addend0,
+                   const int64_t* order, size_t level) {
+  ACE_TRY
+  if (!out0 || !out1 || !digits || !key || !order) return fail("ace_ext_rotate: null argument");
+  if (!level_ok(c, level)) return fail("ace_ext_rotate: level out of range");
+  if (n_parts == 0 || n_parts > c->h.parts) return fail("ace_ext_rotate: number of digits out of range");
+  const size_t T = level + c->h.K, words = T * (size_t)c->h.N;
+  auto overlap = [&](const int64_t* a, const int64_t* b, size_t nb) { return a < b + nb && b < a + words; };
+  if (overlap(out0, digits, n_parts * words) || overlap(out1, digits, n_parts * words) || overlap(out0, out1, words) ||
+      (addend0 && (overlap(out0, addend0, words) || overlap(out1, addend0, words))))
+    return fail("ace_ext_rotate: the results must not overlap the operands (the automorphism is applied on the way in)");
+  LimbMap lm = poly_lm(c, level, true), kp = key_pos(c, level);
+  launch_ext_rotate(c->stream, c->d, U(out0), U(out1), U(digits), words, U(key), key_half_words, key_stride,
+                    (u32)n_parts, addend0 ? U(addend0) : nullptr, order, lm, kp, (u32)T);
+  ACE_CATCH_INT
+}
+
 // ---- ciphertext level ------------------------------------------------------------
 int ace_mul_ciph3(ace_ctx* c, int64_t* d0, int64_t* d1, int64_t* d2, const int64_t* a0, const int64_t* a1,
                   const int64_t* b0, const int64_t* b1, size_t level) {

@@ -493,16 +493,12 @@ static void ext_free(EXT_CT* e) {
 }
 /* both key halves against hoisted digits, then the automorphism (Fast_rotate_ext, evaluator.c:532-566) */
 static void ext_rotate(EXT_CT* out, const int64_t* digits, size_t n_digits, const int64_t* c0_ext, int32_t rot,
-                       size_t level, EXT_CT* tmp) {
+                       size_t level) {
   ROT_KEY* key = Rt_find_rot(rot);
   FMT_ASSERT(key, "cannot find auto key of rotation %d", rot);
-  size_t         half = (G.L + G.K) * G.N;
-  const int64_t* k0   = key->swk._public_keys->dev;
-  ACE_OK(ace_dot_prod(G.ctx, tmp->c0, digits, k0, 2 * half, n_digits, level));
-  ACE_OK(ace_dot_prod(G.ctx, tmp->c1, digits, k0 + half, 2 * half, n_digits, level));
-  if (c0_ext) ACE_OK(ace_poly_add(G.ctx, tmp->c0, tmp->c0, c0_ext, level, 1));
-  ACE_OK(ace_poly_automorphism(G.ctx, out->c0, tmp->c0, key->order, level, 1));
-  ACE_OK(ace_poly_automorphism(G.ctx, out->c1, tmp->c1, key->order, level, 1));
+  size_t half = (G.L + G.K) * G.N;
+  ACE_OK(ace_ext_rotate(G.ctx, out->c0, out->c1, digits, key->swk._public_keys->dev, half, 2 * half, n_digits, c0_ext,
+                        key->order, level));
 }
 static void rotate_iteration(CIPHER ct, BTS_PRECOM* pre, bool encoding, int32_t s, bool is_rem, bool first_step) {
   const FFT_PLAN* p      = encoding ? &pre->enc : &pre->dec;
@@ -515,12 +511,12 @@ static void rotate_iteration(CIPHER ct, BTS_PRECOM* pre, bool encoding, int32_t 
   ACE_OK(ace_precomp(G.ctx, digits, ct->_c1_poly._data, level, 1));
   int64_t* c0_ext = Rt_dev_alloc_raw(T * n);
   ACE_OK(ace_extend(G.ctx, c0_ext, ct->_c0_poly._data, level));
-  EXT_CT  tmp = ext_alloc(level), inner = ext_alloc(level), outer = ext_alloc(level);
+  EXT_CT  inner = ext_alloc(level), outer = ext_alloc(level), turned = ext_alloc(level);
   EXT_CT* rots = (EXT_CT*)calloc((size_t)r.giant, sizeof(EXT_CT));
   for (int32_t j = 0; j < r.giant; ++j) {
     rots[j] = ext_alloc(level);
     if (r.in[j] != 0) {
-      ext_rotate(&rots[j], digits, nd, c0_ext, r.in[j], level, &tmp);
+      ext_rotate(&rots[j], digits, nd, c0_ext, r.in[j], level);
     } else { /* Switch_key_ext: the ciphertext itself, lifted */
       Rt_dev_copy(rots[j].c0, c0_ext, T * n);
       ACE_OK(ace_extend(G.ctx, rots[j].c1, ct->_c1_poly._data, level));
@@ -552,9 +548,9 @@ static void rotate_iteration(CIPHER ct, BTS_PRECOM* pre, bool encoding, int32_t 
       ACE_OK(ace_poly_add(G.ctx, first, first, moved, level, 1));
       ACE_OK(ace_mod_down(G.ctx, low, inner.c1, level, 1));
       ACE_OK(ace_precomp(G.ctx, low_digits, low, level, 1));
-      ext_rotate(&inner, low_digits, nd, NULL, r.out[i], level, &tmp);
-      ACE_OK(ace_poly_add(G.ctx, outer.c0, outer.c0, inner.c0, level, 1));
-      ACE_OK(ace_poly_add(G.ctx, outer.c1, outer.c1, inner.c1, level, 1));
+      ext_rotate(&turned, low_digits, nd, NULL, r.out[i], level);
+      ACE_OK(ace_poly_add(G.ctx, outer.c0, outer.c0, turned.c0, level, 1));
+      ACE_OK(ace_poly_add(G.ctx, outer.c1, outer.c1, turned.c1, level, 1));
     } else {
       ACE_OK(ace_poly_add(G.ctx, first, first, inner.c0, level, 1));
       ACE_OK(ace_poly_add(G.ctx, outer.c1, outer.c1, inner.c1, level, 1));
@@ -568,7 +564,7 @@ static void rotate_iteration(CIPHER ct, BTS_PRECOM* pre, bool encoding, int32_t 
 
   for (int32_t j = 0; j < r.giant; ++j) ext_free(&rots[j]);
   free(rots);
-  ext_free(&tmp);
+  ext_free(&turned);
   ext_free(&inner);
   ext_free(&outer);
   Rt_dev_free(digits);

@@ -239,6 +239,38 @@ def test_mod_down_rescale_extend(pair):
             g.rescale(g.alloc(N), g.alloc(N), 1, True)
 
 
+def test_ext_rotate_equals_its_parts(pair):
+    """The fused extended-basis rotation = two inner products with the key halves, the addend, two automorphisms
+    (each of which is checked against the oracle on its own)."""
+    g = pair.g
+    N = g.N
+    for level in sorted({g.L, max(1, g.L - 1)}):
+        nd, T = g.num_decomp(level), level + g.K
+        pr = [g.primes[i] for i in g.limb_primes(level)]
+        digits = g.upload(np.concatenate([seeded.uniform_poly(8000 + d, pr, N) for d in range(nd)]))
+        swk = g.upload(make_swk(g, 8100 + level))
+        addend = g.upload(seeded.uniform_poly(8200, pr, N))
+        half = (g.L + g.K) * N
+        for rot in (1, -3):
+            order = g.automorphism_order(g.find_automorphism_index(rot), True)
+            t0, t1, w0, w1 = (g.alloc(T * N) for _ in range(4))
+            g.dot_prod(t0, digits, swk, 2 * half, nd, level)
+            g.dot_prod(t1, digits, swk.view(half, swk.n - half), 2 * half, nd, level)
+            for with_addend in (True, False):
+                if with_addend:
+                    g.poly("add", t0, t0, addend, level, True)
+                g.poly("automorphism", w0, t0, order, level, True)
+                g.poly("automorphism", w1, t1, order, level, True)
+                r0, r1 = g.alloc(T * N), g.alloc(T * N)
+                g.ext_rotate(r0, r1, digits, swk, half, 2 * half, nd, addend if with_addend else None, order, level)
+                eq(r0, w0.get(), "first half, level %d rot %d addend %d" % (level, rot, with_addend))
+                eq(r1, w1.get(), "second half, level %d rot %d" % (level, rot))
+                if with_addend:  # undo for the pass without
+                    g.dot_prod(t0, digits, swk, 2 * half, nd, level)
+            with pytest.raises(acefhe.AceError):
+                g.ext_rotate(digits.view(0, T * N), r1, digits, swk, half, 2 * half, nd, None, order, level)
+
+
 def test_mod_down_and_rescale_issued_in_pairs(pair):
     """Two Mod_down (or Rescale) calls in a row go through one set of launches when their buffers allow it; the
     results are those of the calls made one at a time, also when the second reads what the first wrote, when both
