@@ -74,6 +74,7 @@ def _sig(lib):
     f("ace_host_fft_tables", C.c_int, _vp, _vp, _vp)
     f("ace_embedding_inv", C.c_int, _vp, _vp, _vp, _sz)
     f("ace_encode", C.c_int, _vp, _vp, _vp, _sz, C.c_uint32, _sz, C.c_uint32, _sz)
+    f("ace_ext_plain_mac_groups", C.c_int, _vp, _vp, _vp, _sz, _vp, _vp, _sz, _vp, _sz, _sz)
     f("ace_ext_rotate", C.c_int, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp, _sz)
     f("ace_encode_real", C.c_int, _vp, _vp, _vp, C.c_int, _sz, C.c_uint32, _sz, C.c_uint32, _sz)
     f("ace_mod_down_rescale", C.c_int, _vp, _vp, _vp, _sz, C.c_int)
@@ -113,7 +114,7 @@ EXPORTS = [
     "ace_hw_modsub_scalar", "ace_hw_modmul_scalar", "ace_hw_modmuladd_scalar", "ace_hw_rotate",
     "ace_find_automorphism_index", "ace_automorphism_order", "ace_poly_add", "ace_poly_sub", "ace_poly_mul",
     "ace_poly_automorphism", "ace_decomp_modup", "ace_mod_up", "ace_mod_down_rescale",
-    "ace_reduce_rescale_modup", "ace_transform_from_level0", "ace_host_fft_tables", "ace_embedding_inv", "ace_encode", "ace_encode_real", "ace_ext_rotate", "ace_precomp", "ace_mod_down", "ace_rescale", "ace_extend",
+    "ace_reduce_rescale_modup", "ace_transform_from_level0", "ace_host_fft_tables", "ace_embedding_inv", "ace_encode", "ace_encode_real", "ace_ext_rotate", "ace_ext_plain_mac_groups", "ace_precomp", "ace_mod_down", "ace_rescale", "ace_extend",
     "ace_dot_prod", "ace_mul_ciph3", "ace_fast_switch_key", "ace_relin", "ace_rescale_ciph",
     "ace_mul_relin_rescale", "ace_mul_relin_rescale_batch", "ace_fast_rotate", "ace_rotate_batch",
 ]
@@ -413,6 +414,17 @@ class Context:
         pp = (_vp * n)(*[a.ptr for a in plains])
         self._chk(self.lib.ace_ext_plain_mac(self.h, r0.ptr, r1.ptr, p0, p1, pp, C.c_size_t(n), C.c_size_t(level),
                                              C.c_size_t(plain_level), C.c_int(int(accumulate))))
+
+    def ext_plain_mac_groups(self, r0s, r1s, a0s, a1s, plains, level, plain_level):
+        """plains[g][j]: the plaintext of group g, operand j, or None."""
+        ng, n = len(r0s), len(a0s)
+        q0 = (_vp * ng)(*[r.ptr for r in r0s])
+        q1 = (_vp * ng)(*[r.ptr for r in r1s])
+        p0 = (_vp * n)(*[a.ptr for a in a0s])
+        p1 = (_vp * n)(*[a.ptr for a in a1s])
+        pp = (_vp * (ng * n))(*[(plains[g][j].ptr if plains[g][j] is not None else None) for g in range(ng) for j in range(n)])
+        self._chk(self.lib.ace_ext_plain_mac_groups(self.h, q0, q1, C.c_size_t(ng), p0, p1, C.c_size_t(n), pp,
+                                                    C.c_size_t(level), C.c_size_t(plain_level)))
 
     def rotate_batch(self, r0s, r1s, c0, c1, swks, orders, level):
         n = len(swks)

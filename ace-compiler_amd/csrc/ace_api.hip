@@ -1353,6 +1353,47 @@ int ace_ext_plain_mac(ace_ctx* c, int64_t* r0, int64_t* r1, const int64_t* const
   ACE_CATCH_INT
 }
 
+int ace_ext_plain_mac_groups(ace_ctx* c, int64_t* const* r0, int64_t* const* r1, size_t n_groups,
+                             const int64_t* const* a0, const int64_t* const* a1, size_t count,
+                             const int64_t* const* plain, size_t level, size_t plain_level) {
+  ACE_TRY
+  if (!r0 || !r1 || !a0 || !a1 || !plain) return fail("ace_ext_plain_mac_groups: null argument");
+  if (!level_ok(c, level) || !level_ok(c, plain_level) || plain_level < level)
+    return fail("ace_ext_plain_mac_groups: levels out of range (the plaintext may not sit below the ciphertext)");
+  if (!count || !n_groups) return fail("ace_ext_plain_mac_groups: no operands");
+  for (size_t g = 0; g < n_groups; ++g) {
+    if (!r0[g] || !r1[g]) return fail("ace_ext_plain_mac_groups: null result");
+    for (size_t h = 0; h < n_groups; ++h)
+      if (r0[g] == r1[h] || (g != h && (r0[g] == r0[h] || r1[g] == r1[h])))
+        return fail("ace_ext_plain_mac_groups: two results share a buffer");
+    for (size_t j = 0; j < count; ++j) {
+      if (!a0[j] || !a1[j]) return fail("ace_ext_plain_mac_groups: null operand");
+      if (a0[j] == r0[g] || a0[j] == r1[g] || a1[j] == r0[g] || a1[j] == r1[g])
+        return fail("ace_ext_plain_mac_groups: an operand aliases a result");
+    }
+  }
+  LimbMap lm = poly_lm(c, level, true);
+  for (size_t g0 = 0; g0 < n_groups; g0 += kMacGroups) {
+    for (size_t done = 0; done < count; done += kMacGroupOps) {
+      MacGroups ops{};
+      ops.n_groups = (u32)std::min<size_t>(kMacGroups, n_groups - g0);
+      ops.n_ops = (u32)std::min<size_t>(kMacGroupOps, count - done);
+      for (u32 g = 0; g < ops.n_groups; ++g) {
+        ops.r0[g] = U(r0[g0 + g]);
+        ops.r1[g] = U(r1[g0 + g]);
+        for (u32 j = 0; j < ops.n_ops; ++j) ops.p[g][j] = U(plain[(g0 + g) * count + done + j]);
+      }
+      for (u32 j = 0; j < ops.n_ops; ++j) {
+        ops.a0[j] = U(a0[done + j]);
+        ops.a1[j] = U(a1[done + j]);
+      }
+      launch_plain_mac_groups(c->stream, c->d, ops, lm, (u32)(level + c->h.K), (u32)level, (u32)plain_level, done != 0,
+                              c->h.N);
+    }
+  }
+  ACE_CATCH_INT
+}
+
 static int poly_scalars(ace_ctx* c, bool mul, int64_t* r, const int64_t* a, const int64_t* scalars, size_t level) {
   ACE_TRY
   if (!r || !a || !scalars) return fail("ace_poly_scalars: null argument");

@@ -66,6 +66,19 @@ struct MacSet { // operands of one multiply-accumulate launch
 // at plain_level + (t - level) above it
 void launch_plain_mac(hipStream_t st, const DevCtx& c, u64* r0, u64* r1, const MacSet& ops, const LimbMap& lm,
                       u32 n_limbs, u32 level, u32 plain_level, bool accumulate, u64 n);
+// The same for up to kMacGroups groups that share the operands (a0_j, a1_j) and differ in their plaintexts: the
+// operands, two thirds of the traffic of a single group, are read once.  p[g][j] == nullptr: group g has no term j.
+constexpr int kMacGroups = 4, kMacGroupOps = 16;
+struct MacGroups {
+  u64* r0[kMacGroups];
+  u64* r1[kMacGroups];
+  const u64* a0[kMacGroupOps];
+  const u64* a1[kMacGroupOps];
+  const u64* p[kMacGroups][kMacGroupOps];
+  u32 n_groups, n_ops;
+};
+void launch_plain_mac_groups(hipStream_t st, const DevCtx& c, const MacGroups& ops, const LimbMap& lm, u32 n_limbs,
+                             u32 level, u32 plain_level, bool accumulate, u64 n);
 // a run of Hw_* calls executed as one launch: thread i carries out every entry for element i, in order
 enum BatchKind : u32 { BATCH_ROTATE = 100, BATCH_COPY = 101, BATCH_ZERO = 102 };
 // flag on BatchOp::op: the result is handed to the next entry of the chain in a register and overwritten later in

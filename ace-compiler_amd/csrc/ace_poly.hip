@@ -85,6 +85,48 @@ void launch_plain_mac(hipStream_t st, const DevCtx& c, u64* r0, u64* r1, const M
                      plain_level, accumulate ? 1 : 0, n);
 }
 
+__global__ __launch_bounds__(kThreads) void plain_mac_groups_kernel(DevCtx c, MacGroups ops, LimbMap lm, u32 level,
+                                                                    u32 plain_level, int accumulate, u64 n) {
+  const u32 limb = blockIdx.y;
+  const DevPrime P = c.primes[lm.prime[limb]];
+  const u64 base = (u64)limb * n;
+  const u64 pbase = (u64)(limb < level ? limb : plain_level + (limb - level)) * n;
+#pragma unroll
+  ACE_EW_LOOP(i, n) {
+    u64 s0[kMacGroups], s1[kMacGroups];
+#pragma unroll
+    for (int g = 0; g < kMacGroups; ++g) {
+      const bool on = g < (int)ops.n_groups && accumulate;
+      s0[g] = on ? ops.r0[g][base + i] : 0;
+      s1[g] = on ? ops.r1[g][base + i] : 0;
+    }
+    for (u32 j = 0; j < ops.n_ops; ++j) {
+      const u64 x0 = ops.a0[j][base + i], x1 = ops.a1[j][base + i];
+#pragma unroll
+      for (int g = 0; g < kMacGroups; ++g) {
+        if (g < (int)ops.n_groups && ops.p[g][j]) {
+          const u64 w = ops.p[g][j][pbase + i];
+          s0[g] = add_mod(s0[g], mulmod(x0, w, P), P.q);
+          s1[g] = add_mod(s1[g], mulmod(x1, w, P), P.q);
+        }
+      }
+    }
+#pragma unroll
+    for (int g = 0; g < kMacGroups; ++g) {
+      if (g < (int)ops.n_groups) {
+        ops.r0[g][base + i] = s0[g];
+        ops.r1[g][base + i] = s1[g];
+      }
+    }
+  }
+}
+void launch_plain_mac_groups(hipStream_t st, const DevCtx& c, const MacGroups& ops, const LimbMap& lm, u32 n_limbs,
+                             u32 level, u32 plain_level, bool accumulate, u64 n) {
+  if (!n || !n_limbs || !ops.n_ops || !ops.n_groups) return;
+  hipLaunchKernelGGL(plain_mac_groups_kernel, ew_grid(n, n_limbs), dim3(kThreads), 0, st, c, ops, lm, level,
+                     plain_level, accumulate ? 1 : 0, n);
+}
+
 // ---- a recorded run of Hw_* calls (hal/src/hal.c:15-138) in one launch --------------------------------
 // The host splits a run into chains that share no written range; a chain's entries are carried out in order by
 // the thread of element i, so an entry may read what an earlier one of its chain wrote (identical ranges only;

@@ -524,38 +524,57 @@ static void rotate_iteration(CIPHER ct, BTS_PRECOM* pre, bool encoding, int32_t 
   }
   int64_t *first = Rt_dev_alloc_raw(T * n), *moved = Rt_dev_alloc_raw(T * n), *low = Rt_dev_alloc_raw(level * n);
   int64_t* low_digits = Rt_dev_alloc_raw(nd * T * n);
-  const int64_t *in0[64], *in1[64], *inp[64];
+  /* the inner sums of all baby-step groups first: the groups share the rotated ciphertexts, which are read once
+   * for every four groups (ace_ext_plain_mac_groups) */
+  EXT_CT*         inners = (EXT_CT*)calloc((size_t)r.baby, sizeof(EXT_CT));
+  int64_t **      in_r0 = (int64_t**)calloc((size_t)r.baby, sizeof(int64_t*)), **in_r1 = (int64_t**)calloc((size_t)r.baby, sizeof(int64_t*));
+  const int64_t** inp   = (const int64_t**)calloc((size_t)r.baby * (size_t)r.giant, sizeof(int64_t*));
+  const int64_t * in0[64], *in1[64];
+  FMT_ASSERT(r.giant <= 64, "too many rotations in one baby-step group");
+  size_t plain_level = 0;
+  for (int32_t j = 0; j < r.giant; ++j) {
+    in0[j] = rots[j].c0;
+    in1[j] = rots[j].c1;
+  }
   for (int32_t i = 0; i < r.baby; ++i) {
-    size_t count = 0, plain_level = 0;
+    inners[i] = i == 0 ? inner : ext_alloc(level);
+    in_r0[i]  = inners[i].c0;
+    in_r1[i]  = inners[i].c1;
     for (int32_t j = 0; j < r.giant; ++j) {
       int32_t d = r.giant * i + j;
-      if (d == r.num_rot) continue;
+      if (d == r.num_rot) continue; /* stays NULL: no such term */
       FMT_ASSERT(plains[d]._poly._num_primes >= level, "bootstrap plaintext below the ciphertext level");
-      plain_level  = plains[d]._poly._num_primes;
-      in0[count]   = rots[j].c0;
-      in1[count]   = rots[j].c1;
-      inp[count++] = plains[d]._poly._data;
+      plain_level            = plains[d]._poly._num_primes;
+      inp[i * r.giant + j] = plains[d]._poly._data;
     }
-    ACE_OK(ace_ext_plain_mac(G.ctx, inner.c0, inner.c1, in0, in1, inp, count, level, plain_level, 0));
+  }
+  ACE_OK(ace_ext_plain_mac_groups(G.ctx, in_r0, in_r1, (size_t)r.baby, in0, in1, (size_t)r.giant, inp, level, plain_level));
+  for (int32_t i = 0; i < r.baby; ++i) {
+    EXT_CT* in = &inners[i];
     if (i == 0) { /* the c0 parts are summed aside and meet the c1 parts at the end */
-      Rt_dev_copy(first, inner.c0, T * n);
+      Rt_dev_copy(first, in->c0, T * n);
       ACE_OK(ace_zero(G.ctx, outer.c0, T * n));
-      Rt_dev_copy(outer.c1, inner.c1, T * n);
+      Rt_dev_copy(outer.c1, in->c1, T * n);
     } else if (r.out[i] != 0) {
       ROT_KEY* key = Rt_find_rot(r.out[i]);
       FMT_ASSERT(key, "cannot find auto key of rotation %d", r.out[i]);
-      ACE_OK(ace_poly_automorphism(G.ctx, moved, inner.c0, key->order, level, 1));
+      ACE_OK(ace_poly_automorphism(G.ctx, moved, in->c0, key->order, level, 1));
       ACE_OK(ace_poly_add(G.ctx, first, first, moved, level, 1));
-      ACE_OK(ace_mod_down(G.ctx, low, inner.c1, level, 1));
+      ACE_OK(ace_mod_down(G.ctx, low, in->c1, level, 1));
       ACE_OK(ace_precomp(G.ctx, low_digits, low, level, 1));
       ext_rotate(&turned, low_digits, nd, NULL, r.out[i], level);
       ACE_OK(ace_poly_add(G.ctx, outer.c0, outer.c0, turned.c0, level, 1));
       ACE_OK(ace_poly_add(G.ctx, outer.c1, outer.c1, turned.c1, level, 1));
     } else {
-      ACE_OK(ace_poly_add(G.ctx, first, first, inner.c0, level, 1));
-      ACE_OK(ace_poly_add(G.ctx, outer.c1, outer.c1, inner.c1, level, 1));
+      ACE_OK(ace_poly_add(G.ctx, first, first, in->c0, level, 1));
+      ACE_OK(ace_poly_add(G.ctx, outer.c1, outer.c1, in->c1, level, 1));
     }
   }
+  for (int32_t i = 1; i < r.baby; ++i) ext_free(&inners[i]);
+  free(inners);
+  free(in_r0);
+  free(in_r1);
+  free((void*)inp);
   ACE_OK(ace_poly_add(G.ctx, outer.c0, outer.c0, first, level, 1));
   ACE_OK(ace_mod_down(G.ctx, ct->_c0_poly._data, outer.c0, level, 1));
   ACE_OK(ace_mod_down(G.ctx, ct->_c1_poly._data, outer.c1, level, 1));

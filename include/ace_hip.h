@@ -168,6 +168,12 @@ int ace_expand_small(ace_ctx* ctx, int64_t* res, const int64_t* small_host, size
  * device pointers; no operand may alias the result. */
 int ace_ext_plain_mac(ace_ctx* ctx, int64_t* r0, int64_t* r1, const int64_t* const* a0, const int64_t* const* a1,
                       const int64_t* const* plain, size_t count, size_t level, size_t plain_level, int accumulate);
+/* The same for n_groups baby-step groups over the same operands: (r0[g], r1[g]) = sum_j (a0[j], a1[j]) *
+ * plain[g * count + j]; a NULL plaintext means group g has no term j.  The operands are read once for up to four
+ * groups.  No result may share a buffer with an operand or with another result. */
+int ace_ext_plain_mac_groups(ace_ctx* ctx, int64_t* const* r0, int64_t* const* r1, size_t n_groups,
+                             const int64_t* const* a0, const int64_t* const* a1, size_t count,
+                             const int64_t* const* plain, size_t level, size_t plain_level);
 /* Decomp_modup (:160-258) (== Decomp :74-105 + Mod_up :107-158): digit `part`
  * of src (level limbs) raised to level+num_p limbs. */
 int ace_decomp_modup(ace_ctx* ctx, int64_t* res, const int64_t* src, size_t level, size_t part, int is_ntt);

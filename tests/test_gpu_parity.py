@@ -613,6 +613,36 @@ def test_ext_plain_mac(pair):
         g.ext_plain_mac(r0, r1, d0[:1], d1[:1], dp[:1], L, level)
 
 
+def test_ext_plain_mac_groups_equal_single_groups(pair):
+    """Several baby-step groups over the same operands in one call = one ace_ext_plain_mac per group (checked against
+    the oracle above): 6 groups (two launches of up to four), 19 operands (two launches of up to sixteen), terms
+    missing from some groups."""
+    g = pair.g
+    N, L, K = g.N, g.L, g.K
+    if N > 16384:
+        pytest.skip("covered at the smaller rings")
+    level = max(1, L - 1)
+    primes_ct = list(g.primes[:level]) + list(g.primes[L:])
+    count, groups = 19, 6
+    d0 = [g.upload(seeded.uniform_poly(3300 + j, primes_ct, N)) for j in range(count)]
+    d1 = [g.upload(seeded.uniform_poly(3400 + j, primes_ct, N)) for j in range(count)]
+    dp = [[g.upload(seeded.uniform_poly(3500 + 40 * b + j, list(g.primes), N)) for j in range(count)] for b in range(groups)]
+    dp[1][4] = dp[5][18] = dp[5][0] = None
+    T = level + K
+    r0s, r1s = [g.alloc(T * N) for _ in range(groups)], [g.alloc(T * N) for _ in range(groups)]
+    g.ext_plain_mac_groups(r0s, r1s, d0, d1, dp, level, L)
+    w0, w1 = g.alloc(T * N), g.alloc(T * N)
+    for b in range(groups):
+        keep = [j for j in range(count) if dp[b][j] is not None]
+        g.ext_plain_mac(w0, w1, [d0[j] for j in keep], [d1[j] for j in keep], [dp[b][j] for j in keep], level, L)
+        eq(r0s[b].get(), w0.get(), "group %d, first half" % b)
+        eq(r1s[b].get(), w1.get(), "group %d, second half" % b)
+    with pytest.raises(RuntimeError):
+        g.ext_plain_mac_groups([r0s[0], r0s[0]], r1s[:2], d0, d1, dp[:2], level, L)
+    with pytest.raises(RuntimeError):
+        g.ext_plain_mac_groups([d0[0]], r1s[:1], d0, d1, dp[:1], level, L)
+
+
 def test_limb_scalars_and_weighted_sum(pair):
     """Per-limb scalar add / multiply and the weighted sum of ciphertexts against limb-wise oracle calls."""
     g, o = pair.g, pair.o
