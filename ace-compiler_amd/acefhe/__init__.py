@@ -75,7 +75,7 @@ def _sig(lib):
     f("ace_embedding_inv", C.c_int, _vp, _vp, _vp, _sz)
     f("ace_encode", C.c_int, _vp, _vp, _vp, _sz, C.c_uint32, _sz, C.c_uint32, _sz)
     f("ace_ext_plain_mac_groups", C.c_int, _vp, _vp, _vp, _sz, _vp, _vp, _sz, _vp, _sz, _sz)
-    f("ace_ext_rotate", C.c_int, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp, _sz)
+    f("ace_ext_rotate", C.c_int, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp, _sz, C.c_int)
     f("ace_encode_real", C.c_int, _vp, _vp, _vp, C.c_int, _sz, C.c_uint32, _sz, C.c_uint32, _sz)
     f("ace_mod_down_rescale", C.c_int, _vp, _vp, _vp, _sz, C.c_int)
     f("ace_reduce_rescale_modup", C.c_int, _vp, _vp, _vp, _vp, _sz, C.c_int)
@@ -353,9 +353,11 @@ class Context:
     def extend(self, res, src, level):
         self._chk(self.lib.ace_extend(self.h, res.ptr, src.ptr, level))
 
-    def ext_rotate(self, out0, out1, digits, key, key_half_words, key_stride, n_parts, addend0, order, level):
+    def ext_rotate(self, out0, out1, digits, key, key_half_words, key_stride, n_parts, addend0, order, level,
+                   accumulate=0):
         self._chk(self.lib.ace_ext_rotate(self.h, out0.ptr, out1.ptr, digits.ptr, key.ptr, key_half_words, key_stride,
-                                          n_parts, addend0.ptr if addend0 is not None else None, order.ptr, level))
+                                          n_parts, addend0.ptr if addend0 is not None else None, order.ptr, level,
+                                          accumulate))
 
     def dot_prod(self, res, digits, key, key_stride, n_parts, level):
         self._chk(self.lib.ace_dot_prod(self.h, res.ptr, digits.ptr, key.ptr, key_stride, n_parts, level))

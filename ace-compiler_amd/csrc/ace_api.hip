@@ -1663,7 +1663,7 @@ int ace_dot_prod(ace_ctx* c, int64_t* res, const int64_t* digits, const int64_t*
 
 int ace_ext_rotate(ace_ctx* c, int64_t* out0, int64_t* out1, const int64_t* digits, const int64_t* key,
                    size_t key_half_words, size_t key_stride, size_t n_parts, const int64_t* addend0,
-                   const int64_t* order, size_t level) {
+                   const int64_t* order, size_t level, int accumulate) {
   ACE_TRY
   if (!out0 || !out1 || !digits || !key || !order) return fail("ace_ext_rotate: null argument");
   if (!level_ok(c, level)) return fail("ace_ext_rotate: level out of range");
@@ -1675,7 +1675,7 @@ int ace_ext_rotate(ace_ctx* c, int64_t* out0, int64_t* out1, const int64_t* digi
     return fail("ace_ext_rotate: the results must not overlap the operands (the automorphism is applied on the way in)");
   LimbMap lm = poly_lm(c, level, true), kp = key_pos(c, level);
   launch_ext_rotate(c->stream, c->d, U(out0), U(out1), U(digits), words, U(key), key_half_words, key_stride,
-                    (u32)n_parts, addend0 ? U(addend0) : nullptr, order, lm, kp, (u32)T);
+                    (u32)n_parts, addend0 ? U(addend0) : nullptr, order, accumulate & 3, lm, kp, (u32)T);
   ACE_CATCH_INT
 }
 

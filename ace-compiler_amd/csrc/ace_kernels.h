@@ -137,10 +137,11 @@ void launch_digit_copy(hipStream_t st, const DevCtx& c, u64* res, const u64* src
 void launch_dotprod(hipStream_t st, const DevCtx& c, u64* out0, u64* out1, u64 out_stride, const u64* digits,
                     u64 digit_stride, u64 digits_op_stride, const KeySet& keys, u64 key1_off, u64 key_stride,
                     u32 n_parts, const LimbMap& lm, const LimbMap& key_limb, u32 n_limbs, u32 n_ops);
-// out0[i] = (sum_d digit_d * key0_d)[order[i]] (+ addend0[order[i]]), out1[i] = (sum_d digit_d * key1_d)[order[i]]
+// out0[i] (+)= (sum_d digit_d * key0_d)[order[i]] (+ addend0[order[i]]), out1[i] (+)= (sum_d digit_d * key1_d)[order[i]];
+// accumulate bit 0 / 1: add to what out0 / out1 holds
 void launch_ext_rotate(hipStream_t st, const DevCtx& c, u64* out0, u64* out1, const u64* digits, u64 digit_stride,
                        const u64* key0, u64 key1_off, u64 key_stride, u32 n_parts, const u64* addend0, const i64* order,
-                       const LimbMap& lm, const LimbMap& key_limb, u32 n_limbs);
+                       int accumulate, const LimbMap& lm, const LimbMap& key_limb, u32 n_limbs);
 // Mod_down tail for n_polys polynomials: out = (src - y) * pinv (+ addend), per limb constants cst[2t], cst[2t+1];
 // addend_mode 0 none, 1 every polynomial, 2 even polynomials only.  With `orders` the result is permuted on the
 // way out: out[i] = value at orders[p / 2][i] (the automorphism closing a rotation; out must not alias an input).

@@ -529,13 +529,13 @@ __global__ __launch_bounds__(kThreads) void dotprod_kernel(DevCtx c, u64* __rest
 // A rotation in the extended basis without its Mod_down (Fast_rotate_ext, evaluator.c:503-566, as bootstrapping
 // uses it): both halves of the inner product with the rotation key, an optional addend on the first half, and the
 // automorphism, in one pass.  The gather is applied on the way in: out[i] = value at order[i], so writes stay
-// coalesced.  NTT form only (no negative index entries).
+// coalesced.  NTT form only (no negative index entries).  accumulate: bit 0 adds to what out0 holds, bit 1 to out1.
 __global__ __launch_bounds__(kThreads) void ext_rotate_kernel(DevCtx c, u64* __restrict__ out0, u64* __restrict__ out1,
                                                               const u64* __restrict__ digits, u64 digit_stride,
                                                               const u64* __restrict__ key0, u64 key1_off, u64 key_stride,
                                                               u32 n_parts, const u64* __restrict__ addend0,
-                                                              const i64* __restrict__ order, LimbMap lm,
-                                                              LimbMap key_limb) {
+                                                              const i64* __restrict__ order, int accumulate,
+                                                              LimbMap lm, LimbMap key_limb) {
   const u32 limb = blockIdx.y;
   const DevPrime P = c.primes[lm.prime[limb]];
   const u64 n = c.N, dbase = (u64)limb * n, kbase = (u64)key_limb.prime[limb] * n;
@@ -553,18 +553,20 @@ __global__ __launch_bounds__(kThreads) void ext_rotate_kernel(DevCtx c, u64* __r
         l1 = barrett128(h1, l1, P); h1 = 0;
       }
     }
-    u64 v0 = barrett128(h0, l0, P);
+    u64 v0 = barrett128(h0, l0, P), v1 = barrett128(h1, l1, P);
     if (addend0) v0 = add_mod(v0, addend0[dbase + j], P.q);
+    if (accumulate & 1) v0 = add_mod(v0, out0[dbase + i], P.q);
+    if (accumulate & 2) v1 = add_mod(v1, out1[dbase + i], P.q);
     out0[dbase + i] = v0;
-    out1[dbase + i] = barrett128(h1, l1, P);
+    out1[dbase + i] = v1;
   }
 }
 void launch_ext_rotate(hipStream_t st, const DevCtx& c, u64* out0, u64* out1, const u64* digits, u64 digit_stride,
                        const u64* key0, u64 key1_off, u64 key_stride, u32 n_parts, const u64* addend0, const i64* order,
-                       const LimbMap& lm, const LimbMap& key_limb, u32 n_limbs) {
+                       int accumulate, const LimbMap& lm, const LimbMap& key_limb, u32 n_limbs) {
   if (!n_limbs) return;
   hipLaunchKernelGGL(ext_rotate_kernel, ew_grid(c.N, n_limbs, 1), dim3(kThreads), 0, st, c, out0, out1, digits,
-                     digit_stride, key0, key1_off, key_stride, n_parts, addend0, order, lm, key_limb);
+                     digit_stride, key0, key1_off, key_stride, n_parts, addend0, order, accumulate, lm, key_limb);
 }
 
 // The same for operands that share one key: each thread keeps its 2*NP key

@@ -492,13 +492,15 @@ static void ext_free(EXT_CT* e) {
   Rt_dev_free(e->c1);
 }
 /* both key halves against hoisted digits, then the automorphism (Fast_rotate_ext, evaluator.c:532-566) */
+/* (out.c0, out.c1) = the rotation by `rot` of (sum of digits * key halves) + (c0_ext, 0), all in the extended basis;
+ * accumulate bit 0 / 1: added to what out.c0 / out.c1 holds */
 static void ext_rotate(EXT_CT* out, const int64_t* digits, size_t n_digits, const int64_t* c0_ext, int32_t rot,
-                       size_t level) {
+                       size_t level, int accumulate) {
   ROT_KEY* key = Rt_find_rot(rot);
   FMT_ASSERT(key, "cannot find auto key of rotation %d", rot);
   size_t half = (G.L + G.K) * G.N;
   ACE_OK(ace_ext_rotate(G.ctx, out->c0, out->c1, digits, key->swk._public_keys->dev, half, 2 * half, n_digits, c0_ext,
-                        key->order, level));
+                        key->order, level, accumulate));
 }
 static void rotate_iteration(CIPHER ct, BTS_PRECOM* pre, bool encoding, int32_t s, bool is_rem, bool first_step) {
   const FFT_PLAN* p      = encoding ? &pre->enc : &pre->dec;
@@ -511,18 +513,18 @@ static void rotate_iteration(CIPHER ct, BTS_PRECOM* pre, bool encoding, int32_t 
   ACE_OK(ace_precomp(G.ctx, digits, ct->_c1_poly._data, level, 1));
   int64_t* c0_ext = Rt_dev_alloc_raw(T * n);
   ACE_OK(ace_extend(G.ctx, c0_ext, ct->_c0_poly._data, level));
-  EXT_CT  inner = ext_alloc(level), outer = ext_alloc(level), turned = ext_alloc(level);
+  EXT_CT  inner = ext_alloc(level), outer = ext_alloc(level);
   EXT_CT* rots = (EXT_CT*)calloc((size_t)r.giant, sizeof(EXT_CT));
   for (int32_t j = 0; j < r.giant; ++j) {
     rots[j] = ext_alloc(level);
     if (r.in[j] != 0) {
-      ext_rotate(&rots[j], digits, nd, c0_ext, r.in[j], level);
+      ext_rotate(&rots[j], digits, nd, c0_ext, r.in[j], level, 0);
     } else { /* Switch_key_ext: the ciphertext itself, lifted */
       Rt_dev_copy(rots[j].c0, c0_ext, T * n);
       ACE_OK(ace_extend(G.ctx, rots[j].c1, ct->_c1_poly._data, level));
     }
   }
-  int64_t *first = Rt_dev_alloc_raw(T * n), *moved = Rt_dev_alloc_raw(T * n), *low = Rt_dev_alloc_raw(level * n);
+  int64_t* low = Rt_dev_alloc_raw(level * n);
   int64_t* low_digits = Rt_dev_alloc_raw(nd * T * n);
   /* the inner sums of all baby-step groups first: the groups share the rotated ciphertexts, which are read once
    * for every four groups (ace_ext_plain_mac_groups) */
@@ -549,47 +551,41 @@ static void rotate_iteration(CIPHER ct, BTS_PRECOM* pre, bool encoding, int32_t 
     }
   }
   ACE_OK(ace_ext_plain_mac_groups(G.ctx, in_r0, in_r1, (size_t)r.baby, in0, in1, (size_t)r.giant, inp, level, plain_level));
-  for (int32_t i = 0; i < r.baby; ++i) {
+  /* The result is sum_i rotation_i(inner sum i).  Group 0 is not rotated: its two halves start the running sums
+   * `first` (c0 parts that need no key switch) and `sum1`.  A rotated group's c1 part is brought down, raised again
+   * and rotated with its key; its c0 part rides along as the addend; both land in (outer.c0, sum1). */
+  int64_t *first = inners[0].c0, *sum1 = inners[0].c1;
+  bool     outer0_set = false;
+  for (int32_t i = 1; i < r.baby; ++i) {
     EXT_CT* in = &inners[i];
-    if (i == 0) { /* the c0 parts are summed aside and meet the c1 parts at the end */
-      Rt_dev_copy(first, in->c0, T * n);
-      ACE_OK(ace_zero(G.ctx, outer.c0, T * n));
-      Rt_dev_copy(outer.c1, in->c1, T * n);
-    } else if (r.out[i] != 0) {
-      ROT_KEY* key = Rt_find_rot(r.out[i]);
-      FMT_ASSERT(key, "cannot find auto key of rotation %d", r.out[i]);
-      ACE_OK(ace_poly_automorphism(G.ctx, moved, in->c0, key->order, level, 1));
-      ACE_OK(ace_poly_add(G.ctx, first, first, moved, level, 1));
+    if (r.out[i] != 0) {
       ACE_OK(ace_mod_down(G.ctx, low, in->c1, level, 1));
       ACE_OK(ace_precomp(G.ctx, low_digits, low, level, 1));
-      ext_rotate(&turned, low_digits, nd, NULL, r.out[i], level);
-      ACE_OK(ace_poly_add(G.ctx, outer.c0, outer.c0, turned.c0, level, 1));
-      ACE_OK(ace_poly_add(G.ctx, outer.c1, outer.c1, turned.c1, level, 1));
+      EXT_CT into = {outer.c0, sum1};
+      ext_rotate(&into, low_digits, nd, in->c0, r.out[i], level, (outer0_set ? 1 : 0) | 2);
+      outer0_set = true;
     } else {
       ACE_OK(ace_poly_add(G.ctx, first, first, in->c0, level, 1));
-      ACE_OK(ace_poly_add(G.ctx, outer.c1, outer.c1, in->c1, level, 1));
+      ACE_OK(ace_poly_add(G.ctx, sum1, sum1, in->c1, level, 1));
     }
   }
+  if (outer0_set) ACE_OK(ace_poly_add(G.ctx, first, first, outer.c0, level, 1));
   for (int32_t i = 1; i < r.baby; ++i) ext_free(&inners[i]);
   free(inners);
   free(in_r0);
   free(in_r1);
   free((void*)inp);
-  ACE_OK(ace_poly_add(G.ctx, outer.c0, outer.c0, first, level, 1));
-  ACE_OK(ace_mod_down(G.ctx, ct->_c0_poly._data, outer.c0, level, 1));
-  ACE_OK(ace_mod_down(G.ctx, ct->_c1_poly._data, outer.c1, level, 1));
+  ACE_OK(ace_mod_down(G.ctx, ct->_c0_poly._data, first, level, 1));
+  ACE_OK(ace_mod_down(G.ctx, ct->_c1_poly._data, sum1, level, 1));
   ct->_scaling_factor *= G.sc;
   ct->_sf_degree += 1;
 
   for (int32_t j = 0; j < r.giant; ++j) ext_free(&rots[j]);
   free(rots);
-  ext_free(&turned);
   ext_free(&inner);
   ext_free(&outer);
   Rt_dev_free(digits);
   Rt_dev_free(c0_ext);
-  Rt_dev_free(first);
-  Rt_dev_free(moved);
   Rt_dev_free(low);
   Rt_dev_free(low_digits);
 }

@@ -225,11 +225,12 @@ int ace_dot_prod(ace_ctx* ctx, int64_t* res, const int64_t* digits, const int64_
 /* Fast_rotate_ext without its Mod_down (evaluator.c:503-566, as Rotate_iteration of bootstrap.c:1233-1373 uses it):
  * out0 = sigma(sum_d digit_d * key_d.b + addend0), out1 = sigma(sum_d digit_d * key_d.a), level + num_p limbs each,
  * NTT form; sigma is the automorphism given by `order` (ace_automorphism_order, NTT form).  key points at digit 0's b
- * half, its a half lies key_half_words further, digit d's pair key_stride words further; addend0 may be NULL.  The
- * results must not overlap the operands. */
+ * half, its a half lies key_half_words further, digit d's pair key_stride words further; addend0 may be NULL.
+ * accumulate: bit 0 adds the first result to what out0 holds, bit 1 the second to out1 (the running sums of the
+ * giant steps).  The results must not overlap the operands. */
 int ace_ext_rotate(ace_ctx* ctx, int64_t* out0, int64_t* out1, const int64_t* digits, const int64_t* key,
                    size_t key_half_words, size_t key_stride, size_t n_parts, const int64_t* addend0,
-                   const int64_t* order, size_t level);
+                   const int64_t* order, size_t level, int accumulate);
 
 /* ---- ciphertext level (ckks/src/evaluator.c, ckks/src/cipher.c) ------------
  * A ciphertext at level l is two polynomials (c0, c1) of l limbs.  A switch

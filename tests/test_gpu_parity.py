@@ -265,8 +265,24 @@ def test_ext_rotate_equals_its_parts(pair):
                 g.ext_rotate(r0, r1, digits, swk, half, 2 * half, nd, addend if with_addend else None, order, level)
                 eq(r0, w0.get(), "first half, level %d rot %d addend %d" % (level, rot, with_addend))
                 eq(r1, w1.get(), "second half, level %d rot %d" % (level, rot))
+                # running sums: the second call adds to the first half only, the third to both
+                g.ext_rotate(r0, r1, digits, swk, half, 2 * half, nd, addend if with_addend else None, order, level, 1)
+                g.poly("add", w0, w0, w0, level, True)
+                eq(r0, w0.get(), "first half accumulated")
+                eq(r1, w1.get(), "second half overwritten")
+                g.ext_rotate(r0, r1, digits, swk, half, 2 * half, nd, None, order, level, 3)
+                g.poly("automorphism", w0, t0, order, level, True)  # t0 still holds dot (+ addend)
                 if with_addend:  # undo for the pass without
                     g.dot_prod(t0, digits, swk, 2 * half, nd, level)
+                plain0 = g.alloc(T * N)
+                g.poly("automorphism", plain0, t0, order, level, True)
+                # r0 = 2 * sigma(dot + addend) + sigma(dot), r1 = 2 * sigma(dot1)
+                want0, want1 = g.alloc(T * N), g.alloc(T * N)
+                g.poly("add", want0, w0, w0, level, True)
+                g.poly("add", want0, want0, plain0, level, True)
+                g.poly("add", want1, w1, w1, level, True)
+                eq(r0, want0.get(), "first half accumulated twice")
+                eq(r1, want1.get(), "second half accumulated")
             with pytest.raises(acefhe.AceError):
                 g.ext_rotate(digits.view(0, T * N), r1, digits, swk, half, 2 * half, nd, None, order, level)
 
