@@ -1112,7 +1112,10 @@ int ace_copy(ace_ctx* c, int64_t* dst, const int64_t* src, size_t n) {
   if (!dst || !src) return fail("ace_copy: null argument");
   if (dst == src || n == 0) return 0;
   if (c->batching && n <= kRecordedWords) {  // a copy is an elementwise entry like any other
-    c->run_append(BatchOp{U(dst), U(src), nullptr, 0, (u32)BATCH_COPY, 0}, n);
+    // whole limbs go in limb by limb, so that they join the limb-sized calls around them in one run
+    const size_t N = c->h.N, pieces = (n % N == 0 && n / N <= 16) ? n / N : 1, each = n / pieces;
+    for (size_t t = 0; t < pieces; ++t)
+      c->run_append(BatchOp{U(dst) + t * each, U(src) + t * each, nullptr, 0, (u32)BATCH_COPY, 0}, each);
     return 0;
   }
   c->flush_run();
@@ -1124,7 +1127,9 @@ int ace_zero(ace_ctx* c, int64_t* dst, size_t n) {
   if (!dst) return fail("ace_zero: null argument");
   if (n == 0) return 0;
   if (c->batching && n <= kRecordedWords) {
-    c->run_append(BatchOp{U(dst), nullptr, nullptr, 0, (u32)BATCH_ZERO, 0}, n);
+    const size_t N = c->h.N, pieces = (n % N == 0 && n / N <= 16) ? n / N : 1, each = n / pieces;
+    for (size_t t = 0; t < pieces; ++t)
+      c->run_append(BatchOp{U(dst) + t * each, nullptr, nullptr, 0, (u32)BATCH_ZERO, 0}, each);
     return 0;
   }
   c->flush_run();
