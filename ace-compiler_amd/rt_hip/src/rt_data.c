@@ -48,7 +48,7 @@ static struct {
 /* Encoded weight plaintexts kept in HBM.  A program encodes the same entries for every input it is run on (the
  * reference avoids that only with files of pre-encoded plaintexts); with a few hundred GB of HBM the encoded
  * polynomial of each (entry, range, scale degree, level) is kept after its first use and copied from then on.
- * RT_HIP_PLAINTEXT_CACHE_GB bounds the space (default 48; 0 switches it off). */
+ * RT_HIP_PLAINTEXT_CACHE_GB bounds the space (default 96; 0 switches it off). */
 typedef struct {
   uint64_t k1, k2; /* (index, scale, level), (offset, length); k1 == 0 marks a free cell (level is never 0) */
   int64_t* dev;
@@ -100,7 +100,7 @@ static void cache_clear(void) {
 bool Pt_mgr_init(const char* fname) {
   const char* gb    = getenv("RT_HIP_PLAINTEXT_CACHE_GB");
   cache_clear();
-  Cache.limit_words = (size_t)((gb ? atof(gb) : 48.0) * (double)(1ull << 27));
+  Cache.limit_words = (size_t)((gb ? atof(gb) : 96.0) * (double)(1ull << 27));
   const char* over = getenv("RT_HIP_DATA_FILE");
   const char* syn  = getenv("RT_HIP_SYNTHETIC_WEIGHTS");
   if (over && *over) fname = over;
