@@ -152,6 +152,10 @@ void HostContext::build(uint32_t degree, const std::vector<i64>& q, size_t num_p
   parts = num_parts;
   part_size = (L + parts - 1) / parts;
   if (L <= part_size * (parts - 1)) throw std::runtime_error("invalid number of q parts");
+  // the device arithmetic keeps lazily reduced words below 8q in 64 bits (the reference's parameter sets stop at
+  // 60-bit primes)
+  for (i64 v : q)
+    if (v < 3 || v >= ((i64)1 << 61)) throw std::runtime_error("primes must be below 2^61");
   size_t max_bits = 0;
   for (size_t j = 0; j < parts; ++j) {
     size_t lo = j * part_size, hi = std::min(L, lo + part_size);

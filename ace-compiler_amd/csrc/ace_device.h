@@ -1,6 +1,6 @@
 // Device-side data structures and 64-bit modular arithmetic for gfx950.
 //
-// All residues are 64-bit words in [0, q), q < 2^62.  There is no 64x64->128
+// All residues are 64-bit words in [0, q), q < 2^61.  There is no 64x64->128
 // VALU multiply on CDNA4; __umul64hi and `*` lower to v_mad_u64_u32 chains.
 // Three reductions are used, each value-identical to the reference's because
 // the canonical residue of an integer is unique:
@@ -85,6 +85,14 @@ __device__ __forceinline__ u64 csub(u64 a, u64 q) { return a >= q ? a - q : a; }
 // a*w mod q up to one extra q: result in [0, 2q) for any a < 2^64
 __device__ __forceinline__ u64 shoup_lazy(u64 a, u64 w, u64 wp, u64 q) {
   return a * w - __umul64hi(a, wp) * q;
+}
+// The same with the quotient a*wp / 2^64 estimated from three of the four partial products (the low x low one and
+// the carries of the middle sum are dropped): at most 2 too small, so the result is in [0, 4q).  Five instructions
+// for the quotient instead of about ten; for the NTT butterflies, whose lazy ranges absorb the slack (q < 2^61).
+__device__ __forceinline__ u64 shoup_lazier(u64 a, u64 w, u64 wp, u64 q) {
+  const u32 ah = (u32)(a >> 32), al = (u32)a, ph = (u32)(wp >> 32), pl = (u32)wp;
+  const u64 quot = (u64)ah * ph + __umulhi(ah, pl) + __umulhi(al, ph);
+  return a * w - quot * q;
 }
 __device__ __forceinline__ u64 shoup_mul(u64 a, u64 w, u64 wp, u64 q) {
   return csub(shoup_lazy(a, w, wp, q), q);

@@ -20,10 +20,11 @@
 // N <= 4096 uses one workgroup per limb with the limb in LDS.
 //
 // Two arithmetic back ends share the index logic:
-//   ArithInt  64-bit integers, Harvey lazy butterflies (forward < 4q, inverse
-//             < 2q) with Shoup twiddles; any prime below 2^62.  About 30 VALU
-//             instructions per butterfly, which makes the chunk pass
-//             instruction-bound.
+//   ArithInt  64-bit integers, Harvey lazy butterflies (forward < 8q, inverse
+//             < 4q) with Shoup twiddles whose quotient is estimated from three
+//             partial products (up to 2 too small); any prime below 2^61.
+//             About 27 VALU instructions per butterfly, which makes the chunk
+//             pass instruction-bound.
 //   ArithFp   for primes below 2^50.2: residues are carried as exact integers
 //             in FP64 (|x| < 2^53).  A twiddle product is y*w - rint(y*(w/q))*q
 //             evaluated exactly with one FMA for the low half of y*w and one
@@ -54,13 +55,14 @@ __device__ __forceinline__ int lds_pos(int e) { return e + (e >> 4); }
 // ---------------------------------------------------------------------------
 struct ArithInt {
   typedef u64 T;
-  u64 q, q2;
+  u64 q, q2, q4;
   const u64 *w, *wp;  // twiddle, Shoup companion
   u64 sc, scp;        // inverse: final scale constant
   __device__ __forceinline__ void init(const DevCtx& c, u32 pi, bool inverse, const u64* scale, u32 sidx) {
     const DevPrime& P = c.primes[pi];
     q = P.q;
     q2 = q << 1;
+    q4 = q << 2;
     w = (inverse ? c.irou : c.rou) + (u64)pi * c.N;
     wp = (inverse ? c.irou_p : c.rou_p) + (u64)pi * c.N;
     sc = P.ninv;
@@ -91,21 +93,21 @@ struct ArithInt {
   __device__ __forceinline__ T in_mid(u64 v) const { return v; }
   __device__ __forceinline__ u64 out_mid(T v) const { return v; }
   __device__ __forceinline__ void reduce(T&) const {}
-  // forward, Harvey: x,y < 4q -> < 4q
+  // forward, Harvey butterflies with the cheaper quotient estimate (product in [0, 4q)): x,y < 8q -> < 8q
   __device__ __forceinline__ void ct(T& x, T& y, const TW& tw) const {
-    u64 a = csub(x, q2);
-    u64 t = shoup_lazy(y, tw.w, tw.wp, q);
+    u64 a = csub(x, q4);
+    u64 t = shoup_lazier(y, tw.w, tw.wp, q);
     x = a + t;
-    y = a - t + q2;
+    y = a - t + q4;
   }
-  // inverse: x,y < 2q -> < 2q
+  // inverse: x,y < 4q -> < 4q
   __device__ __forceinline__ void gs(T& x, T& y, const TW& tw) const {
-    u64 s = csub(x + y, q2);
-    u64 d = x - y + q2;
+    u64 s = csub(x + y, q4);
+    u64 d = x - y + q4;
     x = s;
-    y = shoup_lazy(d, tw.w, tw.wp, q);
+    y = shoup_lazier(d, tw.w, tw.wp, q);
   }
-  __device__ __forceinline__ u64 out_canon(T v) const { return csub(csub(v, q2), q); }
+  __device__ __forceinline__ u64 out_canon(T v) const { return csub(csub(csub(v, q4), q2), q); }
   __device__ __forceinline__ u64 out_scaled(T v) const { return shoup_mul(v, sc, scp, q); }
 };
 
