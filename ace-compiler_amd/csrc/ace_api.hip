@@ -116,8 +116,7 @@ struct ace_ctx {
   }
   PendingRun run;
   bool batching = true;      // record Hw_* calls and launch them together
-  BatchOp* run_dev = nullptr;
-  u32* run_chain_dev = nullptr;
+  BatchOpDev* run_dev = nullptr;
   static constexpr size_t kMaxRun = 2048;
   void flush_run();
   // A Mod_down or Rescale of one polynomial waits for the next call: generated code issues them in pairs (c0, then
@@ -508,18 +507,7 @@ void ace_ctx::run_append(const BatchOp& o, u64 n) {
 
 void ace_ctx::flush_run() {
   if (run.ops.empty()) return;
-  const size_t count = run.ops.size();
-  // chains: entries joined whenever one writes a range the other reads or writes (union-find over entries)
-  std::vector<u32> parent(count);
-  for (u32 k = 0; k < count; ++k) parent[k] = k;
-  auto find = [&](u32 x) {
-    while (parent[x] != x) x = parent[x] = parent[parent[x]];
-    return x;
-  };
-  auto join = [&](u32 x, u32 y) {
-    x = find(x), y = find(y);
-    if (x != y) parent[std::max(x, y)] = std::min(x, y);
-  };
+  size_t count = run.ops.size();
   // Scratch results: entry k's range is read by entry k+1 (which the kernel serves from a register), by nothing
   // else before a later entry overwrites it.  Such a store is dropped, and the range then ties k to k+1 only:
   // the limb-by-limb products of an inner product (Hw_modmul into one scratch limb, Hw_modadd from it) become
@@ -557,6 +545,44 @@ void ace_ctx::flush_run() {
       scratch_read[k + 1] = 1;
     }
   }
+  // A product into such a scratch limb followed by the sum that adds it to its own destination is one
+  // multiply-add entry (the same canonical value): half the entries, so more runs travel as kernel arguments.
+  {
+    std::vector<BatchOp> merged;
+    std::vector<uint8_t> merged_read;
+    merged.reserve(count);
+    for (u32 k = 0; k < count; ++k) {
+      const BatchOp& o = run.ops[k];
+      const u32 op = o.op & ~kBatchDeadStore;
+      if ((o.op & kBatchDeadStore) && (op == EW_MUL || op == EW_MUL_S) && !scratch_read[k] && k + 1 < count) {
+        const BatchOp& n = run.ops[k + 1];
+        const bool sum_to_self = n.op == EW_ADD && n.prime == o.prime && n.r != o.r &&
+                                 ((n.a == n.r && n.b == o.r) || (n.b == n.r && n.a == o.r));
+        if (sum_to_self) {
+          merged.push_back(BatchOp{n.r, o.a, o.b, o.scalar, (u32)(op == EW_MUL ? EW_MULADD : EW_MULADD_S), o.prime});
+          merged_read.push_back(0);
+          ++k;
+          continue;
+        }
+      }
+      merged.push_back(o);
+      merged_read.push_back(scratch_read[k]);
+    }
+    run.ops.swap(merged);
+    scratch_read.swap(merged_read);
+    count = run.ops.size();
+  }
+  // chains: entries joined whenever one writes a range the other reads or writes (union-find over entries)
+  std::vector<u32> parent(count);
+  for (u32 k = 0; k < count; ++k) parent[k] = k;
+  auto find = [&](u32 x) {
+    while (parent[x] != x) x = parent[x] = parent[parent[x]];
+    return x;
+  };
+  auto join = [&](u32 x, u32 y) {
+    x = find(x), y = find(y);
+    if (x != y) parent[std::max(x, y)] = std::min(x, y);
+  };
   std::unordered_map<uintptr_t, u32> writer;                // last entry that wrote the range
   std::unordered_map<uintptr_t, std::vector<u32>> readers;  // entries that read it since
   for (u32 k = 0; k < count; ++k) {
@@ -601,22 +627,30 @@ void ace_ctx::flush_run() {
   run.written.clear();
   run.rot_res.clear();
   run.rot_src.clear();
+  auto compact = [](const BatchOp& o) {
+    const u32 op = o.op & ~kBatchDeadStore;
+    const bool scalar = op >= EW_ADD_S && op <= EW_MULADD_S;
+    return BatchOpDev{o.r, o.a, scalar ? o.scalar : (u64)(uintptr_t)o.b, o.op, o.prime};
+  };
   if (count <= kSmallRun) {
     SmallRun small{};
-    for (u32 k = 0; k < count; ++k) small.ops[k] = sorted[k];
+    for (u32 k = 0; k < count; ++k) small.ops[k] = compact(sorted[k]);
     for (size_t k = 0; k < chain_start.size(); ++k) small.chain_start[k] = (uint16_t)chain_start[k];
     launch_ew_batch_small(stream, d, small, n_chains, n);
     return;
   }
+  // entries and chain starts travel in one copy: [entries | chain starts]
   if (!run_dev) {
-    HIP_OK(hipMalloc((void**)&run_dev, kMaxRun * sizeof(BatchOp)));
+    HIP_OK(hipMalloc((void**)&run_dev, kMaxRun * sizeof(BatchOpDev) + (kMaxRun + 1) * sizeof(u32)));
     owned.push_back(run_dev);
-    HIP_OK(hipMalloc((void**)&run_chain_dev, (kMaxRun + 1) * sizeof(u32)));
-    owned.push_back(run_chain_dev);
   }
-  h2d(run_dev, sorted.data(), count * sizeof(BatchOp));
-  h2d(run_chain_dev, chain_start.data(), chain_start.size() * sizeof(u32));
-  launch_ew_batch(stream, d, run_dev, run_chain_dev, n_chains, n);
+  const size_t ops_bytes = count * sizeof(BatchOpDev), chain_bytes = chain_start.size() * sizeof(u32);
+  std::vector<unsigned char> image(ops_bytes + chain_bytes);
+  for (u32 k = 0; k < count; ++k) reinterpret_cast<BatchOpDev*>(image.data())[k] = compact(sorted[k]);
+  std::memcpy(image.data() + ops_bytes, chain_start.data(), chain_bytes);
+  h2d(run_dev, image.data(), image.size());
+  launch_ew_batch(stream, d, run_dev, reinterpret_cast<const u32*>(reinterpret_cast<const unsigned char*>(run_dev) + ops_bytes),
+                  n_chains, n);
 }
 
 namespace {

@@ -92,14 +92,21 @@ struct BatchOp {
   u32 op;        // an EwOp, or BATCH_ROTATE
   u32 prime;
 };
-constexpr u32 kSmallRun = 64;  // runs up to this many entries travel as kernel arguments, no copy
+// an entry as the kernels read it: b is the second operand, the index table of a rotate, or the scalar
+struct BatchOpDev {
+  u64* r;
+  const u64* a;
+  u64 b;
+  u32 op, prime;
+};
+constexpr u32 kSmallRun = 96;  // runs up to this many entries travel as kernel arguments (3.3 KB), no copy
 struct SmallRun {
-  BatchOp ops[kSmallRun];
+  BatchOpDev ops[kSmallRun];
   uint16_t chain_start[kSmallRun + 1];
 };
 void launch_ew_batch_small(hipStream_t st, const DevCtx& c, const SmallRun& run, u32 n_chains, u64 n);
 // chain y (blockIdx.y) is the entries [chain_start[y], chain_start[y+1]): chains share no written range, so they run side by side
-void launch_ew_batch(hipStream_t st, const DevCtx& c, const BatchOp* dev_ops, const u32* dev_chain_start, u32 n_chains, u64 n);
+void launch_ew_batch(hipStream_t st, const DevCtx& c, const BatchOpDev* dev_ops, const u32* dev_chain_start, u32 n_chains, u64 n);
 void launch_sample_uniform(hipStream_t st, const DevCtx& c, u64* r, u64 seed, u64 stream, const LimbMap& lm,
                            u32 n_limbs, u64 n);
 void launch_expand_small(hipStream_t st, const DevCtx& c, u64* r, const i64* v, const LimbMap& lm, u32 n_limbs, u64 n);

@@ -131,8 +131,8 @@ void launch_plain_mac_groups(hipStream_t st, const DevCtx& c, const MacGroups& o
 // The host splits a run into chains that share no written range; a chain's entries are carried out in order by
 // the thread of element i, so an entry may read what an earlier one of its chain wrote (identical ranges only;
 // a rotate never reads or overwrites anything the run touches).
-__device__ __forceinline__ void run_chain(const DevCtx& c, const BatchOp* ops, u32 first, u32 last, u64 i);
-__global__ __launch_bounds__(kThreads) void ew_batch_kernel(DevCtx c, const BatchOp* ops, const u32* chain_start, u64 n) {
+__device__ __forceinline__ void run_chain(const DevCtx& c, const BatchOpDev* ops, u32 first, u32 last, u64 i);
+__global__ __launch_bounds__(kThreads) void ew_batch_kernel(DevCtx c, const BatchOpDev* ops, const u32* chain_start, u64 n) {
   const u64 i = (u64)blockIdx.x * kThreads + threadIdx.x;
   if (i >= n) return;
   run_chain(c, ops, chain_start[blockIdx.y], chain_start[blockIdx.y + 1], i);
@@ -142,17 +142,18 @@ __global__ __launch_bounds__(kThreads) void ew_batch_small_kernel(DevCtx c, Smal
   if (i >= n) return;
   run_chain(c, run.ops, run.chain_start[blockIdx.y], run.chain_start[blockIdx.y + 1], i);
 }
-__device__ __forceinline__ void run_chain(const DevCtx& c, const BatchOp* ops, u32 first, u32 last, u64 i) {
+__device__ __forceinline__ void run_chain(const DevCtx& c, const BatchOpDev* ops, u32 first, u32 last, u64 i) {
   // what the previous entry produced stays in a register: an operand that names that range is not loaded again
   const u64* prev_r = nullptr;
   u64 prev_v = 0;
   for (u32 k = first; k < last; ++k) {
-    const BatchOp o = ops[k];
+    const BatchOpDev o = ops[k];
+    const u64* ob = reinterpret_cast<const u64*>(o.b);
     const u32 op = o.op & ~kBatchDeadStore;
     const DevPrime P = c.primes[o.prime];
     u64 v;
     if (op == BATCH_ROTATE) {
-      const i64 src = reinterpret_cast<const i64*>(o.b)[i];
+      const i64 src = reinterpret_cast<const i64*>(ob)[i];
       v = src >= 0 ? o.a[src] : P.q - o.a[-src];
     } else if (op == BATCH_COPY) {
       v = o.a == prev_r ? prev_v : o.a[i];
@@ -160,7 +161,7 @@ __device__ __forceinline__ void run_chain(const DevCtx& c, const BatchOp* ops, u
       v = 0;
     } else {
       const u64 x = o.a == prev_r ? prev_v : o.a[i];
-      const u64 y = op >= EW_ADD_S ? o.scalar : (o.b == prev_r ? prev_v : o.b[i]);
+      const u64 y = op >= EW_ADD_S ? o.b : (ob == prev_r ? prev_v : ob[i]);
       if (op == EW_ADD || op == EW_ADD_S) v = add_mod(x, y, P.q);
       else if (op == EW_SUB || op == EW_SUB_S) v = sub_mod(x, y, P.q);
       else if (op == EW_MUL || op == EW_MUL_S) v = mulmod(x, y, P);
@@ -177,7 +178,7 @@ void launch_ew_batch_small(hipStream_t st, const DevCtx& c, const SmallRun& run,
   dim3 g((unsigned)((n + kThreads - 1) / kThreads), n_chains, 1);
   hipLaunchKernelGGL(ew_batch_small_kernel, g, dim3(kThreads), 0, st, c, run, n);
 }
-void launch_ew_batch(hipStream_t st, const DevCtx& c, const BatchOp* dev_ops, const u32* dev_chain_start, u32 n_chains, u64 n) {
+void launch_ew_batch(hipStream_t st, const DevCtx& c, const BatchOpDev* dev_ops, const u32* dev_chain_start, u32 n_chains, u64 n) {
   if (!n || !n_chains) return;
   dim3 g((unsigned)((n + kThreads - 1) / kThreads), n_chains, 1);
   hipLaunchKernelGGL(ew_batch_kernel, g, dim3(kThreads), 0, st, c, dev_ops, dev_chain_start, n);
