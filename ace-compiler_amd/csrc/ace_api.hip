@@ -806,11 +806,11 @@ void do_rescale(ace_ctx* c, const PolySeq& res, const PolySeq& src, size_t np, s
   size_t mark = c->ws_used;
   u64* last = c->take(np * N);
   u64* u = c->take(np * (level - 1) * N);
-  launch_pick_limb(c->stream, c->d, last, src, (u32)(level - 1), (u32)np);
   LimbMap one{};
   one.prime[0] = (uint8_t)(level - 1);
   PolySeq ls = seq_strided(last, N), us = seq_strided(u, (level - 1) * N);
-  launch_ntt(c->stream, c->d, ls, ls, one, nullptr, 1, (u32)np, true, nullptr);
+  // the inverse transform reads the last limb where it lies
+  launch_ntt(c->stream, c->d, ls, shifted(src, (level - 1) * N), one, nullptr, 1, (u32)np, true, nullptr);
   if (c->d.logN > 12) {  // modulus switch and tail ride on the transform's first and last kernels
     FwdFuse f{};
     f.pro = 1;

@@ -169,8 +169,6 @@ void launch_moddown_rescale(hipStream_t st, const DevCtx& c, u64* out, const u64
                             const u64* pinv, const u64* qlinv, u32 level);
 // out[0] = src, out[i] = Switch_modulus(src, q_0 -> q_i) for i < level
 void launch_from_level0(hipStream_t st, const DevCtx& c, u64* out, const u64* src, u32 level);
-// dst[p][i] = limb `limb` of polynomial p of src
-void launch_pick_limb(hipStream_t st, const DevCtx& c, u64* dst, const PolySeq& src, u32 limb, u32 n_polys);
 // out[t] = src[t] * cst[2t] (Shoup constant per limb)
 void launch_mul_const(hipStream_t st, const DevCtx& c, u64* out, const u64* src, const u64* cst, const LimbMap& lm,
                       u32 n_limbs);

@@ -885,19 +885,6 @@ void launch_from_level0(hipStream_t st, const DevCtx& c, u64* out, const u64* sr
   hipLaunchKernelGGL(from_level0_kernel, ew_grid(c.N, level), dim3(kThreads), 0, st, c, out, src);
 }
 
-// gathers limb `limb` of every polynomial of a sequence into a dense buffer
-__global__ __launch_bounds__(kThreads) void pick_limb_kernel(u64* __restrict__ dst, PolySeq srcs, u64 n, u32 limb) {
-  const u32 p = blockIdx.z;
-  const u64* __restrict__ s = srcs.at(p) + (u64)limb * n;
-  u64* __restrict__ d = dst + (u64)p * n;
-#pragma unroll
-  ACE_EW_LOOP(i, n) d[i] = s[i];
-}
-void launch_pick_limb(hipStream_t st, const DevCtx& c, u64* dst, const PolySeq& src, u32 limb, u32 n_polys) {
-  if (!n_polys) return;
-  hipLaunchKernelGGL(pick_limb_kernel, ew_grid(c.N, 1, n_polys), dim3(kThreads), 0, st, dst, src, (u64)c.N, limb);
-}
-
 // ---- multiply every limb by its own constant (Extend, rns_poly.c:483-500) ---
 __global__ __launch_bounds__(kThreads) void mul_const_kernel(DevCtx c, u64* __restrict__ out,
                                                              const u64* __restrict__ src,
