@@ -686,15 +686,20 @@ PolySeq shifted(const PolySeq& s, u64 words) {
 void do_decomp_modup(ace_ctx* c, u64* res, const u64* digit, size_t level, size_t part, bool is_ntt) {
   const ModUpDev& m = c->modup_at(level, part);
   const size_t N = c->h.N, nd = m.t.digit.size(), nc = m.t.compl_idx.size(), start = c->h.part_size * part;
-  if (res + start * N != digit)
+  // the digit's own limbs pass through; the inverse transform of a large ring drops that copy as it reads them
+  const bool pass_through = res + start * N != digit, by_transform = pass_through && is_ntt && c->d.logN > 12;
+  if (pass_through && !by_transform)
     HIP_OK(hipMemcpyAsync(res + start * N, digit, nd * N * sizeof(u64), hipMemcpyDeviceToDevice, c->stream));
   size_t mark = c->ws_used;
   u64* t = c->take(nd * N);
-  if (is_ntt)
-    launch_ntt(c->stream, c->d, seq_strided(t, 0), seq_strided(digit, 0), m.digit_lm, nullptr, (u32)nd, 1, true,
-               m.scale_ntt);
-  else
+  if (is_ntt) {
+    const PolySeq through = seq_strided(res + start * N, 0);
+    if (!launch_ntt(c->stream, c->d, seq_strided(t, 0), seq_strided(digit, 0), m.digit_lm, nullptr, (u32)nd, 1, true,
+                    m.scale_ntt, 3, nullptr, by_transform ? &through : nullptr))
+      throw std::runtime_error("internal: Mod_up transform rejected");
+  } else {
     launch_mul_const(c->stream, c->d, t, digit, m.scale_coef, m.digit_lm, (u32)nd);
+  }
   ConvBatch b{};
   b.n_jobs = 1;
   b.job[0] = m.job;

@@ -498,8 +498,8 @@ __global__ __launch_bounds__(kChunkThreads, EPI == 1 ? 6 : 8) void ntt_fwd_chunk
 // are those of the forward pass in reverse order.
 template <class A>
 __device__ __forceinline__ void inv_chunk_body(u64* lds_words, const DevCtx& c, const PolySeq& dsts,
-                                               const PolySeq& srcs, const LimbMap& pos, u32 n_polys, u32 chunk,
-                                               u32 limb, u32 pblk, u32 pi) {
+                                               const PolySeq& srcs, const PolySeq& copies, const LimbMap& pos,
+                                               u32 n_polys, u32 chunk, u32 limb, u32 pblk, u32 pi) {
   typedef typename A::T T;
   T* lds = reinterpret_cast<T*>(lds_words);
   const int t = threadIdx.x;
@@ -522,6 +522,11 @@ __device__ __forceinline__ void inv_chunk_body(u64* lds_words, const DevCtx& c, 
       const u64* src = srcs.at(poly0 + it + 1);
 #pragma unroll
       for (int r = 0; r < 8; ++r) nxt[r] = src[off + t + 512 * r];
+    }
+    if (copies.b[0]) {  // the untransformed words are wanted elsewhere too (the digit that Mod_up passes through)
+      u64* cp = copies.at(poly0 + it);
+#pragma unroll
+      for (int r = 0; r < 8; ++r) cp[off + t + 512 * r] = raw[r];
     }
     T v[8];
 #pragma unroll
@@ -571,14 +576,14 @@ __device__ __forceinline__ void inv_chunk_body(u64* lds_words, const DevCtx& c, 
     for (int r = 0; r < 8; ++r) raw[r] = nxt[r];
   }
 }
-__global__ __launch_bounds__(kChunkThreads, 8) void ntt_inv_chunk(DevCtx c, PolySeq dsts, PolySeq srcs, LimbMap lm,
-                                                                  LimbMap pos, u32 n_limbs, u32 n_polys) {
+__global__ __launch_bounds__(kChunkThreads, 8) void ntt_inv_chunk(DevCtx c, PolySeq dsts, PolySeq srcs, PolySeq copies,
+                                                                  LimbMap lm, LimbMap pos, u32 n_limbs, u32 n_polys) {
   __shared__ u64 lds[kChunk + kChunk / 16];
   u32 chunk, limb, pblk;
   if (!chunk_block(c, n_limbs, (n_polys + kPolysPerBlock - 1) / kPolysPerBlock, chunk, limb, pblk)) return;
   const u32 pi = lm.prime[limb];
-  if (c.fp_ok[pi]) inv_chunk_body<ArithFp>(lds, c, dsts, srcs, pos, n_polys, chunk, limb, pblk, pi);
-  else inv_chunk_body<ArithInt>(lds, c, dsts, srcs, pos, n_polys, chunk, limb, pblk, pi);
+  if (c.fp_ok[pi]) inv_chunk_body<ArithFp>(lds, c, dsts, srcs, copies, pos, n_polys, chunk, limb, pblk, pi);
+  else inv_chunk_body<ArithInt>(lds, c, dsts, srcs, copies, pos, n_polys, chunk, limb, pblk, pi);
 }
 
 // inverse, strided pass: spans 4096..N/2, then scale every word by the limb's
@@ -656,7 +661,7 @@ __global__ __launch_bounds__(256) void ntt_small(DevCtx c, PolySeq dsts, PolySeq
 template <int LOGR>
 static void run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolySeq& src, const LimbMap& lm,
                       const LimbMap& pos, u32 n_limbs, u32 n_polys, bool inverse, const u64* scale, int passes,
-                      const FwdFuse& f) {
+                      const FwdFuse& f, const PolySeq& copies) {
   dim3 gs((c.N >> LOGR) / 256, n_limbs, n_polys),
       gc(chunk_grid(c, n_limbs, (n_polys + kPolysPerBlock - 1) / kPolysPerBlock));
   if (!inverse) {
@@ -680,7 +685,7 @@ static void run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst, const
     }
   } else {
     if (passes & 1)
-      hipLaunchKernelGGL(ntt_inv_chunk, gc, dim3(kChunkThreads), 0, st, c, dst, src, lm, pos, n_limbs, n_polys);
+      hipLaunchKernelGGL(ntt_inv_chunk, gc, dim3(kChunkThreads), 0, st, c, dst, src, copies, lm, pos, n_limbs, n_polys);
     if (passes & 2) {
       u32 n_fp = 0;
       for (u32 t = 0; t < n_limbs; ++t) n_fp += c.fp_ok[lm.prime[t]] ? 1 : 0;
@@ -696,8 +701,13 @@ static void run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst, const
 
 bool launch_ntt(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolySeq& src, const LimbMap& lm,
                 const LimbMap* pos_in, u32 n_limbs, u32 n_polys, bool inverse, const u64* scale, int passes,
-                const FwdFuse* fuse) {
+                const FwdFuse* fuse, const PolySeq* copy_src_to) {
   if (n_limbs == 0 || n_polys == 0) return true;
+  PolySeq copies{};
+  if (copy_src_to) {  // only the inverse chunk pass can drop a copy of what it reads
+    if (!inverse || c.logN <= kLogChunk || !(passes & 1)) return false;
+    copies = *copy_src_to;
+  }
   FwdFuse f{};
   if (fuse) {
     if (inverse || c.logN <= kLogChunk || passes != 3) return false;  // only whole forward transforms of N > 4096
@@ -715,7 +725,7 @@ bool launch_ntt(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolyS
   switch (c.logN - kLogChunk) {
 #define ACE_NTT_CASE(LR)                                                                      \
   case LR:                                                                                    \
-    run_large<LR>(st, c, dst, src, lm, pos, n_limbs, n_polys, inverse, scale, passes, f);     \
+    run_large<LR>(st, c, dst, src, lm, pos, n_limbs, n_polys, inverse, scale, passes, f, copies); \
     return true;
     ACE_NTT_CASE(1)
     ACE_NTT_CASE(2)
