@@ -190,9 +190,9 @@ struct ace_ctx {
   ShoupConst sc(u64 w, size_t prime) const { return {w, shoup(w, h.primes[prime].q)}; }
 
   // FP64 tables of a base conversion (ConvJob::fw / fq): targets below the FP64 limit convert in
-  // exact double arithmetic; sources above it are split into two 30-bit-and-rest halves
+  // exact double arithmetic; sources at or above kFpConvSourceLimit are split into their low 30 bits and the rest
   bool conv_fp = true;
-  bool digits_narrow = true;  // every Q prime is below the FP64 limit: digit conversions need no splitting
+  bool digits_narrow = true;  // every Q prime is below the conversion's source limit: digits need no splitting
   void conv_fp_tables(ConvJob& j, const std::vector<size_t>& src, const std::vector<size_t>& tgt, const u64* hat,
                       size_t hat_stride, bool force_split, size_t pad_sources) {
     j.fw = j.fq = nullptr;
@@ -205,7 +205,7 @@ struct ace_ctx {
       any |= j.fp_target[jj] != 0;
     }
     for (size_t s : src) {
-      narrow &= h.primes[s].q < kFpPrimeLimit;
+      narrow &= h.primes[s].q < kFpConvSourceLimit;
       fits &= h.primes[s].q < ((u64)1 << 62);
     }
     if (!any || !fits) {
@@ -371,7 +371,7 @@ struct ace_ctx {
       // FP64 twiddles for the primes the FP64 NTT back end can take
       const char* force_int = std::getenv("ACE_NTT_FORCE_INT");
       conv_fp = !(force_int && force_int[0] == '1');
-      for (size_t i = 0; i < h.L; ++i) digits_narrow &= h.primes[i].q < kFpPrimeLimit;
+      for (size_t i = 0; i < h.L; ++i) digits_narrow &= h.primes[i].q < kFpConvSourceLimit;
       bool use_fp = conv_fp && h.logN > 12;
       std::vector<double> w(T * h.N, 0.0), iw(T * h.N, 0.0);
       for (size_t i = 0; i < T; ++i) {

@@ -12,7 +12,7 @@ constexpr int kMaxBatchPtrs = 32; // keys / index tables per batched launch
 
 // one digit's base conversion: out[map.out_limb[j]][i] = (sum_k t[k][i] * hat[k*hat_stride + j]) mod prime map.prime[j]
 // Targets below the FP64 limit can take the conversion in exact double arithmetic (fp_mode != 0):
-//   fp_mode 1: every source prime is below the limit too; term k is t_k with cofactor fw[k][j]
+//   fp_mode 1: every source prime is below kFpConvSourceLimit; term k is t_k with cofactor fw[k][j]
 //   fp_mode 2: sources may be up to 2^62: t_k is split into its low 30 bits and the rest,
 //              term 2k is the low part with fw[2k][j] = hat, term 2k+1 the high part with
 //              fw[2k+1][j] = hat * 2^30 mod m_j

@@ -104,6 +104,43 @@ def test_ntt_largest_primes_of_the_fp64_back_end(N, primes):
         o.close()
 
 
+def test_conversion_from_a_51_bit_prime_taken_whole():
+    """A 51-bit first prime over 46-bit ones (the shape of the reference's model programs): the base conversion's
+    FP64 path takes such a source without splitting it.  Inputs are chosen so that the words entering the
+    conversion are q-1, (q+1)/2 or 1 in every source limb, besides seeded uniform ones."""
+    cfg = (8192, 7, 51, 46, 3)
+    g, o = acefhe.Context(*cfg), Oracle(*cfg)
+    try:
+        N, level = g.N, g.L
+        q = [int(x) for x in g.primes[:level]]
+        assert 2 ** 50.9 < q[0] < 3 << 50 and all(x < 1 << 47 for x in q[1:])
+        rng = np.random.Generator(np.random.PCG64(51))
+        for case in range(4):
+            limbs = []
+            for t in range(level):
+                part = t // g.part_size
+                digit = q[part * g.part_size:min(level, (part + 1) * g.part_size)]
+                rest = 1
+                for m in digit:
+                    rest *= m if m != q[t] else 1
+                pool = [(v * rest) % q[t] for v in (q[t] - 1, (q[t] + 1) // 2, 1)]
+                if case == 3:
+                    limbs.append(rng.integers(0, q[t], N))
+                else:
+                    limbs.append(np.array(pool, np.int64)[rng.integers(0, 3, N) if case else np.zeros(N, np.int64)])
+            x = np.concatenate(limbs).astype(np.int64)
+            dx = g.upload(x)
+            for is_ntt in (False, True):
+                dr = g.alloc(g.num_decomp(level) * (level + g.K) * N)
+                g.precomp(dr, dx, level, is_ntt)
+                eq(dr, o.precomp(x, level, is_ntt), "precomp case %d ntt %d" % (case, is_ntt))
+                dr.free()
+            dx.free()
+    finally:
+        g.close()
+        o.close()
+
+
 def test_ntt_batched_polys(pair):
     g, o = pair.g, pair.o
     N = g.N
