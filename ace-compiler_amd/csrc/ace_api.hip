@@ -632,11 +632,20 @@ void ace_ctx::flush_run() {
     const bool scalar = op >= EW_ADD_S && op <= EW_MULADD_S;
     return BatchOpDev{o.r, o.a, scalar ? o.scalar : (u64)(uintptr_t)o.b, o.op, o.prime};
   };
+  // two elements per thread when every range of the run allows 16-byte accesses
+  bool pairs = n % 2 == 0;
+  for (u32 k = 0; k < count && pairs; ++k) {
+    const BatchOp& o = sorted[k];
+    uintptr_t rd[3];
+    reads_of(o, rd);
+    const uintptr_t table = o.op == BATCH_ROTATE ? (uintptr_t)o.b : 0;
+    pairs = (((uintptr_t)o.r | rd[0] | rd[1] | table) & 15) == 0;
+  }
   if (count <= kSmallRun) {
     SmallRun small{};
     for (u32 k = 0; k < count; ++k) small.ops[k] = compact(sorted[k]);
     for (size_t k = 0; k < chain_start.size(); ++k) small.chain_start[k] = (uint16_t)chain_start[k];
-    launch_ew_batch_small(stream, d, small, n_chains, n);
+    launch_ew_batch_small(stream, d, small, n_chains, n, pairs);
     return;
   }
   // entries and chain starts travel in one copy: [entries | chain starts]
@@ -650,7 +659,7 @@ void ace_ctx::flush_run() {
   std::memcpy(image.data() + ops_bytes, chain_start.data(), chain_bytes);
   h2d(run_dev, image.data(), image.size());
   launch_ew_batch(stream, d, run_dev, reinterpret_cast<const u32*>(reinterpret_cast<const unsigned char*>(run_dev) + ops_bytes),
-                  n_chains, n);
+                  n_chains, n, pairs);
 }
 
 namespace {
@@ -758,7 +767,7 @@ void do_precomp(ace_ctx* c, u64* res, u64 res_stride, const u64* src, u64 src_st
 // 1 add addend.at(p) to every polynomial, 2 only to even p
 void do_mod_down(ace_ctx* c, const PolySeq& res, const PolySeq& src, size_t np, size_t level, bool is_ntt,
                  const PolySeq* addend, int addend_mode, const OrderSet* orders = nullptr) {
-  const size_t N = c->h.N, K = c->h.K, L = c->h.L;
+  const size_t N = c->h.N, K = c->h.K;
   size_t mark = c->ws_used;
   u64* t = c->take(np * K * N);
   u64* y = c->take(np * level * N);

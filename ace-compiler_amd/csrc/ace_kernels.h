@@ -104,9 +104,10 @@ struct SmallRun {
   BatchOpDev ops[kSmallRun];
   uint16_t chain_start[kSmallRun + 1];
 };
-void launch_ew_batch_small(hipStream_t st, const DevCtx& c, const SmallRun& run, u32 n_chains, u64 n);
+void launch_ew_batch_small(hipStream_t st, const DevCtx& c, const SmallRun& run, u32 n_chains, u64 n, bool pairs);
 // chain y (blockIdx.y) is the entries [chain_start[y], chain_start[y+1]): chains share no written range, so they run side by side
-void launch_ew_batch(hipStream_t st, const DevCtx& c, const BatchOpDev* dev_ops, const u32* dev_chain_start, u32 n_chains, u64 n);
+void launch_ew_batch(hipStream_t st, const DevCtx& c, const BatchOpDev* dev_ops, const u32* dev_chain_start, u32 n_chains,
+                     u64 n, bool pairs);
 void launch_sample_uniform(hipStream_t st, const DevCtx& c, u64* r, u64 seed, u64 stream, const LimbMap& lm,
                            u32 n_limbs, u64 n);
 void launch_expand_small(hipStream_t st, const DevCtx& c, u64* r, const i64* v, const LimbMap& lm, u32 n_limbs, u64 n);

@@ -131,57 +131,110 @@ void launch_plain_mac_groups(hipStream_t st, const DevCtx& c, const MacGroups& o
 // The host splits a run into chains that share no written range; a chain's entries are carried out in order by
 // the thread of element i, so an entry may read what an earlier one of its chain wrote (identical ranges only;
 // a rotate never reads or overwrites anything the run touches).
-__device__ __forceinline__ void run_chain(const DevCtx& c, const BatchOpDev* ops, u32 first, u32 last, u64 i);
-__global__ __launch_bounds__(kThreads) void ew_batch_kernel(DevCtx c, const BatchOpDev* ops, const u32* chain_start, u64 n) {
-  const u64 i = (u64)blockIdx.x * kThreads + threadIdx.x;
-  if (i >= n) return;
-  run_chain(c, ops, chain_start[blockIdx.y], chain_start[blockIdx.y + 1], i);
+// A thread carries V consecutive elements (V = 2 when every range of the run is 16-byte aligned: 16-byte loads
+// and stores, half the waves).
+template <int V>
+struct Words {
+  u64 v[V];
+};
+template <int V>
+__device__ __forceinline__ Words<V> load_words(const u64* p) {
+  Words<V> w;
+  if constexpr (V == 2) {
+    const ulonglong2 t = *reinterpret_cast<const ulonglong2*>(p);
+    w.v[0] = t.x;
+    w.v[1] = t.y;
+  } else {
+    w.v[0] = p[0];
+  }
+  return w;
 }
-__global__ __launch_bounds__(kThreads) void ew_batch_small_kernel(DevCtx c, SmallRun run, u64 n) {
-  const u64 i = (u64)blockIdx.x * kThreads + threadIdx.x;
-  if (i >= n) return;
-  run_chain(c, run.ops, run.chain_start[blockIdx.y], run.chain_start[blockIdx.y + 1], i);
+template <int V>
+__device__ __forceinline__ void store_words(u64* p, const Words<V>& w) {
+  if constexpr (V == 2) *reinterpret_cast<ulonglong2*>(p) = make_ulonglong2(w.v[0], w.v[1]);
+  else p[0] = w.v[0];
 }
+
+template <int V>
 __device__ __forceinline__ void run_chain(const DevCtx& c, const BatchOpDev* ops, u32 first, u32 last, u64 i) {
-  // what the previous entry produced stays in a register: an operand that names that range is not loaded again
+  // what the previous entry produced stays in registers: an operand that names that range is not loaded again
   const u64* prev_r = nullptr;
-  u64 prev_v = 0;
+  Words<V> prev{};
   for (u32 k = first; k < last; ++k) {
     const BatchOpDev o = ops[k];
     const u64* ob = reinterpret_cast<const u64*>(o.b);
     const u32 op = o.op & ~kBatchDeadStore;
     const DevPrime P = c.primes[o.prime];
-    u64 v;
+    Words<V> v;
     if (op == BATCH_ROTATE) {
-      const i64 src = reinterpret_cast<const i64*>(ob)[i];
-      v = src >= 0 ? o.a[src] : P.q - o.a[-src];
+      const Words<V> src = load_words<V>(ob + i);
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        const i64 j = (i64)src.v[e];
+        v.v[e] = j >= 0 ? o.a[j] : P.q - o.a[-j];
+      }
     } else if (op == BATCH_COPY) {
-      v = o.a == prev_r ? prev_v : o.a[i];
+      v = o.a == prev_r ? prev : load_words<V>(o.a + i);
     } else if (op == BATCH_ZERO) {
-      v = 0;
+#pragma unroll
+      for (int e = 0; e < V; ++e) v.v[e] = 0;
     } else {
-      const u64 x = o.a == prev_r ? prev_v : o.a[i];
-      const u64 y = op >= EW_ADD_S ? o.b : (ob == prev_r ? prev_v : ob[i]);
-      if (op == EW_ADD || op == EW_ADD_S) v = add_mod(x, y, P.q);
-      else if (op == EW_SUB || op == EW_SUB_S) v = sub_mod(x, y, P.q);
-      else if (op == EW_MUL || op == EW_MUL_S) v = mulmod(x, y, P);
-      else v = add_mod(o.r == prev_r ? prev_v : o.r[i], mulmod(x, y, P), P.q);
+      const Words<V> x = o.a == prev_r ? prev : load_words<V>(o.a + i);
+      Words<V> y;
+      if (op >= EW_ADD_S) {
+#pragma unroll
+        for (int e = 0; e < V; ++e) y.v[e] = o.b;
+      } else {
+        y = ob == prev_r ? prev : load_words<V>(ob + i);
+      }
+      if (op == EW_ADD || op == EW_ADD_S) {
+#pragma unroll
+        for (int e = 0; e < V; ++e) v.v[e] = add_mod(x.v[e], y.v[e], P.q);
+      } else if (op == EW_SUB || op == EW_SUB_S) {
+#pragma unroll
+        for (int e = 0; e < V; ++e) v.v[e] = sub_mod(x.v[e], y.v[e], P.q);
+      } else if (op == EW_MUL || op == EW_MUL_S) {
+#pragma unroll
+        for (int e = 0; e < V; ++e) v.v[e] = mulmod(x.v[e], y.v[e], P);
+      } else {
+        const Words<V> acc = o.r == prev_r ? prev : load_words<V>(o.r + i);
+#pragma unroll
+        for (int e = 0; e < V; ++e) v.v[e] = add_mod(acc.v[e], mulmod(x.v[e], y.v[e], P), P.q);
+      }
     }
-    if (!(o.op & kBatchDeadStore)) o.r[i] = v;
+    if (!(o.op & kBatchDeadStore)) store_words<V>(o.r + i, v);
     // a rotate's result is never read inside its run
     prev_r = op == BATCH_ROTATE ? nullptr : o.r;
-    prev_v = v;
+    prev = v;
   }
 }
-void launch_ew_batch_small(hipStream_t st, const DevCtx& c, const SmallRun& run, u32 n_chains, u64 n) {
-  if (!n || !n_chains) return;
-  dim3 g((unsigned)((n + kThreads - 1) / kThreads), n_chains, 1);
-  hipLaunchKernelGGL(ew_batch_small_kernel, g, dim3(kThreads), 0, st, c, run, n);
+template <int V>
+__global__ __launch_bounds__(kThreads) void ew_batch_kernel(DevCtx c, const BatchOpDev* ops, const u32* chain_start, u64 n) {
+  const u64 i = ((u64)blockIdx.x * kThreads + threadIdx.x) * V;
+  if (i >= n) return;
+  run_chain<V>(c, ops, chain_start[blockIdx.y], chain_start[blockIdx.y + 1], i);
 }
-void launch_ew_batch(hipStream_t st, const DevCtx& c, const BatchOpDev* dev_ops, const u32* dev_chain_start, u32 n_chains, u64 n) {
+template <int V>
+__global__ __launch_bounds__(kThreads) void ew_batch_small_kernel(DevCtx c, SmallRun run, u64 n) {
+  const u64 i = ((u64)blockIdx.x * kThreads + threadIdx.x) * V;
+  if (i >= n) return;
+  run_chain<V>(c, run.ops, run.chain_start[blockIdx.y], run.chain_start[blockIdx.y + 1], i);
+}
+// pairs: every range of the run starts on a 16-byte boundary and n is even
+void launch_ew_batch_small(hipStream_t st, const DevCtx& c, const SmallRun& run, u32 n_chains, u64 n, bool pairs) {
   if (!n || !n_chains) return;
-  dim3 g((unsigned)((n + kThreads - 1) / kThreads), n_chains, 1);
-  hipLaunchKernelGGL(ew_batch_kernel, g, dim3(kThreads), 0, st, c, dev_ops, dev_chain_start, n);
+  const u64 per_block = (u64)kThreads * (pairs ? 2 : 1);
+  dim3 g((unsigned)((n + per_block - 1) / per_block), n_chains, 1);
+  if (pairs) hipLaunchKernelGGL(ew_batch_small_kernel<2>, g, dim3(kThreads), 0, st, c, run, n);
+  else hipLaunchKernelGGL(ew_batch_small_kernel<1>, g, dim3(kThreads), 0, st, c, run, n);
+}
+void launch_ew_batch(hipStream_t st, const DevCtx& c, const BatchOpDev* dev_ops, const u32* dev_chain_start, u32 n_chains,
+                     u64 n, bool pairs) {
+  if (!n || !n_chains) return;
+  const u64 per_block = (u64)kThreads * (pairs ? 2 : 1);
+  dim3 g((unsigned)((n + per_block - 1) / per_block), n_chains, 1);
+  if (pairs) hipLaunchKernelGGL(ew_batch_kernel<2>, g, dim3(kThreads), 0, st, c, dev_ops, dev_chain_start, n);
+  else hipLaunchKernelGGL(ew_batch_kernel<1>, g, dim3(kThreads), 0, st, c, dev_ops, dev_chain_start, n);
 }
 
 // ---- key-generation helpers: uniform residues and small signed polynomials spread over limbs ------------
