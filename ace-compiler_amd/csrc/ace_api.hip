@@ -702,7 +702,7 @@ void do_decomp_modup(ace_ctx* c, u64* res, const u64* digit, size_t level, size_
   size_t mark = c->ws_used;
   u64* t = c->take(nd * N);
   if (is_ntt) {
-    const PolySeq through = seq_strided(res + start * N, 0);
+    const CopyThrough through{seq_strided(res + start * N, 0), 0, ~0u};
     if (!launch_ntt(c->stream, c->d, seq_strided(t, 0), seq_strided(digit, 0), m.digit_lm, nullptr, (u32)nd, 1, true,
                     m.scale_ntt, 3, nullptr, by_transform ? &through : nullptr))
       throw std::runtime_error("internal: Mod_up transform rejected");
@@ -730,15 +730,20 @@ void do_precomp(ace_ctx* c, u64* res, u64 res_stride, const u64* src, u64 src_st
   const size_t N = c->h.N, nd = c->h.num_decomp(level), T = level + c->h.K;
   size_t mark = c->ws_used;
   u64* t = c->take(nb * level * N);
+  // the digits' own limbs pass through; the inverse transform of a large ring drops that copy as it reads them
+  const bool by_transform = is_ntt && c->d.logN > 12;
   if (is_ntt) {
-    launch_ntt(c->stream, c->d, seq_strided(t, level * N), seq_strided(src, src_stride), c->q_lm, nullptr, (u32)level,
-               (u32)nb, true, pd.scale_ntt);
+    const CopyThrough through{seq_strided(res, res_stride), (u64)(T * N), (u32)c->h.part_size};
+    if (!launch_ntt(c->stream, c->d, seq_strided(t, level * N), seq_strided(src, src_stride), c->q_lm, nullptr,
+                    (u32)level, (u32)nb, true, pd.scale_ntt, 3, nullptr, by_transform ? &through : nullptr))
+      throw std::runtime_error("internal: Mod_up transform rejected");
   } else {
     for (size_t o = 0; o < nb; ++o)
       launch_mul_const(c->stream, c->d, t + o * level * N, src + o * src_stride, pd.scale_coef, c->q_lm, (u32)level);
   }
-  launch_digit_copy(c->stream, c->d, res, src, (u32)level, (u32)c->h.part_size, (u32)nd, T * N, res_stride, src_stride,
-                    (u32)nb);
+  if (!by_transform)
+    launch_digit_copy(c->stream, c->d, res, src, (u32)level, (u32)c->h.part_size, (u32)nd, T * N, res_stride,
+                      src_stride, (u32)nb);
   for (size_t j0 = 0; j0 < nd; j0 += kMaxConvJobs) {
     ConvBatch b{};
     b.n_jobs = (u32)std::min<size_t>(kMaxConvJobs, nd - j0);

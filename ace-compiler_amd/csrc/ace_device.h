@@ -78,6 +78,14 @@ inline PolySeq seq_pair(const u64* c0, const u64* c1, u64 op_stride) {
   return s;
 }
 
+// where an inverse transform drops a copy of the words it reads: limb t of polynomial p goes to
+// seq.at(p) + (t / part_size) * digit_stride + t * N (the digits' own limbs inside raised polynomials)
+struct CopyThrough {
+  PolySeq seq;
+  u64 digit_stride;
+  u32 part_size;
+};
+
 // base conversion: target j -> prime index and limb position in the output
 struct ConvMap {
   uint8_t prime[kMaxPrimes];

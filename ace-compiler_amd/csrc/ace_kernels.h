@@ -53,7 +53,7 @@ struct OrderSet { // one automorphism table per rotation, or one shared (n == 1)
 // only holds the intermediate between the two kernels.  Returns false when the request cannot be served.
 bool launch_ntt(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolySeq& src, const LimbMap& lm,
                 const LimbMap* pos, u32 n_limbs, u32 n_polys, bool inverse, const u64* scale, int passes = 3,
-                const FwdFuse* fuse = nullptr, const PolySeq* copy_src_to = nullptr);
+                const FwdFuse* fuse = nullptr, const CopyThrough* copy_src_to = nullptr);
 
 constexpr u32 kMaxMacOps = 32;
 struct MacSet { // operands of one multiply-accumulate launch

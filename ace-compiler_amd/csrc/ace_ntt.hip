@@ -498,7 +498,7 @@ __global__ __launch_bounds__(kChunkThreads, EPI == 1 ? 6 : 8) void ntt_fwd_chunk
 // are those of the forward pass in reverse order.
 template <class A>
 __device__ __forceinline__ void inv_chunk_body(u64* lds_words, const DevCtx& c, const PolySeq& dsts,
-                                               const PolySeq& srcs, const PolySeq& copies, const LimbMap& pos,
+                                               const PolySeq& srcs, const CopyThrough& copies, const LimbMap& pos,
                                                u32 n_polys, u32 chunk, u32 limb, u32 pblk, u32 pi) {
   typedef typename A::T T;
   T* lds = reinterpret_cast<T*>(lds_words);
@@ -523,8 +523,8 @@ __device__ __forceinline__ void inv_chunk_body(u64* lds_words, const DevCtx& c, 
 #pragma unroll
       for (int r = 0; r < 8; ++r) nxt[r] = src[off + t + 512 * r];
     }
-    if (copies.b[0]) {  // the untransformed words are wanted elsewhere too (the digit that Mod_up passes through)
-      u64* cp = copies.at(poly0 + it);
+    if (copies.seq.b[0]) {  // the untransformed words are wanted elsewhere too (the digits that Mod_up passes through)
+      u64* cp = copies.seq.at(poly0 + it) + (u64)(pos.prime[limb] / copies.part_size) * copies.digit_stride;
 #pragma unroll
       for (int r = 0; r < 8; ++r) cp[off + t + 512 * r] = raw[r];
     }
@@ -576,7 +576,7 @@ __device__ __forceinline__ void inv_chunk_body(u64* lds_words, const DevCtx& c, 
     for (int r = 0; r < 8; ++r) raw[r] = nxt[r];
   }
 }
-__global__ __launch_bounds__(kChunkThreads, 8) void ntt_inv_chunk(DevCtx c, PolySeq dsts, PolySeq srcs, PolySeq copies,
+__global__ __launch_bounds__(kChunkThreads, 8) void ntt_inv_chunk(DevCtx c, PolySeq dsts, PolySeq srcs, CopyThrough copies,
                                                                   LimbMap lm, LimbMap pos, u32 n_limbs, u32 n_polys) {
   __shared__ u64 lds[kChunk + kChunk / 16];
   u32 chunk, limb, pblk;
@@ -661,7 +661,7 @@ __global__ __launch_bounds__(256) void ntt_small(DevCtx c, PolySeq dsts, PolySeq
 template <int LOGR>
 static void run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolySeq& src, const LimbMap& lm,
                       const LimbMap& pos, u32 n_limbs, u32 n_polys, bool inverse, const u64* scale, int passes,
-                      const FwdFuse& f, const PolySeq& copies) {
+                      const FwdFuse& f, const CopyThrough& copies) {
   dim3 gs((c.N >> LOGR) / 256, n_limbs, n_polys),
       gc(chunk_grid(c, n_limbs, (n_polys + kPolysPerBlock - 1) / kPolysPerBlock));
   if (!inverse) {
@@ -701,11 +701,12 @@ static void run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst, const
 
 bool launch_ntt(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolySeq& src, const LimbMap& lm,
                 const LimbMap* pos_in, u32 n_limbs, u32 n_polys, bool inverse, const u64* scale, int passes,
-                const FwdFuse* fuse, const PolySeq* copy_src_to) {
+                const FwdFuse* fuse, const CopyThrough* copy_src_to) {
   if (n_limbs == 0 || n_polys == 0) return true;
-  PolySeq copies{};
+  CopyThrough copies{};
   if (copy_src_to) {  // only the inverse chunk pass can drop a copy of what it reads
     if (!inverse || c.logN <= kLogChunk || !(passes & 1)) return false;
+    if (!copy_src_to->part_size) return false;
     copies = *copy_src_to;
   }
   FwdFuse f{};
