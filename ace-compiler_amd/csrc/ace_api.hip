@@ -189,36 +189,22 @@ struct ace_ctx {
   }
   ShoupConst sc(u64 w, size_t prime) const { return {w, shoup(w, h.primes[prime].q)}; }
 
-  // FP64 tables of a base conversion (ConvJob::fw / fq): targets below the FP64 limit convert in
-  // exact double arithmetic; sources at or above kFpConvSourceLimit are split into their low 30 bits and the rest
+  // FP64 tables of a base conversion (ConvJob::fw / fq) for the targets below kFpConvTargetLimit
   bool conv_fp = true;
-  bool digits_narrow = true;  // every Q prime is below the conversion's source limit: digits need no splitting
   void conv_fp_tables(ConvJob& j, const std::vector<size_t>& src, const std::vector<size_t>& tgt, const u64* hat,
-                      size_t hat_stride, bool force_split, size_t pad_sources) {
+                      size_t hat_stride) {
     j.fw = j.fq = nullptr;
-    j.fp_mode = j.fw_stride = j.fp_pad = 0;
+    j.fw_stride = 0;
     std::memset(j.fp_target, 0, sizeof(j.fp_target));
-    if (!conv_fp) return;
-    bool any = false, narrow = !force_split, fits = pad_sources != 0 && src.size() <= pad_sources;
+    if (!conv_fp || src.size() > 16) return;  // 48 products at most in a sum
+    bool any = false;
     for (size_t jj = 0; jj < tgt.size(); ++jj) {
-      j.fp_target[jj] = h.primes[tgt[jj]].q < kFpPrimeLimit ? 1 : 0;
+      j.fp_target[jj] = h.primes[tgt[jj]].q < kFpConvTargetLimit ? 1 : 0;
       any |= j.fp_target[jj] != 0;
     }
-    for (size_t s : src) {
-      narrow &= h.primes[s].q < kFpConvSourceLimit;
-      fits &= h.primes[s].q < ((u64)1 << 62);
-    }
-    if (!any || !fits) {
-      std::memset(j.fp_target, 0, sizeof(j.fp_target));
-      return;
-    }
+    if (!any) return;
     const size_t nd = src.size(), nc = tgt.size();
-    const size_t terms = pad_sources * (narrow ? 1 : 2);  // zero rows past the real sources
-    std::vector<double> fw(terms * nc * 2, 0.0), fq(nc * 2, 0.0);
-    auto put = [&](size_t term, size_t jj, u64 w, u64 q) {
-      fw[2 * (term * nc + jj)] = (double)w;
-      fw[2 * (term * nc + jj) + 1] = (double)((long double)w / (long double)q);
-    };
+    std::vector<double> fw(3 * nd * nc * 2 + 8, 0.0), fq(nc * 2, 0.0);  // a margin of four entries for grouped reads
     for (size_t jj = 0; jj < nc; ++jj) {
       const u64 q = h.primes[tgt[jj]].q;
       fq[2 * jj] = (double)q;
@@ -226,19 +212,16 @@ struct ace_ctx {
       if (!j.fp_target[jj]) continue;
       for (size_t k = 0; k < nd; ++k) {
         const u64 w = hat[k * hat_stride + jj];
-        if (narrow) {
-          put(k, jj, w, q);
-        } else {
-          put(2 * k, jj, w, q);
-          put(2 * k + 1, jj, mul_mod(w, ((u64)1 << 30) % q, q), q);
+        for (size_t i = 0; i < 3; ++i) {
+          const u64 wi = mul_mod(w, ((u64)1 << (21 * i)) % q, q);
+          fw[2 * ((3 * k + i) * nc + jj)] = (double)(wi >> 26);
+          fw[2 * ((3 * k + i) * nc + jj) + 1] = (double)(wi & (((u64)1 << 26) - 1));
         }
       }
     }
     j.fw = upload_vec(fw);
     j.fq = upload_vec(fq);
-    j.fp_mode = narrow ? 1 : 2;
     j.fw_stride = (u32)nc;
-    j.fp_pad = (u32)pad_sources;
   }
 
   void ensure_ws(size_t words) {
@@ -292,8 +275,7 @@ struct ace_ctx {
     m.job.nc = (u32)nc;
     m.job.map = m.conv;
     conv_fp_tables(m.job, std::vector<size_t>(m.t.digit.begin(), m.t.digit.end()),
-                   std::vector<size_t>(m.t.compl_idx.begin(), m.t.compl_idx.end()), m.t.hat.data(), nc,
-                   !digits_narrow, (size_t)conv_padded_sources((u32)h.part_size));
+                   std::vector<size_t>(m.t.compl_idx.begin(), m.t.compl_idx.end()), m.t.hat.data(), nc);
     return modup.emplace(key, std::move(m)).first->second;
   }
 
@@ -371,7 +353,6 @@ struct ace_ctx {
       // FP64 twiddles for the primes the FP64 NTT back end can take
       const char* force_int = std::getenv("ACE_NTT_FORCE_INT");
       conv_fp = !(force_int && force_int[0] == '1');
-      for (size_t i = 0; i < h.L; ++i) digits_narrow &= h.primes[i].q < kFpConvSourceLimit;
       bool use_fp = conv_fp && h.logN > 12;
       std::vector<double> w(T * h.N, 0.0), iw(T * h.N, 0.0);
       for (size_t i = 0; i < T; ++i) {
@@ -428,7 +409,7 @@ struct ace_ctx {
       p2q_job.hat_stride = (u32)h.L;
       p2q_job.nd = (u32)h.K;
       p2q_job.nc = (u32)h.L;
-      conv_fp_tables(p2q_job, src, tgt, ph.data(), h.L, true, (size_t)conv_padded_sources((u32)h.K));
+      conv_fp_tables(p2q_job, src, tgt, ph.data(), h.L);
     }
     pscale_ntt = upload_vec(sn);
     pscale_coef = upload_vec(scf);

@@ -44,10 +44,9 @@ struct DevCtx {
 // largest prime the FP64 back end accepts: below 2^50.2, so that eight stages'
 // worth of lazily accumulated magnitude stays under 2^53 (see ace_ntt.hip)
 constexpr u64 kFpPrimeLimit = 1290000000000000ull;
-// largest source prime the FP64 base conversion takes whole (3 * 2^50).  A term x*w mod m with
-// x below this limit comes out within (1/2 + x 2^-52) m <= 1.25 m; four terms on top of a
-// re-centred sum stay below 5.5 m < 2^53 for every target m below kFpPrimeLimit.
-constexpr u64 kFpConvSourceLimit = (u64)3 << 50;
+// largest target prime of the FP64 base conversion (3 * 2^50): the halves of a cofactor stay below 2^26, so 48
+// products with 21-bit pieces of the sources add up below 2^53, and 1.4 m < 2^53 in the final reduction
+constexpr u64 kFpConvTargetLimit = (u64)3 << 50;
 
 // limb t of a launch -> prime index
 struct LimbMap {

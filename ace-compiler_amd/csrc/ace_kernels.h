@@ -11,13 +11,10 @@ constexpr int kMaxConvJobs = 4;   // digits converted per base-conversion launch
 constexpr int kMaxBatchPtrs = 32; // keys / index tables per batched launch
 
 // one digit's base conversion: out[map.out_limb[j]][i] = (sum_k t[k][i] * hat[k*hat_stride + j]) mod prime map.prime[j]
-// Targets below the FP64 limit can take the conversion in exact double arithmetic (fp_mode != 0):
-//   fp_mode 1: every source prime is below kFpConvSourceLimit; term k is t_k with cofactor fw[k][j]
-//   fp_mode 2: sources may be up to 2^62: t_k is split into its low 30 bits and the rest,
-//              term 2k is the low part with fw[2k][j] = hat, term 2k+1 the high part with
-//              fw[2k+1][j] = hat * 2^30 mod m_j
-// fw: [terms][fw_stride][2] = (cofactor, cofactor / m_j) as doubles, the terms padded with zero rows to
-//     fp_pad sources; fq: [nc][2] = (m_j, 1 / m_j);
+// Targets below kFpConvTargetLimit take the conversion in exact double arithmetic when the job has tables (fw):
+// a source word is cut into three 21-bit pieces, row 3k+i of fw belongs to piece i of source k:
+// fw: [3 nd][fw_stride][2] = the halves above and below bit 26 of hat * 2^(21 i) mod m_j as doubles (plus a margin of
+//     four entries); fq: [nc][2] = (m_j, 1 / m_j);
 // fp_target[j] says whether target j uses them.
 struct ConvJob {
   const u64* hat;
@@ -26,7 +23,7 @@ struct ConvJob {
   ConvMap map;
   const double* fw;
   const double* fq;
-  u32 fp_mode, fw_stride, fp_pad;  // fp_pad: sources the tables are padded to (4, 8, 12 or 16)
+  u32 fw_stride;
   uint8_t fp_target[kMaxPrimes];
 };
 struct ConvBatch {
@@ -135,7 +132,6 @@ void launch_tensor(hipStream_t st, const DevCtx& c, u64* d0, u64* d1, u64* d2, c
                    const u64* b0, const u64* b1, const LimbMap& lm, u32 n_limbs, u32 n_ops, u64 d01_stride,
                    u64 d2_stride, u64 in_stride);
 // fast base conversion of b.n_jobs digits for each of n_ops operands
-int conv_padded_sources(u32 nd);
 void launch_baseconv(hipStream_t st, const DevCtx& c, u64* out, const u64* t, const ConvBatch& b, u32 n_ops);
 // digit limbs of src copied into the raised polynomials (see digit_copy_kernel)
 void launch_digit_copy(hipStream_t st, const DevCtx& c, u64* res, const u64* src, u32 level, u32 part_size,

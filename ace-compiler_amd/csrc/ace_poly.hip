@@ -396,44 +396,39 @@ void launch_tensor(hipStream_t st, const DevCtx& c, u64* d0, u64* d1, u64* d2, c
 }
 
 // ---- fast base conversion (rns_poly.c:218-242, rns_poly_impl.c:324-336) ----
-// One thread per coefficient and kConvTargets targets; the nd source words
-// stay in registers, the cofactor table is read through wave-uniform loads.
-// blockIdx.z enumerates (operand, job): a job is one digit's conversion, all
-// jobs of a launch share the operand strides.
+// One thread per coefficient and kConvTargets targets.  blockIdx.z enumerates (operand, job): a job is one
+// digit's conversion, all jobs of a launch share the operand strides.
+//
+// Targets below kFpConvTargetLimit are converted in exact FP64 arithmetic: a source word (< 2^63) is cut into
+// three 21-bit pieces; the table holds, for piece i of source k, the two halves (above and below bit 26) of
+// hat * 2^(21 i) mod m.  3 * 16 products below 2^47 add up exactly in each of the two sums (below 2^52.6 < 2^53,
+// one FMA each), and high * 2^26 + low is reduced once per target.  A group whose targets are all of that kind
+// makes one pass over the sources with the table read through wave-uniform loads, a row of it holding the group's
+// entries side by side.  Larger targets (the 60-bit special primes) take nd 128-bit multiply-adds and one
+// Barrett reduction each, from source words kept in registers.
 constexpr int kConvTargets = 4;
 
-// exact x*w mod q in doubles: |result| <= (1/2 + |x| 2^-52) q; w, wi = w/q, q as doubles
-__device__ __forceinline__ double conv_fp_term(double x, double w, double wi, double q) {
-#pragma clang fp contract(off)
-  double c = __builtin_rint(x * wi);
-  double h = x * w;
-  double l = __builtin_fma(x, w, -h);
-  double d = __builtin_fma(-c, q, h);
-  return d + l;
+__device__ __forceinline__ void conv_pieces(u64 x, double piece[3]) {
+  piece[0] = (double)((u32)x & 0x1FFFFFu);
+  piece[1] = (double)((u32)(x >> 21) & 0x1FFFFFu);
+  piece[2] = (double)(u32)(x >> 42);
 }
 
-// one target in FP64: TERMS exact products accumulated as integers below 2^53
-// (re-centred every 4 terms), result canonical.  The table holds TERMS rows
-// (rows past the real sources are zero), so the loop has no guards.
-template <int TERMS>
-__device__ __forceinline__ u64 conv_fp_target(const double* xd, const double* __restrict__ fw, u32 stride, u32 j,
-                                              double q, double qinv) {
+__device__ __forceinline__ u64 conv_fp_finish(double hi, double lo, double q, double qinv) {
 #pragma clang fp contract(off)
-  double acc = 0.0;
-#pragma unroll
-  for (int k = 0; k < TERMS; ++k) {
-    const double2 ww = *reinterpret_cast<const double2*>(fw + 2 * ((u64)k * stride + j));
-    acc += conv_fp_term(xd[k], ww.x, ww.y, q);
-    if ((k & 3) == 3 && k + 1 < TERMS) acc = __builtin_fma(-__builtin_rint(acc * qinv), q, acc);
-  }
+  hi = __builtin_fma(-__builtin_rint(hi * qinv), q, hi);  // |hi| <= m/2
+  lo = __builtin_fma(-__builtin_rint(lo * qinv), q, lo);
+  // hi * 2^26 mod m: the product is exact (a power of two), the quotient is off by less than 1/2 + |hi| 2^-52
+  const double c = __builtin_rint(hi * (67108864.0 * qinv));
+  double acc = __builtin_fma(-c, q, hi * 67108864.0) + lo;  // |acc| < 1.4 m < 2^53
   acc = __builtin_fma(-__builtin_rint(acc * qinv), q, acc);
   acc = acc < 0.0 ? acc + q : acc;
   return (u64)__double_as_longlong(acc + 4503599627370496.0) & 0x000FFFFFFFFFFFFFull;
 }
 
-// MAXS: compile-time bound on the number of source limbs (register arrays); 0 = any number, looped.
-// MODE: ConvJob::fp_mode of every job of the launch (0: integer arithmetic only).
-template <int MAXS, int MODE>
+// MAXS: compile-time bound on the number of source limbs (register array of the integer path); 0 = any number,
+// looped, integer arithmetic only.  FP: every job of the launch has FP64 tables.
+template <int MAXS, int FP>
 __global__ __launch_bounds__(kThreads) void baseconv_kernel(DevCtx c, u64* __restrict__ out_base,
                                                             const u64* __restrict__ t_base, ConvBatch b) {
   const u64 n = c.N;
@@ -448,29 +443,63 @@ __global__ __launch_bounds__(kThreads) void baseconv_kernel(DevCtx c, u64* __res
   const u32 j0 = blockIdx.y * kConvTargets;
   if (j0 >= nc) return;
   if constexpr (MAXS > 0) {
+    if constexpr (FP != 0) {
+      bool all_fp = true;  // wave-uniform
+#pragma unroll
+      for (int jj = 0; jj < kConvTargets; ++jj) all_fp &= j0 + jj >= nc || J.fp_target[j0 + jj] != 0;
+      if (all_fp) {
+        // rows are read up to three entries past a ragged last group: the table is allocated with that margin
+        double hi[kConvTargets], lo[kConvTargets];
+#pragma unroll
+        for (int jj = 0; jj < kConvTargets; ++jj) hi[jj] = lo[jj] = 0.0;
+        const double2* __restrict__ row = reinterpret_cast<const double2*>(J.fw) + j0;
+        const u32 stride = J.fw_stride;
+#pragma unroll 2
+        for (u32 k = 0; k < nd; ++k) {
+          double piece[3];
+          conv_pieces(t[(u64)k * n + i], piece);
+#pragma unroll
+          for (int pc = 0; pc < 3; ++pc) {
+#pragma unroll
+            for (int jj = 0; jj < kConvTargets; ++jj) {
+              const double2 ww = row[(u64)(3 * k + pc) * stride + jj];
+              hi[jj] = __builtin_fma(piece[pc], ww.x, hi[jj]);
+              lo[jj] = __builtin_fma(piece[pc], ww.y, lo[jj]);
+            }
+          }
+        }
+#pragma unroll
+        for (int jj = 0; jj < kConvTargets; ++jj) {
+          const u32 j = j0 + jj;
+          if (j < nc) out[(u64)J.map.out_limb[j] * n + i] = conv_fp_finish(hi[jj], lo[jj], J.fq[2 * j], J.fq[2 * j + 1]);
+        }
+        return;
+      }
+    }
     u64 x[MAXS];
 #pragma unroll
     for (int k = 0; k < MAXS; ++k) x[k] = (u32)k < nd ? t[(u64)k * n + i] : 0;
-    constexpr int TERMS = MODE == 1 ? MAXS : (MODE == 2 ? 2 * MAXS : 1);
-    double xd[TERMS];
-    if constexpr (MODE == 1) {
-#pragma unroll
-      for (int k = 0; k < MAXS; ++k)
-        xd[k] = __longlong_as_double((long long)(x[k] | 0x4330000000000000ull)) - 4503599627370496.0;
-    } else if constexpr (MODE == 2) {
-#pragma unroll
-      for (int k = 0; k < MAXS; ++k) {
-        xd[2 * k] = (double)(u32)(x[k] & 0x3FFFFFFFu);
-        xd[2 * k + 1] = (double)(u32)(x[k] >> 30);
-      }
-    }
 #pragma unroll
     for (int jj = 0; jj < kConvTargets; ++jj) {
       u32 j = j0 + jj;
       if (j >= nc) break;
-      if (MODE != 0 && J.fp_target[j]) {  // wave-uniform
-        out[(u64)J.map.out_limb[j] * n + i] =
-            conv_fp_target<TERMS>(xd, J.fw, J.fw_stride, j, J.fq[2 * j], J.fq[2 * j + 1]);
+      if (FP != 0 && J.fp_target[j]) {  // wave-uniform: an FP64 target in a group that has others too
+        double hi = 0.0, lo = 0.0;
+        const double2* __restrict__ col = reinterpret_cast<const double2*>(J.fw) + j;
+#pragma unroll
+        for (int k = 0; k < MAXS; ++k) {
+          if ((u32)k < nd) {
+            double piece[3];
+            conv_pieces(x[k], piece);
+#pragma unroll
+            for (int pc = 0; pc < 3; ++pc) {
+              const double2 ww = col[(u64)(3 * k + pc) * J.fw_stride];
+              hi = __builtin_fma(piece[pc], ww.x, hi);
+              lo = __builtin_fma(piece[pc], ww.y, lo);
+            }
+          }
+        }
+        out[(u64)J.map.out_limb[j] * n + i] = conv_fp_finish(hi, lo, J.fq[2 * j], J.fq[2 * j + 1]);
         continue;
       }
       u64 hi = 0, lo = 0;
@@ -494,24 +523,24 @@ __global__ __launch_bounds__(kThreads) void baseconv_kernel(DevCtx c, u64* __res
   }
 }
 
-// register-array size used for nd source limbs (0: the looped kernel); the FP64 tables are padded to it
-int conv_padded_sources(u32 nd) { return nd <= 4 ? 4 : nd <= 8 ? 8 : nd <= 12 ? 12 : nd <= 16 ? 16 : 0; }
+// register-array size used for nd source limbs (0: the looped kernel)
+static int conv_padded_sources(u32 nd) { return nd <= 4 ? 4 : nd <= 8 ? 8 : nd <= 12 ? 12 : nd <= 16 ? 16 : 0; }
 
 void launch_baseconv(hipStream_t st, const DevCtx& c, u64* out, const u64* t, const ConvBatch& b, u32 n_ops) {
   if (!b.n_jobs || !n_ops) return;
-  u32 max_nc = 0, max_nd = 0, mode = b.job[0].fp_mode, pad = b.job[0].fp_pad;
+  u32 max_nc = 0, max_nd = 0;
+  bool fp = true;  // jobs without FP64 tables keep the launch to integer arithmetic
   for (u32 k = 0; k < b.n_jobs; ++k) {
     max_nc = b.job[k].nc > max_nc ? b.job[k].nc : max_nc;
     max_nd = b.job[k].nd > max_nd ? b.job[k].nd : max_nd;
-    if (b.job[k].fp_mode != mode || b.job[k].fp_pad != pad) mode = 0;  // mixed launches keep to integer arithmetic
+    fp &= b.job[k].fw != nullptr;
   }
   if (!max_nc) return;
-  if (mode != 0 && max_nd > pad) mode = 0;
-  const int maxs = mode != 0 ? (int)pad : conv_padded_sources(max_nd);
+  const int maxs = conv_padded_sources(max_nd);
   dim3 g((c.N + kThreads - 1) / kThreads, (max_nc + kConvTargets - 1) / kConvTargets, b.n_jobs * n_ops);
 #define ACE_BC(S, M) hipLaunchKernelGGL((baseconv_kernel<S, M>), g, dim3(kThreads), 0, st, c, out, t, b)
 #define ACE_BC_MODES(S) \
-  do { if (mode == 1) ACE_BC(S, 1); else if (mode == 2) ACE_BC(S, 2); else ACE_BC(S, 0); } while (0)
+  do { if (fp) ACE_BC(S, 1); else ACE_BC(S, 0); } while (0)
   switch (maxs) {
     case 4: ACE_BC_MODES(4); break;
     case 8: ACE_BC_MODES(8); break;

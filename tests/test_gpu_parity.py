@@ -104,9 +104,9 @@ def test_ntt_largest_primes_of_the_fp64_back_end(N, primes):
         o.close()
 
 
-def test_conversion_from_a_51_bit_prime_taken_whole():
-    """A 51-bit first prime over 46-bit ones (the shape of the reference's model programs): the base conversion's
-    FP64 path takes such a source without splitting it.  Inputs are chosen so that the words entering the
+def test_conversion_with_a_51_bit_first_prime():
+    """A 51-bit first prime over 46-bit ones (the shape of the reference's model programs): the prime is both a
+    source and a target of the base conversion's FP64 path.  Inputs are chosen so that the words entering the
     conversion are q-1, (q+1)/2 or 1 in every source limb, besides seeded uniform ones."""
     cfg = (8192, 7, 51, 46, 3)
     g, o = acefhe.Context(*cfg), Oracle(*cfg)
@@ -136,6 +136,19 @@ def test_conversion_from_a_51_bit_prime_taken_whole():
                 eq(dr, o.precomp(x, level, is_ntt), "precomp case %d ntt %d" % (case, is_ntt))
                 dr.free()
             dx.free()
+        # Mod_down: the 60-bit special primes are the sources, the 51-bit prime one of the targets
+        pr = [g.primes[i] for i in g.limb_primes(level)]
+        for case in range(2):
+            e = seeded.uniform_poly(5100 + case, pr, N)
+            if case:  # the largest source words
+                e = np.concatenate([np.full(N, int(m) - 1, np.int64) for m in pr])
+            de = g.upload(e)
+            for is_ntt in (False, True):
+                dr = g.alloc(level * N)
+                g.mod_down(dr, de, level, is_ntt)
+                eq(dr, o.mod_down(e, level, is_ntt), "mod_down case %d ntt %d" % (case, is_ntt))
+                dr.free()
+            de.free()
     finally:
         g.close()
         o.close()
