@@ -454,7 +454,7 @@ __global__ __launch_bounds__(kThreads) void baseconv_kernel(DevCtx c, u64* __res
         for (int jj = 0; jj < kConvTargets; ++jj) hi[jj] = lo[jj] = 0.0;
         const double2* __restrict__ row = reinterpret_cast<const double2*>(J.fw) + j0;
         const u32 stride = J.fw_stride;
-#pragma unroll 2
+#pragma unroll 4
         for (u32 k = 0; k < nd; ++k) {
           double piece[3];
           conv_pieces(t[(u64)k * n + i], piece);
