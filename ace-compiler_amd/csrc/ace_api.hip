@@ -65,6 +65,29 @@ struct RescaleDev {
   u64* tail = nullptr;  // [level-1][2]: q_l^-1, Shoup
 };
 
+// Scratch of ace_mod_down_noalloc: the intermediates of one Mod_down (the scaled inverse transform of the P limbs
+// and their conversion to the Q basis), held in a device array that exists from the moment the library is loaded.
+// Each GPU has its own copy at its own address; host code reaches it only through the pointer that
+// hipGetSymbolAddress returned for that GPU (static_scratch_of).
+constexpr size_t kStaticScratchWords = (size_t)1 << 21;  // 16 MiB
+static __device__ __align__(256) __attribute__((used)) unsigned long long scratch[kStaticScratchWords];
+constexpr int kMaxDevices = 64;
+u64* g_static_scratch[kMaxDevices] = {nullptr};
+
+// the address of `scratch` on the current device, looked up once per device
+u64* static_scratch_of_current_device() {
+  int dev = -1;
+  HIP_OK(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) throw std::runtime_error("device ordinal out of range");
+  if (!g_static_scratch[dev]) {
+    void* ptr = nullptr;
+    HIP_OK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    if (!ptr) throw std::runtime_error("hipGetSymbolAddress returned no address for the static scratch");
+    g_static_scratch[dev] = static_cast<u64*>(ptr);
+  }
+  return g_static_scratch[dev];
+}
+
 }  // namespace
 
 // Hw_* calls recorded for one launch (see flush_run)
@@ -178,6 +201,7 @@ struct ace_ctx {
   // scratch arena
   u64* ws = nullptr;
   size_t ws_words = 0, ws_used = 0;
+  u64* static_scratch = nullptr;  // this GPU's copy of the device array `scratch` (ace_mod_down_noalloc)
 
   template <class T>
   T* upload_vec(const std::vector<T>& v) {
@@ -333,6 +357,7 @@ struct ace_ctx {
   }
 
   void init_device() {
+    static_scratch = static_scratch_of_current_device();
     HIP_OK(hipStreamCreateWithFlags(&stream, hipStreamNonBlocking));
     HIP_OK(hipEventCreate(&ev0));
     HIP_OK(hipEventCreate(&ev1));
@@ -1543,6 +1568,41 @@ int ace_mod_down(ace_ctx* c, int64_t* res, const int64_t* src, size_t level, int
   if (!level_ok(c, level)) return fail("ace_mod_down: level out of range");
   c->flush_run();
   c->submit_poly(1, U(res), U(src), level, is_ntt != 0);
+  ACE_CATCH_INT
+}
+
+int ace_mod_down_noalloc(ace_ctx* c, int64_t* res, const int64_t* src, size_t level, int is_ntt) {
+  ACE_TRY_BARE
+  if (!res || !src) return fail("ace_mod_down_noalloc: null argument");
+  if (!level_ok(c, level)) return fail("ace_mod_down_noalloc: level out of range");
+  const size_t need = (level + c->h.K) * (size_t)c->h.N;
+  if (need > kStaticScratchWords)
+    return fail("ace_mod_down_noalloc: (level + num_p) * degree = " + std::to_string(need) + " words exceeds the static "
+                "scratch of " + std::to_string(kStaticScratchWords) + " words (16 MiB); use ace_mod_down");
+  // Recorded calls that are pending go first, as before every entry point.  A short run travels as kernel
+  // arguments; a longer one is staged through buffers that may have to be allocated, and a pending Mod_down or
+  // Rescale takes its scratch from the arena, which may have to grow: those are refused here.
+  if (c->ppoly.kind || c->run.ops.size() > kSmallRun)
+    return fail("ace_mod_down_noalloc: more recorded calls are pending than can be launched without allocating; "
+                "call ace_sync() first");
+  c->flush_run();
+  // the sequencer takes its intermediates from the arena: point the arena at the static array for this call
+  struct ArenaSwap {
+    ace_ctx* c;
+    u64* ws;
+    size_t words, used;
+    ArenaSwap(ace_ctx* c_, u64* p, size_t n) : c(c_), ws(c_->ws), words(c_->ws_words), used(c_->ws_used) {
+      c->ws = p;
+      c->ws_words = n;
+      c->ws_used = 0;
+    }
+    ~ArenaSwap() {
+      c->ws = ws;
+      c->ws_words = words;
+      c->ws_used = used;
+    }
+  } swap(c, c->static_scratch, kStaticScratchWords);
+  do_mod_down(c, seq_strided(U(res), 0), seq_strided(const_cast<u64*>(U(src)), 0), 1, level, is_ntt != 0, nullptr, 0);
   ACE_CATCH_INT
 }
 

@@ -184,6 +184,16 @@ int ace_mod_up(ace_ctx* ctx, int64_t* res, const int64_t* digit, size_t level, s
 int ace_precomp(ace_ctx* ctx, int64_t* res, const int64_t* src, size_t level, int is_ntt);
 /* Mod_down (:260-308): src level+num_p limbs -> res level limbs */
 int ace_mod_down(ace_ctx* ctx, int64_t* res, const int64_t* src, size_t level, int is_ntt);
+/* Mod_down for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same operands and result as ace_mod_down;
+ * the intermediates live in a 16 MiB device array that is part of the library image (one copy per GPU, held until
+ * the process ends), so the call performs no hipMalloc / hipFree and takes nothing from the context's arena.
+ * Rejected when (level + num_p) * degree exceeds 2^21 words, and while more than 96 recorded ace_hw_* calls or a
+ * paired Mod_down / Rescale are pending (their launch may allocate: ace_sync first; up to 96 recorded calls are
+ * launched first, as kernel arguments).  Every call on one GPU shares that array: calls that overlap in time on one GPU (two
+ * contexts, two streams) race; calls on one context are ordered by its stream.  Nothing in the array needs to
+ * start at zero: each call writes every word it later reads. */
+int ace_mod_down_noalloc(ace_ctx* ctx, int64_t* res, const int64_t* src, size_t level, int is_ntt);
 /* Rescale (:310-404): src level limbs -> res level-1 limbs */
 int ace_rescale(ace_ctx* ctx, int64_t* res, const int64_t* src, size_t level, int is_ntt);
 /* Mod_down_rescale (:531-597): Mod_down and rescale in one pass over the coefficient
