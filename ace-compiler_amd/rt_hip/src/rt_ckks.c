@@ -6,6 +6,7 @@
  */
 #include <complex.h>
 #include <math.h>
+#include <sys/random.h>
 
 #include "rt_internal.h"
 
@@ -148,9 +149,20 @@ void Rt_generate_keys(uint64_t seed) {
   if (!seed) {
     const char* env = getenv("RT_HIP_SEED");
     seed = env ? strtoull(env, NULL, 0) : 0;
-    if (!seed) seed = (uint64_t)time(NULL) ^ ((uint64_t)clock() << 32) ^ 0x5DEECE66Dull;
   }
-  rng_seed(seed);
+  if (seed) {
+    rng_seed(seed); /* a fixed seed: reproducible runs for tests and benchmarks only */
+  } else {
+    /* no seed given: the whole generator state comes from the operating system's entropy pool (the reference seeds
+     * its generator from /dev/urandom, util/src/prng.c:56-109), so the secret cannot be found by a seed search */
+    if (getrandom(Rng, sizeof(Rng), 0) != (ssize_t)sizeof(Rng)) {
+      FILE* f = fopen("/dev/urandom", "rb");
+      FMT_ASSERT(f && fread(Rng, sizeof(Rng), 1, f) == 1, "no entropy source for key generation");
+      fclose(f);
+    }
+    FMT_ASSERT(Rng[0] | Rng[1] | Rng[2] | Rng[3], "entropy source returned zeros");
+    seed = rng_next(); /* the device-side stream of public uniform polynomials */
+  }
   Seed   = seed;
   Stream = 0;
   Rt_ckks_finalize(); /* a second call replaces the keys */
@@ -427,6 +439,7 @@ static uint64_t powmod64(uint64_t a, uint64_t e, uint64_t q) {
  * mpz_get_d: mixed-radix digits, exact multi-word evaluation, comparison with Q/2 */
 static double crt_to_double(const int64_t* v, size_t level, const uint64_t* inv /* [level]: (q_0..q_{i-1})^-1 mod q_i */) {
   uint64_t d[64];
+  FMT_ASSERT(level <= 64, "decoding supports at most 64 limbs, the ciphertext has %zu", level);
   for (size_t i = 0; i < level; ++i) {
     uint64_t q = (uint64_t)G.q[i]._val, acc = 0, prod = 1;
     for (size_t j = 0; j < i; ++j) {

@@ -74,7 +74,7 @@ static void free_slots(IO_SLOT* s, size_t n) {
 
 void Finalize_context(void) {
   if (!G.ctx) return;
-  if (Get_rt_data_info && Get_rt_data_info()) Pt_mgr_fini();
+  Pt_mgr_fini(); /* always: the kept plaintexts are device buffers of this context */
   Rt_bootstrap_finalize();
   Rt_ckks_finalize();
   free_key(&G.relin);

@@ -187,31 +187,40 @@ def bootstrap_leg():
 def resnet20_leg():
     """The reference's generated ResNet-20/CIFAR-10 program (rtlib/ant/dataset/resnet20_cifar10_pre.onnx.inc,
     N=65536, 34 limbs, 197 rotation keys, 19 bootstraps), built unchanged against the host runtime where the reference
-    tree was present.  Its weight file is not available, so the weights are pseudo-random
-    (RT_HIP_SYNTHETIC_WEIGHTS): the run measures time per image, not accuracy.  The reference's published run takes
-    1453.96 s per image on one CPU thread."""
+    tree was present, on the 60/56-bit chain the reference's build script compiles it with
+    (scripts/build_resnet20_cifar10.sh:13-14,32; the committed program carries the compiler's defaults 51/46, on which
+    its bootstraps are far outside their precision).  Its weight file is not available, so the weights are
+    pseudo-random (RT_HIP_SYNTHETIC_WEIGHTS): the run measures time per image, and a second run under other keys
+    measures how far the logits depend on the keys and the noise."""
     exe = os.path.join(ROOT, "oracle", "_ref", "models", "resnet20_cifar10_pre.onnx")
     if not os.path.exists(exe):
         return {"resnet20": {"skipped": "the model binary is built only where the reference tree is present"}}
     try:
-        env = dict(os.environ, RT_HIP_SYNTHETIC_WEIGHTS="0.05")
+        env = dict(os.environ, RT_HIP_SYNTHETIC_WEIGHTS="0.15", MODEL_Q0_BITS="60", MODEL_SF_BITS="56", MODEL_KEY_SEED="11")
         # three images one after another: the first pays for encoding every weight plaintext, the later ones find
         # the encoded polynomials in HBM
         r = subprocess.run([exe, "3", "32", "32", "10", "1", "3"], capture_output=True, text=True, timeout=400, env=env)
         line = [l for l in r.stdout.splitlines() if l.startswith("context_s")][0].split()
         vals = dict(zip(line[0::2], (float(v) for v in line[1::2])))
         later = [float(l.split()[5]) for l in r.stdout.splitlines() if l.startswith("image ")]
-        out = {"workload": "ResNet-20 CIFAR-10 inference, the reference's generated program, synthetic weights and "
-                           "images, three images one after another", "main_graph_s": vals["main_graph_s"],
+        logits = [float(v) for v in [l for l in r.stdout.splitlines() if l.startswith("output:")][0].split()[1:]]
+        out = {"workload": "ResNet-20 CIFAR-10 inference, the reference's generated program on the 60/56-bit chain, "
+                           "synthetic weights and images, three images one after another",
+               "main_graph_s": vals["main_graph_s"],
+               "main_graph_s_note": "first image: every weight plaintext is encoded on the fly, as the reference does "
+                                    "for every image (the like-for-like figure)",
                "keygen_s": vals["keygen_s"], "input_s": vals["input_s"], "output_s": vals["output_s"],
                "exit_status": r.returncode, "published_cpu_s": 1453.96,
-               "published_cpu_note": "the reference's published run uses a 60/56-bit chain and trained weights on "
-                                     "other hardware; this program's chain is 51/46 bits: times are not comparable "
-                                     "as a ratio",
-               "later_images_note": "later images reuse the encoded weight plaintexts kept in HBM; the first image "
-                                    "encodes them all, as the reference does for every image"}
+               "published_cpu_note": "the reference's published run: same chain, trained weights, one CPU thread of "
+                                     "other hardware; not a same-run baseline"}
         if later:
             out["main_graph_s_later_images"] = later
+            out["later_images_note"] = "later images reuse the encoded weight plaintexts kept in HBM"
+        env["MODEL_KEY_SEED"] = "22"
+        r2 = subprocess.run([exe, "3", "32", "32", "10", "1"], capture_output=True, text=True, timeout=400, env=env)
+        again = [float(v) for v in [l for l in r2.stdout.splitlines() if l.startswith("output:")][0].split()[1:]]
+        out["logits_first_image"] = logits
+        out["logit_spread_under_other_keys"] = max(abs(x - y) for x, y in zip(logits, again))
         return {"resnet20": out}
     except Exception as e:
         return {"resnet20": {"error": repr(e)[:200]}}

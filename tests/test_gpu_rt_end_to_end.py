@@ -136,11 +136,71 @@ def test_bootstrap_refreshes_levels(args, env):
 RESNET20 = os.path.join(rt_program.ROOT, "oracle", "_ref", "models", "resnet20_cifar10_pre.onnx")
 
 
-def test_reference_resnet20_program_runs():
+def bootstrap_error(args):
+    """max_err printed by bootstrap_program (its exit status says whether that is below 1e-3)."""
+    print("running bootstrap_program", args, flush=True)
+    r = subprocess.run([BOOTSTRAP] + args.split(), capture_output=True, text=True, timeout=200)
+    assert r.returncode in (0, 1) and "max_err" in r.stdout, r.stdout + r.stderr
+    f = r.stdout.split()
+    return float(f[f.index("max_err") + 1]), r.returncode
+
+
+def test_bootstrap_precision_at_the_model_ring():
+    """N = 65536, 34 limbs, Hamming weight 192, 32768 slots, refreshed to level 15 (the call of the ResNet programs).
+    On the chain the reference's build scripts compile the models with (q0 = 60, scale = 56 bits:
+    scripts/build_resnet20_cifar10.sh:13-14,32) the error stays below 1e-3.  The scale is tracked nominally, as in the
+    reference (Rescale_ciphertext divides the recorded scale by 2^scale_bits, ckks/src/evaluator.c:342-362, with
+    _scaling_factor = 1 << scaling_mod_size, ckks/src/param.c:68), so every rescale leaves the relative error
+    d_l = q_l / 2^scale_bits - 1 of its prime in the value; the sine evaluation sees it multiplied by the integer
+    part, q0 / scale and, after the slot transform, sqrt(N).  d_l is the distance of the primes = 1 mod 2N from
+    2^scale_bits, so it grows with N and falls with 2^scale_bits: the error follows that law across rings and
+    chains, and the defaults compiled into the committed programs (51 / 46 bits) are far outside 1e-3 at this ring."""
+    assert os.path.exists(BOOTSTRAP), "tests/programs/bootstrap_program is not built"
+    good, rc = bootstrap_error("65536 33 60 56 192 32768 15 1")
+    assert rc == 0 and good < 1e-3, good
+    e46, _ = bootstrap_error("65536 33 51 46 192 32768 15 1")
+    e50, _ = bootstrap_error("65536 33 55 50 192 32768 15 1")
+    e46_small, _ = bootstrap_error("16384 33 51 46 192 8192 15 1")
+    print("max_err: 60/56 %.3g  55/50 %.3g  51/46 %.3g  51/46 at N=16384 %.3g" % (good, e50, e46, e46_small), flush=True)
+    assert 1e-2 < e46 < 1.0
+    # 4 more scale bits: d_l / 16; a quarter of the ring: d_l / 4 and sqrt(N) / 2 -- each within a factor 3
+    assert 16 / 3 < e46 / e50 < 16 * 3, (e46, e50)
+    assert 8 / 3 < e46 / e46_small < 8 * 3, (e46, e46_small)
+
+
+def resnet20_logits(chain, key_seed, amplitude="0.15"):
+    env = dict(os.environ, RT_HIP_SYNTHETIC_WEIGHTS=amplitude, MODEL_Q0_BITS=str(chain[0]), MODEL_SF_BITS=str(chain[1]),
+               MODEL_KEY_SEED=str(key_seed))
+    print("running", RESNET20, "chain", chain, "key seed", key_seed, flush=True)
+    r = subprocess.run([RESNET20, "3", "32", "32", "10", "1"], capture_output=True, text=True, timeout=230, env=env)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    out = [l for l in r.stdout.splitlines() if l.startswith("output:")][0].split()[1:]
+    assert len(out) == 10
+    return [float(v) for v in out]
+
+
+def test_reference_resnet20_program_is_stable_under_the_keys():
     """The compiler's ResNet-20 program (7000 lines of generated C at N=65536, 34 limbs, 197 rotation keys, 19
-    bootstraps, 1038 weight plaintexts encoded on the fly), unchanged, to the end.  The weight file is not part of the
-    reference tree, so the weights are pseudo-random and only completion and finite outputs are checked; the
-    operators it is made of are checked with expected values by the reference's examples above."""
+    bootstraps, 1038 weight plaintexts encoded on the fly), unchanged, on the chain the reference's build script
+    compiles it with (60 / 56 bits).  The weight file is not part of the reference tree, so weights and image are
+    pseudo-random and there is no expected output; what is checked is that the ten logits do not depend on the
+    secret key, the encryption randomness or the key-switching noise: two runs that differ in all of those agree
+    within 1e-3 (a numerically meaningless run, as on the compiled-in 51 / 46 chain, fails this by orders of
+    magnitude).  The operators the program is made of are checked with expected values by the reference's examples."""
+    if not os.path.exists(RESNET20):
+        pytest.skip("built only where the reference tree is present")
+    a, b = resnet20_logits((60, 56), 11), resnet20_logits((60, 56), 22)
+    spread = max(abs(x - y) for x, y in zip(a, b))
+    print("logits", a, "spread", spread, flush=True)
+    assert all(v == v and abs(v) < 10 for v in a)
+    assert max(abs(v) for v in a) > 5e-3, "the logits carry no signal"
+    assert spread < 1e-3 and spread < 0.05 * max(abs(v) for v in a), spread
+
+
+def test_reference_resnet20_program_runs_on_its_compiled_in_chain():
+    """The same program with the parameters it carries (51 / 46 bits): runs to the end.  Its bootstraps are far
+    outside their precision on this chain (test_bootstrap_precision_at_the_model_ring), in the reference's arithmetic
+    as here, so nothing is asserted about the values beyond their being numbers."""
     if not os.path.exists(RESNET20):
         pytest.skip("built only where the reference tree is present")
     env = dict(os.environ, RT_HIP_SYNTHETIC_WEIGHTS="0.05")
