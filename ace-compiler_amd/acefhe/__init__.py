@@ -76,6 +76,7 @@ def _sig(lib):
     f("ace_encode", C.c_int, _vp, _vp, _vp, _sz, C.c_uint32, _sz, C.c_uint32, _sz)
     f("ace_ext_plain_mac_groups", C.c_int, _vp, _vp, _vp, _sz, _vp, _vp, _sz, _vp, _sz, _sz)
     f("ace_ext_rotate", C.c_int, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp, _sz, C.c_int)
+    f("ace_encode_scaled", C.c_int, _vp, _vp, _vp, _sz, C.c_uint32, _sz, C.c_double, _sz)
     f("ace_encode_real", C.c_int, _vp, _vp, _vp, C.c_int, _sz, C.c_uint32, _sz, C.c_uint32, _sz)
     f("ace_mod_down_rescale", C.c_int, _vp, _vp, _vp, _sz, C.c_int)
     f("ace_reduce_rescale_modup", C.c_int, _vp, _vp, _vp, _vp, _sz, C.c_int)
@@ -115,7 +116,7 @@ EXPORTS = [
     "ace_hw_modsub_scalar", "ace_hw_modmul_scalar", "ace_hw_modmuladd_scalar", "ace_hw_rotate",
     "ace_find_automorphism_index", "ace_automorphism_order", "ace_poly_add", "ace_poly_sub", "ace_poly_mul",
     "ace_poly_automorphism", "ace_decomp_modup", "ace_mod_up", "ace_mod_down_rescale",
-    "ace_reduce_rescale_modup", "ace_transform_from_level0", "ace_host_fft_tables", "ace_embedding_inv", "ace_encode", "ace_encode_real", "ace_ext_rotate", "ace_ext_plain_mac_groups", "ace_precomp", "ace_mod_down", "ace_rescale", "ace_extend",
+    "ace_reduce_rescale_modup", "ace_transform_from_level0", "ace_host_fft_tables", "ace_embedding_inv", "ace_encode", "ace_encode_scaled", "ace_encode_real", "ace_ext_rotate", "ace_ext_plain_mac_groups", "ace_precomp", "ace_mod_down", "ace_rescale", "ace_extend",
     "ace_dot_prod", "ace_mul_ciph3", "ace_fast_switch_key", "ace_relin", "ace_rescale_ciph",
     "ace_mul_relin_rescale", "ace_mul_relin_rescale_batch", "ace_fast_rotate", "ace_rotate_batch",
 ]
@@ -331,6 +332,11 @@ class Context:
         v = np.ascontiguousarray(values, dtype=np.complex128)
         self._chk(self.lib.ace_encode(self.h, res.ptr, v.ctypes.data_as(C.c_void_p), v.size, slots, level, sf_degree,
                                       p_cnt))
+
+    def encode_scaled(self, res, values, slots, level, scale, p_cnt=0):
+        v = np.ascontiguousarray(values, dtype=np.complex128)
+        self._chk(self.lib.ace_encode_scaled(self.h, res.ptr, v.ctypes.data_as(C.c_void_p), v.size, slots, level,
+                                             float(scale), p_cnt))
 
     def encode_real(self, res, values, slots=0, level=0, sf_degree=1, p_cnt=0):
         """values: a float32 or float64 array of real numbers."""

@@ -1674,8 +1674,10 @@ int ace_embedding_inv(ace_ctx* c, double* host_out, const double* host_in, size_
 
 // kind: 0 complex doubles (re, im interleaved), 1 real doubles, 2 real floats.  Real inputs travel as they are and
 // are widened to complex numbers on the device (a float widens exactly, as the host cast would).
+// explicit_scale > 0: Encode_impl_with_scale (encoder.c:337-403): one multiplication by that scale, rounded without
+// the half that Encode_impl adds first, and no further powers of the scaling factor.
 static int encode_impl(ace_ctx* c, int64_t* res, const void* values, int kind, size_t n_values, uint32_t slots,
-                       size_t level, uint32_t sf_degree, size_t p_cnt) {
+                       size_t level, uint32_t sf_degree, size_t p_cnt, double explicit_scale = 0.0) {
   ACE_TRY
   if (!res || (!values && n_values)) return fail("ace_encode: null argument");
   if (!c->sf_bits) return fail("ace_encode: the context was created from explicit primes and has no scaling factor");
@@ -1686,10 +1688,15 @@ static int encode_impl(ace_ctx* c, int64_t* res, const void* values, int kind, s
   if (n_values > slots) return fail("slot size is too small");
   if (slots > N / 2 || (slots & (slots - 1))) return fail("slot size must be a power of two of at most N/2");
   if (p_cnt != 0 && p_cnt != K) return fail("ace_encode: p_cnt must be 0 or the number of special primes");
-  if (sf_degree < 1 || c->sf_bits * sf_degree >= c->q0_bits + (level - 1) * c->sf_bits)
+  const bool by_scale = explicit_scale > 0.0;
+  if (by_scale) {
+    if ((uint32_t)std::log2(explicit_scale) >= c->q0_bits + (level - 1) * c->sf_bits) return fail("invalid scale for encode");
+    sf_degree = 1;
+  } else if (sf_degree < 1 || c->sf_bits * sf_degree >= c->q0_bits + (level - 1) * c->sf_bits) {
     return fail("invalid scaling factor for encode");
-  const double scaling_factor = std::ldexp(1.0, (int)c->sf_bits);
-  const double scale = std::pow(scaling_factor, (double)sf_degree);
+  }
+  const double scaling_factor = by_scale ? explicit_scale : std::ldexp(1.0, (int)c->sf_bits);
+  const double scale = by_scale ? explicit_scale : std::pow(scaling_factor, (double)sf_degree);
   // Check_msg_range (encoder.c:48-59): the largest scaled coefficient must stay below 2^(valid bits - 1)
   const int valid = (int)c->q0_bits + (int)(level - 1) * (int)c->sf_bits;
   const double range_bound = std::ldexp(1.0, valid - 1);
@@ -1710,8 +1717,8 @@ static int encode_impl(ace_ctx* c, int64_t* res, const void* values, int kind, s
   c->ws_used = 0;
   double2* z = reinterpret_cast<double2*>(c->take(2 * (size_t)slots));
   stage_values(c->stream, z, kind == 0 ? nullptr : c->take(slots));
-  launch_encode(c->stream, c->d, U(res), z, c->fft_rou, c->rot_group, slots, scaling_factor, scale, range_bound, lm,
-                n_limbs, c->d_err);
+  launch_encode(c->stream, c->d, U(res), z, c->fft_rou, c->rot_group, slots, scaling_factor, scale,
+                by_scale ? 0.0 : 0.5, range_bound, lm, n_limbs, c->d_err);
   if (sf_degree > 1) {  // encoder.c:297-312: the Q limbs are multiplied by scaling_factor^(sf_degree-1)
     std::vector<u64> cst(2 * level);
     for (size_t t = 0; t < level; ++t) {
@@ -1736,6 +1743,11 @@ int ace_encode(ace_ctx* c, int64_t* res, const double* values, size_t n_values, 
 int ace_encode_real(ace_ctx* c, int64_t* res, const void* values, int is_f32, size_t n_values, uint32_t slots,
                     size_t level, uint32_t sf_degree, size_t p_cnt) {
   return encode_impl(c, res, values, is_f32 ? 2 : 1, n_values, slots, level, sf_degree, p_cnt);
+}
+int ace_encode_scaled(ace_ctx* c, int64_t* res, const double* values, size_t n_values, uint32_t slots, size_t level,
+                      double scale, size_t p_cnt) {
+  if (!(scale > 0.0)) return fail("invalid scale for encode");
+  return encode_impl(c, res, values, 0, n_values, slots, level, 1, p_cnt, scale);
 }
 
 int ace_extend(ace_ctx* c, int64_t* res, const int64_t* src, size_t level) {

@@ -87,7 +87,8 @@ __device__ __forceinline__ i64 mod_int64(i64 v, i64 m) {
 __global__ __launch_bounds__(kEncThreads) void encode_round_kernel(DevCtx c, u64* __restrict__ out,
                                                                    const double2* __restrict__ r, u32 slots,
                                                                    u32 logslots, double scaling_factor, double scale,
-                                                                   double range_bound, LimbMap lm, int* err) {
+                                                                   double round_add, double range_bound, LimbMap lm,
+                                                                   int* err) {
 #pragma clang fp contract(off)
   const u32 n = blockIdx.x * kEncThreads + threadIdx.x;
   if (n >= c.N) return;
@@ -103,7 +104,7 @@ __global__ __launch_bounds__(kEncThreads) void encode_round_kernel(DevCtx c, u64
     const double2 z = r[src];
     const double v = (imag ? z.y : z.x) * (1.0 / (double)slots);  // slots is a power of two: exact, as the division is
     if (fabs(v * scale) >= range_bound) *err = 1;
-    const double up = v * scaling_factor + 0.5;
+    const double up = v * scaling_factor + round_add;  // 0.5 in Encode_impl, 0 in Encode_impl_with_scale
     if (!(up <= 9223372036854775807.0 && up >= -9223372036854775807.0)) {
       *err = 1;
     } else {
@@ -149,13 +150,13 @@ void launch_widen_real(hipStream_t st, double2* z, const void* raw, bool is_f32,
 }
 
 void launch_encode(hipStream_t st, const DevCtx& c, u64* out, double2* r, const double2* rou, const u32* rot,
-                   u32 slots, double scaling_factor, double scale, double range_bound, const LimbMap& lm,
-                   u32 n_limbs, int* err) {
+                   u32 slots, double scaling_factor, double scale, double round_add, double range_bound,
+                   const LimbMap& lm, u32 n_limbs, int* err) {
   u32 logslots = 0;
   while ((1u << logslots) < slots) ++logslots;
   launch_embed_inv_stages(st, r, rou, rot, 2 * c.N, slots);
   hipLaunchKernelGGL(encode_round_kernel, dim3((c.N + kEncThreads - 1) / kEncThreads, n_limbs), dim3(kEncThreads), 0,
-                     st, c, out, r, slots, logslots, scaling_factor, scale, range_bound, lm, err);
+                     st, c, out, r, slots, logslots, scaling_factor, scale, round_add, range_bound, lm, err);
 }
 
 }  // namespace ace

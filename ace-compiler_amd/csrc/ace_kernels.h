@@ -179,7 +179,7 @@ void launch_embedding_inv(hipStream_t st, const DevCtx& c, double2* out, double2
 // z[i] = (raw[i], 0) for i < n_values, (0, 0) up to slots; raw holds doubles or floats
 void launch_widen_real(hipStream_t st, double2* z, const void* raw, bool is_f32, u32 n_values, u32 slots);
 void launch_encode(hipStream_t st, const DevCtx& c, u64* out, double2* r, const double2* rou, const u32* rot,
-                   u32 slots, double scaling_factor, double scale, double range_bound, const LimbMap& lm,
-                   u32 n_limbs, int* err);
+                   u32 slots, double scaling_factor, double scale, double round_add, double range_bound,
+                   const LimbMap& lm, u32 n_limbs, int* err);
 
 }  // namespace ace

@@ -393,7 +393,9 @@ void Rt_bootstrap_prepare(void) {
   keygen(setup(slots));
 }
 
+static void stage_clear(void);
 void Rt_bootstrap_finalize(void) {
+  stage_clear();
   while (Precoms) {
     BTS_PRECOM* p = Precoms;
     Precoms       = p->next;
@@ -964,6 +966,107 @@ CIPHER Eval_bootstrap_ciph(CIPHER res, CIPHER ct, uint32_t level_after_bts, uint
   if (res->_c0_poly._data) Free_ciph_poly(res, 1);
   *res = work;
   return res;
+}
+
+/* ---- the stages on their own (cipher.c:585-767) ------------------------------------------------------
+ * The same pieces as above, cut where the compiler's staged operators cut them.  The imaginary half of a fully
+ * packed input lives here between the first two calls. */
+static struct {
+  bool       active, full;
+  uint32_t   slots;
+  CIPHERTEXT sub;
+} Stage;
+static void stage_clear(void) {
+  if (Stage.sub._c0_poly._data) Free_ciph_poly(&Stage.sub, 1);
+  memset(&Stage, 0, sizeof(Stage));
+}
+static uint32_t stage_slots(CIPHER ct, uint32_t num_slots) {
+  return num_slots ? num_slots : (ct->_slots ? ct->_slots : (uint32_t)(G.N / 2));
+}
+static CIPHER stage_result(CIPHER res, CIPHER ct, CIPHERTEXT* work) { /* res takes over work's polynomials */
+  if (res->_c0_poly._data && res != ct) Free_ciph_poly(res, 1);
+  if (res == ct) Free_ciph_poly(ct, 1);
+  *res = *work;
+  return res;
+}
+
+CIPHER Eval_bootstrap_coeffs_to_slots_ciph(CIPHER res, CIPHER ct, uint32_t num_slots) {
+  NEED_CTX();
+  stage_clear();
+  uint32_t    slots = stage_slots(ct, num_slots);
+  BTS_PRECOM* pre   = setup(slots);
+  keygen(pre);
+  bool       full = slots == G.N / 2;
+  CIPHERTEXT work, conj;
+  new_ciph(&work), new_ciph(&conj);
+  raise_modulus(&work, ct, (uint32_t)G.L, slots);
+  if (!full) {
+    for (uint32_t j = 1; j < G.N / (2 * slots); j <<= 1) {
+      rotate_into(&conj, &work, (int32_t)(j * slots));
+      Add_ciph(&work, &work, &conj);
+    }
+  }
+  coeff_slots_transform(&work, pre, true);
+  rotate_into(&conj, &work, (int32_t)(2 * G.N - 1));
+  if (full) {
+    new_ciph(&Stage.sub);
+    Sub_ciph(&Stage.sub, &work, &conj);
+    Add_ciph(&work, &work, &conj);
+    Mul_mono_ciph(&Stage.sub, &Stage.sub, (uint32_t)(3 * G.N / 2));
+    while (work._sf_degree > 1) {
+      rescale(&work);
+      rescale(&Stage.sub);
+    }
+  } else {
+    Add_ciph(&work, &work, &conj);
+    while (work._sf_degree > 1) rescale(&work);
+  }
+  Stage.active = true;
+  Stage.full   = full;
+  Stage.slots  = slots;
+  Free_ciph_poly(&conj, 1);
+  return stage_result(res, ct, &work);
+}
+
+CIPHER Eval_bootstrap_eval_mod_ciph(CIPHER res, CIPHER ct, uint32_t num_slots) {
+  NEED_CTX();
+  uint32_t    slots = stage_slots(ct, num_slots);
+  BTS_PRECOM* pre   = setup(slots);
+  keygen(pre);
+  CIPHERTEXT work;
+  new_ciph(&work);
+  Copy_ciph(&work, ct);
+  if (Stage.active && Stage.full && Stage.sub._c0_poly._data && Stage.slots == slots) {
+    eval_approx_mod(&work);
+    eval_approx_mod(&Stage.sub);
+    Mul_mono_ciph(&Stage.sub, &Stage.sub, slots);
+    Add_ciph(&work, &work, &Stage.sub);
+    Free_ciph_poly(&Stage.sub, 1);
+    new_ciph(&Stage.sub);
+  } else {
+    while (work._sf_degree > 1) rescale(&work);
+    eval_approx_mod(&work);
+  }
+  return stage_result(res, ct, &work);
+}
+
+CIPHER Eval_bootstrap_slots_to_coeffs_ciph(CIPHER res, CIPHER ct, uint32_t num_slots) {
+  NEED_CTX();
+  uint32_t    slots = stage_slots(ct, num_slots);
+  BTS_PRECOM* pre   = setup(slots);
+  keygen(pre);
+  CIPHERTEXT work, rot;
+  new_ciph(&work), new_ciph(&rot);
+  Copy_ciph(&work, ct);
+  coeff_slots_transform(&work, pre, false);
+  if (slots != G.N / 2) {
+    rotate_into(&rot, &work, (int32_t)slots);
+    Add_ciph(&work, &work, &rot);
+    Free_ciph_poly(&rot, 1);
+  }
+  finish(&work);
+  stage_clear();
+  return stage_result(res, ct, &work);
 }
 
 CIPHER Bootstrap(CIPHER res, CIPHER ct, uint32_t level_after_bts) {

@@ -70,6 +70,19 @@ static void sample_ternary(int64_t* v, size_t n, size_t weight) {
   }
 }
 
+static bool Rng_ready;
+void Rt_sample_ternary(int64_t* v, size_t n, size_t hamming_weight) {
+  if (!Rng_ready) { /* no key generation has seeded the stream yet: seed it as Rt_generate_keys(0) would */
+    const char* env  = getenv("RT_HIP_SEED");
+    uint64_t    seed = env ? strtoull(env, NULL, 0) : 0;
+    if (seed) rng_seed(seed);
+    else FMT_ASSERT(getrandom(Rng, sizeof(Rng), 0) == (ssize_t)sizeof(Rng) && (Rng[0] | Rng[1] | Rng[2] | Rng[3]),
+                    "no entropy source");
+    Rng_ready = true;
+  }
+  sample_ternary(v, n, hamming_weight);
+}
+
 /* ---- small helpers over the device ------------------------------------------------------------ */
 static uint64_t Seed, Stream; /* of the device-side uniform sampler: one stream per polynomial */
 
@@ -163,8 +176,9 @@ void Rt_generate_keys(uint64_t seed) {
     FMT_ASSERT(Rng[0] | Rng[1] | Rng[2] | Rng[3], "entropy source returned zeros");
     seed = rng_next(); /* the device-side stream of public uniform polynomials */
   }
-  Seed   = seed;
-  Stream = 0;
+  Seed      = seed;
+  Stream    = 0;
+  Rng_ready = true;
   Rt_ckks_finalize(); /* a second call replaces the keys */
   CKKS_PARAMS* prm = Get_context_params();
   size_t       n = G.N, T = G.L + G.K, hw = prm->_hamming_weight;
@@ -335,6 +349,31 @@ void Encode_dcmplx_ext(PLAIN plain, DCMPLX* input, size_t len, uint32_t level, u
   plain->_slots          = G.N / 2;
   p->_is_ntt             = true;
   ACE_OK(ace_encode(G.ctx, p->_data, (const double*)input, len, 0, level, 1, p_cnt));
+}
+/* Encode_float_with_scale (ckks/src/plain.c:104-123): the scale is given, the degree recorded is the least
+ * power of the scaling factor that reaches it (Get_approx_sf_degree, encoder.c:328-335) */
+void Encode_float_with_scale(PLAIN plain, float* input, size_t len, double scale, uint32_t level) {
+  NEED_CTX();
+  if (level == 0) level = (uint32_t)G.L;
+  FMT_ASSERT(level <= G.L, "level should not be larger than mul_depth + 1");
+  FMT_ASSERT(scale > 0 && G.sc != 1, "invalid scale for encode");
+  uint32_t deg = (uint32_t)floor(log2(scale) / log2(G.sc));
+  if (scale > pow(G.sc, deg)) ++deg;
+  init_plain(plain, level, scale, deg, G.N / 2);
+  if (len == 1) { /* Encode_val_at_level_with_scale (encoder.c:580-605) */
+    int64_t words[128];
+    Rt_encode_val_words(words, (double)*input, level, scale);
+    for (uint32_t t = 0; t < level; ++t) {
+      int64_t* limb = plain->_poly._data + (size_t)t * G.N;
+      ACE_OK(ace_zero(G.ctx, limb, G.N));
+      ACE_OK(ace_hw_modadd_scalar(G.ctx, limb, limb, words[t], t, G.N));
+    }
+    return;
+  }
+  double* v = (double*)calloc(2 * len, sizeof(double));
+  for (size_t i = 0; i < len; ++i) v[2 * i] = (double)input[i];
+  ACE_OK(ace_encode_scaled(G.ctx, plain->_poly._data, v, len, 0, level, scale, 0));
+  free(v);
 }
 /* Encode_single_double (ckks/src/plain.c:139-147): `level` host words */
 void Encode_single_double(int64_t* res, double input, uint32_t sc_degree, uint32_t level) {
@@ -611,12 +650,97 @@ double* Get_msg(CIPHER c) {
   free(v);
   return r;
 }
-void Print_cipher_msg(FILE* fp, const char* name, CIPHER c, uint32_t len) {
-  double* m = Get_msg(c);
-  fprintf(fp, "[%s] level %zu, sf_degree %u: {", name, Level(c), c->_sf_degree);
-  for (uint32_t i = 0; i < len; ++i) fprintf(fp, " %g", m[i]);
-  fprintf(fp, " }\n");
+/* the printers of ckks/src/cipher.c:228-338, in the reference's formats */
+static void print_msg_range(FILE* fp, const DCMPLX* msg, uint32_t n) {
+  double   lo_re = creal(msg[0]), hi_re = lo_re, lo_im = cimag(msg[0]), hi_im = lo_im;
+  uint32_t lo_re_at = 0, hi_re_at = 0, lo_im_at = 0, hi_im_at = 0;
+  for (uint32_t i = 1; i < n; ++i) {
+    double re = creal(msg[i]), im = cimag(msg[i]);
+    if (re > hi_re) hi_re = re, hi_re_at = i;
+    else if (re < lo_re) lo_re = re, lo_re_at = i;
+    if (im > hi_im) hi_im = im, hi_im_at = i;
+    else if (im < lo_im) lo_im = im, lo_im_at = i;
+  }
+  fprintf(fp, "msg_range[%d]: real(%.17f[%d] ~ %.17f[%d]), imag(%.17f[%d] ~ %.17f[%d])\n", n, lo_re, lo_re_at, hi_re,
+          hi_re_at, lo_im, lo_im_at, hi_im, hi_im_at);
+}
+static uint32_t slots_of(CIPHER c) { return c->_slots ? c->_slots : G.N / 2; }
+void Print_cipher_info(FILE* fp, const char* name, CIPHER c) {
+  fprintf(fp, "\n[%s] ciph_info: %d %d %ld %ld\n", name, c->_sf_degree, c->_slots, (long)c->_c0_poly._num_primes,
+          (long)c->_c0_poly._num_primes_p);
+}
+static void print_msg(FILE* fp, const char* name, CIPHER c, uint32_t len, uint32_t b_len, bool imag) {
+  DCMPLX*  m = Get_msg_with_imag(c);
+  uint32_t n = slots_of(c);
+  Print_cipher_info(fp, name, c);
+  fprintf(fp, b_len ? "[%s] msg: [ \n" : "[%s] msg: [ ", name);
+  for (uint32_t i = 0; i < len && i < n; ++i) {
+    if (b_len && i % b_len == 0) fprintf(fp, "\n");
+    if (imag) fprintf(fp, "(%.17f, %.17fI) ", creal(m[i]), cimag(m[i]));
+    else fprintf(fp, "%.17f ", creal(m[i]));
+  }
+  fprintf(fp, "] ");
+  print_msg_range(fp, m, n);
   free(m);
+}
+void Print_cipher_msg(FILE* fp, const char* name, CIPHER c, uint32_t len) { print_msg(fp, name, c, len, 0, false); }
+void Print_cipher_msg_by_block_len(FILE* fp, const char* name, CIPHER c, uint32_t len, uint32_t b_len) {
+  FMT_ASSERT(b_len, "block length must not be zero");
+  print_msg(fp, name, c, len, b_len, false);
+}
+void Print_cipher_msg_with_imag(FILE* fp, const char* name, CIPHER c, uint32_t len) { print_msg(fp, name, c, len, 0, true); }
+void Print_cipher_range(FILE* fp, const char* name, CIPHER c) {
+  DCMPLX* m = Get_msg_with_imag(c);
+  fprintf(fp, "[%s] ", name);
+  print_msg_range(fp, m, slots_of(c));
+  free(m);
+}
+void Print_cipher_poly(FILE* fp, const char* name, CIPHER c) {
+  Print_cipher_info(fp, name, c);
+  fprintf(fp, "@c0:\n");
+  Print_poly_lite(fp, &c->_c0_poly);
+  fprintf(fp, "@c1:\n");
+  Print_poly_lite(fp, &c->_c1_poly);
+}
+void Dump_cipher_msg(const char* name, CIPHER c, uint32_t len) { Print_cipher_msg(stderr, name, c, len); }
+
+/* Within_value_range (cipher.c:172-186, encoder.c:48-101): would `msg`, encoded at the ciphertext's scale and
+ * level, stay below half the level's modulus?  The inverse embedding runs on the device. */
+bool Within_value_range(CIPHER c, double* msg, uint32_t len) {
+  uint32_t n = slots_of(c);
+  FMT_ASSERT(len <= n, "length of msg should less than slots");
+  CKKS_PARAMS* prm = Get_context_params();
+  double*      in  = (double*)calloc(2 * (size_t)n, sizeof(double));
+  double*      out = (double*)calloc(2 * (size_t)n, sizeof(double));
+  for (uint32_t i = 0; i < len; ++i) in[2 * i] = msg[i];
+  ACE_OK(ace_embedding_inv(G.ctx, out, in, n));
+  double biggest = 0; /* Transform_msg_within_range, encoder.c:217-231 */
+  for (size_t i = 0; i < 2 * (size_t)n; ++i) {
+    double up = fabs(out[i] * c->_scaling_factor);
+    if (up > biggest) biggest = up;
+  }
+  free(in);
+  free(out);
+  int32_t bits  = (int32_t)(log2(fmax(biggest, __DBL_MIN__))) + 1;
+  int32_t valid = (int32_t)prm->_first_mod_size + (int32_t)(Level(c) - 1) * (int32_t)prm->_scaling_mod_size;
+  return bits < valid;
+}
+
+/* Real_relu (cipher.c:340-366): the exact ReLU through the secret key, for validating the approximated one */
+CIPHER Real_relu(CIPHER c) {
+  uint32_t n = slots_of(c);
+  DCMPLX*  m = Get_msg_with_imag(c);
+  for (uint32_t i = 0; i < n; ++i)
+    if (creal(m[i]) <= 0) m[i] *= 0.0;
+  PLAINTEXT pt;
+  memset(&pt, 0, sizeof(pt));
+  init_plain(&pt, Level(c), pow(G.sc, c->_sf_degree), c->_sf_degree, n);
+  ACE_OK(ace_encode(G.ctx, pt._poly._data, (const double*)m, n, n, Level(c), c->_sf_degree, 0));
+  CIPHER res = (CIPHER)calloc(1, sizeof(CIPHERTEXT));
+  Encrypt(res, &pt);
+  Free_plain_poly(&pt);
+  free(m);
+  return res;
 }
 void Validate_impl(double* res, double* msg, uint32_t len, int32_t epsilon) {
   double error = pow(10, epsilon);
@@ -656,7 +780,7 @@ static DATA_SCHEME* find_scheme(const char* name, bool input) {
   Rt_fatal(__FILE__, __LINE__, "not find the %s \"%s\"", input ? "input" : "output", name);
 }
 
-void Prepare_input(TENSOR* input, const char* name) {
+static void prepare_input(TENSOR* input, const char* name, bool dup) {
   NEED_CTX();
   DATA_SCHEME* sch = find_scheme(name, true);
   FMT_ASSERT(sch->_count > 0, "no desc found in scheme");
@@ -667,9 +791,15 @@ void Prepare_input(TENSOR* input, const char* name) {
     size_t          len;
     double*         v;
     if (d->_count == 0) { /* the whole tensor in one ciphertext */
-      len = total;
-      v   = (double*)calloc(2 * len, sizeof(double));
-      for (size_t k = 0; k < len; ++k) v[2 * k] = input->_vals[k];
+      len = dup ? G.N / 2 : total;
+      FMT_ASSERT(total <= len, "tensor larger than the slot count");
+      v = (double*)calloc(2 * len, sizeof(double));
+      for (size_t k = 0; k < total; ++k) v[2 * k] = input->_vals[k];
+      if (dup) { /* Pre_encode_scheme_dup (rtlib.c:19-33): repeated with the period of the next power of two */
+        size_t period = 1;
+        while (period < total) period <<= 1;
+        for (size_t k = period; k < len; ++k) v[2 * k] = v[2 * (k % period)];
+      }
     } else { /* a chunk with optional padding from its neighbours (Pre_encode_scheme) */
       FMT_ASSERT(d->_kind == NORMAL && d->_stride == 1, "TODO: other kind / stride");
       FMT_ASSERT((size_t)d->_count < total && (size_t)(d->_start + d->_count) <= total, "chunk out of image bound");
@@ -692,6 +822,9 @@ void Prepare_input(TENSOR* input, const char* name) {
     free(v);
   }
 }
+
+void Prepare_input(TENSOR* input, const char* name) { prepare_input(input, name, false); }
+void Prepare_input_dup(TENSOR* input, const char* name) { prepare_input(input, name, true); }
 
 double* Handle_output(const char* name) {
   NEED_CTX();

@@ -4,7 +4,10 @@
  * at offset 0, entries from offset 4096 on, each padded to 2^_ent_align bytes, and a lookup table of
  * 32-byte records at _lut_ofst.  Message files (float or double entries) are read whole at Prepare_context,
  * as Pt_mgr_init does (rtlib/ant/porting/pt_mgr.c:35-99); Pt_from_msg encodes `len` values of entry `index`
- * (pt_mgr.c:188-243).  Files of pre-encoded plaintexts hold host-side polynomial images and are refused.
+ * (pt_mgr.c:188-243).  A file of pre-encoded plaintexts (DE_PLAINTEXT) holds, per entry, a PLAINTEXT_BUFFER
+ * (fhe-cmplr/include/fhe/core/rt_encode_api.h:20-27): magic, version, size, then the host image of a PLAINTEXT
+ * with a null `_data` followed by its words; such files can be far larger than host memory, so their entries
+ * are read one at a time, on demand, and uploaded (Pt_get, pt_mgr.c:117-177).
  *
  * RT_HIP_DATA_FILE names the file when the path compiled into the program does not exist here.
  * RT_HIP_SYNTHETIC_WEIGHTS=<amplitude> replaces a missing file by reproducible pseudo-random values in
@@ -43,6 +46,8 @@ static struct {
   LUT_ENTRY* lut;
   char*      buf; /* the bytes between the first page and the lookup table */
   uint64_t   size;
+  FILE*       file; /* a file of pre-encoded plaintexts stays open */
+  PLAINTEXT** pt;   /* [ent_count]: the entries uploaded so far */
 } Data;
 
 /* Encoded weight plaintexts kept in HBM.  A program encodes the same entries for every input it is run on (the
@@ -118,14 +123,20 @@ bool Pt_mgr_init(const char* fname) {
   }
   FMT_ASSERT(fread(&Data.hdr, sizeof(DATA_HDR), 1, f) == 1, "failed to read rt data file header");
   FMT_ASSERT(memcmp(Data.hdr.magic, "!ANTFHE\0", 8) == 0, "%s is not an rt data file", fname);
-  FMT_ASSERT(Data.hdr.ent_type == DE_MSG_F32 || Data.hdr.ent_type == DE_MSG_F64,
-             "rt data files of pre-encoded plaintexts are not supported: their polynomials are host images");
+  FMT_ASSERT(Data.hdr.ent_type == DE_MSG_F32 || Data.hdr.ent_type == DE_MSG_F64 || Data.hdr.ent_type == DE_PLAINTEXT,
+             "unknown entry type %u in rt data file", (unsigned)Data.hdr.ent_type);
   FMT_ASSERT(Data.hdr.lut_ofst >= DATA_PAGE, "lookup table inside the first page");
   Data.lut = (LUT_ENTRY*)malloc((Data.hdr.ent_count ? Data.hdr.ent_count : 1) * sizeof(LUT_ENTRY));
   FMT_ASSERT(fseek(f, (long)Data.hdr.lut_ofst, SEEK_SET) == 0 &&
                  fread(Data.lut, sizeof(LUT_ENTRY), Data.hdr.ent_count, f) == Data.hdr.ent_count,
              "failed to read rt data file lookup table");
   Data.size = Data.hdr.lut_ofst - DATA_PAGE;
+  if (Data.hdr.ent_type == DE_PLAINTEXT) {
+    Data.file = f;
+    Data.pt   = (PLAINTEXT**)calloc(Data.hdr.ent_count ? Data.hdr.ent_count : 1, sizeof(PLAINTEXT*));
+    Data.open = true;
+    return true;
+  }
   Data.buf  = (char*)malloc(Data.size ? Data.size : 1);
   FMT_ASSERT(fseek(f, DATA_PAGE, SEEK_SET) == 0 && fread(Data.buf, 1, Data.size, f) == Data.size,
              "failed to fill data from file");
@@ -136,6 +147,11 @@ bool Pt_mgr_init(const char* fname) {
 
 void Pt_mgr_fini(void) {
   cache_clear();
+  if (Data.pt)
+    for (uint64_t i = 0; i < Data.hdr.ent_count; ++i)
+      if (Data.pt[i]) Pt_free((uint32_t)i);
+  free(Data.pt);
+  if (Data.file) fclose(Data.file);
   for (size_t i = 0; i < Data.syn_count; ++i) free(Data.syn[i]);
   free(Data.syn);
   free(Data.syn_len);
@@ -263,9 +279,59 @@ void Pt_from_msg_ofst_validate(void* pt, float* buf, uint32_t index, size_t ofst
 void Pt_from_msg_validate(void* pt, float* buf, uint32_t index, size_t len, uint32_t scale, uint32_t level) {
   Pt_from_msg_ofst_validate(pt, buf, index, 0, len, scale, level);
 }
-void* Pt_get(uint32_t index, size_t len, uint32_t scale, uint32_t level) {
-  (void)len, (void)scale, (void)level;
-  Rt_fatal(__FILE__, __LINE__, "Pt_get(%u): pre-encoded plaintext files are not supported; ship messages (f32 / f64)", index);
+/* ---- files of pre-encoded plaintexts ------------------------------------------------------------------- */
+static bool plaintext_file(void) { return Data.open && !Data.synthetic && Data.hdr.ent_type == DE_PLAINTEXT; }
+static PLAINTEXT* load_plain_entry(uint32_t index) {
+  FMT_ASSERT(plaintext_file(), "Pt_get: the program's rt data file does not hold pre-encoded plaintexts");
+  FMT_ASSERT(index < Data.hdr.ent_count, "index out of entry range");
+  if (Data.pt[index]) return Data.pt[index];
+  const LUT_ENTRY* e = &Data.lut[index];
+  FMT_ASSERT(e->ofst >= DATA_PAGE && e->ofst + e->size <= Data.hdr.lut_ofst, "entry offset too large");
+  FMT_ASSERT(e->size >= 16 + sizeof(PLAINTEXT), "Plaintext buffer too small");
+  char* raw = (char*)malloc(e->size);
+  FMT_ASSERT(fseek(Data.file, (long)e->ofst, SEEK_SET) == 0 && fread(raw, 1, e->size, Data.file) == e->size,
+             "failed to fill data from file");
+  uint32_t version, size; /* Cast_buffer_to_plain (ckks/src/plain.c:262-292) */
+  memcpy(&version, raw + 8, 4);
+  memcpy(&size, raw + 12, 4);
+  FMT_ASSERT(memcmp(raw, "ANTPLAIN", 8) == 0, "Plaintext buffer magic mismatch");
+  FMT_ASSERT(version == RT_DATA_VERSION, "Plaintext buffer version mismatch");
+  FMT_ASSERT((uint64_t)size + 16 <= e->size, "Plaintext buffer too small");
+  PLAINTEXT* pt = (PLAINTEXT*)malloc(sizeof(PLAINTEXT));
+  memcpy(pt, raw + 16, sizeof(PLAINTEXT));
+  POLY poly = &pt->_poly;
+  FMT_ASSERT(poly->_data == NULL, "Plaintext poly data is not NULL");
+  size_t words = poly->_num_alloc_primes * (size_t)poly->_ring_degree;
+  FMT_ASSERT(size == words * sizeof(int64_t) + sizeof(PLAINTEXT), "Plaintext size mismatch");
+  FMT_ASSERT(poly->_ring_degree == Degree() && poly->_num_primes >= 1 && poly->_num_primes <= Get_q_cnt() &&
+                 (poly->_num_primes_p == 0 || poly->_num_primes_p == Get_p_cnt()) &&
+                 poly->_num_alloc_primes >= poly->_num_primes + poly->_num_primes_p,
+             "plaintext %u does not fit this context (degree %u, %zu + %zu primes)", index, poly->_ring_degree,
+             poly->_num_primes, poly->_num_primes_p);
+  poly->_data = Rt_dev_alloc_raw(words);
+  ACE_OK(ace_upload(G.ctx, poly->_data, (const int64_t*)(raw + 16 + sizeof(PLAINTEXT)), words)); /* waits for the copy */
+  free(raw);
+  return Data.pt[index] = pt;
 }
-/* Free_data (pt_mgr.c:181-185): the polynomial of a plaintext made by Pt_from_msg */
-void Free_data(void* poly) { Free_poly_data((POLY)poly); }
+void* Pt_get(uint32_t index, size_t len, uint32_t scale, uint32_t level) {
+  (void)len, (void)scale, (void)level; /* the entry carries its own shape, as in the reference */
+  return load_plain_entry(index);
+}
+void Pt_prefetch(uint32_t index) {
+  if (plaintext_file() && index < Data.hdr.ent_count) (void)load_plain_entry(index);
+}
+void Pt_free(uint32_t index) {
+  FMT_ASSERT(plaintext_file() && index < Data.hdr.ent_count && Data.pt[index], "BLOCK_INFO state is not ready");
+  Free_poly_data(&Data.pt[index]->_poly);
+  free(Data.pt[index]);
+  Data.pt[index] = NULL;
+}
+void* Pt_get_validate(float* buf, uint32_t index, size_t len, uint32_t scale, uint32_t level) {
+  (void)buf, (void)len, (void)scale, (void)level;
+  Rt_fatal(__FILE__, __LINE__, "Pt_get_validate(%u): TODO: not implemented", index); /* pt_mgr.c:161-164 */
+}
+/* Free_data (pt_mgr.c:179-183): the polynomial of a plaintext made by Pt_from_msg; a plaintext of Pt_get
+ * belongs to the manager and is left alone */
+void Free_data(void* poly) {
+  if (!plaintext_file()) Free_poly_data((POLY)poly);
+}

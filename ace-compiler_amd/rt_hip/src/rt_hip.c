@@ -580,7 +580,7 @@ uint32_t Get_slots(CIPHER c) { return c->_slots; }
 void     Set_slots(CIPHER c, uint32_t slots) { c->_slots = slots; }
 
 /* shape res like `like` with the given scale; polynomials end up in NTT form at like's level */
-static void shape_ciph(CIPHER res, CIPHER like, double sf, uint32_t deg) {
+void Rt_shape_ciph(CIPHER res, CIPHER like, double sf, uint32_t deg) {
   res->_scaling_factor = sf;
   res->_sf_degree      = deg;
   res->_slots          = like->_slots;
@@ -613,21 +613,21 @@ void Init_ciph_same_scale(CIPHER res, CIPHER a, CIPHER b) {
   CIPHER pick = b ? lower_of(a, b) : a;
   if (pick == b && !a->_c0_poly._data) {
     /* accumulator idiom: an empty first operand becomes a zero ciphertext shaped like the second */
-    shape_ciph(a, b, b->_scaling_factor, b->_sf_degree);
+    Rt_shape_ciph(a, b, b->_scaling_factor, b->_sf_degree);
     a->_c0_poly._is_ntt = b->_c0_poly._is_ntt;
     a->_c1_poly._is_ntt = b->_c1_poly._is_ntt;
   } else if (!pick->_c0_poly._data) {
     memset(res, 0, sizeof(*res));
     return;
   }
-  shape_ciph(res, pick, pick->_scaling_factor, pick->_sf_degree);
+  Rt_shape_ciph(res, pick, pick->_scaling_factor, pick->_sf_degree);
 }
 void Init_ciph_up_scale(CIPHER res, CIPHER a, CIPHER b) {
-  shape_ciph(res, lower_of(a, b), a->_scaling_factor * b->_scaling_factor, a->_sf_degree + b->_sf_degree);
+  Rt_shape_ciph(res, lower_of(a, b), a->_scaling_factor * b->_scaling_factor, a->_sf_degree + b->_sf_degree);
 }
 void Init_ciph_down_scale(CIPHER res, CIPHER c) {
   FMT_ASSERT(c->_sf_degree >= 2, "Scale degree of result dec to zero");
-  shape_ciph(res, c, c->_scaling_factor / G.sc, c->_sf_degree - 1);
+  Rt_shape_ciph(res, c, c->_scaling_factor / G.sc, c->_sf_degree - 1);
 }
 void Init_ciph_same_scale_ciph3(CIPHER res, CIPHER3 c) {
   FMT_ASSERT(res, "invalid ciphertext");
@@ -679,7 +679,7 @@ static CIPHER ciph_ew(poly2_fn fn, CIPHER res, CIPHER a, CIPHER b) {
   FMT_ASSERT(a->_scaling_factor == b->_scaling_factor, "Scaling factors are not equal.");
   size_t la = Level(a), lb = Level(b), l = la < lb ? la : lb;
   CIPHER low = la <= lb ? a : b;
-  if (res != a && res != b) shape_ciph(res, low, low->_scaling_factor, low->_sf_degree);
+  if (res != a && res != b) Rt_shape_ciph(res, low, low->_scaling_factor, low->_sf_degree);
   /* the higher operand is viewed at the common level for the duration of the call */
   CIPHERTEXT va = *a, vb = *b;
   va._c0_poly._num_primes = va._c1_poly._num_primes = l;
@@ -726,17 +726,10 @@ CIPHER Rescale_ciph(CIPHER res, CIPHER c) {
   FMT_ASSERT(level > 1, "rescale: multiply level is not big enought for more operation");
   double   sf  = c->_scaling_factor / G.sc;
   uint32_t deg = c->_sf_degree - 1;
-  shape_ciph(res, c, sf, deg);
+  Rt_shape_ciph(res, c, sf, deg);
   ACE_OK(ace_rescale_ciph(G.ctx, res->_c0_poly._data, res->_c1_poly._data, c->_c0_poly._data, c->_c1_poly._data, level));
   Set_poly_level(&res->_c0_poly, level - 1);
   Set_poly_level(&res->_c1_poly, level - 1);
-  return res;
-}
-
-CIPHER Modswitch_ciph(CIPHER res, CIPHER c) {
-  if (res != c) shape_ciph(res, c, c->_scaling_factor, c->_sf_degree);
-  Modswitch(&res->_c0_poly, &c->_c0_poly);
-  Modswitch(&res->_c1_poly, &c->_c1_poly);
   return res;
 }
 
@@ -764,7 +757,7 @@ void Rotate_batch_ciph(CIPHER res_arr, CIPHER c, const int32_t* rot_idx, uint32_
     ACE_OK(ace_rotate_batch(G.ctx, s0, s1, c->_c0_poly._data, c->_c1_poly._data, keys, orders, m, level));
     for (uint32_t j = 0; j < m; ++j) {
       CIPHER out = &res_arr[where[j]];
-      shape_ciph(out, c, c->_scaling_factor, c->_sf_degree);
+      Rt_shape_ciph(out, c, c->_scaling_factor, c->_sf_degree);
       Rt_dev_copy(out->_c0_poly._data, s0 + j * level * n, level * n);
       Rt_dev_copy(out->_c1_poly._data, s1 + j * level * n, level * n);
     }

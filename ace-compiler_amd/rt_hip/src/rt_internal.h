@@ -61,6 +61,9 @@ void     Rt_install_key(SWITCH_KEY* k, const int64_t* host);
 void     Rt_install_key_dev(SWITCH_KEY* k, int64_t* dev); /* takes ownership of the buffer */
 ROT_KEY* Rt_rot_entry(int32_t rot_idx);
 ROT_KEY* Rt_find_rot(int32_t rot_idx);
+void     Rt_shape_ciph(CIPHER res, CIPHER like, double sf, uint32_t deg); /* res shaped like `like`, NTT form */
+void     Rt_sample_ternary(int64_t* v, size_t n, size_t hamming_weight);  /* the key generator's host stream */
+#define RT_DATA_VERSION 1u /* RT_VERSION_FULL (fhe-cmplr/include/fhe/core/rt_version.h:15-22): 0.0.0 build 1 */
 void     Rt_ckks_finalize(void);
 void     Rt_bootstrap_finalize(void);
 void     Rt_bootstrap_prepare(void);

@@ -225,6 +225,10 @@ int ace_encode(ace_ctx* ctx, int64_t* res, const double* values, size_t n_values
  * (is_f32 = 1), widened to complex numbers with zero imaginary part on the device. */
 int ace_encode_real(ace_ctx* ctx, int64_t* res, const void* values, int is_f32, size_t n_values, uint32_t slots,
                     size_t level, uint32_t sf_degree, size_t p_cnt);
+/* Encode_at_level_with_scale (ckks/src/encoder.c:337-420): complex values at an explicit scale (any positive
+ * double below the level's modulus): one multiplication by `scale`, rounded to nearest. */
+int ace_encode_scaled(ace_ctx* ctx, int64_t* res, const double* values, size_t n_values, uint32_t slots, size_t level,
+                      double scale, size_t p_cnt);
 /* Extend (:483-500): src level limbs -> res level+num_p limbs (P limbs zero) */
 int ace_extend(ace_ctx* ctx, int64_t* res, const int64_t* src, size_t level);
 /* Dot_prod / Fast_dot_prod (:502-529): digits = n_parts x (level+num_p) limbs;

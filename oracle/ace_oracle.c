@@ -1252,8 +1252,22 @@ static i64 mod_int64(i64 v, i64 m) { i64 r = v % m; return r < 0 ? r + m : r; } 
 /* Encode_impl (encoder.c:234-326), 64-bit build.  values: n_values complex numbers
  * (re, im interleaved); out: level Q limbs followed by p_cnt P limbs, NTT form.
  * Returns 1, or 0 where the reference asserts (vector out of range / overflow). */
+static int encode_either(const orc_ctx* c, int64_t* out, const double* values, size_t n_values, uint32_t slots,
+                         size_t level, uint32_t sf_degree, size_t p_cnt, double explicit_scale);
 int orc_encode(const orc_ctx* c, int64_t* out, const double* values, size_t n_values, uint32_t slots, size_t level,
                uint32_t sf_degree, size_t p_cnt) {
+  return encode_either(c, out, values, n_values, slots, level, sf_degree, p_cnt, 0.0);
+}
+/* Encode_impl_with_scale (encoder.c:337-403): the same steps with one multiplication by `scale`, rounded by
+ * llround without the half that Encode_impl adds first, no range assertion on the rounded value and no
+ * further powers of the scaling factor */
+int orc_encode_scaled(const orc_ctx* c, int64_t* out, const double* values, size_t n_values, uint32_t slots,
+                      size_t level, double scale, size_t p_cnt) {
+  ORC_ASSERT(scale > 0, "invalid scale for encode");
+  return encode_either(c, out, values, n_values, slots, level, 1, p_cnt, scale);
+}
+static int encode_either(const orc_ctx* c, int64_t* out, const double* values, size_t n_values, uint32_t slots,
+                         size_t level, uint32_t sf_degree, size_t p_cnt, double explicit_scale) {
   ORC_ASSERT(c->sf_bits, "context has no scaling factor");
   size_t N = c->N;
   double scaling_factor = (double)((u64)1 << c->sf_bits); /* param.c:68 */
@@ -1262,8 +1276,13 @@ int orc_encode(const orc_ctx* c, int64_t* out, const double* values, size_t n_va
   ORC_ASSERT(level <= c->L && n_values <= slots && slots <= N / 2, "encode: bad sizes");
   uint32_t sf_bits = (uint32_t)log2(scaling_factor);
   size_t coeff_bits = c->q0_bits + (level - 1) * c->sf_bits; /* Get_coeff_bit_count */
-  ORC_ASSERT(sf_degree >= 1 && (size_t)sf_bits * sf_degree < coeff_bits, "invalid scaling factor for encode");
   double scale = pow(scaling_factor, sf_degree);
+  if (explicit_scale > 0) {
+    ORC_ASSERT((uint32_t)log2(explicit_scale) < coeff_bits, "invalid scale for encode");
+    scale = explicit_scale;
+  } else {
+    ORC_ASSERT(sf_degree >= 1 && (size_t)sf_bits * sf_degree < coeff_bits, "invalid scaling factor for encode");
+  }
   /* Transform_msg_within_range (encoder.c:198-231) */
   dcmplx* in = (dcmplx*)calloc(slots, sizeof(dcmplx));
   dcmplx* ts = (dcmplx*)calloc(slots, sizeof(dcmplx));
@@ -1281,7 +1300,9 @@ int orc_encode(const orc_ctx* c, int64_t* out, const double* values, size_t n_va
   i64* message = (i64*)calloc(N, sizeof(i64));
   uint32_t gap = (uint32_t)(N / (slots * 2));
   for (uint32_t i = 0; ok && i < slots; i++) {
-    double re = creal(ts[i]) * scaling_factor + 0.5, im = cimag(ts[i]) * scaling_factor + 0.5;
+    double re, im;
+    if (explicit_scale > 0) re = creal(ts[i]) * scale, im = cimag(ts[i]) * scale;
+    else re = creal(ts[i]) * scaling_factor + 0.5, im = cimag(ts[i]) * scaling_factor + 0.5;
     if (!(re <= (double)INT64_MAX && re >= -(double)INT64_MAX && im <= (double)INT64_MAX && im >= -(double)INT64_MAX)) {
       ok = 0;
       break;
@@ -1301,7 +1322,7 @@ int orc_encode(const orc_ctx* c, int64_t* out, const double* values, size_t n_va
         out[t * N + n] = v > big_half ? mod_int64(v - diff, q) : mod_int64(v, q);
       }
     }
-    if (sf_degree > 1) { /* encoder.c:297-312: only the Q limbs */
+    if (sf_degree > 1 && !(explicit_scale > 0)) { /* encoder.c:297-312: only the Q limbs */
       for (size_t t = 0; t < level; t++) {
         i64 q = c->mod[t].val, powp = (i64)scaling_factor;
         for (uint32_t d = 2; d < sf_degree; d++) powp = mul_mod_exact(powp, (i64)scaling_factor, q);

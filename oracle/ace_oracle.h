@@ -169,6 +169,9 @@ void orc_embedding(const orc_ctx* c, double* res, const double* coeffs, size_t l
 /* Encode_impl (encoder.c:234-326): 1 on success, 0 where the reference asserts on range */
 int orc_encode(const orc_ctx* c, int64_t* out, const double* values, size_t n_values, uint32_t slots, size_t level,
                uint32_t sf_degree, size_t p_cnt);
+/* Encode_impl_with_scale (encoder.c:337-403) */
+int orc_encode_scaled(const orc_ctx* c, int64_t* out, const double* values, size_t n_values, uint32_t slots,
+                      size_t level, double scale, size_t p_cnt);
 /* Decode (encoder.c:657-704) */
 void orc_decode(const orc_ctx* c, double* res, const int64_t* poly, size_t level, uint32_t slots, double factor,
                 int is_ntt);

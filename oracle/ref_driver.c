@@ -41,7 +41,7 @@ enum {
   OP_NTT = 1, OP_INTT, OP_HW, OP_DECOMP_MODUP, OP_PRECOMP, OP_MOD_DOWN,
   OP_RESCALE, OP_DOT_PROD, OP_AUTO_ORDER, OP_AUTO_INDEX, OP_AUTOMORPHISM,
   OP_EXTEND, OP_TBL_MODUP, OP_TBL_MODDOWN, OP_TBL_RESCALE, OP_POLY, OP_TWIDDLES,
-  OP_MOD_UP, OP_MOD_DOWN_RESCALE, OP_REDUCE_RESCALE_MODUP, OP_FROM_LEVEL0, OP_ENCODE, OP_DECODE, OP_EMBEDDING, OP_TIME_NTT
+  OP_MOD_UP, OP_MOD_DOWN_RESCALE, OP_REDUCE_RESCALE_MODUP, OP_FROM_LEVEL0, OP_ENCODE, OP_DECODE, OP_EMBEDDING, OP_TIME_NTT, OP_ENCODE_SCALED
 };
 
 static int64_t* in_buf;
@@ -274,6 +274,28 @@ int main(int argc, char** argv) {
         memset(&pt, 0, sizeof(pt));
         if (pc) Encode_ext_at_level(&pt, enc, vals, (uint32_t)lv, (uint32_t)a2, (uint32_t)pc);
         else Encode_at_level_with_sf(&pt, enc, vals, (uint32_t)lv, (uint32_t)a2, (uint32_t)a3);
+        POLYNOMIAL* poly = Get_plain_poly(&pt);
+        size_t n = (Poly_level(poly) + Num_p(poly)) * N;
+        wr1((int64_t)(n + 3));
+        wr(Get_poly_coeffs(poly), Poly_level(poly) * N);
+        if (Num_p(poly)) wr(Get_p_coeffs(poly), Num_p(poly) * N);
+        wr1((int64_t)pt._slots);
+        wr1((int64_t)pt._sf_degree);
+        { double sf = pt._scaling_factor; int64_t bits; memcpy(&bits, &sf, 8); wr1(bits); }
+        Free_poly_data(poly);
+        Free_value_list(vals);
+        break;
+      }
+      case OP_ENCODE_SCALED: { /* a1 level, a2 slots, a3 raw bits of the scale, a4 p_cnt; in = complex doubles */
+        size_t lv = (size_t)a1, nv = n_in / 2;
+        double scale;
+        memcpy(&scale, &a3, 8);
+        CKKS_ENCODER* enc = (CKKS_ENCODER*)Context->_encoder;
+        VALUE_LIST* vals = Alloc_value_list(DCMPLX_TYPE, nv);
+        memcpy(DCMPLX_VALUES(vals), in, nv * sizeof(DCMPLX));
+        PLAINTEXT pt;
+        memset(&pt, 0, sizeof(pt));
+        Encode_at_level_with_scale(&pt, enc, vals, (uint32_t)lv, (uint32_t)a2, scale, (uint32_t)a4);
         POLYNOMIAL* poly = Get_plain_poly(&pt);
         size_t n = (Poly_level(poly) + Num_p(poly)) * N;
         wr1((int64_t)(n + 3));

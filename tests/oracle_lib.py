@@ -255,6 +255,16 @@ class Oracle:
                                 C.c_size_t(level), C.c_uint32(sf_degree), C.c_size_t(p_cnt))
         return out if ok else None
 
+    def encode_scaled(self, values, slots, level, scale, p_cnt=0):
+        """Encode_at_level_with_scale: the plaintext polynomial at an explicit scale, or None on a range failure."""
+        v = np.ascontiguousarray(values, dtype=np.complex128)
+        lv = level or self.L
+        out = np.zeros((lv + p_cnt) * self.N, np.int64)
+        self.L_.orc_encode_scaled.restype = C.c_int
+        ok = self.L_.orc_encode_scaled(self.h, _ptr(out), v.ctypes.data_as(C.c_void_p), C.c_size_t(v.size),
+                                       C.c_uint32(slots), C.c_size_t(level), C.c_double(scale), C.c_size_t(p_cnt))
+        return out if ok else None
+
     def decode(self, poly, level, slots, factor, is_ntt=True):
         poly = np.ascontiguousarray(poly, dtype=np.int64)
         out = np.zeros(slots, np.complex128)

@@ -457,6 +457,11 @@ def test_encode(pair):
             dr = g.alloc((level + pc) * N)
             g.encode(dr, vals, slots, level, deg, pc)
             eq(dr, want, "encode slots=%d level=%d sf_degree=%d p=%d" % (slots, level, deg, pc))
+            if deg == 1:  # an explicit scale that is no power of the scaling factor (Encode_at_level_with_scale)
+                scale = 1.5 * 2.0 ** sf_bits if level > 1 else 2.0 ** (sf_bits - 7) * 1.1
+                if np.log2(scale) + 3 < q0_bits + (level - 1) * sf_bits:
+                    g.encode_scaled(dr, vals, slots, level, scale, pc)
+                    eq(dr, o.encode_scaled(vals, slots, level, scale, pc), "encode_scaled slots=%d level=%d p=%d" % (slots, level, pc))
     # real-valued messages (doubles, floats) are widened on the device: same residues as the complex form, with
     # calls recorded and issued one by one
     for side in (True, False):

@@ -251,3 +251,22 @@ def test_plaintexts_from_a_weight_file(dtype, tmp_path):
     if dtype == "f32":  # an index past the table is refused the way the reference refuses it
         bad = run(args[:9] + ["9", "0", "4"], 0)
         assert bad.returncode != 0 and "index out of entry range" in bad.stderr
+
+
+SURFACE = os.path.join(rt_program.ROOT, "tests", "programs", "surface_program")
+
+
+@pytest.mark.parametrize("args", [
+    "4096 5 60 50 11",
+    "65536 4 60 50 12",
+    "1024 20 60 51 13 bootstrap",
+], ids=["N4096", "N65536", "N1024_staged_bootstrap"])
+def test_less_used_entry_points(args):
+    """One-limb polynomials, per-limb scalars, Alloc_precomp's list, Automorphism_transform, Upscale / Downscale /
+    Raise_mod, Reset_ciph, Encode_float_with_scale, Prepare_input_dup, a file of pre-encoded plaintexts read by
+    Pt_get, and the three staged bootstrap operators: each against the entry points the committed programs use
+    (bit for bit) or the message it must decrypt to."""
+    assert os.path.exists(SURFACE), "tests/programs/surface_program is not built"
+    print("running surface_program", args, flush=True)
+    r = subprocess.run([SURFACE] + args.split(), capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0 and "surface ok" in r.stdout, r.stdout + r.stderr

@@ -46,6 +46,17 @@ def test_embedding_encode_decode(cfg):
                     dec = o.decode(poly, level, slots, sc, bool(is_ntt))
                     want.append(bits(dec))
                     assert np.abs(dec[:n_val] - zz).max() < 1e-6
+        # an explicit scale that is no power of the scaling factor (Encode_at_level_with_scale), with and without P limbs
+        for level, scale, pc in ((o.L, 1.5 * 2.0 ** cfg[3], 0), (2, 2.0 ** (cfg[3] - 7) * 1.1, 0), (o.L, 1.25 * 2.0 ** (cfg[3] + 5), o.K)):
+            if np.log2(scale) + 3 >= cfg[2] + (level - 1) * cfg[3]:
+                continue
+            zz = z[:max(1, slots - 1)] * 3.0
+            s.add(refdrv.OP_ENCODE_SCALED, level, slots, int(bits(np.array([scale]))[0]), pc, bits(zz))
+            pt = o.encode_scaled(zz, slots, level, scale, pc)
+            assert pt is not None
+            deg = int(np.floor(np.log2(scale) / cfg[3]))
+            deg += scale > float(2 ** cfg[3]) ** deg
+            want.append(np.concatenate([pt, [slots, deg], bits(np.array([scale]))]))
     # decode of arbitrary residues: large centred values, both signs
     for level in (o.L, 3, 1):
         poly = seeded.uniform_poly(90 + level, o.primes[:level], N)

@@ -1,0 +1,119 @@
+"""The program-facing surface of the runtime against the reference's headers: every function the reference
+declares for programs (poly, HAL, lpoly, cipher, plain, key, rt_api, pt_mgr, tensor, rt_stat) must be exported by
+librt_hip.so or defined inline by rt_hip.h, with the same number of parameters; what is left out is listed
+here with its reason.  Runs where the reference tree is present (it is read as text only)."""
+import os
+import re
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+RT = "/root/reference/fhe-cmplr/rtlib"
+HEADERS = [
+    "ant/include/poly/rns_poly.h",
+    "ant/include/hal/hal.h",
+    "ant/include/lpoly/poly.h",
+    "ant/include/ckks/cipher.h",
+    "ant/include/ckks/plain.h",
+    "ant/include/ckks/key.h",
+    "include/common/rt_api.h",
+    "include/common/pt_mgr.h",
+    "include/common/tensor.h",
+    "include/common/rt_stat.h",
+]
+# name -> why it is not provided
+LEFT_OUT = {
+    # the program provides these (weak declarations in both headers)
+    "Get_context_params": "defined by the compiled program",
+    "Get_extra_context_params": "defined by the compiled program (optional auxiliary module)",
+    "Get_rt_data_info": "defined by the compiled program",
+    "Get_input_count": "defined by the compiled program",
+    "Get_output_count": "defined by the compiled program",
+    "Get_encode_scheme": "defined by the compiled program",
+    "Get_decode_scheme": "defined by the compiled program",
+    "Main_graph": "defined by the compiled program",
+    # big-integer (GMP) list conversions of the reference's setup and decode code; no emitter produces them
+    "Transform_value_to_rns_poly": "takes a VALUE_LIST of GMP integers; host-side setup helper",
+    "Reconstruct_rns_poly_to_value": "returns a VALUE_LIST of GMP integers; host-side decode helper",
+}
+
+
+def _strip(text):
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = re.sub(r"//[^\n]*", "", text)
+    return re.sub(r"#[^\n]*(\\\n[^\n]*)*", "", text)
+
+
+def _prototypes(text):
+    """name -> number of parameters, for every function declared or defined at file scope"""
+    text = _strip(text)
+    out = {}
+    depth = 0
+    i = 0
+    top = []  # characters at brace depth 0 (function bodies blanked out), extern "C" braces kept transparent
+    text = re.sub(r'extern\s+"C"\s*\{', " ", text)
+    while i < len(text):
+        ch = text[i]
+        if ch == "{":
+            depth += 1
+        elif ch == "}":
+            depth = max(0, depth - 1)
+            top.append(";")
+        elif depth == 0:
+            top.append(ch)
+        i += 1
+    flat = "".join(top)
+    for m in re.finditer(r"([A-Za-z_][A-Za-z0-9_\*\s]*?)\b([A-Z][A-Za-z0-9_]*)\s*\(([^()]*(?:\([^()]*\)[^()]*)*)\)\s*(?:__attribute__\s*\(\(.*?\)\))?\s*;", flat):
+        ret, name, args = m.group(1).strip(), m.group(2), m.group(3).strip()
+        if not ret or ret.split()[-1] in ("return", "else", "typedef"):
+            continue
+        n = 0 if args in ("", "void") else args.count(",") + 1
+        out[name] = n
+    return out
+
+
+@pytest.fixture(scope="module")
+def ours():
+    hdr = open(os.path.join(ROOT, "ace-compiler_amd/rt_hip/include/rt_hip.h")).read()
+    protos = _prototypes(hdr)
+    macros = set(re.findall(r"#define\s+([A-Za-z_][A-Za-z0-9_]*)", hdr))
+    lib = os.path.join(ROOT, "ace-compiler_amd/librt_hip.so")
+    exported = set()
+    for line in subprocess.run(["nm", "-D", "--defined-only", lib], capture_output=True, text=True, check=True).stdout.splitlines():
+        exported.add(line.split()[-1])
+    inline = set(re.findall(r"static inline [^;{]*?\b([A-Za-z_][A-Za-z0-9_]*)\s*\(", _strip(hdr)))
+    return protos, macros, exported, inline
+
+
+@pytest.mark.skipif(not os.path.isdir(RT), reason="the reference tree is not present")
+@pytest.mark.parametrize("header", HEADERS)
+def test_every_declared_function_is_provided(header, ours):
+    protos, macros, exported, inline = ours
+    ref = _prototypes(open(os.path.join(RT, header)).read())
+    assert ref, header
+    missing, arity = [], []
+    for name, n in sorted(ref.items()):
+        if name in LEFT_OUT:
+            continue
+        if name not in exported and name not in inline and name not in macros:
+            missing.append(name)
+        elif name in protos and protos[name] != n:
+            arity.append((name, n, protos[name]))
+    assert not missing, f"{header}: not provided: {missing}"
+    assert not arity, f"{header}: parameter counts differ (name, reference, here): {arity}"
+
+
+def test_left_out_list_is_not_stale(ours):
+    _, macros, exported, inline = ours
+    provided = [n for n in LEFT_OUT if n in exported or n in inline or n in macros]
+    assert not provided, f"now provided, drop from the list: {provided}"
+
+
+def test_declared_functions_are_exported(ours):
+    """every non-inline prototype of rt_hip.h resolves in librt_hip.so"""
+    protos, _, exported, inline = ours
+    weak = {"Get_context_params", "Get_rt_data_info", "Get_input_count", "Get_output_count", "Get_encode_scheme",
+            "Get_decode_scheme", "Main_graph"}
+    lost = [n for n in protos if n not in exported and n not in inline and n not in weak]
+    assert not lost, lost
