@@ -208,6 +208,16 @@ void Rt_generate_keys(uint64_t seed) {
   Rt_bootstrap_prepare();
 }
 
+void Rt_get_secret(int64_t* host_small) {
+  FMT_ASSERT(G.secret_small, "Rt_generate_keys() has not run");
+  memcpy(host_small, G.secret_small, G.N * sizeof(int64_t));
+}
+void Rt_get_public_key(int64_t* host_pk0, int64_t* host_pk1) {
+  FMT_ASSERT(G.pk0, "Rt_generate_keys() has not run");
+  ACE_OK(ace_download(G.ctx, host_pk0, G.pk0, G.L * G.N));
+  ACE_OK(ace_download(G.ctx, host_pk1, G.pk1, G.L * G.N));
+}
+
 void Rt_ckks_finalize(void) {
   free(G.secret_small);
   if (G.secret_ntt) Rt_dev_free(G.secret_ntt);

@@ -86,14 +86,17 @@ class CkksHost:
     def neg(self, a, prime_idx):
         return self.limbwise("modsub", np.zeros_like(a), a, prime_idx)
 
-    def switch_key(self, s_res_ntt, s_src_ntt):
-        """Key taking a polynomial multiplying s_src to a pair decrypting under s_res (all L+k limbs, NTT)."""
+    def switch_key(self, s_res_ntt, s_src_ntt, a_given=None, e_given=None):
+        """Key taking a polynomial multiplying s_src to a pair decrypting under s_res (all L+k limbs, NTT).
+        a_given / e_given: per digit, the uniform polynomial (NTT form) and the small error (signed coefficients)
+        to use instead of drawing them."""
         n, T = self.N, self.L + self.K
         out = []
         for d in range(self.parts):
-            a = self.uniform(self.all_idx)
+            a = a_given[d] if a_given is not None else self.uniform(self.all_idx)
+            e = e_given[d] if e_given is not None else self.error()
             b = self.limbwise("modadd", self.neg(self.limbwise("modmul", a, s_res_ntt, self.all_idx), self.all_idx),
-                              self.small_to_ntt(self.error(), self.all_idx), self.all_idx)
+                              self.small_to_ntt(e, self.all_idx), self.all_idx)
             for i in range(d * self.part_size, min((d + 1) * self.part_size, self.L)):
                 lift = self.o.hw("modmul_scalar", s_src_ntt[i * n:(i + 1) * n], self.P % self.primes[i], i)
                 b[i * n:(i + 1) * n] = self.o.hw("modadd", b[i * n:(i + 1) * n], lift, i)

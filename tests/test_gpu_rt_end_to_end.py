@@ -270,3 +270,79 @@ def test_less_used_entry_points(args):
     print("running surface_program", args, flush=True)
     r = subprocess.run([SURFACE] + args.split(), capture_output=True, text=True, timeout=110)
     assert r.returncode == 0 and "surface ok" in r.stdout, r.stdout + r.stderr
+
+
+KEYGEN = os.path.join(rt_program.ROOT, "tests", "programs", "keygen_program")
+
+
+@pytest.mark.parametrize("cfg,hw", [((8192, 5, 40, 40, 3), 192), ((65536, 6, 60, 50, 3), 192), ((2048, 4, 50, 40, 2), 0)],
+                         ids=["N8192", "N65536", "N2048_uniform_secret"])
+def test_device_built_keys_satisfy_their_defining_equations(cfg, hw, tmp_path):
+    """Keys built in HBM by Rt_generate_keys against Generate_switching_key (key_gen.c:127-262): for every digit,
+    b + a*s_res - P*s_src*[limb in the digit] must be ONE small polynomial (coefficients -1, 0, 1) seen through all
+    L+k limbs -- a dropped term, a wrong sign, the lift on the wrong limbs or a wrong automorphism of the secret
+    leaves residues that are large or differ between limbs -- and rebuilding b on the CPU from the same (a, e, s)
+    gives the device's words bit for bit.  Relinearisation, two rotations, the conjugation, and the public key."""
+    import numpy as np
+
+    from ckks_host import CkksHost
+    from oracle_lib import Oracle
+
+    assert os.path.exists(KEYGEN), "tests/programs/keygen_program is not built"
+    N, num_q, q0_bits, sf_bits, parts = cfg
+    rots = [1, -3, 2 * N - 1]
+    out_path = str(tmp_path / "keys.bin")
+    args = [KEYGEN, out_path, str(N), str(num_q - 1), str(q0_bits), str(sf_bits), str(hw), "77"] + [str(r) for r in rots]
+    print("running keygen_program", args[2:], flush=True)
+    r = subprocess.run(args, capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0, r.stdout + r.stderr
+    o = Oracle(*cfg)
+    L, K, T = o.L, o.K, o.L + o.K
+    raw = np.fromfile(out_path, np.int64)
+    key_words = 2 * parts * T * N
+    assert raw.size == N + 2 * L * N + (1 + len(rots)) * key_words
+    s = raw[:N]
+    assert set(np.unique(s)) <= {-1, 0, 1}
+    if hw:
+        assert int(np.abs(s).sum()) == hw and abs(int((s == 1).sum()) - hw // 2) <= 1
+    else:
+        assert N // 2 < int(np.abs(s).sum()) < 3 * N // 4  # uniform over {-1, 0, 1}
+    h = CkksHost(o, 5, hamming_weight=min(192, N))
+    h.s, h.s_ntt = s, h.small_to_ntt(s, h.all_idx)
+    all_idx, q_idx = h.all_idx, list(range(L))
+
+    def small_poly(res_ntt, idx, what):
+        """the polynomial whose residues res_ntt holds: must be small and the same through every limb"""
+        c = o.intt(res_ntt, idx).reshape(len(idx), N)
+        qs = np.array([o.primes[i] for i in idx], np.int64)[:, None]
+        c = np.where(c > qs // 2, c - qs, c)
+        assert np.abs(c).max() <= 1, "%s: residual is not small (max %d)" % (what, int(np.abs(c).max()))
+        assert (c == c[0]).all(), "%s: residual differs between limbs" % what
+        assert N // 4 < int(np.abs(c[0]).sum()) < 3 * N // 4, "%s: not the triangle distribution" % what
+        return c[0]
+
+    pk0, pk1 = raw[N:N + L * N], raw[N + L * N:N + 2 * L * N]
+    small_poly(h.limbwise("modadd", pk0, h.limbwise("modmul", pk1, h.s_ntt[:L * N], q_idx), q_idx), q_idx, "public key")
+    s2 = h.limbwise("modmul", h.s_ntt, h.s_ntt, all_idx)
+    cases = [("relin", h.s_ntt, s2)]
+    for rot in rots:
+        k = 2 * N - 1 if rot == 2 * N - 1 else o.find_automorphism_index(rot)
+        s_res = h.small_to_ntt(h.automorphism_coeffs(s, pow(int(k), -1, 2 * N)), all_idx)
+        cases.append(("rotation %d" % rot, s_res, h.s_ntt))
+    seen_a = []
+    for ci, (name, s_res, s_src) in enumerate(cases):
+        key = raw[N + 2 * L * N + ci * key_words:N + 2 * L * N + (ci + 1) * key_words]
+        a_list, e_list = [], []
+        for d in range(parts):
+            b, a = key[2 * d * T * N:(2 * d + 1) * T * N], key[(2 * d + 1) * T * N:(2 * d + 2) * T * N]
+            assert all((a[t * N:(t + 1) * N] < o.primes[i]).all() and (a[t * N:(t + 1) * N] >= 0).all() for t, i in enumerate(all_idx))
+            res = h.limbwise("modadd", b, h.limbwise("modmul", a, s_res, all_idx), all_idx)
+            for i in range(d * h.part_size, min((d + 1) * h.part_size, L)):
+                lift = o.hw("modmul_scalar", s_src[i * N:(i + 1) * N], h.P % o.primes[i], i)
+                res[i * N:(i + 1) * N] = o.hw("modsub", res[i * N:(i + 1) * N], lift, i)
+            e_list.append(small_poly(res, all_idx, "%s digit %d" % (name, d)))
+            a_list.append(a)
+            seen_a.append(a[:64].tobytes())
+        assert np.array_equal(h.switch_key(s_res, s_src, a_list, e_list), key), name
+    assert len(set(seen_a)) == len(seen_a), "the uniform polynomials of two digits or keys coincide"
+    o.close()
