@@ -226,6 +226,27 @@ def resnet20_leg():
         return {"resnet20": {"error": repr(e)[:200]}}
 
 
+def keyswitch_cpu_reference(level):
+    """The reference's own key-switch pieces (Alloc_precomp, Dot_prod, Mod_down, Rescale, Automorphism_transform of
+    the compiled reference, oracle/_ref/ref_driver) at this level on this host, one thread, each run once on uniform
+    residues; None where that binary is absent."""
+    import refdrv
+
+    if not refdrv.available():
+        return None
+    s = refdrv.RefSession(*CFG)
+    k = s.add(refdrv.OP_TIME_KEYSWITCH, level, 7)
+    _, res = s.run()
+    pre, dot, down, resc, auto = (int(v) * 1e-9 for v in res[k])
+    note = "the reference's Alloc_precomp / 2 x Dot_prod / 2 x Mod_down / 2 x Rescale / 2 x Automorphism_transform, once each, gcc -O3"
+    return {"keyswitch_cpu_baseline": {"s_per_op": round(pre + dot + down + resc, 3), "cores": 1, "kind": "reference",
+                                       "parts_s": {"precomp": round(pre, 3), "dot_prod_x2": round(dot, 3),
+                                                   "mod_down_x2": round(down, 3), "rescale_x2": round(resc, 3)},
+                                       "sample": note},
+            "rotation_cpu_baseline": {"s_per_rotation": round(dot + down + auto, 3), "hoisted_precomp_s": round(pre, 3),
+                                      "cores": 1, "kind": "reference", "sample": note}}
+
+
 def extra_legs(g, which="all"):
     import headline
     from oracle_lib import Oracle
@@ -244,6 +265,12 @@ def extra_legs(g, which="all"):
     o.close()
     for b in cts + [swk]:
         b.free()
+    ref = keyswitch_cpu_reference(level)
+    if ref:
+        if "keyswitch_ops_per_s" in extra:
+            extra["keyswitch_cpu_baseline"] = ref["keyswitch_cpu_baseline"]
+        if "rotations_per_s" in extra:
+            extra["rotation_cpu_baseline"] = ref["rotation_cpu_baseline"]
     return extra
 
 

@@ -41,7 +41,7 @@ enum {
   OP_NTT = 1, OP_INTT, OP_HW, OP_DECOMP_MODUP, OP_PRECOMP, OP_MOD_DOWN,
   OP_RESCALE, OP_DOT_PROD, OP_AUTO_ORDER, OP_AUTO_INDEX, OP_AUTOMORPHISM,
   OP_EXTEND, OP_TBL_MODUP, OP_TBL_MODDOWN, OP_TBL_RESCALE, OP_POLY, OP_TWIDDLES,
-  OP_MOD_UP, OP_MOD_DOWN_RESCALE, OP_REDUCE_RESCALE_MODUP, OP_FROM_LEVEL0, OP_ENCODE, OP_DECODE, OP_EMBEDDING, OP_TIME_NTT, OP_ENCODE_SCALED
+  OP_MOD_UP, OP_MOD_DOWN_RESCALE, OP_REDUCE_RESCALE_MODUP, OP_FROM_LEVEL0, OP_ENCODE, OP_DECODE, OP_EMBEDDING, OP_TIME_NTT, OP_ENCODE_SCALED, OP_TIME_KEYSWITCH
 };
 
 static int64_t* in_buf;
@@ -146,6 +146,80 @@ int main(int argc, char** argv) {
         wr1(trips);
         wr1(ns);
         wr(data, nl * N);
+        break;
+      }
+      case OP_TIME_KEYSWITCH: { /* a1 = level, a2 = seed; no input.  The pieces of one key switch at `level`, each run
+                                   once on uniform residues and timed on its own: Alloc_precomp, two Dot_prod (the two
+                                   halves of a key), two Mod_down, two Rescale, two Automorphism_transform.
+                                   out = nanoseconds of the five, in that order */
+        size_t lv = (size_t)a1, nd = Get_num_decomp(Get_crt_context(), lv);
+        uint64_t st = (uint64_t)a2 * 0x9E3779B97F4A7C15ull + 1;
+        int64_t* c2 = (int64_t*)malloc(lv * N * sizeof(int64_t));
+        int64_t* key = (int64_t*)malloc(2 * nd * (L + K) * N * sizeof(int64_t));
+        for (size_t t = 0; t < lv; t++) {
+          uint64_t q = (uint64_t)Get_modulus_val(prime_at(t));
+          for (size_t i = 0; i < N; i++) {
+            st = st * 6364136223846793005ull + 1442695040888963407ull;
+            c2[t * N + i] = (int64_t)((st >> 3) % q);
+          }
+        }
+        for (size_t h = 0; h < 2 * nd; h++)
+          for (size_t t = 0; t < L + K; t++) {
+            uint64_t q = (uint64_t)Get_modulus_val(prime_at(t));
+            for (size_t i = 0; i < N; i++) {
+              st = st * 6364136223846793005ull + 1442695040888963407ull;
+              key[(h * (L + K) + t) * N + i] = (int64_t)((st >> 3) % q);
+            }
+          }
+        struct timespec t0, t1;
+        int64_t ns[5];
+#define TICK() clock_gettime(CLOCK_MONOTONIC, &t0)
+#define TOCK(k) (clock_gettime(CLOCK_MONOTONIC, &t1), ns[k] = (int64_t)(t1.tv_sec - t0.tv_sec) * 1000000000 + (t1.tv_nsec - t0.tv_nsec))
+        POLYNOMIAL src, kb[16], ka[16], dg[16], ext[2], down[2], low[2], rot[2];
+        wrap_poly(&src, c2, lv, 0, true);
+        TICK();
+        VALUE_LIST* pl = Alloc_precomp(&src);
+        TOCK(0);
+        for (size_t d = 0; d < nd; d++) {
+          dg[d] = *(POLYNOMIAL*)Get_ptr_value_at(pl, d);
+          wrap_poly(&kb[d], key + (2 * d) * (L + K) * N, L, K, true);
+          wrap_poly(&ka[d], key + (2 * d + 1) * (L + K) * N, L, K, true);
+        }
+        memset(ext, 0, sizeof(ext)), memset(down, 0, sizeof(down)), memset(low, 0, sizeof(low)), memset(rot, 0, sizeof(rot));
+        TICK();
+        Dot_prod(&ext[0], dg, kb, (uint32_t)nd);
+        Dot_prod(&ext[1], dg, ka, (uint32_t)nd);
+        TOCK(1);
+        for (int h = 0; h < 2; h++) {
+          Alloc_poly_data(&down[h], (uint32_t)N, lv, 0);
+          Alloc_poly_data(&low[h], (uint32_t)N, lv - 1, 0);
+          Alloc_poly_data(&rot[h], (uint32_t)N, lv, 0);
+          Set_is_ntt(&down[h], true), Set_is_ntt(&low[h], true), Set_is_ntt(&rot[h], true);
+        }
+        TICK();
+        Mod_down(&down[0], &ext[0]);
+        Mod_down(&down[1], &ext[1]);
+        TOCK(2);
+        VALUE_LIST* order = Alloc_value_list(I64_TYPE, N);
+        Precompute_automorphism_order(order, 5, (uint32_t)N, true);
+        TICK();
+        Automorphism_transform(&rot[0], &down[0], order);
+        Automorphism_transform(&rot[1], &down[1], order);
+        TOCK(4);
+        TICK();
+        Rescale(&low[0], &down[0]);
+        Rescale(&low[1], &down[1]);
+        TOCK(3);
+#undef TICK
+#undef TOCK
+        wr1(5);
+        wr(ns, 5);
+        for (int h = 0; h < 2; h++) {
+          Free_poly_data(&ext[h]), Free_poly_data(&down[h]), Free_poly_data(&low[h]), Free_poly_data(&rot[h]);
+        }
+        Free_value_list(order);
+        Free_precomp(pl);
+        free(c2), free(key);
         break;
       }
       case OP_HW: { /* a1 = which, a2 = prime idx, a3 = n; in = r[n] a[n] b[n] */
