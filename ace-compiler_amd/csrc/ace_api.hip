@@ -385,8 +385,11 @@ struct ace_ctx {
         if (!d.fp_ok[i]) continue;
         for (size_t k = 0; k < h.N; ++k) {
           size_t o = i * h.N + k;
-          w[o] = (double)h.rou[o];
-          iw[o] = (double)h.irou[o];
+          // centred on zero: |w| <= q/2 halves the error of the quotient estimate in a twiddle product, which is
+          // what lets six forward stages run between two reductions (ace_ntt.hip)
+          const i64 q = (i64)h.primes[i].q, a = (i64)h.rou[o], b = (i64)h.irou[o];
+          w[o] = (double)(a > q / 2 ? a - q : a);
+          iw[o] = (double)(b > q / 2 ? b - q : b);
         }
       }
       if (use_fp) {

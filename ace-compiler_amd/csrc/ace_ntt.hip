@@ -52,6 +52,15 @@ constexpr int kLogChunk = 12;
 
 __device__ __forceinline__ int lds_pos(int e) { return e + (e >> 4); }
 
+// Orders the LDS writes of a wave before its own later LDS reads, where no other wave touches those words (the
+// wave <-> octet <-> narrow exchanges of a chunk pass stay inside the 512 words a wave owns): the hardware carries
+// out one wave's LDS instructions in order, so only the compiler has to be kept from moving them.
+__device__ __forceinline__ void wave_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 // ---------------------------------------------------------------------------
 struct ArithInt {
   typedef u64 T;
@@ -233,9 +242,9 @@ __device__ __forceinline__ void reduce_all(const A& ar, typename A::T* v) {
 template <class A, int LOGR, int K = 0>
 __device__ __forceinline__ void fwd_strided_stages(const A& ar, typename A::T* v) {
   if constexpr (K < LOGR) {
-    // four stages is the most the FP64 back end may run between reductions; up to three may start from
-    // canonical residues, four need centred ones
-    if ((K == 0 && LOGR >= 4) || K == 4) reduce_all<A, (1 << LOGR)>(ar, v);
+    // the FP64 back end may run five stages from canonical residues, six from centred ones (see the head of
+    // this file): no reduction here for LOGR <= 5
+    static_assert(LOGR <= 5, "reduce before the sixth stage");
     ct_stage<A, (1 << LOGR), K>(ar, v, 1u << K);
     fwd_strided_stages<A, LOGR, K + 1>(ar, v);
   }
@@ -243,7 +252,7 @@ __device__ __forceinline__ void fwd_strided_stages(const A& ar, typename A::T* v
 template <class A, int LOGR, int K = 0>
 __device__ __forceinline__ void inv_strided_stages(const A& ar, typename A::T* v) {
   if constexpr (K < LOGR) {
-    if ((K & 1) == 0) reduce_all<A, (1 << LOGR)>(ar, v);
+    if (K % 3 == 0) reduce_all<A, (1 << LOGR)>(ar, v);  // an inverse stage doubles the bound: three from centred values
     gs_stage<A, (1 << LOGR), K>(ar, v, (1u << LOGR) >> (K + 1));
     inv_strided_stages<A, LOGR, K + 1>(ar, v);
   }
@@ -409,13 +418,12 @@ __device__ __forceinline__ void fwd_chunk_body(u64* lds_words, const DevCtx& c, 
     // local stages 3..5: local group = (wv << (ls-3)) + g
 #pragma unroll
     for (int r = 0; r < 8; ++r) v[r] = lds[cm.wave + ChunkMap::wave_off(r)];
-    reduce_all<A, 8>(ar, v);
     ct_stage<A, 8, 0>(ar, v, (tw0 << 3) + (cm.wv << 0));
     ct_stage<A, 8, 1>(ar, v, (tw0 << 4) + (cm.wv << 1));
     ct_stage<A, 8, 2>(ar, v, (tw0 << 5) + (cm.wv << 2));
 #pragma unroll
     for (int r = 0; r < 8; ++r) lds[cm.wave + ChunkMap::wave_off(r)] = v[r];
-    __syncthreads();
+    wave_sync();  // the words read next were written by this wave
     // local stages 6..8: local group = (h << (ls-6)) + g
 #pragma unroll
     for (int r = 0; r < 8; ++r) v[r] = lds[cm.octet + ChunkMap::octet_off(r)];
@@ -425,11 +433,10 @@ __device__ __forceinline__ void fwd_chunk_body(u64* lds_words, const DevCtx& c, 
     ct_stage<A, 8, 2>(ar, v, (tw0 << 8) + (cm.h << 2));
 #pragma unroll
     for (int r = 0; r < 8; ++r) lds[cm.octet + ChunkMap::octet_off(r)] = v[r];
-    __syncthreads();
+    wave_sync();  // the words read next were written by this wave
     // local stages 9..11: local group = (t << (ls-9)) + g
 #pragma unroll
     for (int r = 0; r < 8; ++r) v[r] = lds[cm.narrow + ChunkMap::narrow_off(r)];
-    reduce_all<A, 8>(ar, v);
     ct_stage<A, 8, 0>(ar, v, (tw0 << 9) + ((u32)t << 0));
     ct_stage<A, 8, 1>(ar, v, (tw0 << 10) + ((u32)t << 1));
     ct_stage<A, 8, 2>(ar, v, (tw0 << 11) + ((u32)t << 2));
@@ -541,7 +548,7 @@ __device__ __forceinline__ void inv_chunk_body(u64* lds_words, const DevCtx& c, 
     gs_stage<A, 8, 2>(ar, v, (mh >> 2) + (chunk << 9) + ((u32)t << 0));
 #pragma unroll
     for (int r = 0; r < 8; ++r) lds[cm.narrow + ChunkMap::narrow_off(r)] = v[r];
-    __syncthreads();
+    wave_sync();  // the words read next were written by this wave
     // spans 8, 16, 32
 #pragma unroll
     for (int r = 0; r < 8; ++r) v[r] = lds[cm.octet + ChunkMap::octet_off(r)];
@@ -551,7 +558,7 @@ __device__ __forceinline__ void inv_chunk_body(u64* lds_words, const DevCtx& c, 
     gs_stage<A, 8, 2>(ar, v, (mh >> 5) + (chunk << 6) + (cm.h << 0));
 #pragma unroll
     for (int r = 0; r < 8; ++r) lds[cm.octet + ChunkMap::octet_off(r)] = v[r];
-    __syncthreads();
+    wave_sync();  // the words read next were written by this wave
     // spans 64, 128, 256
 #pragma unroll
     for (int r = 0; r < 8; ++r) v[r] = lds[cm.wave + ChunkMap::wave_off(r)];

@@ -39,9 +39,22 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def time_region(g, fn, reps):
-    """Average milliseconds per call of fn over reps calls, by HIP events on the library's stream."""
+def settle(g, fn, ms=60.0):
+    """Untimed calls of fn until the GPU has been busy for `ms` milliseconds: the part's clocks (and with them every
+    kernel time) settle only after some tens of milliseconds of load, and a measurement that starts on an idle GPU
+    reads up to 10 % slow."""
     g.sync()
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < ms:
+        for _ in range(4):
+            fn()
+        g.sync()
+
+
+def time_region(g, fn, reps):
+    """Average milliseconds per call of fn over reps calls, by HIP events on the library's stream, after the
+    clocks have settled under the same load."""
+    settle(g, fn)
     g.timer_start()
     for _ in range(reps):
         fn()
@@ -310,6 +323,8 @@ def main():
 
     if args.only_extra:
         args.warmup, args.steps = 0, 1
+    else:
+        settle(g, step)  # untimed, before the warm-up steps: see settle()
     for _ in range(args.warmup):
         step()
     g.sync()
@@ -351,7 +366,7 @@ def main():
         src = x if which == 1 else scratch
         f = lambda: g.ntt_pass(scratch, src, idx, POLYS, LIMBS, inv, which)
         f()
-        ms = time_region(g, f, 10)
+        ms = time_region(g, f, 20)
         kern[name] = {"ms": round(ms, 4), "GB/s": round(pass_bytes / (ms * 1e-3) / 1e9, 1)}
     dom = max(kern, key=lambda k: kern[k]["ms"])
     roofline = {"bound": "hbm", "kernel": dom, "achieved": kern[dom]["GB/s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
