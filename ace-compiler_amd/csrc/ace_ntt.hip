@@ -14,7 +14,8 @@
 //            three stages with the chunk passing through LDS between rounds
 //            (LDS index padded by e>>4, which keeps every round's accesses
 //            free of bank conflicts), and once more so that the global
-//            store is coalesced.  Eight registers per thread leave room for
+//            store is coalesced.  Two of the exchanges stay inside the 512
+//            words a wave owns and need no work-group barrier.  Eight registers per thread leave room for
 //            eight waves per SIMD, which is what hides the memory waits.
 //   inverse  the same two kernels mirrored (chunk first, strided last).
 // N <= 4096 uses one workgroup per limb with the limb in LDS.
@@ -28,14 +29,19 @@
 //   ArithFp   for primes below 2^50.2: residues are carried as exact integers
 //             in FP64 (|x| < 2^53).  A twiddle product is y*w - rint(y*(w/q))*q
 //             evaluated exactly with one FMA for the low half of y*w and one
-//             for the subtraction (6 full-rate FP64 ops); sums are brought
-//             back to |x| <= q/2 with x - rint(x/q)*q before they can pass
-//             2^53: a forward stage takes a bound of B q to at most
-//             (1.43 B + 0.5) q, an inverse stage doubles it, so forward code
-//             reduces at least every four stages (every three in the chunk
-//             pass) and inverse code every two or three.  All intermediate
-//             values are integers below 2^53, so no rounding ever happens
-//             and the final canonical residue is exact.
+//             for the subtraction (6 full-rate FP64 ops).  The twiddles are
+//             stored centred on zero (|w| <= q/2): the quotient estimate is off
+//             by at most 1/2 + 3*2^-53*|y||w|/q, so a product of a value of
+//             magnitude B q comes out below (0.5 + 0.215 B) q, and a forward
+//             stage takes a bound of B q to at most (1.215 B + 0.5) q.  From
+//             centred values (B = 1/2) six stages reach 6.77 q, from canonical
+//             residues (B = 1) five reach 6.49 q, both below 2^53 / q >= 6.98:
+//             the forward strided pass never reduces, the forward chunk pass
+//             reduces (x - rint(x/q)*q) before its first and its third round.
+//             An inverse stage doubles the bound of its sums, so inverse code
+//             reduces every three stages (0.5 q -> 4 q).  All intermediate
+//             values are integers below 2^53, so no rounding ever happens and
+//             the final canonical residue is exact.
 // Between the two passes the buffer holds back-end specific words (lazily
 // reduced integers, or raw FP64 bits); the second pass stores canonical
 // residues.
@@ -102,6 +108,7 @@ struct ArithInt {
   __device__ __forceinline__ T in_mid(u64 v) const { return v; }
   __device__ __forceinline__ u64 out_mid(T v) const { return v; }
   __device__ __forceinline__ void reduce(T&) const {}
+  __device__ __forceinline__ void recentre_sum_of_four(T&) const {}
   // forward, Harvey butterflies with the cheaper quotient estimate (product in [0, 4q)): x,y < 8q -> < 8q
   __device__ __forceinline__ void ct(T& x, T& y, const TW& tw) const {
     u64 a = csub(x, q4);
@@ -162,6 +169,11 @@ struct ArithFp {
   __device__ __forceinline__ u64 out_mid(T v) const { return (u64)__double_as_longlong(v); }
   // x - rint(x/q)*q: |result| <= (1/2 + 2^-49) q, exact
   __device__ __forceinline__ void reduce(T& x) const { x = __builtin_fma(-__builtin_rint(x * qinv), q, x); }
+  // The first round of an inverse chunk pass starts from canonical residues, all in [0, q).  Instead of centring
+  // all eight values (24 operations), the two sums of four that meet in the third stage, each in [0, 4q), are
+  // shifted by 2q: their sum stays within +-4q, every other value has passed through a twiddle product and is
+  // small, and the round ends with the same bound (4q) as one that starts from centred values.
+  __device__ __forceinline__ void recentre_sum_of_four(T& x) const { x -= q + q; }
   // y*w mod q as a signed integer of magnitude <= (1/2 + 0.43 |y|/q) q, exact
   __device__ __forceinline__ double mulmod(double y, double ww, double wwi) const {
     double c = __builtin_rint(y * wwi);
@@ -342,6 +354,9 @@ static inline unsigned chunk_grid(const DevCtx& c, u32 n_limbs, u32 slots_per_gr
 #define ACE_NTT_PB 1
 #endif
 constexpr int kPolysPerBlock = ACE_NTT_PB;
+#ifndef ACE_NTT_SHIFT
+#define ACE_NTT_SHIFT 1
+#endif
 constexpr int kChunkThreads = 512;  // 8 coefficients per thread
 
 // The four thread -> element maps of a chunk pass (r = 0..7).  Each covers the
@@ -378,7 +393,7 @@ struct ChunkMap {
 // once more so that the global store is coalesced.  A thread writes back the
 // positions it read, so one barrier per round suffices.
 // EPI != 0: the result is not stored back but consumed by FwdFuse::epi.
-template <class A, int EPI>
+template <class A, int EPI, int SKIP>
 __device__ __forceinline__ void fwd_chunk_body(u64* lds_words, const DevCtx& c, const PolySeq& datas,
                                                const LimbMap& pos, u32 logr, u32 n_polys, const FwdFuse& f, u32 chunk,
                                                u32 limb, u32 pblk, u32 pi) {
@@ -409,7 +424,7 @@ __device__ __forceinline__ void fwd_chunk_body(u64* lds_words, const DevCtx& c, 
 #pragma unroll
     for (int r = 0; r < 8; ++r) v[r] = ar.in_mid(raw[r]);
     reduce_all<A, 8>(ar, v);
-    ct_stage<A, 8, 0>(ar, v, tw0 << 0);
+    if (!SKIP) ct_stage<A, 8, 0>(ar, v, tw0 << 0);  // else the strided pass has run this stage as its last
     ct_stage<A, 8, 1>(ar, v, tw0 << 1);
     ct_stage<A, 8, 2>(ar, v, tw0 << 2);
 #pragma unroll
@@ -486,15 +501,15 @@ __device__ __forceinline__ void fwd_chunk_body(u64* lds_words, const DevCtx& c, 
   }
 }
 // (the Mod_down tail keeps three more pointers and constants alive: 80 registers, 6 waves per SIMD)
-template <int EPI>
+template <int EPI, int SKIP>
 __global__ __launch_bounds__(kChunkThreads, EPI == 1 ? 6 : 8) void ntt_fwd_chunk(DevCtx c, PolySeq datas, LimbMap lm, LimbMap pos,
                                                                   u32 logr, u32 n_limbs, u32 n_polys, FwdFuse f) {
   __shared__ u64 lds[kChunk + kChunk / 16];
   u32 chunk, limb, pblk;
   if (!chunk_block(c, n_limbs, (n_polys + kPolysPerBlock - 1) / kPolysPerBlock, chunk, limb, pblk)) return;
   const u32 pi = lm.prime[limb];
-  if (c.fp_ok[pi]) fwd_chunk_body<ArithFp, EPI>(lds, c, datas, pos, logr, n_polys, f, chunk, limb, pblk, pi);
-  else fwd_chunk_body<ArithInt, EPI>(lds, c, datas, pos, logr, n_polys, f, chunk, limb, pblk, pi);
+  if (c.fp_ok[pi]) fwd_chunk_body<ArithFp, EPI, SKIP>(lds, c, datas, pos, logr, n_polys, f, chunk, limb, pblk, pi);
+  else fwd_chunk_body<ArithInt, EPI, SKIP>(lds, c, datas, pos, logr, n_polys, f, chunk, limb, pblk, pi);
 }
 
 // ---------------------------------------------------------------------------
@@ -503,7 +518,7 @@ __global__ __launch_bounds__(kChunkThreads, EPI == 1 ? 6 : 8) void ntt_fwd_chunk
 // by the strided pass that always follows.  At span 2^u the stage has
 // m = N >> (u+1) groups and element j belongs to group j >> (u+1).  The rounds
 // are those of the forward pass in reverse order.
-template <class A>
+template <class A, int SKIP>
 __device__ __forceinline__ void inv_chunk_body(u64* lds_words, const DevCtx& c, const PolySeq& dsts,
                                                const PolySeq& srcs, const CopyThrough& copies, const LimbMap& pos,
                                                u32 n_polys, u32 chunk, u32 limb, u32 pblk, u32 pi) {
@@ -542,9 +557,10 @@ __device__ __forceinline__ void inv_chunk_body(u64* lds_words, const DevCtx& c, 
     // spans 1, 2, 4
 #pragma unroll
     for (int r = 0; r < 8; ++r) v[r] = lds[cm.narrow + ChunkMap::narrow_off(r)];
-    reduce_all<A, 8>(ar, v);
     gs_stage<A, 8, 0>(ar, v, (mh >> 0) + (chunk << 11) + ((u32)t << 2));
     gs_stage<A, 8, 1>(ar, v, (mh >> 1) + (chunk << 10) + ((u32)t << 1));
+    ar.recentre_sum_of_four(v[0]);
+    ar.recentre_sum_of_four(v[4]);
     gs_stage<A, 8, 2>(ar, v, (mh >> 2) + (chunk << 9) + ((u32)t << 0));
 #pragma unroll
     for (int r = 0; r < 8; ++r) lds[cm.narrow + ChunkMap::narrow_off(r)] = v[r];
@@ -576,21 +592,22 @@ __device__ __forceinline__ void inv_chunk_body(u64* lds_words, const DevCtx& c, 
     reduce_all<A, 8>(ar, v);
     gs_stage<A, 8, 0>(ar, v, (mh >> 9) + (chunk << 2));
     gs_stage<A, 8, 1>(ar, v, (mh >> 10) + (chunk << 1));
-    gs_stage<A, 8, 2>(ar, v, (mh >> 11) + (chunk << 0));
+    if (!SKIP) gs_stage<A, 8, 2>(ar, v, (mh >> 11) + (chunk << 0));  // else the strided pass runs it as its first
 #pragma unroll
     for (int r = 0; r < 8; ++r) dst[off + t + 512 * r] = ar.out_mid(v[r]);
 #pragma unroll
     for (int r = 0; r < 8; ++r) raw[r] = nxt[r];
   }
 }
+template <int SKIP>
 __global__ __launch_bounds__(kChunkThreads, 8) void ntt_inv_chunk(DevCtx c, PolySeq dsts, PolySeq srcs, CopyThrough copies,
                                                                   LimbMap lm, LimbMap pos, u32 n_limbs, u32 n_polys) {
   __shared__ u64 lds[kChunk + kChunk / 16];
   u32 chunk, limb, pblk;
   if (!chunk_block(c, n_limbs, (n_polys + kPolysPerBlock - 1) / kPolysPerBlock, chunk, limb, pblk)) return;
   const u32 pi = lm.prime[limb];
-  if (c.fp_ok[pi]) inv_chunk_body<ArithFp>(lds, c, dsts, srcs, copies, pos, n_polys, chunk, limb, pblk, pi);
-  else inv_chunk_body<ArithInt>(lds, c, dsts, srcs, copies, pos, n_polys, chunk, limb, pblk, pi);
+  if (c.fp_ok[pi]) inv_chunk_body<ArithFp, SKIP>(lds, c, dsts, srcs, copies, pos, n_polys, chunk, limb, pblk, pi);
+  else inv_chunk_body<ArithInt, SKIP>(lds, c, dsts, srcs, copies, pos, n_polys, chunk, limb, pblk, pi);
 }
 
 // inverse, strided pass: spans 4096..N/2, then scale every word by the limb's
@@ -665,43 +682,52 @@ __global__ __launch_bounds__(256) void ntt_small(DevCtx c, PolySeq dsts, PolySeq
 }
 
 // ---------------------------------------------------------------------------
-template <int LOGR>
+// LOGR = logN - 12 stages lie outside a 4096-word chunk.  With a shift of 1 the strided pass, which is bound by HBM
+// and has instruction slots to spare, also runs the chunk's widest stage (LOGR + 1 stages on N / 2^(LOGR+1) rows of
+// a column), and the chunk pass skips it.  Measured on 768 limbs at N = 2^16: the chunk passes gain 2 %, the inverse
+// strided pass stays where it was and the forward one, which then needs 122 registers, loses 6 %: the inverse
+// transform shifts (SI), the forward one does not (SF).
+template <int LOGR, int SF, int SI>
 static void run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolySeq& src, const LimbMap& lm,
                       const LimbMap& pos, u32 n_limbs, u32 n_polys, bool inverse, const u64* scale, int passes,
                       const FwdFuse& f, const CopyThrough& copies) {
-  dim3 gs((c.N >> LOGR) / 256, n_limbs, n_polys),
-      gc(chunk_grid(c, n_limbs, (n_polys + kPolysPerBlock - 1) / kPolysPerBlock));
+  dim3 gc(chunk_grid(c, n_limbs, (n_polys + kPolysPerBlock - 1) / kPolysPerBlock));
   if (!inverse) {
+    constexpr int LS = LOGR + SF, SHIFT = SF;
+    dim3 gs((c.N >> LS) / 256, n_limbs, n_polys);
     if (passes & 1) {
       if (f.pro == 0)
-        hipLaunchKernelGGL((ntt_fwd_strided<LOGR, 0>), gs, dim3(256), 0, st, c, dst, src, lm, pos, f);
+        hipLaunchKernelGGL((ntt_fwd_strided<LS, 0>), gs, dim3(256), 0, st, c, dst, src, lm, pos, f);
       else
-        hipLaunchKernelGGL((ntt_fwd_strided<LOGR, 1>), gs, dim3(256), 0, st, c, dst, src, lm, pos, f);
+        hipLaunchKernelGGL((ntt_fwd_strided<LS, 1>), gs, dim3(256), 0, st, c, dst, src, lm, pos, f);
     }
     if (passes & 2) {
       const u32 lr = LOGR;
       if (f.epi == 0)
-        hipLaunchKernelGGL((ntt_fwd_chunk<0>), gc, dim3(kChunkThreads), 0, st, c, dst, lm, pos, lr, n_limbs,
+        hipLaunchKernelGGL((ntt_fwd_chunk<0, SHIFT>), gc, dim3(kChunkThreads), 0, st, c, dst, lm, pos, lr, n_limbs,
                            n_polys, f);
       else if (f.epi == 1)
-        hipLaunchKernelGGL((ntt_fwd_chunk<1>), gc, dim3(kChunkThreads), 0, st, c, dst, lm, pos, lr, n_limbs,
+        hipLaunchKernelGGL((ntt_fwd_chunk<1, SHIFT>), gc, dim3(kChunkThreads), 0, st, c, dst, lm, pos, lr, n_limbs,
                            n_polys, f);
       else
-        hipLaunchKernelGGL((ntt_fwd_chunk<2>), gc, dim3(kChunkThreads), 0, st, c, dst, lm, pos, lr, n_limbs,
+        hipLaunchKernelGGL((ntt_fwd_chunk<2, SHIFT>), gc, dim3(kChunkThreads), 0, st, c, dst, lm, pos, lr, n_limbs,
                            n_polys, f);
     }
   } else {
+    constexpr int LS = LOGR + SI, SHIFT = SI;
+    dim3 gs((c.N >> LS) / 256, n_limbs, n_polys);
     if (passes & 1)
-      hipLaunchKernelGGL(ntt_inv_chunk, gc, dim3(kChunkThreads), 0, st, c, dst, src, copies, lm, pos, n_limbs, n_polys);
+      hipLaunchKernelGGL((ntt_inv_chunk<SHIFT>), gc, dim3(kChunkThreads), 0, st, c, dst, src, copies, lm, pos, n_limbs,
+                         n_polys);
     if (passes & 2) {
       u32 n_fp = 0;
       for (u32 t = 0; t < n_limbs; ++t) n_fp += c.fp_ok[lm.prime[t]] ? 1 : 0;
       if (n_fp == 0)
-        hipLaunchKernelGGL((ntt_inv_strided<LOGR, 1>), gs, dim3(256), 0, st, c, dst, lm, pos, scale);
+        hipLaunchKernelGGL((ntt_inv_strided<LS, 1>), gs, dim3(256), 0, st, c, dst, lm, pos, scale);
       else if (n_fp == n_limbs)
-        hipLaunchKernelGGL((ntt_inv_strided<LOGR, 2>), gs, dim3(256), 0, st, c, dst, lm, pos, scale);
+        hipLaunchKernelGGL((ntt_inv_strided<LS, 2>), gs, dim3(256), 0, st, c, dst, lm, pos, scale);
       else
-        hipLaunchKernelGGL((ntt_inv_strided<LOGR, 0>), gs, dim3(256), 0, st, c, dst, lm, pos, scale);
+        hipLaunchKernelGGL((ntt_inv_strided<LS, 0>), gs, dim3(256), 0, st, c, dst, lm, pos, scale);
     }
   }
 }
@@ -731,15 +757,15 @@ bool launch_ntt(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolyS
     return true;
   }
   switch (c.logN - kLogChunk) {
-#define ACE_NTT_CASE(LR)                                                                      \
-  case LR:                                                                                    \
-    run_large<LR>(st, c, dst, src, lm, pos, n_limbs, n_polys, inverse, scale, passes, f, copies); \
+#define ACE_NTT_CASE(LR, SH)                                                                       \
+  case LR:                                                                                         \
+    run_large<LR, 0, SH>(st, c, dst, src, lm, pos, n_limbs, n_polys, inverse, scale, passes, f, copies); \
     return true;
-    ACE_NTT_CASE(1)
-    ACE_NTT_CASE(2)
-    ACE_NTT_CASE(3)
-    ACE_NTT_CASE(4)
-    ACE_NTT_CASE(5)
+    ACE_NTT_CASE(1, ACE_NTT_SHIFT)
+    ACE_NTT_CASE(2, ACE_NTT_SHIFT)
+    ACE_NTT_CASE(3, ACE_NTT_SHIFT)
+    ACE_NTT_CASE(4, ACE_NTT_SHIFT)
+    ACE_NTT_CASE(5, 0)  // 64 rows of a column would not fit the registers of a thread
 #undef ACE_NTT_CASE
     default:
       return false;  // ring degree above 2^17 not supported
