@@ -801,9 +801,10 @@ void do_mod_down(ace_ctx* c, const PolySeq& res, const PolySeq& src, size_t np, 
   launch_baseconv(c->stream, c->d, y, t, b, (u32)np);
   if (is_ntt) {
     PolySeq ys = seq_strided(y, level * N);
-    if (c->d.logN > 12 && !orders) {  // the tail rides on the transform's last kernel
+    if (c->d.logN > 12) {  // the tail, and with `orders` the automorphism, ride on the transform's last kernel
       FwdFuse f{};
       f.epi = 1;
+      if (orders) f.orders = *orders;
       f.out = res;
       f.src = src;
       f.addend = addend_mode ? *addend : res;

@@ -163,12 +163,23 @@ __device__ __forceinline__ u64 sub_mod(u64 a, u64 b, u64 q) {
 }
 
 
+constexpr int kMaxBatchPtrs = 32;  // keys / index tables per batched launch
+struct OrderSet {  // one automorphism table per rotation, or one shared (n == 1)
+  const i64* p[kMaxBatchPtrs];
+  u32 n;
+};
+
 // Work folded into a forward NTT of N > 4096 (launch_ntt): a prologue that forms
 // the transform's input on the fly, and an epilogue that consumes its output
 // instead of storing it.  Limb t of polynomial p is word offset pos[t]*N.
 //   pro 1  Rescale's modulus switch (rns_poly.c:340-360): input word i of limb t =
 //          Switch_modulus(last[p*last_stride + i], q_last -> q_t) * sw[3t] (Shoup sw[3t+1], sw[3t+2] = q_t - q_last mod q_t)
-//   epi 1  Mod_down tail (rns_poly.c:292-303): out = (src - ntt) * cst[2t] (+ addend)
+//   epi 1  Mod_down tail (rns_poly.c:292-303): out = (src - ntt) * cst[2t] (+ addend).  With index tables
+//          (orders.n != 0; polynomials 2r and 2r+1 use table r) the automorphism that ends a rotation is applied
+//          on the way out: out[i] = the value at orders[i].  The tables must be those of
+//          Precompute_automorphism_order for the NTT form (number_theory.c:211-222): an affine map of the
+//          evaluation index, which in bit-reversed order takes every aligned block of 2^s words onto one such
+//          block, so a 4096-word chunk of the result comes from one chunk of the transform.
 //   epi 2  Rescale tail (rns_poly.c:362-372):  out = src * cst[2t] + ntt
 // addend_mode: 0 none, 1 every polynomial, 2 even polynomials only.
 struct FwdFuse {
@@ -180,6 +191,7 @@ struct FwdFuse {
   PolySeq out, src, addend;
   int addend_mode;
   const u64* cst;
+  OrderSet orders;
 };
 
 }  // namespace ace

@@ -8,7 +8,7 @@ namespace ace {
 enum EwOp { EW_ADD, EW_SUB, EW_MUL, EW_MULADD, EW_ADD_S, EW_SUB_S, EW_MUL_S, EW_MULADD_S };
 
 constexpr int kMaxConvJobs = 4;   // digits converted per base-conversion launch
-constexpr int kMaxBatchPtrs = 32; // keys / index tables per batched launch
+// (kMaxBatchPtrs, the number of keys / index tables per batched launch, and OrderSet live in ace_device.h)
 
 // one digit's base conversion: out[map.out_limb[j]][i] = (sum_k t[k][i] * hat[k*hat_stride + j]) mod prime map.prime[j]
 // Targets below kFpConvTargetLimit take the conversion in exact double arithmetic when the job has tables (fw):
@@ -33,10 +33,6 @@ struct ConvBatch {
 };
 struct KeySet {   // one switch key per operand, or one shared by all (n == 1)
   const u64* p[kMaxBatchPtrs];
-  u32 n;
-};
-struct OrderSet { // one automorphism table per rotation, or one shared (n == 1)
-  const i64* p[kMaxBatchPtrs];
   u32 n;
 };
 

@@ -467,32 +467,67 @@ __device__ __forceinline__ void fwd_chunk_body(u64* lds_words, const DevCtx& c, 
     } else {
       const u32 p = poly0 + it, lt = pos.prime[limb];
       const u64 q = c.primes[pi].q, w = f.cst[2 * lt], wp = f.cst[2 * lt + 1];
-      const u64 o = (u64)lt * c.N + (u64)chunk * kChunk + t;
-      u64* out = f.out.at(p) + o;  // may alias the addend (in-place relinearisation)
-      const u64* __restrict__ src = f.src.at(p) + o;
       const u64* addend =
-          (EPI == 1 && (f.addend_mode == 1 || (f.addend_mode == 2 && !(p & 1)))) ? f.addend.at(p) + o : nullptr;
-      // four words at a time: the operands of all eight would not fit beside the 64 registers of a thread
+          (EPI == 1 && (f.addend_mode == 1 || (f.addend_mode == 2 && !(p & 1)))) ? f.addend.at(p) + (u64)lt * c.N : nullptr;
+      if (EPI == 1 && f.orders.n) {
+        // the automorphism on the way out: this chunk of the transform is the source of one chunk of the result
+        const i64* __restrict__ order = f.orders.p[f.orders.n == 1 ? 0 : (p >> 1)];
+        const u32 n_chunks = c.N >> kLogChunk;
+        u32 dc = chunk;
+        for (u32 cc = 0; cc < n_chunks; ++cc)
+          if ((u32)((u64)order[(u64)cc * kChunk] >> kLogChunk) == chunk) dc = cc;
+        order += (u64)dc * kChunk + t;
+        const u64 so = (u64)lt * c.N + (u64)chunk * kChunk;  // where this chunk's operands lie
+        u64* __restrict__ out = f.out.at(p) + (u64)lt * c.N + (u64)dc * kChunk + t;  // never an operand (checked by the callers)
+        const u64* __restrict__ src = f.src.at(p) + so;
+        if (addend) addend += (u64)chunk * kChunk;
 #pragma unroll
-      for (int r0 = 0; r0 < 8; r0 += 4) {
-        u64 sv[4], av[4];
+        for (int r0 = 0; r0 < 8; r0 += 4) {
+          u32 s[4];
+          u64 sv[4], av[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) sv[r] = src[512 * (r0 + r)];
-        if (addend) {
+          for (int r = 0; r < 4; ++r) s[r] = (u32)order[512 * (r0 + r)] & (u32)(kChunk - 1);
 #pragma unroll
-          for (int r = 0; r < 4; ++r) av[r] = addend[512 * (r0 + r)];
-        }
+          for (int r = 0; r < 4; ++r) sv[r] = src[s[r]];
+          if (addend) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const u64 y = ldsu[cm.wide + ChunkMap::wide_off(r0 + r)];
-          u64 v;
-          if (EPI == 1) {
-            v = shoup_mul(sub_mod(sv[r], y, q), w, wp, q);
-            if (addend) v = add_mod(v, av[r], q);
-          } else {
-            v = add_mod(shoup_mul(sv[r], w, wp, q), y, q);
+            for (int r = 0; r < 4; ++r) av[r] = addend[s[r]];
           }
-          out[512 * (r0 + r)] = v;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            u64 v = shoup_mul(sub_mod(sv[r], ldsu[lds_pos((int)s[r])], q), w, wp, q);
+            if (addend) v = add_mod(v, av[r], q);
+            out[512 * (r0 + r)] = v;
+          }
+        }
+        if (kPolysPerBlock > 1) __syncthreads();  // the gathered LDS reads are not the words this thread writes next
+      } else {
+        const u64 o = (u64)lt * c.N + (u64)chunk * kChunk + t;
+        u64* out = f.out.at(p) + o;  // may alias the addend (in-place relinearisation)
+        const u64* __restrict__ src = f.src.at(p) + o;
+        if (addend) addend += (u64)chunk * kChunk + t;
+        // four words at a time: the operands of all eight would not fit beside the 64 registers of a thread
+#pragma unroll
+        for (int r0 = 0; r0 < 8; r0 += 4) {
+          u64 sv[4], av[4];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) sv[r] = src[512 * (r0 + r)];
+          if (addend) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) av[r] = addend[512 * (r0 + r)];
+          }
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const u64 y = ldsu[cm.wide + ChunkMap::wide_off(r0 + r)];
+            u64 v;
+            if (EPI == 1) {
+              v = shoup_mul(sub_mod(sv[r], y, q), w, wp, q);
+              if (addend) v = add_mod(v, av[r], q);
+            } else {
+              v = add_mod(shoup_mul(sv[r], w, wp, q), y, q);
+            }
+            out[512 * (r0 + r)] = v;
+          }
         }
       }
     }
