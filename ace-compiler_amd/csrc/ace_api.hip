@@ -1241,7 +1241,7 @@ static int ntt_common(ace_ctx* c, int64_t* dst, const int64_t* src, const int32_
   const u64 stride = (u64)stride_limbs * c->h.N;
   if (!launch_ntt(c->stream, c->d, seq_strided(U(dst), stride), seq_strided(U(src), stride), lm, nullptr,
                   (u32)n_limbs, (u32)n_polys, inverse, nullptr, passes))
-    return fail("ace_ntt: ring degree not supported");
+    return fail("ace_ntt: ring degree above 2^17, or a polynomial that does not start on a 16-byte boundary");
   ACE_CATCH_INT
 }
 int ace_ntt(ace_ctx* c, int64_t* dst, const int64_t* src, const int32_t* prime_idx, size_t n_limbs, size_t n_polys,

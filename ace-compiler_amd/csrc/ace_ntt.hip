@@ -36,8 +36,8 @@
 //             stage takes a bound of B q to at most (1.215 B + 0.5) q.  From
 //             centred values (B = 1/2) six stages reach 6.77 q, from canonical
 //             residues (B = 1) five reach 6.49 q, both below 2^53 / q >= 6.98:
-//             the forward strided pass never reduces, the forward chunk pass
-//             reduces (x - rint(x/q)*q) before its first and its third round.
+//             the forward strided pass reduces (x - rint(x/q)*q) only what it
+//             stores, the forward chunk pass only before its third round.
 //             An inverse stage doubles the bound of its sums, so inverse code
 //             reduces every three stages (0.5 q -> 4 q).  All intermediate
 //             values are integers below 2^53, so no rounding ever happens and
@@ -308,6 +308,9 @@ __device__ __forceinline__ void fwd_strided_body(const DevCtx& c, const PolySeq&
     }
   }
   fwd_strided_stages<A, LOGR>(ar, v);
+  // this pass is bound by HBM and has instruction slots to spare: it hands centred values to the chunk pass,
+  // which then runs its first two rounds (six stages) without reducing
+  reduce_all<A, R>(ar, v);
 #pragma unroll
   for (int r = 0; r < R; ++r) (dst + r * rs)[col] = ar.out_mid(v[r]);
 }
@@ -358,6 +361,10 @@ constexpr int kPolysPerBlock = ACE_NTT_PB;
 #define ACE_NTT_SHIFT 1
 #endif
 constexpr int kChunkThreads = 512;  // 8 coefficients per thread
+#ifndef ACE_NTT_WAVES
+#define ACE_NTT_WAVES 8
+#endif
+constexpr int kChunkWaves = ACE_NTT_WAVES;  // waves per SIMD the chunk kernels are compiled for
 
 // The four thread -> element maps of a chunk pass (r = 0..7).  Each covers the
 // chunk once and keeps the eight elements of three consecutive stages' worth of
@@ -422,8 +429,7 @@ __device__ __forceinline__ void fwd_chunk_body(u64* lds_words, const DevCtx& c, 
     T v[8];
     // local stages 0..2
 #pragma unroll
-    for (int r = 0; r < 8; ++r) v[r] = ar.in_mid(raw[r]);
-    reduce_all<A, 8>(ar, v);
+    for (int r = 0; r < 8; ++r) v[r] = ar.in_mid(raw[r]);  // centred by the strided pass
     if (!SKIP) ct_stage<A, 8, 0>(ar, v, tw0 << 0);  // else the strided pass has run this stage as its last
     ct_stage<A, 8, 1>(ar, v, tw0 << 1);
     ct_stage<A, 8, 2>(ar, v, tw0 << 2);
@@ -458,12 +464,16 @@ __device__ __forceinline__ void fwd_chunk_body(u64* lds_words, const DevCtx& c, 
     u64* ldsu = lds_words;
 #pragma unroll
     for (int r = 0; r < 8; ++r) ldsu[cm.narrow + ChunkMap::narrow_off(r)] = ar.out_canon(v[r]);
-    __syncthreads();
-    // each thread reads back the words it will overwrite first in the next
-    // iteration, so no further barrier is needed
+    // The result leaves in the wave order (lane + 64 r inside the 512 words a wave owns): 512 contiguous bytes
+    // per store instruction, and every word a wave stores was written by that wave, so no work-group barrier is
+    // needed.  Only the automorphism gathers from the whole chunk.
+    const bool gathers = EPI == 1 && f.orders.n != 0;
+    if (gathers) __syncthreads();
+    else wave_sync();
+    const u32 wpos = cm.wv * 512 + ((u32)t & 63);  // first of this thread's words in the wave order
     if (EPI == 0) {
 #pragma unroll
-      for (int r = 0; r < 8; ++r) base[t + 512 * r] = ldsu[cm.wide + ChunkMap::wide_off(r)];
+      for (int r = 0; r < 8; ++r) base[wpos + 64 * r] = ldsu[cm.wave + ChunkMap::wave_off(r)];
     } else {
       const u32 p = poly0 + it, lt = pos.prime[limb];
       const u64 q = c.primes[pi].q, w = f.cst[2 * lt], wp = f.cst[2 * lt + 1];
@@ -502,23 +512,23 @@ __device__ __forceinline__ void fwd_chunk_body(u64* lds_words, const DevCtx& c, 
         }
         if (kPolysPerBlock > 1) __syncthreads();  // the gathered LDS reads are not the words this thread writes next
       } else {
-        const u64 o = (u64)lt * c.N + (u64)chunk * kChunk + t;
+        const u64 o = (u64)lt * c.N + (u64)chunk * kChunk + wpos;
         u64* out = f.out.at(p) + o;  // may alias the addend (in-place relinearisation)
         const u64* __restrict__ src = f.src.at(p) + o;
-        if (addend) addend += (u64)chunk * kChunk + t;
+        if (addend) addend += (u64)chunk * kChunk + wpos;
         // four words at a time: the operands of all eight would not fit beside the 64 registers of a thread
 #pragma unroll
         for (int r0 = 0; r0 < 8; r0 += 4) {
           u64 sv[4], av[4];
 #pragma unroll
-          for (int r = 0; r < 4; ++r) sv[r] = src[512 * (r0 + r)];
+          for (int r = 0; r < 4; ++r) sv[r] = src[64 * (r0 + r)];
           if (addend) {
 #pragma unroll
-            for (int r = 0; r < 4; ++r) av[r] = addend[512 * (r0 + r)];
+            for (int r = 0; r < 4; ++r) av[r] = addend[64 * (r0 + r)];
           }
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            const u64 y = ldsu[cm.wide + ChunkMap::wide_off(r0 + r)];
+            const u64 y = ldsu[cm.wave + ChunkMap::wave_off(r0 + r)];
             u64 v;
             if (EPI == 1) {
               v = shoup_mul(sub_mod(sv[r], y, q), w, wp, q);
@@ -526,18 +536,20 @@ __device__ __forceinline__ void fwd_chunk_body(u64* lds_words, const DevCtx& c, 
             } else {
               v = add_mod(shoup_mul(sv[r], w, wp, q), y, q);
             }
-            out[512 * (r0 + r)] = v;
+            out[64 * (r0 + r)] = v;
           }
         }
       }
     }
+    // the next polynomial's first round writes words that other waves may still be reading
+    if (kPolysPerBlock > 1) __syncthreads();
 #pragma unroll
     for (int r = 0; r < 8; ++r) raw[r] = nxt[r];
   }
 }
 // (the Mod_down tail keeps three more pointers and constants alive: 80 registers, 6 waves per SIMD)
 template <int EPI, int SKIP>
-__global__ __launch_bounds__(kChunkThreads, EPI == 1 ? 6 : 8) void ntt_fwd_chunk(DevCtx c, PolySeq datas, LimbMap lm, LimbMap pos,
+__global__ __launch_bounds__(kChunkThreads, kChunkWaves) void ntt_fwd_chunk(DevCtx c, PolySeq datas, LimbMap lm, LimbMap pos,
                                                                   u32 logr, u32 n_limbs, u32 n_polys, FwdFuse f) {
   __shared__ u64 lds[kChunk + kChunk / 16];
   u32 chunk, limb, pblk;
@@ -550,7 +562,8 @@ __global__ __launch_bounds__(kChunkThreads, EPI == 1 ? 6 : 8) void ntt_fwd_chunk
 // ---------------------------------------------------------------------------
 // inverse, chunk pass: spans 1..2048 on 4096 contiguous words; src -> dst.
 // Nothing is scaled here: 1/N (times an optional per-limb constant) is applied
-// by the strided pass that always follows.  At span 2^u the stage has
+// by the strided pass that always follows.  The first round works on the eight
+// consecutive words a thread loads itself.  At span 2^u the stage has
 // m = N >> (u+1) groups and element j belongs to group j >> (u+1).  The rounds
 // are those of the forward pass in reverse order.
 template <class A, int SKIP>
@@ -567,31 +580,32 @@ __device__ __forceinline__ void inv_chunk_body(u64* lds_words, const DevCtx& c, 
   ar.init(c, pi, true, nullptr, 0);
   const ChunkMap cm(t);
   const u32 mh = c.N >> 1;  // groups at span 1
+  // a thread reads the eight consecutive words its first round works on (64 bytes, 16-byte loads): no pass
+  // through LDS before the first stage
   u64 raw[8], nxt[8];
-  {
-    const u64* src = srcs.at(poly0);
+  auto load8 = [&](u64* into, u32 poly) {
+    const ulonglong2* src2 = reinterpret_cast<const ulonglong2*>(srcs.at(poly) + off + 8 * t);
 #pragma unroll
-    for (int r = 0; r < 8; ++r) raw[r] = src[off + t + 512 * r];
-  }
+    for (int k = 0; k < 4; ++k) {
+      const ulonglong2 x = src2[k];
+      into[2 * k] = x.x;
+      into[2 * k + 1] = x.y;
+    }
+  };
+  load8(raw, poly0);
   for (u32 it = 0; it < cnt; ++it) {
     u64* dst = dsts.at(poly0 + it);
-    if (it + 1 < cnt) {
-      const u64* src = srcs.at(poly0 + it + 1);
-#pragma unroll
-      for (int r = 0; r < 8; ++r) nxt[r] = src[off + t + 512 * r];
-    }
+    if (it + 1 < cnt) load8(nxt, poly0 + it + 1);
     if (copies.seq.b[0]) {  // the untransformed words are wanted elsewhere too (the digits that Mod_up passes through)
       u64* cp = copies.seq.at(poly0 + it) + (u64)(pos.prime[limb] / copies.part_size) * copies.digit_stride;
+      ulonglong2* cp2 = reinterpret_cast<ulonglong2*>(cp + off + 8 * t);
 #pragma unroll
-      for (int r = 0; r < 8; ++r) cp[off + t + 512 * r] = raw[r];
+      for (int k = 0; k < 4; ++k) cp2[k] = make_ulonglong2(raw[2 * k], raw[2 * k + 1]);
     }
     T v[8];
-#pragma unroll
-    for (int r = 0; r < 8; ++r) lds[cm.wide + ChunkMap::wide_off(r)] = ar.in_canon(raw[r]);
-    __syncthreads();
     // spans 1, 2, 4
 #pragma unroll
-    for (int r = 0; r < 8; ++r) v[r] = lds[cm.narrow + ChunkMap::narrow_off(r)];
+    for (int r = 0; r < 8; ++r) v[r] = ar.in_canon(raw[r]);
     gs_stage<A, 8, 0>(ar, v, (mh >> 0) + (chunk << 11) + ((u32)t << 2));
     gs_stage<A, 8, 1>(ar, v, (mh >> 1) + (chunk << 10) + ((u32)t << 1));
     ar.recentre_sum_of_four(v[0]);
@@ -630,12 +644,13 @@ __device__ __forceinline__ void inv_chunk_body(u64* lds_words, const DevCtx& c, 
     if (!SKIP) gs_stage<A, 8, 2>(ar, v, (mh >> 11) + (chunk << 0));  // else the strided pass runs it as its first
 #pragma unroll
     for (int r = 0; r < 8; ++r) dst[off + t + 512 * r] = ar.out_mid(v[r]);
+    if (kPolysPerBlock > 1) __syncthreads();  // the next polynomial's first round writes words other waves still read
 #pragma unroll
     for (int r = 0; r < 8; ++r) raw[r] = nxt[r];
   }
 }
 template <int SKIP>
-__global__ __launch_bounds__(kChunkThreads, 8) void ntt_inv_chunk(DevCtx c, PolySeq dsts, PolySeq srcs, CopyThrough copies,
+__global__ __launch_bounds__(kChunkThreads, kChunkWaves) void ntt_inv_chunk(DevCtx c, PolySeq dsts, PolySeq srcs, CopyThrough copies,
                                                                   LimbMap lm, LimbMap pos, u32 n_limbs, u32 n_polys) {
   __shared__ u64 lds[kChunk + kChunk / 16];
   u32 chunk, limb, pblk;
@@ -786,6 +801,16 @@ bool launch_ntt(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolyS
   if (pos_in) pos = *pos_in;
   else
     for (u32 t = 0; t < n_limbs; ++t) pos.prime[t] = (uint8_t)t;
+  if (c.logN > kLogChunk) {
+    // the chunk passes move 16 bytes per access: every polynomial must start on a 16-byte boundary (limbs are
+    // multiples of 4096 words apart, so this is a condition on the base pointers and strides only)
+    auto aligned = [](const PolySeq& q) {
+      return (((uintptr_t)q.b[0] | (uintptr_t)q.b[1]) & 15) == 0 && (q.pair_stride & 1) == 0;
+    };
+    if (!aligned(dst) || !aligned(src)) return false;
+    if (f.epi && (!aligned(f.out) || !aligned(f.src) || (f.addend_mode && !aligned(f.addend)))) return false;
+    if (copies.seq.b[0] && (!aligned(copies.seq) || (copies.digit_stride & 1))) return false;
+  }
   if (c.logN <= kLogChunk) {
     hipLaunchKernelGGL(ntt_small, dim3(1, n_limbs, n_polys), dim3(256), 0, st, c, dst, src, lm, pos, inverse ? 1 : 0,
                        scale);
