@@ -566,7 +566,7 @@ __global__ __launch_bounds__(kChunkThreads, kChunkWaves) void ntt_fwd_chunk(DevC
 // consecutive words a thread loads itself.  At span 2^u the stage has
 // m = N >> (u+1) groups and element j belongs to group j >> (u+1).  The rounds
 // are those of the forward pass in reverse order.
-template <class A, int SKIP>
+template <class A, int SKIP, int COPY>
 __device__ __forceinline__ void inv_chunk_body(u64* lds_words, const DevCtx& c, const PolySeq& dsts,
                                                const PolySeq& srcs, const CopyThrough& copies, const LimbMap& pos,
                                                u32 n_polys, u32 chunk, u32 limb, u32 pblk, u32 pi) {
@@ -580,32 +580,46 @@ __device__ __forceinline__ void inv_chunk_body(u64* lds_words, const DevCtx& c, 
   ar.init(c, pi, true, nullptr, 0);
   const ChunkMap cm(t);
   const u32 mh = c.N >> 1;  // groups at span 1
-  // a thread reads the eight consecutive words its first round works on (64 bytes, 16-byte loads): no pass
-  // through LDS before the first stage
+  // A thread reads the eight consecutive words its first round works on (64 bytes, 16-byte loads): no pass
+  // through LDS before the first stage.  Where a copy of the words is wanted as well (the digits that Mod_up
+  // passes through), they are read in the coalesced order instead, copied from registers 512 contiguous bytes per
+  // store (16-byte stores 64 bytes apart are slow) and brought into the first round's order through LDS.
+  constexpr bool copying = COPY != 0;
   u64 raw[8], nxt[8];
   auto load8 = [&](u64* into, u32 poly) {
-    const ulonglong2* src2 = reinterpret_cast<const ulonglong2*>(srcs.at(poly) + off + 8 * t);
+    if (copying) {
+      const u64* src = srcs.at(poly) + off + t;
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const ulonglong2 x = src2[k];
-      into[2 * k] = x.x;
-      into[2 * k + 1] = x.y;
+      for (int r = 0; r < 8; ++r) into[r] = src[512 * r];
+    } else {
+      const ulonglong2* src2 = reinterpret_cast<const ulonglong2*>(srcs.at(poly) + off + 8 * t);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const ulonglong2 x = src2[k];
+        into[2 * k] = x.x;
+        into[2 * k + 1] = x.y;
+      }
     }
   };
   load8(raw, poly0);
   for (u32 it = 0; it < cnt; ++it) {
     u64* dst = dsts.at(poly0 + it);
     if (it + 1 < cnt) load8(nxt, poly0 + it + 1);
-    if (copies.seq.b[0]) {  // the untransformed words are wanted elsewhere too (the digits that Mod_up passes through)
-      u64* cp = copies.seq.at(poly0 + it) + (u64)(pos.prime[limb] / copies.part_size) * copies.digit_stride;
-      ulonglong2* cp2 = reinterpret_cast<ulonglong2*>(cp + off + 8 * t);
-#pragma unroll
-      for (int k = 0; k < 4; ++k) cp2[k] = make_ulonglong2(raw[2 * k], raw[2 * k + 1]);
-    }
     T v[8];
-    // spans 1, 2, 4
+    if (copying) {
+      u64* cp = copies.seq.at(poly0 + it) + (u64)(pos.prime[limb] / copies.part_size) * copies.digit_stride;
 #pragma unroll
-    for (int r = 0; r < 8; ++r) v[r] = ar.in_canon(raw[r]);
+      for (int r = 0; r < 8; ++r) cp[off + t + 512 * r] = raw[r];
+#pragma unroll
+      for (int r = 0; r < 8; ++r) lds[cm.wide + ChunkMap::wide_off(r)] = ar.in_canon(raw[r]);
+      __syncthreads();
+#pragma unroll
+      for (int r = 0; r < 8; ++r) v[r] = lds[cm.narrow + ChunkMap::narrow_off(r)];
+    } else {
+#pragma unroll
+      for (int r = 0; r < 8; ++r) v[r] = ar.in_canon(raw[r]);
+    }
+    // spans 1, 2, 4
     gs_stage<A, 8, 0>(ar, v, (mh >> 0) + (chunk << 11) + ((u32)t << 2));
     gs_stage<A, 8, 1>(ar, v, (mh >> 1) + (chunk << 10) + ((u32)t << 1));
     ar.recentre_sum_of_four(v[0]);
@@ -649,15 +663,15 @@ __device__ __forceinline__ void inv_chunk_body(u64* lds_words, const DevCtx& c, 
     for (int r = 0; r < 8; ++r) raw[r] = nxt[r];
   }
 }
-template <int SKIP>
+template <int SKIP, int COPY>
 __global__ __launch_bounds__(kChunkThreads, kChunkWaves) void ntt_inv_chunk(DevCtx c, PolySeq dsts, PolySeq srcs, CopyThrough copies,
                                                                   LimbMap lm, LimbMap pos, u32 n_limbs, u32 n_polys) {
   __shared__ u64 lds[kChunk + kChunk / 16];
   u32 chunk, limb, pblk;
   if (!chunk_block(c, n_limbs, (n_polys + kPolysPerBlock - 1) / kPolysPerBlock, chunk, limb, pblk)) return;
   const u32 pi = lm.prime[limb];
-  if (c.fp_ok[pi]) inv_chunk_body<ArithFp, SKIP>(lds, c, dsts, srcs, copies, pos, n_polys, chunk, limb, pblk, pi);
-  else inv_chunk_body<ArithInt, SKIP>(lds, c, dsts, srcs, copies, pos, n_polys, chunk, limb, pblk, pi);
+  if (c.fp_ok[pi]) inv_chunk_body<ArithFp, SKIP, COPY>(lds, c, dsts, srcs, copies, pos, n_polys, chunk, limb, pblk, pi);
+  else inv_chunk_body<ArithInt, SKIP, COPY>(lds, c, dsts, srcs, copies, pos, n_polys, chunk, limb, pblk, pi);
 }
 
 // inverse, strided pass: spans 4096..N/2, then scale every word by the limb's
@@ -766,9 +780,14 @@ static void run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst, const
   } else {
     constexpr int LS = LOGR + SI, SHIFT = SI;
     dim3 gs((c.N >> LS) / 256, n_limbs, n_polys);
-    if (passes & 1)
-      hipLaunchKernelGGL((ntt_inv_chunk<SHIFT>), gc, dim3(kChunkThreads), 0, st, c, dst, src, copies, lm, pos, n_limbs,
-                         n_polys);
+    if (passes & 1) {
+      if (copies.seq.b[0])
+        hipLaunchKernelGGL((ntt_inv_chunk<SHIFT, 1>), gc, dim3(kChunkThreads), 0, st, c, dst, src, copies, lm, pos,
+                           n_limbs, n_polys);
+      else
+        hipLaunchKernelGGL((ntt_inv_chunk<SHIFT, 0>), gc, dim3(kChunkThreads), 0, st, c, dst, src, copies, lm, pos,
+                           n_limbs, n_polys);
+    }
     if (passes & 2) {
       u32 n_fp = 0;
       for (u32 t = 0; t < n_limbs; ++t) n_fp += c.fp_ok[lm.prime[t]] ? 1 : 0;
