@@ -835,10 +835,15 @@ bool launch_ntt(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolyS
                        scale);
     return true;
   }
+  // the shifted inverse (see run_large) halves the threads of the strided pass: only for launches that fill the
+  // machine anyway.  The rule depends on the shape of the launch alone, so the two passes of a transform agree
+  // also when a caller runs them apart.
+  const bool big = (u64)n_limbs * n_polys >= 192;
   switch (c.logN - kLogChunk) {
 #define ACE_NTT_CASE(LR, SH)                                                                       \
   case LR:                                                                                         \
-    run_large<LR, 0, SH>(st, c, dst, src, lm, pos, n_limbs, n_polys, inverse, scale, passes, f, copies); \
+    if (SH && big) run_large<LR, 0, SH>(st, c, dst, src, lm, pos, n_limbs, n_polys, inverse, scale, passes, f, copies); \
+    else run_large<LR, 0, 0>(st, c, dst, src, lm, pos, n_limbs, n_polys, inverse, scale, passes, f, copies);          \
     return true;
     ACE_NTT_CASE(1, ACE_NTT_SHIFT)
     ACE_NTT_CASE(2, ACE_NTT_SHIFT)
