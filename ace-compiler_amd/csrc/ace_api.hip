@@ -175,6 +175,9 @@ struct ace_ctx {
   double2* fft_rou = nullptr;       // [2N] exp(2 pi i k / 2N)
   u32* rot_group = nullptr;         // [N/2] 5^k mod 2N
   int* d_err = nullptr;             // sticky device flag of checks that run inside kernels
+  // decoder: inv[L] then garner[L][L] (see crt_to_double), built on first use; Q = q0..q(level-1) per level
+  u64* decode_tab = nullptr;
+  std::map<size_t, u64*> decode_q;
   void check_deferred() {
     int e = 0;
     HIP_OK(hipMemcpyAsync(&e, d_err, sizeof(int), hipMemcpyDeviceToHost, stream));
@@ -1672,6 +1675,61 @@ int ace_embedding_inv(ace_ctx* c, double* host_out, const double* host_in, size_
   HIP_OK(hipMemcpyAsync(r, host_in, len * sizeof(double2), hipMemcpyHostToDevice, c->stream));
   launch_embedding_inv(c->stream, c->d, o, r, c->fft_rou, c->rot_group, (u32)len);
   HIP_OK(hipMemcpyAsync(host_out, o, len * sizeof(double2), hipMemcpyDeviceToHost, c->stream));
+  HIP_OK(hipStreamSynchronize(c->stream));
+  ACE_CATCH_INT
+}
+
+int ace_decode(ace_ctx* c, double* host_out, const int64_t* poly, size_t level, int is_ntt, uint32_t slots,
+               double factor) {
+  ACE_TRY
+  if (!host_out || !poly) return fail("ace_decode: null argument");
+  const size_t N = c->h.N, L = c->h.L;
+  if (!slots) slots = (uint32_t)(N / 2);
+  if (level == 0 || level > L) return fail("ace_decode: level out of range");
+  if (level > (size_t)kDecodeWords) return fail("ace_decode: more than 64 limbs");
+  if (slots > N / 2 || (slots & (slots - 1))) return fail("slot size must be a power of two of at most N/2");
+  if (!(factor > 0.0)) return fail("ace_decode: the scale must be positive");
+  if (!c->decode_tab) {
+    std::vector<u64> tab(L + L * L, 0);
+    for (size_t i = 0; i < L; ++i) {
+      const u64 q = c->h.primes[i].q;
+      u64 prod = 1;
+      for (size_t j = 0; j < i; ++j) {
+        tab[L + i * L + j] = prod;
+        prod = mul_mod(prod, c->h.primes[j].q % q, q);
+      }
+      tab[i] = i ? inv_mod_prime(prod, q) : 1;
+    }
+    c->decode_tab = c->upload_vec(tab);
+  }
+  u64*& big_q = c->decode_q[level];
+  if (!big_q) {
+    std::vector<u64> w(level, 0);
+    w[0] = 1;
+    for (size_t i = 0; i < level; ++i) {
+      unsigned __int128 carry = 0;
+      for (size_t k = 0; k < level; ++k) {
+        unsigned __int128 t = (unsigned __int128)w[k] * c->h.primes[i].q + carry;
+        w[k] = (u64)t;
+        carry = t >> 64;
+      }
+    }
+    big_q = c->upload_vec(w);
+  }
+  c->ensure_ws(c->std_ws(level));
+  c->ws_used = 0;
+  double2* r = reinterpret_cast<double2*>(c->take(2 * (size_t)slots));
+  const u64* coef = U(poly);
+  if (is_ntt) {  // the operand stays as it is
+    u64* tmp = c->take(level * N);
+    if (!launch_ntt(c->stream, c->d, seq_strided(tmp, 0), seq_strided(const_cast<u64*>(U(poly)), 0), c->q_lm, nullptr,
+                    (u32)level, 1, true, nullptr))
+      return fail("ace_decode: ring degree above 2^17, or a polynomial that does not start on a 16-byte boundary");
+    coef = tmp;
+  }
+  launch_decode(c->stream, c->d, r, coef, (u32)level, slots, factor, c->decode_tab, c->decode_tab + L, (u32)L, big_q,
+                c->fft_rou, c->rot_group);
+  HIP_OK(hipMemcpyAsync(host_out, r, slots * sizeof(double2), hipMemcpyDeviceToHost, c->stream));
   HIP_OK(hipStreamSynchronize(c->stream));
   ACE_CATCH_INT
 }

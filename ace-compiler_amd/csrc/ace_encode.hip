@@ -159,4 +159,114 @@ void launch_encode(hipStream_t st, const DevCtx& c, u64* out, double2* r, const 
                      st, c, out, r, slots, logslots, scaling_factor, scale, round_add, range_bound, lm, err);
 }
 
+// ---- decoding (Decode, ckks/src/encoder.c:657-704) ------------------------------------------------------
+// Reconstruct (util/src/crt.c:1247-1275) followed by mpz_get_d: the centred integer behind the residues of one
+// coefficient as a double, truncated towards zero.  Mixed-radix digits (x = d0 + d1 q0 + d2 q0 q1 + ...) from the
+// table garner[i*stride + j] = q0..q(j-1) mod qi and inv[i] = (q0..q(i-1))^-1 mod qi, then the exact value by
+// Horner's rule in `level` 64-bit words (primes are below 2^61, so it fits), compared with Q = q0..q(level-1).
+__device__ double crt_to_double(const DevCtx& c, const u64* __restrict__ poly, u32 coef, u32 level,
+                                const u64* __restrict__ inv, const u64* __restrict__ garner, u32 stride,
+                                const u64* __restrict__ big_q) {
+  u64 d[kDecodeWords], x[kDecodeWords];
+  for (u32 i = 0; i < level; ++i) {
+    const DevPrime p = c.primes[i];
+    u64 hi = 0, lo = 0;
+    for (u32 j = 0; j < i; ++j) mac128(hi, lo, d[j], garner[(u64)i * stride + j]);
+    const u64 acc = barrett128(hi, lo, p);
+    u64 v = poly[(u64)i * c.N + coef];
+    if (v >= p.q) v %= p.q;
+    const u64 t = v >= acc ? v - acc : v + p.q - acc;
+    d[i] = i ? mulmod(t, inv[i], p) : t;
+  }
+  for (u32 k = 0; k < level; ++k) x[k] = 0;
+  for (u32 i = level; i-- > 0;) {  // x = x * q_i + d_i
+    const u64 q = c.primes[i].q;
+    u64 carry = d[i];
+    for (u32 k = 0; k < level; ++k) {
+      const u64 lo = x[k] * q, hi = __umul64hi(x[k], q), s = lo + carry;
+      x[k] = s;
+      carry = hi + (s < lo);
+    }
+  }
+  // negative when 2x > Q (Q is odd); 2x still fits the words: x < 2^(61 level)
+  bool neg = false;
+  for (u32 k = level; k-- > 0;) {
+    const u64 twice = (x[k] << 1) | (k ? x[k - 1] >> 63 : 0);
+    if (twice != big_q[k]) {
+      neg = twice > big_q[k];
+      break;
+    }
+  }
+  if (neg) {  // x = Q - x
+    u64 borrow = 0;
+    for (u32 k = 0; k < level; ++k) {
+      const u64 a = big_q[k], b = x[k], t = a - b - borrow;
+      borrow = (a < b) || (a == b && borrow);
+      x[k] = t;
+    }
+  }
+  u32 top = level;
+  while (top > 0 && x[top - 1] == 0) --top;
+  if (!top) return 0.0;
+  const u32 hb = 63 - (u32)__clzll((long long)x[top - 1]), bitlen = (top - 1) * 64 + hb + 1;
+  double r;
+  if (bitlen <= 53) {
+    r = (double)x[0];
+  } else {  // the 53 leading bits, the rest cut off
+    const u32 sh = bitlen - 53, w = sh / 64, b = sh % 64;
+    u64 m = x[w] >> b;
+    if (b && w + 1 < top) m |= x[w + 1] << (64 - b);
+    m &= ((u64)1 << 53) - 1;
+    r = ldexp((double)m, (int)sh);
+  }
+  return neg ? -r : r;
+}
+
+// thread n < slots: the real part of slot n (coefficient n*gap), n >= slots: the imaginary part (coefficient
+// (n-slots)*gap + N/2); each divided by the plaintext's scale and stored where the embedding's bit reversal
+// wants it
+__global__ __launch_bounds__(kEncThreads) void decode_crt_kernel(DevCtx c, double2* __restrict__ r,
+                                                                 const u64* __restrict__ poly, u32 level, u32 slots,
+                                                                 u32 logslots, double factor,
+                                                                 const u64* __restrict__ inv,
+                                                                 const u64* __restrict__ garner, u32 stride,
+                                                                 const u64* __restrict__ big_q) {
+  const u32 n = blockIdx.x * kEncThreads + threadIdx.x;
+  if (n >= 2 * slots) return;
+  const bool imag = n >= slots;
+  const u32 i = imag ? n - slots : n, gap = c.N / (2 * slots);
+  const double v = crt_to_double(c, poly, i * gap + (imag ? c.N / 2 : 0), level, inv, garner, stride, big_q) / factor;
+  double* out = reinterpret_cast<double*>(r + (logslots ? (__brev(i) >> (32 - logslots)) : 0));
+  out[imag ? 1 : 0] = v;
+}
+
+// stage logm of Embedding (util/src/ntt.c:598-629) on bit-reversed input: (x, y) -> (x + w y, x - w y)
+__global__ __launch_bounds__(kEncThreads) void embed_fwd_stage_kernel(double2* __restrict__ r,
+                                                                      const double2* __restrict__ rou,
+                                                                      const u32* __restrict__ rot, u32 M, u32 logm,
+                                                                      u32 len) {
+#pragma clang fp contract(off)
+  const u32 t = blockIdx.x * kEncThreads + threadIdx.x;
+  if (t >= (len >> 1)) return;
+  const u32 num = 1u << (logm - 1), i = t & (num - 1), ie = ((t >> (logm - 1)) << logm) | i, io = ie + num;
+  const u32 idx_mod = 1u << (logm + 2), gap = M / idx_mod;
+  const double2 w = rou[(rot[i] & (idx_mod - 1)) * gap], x = r[ie], y = r[io];
+  const double pr = w.x * y.x, qr = w.y * y.y, pi = w.x * y.y, qi = w.y * y.x;
+  const double omr = pr - qr, omi = pi + qi;
+  r[ie] = make_double2(x.x + omr, x.y + omi);
+  r[io] = make_double2(x.x - omr, x.y - omi);
+}
+
+void launch_decode(hipStream_t st, const DevCtx& c, double2* r, const u64* poly, u32 level, u32 slots, double factor,
+                   const u64* inv, const u64* garner, u32 stride, const u64* big_q, const double2* rou,
+                   const u32* rot) {
+  u32 logslots = 0;
+  while ((1u << logslots) < slots) ++logslots;
+  hipLaunchKernelGGL(decode_crt_kernel, dim3((2 * slots + kEncThreads - 1) / kEncThreads), dim3(kEncThreads), 0, st, c,
+                     r, poly, level, slots, logslots, factor, inv, garner, stride, big_q);
+  for (u32 logm = 1; logm <= logslots; ++logm)
+    hipLaunchKernelGGL(embed_fwd_stage_kernel, dim3(((slots >> 1) + kEncThreads - 1) / kEncThreads),
+                       dim3(kEncThreads), 0, st, r, rou, rot, 2 * c.N, logm, slots);
+}
+
 }  // namespace ace

@@ -177,5 +177,10 @@ void launch_widen_real(hipStream_t st, double2* z, const void* raw, bool is_f32,
 void launch_encode(hipStream_t st, const DevCtx& c, u64* out, double2* r, const double2* rou, const u32* rot,
                    u32 slots, double scaling_factor, double scale, double round_add, double range_bound,
                    const LimbMap& lm, u32 n_limbs, int* err);
+constexpr int kDecodeWords = 64;  // most limbs of a polynomial the decoder reconstructs
+// Decode (ckks/src/encoder.c:657-704) of a polynomial in coefficient form: r receives the `slots` complex values
+void launch_decode(hipStream_t st, const DevCtx& c, double2* r, const u64* poly, u32 level, u32 slots, double factor,
+                   const u64* inv, const u64* garner, u32 stride, const u64* big_q, const double2* rou,
+                   const u32* rot);
 
 }  // namespace ace

@@ -223,12 +223,8 @@ void Rt_ckks_finalize(void) {
   if (G.secret_ntt) Rt_dev_free(G.secret_ntt);
   if (G.pk0) Rt_dev_free(G.pk0);
   if (G.pk1) Rt_dev_free(G.pk1);
-  free(G.fft_rou);
-  free(G.rot_group);
   G.secret_small = NULL;
   G.secret_ntt = G.pk0 = G.pk1 = NULL;
-  G.fft_rou   = NULL;
-  G.rot_group = NULL;
 }
 
 /* ---- plaintexts ------------------------------------------------------------------------------------- */
@@ -474,157 +470,13 @@ void Rt_decrypt(PLAIN res, CIPHER c) {
   ACE_OK(ace_poly_add(G.ctx, res->_poly._data, res->_poly._data, c->_c0_poly._data, level, 0));
 }
 
-/* ---- decoding (ckks/src/encoder.c:657-704, util/src/crt.c:1247-1275, util/src/ntt.c:598-629) ---------- */
-typedef unsigned __int128 u128;
-static uint64_t mulmod64(uint64_t a, uint64_t b, uint64_t q) { return (uint64_t)((u128)a * b % q); }
-static uint64_t powmod64(uint64_t a, uint64_t e, uint64_t q) {
-  uint64_t r = 1;
-  for (a %= q; e; e >>= 1, a = mulmod64(a, a, q))
-    if (e & 1) r = mulmod64(r, a, q);
-  return r;
-}
-
-/* the centred integer with residues v[0..level) as a double, truncated towards zero like
- * mpz_get_d: mixed-radix digits, exact multi-word evaluation, comparison with Q/2 */
-static double crt_to_double(const int64_t* v, size_t level, const uint64_t* inv /* [level]: (q_0..q_{i-1})^-1 mod q_i */) {
-  uint64_t d[64];
-  FMT_ASSERT(level <= 64, "decoding supports at most 64 limbs, the ciphertext has %zu", level);
-  for (size_t i = 0; i < level; ++i) {
-    uint64_t q = (uint64_t)G.q[i]._val, acc = 0, prod = 1;
-    for (size_t j = 0; j < i; ++j) {
-      acc  = (acc + mulmod64(d[j] % q, prod, q)) % q;
-      prod = mulmod64(prod, (uint64_t)G.q[j]._val % q, q);
-    }
-    uint64_t t = ((uint64_t)v[i] % q + q - acc) % q;
-    d[i]       = i ? mulmod64(t, inv[i], q) : t;
-  }
-  uint64_t x[66] = {0}, Q[66] = {0}, x2[67] = {0};
-  size_t   nx = 1, nQ = 1;
-  Q[0]        = 1;
-  for (size_t i = level; i-- > 0;) { /* Horner from the top digit */
-    u128 carry = 0;
-    for (size_t k = 0; k < nx; ++k) {
-      u128 p = (u128)x[k] * (uint64_t)G.q[i]._val + carry;
-      x[k]   = (uint64_t)p;
-      carry  = p >> 64;
-    }
-    if (carry) x[nx++] = (uint64_t)carry;
-    u128 a = (u128)x[0] + d[i];
-    x[0]   = (uint64_t)a;
-    for (size_t k = 1; (a >> 64) && k <= nx; ++k) {
-      a    = (u128)x[k] + 1;
-      x[k] = (uint64_t)a;
-      if (k == nx) nx++;
-    }
-  }
-  for (size_t i = 0; i < level; ++i) {
-    u128 carry = 0;
-    for (size_t k = 0; k < nQ; ++k) {
-      u128 p = (u128)Q[k] * (uint64_t)G.q[i]._val + carry;
-      Q[k]   = (uint64_t)p;
-      carry  = p >> 64;
-    }
-    if (carry) Q[nQ++] = (uint64_t)carry;
-  }
-  size_t n = nQ > nx ? nQ : nx;
-  for (size_t k = 0; k < n; ++k) x2[k] = (x[k] << 1) | (k ? x[k - 1] >> 63 : 0);
-  x2[n]   = x[n - 1] >> 63;
-  int neg = x2[n] != 0;
-  if (!neg)
-    for (size_t k = n; k-- > 0;)
-      if (x2[k] != Q[k]) {
-        neg = x2[k] > Q[k];
-        break;
-      }
-  if (neg) {
-    uint64_t borrow = 0;
-    for (size_t k = 0; k < n; ++k) {
-      u128 t = (u128)Q[k] - x[k] - borrow;
-      x[k]   = (uint64_t)t;
-      borrow = (uint64_t)(t >> 64) & 1;
-    }
-  }
-  size_t top = n;
-  while (top > 0 && x[top - 1] == 0) top--;
-  if (!top) return 0.0;
-  int    hb     = 63 - __builtin_clzll(x[top - 1]);
-  size_t bitlen = (top - 1) * 64 + (size_t)hb + 1;
-  double r;
-  if (bitlen <= 53) {
-    r = (double)x[0];
-  } else {
-    size_t   sh = bitlen - 53, w = sh / 64, b = sh % 64;
-    uint64_t m  = x[w] >> b;
-    if (b && w + 1 < top) m |= x[w + 1] << (64 - b);
-    m &= ((uint64_t)1 << 53) - 1;
-    r = ldexp((double)m, (int)sh);
-  }
-  return neg ? -r : r;
-}
-
-static void need_fft_tables(void) {
-  if (G.fft_rou) return;
-  G.fft_rou   = (double*)malloc(4 * (size_t)G.N * sizeof(double));
-  G.rot_group = (uint32_t*)malloc((G.N / 2 ? G.N / 2 : 1) * sizeof(uint32_t));
-  ACE_OK(ace_host_fft_tables(G.ctx, G.fft_rou, G.rot_group));
-}
-
-/* Embedding (util/src/ntt.c:598-629) on the host */
-static void embedding(DCMPLX* res, const DCMPLX* coeffs, size_t len) {
-  need_fft_tables();
-  size_t M = 2 * (size_t)G.N, logn = 0;
-  while (((size_t)1 << logn) < len) logn++;
-  for (size_t i = 0; i < len; ++i) {
-    size_t r = 0;
-    for (size_t b = 0; b < logn; ++b) r |= ((i >> b) & 1) << (logn - 1 - b);
-    res[i] = coeffs[r];
-  }
-  for (size_t logm = 1; logm < logn + 1; ++logm) {
-    size_t idx_mod = (size_t)1 << (logm + 2), gap = M / idx_mod, num = (size_t)1 << (logm - 1);
-    for (size_t j = 0; j < len; j += (size_t)1 << logm)
-      for (size_t i = 0; i < num; ++i) {
-        size_t ie = j + i, io = ie + num, ri = ((size_t)G.rot_group[i] % idx_mod) * gap;
-        DCMPLX om = (G.fft_rou[2 * ri] + G.fft_rou[2 * ri + 1] * I) * res[io];
-        DCMPLX plus = res[ie] + om, minus = res[ie] - om;
-        res[ie] = plus;
-        res[io] = minus;
-      }
-  }
-}
-
+/* ---- decoding (ckks/src/encoder.c:657-704): Reconstruct, the conversion to double and the embedding run on the
+ * device (ace_decode); only the slots' complex numbers come back ------------------------------------------ */
 void Rt_decode(DCMPLX* res, PLAIN plain) {
-  POLY     p = &plain->_poly;
-  size_t   level = p->_num_primes, n = G.N, half = n / 2;
-  uint32_t slots = plain->_slots ? plain->_slots : (uint32_t)half, gap = (uint32_t)(half / slots);
-  int64_t* host = (int64_t*)malloc(level * n * sizeof(int64_t));
-  if (p->_is_ntt) { /* the plaintext itself stays as it is */
-    int32_t idx[128];
-    for (size_t t = 0; t < level; ++t) idx[t] = (int32_t)t;
-    int64_t* tmp = Rt_dev_alloc(level * n);
-    ACE_OK(ace_intt(G.ctx, tmp, p->_data, idx, level, 1, 0));
-    ACE_OK(ace_download(G.ctx, host, tmp, level * n));
-    Rt_dev_free(tmp);
-  } else {
-    ACE_OK(ace_download(G.ctx, host, p->_data, level * n));
-  }
-  uint64_t inv[64];
-  for (size_t i = 1; i < level; ++i) {
-    uint64_t q = (uint64_t)G.q[i]._val, prod = 1;
-    for (size_t j = 0; j < i; ++j) prod = mulmod64(prod, (uint64_t)G.q[j]._val % q, q);
-    inv[i] = powmod64(prod, q - 2, q);
-  }
-  DCMPLX* msg = (DCMPLX*)malloc(slots * sizeof(DCMPLX));
-  int64_t v[64];
-  for (uint32_t i = 0; i < slots; ++i) {
-    for (size_t t = 0; t < level; ++t) v[t] = host[t * n + (size_t)i * gap];
-    double re = crt_to_double(v, level, inv) / plain->_scaling_factor;
-    for (size_t t = 0; t < level; ++t) v[t] = host[t * n + (size_t)i * gap + half];
-    double im = crt_to_double(v, level, inv) / plain->_scaling_factor;
-    msg[i]    = re + im * I;
-  }
-  embedding(res, msg, slots);
-  free(msg);
-  free(host);
+  POLY     p     = &plain->_poly;
+  uint32_t slots = plain->_slots ? plain->_slots : (uint32_t)(G.N / 2);
+  FMT_ASSERT(p->_num_primes_p == 0, "decoding an extended plaintext is not supported");
+  ACE_OK(ace_decode(G.ctx, (double*)res, p->_data, p->_num_primes, p->_is_ntt, slots, plain->_scaling_factor));
 }
 
 DCMPLX* Get_dcmplx_msg_from_plain(PLAIN plain) {

@@ -42,8 +42,6 @@ struct rt_state {
   int64_t* secret_small; /* host: N signed coefficients */
   int64_t* secret_ntt;   /* device: (L+k) limbs */
   int64_t *pk0, *pk1;    /* device: L limbs each */
-  double*   fft_rou;     /* host: 2N (cos, sin) pairs */
-  uint32_t* rot_group;   /* host: N/2 powers of 5 */
 };
 extern struct rt_state G;
 

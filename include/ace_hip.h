@@ -211,6 +211,13 @@ int ace_reduce_rescale_modup(ace_ctx* ctx, int64_t* res, int64_t* raised, int64_
 int ace_transform_from_level0(ace_ctx* ctx, int64_t* res, const int64_t* src, size_t level);
 /* Embedding_inv (util/src/ntt.c:631-675) on `len` complex numbers, host to host through the device */
 int ace_embedding_inv(ace_ctx* ctx, double* host_out, const double* host_in, size_t len);
+/* Decode (ckks/src/encoder.c:657-704): the message of a plaintext polynomial at `level` (NTT or coefficient form,
+ * left unchanged): Reconstruct (util/src/crt.c:1247-1275) of the coefficients the slots use to centred integers, their
+ * conversion to double as mpz_get_d truncates, division by `factor` (the plaintext's scale) and Embedding
+ * (util/src/ntt.c:598-629), all on the device.  host_out receives `slots` complex numbers (re, im interleaved);
+ * slots = 0 means N/2.  Synchronises.  At most 64 limbs. */
+int ace_decode(ace_ctx* ctx, double* host_out, const int64_t* poly, size_t level, int is_ntt, uint32_t slots,
+               double factor);
 /* Encode_impl (ckks/src/encoder.c:234-326; Encode_at_level_with_sf, Encode_ext_at_level): `values` is a
  * HOST array of n_values complex numbers (re, im interleaved), zero-padded to `slots` (0: N/2); the
  * plaintext polynomial lands in res: level (0: all) Q limbs followed by p_cnt (0 or num_p) P limbs, NTT

@@ -439,6 +439,50 @@ def test_mod_down_rescale_family(pair):
         g.mod_down_rescale(g.alloc(N), g.alloc(N), 1, True)
 
 
+def test_decode(pair):
+    """Device decoder vs the oracle's (itself matched against the reference's compiled Decode): the same doubles.
+    Operands: encoded messages (small centred values), and uniformly random residues (integers as large as Q, both
+    signs, every word of the multi-word reconstruction in use), in NTT and in coefficient form."""
+    g, o = pair.g, pair.o
+    N, (q0_bits, sf_bits) = g.N, pair.cfg[2:4]
+    rng = np.random.default_rng(N + 5)
+    for slots in sorted({N // 2, max(1, N // 8), min(4, N // 2), 1}):
+        z = rng.uniform(-1, 1, slots) + 1j * rng.uniform(-1, 1, slots)
+        for level in sorted({g.L, min(2, g.L), 1, max(1, g.L - 1)}):
+            if sf_bits >= q0_bits + (level - 1) * sf_bits:
+                continue
+            enc = o.encode(z, slots, level, 1, 0)
+            factor = 2.0 ** sf_bits
+            got = g.decode(g.upload(enc), level, slots, factor, True)
+            want = o.decode(enc, level, slots, factor, True)
+            assert np.array_equal(got.view(np.uint64), want.view(np.uint64)), "decode slots=%d level=%d" % (slots, level)
+            assert np.abs(got - z).max() < 1e-6
+            noise = np.concatenate([rng.integers(0, q, N, dtype=np.int64) for q in g.primes[:level]])
+            for is_ntt in (True, False):
+                d = g.upload(noise)
+                got = g.decode(d, level, slots, factor * 3.0, is_ntt)
+                want = o.decode(noise, level, slots, factor * 3.0, is_ntt)
+                assert np.array_equal(got.view(np.uint64), want.view(np.uint64)), "decode of random residues slots=%d level=%d ntt=%d" % (slots, level, is_ntt)
+                assert np.array_equal(d.get(), noise)  # the operand is left as it was
+    # the integers at the sign change and the ends of the range: x = 0, 1, (Q-1)/2, (Q+1)/2, Q-1
+    level = g.L
+    Q = 1
+    for q in g.primes[:level]:
+        Q *= int(q)
+    vals = [0, 1, (Q - 1) // 2, (Q + 1) // 2, Q - 1, Q // 3][:N]
+    poly = np.zeros((level, N), np.int64)
+    for k, v in enumerate(vals):
+        for t, q in enumerate(g.primes[:level]):
+            poly[t, k] = v % int(q)
+    got = g.decode(g.upload(poly.reshape(-1)), level, N // 2, 1.0, False)
+    want = o.decode(poly.reshape(-1), level, N // 2, 1.0, False)
+    assert np.array_equal(got.view(np.uint64), want.view(np.uint64))
+    with pytest.raises(acefhe.AceError):
+        g.decode(g.upload(poly.reshape(-1)), g.L + 1, 0, 1.0, False)
+    with pytest.raises(acefhe.AceError):
+        g.decode(g.upload(poly.reshape(-1)), 1, 3, 1.0, False)
+
+
 def test_encode(pair):
     """Device encoder vs the oracle's (itself matched against the reference's compiled encoder): same residues."""
     g, o = pair.g, pair.o
