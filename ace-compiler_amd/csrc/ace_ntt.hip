@@ -70,6 +70,7 @@ __device__ __forceinline__ void wave_sync() {
 // ---------------------------------------------------------------------------
 struct ArithInt {
   typedef u64 T;
+  static constexpr bool kFp = false;
   u64 q, q2, q4;
   const u64 *w, *wp;  // twiddle, Shoup companion
   u64 sc, scp;        // inverse: final scale constant
@@ -129,6 +130,7 @@ struct ArithInt {
 
 struct ArithFp {
   typedef double T;
+  static constexpr bool kFp = true;
   double q, qinv;
   const double* w;  // twiddles as exact FP64 integers
   double sc, sci;
@@ -295,6 +297,24 @@ __device__ __forceinline__ void fwd_strided_body(const DevCtx& c, const PolySeq&
     const u64 ql = c.primes[f.last_prime].q, half = ql >> 1;
     const u64 K = f.sw[3 * lt], Kp = f.sw[3 * lt + 1], diff = f.sw[3 * lt + 2];
     const u64* __restrict__ last = f.last + blockIdx.z * f.last_stride + col;
+    if constexpr (A::kFp) {
+      // Both primes small enough for FP64: the centred value of the last limb's word (|x| <= ql/2 <= q) times the
+      // centred constant is one exact FP64 product, about a fifth of the integer path's instructions; its result
+      // (below 0.72 q) is what the stages take.
+      if (ql < ((u64)1 << 52) && ql <= 2 * P.q) {
+        const double qld = (double)ql, halfd = (double)half;
+        double kc = ar.in_canon(K);
+        if (K > (P.q >> 1)) kc -= ar.q;
+        const double kci = kc * ar.qinv;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          double x = ar.in_canon(last[r * rs]);
+          x = x > halfd ? x - qld : x;
+          v[r] = ar.mulmod(x, kc, kci);
+        }
+        goto stages;
+      }
+    }
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       u64 x = last[r * rs];
@@ -307,6 +327,7 @@ __device__ __forceinline__ void fwd_strided_body(const DevCtx& c, const PolySeq&
       v[r] = ar.in_canon(shoup_mul(x, K, Kp, P.q));
     }
   }
+stages:
   fwd_strided_stages<A, LOGR>(ar, v);
   // this pass is bound by HBM and has instruction slots to spare: it hands centred values to the chunk pass,
   // which then runs its first two rounds (six stages) without reducing
