@@ -911,7 +911,7 @@ static void finish(CIPHER res) {
   while (res->_sf_degree > 1) rescale(res);
 }
 
-CIPHER Eval_bootstrap_ciph(CIPHER res, CIPHER ct, uint32_t level_after_bts, uint32_t num_slots) {
+static CIPHER eval_bootstrap(CIPHER res, CIPHER ct, uint32_t level_after_bts, uint32_t num_slots) {
   NEED_CTX();
   FMT_ASSERT(Level(ct) > 0, "Input cipher level is exhausted");
   uint32_t    slots = num_slots ? num_slots : (ct->_slots ? ct->_slots : (uint32_t)(G.N / 2));
@@ -965,6 +965,13 @@ CIPHER Eval_bootstrap_ciph(CIPHER res, CIPHER ct, uint32_t level_after_bts, uint
   Free_ciph_poly(&sub, 1);
   if (res->_c0_poly._data) Free_ciph_poly(res, 1);
   *res = work;
+  return res;
+}
+
+CIPHER Eval_bootstrap_ciph(CIPHER res, CIPHER ct, uint32_t level_after_bts, uint32_t num_slots) {
+  RTLIB_TM_START(RTM_BOOTSTRAP, rtm);
+  eval_bootstrap(res, ct, level_after_bts, num_slots);
+  RTLIB_TM_END(RTM_BOOTSTRAP, rtm);
   return res;
 }
 

@@ -604,17 +604,6 @@ CIPHER Real_relu(CIPHER c) {
   free(m);
   return res;
 }
-void Validate_impl(double* res, double* msg, uint32_t len, int32_t epsilon) {
-  double error = pow(10, epsilon);
-  for (uint32_t i = 0; i < len; ++i)
-    if (fabs(res[i] - msg[i]) > error) Rt_fatal(__FILE__, __LINE__, "ERROR: validation failed at %u. %f != %f", i, res[i], msg[i]);
-}
-void Validate(CIPHER c, double* msg, uint32_t len, int32_t epsilon) {
-  double* res = Get_msg(c);
-  Validate_impl(res, msg, len, epsilon);
-  free(res);
-}
-
 /* ---- tensors, program inputs and outputs (common/tensor.h, ckks/src/rtlib.c:66-229) ---------------- */
 TENSOR* Alloc_tensor(size_t n, size_t c, size_t h, size_t w, const double* val) {
   size_t  len = n * c * h * w;

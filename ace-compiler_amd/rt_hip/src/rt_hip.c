@@ -88,12 +88,16 @@ void Finalize_context(void) {
   free(G.q);
   ace_ctx_destroy(G.ctx);
   memset(&G, 0, sizeof(G));
+  Report_rtlib_timing(); /* ckks_context.c:207-210: the table of times, if the environment asks for one */
+  Close_trace_file();
 }
 
 void Run_main_graph(void) {
   NEED_CTX();
   FMT_ASSERT(Main_graph, "the program does not define Main_graph()");
+  RTLIB_TM_START(RTM_MAIN_GRAPH, rtm);
   FMT_ASSERT(Main_graph(), "Main_graph() reported failure");
+  RTLIB_TM_END(RTM_MAIN_GRAPH, rtm);
 }
 
 /* ---- context getters ----------------------------------------------------------- */

@@ -211,6 +211,36 @@ def test_reference_resnet20_program_runs_on_its_compiled_in_chain():
     assert len(out) == 10 and all(v == v and abs(v) != float("inf") for v in map(float, out))
 
 
+CONV_PROGRAMS = ["conv_3x16x32x3", "conv_16x16x32x3", "conv_32x32x16x3", "conv_64x64x8x3", "conv_128x128x28x3",
+                 "conv_256x256x14x3", "conv_512x512x7x3"]
+
+
+@pytest.mark.parametrize("name", CONV_PROGRAMS)
+def test_reference_conv_programs_run(name, tmp_path):
+    """The reference's single-layer convolution programs (rtlib/ant/dataset/conv_*.cxx: the compiler's output plus a
+    driver with the input, the expected output and, in three of them, the comparison), built unchanged, run to the end.  Their
+    weight files are not in the reference tree, so the weights are pseudo-random and the comparison with the expected
+    output cannot succeed: what is checked is that every runtime call of these programs is there and works (they
+    use the per-event timing marks, whose table must list the convolution), and that the output is finite."""
+    exe = os.path.join(rt_program.ROOT, "oracle", "_ref", "models", name)
+    if not os.path.exists(exe):
+        pytest.skip("built only where the reference tree is present")
+    table = tmp_path / "timing.txt"
+    env = dict(os.environ, RT_HIP_SYNTHETIC_WEIGHTS="0.05", RTLIB_TIMING_OUTPUT=str(table), PRINT_ALL="1")
+    print("running", exe, flush=True)
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=200, env=env)
+    assert r.returncode in (0, 1), r.stdout[-1500:] + r.stderr[-1500:]
+    # some of the drivers have their comparison commented out and only run the graph
+    if "expect absolute error" in r.stdout:
+        assert "FAILED!" in r.stdout or "SUCCESS!" in r.stdout, r.stdout[-1500:]
+        values = [float(l.split("result: ")[1].split(",")[0]) for l in r.stdout.splitlines() if l.startswith("index: ") and "result: " in l]
+        assert len(values) >= 1024 and all(v == v and abs(v) < 1e6 for v in values)
+    else:
+        assert r.returncode == 0
+    text = table.read_text()
+    assert "RTLib functions" in text and "NN_CONV" in text, text
+
+
 MSG = os.path.join(rt_program.ROOT, "tests", "programs", "msg_program")
 
 
