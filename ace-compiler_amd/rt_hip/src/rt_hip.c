@@ -105,6 +105,9 @@ uint32_t Degree(void) { return G.N; }
 size_t   Get_q_cnt(void) { return G.L; }
 size_t   Get_p_cnt(void) { return G.K; }
 size_t   Get_q_parts(void) { return G.parts; }
+CRT_CONTEXT* Get_crt_context(void) { return G.ctx; }
+NTT_CONTEXT* Get_ntt_ctx(void) { return G.ctx; }
+size_t       Get_part_size(void) { return G.ctx ? ace_part_size(G.ctx) : 0; }
 MODULUS* Q_modulus(void) { return G.q; }
 MODULUS* P_modulus(void) { return G.p; }
 double   Get_default_sc(void) { return G.sc; }
