@@ -30,7 +30,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 # HBM bytes per launch of each NTT kernel on this workload, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs of this script, calibrated against the plain copy of the same buffer
 # (profiles/ntt_batch_N65536_L24.md).  Algorithmic bytes per launch are 805306368.
-TRAFFIC_BYTES = {'ntt_fwd_strided': 805563376, 'ntt_fwd_chunk': 818312660, 'ntt_inv_chunk': 818259824, 'ntt_inv_strided': 806260884}
+TRAFFIC_BYTES = {'ntt_fwd_strided': 805492216, 'ntt_fwd_chunk': 818298120, 'ntt_inv_chunk': 818245899, 'ntt_inv_strided': 805688097}
 N, LIMBS, POLYS = 65536, 24, 32
 CFG = (N, LIMBS, 50, 50, 3)
 
