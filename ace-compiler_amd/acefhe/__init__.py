@@ -73,6 +73,8 @@ def _sig(lib):
     f("ace_mod_up", C.c_int, _vp, _vp, _vp, _sz, _sz, C.c_int)
     f("ace_host_fft_tables", C.c_int, _vp, _vp, _vp)
     f("ace_embedding_inv", C.c_int, _vp, _vp, _vp, _sz)
+    for n in ("ace_fork", "ace_fork_switch", "ace_join"):
+        f(n, C.c_int, _vp)
     f("ace_decode", C.c_int, _vp, _vp, _vp, _sz, C.c_int, C.c_uint32, C.c_double)
     f("ace_encode", C.c_int, _vp, _vp, _vp, _sz, C.c_uint32, _sz, C.c_uint32, _sz)
     f("ace_ext_plain_mac_groups", C.c_int, _vp, _vp, _vp, _sz, _vp, _vp, _sz, _vp, _sz, _sz)
@@ -117,7 +119,7 @@ EXPORTS = [
     "ace_hw_modsub_scalar", "ace_hw_modmul_scalar", "ace_hw_modmuladd_scalar", "ace_hw_rotate",
     "ace_find_automorphism_index", "ace_automorphism_order", "ace_poly_add", "ace_poly_sub", "ace_poly_mul",
     "ace_poly_automorphism", "ace_decomp_modup", "ace_mod_up", "ace_mod_down_rescale",
-    "ace_reduce_rescale_modup", "ace_transform_from_level0", "ace_host_fft_tables", "ace_embedding_inv", "ace_decode", "ace_encode", "ace_encode_scaled", "ace_encode_real", "ace_ext_rotate", "ace_ext_plain_mac_groups", "ace_precomp", "ace_mod_down", "ace_rescale", "ace_extend",
+    "ace_reduce_rescale_modup", "ace_transform_from_level0", "ace_host_fft_tables", "ace_embedding_inv", "ace_decode", "ace_fork", "ace_fork_switch", "ace_join", "ace_encode", "ace_encode_scaled", "ace_encode_real", "ace_ext_rotate", "ace_ext_plain_mac_groups", "ace_precomp", "ace_mod_down", "ace_rescale", "ace_extend",
     "ace_dot_prod", "ace_mul_ciph3", "ace_fast_switch_key", "ace_relin", "ace_rescale_ciph",
     "ace_mul_relin_rescale", "ace_mul_relin_rescale_batch", "ace_fast_rotate", "ace_rotate_batch",
 ]
@@ -260,6 +262,15 @@ class Context:
 
     def copy(self, dst, src, n_words=None):
         self._chk(self.lib.ace_copy(self.h, dst.ptr, src.ptr, src.n if n_words is None else n_words))
+
+    def fork(self):
+        self._chk(self.lib.ace_fork(self.h))
+
+    def fork_switch(self):
+        self._chk(self.lib.ace_fork_switch(self.h))
+
+    def join(self):
+        self._chk(self.lib.ace_join(self.h))
 
     def sync(self):
         self._chk(self.lib.ace_sync(self.h))

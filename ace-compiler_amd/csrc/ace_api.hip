@@ -114,7 +114,7 @@ struct ace_ctx {
     hipEvent_t done = nullptr;
     bool pending = false;
   };
-  static constexpr int kStages = 16;
+  static constexpr int kStages = 256;
   Stage stages[kStages];
   int next_stage = 0;
   void h2d(void* dev_dst, const void* src, size_t bytes) {
@@ -205,6 +205,30 @@ struct ace_ctx {
   u64* ws = nullptr;
   size_t ws_words = 0, ws_used = 0;
   u64* static_scratch = nullptr;  // this GPU's copy of the device array `scratch` (ace_mod_down_noalloc)
+  // A second lane for calls that may overlap with those of the first (ace_fork / ace_fork_switch / ace_join): its
+  // own stream (same priority), scratch arena, buffer pool and run image; everything else (tables, the map of live
+  // buffers) is shared.  `idle` holds the lane that is not in use; swapping makes every entry point work on the other
+  // lane without knowing.  A buffer freed on a lane joins that lane's pool, so its next use is ordered on the stream
+  // that last touched it (or on one that has waited for it at the fork or the join).
+  struct Lane {
+    hipStream_t stream = nullptr;
+    u64* ws = nullptr;
+    size_t ws_words = 0, ws_used = 0;
+    std::multimap<size_t, void*> pool;
+    size_t pooled_words = 0;
+    BatchOpDev* run_dev = nullptr;
+  } idle;
+  int fork_state = 0;  // 0 one lane; 1 issuing on the second lane; 2 back on the first, the second's work in flight
+  hipEvent_t fork_ev = nullptr, join_ev = nullptr;
+  void swap_lanes() {
+    std::swap(stream, idle.stream);
+    std::swap(ws, idle.ws);
+    std::swap(ws_words, idle.ws_words);
+    std::swap(ws_used, idle.ws_used);
+    std::swap(pool, idle.pool);
+    std::swap(pooled_words, idle.pooled_words);
+    std::swap(run_dev, idle.run_dev);
+  }
 
   template <class T>
   T* upload_vec(const std::vector<T>& v) {
@@ -458,8 +482,15 @@ struct ace_ctx {
       if (st.host) (void)hipHostFree(st.host);
       if (st.done) (void)hipEventDestroy(st.done);
     }
+    if (fork_state == 1) swap_lanes();  // destroyed in the middle of a fork: back to the first lane
+    if (idle.stream) (void)hipStreamSynchronize(idle.stream);
     for (void* p : owned) (void)hipFree(p);
     drop_pool();
+    for (auto& kv : idle.pool) (void)hipFree(kv.second);
+    if (idle.ws) (void)hipFree(idle.ws);
+    if (idle.stream) (void)hipStreamDestroy(idle.stream);
+    if (fork_ev) (void)hipEventDestroy(fork_ev);
+    if (join_ev) (void)hipEventDestroy(join_ev);
     if (ws) (void)hipFree(ws);
     if (ev0) (void)hipEventDestroy(ev0);
     if (ev1) (void)hipEventDestroy(ev1);
@@ -1207,6 +1238,42 @@ int ace_sync(ace_ctx* c) {
   c->check_deferred();
   ACE_CATCH_INT
 }
+// ---- two lanes ------------------------------------------------------------------
+int ace_fork(ace_ctx* c) {
+  ACE_TRY
+  if (c->fork_state) return fail("ace_fork: the context is forked already");
+  if (!c->idle.stream) {
+    HIP_OK(hipStreamCreateWithFlags(&c->idle.stream, hipStreamNonBlocking));
+    HIP_OK(hipEventCreateWithFlags(&c->fork_ev, hipEventDisableTiming));
+    HIP_OK(hipEventCreateWithFlags(&c->join_ev, hipEventDisableTiming));
+  }
+  HIP_OK(hipEventRecord(c->fork_ev, c->stream));
+  c->swap_lanes();
+  HIP_OK(hipStreamWaitEvent(c->stream, c->fork_ev, 0));
+  c->fork_state = 1;
+  ACE_CATCH_INT
+}
+int ace_fork_switch(ace_ctx* c) {
+  ACE_TRY  // launches what is still recorded, on the second lane
+  if (c->fork_state != 1) return fail("ace_fork_switch: not on the second lane");
+  HIP_OK(hipEventRecord(c->join_ev, c->stream));
+  c->swap_lanes();
+  c->fork_state = 2;
+  ACE_CATCH_INT
+}
+int ace_join(ace_ctx* c) {
+  ACE_TRY
+  if (c->fork_state == 1) {
+    HIP_OK(hipEventRecord(c->join_ev, c->stream));
+    c->swap_lanes();
+    c->fork_state = 2;
+  }
+  if (c->fork_state != 2) return fail("ace_join: the context is not forked");
+  HIP_OK(hipStreamWaitEvent(c->stream, c->join_ev, 0));
+  c->fork_state = 0;
+  ACE_CATCH_INT
+}
+
 int ace_timer_start(ace_ctx* c) {
   ACE_TRY
   HIP_OK(hipEventRecord(c->ev0, c->stream));

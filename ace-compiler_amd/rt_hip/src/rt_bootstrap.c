@@ -394,7 +394,9 @@ void Rt_bootstrap_prepare(void) {
 }
 
 static void stage_clear(void);
+static void mono_clear(void);
 void Rt_bootstrap_finalize(void) {
+  mono_clear();
   stage_clear();
   while (Precoms) {
     BTS_PRECOM* p = Precoms;
@@ -450,17 +452,43 @@ static void set_level(CIPHER c, size_t level) {
   Set_poly_level(&c->_c1_poly, level);
 }
 
-CIPHER Mul_mono_ciph(CIPHER res, CIPHER c, uint32_t power) { /* Mul_by_monomial (evaluator.c:260-286) */
-  size_t   l = Level(c), n = G.N;
+/* The monomial X^power over all Q limbs in NTT form, kept on the device once built: a bootstrap multiplies by the
+ * same two monomials every time, and building one means a host buffer of a whole polynomial, an upload (which waits
+ * for the GPU to finish everything issued so far) and a transform. */
+#define MONO_SLOTS 8
+static struct {
+  uint32_t power;
+  int64_t* dev;
+} Mono[MONO_SLOTS];
+static size_t Mono_n;
+static void   mono_clear(void) {
+  for (size_t i = 0; i < Mono_n; ++i) Rt_dev_free(Mono[i].dev);
+  Mono_n = 0;
+}
+static int64_t* monomial(uint32_t power) {
+  size_t n = G.N, l = G.L;
+  power %= (uint32_t)(2 * n);
+  for (size_t i = 0; i < Mono_n; ++i)
+    if (Mono[i].power == power) return Mono[i].dev;
+  if (Mono_n == MONO_SLOTS) mono_clear();
   int64_t* host = (int64_t*)calloc(l * n, sizeof(int64_t));
   int64_t* mono = Rt_dev_alloc(l * n);
   int32_t  idx[128];
   for (size_t t = 0; t < l; ++t) {
-    host[t * n + power % n] = power % (2 * n) < n ? 1 : G.q[t]._val - 1;
+    host[t * n + power % n] = power < n ? 1 : G.q[t]._val - 1;
     idx[t]                  = (int32_t)t;
   }
   ACE_OK(ace_upload(G.ctx, mono, host, l * n));
   ACE_OK(ace_ntt(G.ctx, mono, mono, idx, l, 1, 0));
+  free(host);
+  Mono[Mono_n].power = power;
+  Mono[Mono_n].dev   = mono;
+  Mono_n++;
+  return mono;
+}
+CIPHER Mul_mono_ciph(CIPHER res, CIPHER c, uint32_t power) { /* Mul_by_monomial (evaluator.c:260-286) */
+  size_t   l    = Level(c);
+  int64_t* mono = monomial(power); /* limb t of a polynomial at any level is limb t of the chain */
   if (res != c) {
     Init_poly(&res->_c0_poly, &c->_c0_poly);
     Init_poly(&res->_c1_poly, &c->_c1_poly);
@@ -471,8 +499,6 @@ CIPHER Mul_mono_ciph(CIPHER res, CIPHER c, uint32_t power) { /* Mul_by_monomial 
   ACE_OK(ace_poly_mul(G.ctx, res->_c0_poly._data, c->_c0_poly._data, mono, l, 0));
   ACE_OK(ace_poly_mul(G.ctx, res->_c1_poly._data, c->_c1_poly._data, mono, l, 0));
   res->_c0_poly._is_ntt = res->_c1_poly._is_ntt = true;
-  Rt_dev_free(mono);
-  free(host);
   return res;
 }
 
@@ -857,6 +883,24 @@ static void eval_chebyshev(CIPHER ct, const double* coeff, uint32_t n_coeff, boo
 }
 
 /* Eval_approx_mod (bootstrap.c:1524-1559): the series, then the double-angle steps */
+static void eval_approx_mod(CIPHER ct);
+/* The real and the imaginary half of a fully packed ciphertext go through the same series independently: the second
+ * is issued on the library's second lane, so that its kernels (one polynomial each, too small for the machine)
+ * overlap with the first's.  RT_HIP_ONE_LANE=1 issues them one after the other. */
+static void eval_approx_mod_pair(CIPHER a, CIPHER b) {
+  static int one_lane = -1;
+  if (one_lane < 0) one_lane = getenv("RT_HIP_ONE_LANE") && atoi(getenv("RT_HIP_ONE_LANE")) != 0;
+  if (one_lane) {
+    eval_approx_mod(a);
+    eval_approx_mod(b);
+    return;
+  }
+  ACE_OK(ace_fork(G.ctx));
+  eval_approx_mod(b);
+  ACE_OK(ace_fork_switch(G.ctx));
+  eval_approx_mod(a);
+  ACE_OK(ace_join(G.ctx));
+}
 static void eval_approx_mod(CIPHER ct) {
   const SIN_POLY* p = sin_poly();
   if (p->even) add_const(ct, -1.0 / (4.0 * p->k_bound));
@@ -945,8 +989,7 @@ static CIPHER eval_bootstrap(CIPHER res, CIPHER ct, uint32_t level_after_bts, ui
       rescale(&work);
       rescale(&sub);
     }
-    eval_approx_mod(&work);
-    eval_approx_mod(&sub);
+    eval_approx_mod_pair(&work, &sub);
     Mul_mono_ciph(&sub, &sub, (uint32_t)(G.N / 2));
     Add_ciph(&work, &work, &sub);
   } else {
@@ -1044,8 +1087,7 @@ CIPHER Eval_bootstrap_eval_mod_ciph(CIPHER res, CIPHER ct, uint32_t num_slots) {
   new_ciph(&work);
   Copy_ciph(&work, ct);
   if (Stage.active && Stage.full && Stage.sub._c0_poly._data && Stage.slots == slots) {
-    eval_approx_mod(&work);
-    eval_approx_mod(&Stage.sub);
+    eval_approx_mod_pair(&work, &Stage.sub);
     Mul_mono_ciph(&Stage.sub, &Stage.sub, slots);
     Add_ciph(&work, &work, &Stage.sub);
     Free_ciph_poly(&Stage.sub, 1);

@@ -129,7 +129,7 @@ VALUE_LIST* Alloc_precomp(POLY input) {
 }
 void Free_precomp(VALUE_LIST* precompute) {
   if (!precompute) return;
-  Free_polys((POLY_ARR)PTR_VALUE_AT(precompute, 0)); /* the digits are one array over one slab */
+  if (LIST_LEN(precompute)) Free_polys((POLY_ARR)PTR_VALUE_AT(precompute, 0)); /* the digits are one array over one slab */
   Free_value_list(precompute);
 }
 

@@ -91,6 +91,20 @@ int      ace_download(ace_ctx* ctx, int64_t* host_dst, const int64_t* dev_src, s
 int      ace_copy(ace_ctx* ctx, int64_t* dev_dst, const int64_t* dev_src, size_t n_words);
 int      ace_zero(ace_ctx* ctx, int64_t* dev_dst, size_t n_words);
 int      ace_sync(ace_ctx* ctx);
+/* Two lanes.  No counterpart in the reference, whose runtime is synchronous: calls enqueue on one stream per context
+ * and therefore run one after another on the GPU, although a single polynomial's kernels do not fill the machine.
+ * Where a program has two independent pieces of work (the two sine evaluations of a fully packed bootstrap):
+ *   ace_fork(ctx);         the calls that follow are issued on a second stream, which first waits for everything
+ *                          issued so far;
+ *   ace_fork_switch(ctx);  back to the first stream: the calls that follow may run at the same time as those issued
+ *                          since ace_fork;
+ *   ace_join(ctx);         the first stream waits for the second (ace_join straight after ace_fork works too).
+ * Between ace_fork and ace_join the two sequences must not touch each other's buffers (what either reads may have
+ * been written before the fork); results are those of issuing both sequences one after the other.  Buffers may be
+ * allocated and freed on either lane. */
+int      ace_fork(ace_ctx* ctx);
+int      ace_fork_switch(ace_ctx* ctx);
+int      ace_join(ace_ctx* ctx);
 /* HIP-event stopwatch on the context's stream (for benchmarks) */
 int      ace_timer_start(ace_ctx* ctx);
 float    ace_timer_stop_ms(ace_ctx* ctx); /* synchronises; <0 on error */

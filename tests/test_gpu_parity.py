@@ -634,6 +634,57 @@ def test_mul_relin_rescale_batch(pair):
         g.mul_relin_rescale_batch(r0, r1, n - 1, dev[0], dev[1], dev[2], dev[3], in_stride, dk, level, 2)  # overlap
 
 
+def test_two_lanes_equal_one(pair):
+    """ace_fork / ace_fork_switch / ace_join: two independent sequences of calls (HMult + relinearise + rescale, a
+    transform there and back, recorded elementwise calls, buffers allocated and freed on the way) issued on the two
+    lanes give the results of issuing them one after the other, repeatedly, with the lanes' buffer pools warm and
+    cold; misuse is rejected."""
+    g = pair.g
+    N = g.N
+    if g.L < 2:
+        pytest.skip("needs two levels")
+    big_ring_skip(N)
+    level = g.L
+    pr = g.primes[:level]
+    dk = g.upload(make_swk(g, 1900))
+    idx = list(range(level - 1))
+
+    def sequence(seed):
+        a0, a1, b0, b1 = (g.upload(seeded.uniform_poly(seed + i, pr, N)) for i in range(4))
+        r0, r1 = g.alloc((level - 1) * N), g.alloc((level - 1) * N)
+        g.mul_relin_rescale(r0, r1, a0, a1, b0, b1, dk, level)
+        t = g.alloc((level - 1) * N)
+        g.intt(t, r0, idx)
+        g.ntt(t, t, idx)
+        for limb in range(level - 1):  # recorded calls: r1 += t * r0, limb by limb
+            g.hw("modmuladd", r1.view(limb * N, N), t.view(limb * N, N), r0.view(limb * N, N), limb)
+        for b in (a0, a1, b0, b1, t):
+            b.free()
+        return r0, r1
+
+    want = [[x.get() for x in sequence(2000 + 10 * k)] for k in range(2)]
+    for rep in range(4):
+        g.fork()
+        second = sequence(2010)
+        g.fork_switch()
+        first = sequence(2000)
+        g.join()
+        for k, res in enumerate((first, second)):
+            for j in range(2):
+                eq(res[j], want[k][j], "lane %d result %d, repetition %d" % (k, j, rep))
+                res[j].free()
+    g.fork()
+    g.join()  # nothing issued on the second lane
+    with pytest.raises(acefhe.AceError):
+        g.join()
+    with pytest.raises(acefhe.AceError):
+        g.fork_switch()
+    g.fork()
+    with pytest.raises(acefhe.AceError):
+        g.fork()
+    g.join()
+
+
 def test_rotation_many(pair):
     """More rotations than one batched launch holds (small rings only: the oracle does each one)."""
     g, o = pair.g, pair.o
