@@ -145,6 +145,22 @@ def bootstrap_error(args):
     return float(f[f.index("max_err") + 1]), r.returncode
 
 
+def test_bootstrap_on_two_lanes_equals_one_lane():
+    """A fully packed bootstrap issues its two sine evaluations on the library's two lanes; with RT_HIP_ONE_LANE=1 it
+    issues them one after the other.  Same keys, same input: the decrypted results are the same numbers to the last
+    printed digit (the ciphertexts are bit-identical, the arithmetic being exact)."""
+    assert os.path.exists(BOOTSTRAP), "tests/programs/bootstrap_program is not built"
+    lines = []
+    for one in ("0", "1"):
+        print("running bootstrap_program, RT_HIP_ONE_LANE=" + one, flush=True)
+        r = subprocess.run([BOOTSTRAP] + "1024 20 60 51 64 512 0 4".split(), capture_output=True, text=True, timeout=110,
+                           env=dict(os.environ, RT_HIP_ONE_LANE=one))
+        assert r.returncode == 0, r.stdout + r.stderr
+        f = r.stdout.split()
+        lines.append((f[f.index("max_err") + 1], f[f.index("square_err") + 1], f[f.index("level") + 1]))
+    assert lines[0] == lines[1], lines
+
+
 def test_bootstrap_precision_at_the_model_ring():
     """N = 65536, 34 limbs, Hamming weight 192, 32768 slots, refreshed to level 15 (the call of the ResNet programs).
     On the chain the reference's build scripts compile the models with (q0 = 60, scale = 56 bits:
