@@ -80,6 +80,7 @@ def _sig(lib):
     f("ace_ext_plain_mac_groups", C.c_int, _vp, _vp, _vp, _sz, _vp, _vp, _sz, _vp, _sz, _sz)
     f("ace_ext_rotate", C.c_int, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp, _sz, C.c_int)
     f("ace_encode_scaled", C.c_int, _vp, _vp, _vp, _sz, C.c_uint32, _sz, C.c_double, _sz)
+    f("ace_encode_real_batch", C.c_int, _vp, _vp, _sz, _vp, C.c_int, _sz, _sz, C.c_uint32, _sz, C.c_uint32, _sz)
     f("ace_encode_real", C.c_int, _vp, _vp, _vp, C.c_int, _sz, C.c_uint32, _sz, C.c_uint32, _sz)
     f("ace_mod_down_rescale", C.c_int, _vp, _vp, _vp, _sz, C.c_int)
     f("ace_reduce_rescale_modup", C.c_int, _vp, _vp, _vp, _vp, _sz, C.c_int)
@@ -119,7 +120,7 @@ EXPORTS = [
     "ace_hw_modsub_scalar", "ace_hw_modmul_scalar", "ace_hw_modmuladd_scalar", "ace_hw_rotate",
     "ace_find_automorphism_index", "ace_automorphism_order", "ace_poly_add", "ace_poly_sub", "ace_poly_mul",
     "ace_poly_automorphism", "ace_decomp_modup", "ace_mod_up", "ace_mod_down_rescale",
-    "ace_reduce_rescale_modup", "ace_transform_from_level0", "ace_host_fft_tables", "ace_embedding_inv", "ace_decode", "ace_fork", "ace_fork_switch", "ace_join", "ace_encode", "ace_encode_scaled", "ace_encode_real", "ace_ext_rotate", "ace_ext_plain_mac_groups", "ace_precomp", "ace_mod_down", "ace_rescale", "ace_extend",
+    "ace_reduce_rescale_modup", "ace_transform_from_level0", "ace_host_fft_tables", "ace_embedding_inv", "ace_decode", "ace_fork", "ace_fork_switch", "ace_join", "ace_encode", "ace_encode_scaled", "ace_encode_real", "ace_encode_real_batch", "ace_ext_rotate", "ace_ext_plain_mac_groups", "ace_precomp", "ace_mod_down", "ace_rescale", "ace_extend",
     "ace_dot_prod", "ace_mul_ciph3", "ace_fast_switch_key", "ace_relin", "ace_rescale_ciph",
     "ace_mul_relin_rescale", "ace_mul_relin_rescale_batch", "ace_fast_rotate", "ace_rotate_batch",
 ]
@@ -362,6 +363,14 @@ class Context:
         assert v.dtype in (np.float32, np.float64)
         self._chk(self.lib.ace_encode_real(self.h, res.ptr, v.ctypes.data_as(C.c_void_p), int(v.dtype == np.float32), v.size,
                                            slots, level, sf_degree, p_cnt))
+
+    def encode_real_batch(self, res, res_stride, vectors, slots=0, level=0, sf_degree=1, p_cnt=0):
+        """vectors: equally long float32 or float64 arrays, one per polynomial."""
+        vs = [np.ascontiguousarray(v) for v in vectors]
+        assert vs and all(v.dtype == vs[0].dtype and v.size == vs[0].size for v in vs)
+        ptrs = (C.c_void_p * len(vs))(*[v.ctypes.data for v in vs])
+        self._chk(self.lib.ace_encode_real_batch(self.h, res.ptr, res_stride, ptrs, int(vs[0].dtype == np.float32),
+                                                 vs[0].size, len(vs), slots, level, sf_degree, p_cnt))
 
     def mod_up(self, res, digit, level, part, is_ntt=True):
         self._chk(self.lib.ace_mod_up(self.h, res.ptr, digit.ptr, level, part, int(is_ntt)))

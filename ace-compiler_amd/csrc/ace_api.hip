@@ -1805,10 +1805,19 @@ int ace_decode(ace_ctx* c, double* host_out, const int64_t* poly, size_t level, 
 // are widened to complex numbers on the device (a float widens exactly, as the host cast would).
 // explicit_scale > 0: Encode_impl_with_scale (encoder.c:337-403): one multiplication by that scale, rounded without
 // the half that Encode_impl adds first, and no further powers of the scaling factor.
+// n_vec > 1: that many vectors (vecs[v], each n_values long, real-valued kinds only) are encoded in one set of
+// launches into res + v * res_stride.
 static int encode_impl(ace_ctx* c, int64_t* res, const void* values, int kind, size_t n_values, uint32_t slots,
-                       size_t level, uint32_t sf_degree, size_t p_cnt, double explicit_scale = 0.0) {
+                       size_t level, uint32_t sf_degree, size_t p_cnt, double explicit_scale = 0.0,
+                       const void* const* vecs = nullptr, size_t n_vec = 1, size_t res_stride = 0) {
   ACE_TRY
-  if (!res || (!values && n_values)) return fail("ace_encode: null argument");
+  if (n_vec == 0) return 0;
+  if (!vecs) vecs = &values;
+  if (!res) return fail("ace_encode: null argument");
+  for (size_t v = 0; v < n_vec; ++v)
+    if (!vecs[v] && n_values) return fail("ace_encode: null argument");
+  if (n_vec > 1 && (kind == 0 || n_values == 0)) return fail("ace_encode: batches take real-valued vectors");
+  if (n_vec > 65535) return fail("ace_encode: more than 65535 vectors per call");
   if (!c->sf_bits) return fail("ace_encode: the context was created from explicit primes and has no scaling factor");
   const size_t N = c->h.N, K = c->h.K;
   if (!slots) slots = (uint32_t)(N / 2);
@@ -1832,22 +1841,25 @@ static int encode_impl(ace_ctx* c, int64_t* res, const void* values, int kind, s
   LimbMap lm = poly_lm(c, level, p_cnt != 0);
   const u32 n_limbs = (u32)(level + p_cnt);
   const size_t value_bytes = kind == 0 ? sizeof(double2) : kind == 1 ? sizeof(double) : sizeof(float);
+  const size_t poly_words = (size_t)n_limbs * N;
+  if (n_vec > 1 && res_stride < poly_words) return fail("ace_encode: result stride smaller than a polynomial");
   auto stage_values = [&](hipStream_t st, double2* z, void* raw) {  // z = the values, zero-padded to `slots`
     if (kind == 0) {
       if (n_values < slots)
         launch_fill_zero(st, reinterpret_cast<u64*>(z + n_values), 2 * (size_t)(slots - n_values));
-      c->h2d(z, values, n_values * value_bytes);
+      c->h2d(z, vecs[0], n_values * value_bytes);
     } else {
-      c->h2d(raw, values, n_values * value_bytes);
-      launch_widen_real(st, z, raw, kind == 2, (u32)n_values, slots);
+      for (size_t v = 0; v < n_vec; ++v)
+        c->h2d(static_cast<char*>(raw) + v * n_values * value_bytes, vecs[v], n_values * value_bytes);
+      launch_widen_real(st, z, raw, kind == 2, (u32)n_values, slots, (u32)n_vec);
     }
   };
-  c->ensure_ws(c->std_ws(level));
+  c->ensure_ws(std::max(c->std_ws(level), 3 * (size_t)slots * n_vec + 2 * level + 64));
   c->ws_used = 0;
-  double2* z = reinterpret_cast<double2*>(c->take(2 * (size_t)slots));
-  stage_values(c->stream, z, kind == 0 ? nullptr : c->take(slots));
+  double2* z = reinterpret_cast<double2*>(c->take(2 * (size_t)slots * n_vec));
+  stage_values(c->stream, z, kind == 0 ? nullptr : c->take((size_t)slots * n_vec));
   launch_encode(c->stream, c->d, U(res), z, c->fft_rou, c->rot_group, slots, scaling_factor, scale,
-                by_scale ? 0.0 : 0.5, range_bound, lm, n_limbs, c->d_err);
+                by_scale ? 0.0 : 0.5, range_bound, lm, n_limbs, c->d_err, (u32)n_vec, res_stride);
   if (sf_degree > 1) {  // encoder.c:297-312: the Q limbs are multiplied by scaling_factor^(sf_degree-1)
     std::vector<u64> cst(2 * level);
     for (size_t t = 0; t < level; ++t) {
@@ -1858,11 +1870,11 @@ static int encode_impl(ace_ctx* c, int64_t* res, const void* values, int kind, s
     }
     u64* dc = c->take(2 * level);
     c->h2d(dc, cst.data(), cst.size() * sizeof(u64));
-    HIP_OK(hipStreamSynchronize(c->stream));  // cst is a local
-    launch_mul_const(c->stream, c->d, U(res), U(res), dc, c->q_lm, (u32)level);
+    for (size_t v = 0; v < n_vec; ++v)
+      launch_mul_const(c->stream, c->d, U(res) + v * res_stride, U(res) + v * res_stride, dc, c->q_lm, (u32)level);
   }
-  PolySeq rs = seq_strided(U(res), 0);
-  launch_ntt(c->stream, c->d, rs, rs, lm, nullptr, n_limbs, 1, false, nullptr);
+  PolySeq rs = seq_strided(U(res), res_stride);
+  launch_ntt(c->stream, c->d, rs, rs, lm, nullptr, n_limbs, (u32)n_vec, false, nullptr);
   ACE_CATCH_INT
 }
 int ace_encode(ace_ctx* c, int64_t* res, const double* values, size_t n_values, uint32_t slots, size_t level,
@@ -1872,6 +1884,13 @@ int ace_encode(ace_ctx* c, int64_t* res, const double* values, size_t n_values, 
 int ace_encode_real(ace_ctx* c, int64_t* res, const void* values, int is_f32, size_t n_values, uint32_t slots,
                     size_t level, uint32_t sf_degree, size_t p_cnt) {
   return encode_impl(c, res, values, is_f32 ? 2 : 1, n_values, slots, level, sf_degree, p_cnt);
+}
+int ace_encode_real_batch(ace_ctx* c, int64_t* res, size_t res_stride, const void* const* values, int is_f32,
+                          size_t n_values, size_t n_vec, uint32_t slots, size_t level, uint32_t sf_degree,
+                          size_t p_cnt) {
+  if (!values) return fail("ace_encode_real_batch: null argument");
+  return encode_impl(c, res, nullptr, is_f32 ? 2 : 1, n_values, slots, level, sf_degree, p_cnt, 0.0, values, n_vec,
+                     res_stride);
 }
 int ace_encode_scaled(ace_ctx* c, int64_t* res, const double* values, size_t n_values, uint32_t slots, size_t level,
                       double scale, size_t p_cnt) {

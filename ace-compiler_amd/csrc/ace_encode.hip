@@ -19,9 +19,10 @@ constexpr int kTileThreads = 1024;  // one butterfly per thread and stage on a f
 __global__ __launch_bounds__(kTileThreads) void embed_inv_tile_kernel(double2* __restrict__ r,
                                                                      const double2* __restrict__ rou,
                                                                      const u32* __restrict__ rot, u32 M, u32 logm_hi,
-                                                                     u32 logm_lo, u32 log_w) {
+                                                                     u32 logm_lo, u32 log_w, u32 len) {
 #pragma clang fp contract(off)
   __shared__ double2 tile[1u << kTileLog];
+  r += (u64)blockIdx.y * len;  // blockIdx.y: which of the vectors of a batch
   const u32 S = logm_hi - logm_lo + 1, low_bits = logm_lo - 1;  // low_bits index bits lie below the paired ones
   const u32 tile_elems = 1u << (S + log_w);
   // blockIdx.x enumerates (high part, group of W low values)
@@ -53,7 +54,8 @@ __global__ __launch_bounds__(kTileThreads) void embed_inv_tile_kernel(double2* _
 }
 
 // all stages of Embedding_inv over `len` elements: the top stages in tiles of strided runs, then the rest
-static void launch_embed_inv_stages(hipStream_t st, double2* r, const double2* rou, const u32* rot, u32 M, u32 len) {
+static void launch_embed_inv_stages(hipStream_t st, double2* r, const double2* rou, const u32* rot, u32 M, u32 len,
+                                    u32 n_vec = 1) {
   u32 loglen = 0;
   while ((1u << loglen) < len) ++loglen;
   u32 hi = loglen;
@@ -61,14 +63,14 @@ static void launch_embed_inv_stages(hipStream_t st, double2* r, const double2* r
   const u32 threads = half >= (u32)kTileThreads ? (u32)kTileThreads : (half < 64 ? 64 : half);
   while (hi > kTileLog) {  // stages hi .. lo on tiles of 2^S x W elements, W >= 16 for coalesced runs
     const u32 S = (hi - kTileLog) < 7 ? (hi - kTileLog) : 7, lo = hi - S + 1, log_w = kTileLog - S;
-    hipLaunchKernelGGL(embed_inv_tile_kernel, dim3(len >> kTileLog), dim3(threads), 0, st, r, rou, rot, M, hi, lo,
-                       log_w);
+    hipLaunchKernelGGL(embed_inv_tile_kernel, dim3(len >> kTileLog, n_vec), dim3(threads), 0, st, r, rou, rot, M, hi,
+                       lo, log_w, len);
     hi = lo - 1;
   }
   if (hi >= 1) {
     const u32 tile_log = hi;  // hi <= kTileLog: stages hi .. 1 on tiles of 2^hi consecutive elements
-    hipLaunchKernelGGL(embed_inv_tile_kernel, dim3(len >> tile_log), dim3(threads), 0, st, r, rou, rot, M, hi, 1u,
-                       0u);
+    hipLaunchKernelGGL(embed_inv_tile_kernel, dim3(len >> tile_log, n_vec), dim3(threads), 0, st, r, rou, rot, M, hi,
+                       1u, 0u, len);
   }
 }
 
@@ -88,10 +90,12 @@ __global__ __launch_bounds__(kEncThreads) void encode_round_kernel(DevCtx c, u64
                                                                    const double2* __restrict__ r, u32 slots,
                                                                    u32 logslots, double scaling_factor, double scale,
                                                                    double round_add, double range_bound, LimbMap lm,
-                                                                   int* err) {
+                                                                   int* err, u64 out_stride) {
 #pragma clang fp contract(off)
   const u32 n = blockIdx.x * kEncThreads + threadIdx.x;
   if (n >= c.N) return;
+  out += blockIdx.z * out_stride;  // blockIdx.z: which of the vectors of a batch
+  r += (u64)blockIdx.z * slots;
   const u32 limb = blockIdx.y;
   const i64 q = (i64)c.primes[lm.prime[limb]].q;
   const u32 gap = c.N / (slots * 2);
@@ -140,23 +144,25 @@ __global__ __launch_bounds__(256) void widen_real_kernel(double2* __restrict__ z
                                                          int is_f32, u32 n_values, u32 slots) {
   const u32 i = blockIdx.x * 256 + threadIdx.x;
   if (i >= slots) return;
+  const u64 at = (u64)blockIdx.y * n_values + i;  // blockIdx.y: which of the vectors of a batch, stored back to back
   double v = 0.0;
-  if (i < n_values) v = is_f32 ? (double)static_cast<const float*>(raw)[i] : static_cast<const double*>(raw)[i];
-  z[i] = make_double2(v, 0.0);
+  if (i < n_values) v = is_f32 ? (double)static_cast<const float*>(raw)[at] : static_cast<const double*>(raw)[at];
+  z[(u64)blockIdx.y * slots + i] = make_double2(v, 0.0);
 }
-void launch_widen_real(hipStream_t st, double2* z, const void* raw, bool is_f32, u32 n_values, u32 slots) {
-  hipLaunchKernelGGL(widen_real_kernel, dim3((slots + 255) / 256), dim3(256), 0, st, z, raw, is_f32 ? 1 : 0, n_values,
-                     slots);
+void launch_widen_real(hipStream_t st, double2* z, const void* raw, bool is_f32, u32 n_values, u32 slots, u32 n_vec) {
+  hipLaunchKernelGGL(widen_real_kernel, dim3((slots + 255) / 256, n_vec), dim3(256), 0, st, z, raw, is_f32 ? 1 : 0,
+                     n_values, slots);
 }
 
 void launch_encode(hipStream_t st, const DevCtx& c, u64* out, double2* r, const double2* rou, const u32* rot,
                    u32 slots, double scaling_factor, double scale, double round_add, double range_bound,
-                   const LimbMap& lm, u32 n_limbs, int* err) {
+                   const LimbMap& lm, u32 n_limbs, int* err, u32 n_vec, u64 out_stride) {
   u32 logslots = 0;
   while ((1u << logslots) < slots) ++logslots;
-  launch_embed_inv_stages(st, r, rou, rot, 2 * c.N, slots);
-  hipLaunchKernelGGL(encode_round_kernel, dim3((c.N + kEncThreads - 1) / kEncThreads, n_limbs), dim3(kEncThreads), 0,
-                     st, c, out, r, slots, logslots, scaling_factor, scale, round_add, range_bound, lm, err);
+  launch_embed_inv_stages(st, r, rou, rot, 2 * c.N, slots, n_vec);
+  hipLaunchKernelGGL(encode_round_kernel, dim3((c.N + kEncThreads - 1) / kEncThreads, n_limbs, n_vec),
+                     dim3(kEncThreads), 0, st, c, out, r, slots, logslots, scaling_factor, scale, round_add,
+                     range_bound, lm, err, out_stride);
 }
 
 // ---- decoding (Decode, ckks/src/encoder.c:657-704) ------------------------------------------------------

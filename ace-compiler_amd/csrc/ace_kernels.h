@@ -173,10 +173,11 @@ void launch_embedding_inv(hipStream_t st, const DevCtx& c, double2* out, double2
 // message) and is used as scratch; rou = exp(2 pi i k / 2N), k < 2N; rot = 5^k mod 2N, k < N/2.
 // out: n_limbs limbs of N words (limb t uses lm.prime[t]).  *err is set to 1 where the reference asserts.
 // z[i] = (raw[i], 0) for i < n_values, (0, 0) up to slots; raw holds doubles or floats
-void launch_widen_real(hipStream_t st, double2* z, const void* raw, bool is_f32, u32 n_values, u32 slots);
+void launch_widen_real(hipStream_t st, double2* z, const void* raw, bool is_f32, u32 n_values, u32 slots,
+                       u32 n_vec = 1);  // n_vec vectors of n_values back to back in raw, of slots in z
 void launch_encode(hipStream_t st, const DevCtx& c, u64* out, double2* r, const double2* rou, const u32* rot,
                    u32 slots, double scaling_factor, double scale, double round_add, double range_bound,
-                   const LimbMap& lm, u32 n_limbs, int* err);
+                   const LimbMap& lm, u32 n_limbs, int* err, u32 n_vec = 1, u64 out_stride = 0);
 constexpr int kDecodeWords = 64;  // most limbs of a polynomial the decoder reconstructs
 // Decode (ckks/src/encoder.c:657-704) of a polynomial in coefficient form: r receives the `slots` complex values
 void launch_decode(hipStream_t st, const DevCtx& c, double2* r, const u64* poly, u32 level, u32 slots, double factor,

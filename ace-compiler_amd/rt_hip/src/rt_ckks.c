@@ -317,6 +317,14 @@ void Rt_encode_real(PLAIN plain, const void* values, int is_f32, size_t len, uin
   ACE_OK(ace_encode_real(G.ctx, plain->_poly._data, values, is_f32, len, 0, level, sc_degree, 0));
 }
 
+/* n_vec real-valued vectors into the polynomials dev_base + v * stride (level limbs each, NTT form) */
+void Rt_encode_real_batch(int64_t* dev_base, size_t stride, const void* const* values, int is_f32, size_t len,
+                          size_t n_vec, uint32_t sc_degree, uint32_t level) {
+  if (level == 0) level = (uint32_t)G.L;
+  FMT_ASSERT(level <= G.L, "level should not be larger than mul_depth + 1");
+  ACE_OK(ace_encode_real_batch(G.ctx, dev_base, stride, values, is_f32, len, n_vec, 0, level, sc_degree, 0));
+}
+
 void Encode_double(PLAIN plain, double* input, size_t len, uint32_t sc_degree, uint32_t level) {
   if (len == 1) {
     encode_value(plain, *input, sc_degree, level);

@@ -78,6 +78,15 @@ static int64_t* cache_room(size_t words) {
   return p;
 }
 
+/* room for `count` polynomials of `words` words one after the other (a batch is encoded straight into it) */
+static int64_t* cache_room_run(size_t words, size_t count) {
+  if (words * count > PT_SLAB_WORDS) return NULL;
+  if (Cache.slab_left < words * count) Cache.slab_left = 0; /* the rest of the slab stays unused */
+  int64_t* first = cache_room(words);
+  for (size_t i = 1; first && i < count; ++i) (void)cache_room(words);
+  return first;
+}
+
 static PT_CELL* cache_find(uint64_t k1, uint64_t k2) {
   if (!Cache.cap) return NULL;
   uint64_t h = (k1 * 0x9E3779B97F4A7C15ull) ^ (k2 * 0xC2B2AE3D27D4EB4Full);
@@ -230,9 +239,61 @@ static const void* entry_bytes(uint32_t index, size_t first, size_t len, int* is
   return Data.buf + (e->ofst - DATA_PAGE) + first * width;
 }
 
+/* Programs ask for the entries of a tensor one after the other (index, index + 1, ... with the same range, scale
+ * and level: the taps and channels of a convolution), each a handful of small launches on one polynomial.  On a
+ * miss the entries that follow are therefore encoded along with the one asked for, in one set of launches
+ * (ace_encode_real_batch: the same bits), straight into the kept plaintexts; a guess that the program does not
+ * follow costs the encodes it does not use.  RT_HIP_PLAINTEXT_AHEAD sets how many (default 16, 1 = none). */
+#define PT_AHEAD_MAX 64
+static bool entry_has(uint32_t index, size_t first, size_t len) {
+  if (Data.synthetic) return true;
+  if (index >= Data.hdr.ent_count) return false;
+  size_t           width = Data.hdr.ent_type == DE_MSG_F32 ? sizeof(float) : sizeof(double);
+  const LUT_ENTRY* e     = &Data.lut[index];
+  return e->size >= (first + len) * width && e->ofst >= DATA_PAGE && e->ofst - DATA_PAGE + (first + len) * width <= Data.size;
+}
+static uint64_t cache_key1(uint32_t index, uint32_t scale, uint32_t level) {
+  return ((uint64_t)index << 32) | ((uint64_t)(scale & 0xFFFF) << 16) | (level ? level : Get_q_cnt());
+}
+static bool encode_ahead(void* pt, uint32_t index, size_t ofst, size_t len, uint32_t scale, uint32_t level, size_t words) {
+  static size_t ahead;
+  if (!ahead) {
+    const char* env = getenv("RT_HIP_PLAINTEXT_AHEAD");
+    ahead           = env ? (size_t)atoi(env) : 16;
+    if (ahead < 1) ahead = 1;
+    if (ahead > PT_AHEAD_MAX) ahead = PT_AHEAD_MAX;
+  }
+  if (ahead < 2) return false;
+  const uint64_t k2 = ((uint64_t)ofst << 32) | (uint64_t)len;
+  const void*    vals[PT_AHEAD_MAX];
+  int            is_f32 = 0;
+  size_t         n      = 0;
+  while (4 * (Cache.count + ahead + 1) > 3 * Cache.cap) cache_grow();
+  for (; n < ahead && (uint64_t)index + n < (1ull << 32); ++n) {
+    uint32_t idx = index + (uint32_t)n;
+    if (Cache.words + (n + 1) * words > Cache.limit_words || !entry_has(idx, ofst, len)) break;
+    if (cache_find(cache_key1(idx, scale, level), k2)->k1) break; /* kept already: the run ends here */
+    vals[n] = entry_bytes(idx, ofst, len, &is_f32);
+  }
+  if (n < 2) return false;
+  int64_t* base = cache_room_run(words, n);
+  if (!base) return false;
+  Rt_encode_real_batch(base, words, vals, is_f32, len, n, scale, level);
+  for (size_t i = 0; i < n; ++i) {
+    PT_CELL* c = cache_find(cache_key1(index + (uint32_t)i, scale, level), k2);
+    c->k1      = cache_key1(index + (uint32_t)i, scale, level);
+    c->k2      = k2;
+    c->dev     = base + i * words;
+    ++Cache.count;
+    Cache.words += words;
+  }
+  Rt_copy_words(Rt_plain_prepare((PLAIN)pt, scale, level), base, words);
+  return true;
+}
+
 void* Pt_from_msg_ofst(void* pt, uint32_t index, size_t ofst, size_t len, uint32_t scale, uint32_t level) {
   const size_t   words = (size_t)(level ? level : Get_q_cnt()) * Degree();
-  const uint64_t k1    = ((uint64_t)index << 32) | ((uint64_t)(scale & 0xFFFF) << 16) | (level ? level : Get_q_cnt());
+  const uint64_t k1    = cache_key1(index, scale, level);
   const uint64_t k2    = ((uint64_t)ofst << 32) | (uint64_t)len;
   PT_CELL*       cell  = NULL;
   if (Cache.limit_words && len > 1 && ofst < (1ull << 32) && len < (1ull << 32) && scale < 0x10000) {
@@ -243,6 +304,8 @@ void* Pt_from_msg_ofst(void* pt, uint32_t index, size_t ofst, size_t len, uint32
       return pt;
     }
     if (Cache.words + words > Cache.limit_words) cell = NULL;
+    if (cell && encode_ahead(pt, index, ofst, len, scale, level, words)) return pt;
+    if (cell) cell = cache_find(k1, k2); /* the table may have grown */
   }
   Pt_encode_entry(pt, index, ofst, len, scale, level);
   if (cell && (cell->dev = cache_room(words)) != NULL) {

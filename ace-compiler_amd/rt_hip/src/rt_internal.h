@@ -72,5 +72,7 @@ void     Rt_encode_val_words(int64_t* res, double value, uint32_t level, double 
 void     Rt_copy_words(int64_t* dst, const int64_t* src, size_t n_words);
 int64_t* Rt_plain_prepare(PLAIN plain, uint32_t sc_degree, uint32_t level);
 void     Rt_encode_real(PLAIN plain, const void* values, int is_f32, size_t len, uint32_t sc_degree, uint32_t level);
+void     Rt_encode_real_batch(int64_t* dev_base, size_t stride, const void* const* values, int is_f32, size_t len,
+                              size_t n_vec, uint32_t sc_degree, uint32_t level);
 
 #endif

@@ -246,6 +246,12 @@ int ace_encode(ace_ctx* ctx, int64_t* res, const double* values, size_t n_values
  * (is_f32 = 1), widened to complex numbers with zero imaginary part on the device. */
 int ace_encode_real(ace_ctx* ctx, int64_t* res, const void* values, int is_f32, size_t n_values, uint32_t slots,
                     size_t level, uint32_t sf_degree, size_t p_cnt);
+/* The same for `n_vec` vectors of `n_values` values each (values[v] points to vector v) in one set of launches:
+ * vector v is encoded into res + v * res_stride words, bit for bit as ace_encode_real would.  For weight files, whose
+ * entries a program asks for one after the other. */
+int ace_encode_real_batch(ace_ctx* ctx, int64_t* res, size_t res_stride, const void* const* values, int is_f32,
+                          size_t n_values, size_t n_vec, uint32_t slots, size_t level, uint32_t sf_degree,
+                          size_t p_cnt);
 /* Encode_at_level_with_scale (ckks/src/encoder.c:337-420): complex values at an explicit scale (any positive
  * double below the level's modulus): one multiplication by `scale`, rounded to nearest. */
 int ace_encode_scaled(ace_ctx* ctx, int64_t* res, const double* values, size_t n_values, uint32_t slots, size_t level,

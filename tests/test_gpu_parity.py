@@ -439,6 +439,35 @@ def test_mod_down_rescale_family(pair):
         g.mod_down_rescale(g.alloc(N), g.alloc(N), 1, True)
 
 
+def test_encode_real_batch_equals_single_encodes(pair):
+    """ace_encode_real_batch: several real-valued vectors in one set of launches give, each, the polynomial of its
+    own ace_encode_real call (which test_encode compares with the oracle), with padding between the results left
+    alone, for floats and doubles, scale degrees 1 and 2, with and without P limbs."""
+    g = pair.g
+    N, (q0_bits, sf_bits) = g.N, pair.cfg[2:4]
+    rng = np.random.default_rng(N + 77)
+    for slots, n in ((N // 2, N // 2), (N // 2, max(1, N // 8)), (max(1, N // 4), max(1, N // 4))):
+        for level, deg, pc in ((g.L, 1, 0), (g.L, 2, 0), (max(1, g.L - 1), 1, g.K)):
+            if deg * sf_bits >= q0_bits + (level - 1) * sf_bits:
+                continue
+            words = (level + pc) * N
+            stride = words + N  # one limb of padding
+            for dt in (np.float32, np.float64):
+                vecs = [rng.uniform(-2, 2, n).astype(dt) for _ in range(5)]
+                out = g.alloc(5 * stride)
+                g.encode_real_batch(out, stride, vecs, slots, level, deg, pc)
+                got = out.get()
+                one = g.alloc(words)
+                for v, x in enumerate(vecs):
+                    g.encode_real(one, x, slots, level, deg, pc)
+                    eq(got[v * stride:v * stride + words], one.get(), "vector %d of the batch (%s, slots %d, n %d, level %d, degree %d, p %d)" % (v, dt.__name__, slots, n, level, deg, pc))
+                    assert not got[v * stride + words:(v + 1) * stride].any(), "padding written"
+                out.free()
+                one.free()
+    with pytest.raises(acefhe.AceError):
+        g.encode_real_batch(g.alloc(4 * N * g.L), N, [np.zeros(4), np.zeros(4)], 0, g.L, 1, 0)  # stride too small
+
+
 def test_decode(pair):
     """Device decoder vs the oracle's (itself matched against the reference's compiled Decode): the same doubles.
     Operands: encoded messages (small centred values), and uniformly random residues (integers as large as Q, both
