@@ -158,6 +158,30 @@ struct ace_ctx {
     flush_poly();
     flush_run();
   }
+  // The same for an entry point that names everything it touches: `writes` are ranges it fills completely without
+  // reading them, `reads` everything else it reads or writes.  A recorded zero fill that nothing recorded after it
+  // touches (the fill of a fresh buffer, which Alloc_poly promises) is then dropped if it lies inside a range the
+  // entry point overwrites, and moved behind the entry point's own launches, into the next run, if the entry point
+  // does not touch it at all; only a fill it reads is carried out now.
+  struct Span {
+    uintptr_t lo, hi;
+  };
+  static Span span(const void* p, size_t words) { return Span{(uintptr_t)p, (uintptr_t)p + words * sizeof(u64)}; }
+  std::vector<Span> decl_writes, decl_reads;
+  bool decl_active = false;
+  void flush_pending_declared(std::initializer_list<Span> writes, std::initializer_list<Span> reads,
+                              bool keep_poly = false) {
+    if (!keep_poly) flush_poly();
+    decl_writes.assign(writes.begin(), writes.end());
+    decl_reads.assign(reads.begin(), reads.end());
+    decl_active = true;
+    flush_run();
+    decl_active = false;
+  }
+  void flush_pending_overwriting(const void* out, size_t out_words, const void* in, size_t in_words,
+                                 bool keep_poly = false) {
+    flush_pending_declared({span(out, out_words)}, {span(in, in_words)}, keep_poly);
+  }
   bool run_accepts(const BatchOp& o, u64 n) const;
   void run_append(const BatchOp& o, u64 n);
   std::map<std::pair<size_t, size_t>, ModUpDev> modup;
@@ -550,6 +574,72 @@ void ace_ctx::run_append(const BatchOp& o, u64 n) {
 
 void ace_ctx::flush_run() {
   if (run.ops.empty()) return;
+  // Zero fills that nobody can see yet: the range is written by a later entry of the run before any entry reads it
+  // (dropped), or the rest of the run leaves it alone and the flushing entry point, having named its operands,
+  // overwrites it (dropped) or does not touch it (moved into the next run).  Ranges of a run that overlap are
+  // identical, so the start address names the range.
+  std::vector<BatchOp> carried;
+  {
+    const uintptr_t bytes = (uintptr_t)run.n * sizeof(u64);
+    auto overlaps = [&](const std::vector<Span>& v, uintptr_t r) {
+      for (const Span& x : v)
+        if (r < x.hi && x.lo < r + bytes) return true;
+      return false;
+    };
+    auto inside = [&](const std::vector<Span>& v, uintptr_t r) {
+      for (const Span& x : v)
+        if (r >= x.lo && r + bytes <= x.hi) return true;
+      return false;
+    };
+    std::vector<BatchOp> kept;
+    kept.reserve(run.ops.size());
+    for (size_t k = 0; k < run.ops.size(); ++k) {
+      const BatchOp& o = run.ops[k];
+      bool dead = false, carry = false;
+      if (o.op == BATCH_ZERO) {
+        const uintptr_t r = (uintptr_t)o.r;
+        bool touched = run.ops.size() - k > 512;  // a longer look ahead is not worth its time: the fill stays
+        for (size_t j = k + 1; j < run.ops.size() && !touched; ++j) {
+          BatchOp& n = run.ops[j];
+          const bool reads_b = !(n.op == BATCH_COPY || n.op == BATCH_ZERO || (n.op >= EW_ADD_S && n.op <= EW_MULADD_S));
+          const bool reads_r = n.op == EW_MULADD || n.op == EW_MULADD_S;
+          const bool a_is_r = n.op != BATCH_ZERO && (uintptr_t)n.a == r, b_is_r = reads_b && (uintptr_t)n.b == r;
+          if (reads_r && (uintptr_t)n.r == r && !a_is_r && !b_is_r) {
+            // the first thing that happens to the zeros is a product added to them: the product alone
+            n.op = n.op == EW_MULADD ? (u32)EW_MUL : (u32)EW_MUL_S;
+            touched = dead = true;
+          } else if (n.op == EW_ADD && (uintptr_t)n.r == r && a_is_r != b_is_r) {
+            // ... or a sum with them: a copy of the other operand (residues are canonical, 0 + x = x)
+            n = BatchOp{n.r, a_is_r ? n.b : n.a, nullptr, 0, (u32)BATCH_COPY, n.prime};
+            touched = dead = true;
+          } else if (a_is_r || b_is_r || (reads_r && (uintptr_t)n.r == r)) {
+            touched = true;  // read first: the zeros are needed
+          } else if ((uintptr_t)n.r == r) {
+            touched = dead = true;  // written first
+          }
+        }
+        if (!touched && decl_active && !overlaps(decl_reads, r)) {
+          if (inside(decl_writes, r)) dead = true;
+          else if (!overlaps(decl_writes, r)) carry = true;
+        }
+      }
+      if (carry) carried.push_back(o);
+      else if (!dead) kept.push_back(o);
+    }
+    run.ops.swap(kept);
+  }
+  const u64 carried_n = run.n;
+  auto recarry = [&]() {  // the fills that wait: first entries of the next run
+    for (const BatchOp& o : carried) run_append(o, carried_n);
+  };
+  if (run.ops.empty()) {
+    run.touched.clear();
+    run.written.clear();
+    run.rot_res.clear();
+    run.rot_src.clear();
+    recarry();
+    return;
+  }
   size_t count = run.ops.size();
   // Scratch results: entry k's range is read by entry k+1 (which the kernel serves from a register), by nothing
   // else before a later entry overwrites it.  Such a store is dropped, and the range then ties k to k+1 only:
@@ -603,6 +693,12 @@ void ace_ctx::flush_run() {
                                  ((n.a == n.r && n.b == o.r) || (n.b == n.r && n.a == o.r));
         if (sum_to_self) {
           merged.push_back(BatchOp{n.r, o.a, o.b, o.scalar, (u32)(op == EW_MUL ? EW_MULADD : EW_MULADD_S), o.prime});
+          merged_read.push_back(0);
+          ++k;
+          continue;
+        }
+        if (n.op == BATCH_COPY && n.a == o.r && n.r != o.r) {  // ... or by its copy: the product goes there
+          merged.push_back(BatchOp{n.r, o.a, o.b, o.scalar, op, o.prime});
           merged_read.push_back(0);
           ++k;
           continue;
@@ -670,6 +766,7 @@ void ace_ctx::flush_run() {
   run.written.clear();
   run.rot_res.clear();
   run.rot_src.clear();
+  recarry();
   auto compact = [](const BatchOp& o) {
     const u32 op = o.op & ~kBatchDeadStore;
     const bool scalar = op >= EW_ADD_S && op <= EW_MULADD_S;
@@ -1174,12 +1271,12 @@ void ace_free(ace_ctx* c, int64_t* p) {
   if (!p || !c || !c->device_ok) return;
   auto it = c->live.find(p);
   if (it == c->live.end()) return;  // not from ace_alloc of this context (a view, or freed twice)
-  try {
-    c->flush_pending();  // recorded calls may still name this buffer
+  const size_t words = it->second;
+  try {  // recorded calls may still name this buffer; a zero fill of it that nothing has looked at is moot
+    c->flush_pending_declared({ace_ctx::span(p, words)}, {});
   } catch (const std::exception& e) {
     (void)fail(e.what());
   }
-  const size_t words = it->second;
   c->live.erase(it);
   if (c->pooled_words + words <= ace_ctx::kPoolLimitWords) {
     c->pool.emplace(words, p);
@@ -1605,10 +1702,11 @@ int ace_poly_automorphism(ace_ctx* c, int64_t* r, const int64_t* a, const int64_
 }
 
 int ace_decomp_modup(ace_ctx* c, int64_t* res, const int64_t* src, size_t level, size_t part, int is_ntt) {
-  ACE_TRY
+  ACE_TRY_BARE
   if (!res || !src) return fail("ace_decomp_modup: null argument");
   if (!level_ok(c, level)) return fail("ace_decomp_modup: level out of range");
   if (part >= c->h.num_decomp(level)) return fail("ace_decomp_modup: digit index out of range");
+  c->flush_pending_overwriting(res, (level + c->h.K) * (size_t)c->h.N, src, level * (size_t)c->h.N);
   c->ensure_ws(c->std_ws(level));
   c->ws_used = 0;
   do_decomp_modup(c, U(res), U(src) + c->h.part_size * part * (size_t)c->h.N, level, part, is_ntt != 0);
@@ -1616,10 +1714,11 @@ int ace_decomp_modup(ace_ctx* c, int64_t* res, const int64_t* src, size_t level,
 }
 
 int ace_mod_up(ace_ctx* c, int64_t* res, const int64_t* digit, size_t level, size_t part, int is_ntt) {
-  ACE_TRY
+  ACE_TRY_BARE
   if (!res || !digit) return fail("ace_mod_up: null argument");
   if (!level_ok(c, level)) return fail("ace_mod_up: level out of range");
   if (part >= c->h.num_decomp(level)) return fail("ace_mod_up: digit index out of range");
+  c->flush_pending_overwriting(res, (level + c->h.K) * (size_t)c->h.N, digit, c->h.part_size * (size_t)c->h.N);
   c->ensure_ws(c->std_ws(level));
   c->ws_used = 0;
   do_decomp_modup(c, U(res), U(digit), level, part, is_ntt != 0);
@@ -1627,9 +1726,11 @@ int ace_mod_up(ace_ctx* c, int64_t* res, const int64_t* digit, size_t level, siz
 }
 
 int ace_precomp(ace_ctx* c, int64_t* res, const int64_t* src, size_t level, int is_ntt) {
-  ACE_TRY
+  ACE_TRY_BARE
   if (!res || !src) return fail("ace_precomp: null argument");
   if (!level_ok(c, level)) return fail("ace_precomp: level out of range");
+  c->flush_pending_overwriting(res, c->h.num_decomp(level) * (level + c->h.K) * (size_t)c->h.N, src,
+                               level * (size_t)c->h.N);
   c->ensure_ws(c->std_ws(level));
   c->ws_used = 0;
   do_precomp(c, U(res), 0, U(src), 0, 1, level, is_ntt != 0);
@@ -1640,7 +1741,7 @@ int ace_mod_down(ace_ctx* c, int64_t* res, const int64_t* src, size_t level, int
   ACE_TRY_BARE
   if (!res || !src) return fail("ace_mod_down: null argument");
   if (!level_ok(c, level)) return fail("ace_mod_down: level out of range");
-  c->flush_run();
+  c->flush_pending_overwriting(res, level * (size_t)c->h.N, src, (level + c->h.K) * (size_t)c->h.N, true);
   c->submit_poly(1, U(res), U(src), level, is_ntt != 0);
   ACE_CATCH_INT
 }
@@ -1684,7 +1785,7 @@ int ace_rescale(ace_ctx* c, int64_t* res, const int64_t* src, size_t level, int 
   ACE_TRY_BARE
   if (!res || !src) return fail("ace_rescale: null argument");
   if (level < 2 || level > c->h.L) return fail("Level of rescale opnd is too small");
-  c->flush_run();
+  c->flush_pending_overwriting(res, (level - 1) * (size_t)c->h.N, src, level * (size_t)c->h.N, true);
   c->submit_poly(2, U(res), U(src), level, is_ntt != 0);
   ACE_CATCH_INT
 }
@@ -1941,9 +2042,14 @@ int ace_ext_rotate(ace_ctx* c, int64_t* out0, int64_t* out1, const int64_t* digi
 // ---- ciphertext level ------------------------------------------------------------
 int ace_mul_ciph3(ace_ctx* c, int64_t* d0, int64_t* d1, int64_t* d2, const int64_t* a0, const int64_t* a1,
                   const int64_t* b0, const int64_t* b1, size_t level) {
-  ACE_TRY
+  ACE_TRY_BARE
   if (!d0 || !d1 || !d2 || !a0 || !a1 || !b0 || !b1) return fail("ace_mul_ciph3: null argument");
   if (!level_ok(c, level)) return fail("ace_mul_ciph3: level out of range");
+  {
+    const size_t w = level * (size_t)c->h.N;
+    c->flush_pending_declared({ace_ctx::span(d0, w), ace_ctx::span(d1, w), ace_ctx::span(d2, w)},
+                              {ace_ctx::span(a0, w), ace_ctx::span(a1, w), ace_ctx::span(b0, w), ace_ctx::span(b1, w)});
+  }
   launch_tensor(c->stream, c->d, U(d0), U(d1), U(d2), U(a0), U(a1), U(b0), U(b1), c->q_lm, (u32)level, 1, 0, 0, 0);
   ACE_CATCH_INT
 }

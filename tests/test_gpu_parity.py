@@ -993,6 +993,62 @@ def test_recorded_inner_product_through_a_scratch_limb(pair):
         eq(x, w, what)
 
 
+def test_recorded_zero_fills_that_nothing_sees(pair):
+    """Generated code zero-fills every polynomial it allocates and then overwrites or accumulates into it.  Recorded,
+    a fill that is overwritten before it is read is dropped, a product or a sum added to fresh zeros becomes the
+    product or a copy, and a fill the flushing entry point does not touch waits for the next run.  Every buffer must
+    hold what one launch per call leaves -- including a recycled buffer that held other values, which must read as
+    zeros once it is looked at."""
+    g = pair.g
+    N, L, K = g.N, g.L, g.K
+    big_ring_skip(N)
+    level = min(L, 4)
+    T = level
+    mk = lambda seed: np.concatenate([seeded.uniform_poly(seed + t, [g.primes[t]], N) for t in range(T)])
+    hx, hy = mk(7400), mk(7500)
+    hext = seeded.uniform_poly(7600, [g.primes[i] for i in g.limb_primes(level)], N)
+
+    def program():
+        limb = lambda buf, t: buf.view(t * N, N)
+        x, y, ext = g.upload(hx), g.upload(hy), g.upload(hext)
+        dirty = g.alloc(T * N)
+        for t in range(T):
+            g.hw("modadd_scalar", limb(dirty, t), limb(dirty, t), 12345 + t, t)
+        dirty.free()
+        recycled = g.alloc(T * N)  # the buffer that held 12345...: nothing touches it until it is read back
+        acc, via_tmp, over, summed, read_first, doubled, waits = (g.alloc(T * N) for _ in range(7))
+        down, tmp, spare = g.alloc(level * N), g.alloc(N), g.alloc(T * N)
+        for t in range(T):
+            g.hw("modmuladd", limb(acc, t), limb(x, t), limb(y, t), t)  # a product added to fresh zeros
+            g.hw("modmul", tmp, limb(x, t), limb(x, t), t)  # ... through a scratch limb
+            g.hw("modadd", limb(via_tmp, t), limb(via_tmp, t), tmp, t)
+            g.hw("modmul", limb(over, t), limb(y, t), limb(y, t), t)  # overwritten before anyone reads
+            g.hw("modadd", limb(summed, t), limb(y, t), limb(summed, t), t)  # a sum with fresh zeros
+            g.hw("modsub", limb(spare, t), limb(read_first, t), limb(x, t), t)  # the zeros are read
+            g.hw("modadd_scalar", limb(read_first, t), limb(read_first, t), 77, t)
+            g.hw("modadd", limb(doubled, t), limb(doubled, t), limb(doubled, t), t)  # 0 + 0
+            g.hw("modmuladd", limb(acc, t), limb(y, t), limb(y, t), t)  # a second product on top
+        g.mod_down(down, ext, level)  # names its operands: fills of other buffers wait, its result's fill is moot
+        for t in range(T):
+            g.hw("modmuladd_scalar", limb(waits, t), limb(x, t), 3 + t, t)
+        bufs = (acc, via_tmp, over, summed, read_first, doubled, waits, recycled, down, spare)
+        out = [b.get() for b in bufs]
+        for b in bufs + (x, y, ext, tmp):
+            b.free()
+        return out
+
+    g.set_batching(False)
+    want = program()
+    g.set_batching(True)
+    got = program()
+    names = ("product on zeros", "product through a scratch limb", "overwritten", "sum with zeros", "zeros read first",
+             "zeros added to themselves", "fill that waited, then a scalar product", "recycled buffer", "mod_down result",
+             "difference from zeros")
+    for w, x, what in zip(want, got, names):
+        eq(x, w, what)
+    assert not got[7].any() and not got[5].any()
+
+
 def test_key_generation_helpers(pair):
     """ace_expand_small exactly; ace_sample_uniform: in range, reproducible, streams differ, and roughly uniform
     (mean, and a chi-square over 16 buckets at 6 sigma) -- it has no counterpart to compare bits with."""
