@@ -266,6 +266,7 @@ struct ace_ctx {
 
   // FP64 tables of a base conversion (ConvJob::fw / fq) for the targets below kFpConvTargetLimit
   bool conv_fp = true;
+  bool conv_matrix = true;  // base conversions on the matrix cores (ACE_CONV_MATRIX=0 in the environment: off)
   void conv_fp_tables(ConvJob& j, const std::vector<size_t>& src, const std::vector<size_t>& tgt, const u64* hat,
                       size_t hat_stride) {
     j.fw = j.fq = nullptr;
@@ -297,6 +298,48 @@ struct ace_ctx {
     j.fw = upload_vec(fw);
     j.fq = upload_vec(fq);
     j.fw_stride = (u32)nc;
+  }
+
+  // Operands of a base conversion on the matrix cores (ConvJob::mx / mq): for targets j, source k and byte a of
+  // a source word the constant hat_kj * 2^(8a) mod m_j in signed bytes, laid out as the MFMA's A operand: lane l of
+  // (quad, step) holds row l % 32 and inner indices 16 (l / 32) .. + 15, inner index t of step s being byte t % 8 of
+  // source 4 s + t / 8; row rho is byte 4 (rho / 8) + rho % 4 (below 8: the first, from 8: the second) of the two
+  // targets lane half (rho / 4) % 2 finds in its result registers.
+  void conv_matrix_tables(ConvJob& j, const std::vector<size_t>& tgt, const u64* hat, size_t hat_stride, size_t nd) {
+    j.mx = nullptr;
+    j.mt = nullptr;
+    if (nd > 4 * kMxSteps) return;
+    for (size_t p : tgt)
+      if (h.primes[p].q >> 61) return;
+    const size_t nc = tgt.size(), quads = (nc + 3) / 4;
+    std::vector<ConvTarget> mt((quads + 1) * 4, ConvTarget{1, 1.0, 0, 0});  // a spare quad: the kernel reads one ahead
+    std::vector<u64> signed_bytes(nc * nd * 8);
+    for (size_t jj = 0; jj < nc; ++jj) {
+      const u64 q = h.primes[tgt[jj]].q;
+      mt[jj] = ConvTarget{q, (double)(1.0L / (long double)q), (u64)j.map.out_limb[jj] * h.N, 0};
+      for (size_t k = 0; k < nd; ++k) {
+        u64 cst = hat[k * hat_stride + jj] % q;
+        for (size_t a = 0; a < 8; ++a) {
+          signed_bytes[(jj * nd + k) * 8 + a] = (cst + 0x8080808080808080ull) ^ 0x8080808080808080ull;
+          cst = mul_mod(cst, 256 % q, q);
+        }
+      }
+    }
+    std::vector<uint8_t> tab((quads + 1) * kMxSteps * 64 * 16, 0);
+    for (size_t quad = 0; quad < quads; ++quad)
+      for (size_t s = 0; s < kMxSteps; ++s)
+        for (size_t lane = 0; lane < 64; ++lane) {
+          const size_t rho = lane % 32, kb = lane / 32, half = (rho / 4) % 2, r = (rho / 8) * 4 + rho % 4;
+          const size_t jj = quad * 4 + 2 * half + r / 8, byte = r % 8;
+          if (jj >= nc) continue;
+          for (size_t t = 0; t < 16; ++t) {
+            const size_t k = 4 * s + 2 * kb + t / 8, a = t % 8;
+            if (k >= nd) continue;
+            tab[((quad * kMxSteps + s) * 64 + lane) * 16 + t] = (uint8_t)(signed_bytes[(jj * nd + k) * 8 + a] >> (8 * byte));
+          }
+        }
+    j.mx = reinterpret_cast<const uint4*>(upload_vec(tab));
+    j.mt = upload_vec(mt);
   }
 
   void ensure_ws(size_t words) {
@@ -351,6 +394,7 @@ struct ace_ctx {
     m.job.map = m.conv;
     conv_fp_tables(m.job, std::vector<size_t>(m.t.digit.begin(), m.t.digit.end()),
                    std::vector<size_t>(m.t.compl_idx.begin(), m.t.compl_idx.end()), m.t.hat.data(), nc);
+    conv_matrix_tables(m.job, std::vector<size_t>(m.t.compl_idx.begin(), m.t.compl_idx.end()), m.t.hat.data(), nc, nd);
     return modup.emplace(key, std::move(m)).first->second;
   }
 
@@ -429,6 +473,8 @@ struct ace_ctx {
       // FP64 twiddles for the primes the FP64 NTT back end can take
       const char* force_int = std::getenv("ACE_NTT_FORCE_INT");
       conv_fp = !(force_int && force_int[0] == '1');
+      const char* no_matrix = std::getenv("ACE_CONV_MATRIX");
+      conv_matrix = !(no_matrix && no_matrix[0] == '0');
       bool use_fp = conv_fp && h.logN > 12;
       std::vector<double> w(T * h.N, 0.0), iw(T * h.N, 0.0);
       for (size_t i = 0; i < T; ++i) {
@@ -489,6 +535,7 @@ struct ace_ctx {
       p2q_job.nd = (u32)h.K;
       p2q_job.nc = (u32)h.L;
       conv_fp_tables(p2q_job, src, tgt, ph.data(), h.L);
+      conv_matrix_tables(p2q_job, tgt, ph.data(), h.L, h.K);
     }
     pscale_ntt = upload_vec(sn);
     pscale_coef = upload_vec(scf);
@@ -850,6 +897,7 @@ void do_decomp_modup(ace_ctx* c, u64* res, const u64* digit, size_t level, size_
     launch_mul_const(c->stream, c->d, t, digit, m.scale_coef, m.digit_lm, (u32)nd);
   }
   ConvBatch b{};
+  b.matrix = c->conv_matrix;
   b.n_jobs = 1;
   b.job[0] = m.job;
   launch_baseconv(c->stream, c->d, res, t, b, 1);
@@ -886,6 +934,7 @@ void do_precomp(ace_ctx* c, u64* res, u64 res_stride, const u64* src, u64 src_st
                       src_stride, (u32)nb);
   for (size_t j0 = 0; j0 < nd; j0 += kMaxConvJobs) {
     ConvBatch b{};
+    b.matrix = c->conv_matrix;
     b.n_jobs = (u32)std::min<size_t>(kMaxConvJobs, nd - j0);
     for (u32 k = 0; k < b.n_jobs; ++k) b.job[k] = pd.jobs[j0 + k];
     b.t_stride = level * N;
@@ -924,6 +973,7 @@ void do_mod_down(ace_ctx* c, const PolySeq& res, const PolySeq& src, size_t np, 
       launch_mul_const(c->stream, c->d, t + p * K * N, src.at((u32)p) + level * N, c->pscale_coef, c->p_lm, (u32)K);
   }
   ConvBatch b{};
+  b.matrix = c->conv_matrix;
   b.n_jobs = 1;
   b.job[0] = c->p2q_job;
   b.job[0].nc = (u32)level;
@@ -1010,6 +1060,7 @@ void do_moddown_rescale_core(ace_ctx* c, u64* x, u64* y, u64* last_out, u64* pol
   u64* t = c->take(K * N);
   launch_mul_const(c->stream, c->d, t, poly + level * N, c->pscale_coef, c->p_lm, (u32)K);
   ConvBatch b{};
+  b.matrix = c->conv_matrix;
   b.n_jobs = 1;
   b.job[0] = c->p2q_job;
   b.job[0].nc = (u32)level;

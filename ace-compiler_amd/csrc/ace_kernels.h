@@ -16,9 +16,21 @@ constexpr int kMaxConvJobs = 4;   // digits converted per base-conversion launch
 // fw: [3 nd][fw_stride][2] = the halves above and below bit 26 of hat * 2^(21 i) mod m_j as doubles (plus a margin of
 //     four entries); fq: [nc][2] = (m_j, 1 / m_j);
 // fp_target[j] says whether target j uses them.
+// mx: operands of the conversion on the matrix cores (null: not available for this job), [quad][kMxSteps][64 lanes]
+//     of 16 bytes each, a quad being four consecutive targets and a step four source limbs; mt: [4 quads] for each
+//     target its modulus, the reciprocal as a double and the word offset of its limb in the output polynomial.
+constexpr u32 kMxSteps = 4;
+struct ConvTarget {
+  u64 m;
+  double minv;
+  u64 out_off;
+  u64 pad;
+};
 struct ConvJob {
   const u64* hat;
   u32 hat_stride, nd, nc;
+  const uint4* mx;
+  const ConvTarget* mt;
   u64 t_off, out_off;  // word offsets of this job's source limbs / output polynomial inside one operand
   ConvMap map;
   const double* fw;
@@ -29,6 +41,7 @@ struct ConvJob {
 struct ConvBatch {
   ConvJob job[kMaxConvJobs];
   u32 n_jobs;
+  u32 matrix;                // take the matrix-core kernel where the jobs have its tables
   u64 t_stride, out_stride;  // word strides between operands
 };
 struct KeySet {   // one switch key per operand, or one shared by all (n == 1)

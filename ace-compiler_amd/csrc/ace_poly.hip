@@ -523,6 +523,132 @@ __global__ __launch_bounds__(kThreads) void baseconv_kernel(DevCtx c, u64* __res
   }
 }
 
+// ---- the same conversion on the matrix cores ------------------------------------------------------------------
+// out_j = sum_k x_k * hat_kj (mod m_j) is a matrix product over the bytes of the source words: with the signed bytes
+// d_ka of x_k (x_k = sum_a d_ka 2^(8a), d in [-128, 127]) and the constants C_kaj = hat_kj * 2^(8a) mod m_j cut
+// into signed bytes the same way (C = sum_p e_kajp 2^(8p)), V_j = sum_p 2^(8p) sum_(k,a) d_ka e_kajp is congruent to
+// the sum mod m_j.  The inner sums are one int8 MFMA product: rows (target, p), columns = coefficients, inner index
+// (k, a) -- a source word as it lies in memory is eight consecutive inner indices.  |V_j| < 2^14 m_j, so the
+// quotient has 15 bits, an FP64 estimate of it is off by less than one, and V_j - Q m_j is taken in wrapping 64-bit
+// arithmetic: the canonical residue, the same word the multiply-accumulate path gives.
+// v_mfma_i32_32x32x32_i8: lane l holds row (column) l % 32 and inner indices 16 (l / 32) .. + 15 of the A (B) operand;
+// result register r of lane l is row 8 (r / 4) + 4 (l / 32) + r % 4 of column l % 32.  The table's rows are permuted so
+// that registers 0-7 of a lane are the eight byte sums of target 2 (l / 32) of the quad, registers 8-15 those of target
+// 2 (l / 32) + 1.
+// Source words must be below 2^63 - 2^56 (residues of primes below 2^61 are).
+typedef int conv_v16i __attribute__((ext_vector_type(16)));
+typedef int conv_v4i __attribute__((ext_vector_type(4)));
+constexpr u64 kSignedBytes = 0x8080808080808080ull;
+constexpr u32 kMxThreads = 256, kMxCoefPerBlock = 64 * (kMxThreads / 64);
+
+// one quad of targets for the wave's two tiles; FULL: all four targets exist (no lane is left out, so the stores
+// are unconditional and the waits the compiler places do not have to allow for a path without them)
+template <int STEPS, bool FULL>
+__device__ __forceinline__ void conv_mx_quad(const uint4 (&row)[STEPS], const ConvTarget (&tg)[2],
+                                             const conv_v4i (&x)[2][STEPS], u64* __restrict__ out, u32 first_target,
+                                             u32 nc) {
+  conv_v16i acc[2];
+#pragma unroll
+  for (u32 tile = 0; tile < 2; ++tile) {
+    acc[tile] = conv_v16i{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      const conv_v4i a = {(int)row[s].x, (int)row[s].y, (int)row[s].z, (int)row[s].w};
+      acc[tile] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, x[tile][s], acc[tile], 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int w = 0; w < 2; ++w) {
+    const u64 m = tg[w].m;
+    u64 res[2];
+#pragma unroll
+    for (u32 tile = 0; tile < 2; ++tile) {
+      const conv_v16i& S = acc[tile];
+      // byte sums are below 2^21 in size: two of them, one shifted by a byte, fit a 32-bit word
+      const int u0 = S[8 * w + 0] + (S[8 * w + 1] << 8), v0 = S[8 * w + 2] + (S[8 * w + 3] << 8);
+      const int u1 = S[8 * w + 4] + (S[8 * w + 5] << 8), v1 = S[8 * w + 6] + (S[8 * w + 7] << 8);
+      const i64 t0 = (i64)u0 + ((i64)v0 << 16), t1 = (i64)u1 + ((i64)v1 << 16);
+      const u64 v_lo = (u64)t0 + ((u64)t1 << 32);  // V mod 2^64
+      const double d0 = __builtin_fma((double)v0, 65536.0, (double)u0);  // exact
+      const double d1 = __builtin_fma((double)v1, 65536.0, (double)u1);
+      const double vd = __builtin_fma(d1, 4294967296.0, d0);  // V to 53 bits
+      // |V / m| < 2^14 and the estimate is off by far less than 1/2: V - Q m lies within (1/2 + 2^-30) m of zero
+      const int quot = (int)__builtin_rint(vd * tg[w].minv);
+      const i64 r = (i64)(v_lo - (u64)(i64)quot * m);
+      res[tile] = (u64)(r < 0 ? r + (i64)m : r);
+    }
+    if (FULL || first_target + w < nc)
+      *reinterpret_cast<ulonglong2*>(out + tg[w].out_off) = make_ulonglong2(res[0], res[1]);
+  }
+}
+
+// A wave converts 64 coefficients as two tiles of 32 (lane column c of tile e is coefficient 2 c + e, so a lane
+// loads and stores its two coefficients as one 16-byte word), one quad of targets after the other; the table rows of
+// the next quad are requested before the current one is worked on (the tables end with a spare quad).
+template <int STEPS>
+__global__ __launch_bounds__(kMxThreads) void baseconv_mx_kernel(DevCtx c, u64* __restrict__ out_base,
+                                                                 const u64* __restrict__ t_base, ConvBatch b,
+                                                                 u32 quads_per_block) {
+  const u64 n = c.N;
+  const u32 lane = threadIdx.x & 63, half = lane >> 5;
+  const u64 i = ((u64)blockIdx.x * (kMxThreads / 64) + (threadIdx.x >> 6)) * 64 + 2 * (lane & 31);
+  const u32 jobi = blockIdx.z % b.n_jobs, op = blockIdx.z / b.n_jobs;
+  const ConvJob& J = b.job[jobi];
+  const u32 nd = J.nd, nc = J.nc;
+  const u32 quad0 = blockIdx.y * quads_per_block;
+  if (quad0 * 4 >= nc) return;
+  const u32 quad1 = min(quad0 + quads_per_block, (nc + 3) / 4);
+  const u32 full1 = min(quad1, nc / 4);  // quads below this one have all four targets
+  const u64* __restrict__ t = t_base + op * b.t_stride + J.t_off + i;
+  u64* __restrict__ out = out_base + op * b.out_stride + J.out_off + i;
+  conv_v4i x[2][STEPS];
+  {
+    ulonglong2 v[STEPS][2];
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s)
+#pragma unroll
+      for (int w = 0; w < 2; ++w) {
+        const u32 k = 4 * s + 2 * half + w;
+        v[s][w] = *reinterpret_cast<const ulonglong2*>(t + (u64)min(k, nd - 1) * n);
+      }
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s)
+#pragma unroll
+      for (int w = 0; w < 2; ++w) {
+        const bool live = 4 * s + 2 * half + w < nd;
+        const u64 e0 = live ? (v[s][w].x + kSignedBytes) ^ kSignedBytes : 0;
+        const u64 e1 = live ? (v[s][w].y + kSignedBytes) ^ kSignedBytes : 0;
+        x[0][s][2 * w] = (int)(u32)e0;
+        x[0][s][2 * w + 1] = (int)(u32)(e0 >> 32);
+        x[1][s][2 * w] = (int)(u32)e1;
+        x[1][s][2 * w + 1] = (int)(u32)(e1 >> 32);
+      }
+  }
+  const uint4* __restrict__ mx = J.mx + (u64)quad0 * kMxSteps * 64 + lane;
+  const ConvTarget* __restrict__ mt = J.mt + quad0 * 4 + 2 * half;
+  uint4 row[STEPS];
+  ConvTarget tg[2];
+#pragma unroll
+  for (int s = 0; s < STEPS; ++s) row[s] = mx[s * 64];
+  tg[0] = mt[0];
+  tg[1] = mt[1];
+  u32 quad = quad0;
+  for (; quad < full1; ++quad) {
+    mx += kMxSteps * 64;
+    mt += 4;
+    uint4 row_next[STEPS];
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) row_next[s] = mx[s * 64];
+    const ConvTarget tg_next[2] = {mt[0], mt[1]};
+    conv_mx_quad<STEPS, true>(row, tg, x, out, quad * 4 + 2 * half, nc);
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) row[s] = row_next[s];
+    tg[0] = tg_next[0];
+    tg[1] = tg_next[1];
+  }
+  if (quad < quad1) conv_mx_quad<STEPS, false>(row, tg, x, out, quad * 4 + 2 * half, nc);
+}
+
 // register-array size used for nd source limbs (0: the looped kernel)
 static int conv_padded_sources(u32 nd) { return nd <= 4 ? 4 : nd <= 8 ? 8 : nd <= 12 ? 12 : nd <= 16 ? 16 : 0; }
 
@@ -536,6 +662,27 @@ void launch_baseconv(hipStream_t st, const DevCtx& c, u64* out, const u64* t, co
     fp &= b.job[k].fw != nullptr;
   }
   if (!max_nc) return;
+  bool mx = b.matrix && c.N % kMxCoefPerBlock == 0 && max_nd <= 4 * kMxSteps &&
+            ((uintptr_t)out | (uintptr_t)t) % 16 == 0 && (b.out_stride | b.t_stride) % 2 == 0;
+  for (u32 k = 0; k < b.n_jobs; ++k) mx &= b.job[k].mx != nullptr;
+  if (mx) {
+    const u32 quads = (max_nc + 3) / 4, steps = (max_nd + 3) / 4;
+    // all targets of a job in one block (the source words are loaded once) unless that leaves the machine empty
+    const u32 blocks = (u32)(c.N / kMxCoefPerBlock) * b.n_jobs * n_ops;
+    u32 split = blocks >= 1024 ? 1 : (1024 + blocks - 1) / blocks;
+    split = split > quads ? quads : split;
+    const u32 per_block = (quads + split - 1) / split;
+    dim3 g((u32)(c.N / kMxCoefPerBlock), (quads + per_block - 1) / per_block, b.n_jobs * n_ops);
+#define ACE_BCX(S) hipLaunchKernelGGL((baseconv_mx_kernel<S>), g, dim3(kMxThreads), 0, st, c, out, t, b, per_block)
+    switch (steps) {
+      case 1: ACE_BCX(1); break;
+      case 2: ACE_BCX(2); break;
+      case 3: ACE_BCX(3); break;
+      default: ACE_BCX(4); break;
+    }
+#undef ACE_BCX
+    return;
+  }
   const int maxs = conv_padded_sources(max_nd);
   dim3 g((c.N + kThreads - 1) / kThreads, (max_nc + kConvTargets - 1) / kConvTargets, b.n_jobs * n_ops);
 #define ACE_BC(S, M) hipLaunchKernelGGL((baseconv_kernel<S, M>), g, dim3(kThreads), 0, st, c, out, t, b)

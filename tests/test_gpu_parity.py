@@ -173,6 +173,61 @@ def test_conversion_with_a_51_bit_first_prime():
         o.close()
 
 
+@pytest.mark.parametrize("matrix", ["1", "0"], ids=["matrix_cores", "vector_units"])
+@pytest.mark.parametrize("cfg", [(8192, 7, 51, 46, 3), (2048, 9, 60, 56, 3), (256, 5, 60, 59, 2), (65536, 13, 60, 56, 4)],
+                         ids=lambda c: "N%d_L%d_%d_%d" % c[:4])
+def test_conversion_on_the_matrix_cores_and_on_the_vector_units(cfg, matrix, monkeypatch):
+    """The base conversion has two implementations for rings of 256 coefficients and more: int8 matrix products over
+    the signed bytes of the source words (the default) and 128-bit / FP64 multiply-accumulates (ACE_CONV_MATRIX=0 when
+    the context is made).  Both must give the oracle's words, also where the words entering the conversion are
+    m-1, (m+1)/2, 1, or have every byte at 0x80, 0x7F or 0xFF (where the signed bytes carry), in every source limb."""
+    monkeypatch.setenv("ACE_CONV_MATRIX", matrix)
+    g, o = acefhe.Context(*cfg), Oracle(*cfg)
+    try:
+        N, level = g.N, g.L
+        q = [int(x) for x in g.primes[:level]]
+        rng = np.random.Generator(np.random.PCG64(77))
+        for case in range(3):
+            limbs = []
+            for t in range(level):
+                part = t // g.part_size
+                digit = q[part * g.part_size:min(level, (part + 1) * g.part_size)]
+                rest = 1
+                for m in digit:
+                    rest *= m if m != q[t] else 1
+                want = [q[t] - 1, (q[t] + 1) // 2, 1, 0x8080808080808080 % q[t], 0x7F7F7F7F7F7F7F7F % q[t],
+                        0xFFFFFFFFFFFFFFFF % q[t], 0x0080008000800080 % q[t]]
+                pool = np.array([(v * rest) % q[t] for v in want], np.int64)  # times (Q_d / q_t)^-1 these become `want`
+                if case == 2:
+                    limbs.append(rng.integers(0, q[t], N))
+                else:
+                    limbs.append(pool[rng.integers(0, len(pool), N)] if case else np.full(N, pool[0]))
+            x = np.concatenate(limbs).astype(np.int64)
+            dx = g.upload(x)
+            for is_ntt in (False, True):
+                dr = g.alloc(g.num_decomp(level) * (level + g.K) * N)
+                g.precomp(dr, dx, level, is_ntt)
+                eq(dr, o.precomp(x, level, is_ntt), "precomp case %d ntt %d" % (case, is_ntt))
+                dr.free()
+            dx.free()
+        for lvl in sorted({level, max(1, level - 3)}):
+            pr = [g.primes[i] for i in g.limb_primes(lvl)]
+            for case in range(2):
+                e = seeded.uniform_poly(5200 + case, pr, N)
+                if case:  # the largest source words
+                    e = np.concatenate([np.full(N, int(m) - 1, np.int64) for m in pr])
+                de = g.upload(e)
+                for is_ntt in (False, True):
+                    dr = g.alloc(lvl * N)
+                    g.mod_down(dr, de, lvl, is_ntt)
+                    eq(dr, o.mod_down(e, lvl, is_ntt), "mod_down level %d case %d ntt %d" % (lvl, case, is_ntt))
+                    dr.free()
+                de.free()
+    finally:
+        g.close()
+        o.close()
+
+
 def test_ntt_batched_polys(pair):
     g, o = pair.g, pair.o
     N = g.N
