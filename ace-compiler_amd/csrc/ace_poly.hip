@@ -68,14 +68,15 @@ __global__ __launch_bounds__(kThreads) void plain_mac_kernel(DevCtx c, u64* __re
   const u64 pbase = (u64)(limb < level ? limb : plain_level + (limb - level)) * n;
 #pragma unroll
   ACE_EW_LOOP(i, n) {
-    u64 s0 = accumulate ? r0[base + i] : 0, s1 = accumulate ? r1[base + i] : 0;
+    // summed in 128 bits, reduced once: at most kMaxMacOps = 32 products of residues below 2^61 and the running sum
+    u64 l0 = accumulate ? r0[base + i] : 0, l1 = accumulate ? r1[base + i] : 0, h0 = 0, h1 = 0;
     for (u32 j = 0; j < ops.n; ++j) {
       u64 w = ops.p[j][pbase + i];
-      s0 = add_mod(s0, mulmod(ops.a0[j][base + i], w, P), P.q);
-      s1 = add_mod(s1, mulmod(ops.a1[j][base + i], w, P), P.q);
+      mac128(h0, l0, ops.a0[j][base + i], w);
+      mac128(h1, l1, ops.a1[j][base + i], w);
     }
-    r0[base + i] = s0;
-    r1[base + i] = s1;
+    r0[base + i] = barrett128(h0, l0, P);
+    r1[base + i] = barrett128(h1, l1, P);
   }
 }
 void launch_plain_mac(hipStream_t st, const DevCtx& c, u64* r0, u64* r1, const MacSet& ops, const LimbMap& lm,
@@ -93,12 +94,15 @@ __global__ __launch_bounds__(kThreads) void plain_mac_groups_kernel(DevCtx c, Ma
   const u64 pbase = (u64)(limb < level ? limb : plain_level + (limb - level)) * n;
 #pragma unroll
   ACE_EW_LOOP(i, n) {
-    u64 s0[kMacGroups], s1[kMacGroups];
+    // The products of a group are summed in 128 bits and reduced once (at most kMaxMacOps = 32 products of residues
+    // below 2^61, plus the running sum: below 2^128); the canonical residue is the one a reduction per product gives.
+    u64 l0[kMacGroups], h0[kMacGroups], l1[kMacGroups], h1[kMacGroups];
 #pragma unroll
     for (int g = 0; g < kMacGroups; ++g) {
       const bool on = g < (int)ops.n_groups && accumulate;
-      s0[g] = on ? ops.r0[g][base + i] : 0;
-      s1[g] = on ? ops.r1[g][base + i] : 0;
+      l0[g] = on ? ops.r0[g][base + i] : 0;
+      l1[g] = on ? ops.r1[g][base + i] : 0;
+      h0[g] = h1[g] = 0;
     }
     for (u32 j = 0; j < ops.n_ops; ++j) {
       const u64 x0 = ops.a0[j][base + i], x1 = ops.a1[j][base + i];
@@ -106,16 +110,16 @@ __global__ __launch_bounds__(kThreads) void plain_mac_groups_kernel(DevCtx c, Ma
       for (int g = 0; g < kMacGroups; ++g) {
         if (g < (int)ops.n_groups && ops.p[g][j]) {
           const u64 w = ops.p[g][j][pbase + i];
-          s0[g] = add_mod(s0[g], mulmod(x0, w, P), P.q);
-          s1[g] = add_mod(s1[g], mulmod(x1, w, P), P.q);
+          mac128(h0[g], l0[g], x0, w);
+          mac128(h1[g], l1[g], x1, w);
         }
       }
     }
 #pragma unroll
     for (int g = 0; g < kMacGroups; ++g) {
       if (g < (int)ops.n_groups) {
-        ops.r0[g][base + i] = s0[g];
-        ops.r1[g][base + i] = s1[g];
+        ops.r0[g][base + i] = barrett128(h0[g], l0[g], P);
+        ops.r1[g][base + i] = barrett128(h1[g], l1[g], P);
       }
     }
   }
@@ -308,14 +312,16 @@ __global__ __launch_bounds__(kThreads) void wsum_kernel(DevCtx c, u64* __restric
   const u64 base = (u64)limb * n;
 #pragma unroll
   ACE_EW_LOOP(i, n) {
-    u64 s0 = 0, s1 = 0;
+    // summed in 128 bits, reduced once: at most kMaxMacOps = 32 products of residues below 2^61 (the weights are
+    // checked to be residues by the caller)
+    u64 l0 = 0, l1 = 0, h0 = 0, h1 = 0;
     for (u32 j = 0; j < ops.n; ++j) {
       u64 v = w[j * n_limbs + limb];
-      s0 = add_mod(s0, mulmod(ops.a0[j][base + i], v, P), P.q);
-      s1 = add_mod(s1, mulmod(ops.a1[j][base + i], v, P), P.q);
+      mac128(h0, l0, ops.a0[j][base + i], v);
+      mac128(h1, l1, ops.a1[j][base + i], v);
     }
-    r0[base + i] = s0;
-    r1[base + i] = s1;
+    r0[base + i] = barrett128(h0, l0, P);
+    r1[base + i] = barrett128(h1, l1, P);
   }
 }
 void launch_wsum(hipStream_t st, const DevCtx& c, u64* r0, u64* r1, const MacSet& ops, const u64* w,
