@@ -88,6 +88,8 @@ def _sig(lib):
     f("ace_precomp", C.c_int, _vp, _vp, _vp, _sz, C.c_int)
     f("ace_mod_down", C.c_int, _vp, _vp, _vp, _sz, C.c_int)
     f("ace_mod_down_noalloc", C.c_int, _vp, _vp, _vp, _sz, C.c_int)
+    f("ace_precomp_batch", C.c_int, _vp, _vp, _sz, _vp, _sz, _sz, _sz, C.c_int)
+    f("ace_mod_down_batch", C.c_int, _vp, _vp, _sz, _vp, _sz, _sz, _sz, C.c_int)
     f("ace_rescale", C.c_int, _vp, _vp, _vp, _sz, C.c_int)
     f("ace_extend", C.c_int, _vp, _vp, _vp, _sz)
     f("ace_dot_prod", C.c_int, _vp, _vp, _vp, _vp, _sz, _sz, _sz)
@@ -111,7 +113,7 @@ def _sig(lib):
 
 # every symbol include/ace_hip.h declares
 EXPORTS = [
-    "ace_mod_down_noalloc", "ace_sample_uniform", "ace_expand_small", "ace_set_batching", "ace_ext_plain_mac", "ace_poly_add_scalars", "ace_poly_mul_scalars", "ace_ciph_wsum", "ace_alloc_uninit", "ace_ctx_create", "ace_ctx_create_with_primes", "ace_ctx_destroy", "ace_has_device", "ace_last_error",
+    "ace_mod_down_noalloc", "ace_precomp_batch", "ace_mod_down_batch", "ace_sample_uniform", "ace_expand_small", "ace_set_batching", "ace_ext_plain_mac", "ace_poly_add_scalars", "ace_poly_mul_scalars", "ace_ciph_wsum", "ace_alloc_uninit", "ace_ctx_create", "ace_ctx_create_with_primes", "ace_ctx_destroy", "ace_has_device", "ace_last_error",
     "ace_degree", "ace_num_q", "ace_num_p", "ace_num_parts", "ace_part_size", "ace_num_decomp", "ace_prime",
     "ace_root", "ace_modulus", "ace_host_twiddles", "ace_host_tbl_modup", "ace_host_tbl_moddown",
     "ace_host_tbl_rescale", "ace_host_automorphism_order", "ace_alloc", "ace_free", "ace_upload", "ace_download",
@@ -380,6 +382,12 @@ class Context:
 
     def mod_down(self, res, src, level, is_ntt=True):
         self._chk(self.lib.ace_mod_down(self.h, res.ptr, src.ptr, level, int(is_ntt)))
+
+    def precomp_batch(self, res, res_stride, src, src_stride, count, level, is_ntt=True):
+        self._chk(self.lib.ace_precomp_batch(self.h, res.ptr, res_stride, src.ptr, src_stride, count, level, int(is_ntt)))
+
+    def mod_down_batch(self, res, res_stride, src, src_stride, count, level, is_ntt=True):
+        self._chk(self.lib.ace_mod_down_batch(self.h, res.ptr, res_stride, src.ptr, src_stride, count, level, int(is_ntt)))
 
     def mod_down_noalloc(self, res, src, level, is_ntt=True):
         self._chk(self.lib.ace_mod_down_noalloc(self.h, res.ptr, src.ptr, level, int(is_ntt)))

@@ -1797,6 +1797,52 @@ int ace_mod_down(ace_ctx* c, int64_t* res, const int64_t* src, size_t level, int
   ACE_CATCH_INT
 }
 
+// Precomp / Mod_down of `count` polynomials at constant strides in one set of launches
+static int batch_args_ok(const char* who, const void* res, size_t res_stride, size_t res_words, const void* src,
+                         size_t src_stride, size_t src_words, size_t count) {
+  if (!res || !src) return fail(std::string(who) + ": null argument");
+  if (!count) return fail(std::string(who) + ": count is zero");
+  if (count > 1 && (res_stride < res_words || src_stride < src_words))
+    return fail(std::string(who) + ": a stride is shorter than the polynomial it steps over");
+  const uintptr_t r0 = (uintptr_t)res, r1 = r0 + ((count - 1) * res_stride + res_words) * sizeof(u64);
+  const uintptr_t s0 = (uintptr_t)src, s1 = s0 + ((count - 1) * src_stride + src_words) * sizeof(u64);
+  if (r0 < s1 && s0 < r1) return fail(std::string(who) + ": results and operands overlap");
+  return 0;
+}
+
+int ace_precomp_batch(ace_ctx* c, int64_t* res, size_t res_stride, const int64_t* src, size_t src_stride, size_t count,
+                      size_t level, int is_ntt) {
+  ACE_TRY_BARE
+  if (!level_ok(c, level)) return fail("ace_precomp_batch: level out of range");
+  const size_t N = c->h.N, res_words = c->h.num_decomp(level) * (level + c->h.K) * N, src_words = level * N;
+  if (int rc = batch_args_ok("ace_precomp_batch", res, res_stride, res_words, src, src_stride, src_words, count)) return rc;
+  // only a result range without gaps is overwritten as a whole
+  if (res_stride == res_words || count == 1)
+    c->flush_pending_overwriting(res, ((count - 1) * res_stride + res_words), src, (count - 1) * src_stride + src_words);
+  else
+    c->flush_pending();
+  c->ensure_ws(c->std_ws(level) * count);
+  c->ws_used = 0;
+  do_precomp(c, U(res), res_stride, U(src), src_stride, count, level, is_ntt != 0);
+  ACE_CATCH_INT
+}
+
+int ace_mod_down_batch(ace_ctx* c, int64_t* res, size_t res_stride, const int64_t* src, size_t src_stride, size_t count,
+                       size_t level, int is_ntt) {
+  ACE_TRY_BARE
+  if (!level_ok(c, level)) return fail("ace_mod_down_batch: level out of range");
+  const size_t N = c->h.N, res_words = level * N, src_words = (level + c->h.K) * N;
+  if (int rc = batch_args_ok("ace_mod_down_batch", res, res_stride, res_words, src, src_stride, src_words, count)) return rc;
+  if (res_stride == res_words || count == 1)
+    c->flush_pending_overwriting(res, ((count - 1) * res_stride + res_words), src, (count - 1) * src_stride + src_words);
+  else
+    c->flush_pending();
+  c->ensure_ws(c->std_ws(level) * count);
+  c->ws_used = 0;
+  do_mod_down(c, seq_strided(U(res), res_stride), seq_strided(U(src), src_stride), count, level, is_ntt != 0, nullptr, 0);
+  ACE_CATCH_INT
+}
+
 int ace_mod_down_noalloc(ace_ctx* c, int64_t* res, const int64_t* src, size_t level, int is_ntt) {
   ACE_TRY_BARE
   if (!res || !src) return fail("ace_mod_down_noalloc: null argument");

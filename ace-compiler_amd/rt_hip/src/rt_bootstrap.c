@@ -541,7 +541,7 @@ static void rotate_iteration(CIPHER ct, BTS_PRECOM* pre, bool encoding, int32_t 
   ACE_OK(ace_precomp(G.ctx, digits, ct->_c1_poly._data, level, 1));
   int64_t* c0_ext = Rt_dev_alloc_raw(T * n);
   ACE_OK(ace_extend(G.ctx, c0_ext, ct->_c0_poly._data, level));
-  EXT_CT  inner = ext_alloc(level), outer = ext_alloc(level);
+  EXT_CT  outer = ext_alloc(level);
   EXT_CT* rots = (EXT_CT*)calloc((size_t)r.giant, sizeof(EXT_CT));
   for (int32_t j = 0; j < r.giant; ++j) {
     rots[j] = ext_alloc(level);
@@ -552,10 +552,12 @@ static void rotate_iteration(CIPHER ct, BTS_PRECOM* pre, bool encoding, int32_t 
       ACE_OK(ace_extend(G.ctx, rots[j].c1, ct->_c1_poly._data, level));
     }
   }
-  int64_t* low = Rt_dev_alloc_raw(level * n);
-  int64_t* low_digits = Rt_dev_alloc_raw(nd * T * n);
   /* the inner sums of all baby-step groups first: the groups share the rotated ciphertexts, which are read once
-   * for every four groups (ace_ext_plain_mac_groups) */
+   * for every four groups (ace_ext_plain_mac_groups).  The sums lie side by side in one buffer, so that the c1 parts
+   * of consecutive groups are a sequence at a constant stride for the batched calls below. */
+  int64_t*        inner_slab = Rt_dev_alloc_raw((size_t)r.baby * 2 * T * n);
+  int64_t*        low        = Rt_dev_alloc_raw((size_t)r.baby * level * n);
+  int64_t*        low_digits = Rt_dev_alloc_raw((size_t)r.baby * nd * T * n);
   EXT_CT*         inners = (EXT_CT*)calloc((size_t)r.baby, sizeof(EXT_CT));
   int64_t **      in_r0 = (int64_t**)calloc((size_t)r.baby, sizeof(int64_t*)), **in_r1 = (int64_t**)calloc((size_t)r.baby, sizeof(int64_t*));
   const int64_t** inp   = (const int64_t**)calloc((size_t)r.baby * (size_t)r.giant, sizeof(int64_t*));
@@ -567,7 +569,8 @@ static void rotate_iteration(CIPHER ct, BTS_PRECOM* pre, bool encoding, int32_t 
     in1[j] = rots[j].c1;
   }
   for (int32_t i = 0; i < r.baby; ++i) {
-    inners[i] = i == 0 ? inner : ext_alloc(level);
+    inners[i].c0 = inner_slab + (size_t)i * 2 * T * n;
+    inners[i].c1 = inners[i].c0 + T * n;
     in_r0[i]  = inners[i].c0;
     in_r1[i]  = inners[i].c1;
     for (int32_t j = 0; j < r.giant; ++j) {
@@ -582,23 +585,32 @@ static void rotate_iteration(CIPHER ct, BTS_PRECOM* pre, bool encoding, int32_t 
   /* The result is sum_i rotation_i(inner sum i).  Group 0 is not rotated: its two halves start the running sums
    * `first` (c0 parts that need no key switch) and `sum1`.  A rotated group's c1 part is brought down, raised again
    * and rotated with its key; its c0 part rides along as the addend; both land in (outer.c0, sum1). */
+  /* One polynomial's Mod_down and Precomp leave most of the machine idle, so consecutive rotated groups go through
+   * them together (ace_mod_down_batch, ace_precomp_batch: the words of single calls). */
   int64_t *first = inners[0].c0, *sum1 = inners[0].c1;
   bool     outer0_set = false;
-  for (int32_t i = 1; i < r.baby; ++i) {
+  for (int32_t i = 1; i < r.baby;) {
     EXT_CT* in = &inners[i];
-    if (r.out[i] != 0) {
-      ACE_OK(ace_mod_down(G.ctx, low, in->c1, level, 1));
-      ACE_OK(ace_precomp(G.ctx, low_digits, low, level, 1));
-      EXT_CT into = {outer.c0, sum1};
-      ext_rotate(&into, low_digits, nd, in->c0, r.out[i], level, (outer0_set ? 1 : 0) | 2);
-      outer0_set = true;
-    } else {
+    if (r.out[i] == 0) {
       ACE_OK(ace_poly_add(G.ctx, first, first, in->c0, level, 1));
       ACE_OK(ace_poly_add(G.ctx, sum1, sum1, in->c1, level, 1));
+      ++i;
+      continue;
     }
+    int32_t end = i;
+    while (end < r.baby && r.out[end] != 0) ++end;
+    size_t cnt = (size_t)(end - i);
+    ACE_OK(ace_mod_down_batch(G.ctx, low, level * n, in->c1, 2 * T * n, cnt, level, 1));
+    ACE_OK(ace_precomp_batch(G.ctx, low_digits, nd * T * n, low, level * n, cnt, level, 1));
+    for (int32_t g = i; g < end; ++g) {
+      EXT_CT into = {outer.c0, sum1};
+      ext_rotate(&into, low_digits + (size_t)(g - i) * nd * T * n, nd, inners[g].c0, r.out[g], level,
+                 (outer0_set ? 1 : 0) | 2);
+      outer0_set = true;
+    }
+    i = end;
   }
   if (outer0_set) ACE_OK(ace_poly_add(G.ctx, first, first, outer.c0, level, 1));
-  for (int32_t i = 1; i < r.baby; ++i) ext_free(&inners[i]);
   free(inners);
   free(in_r0);
   free(in_r1);
@@ -610,7 +622,7 @@ static void rotate_iteration(CIPHER ct, BTS_PRECOM* pre, bool encoding, int32_t 
 
   for (int32_t j = 0; j < r.giant; ++j) ext_free(&rots[j]);
   free(rots);
-  ext_free(&inner);
+  Rt_dev_free(inner_slab);
   ext_free(&outer);
   Rt_dev_free(digits);
   Rt_dev_free(c0_ext);

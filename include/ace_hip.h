@@ -198,6 +198,14 @@ int ace_mod_up(ace_ctx* ctx, int64_t* res, const int64_t* digit, size_t level, s
 int ace_precomp(ace_ctx* ctx, int64_t* res, const int64_t* src, size_t level, int is_ntt);
 /* Mod_down (:260-308): src level+num_p limbs -> res level limbs */
 int ace_mod_down(ace_ctx* ctx, int64_t* res, const int64_t* src, size_t level, int is_ntt);
+/* Precomp (:416-481) / Mod_down (:260-308) of `count` polynomials in one set of launches: polynomial o is read at
+ * src + o * src_stride and written at res + o * res_stride (strides in words, at least the size of one operand /
+ * result; results and operands must not overlap).  The words are those of `count` single calls; the batch exists
+ * because one polynomial's kernels leave most of the machine idle (the rotated inner sums of a bootstrap level). */
+int ace_precomp_batch(ace_ctx* ctx, int64_t* res, size_t res_stride, const int64_t* src, size_t src_stride,
+                      size_t count, size_t level, int is_ntt);
+int ace_mod_down_batch(ace_ctx* ctx, int64_t* res, size_t res_stride, const int64_t* src, size_t src_stride,
+                       size_t count, size_t level, int is_ntt);
 /* Mod_down for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same operands and result as ace_mod_down;
  * the intermediates live in a 16 MiB device array that is part of the library image (one copy per GPU, held until

@@ -228,6 +228,38 @@ def test_conversion_on_the_matrix_cores_and_on_the_vector_units(cfg, matrix, mon
         o.close()
 
 
+def test_precomp_and_mod_down_batches_equal_single_calls(pair):
+    """ace_precomp_batch / ace_mod_down_batch over polynomials at a constant stride (with a gap between them, as the
+    c1 halves of a bootstrap level's inner sums lie) give the words of one call per polynomial, which the oracle pins."""
+    g, o = pair.g, pair.o
+    N, K = g.N, g.K
+    big_ring_skip(N)
+    count = 3
+    for level in levels_of(g)[-2:]:
+        T, nd = level + K, g.num_decomp(level)
+        pr = [g.primes[i] for i in g.limb_primes(level)]
+        for is_ntt in (True, False):
+            ext = [seeded.uniform_poly(7700 + 10 * level + k, pr, N) for k in range(count)]
+            stride = 2 * T * N  # every other polynomial of the buffer
+            slab = np.zeros(count * stride, np.int64)
+            for k in range(count):
+                slab[k * stride + T * N:(k + 1) * stride] = ext[k]
+            dslab = g.upload(slab)
+            low = g.alloc(count * level * N)
+            g.mod_down_batch(low, level * N, dslab.view(T * N, (count - 1) * stride + T * N), stride, count, level, is_ntt)
+            want_low = [o.mod_down(e, level, is_ntt) for e in ext]
+            eq(low, np.concatenate(want_low), "mod_down_batch l=%d ntt=%d" % (level, is_ntt))
+            eq(dslab, slab, "mod_down_batch leaves its operands")
+            dig = g.alloc(count * nd * T * N)
+            g.precomp_batch(dig, nd * T * N, low, level * N, count, level, is_ntt)
+            eq(dig, np.concatenate([o.precomp(w, level, is_ntt) for w in want_low]), "precomp_batch l=%d ntt=%d" % (level, is_ntt))
+            for b in (dslab, low, dig):
+                b.free()
+    with pytest.raises(acefhe.AceError):
+        a = g.alloc(2 * (g.L + K) * N)
+        g.mod_down_batch(a, g.L * N, a, (g.L + K) * N, 2, g.L)  # results over operands
+
+
 def test_ntt_batched_polys(pair):
     g, o = pair.g, pair.o
     N = g.N
