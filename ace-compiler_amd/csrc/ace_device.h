@@ -117,6 +117,16 @@ __device__ __forceinline__ u64 mulmod(u64 a, u64 b, const DevPrime& p) {
   return csub(csub(r, p.q), p.q);
 }
 
+// (hi:lo) mod q for a value below 2^(shift + 64), e.g. a sum of up to sum_terms(p) products of residues: the
+// single-word Barrett step of mulmod, a third of barrett128's multiplies, and the same canonical residue
+__device__ __forceinline__ u64 barrett_sum(u64 hi, u64 lo, const DevPrime& p) {
+  u64 x1 = (hi << (64 - p.shift)) | (lo >> p.shift);
+  u64 r  = lo - __umul64hi(x1, p.mu_sh) * p.q;  // < 3q
+  return csub(csub(r, p.q), p.q);
+}
+// how many products of residues (each below 2^(2 shift + 2)) stay below 2^(shift + 64) when added up
+__device__ __forceinline__ u32 sum_terms(const DevPrime& p) { return p.shift >= 60 ? 4u : p.shift == 59 ? 8u : 16u; }
+
 // (hi:lo) mod q for any 128-bit value
 __device__ __forceinline__ u64 barrett128(u64 hi, u64 lo, const DevPrime& p) {
   u64 ll_hi = __umul64hi(lo, p.mu_lo);

@@ -727,10 +727,9 @@ void launch_digit_copy(hipStream_t st, const DevCtx& c, u64* res, const u64* src
 }
 
 // ---- Dot_prod (rns_poly.c:502-529, rns_poly_impl.c:102-162) ----------------
-// Both key halves in one pass so the digits are read once.  Up to 8 products
-// are accumulated in 128 bits before one Barrett-128 (the reference's
-// Fast_dotprod_poly); the result equals the reference's default
-// multiply-reduce-add chain because canonical residues are unique.
+// Both key halves in one pass so the digits are read once.  Products of residues are accumulated in 128 bits
+// (the reference's Fast_dotprod_poly) and reduced by one single-word Barrett step while the sum stays below
+// 2^(shift + 64); the result equals the reference's multiply-reduce-add chain because canonical residues are unique.
 template <bool TWO>
 __global__ __launch_bounds__(kThreads) void dotprod_kernel(DevCtx c, u64* __restrict__ out0, u64* __restrict__ out1,
                                                            u64 out_stride, const u64* __restrict__ digits,
@@ -745,20 +744,23 @@ __global__ __launch_bounds__(kThreads) void dotprod_kernel(DevCtx c, u64* __rest
   digits += op * digits_op_stride;
   out0 += op * out_stride;
   if (TWO) out1 += op * out_stride;
+  const u32 max_terms = sum_terms(P);
 #pragma unroll
   ACE_EW_LOOP(i, n) {
     u64 h0 = 0, l0 = 0, h1 = 0, l1 = 0;
+    u32 terms = 0;
     for (u32 d = 0; d < n_parts; ++d) {
       u64 x = digits[d * digit_stride + dbase + i];
       mac128(h0, l0, x, key0[d * key_stride + kbase + i]);
       if (TWO) mac128(h1, l1, x, key1[d * key_stride + kbase + i]);
-      if ((d & 7) == 7 && d + 1 < n_parts) {
-        l0 = barrett128(h0, l0, P); h0 = 0;
-        if (TWO) { l1 = barrett128(h1, l1, P); h1 = 0; }
+      if (++terms == max_terms && d + 1 < n_parts) {  // the reduced sum counts as one term
+        l0 = barrett_sum(h0, l0, P); h0 = 0;
+        if (TWO) { l1 = barrett_sum(h1, l1, P); h1 = 0; }
+        terms = 1;
       }
     }
-    out0[dbase + i] = barrett128(h0, l0, P);
-    if (TWO) out1[dbase + i] = barrett128(h1, l1, P);
+    out0[dbase + i] = barrett_sum(h0, l0, P);
+    if (TWO) out1[dbase + i] = barrett_sum(h1, l1, P);
   }
 }
 
@@ -776,20 +778,23 @@ __global__ __launch_bounds__(kThreads) void ext_rotate_kernel(DevCtx c, u64* __r
   const DevPrime P = c.primes[lm.prime[limb]];
   const u64 n = c.N, dbase = (u64)limb * n, kbase = (u64)key_limb.prime[limb] * n;
   const u64* __restrict__ key1 = key0 + key1_off;
+  const u32 max_terms = sum_terms(P);
 #pragma unroll
   ACE_EW_LOOP(i, n) {
     const u64 j = (u64)order[i];
     u64 h0 = 0, l0 = 0, h1 = 0, l1 = 0;
+    u32 terms = 0;
     for (u32 d = 0; d < n_parts; ++d) {
       const u64 x = digits[d * digit_stride + dbase + j];
       mac128(h0, l0, x, key0[d * key_stride + kbase + j]);
       mac128(h1, l1, x, key1[d * key_stride + kbase + j]);
-      if ((d & 7) == 7 && d + 1 < n_parts) {
-        l0 = barrett128(h0, l0, P); h0 = 0;
-        l1 = barrett128(h1, l1, P); h1 = 0;
+      if (++terms == max_terms && d + 1 < n_parts) {  // the reduced sum counts as one term
+        l0 = barrett_sum(h0, l0, P); h0 = 0;
+        l1 = barrett_sum(h1, l1, P); h1 = 0;
+        terms = 1;
       }
     }
-    u64 v0 = barrett128(h0, l0, P), v1 = barrett128(h1, l1, P);
+    u64 v0 = barrett_sum(h0, l0, P), v1 = barrett_sum(h1, l1, P);
     if (addend0) v0 = add_mod(v0, addend0[dbase + j], P.q);
     if (accumulate & 1) v0 = add_mod(v0, out0[dbase + i], P.q);
     if (accumulate & 2) v1 = add_mod(v1, out1[dbase + i], P.q);
@@ -849,9 +854,9 @@ __global__ __launch_bounds__(kThreads) void dotprod_shared_key_kernel(
         mac128(h0, l0, x[u][d], k0[u][d]);
         mac128(h1, l1, x[u][d], k1[u][d]);
       }
-      if (i < n) {
-        out0[op * out_stride + dbase + i] = barrett128(h0, l0, P);
-        out1[op * out_stride + dbase + i] = barrett128(h1, l1, P);
+      if (i < n) {  // NP <= 4 products: below 2^(shift + 64) for every prime below 2^61
+        out0[op * out_stride + dbase + i] = barrett_sum(h0, l0, P);
+        out1[op * out_stride + dbase + i] = barrett_sum(h1, l1, P);
       }
     }
   }
@@ -899,9 +904,9 @@ __global__ __launch_bounds__(kThreads) void dotprod_shared_digits_kernel(
         mac128(h0, l0, x[u][d], k0[u][d]);
         mac128(h1, l1, x[u][d], k1[u][d]);
       }
-      if (i < n) {
-        out0[op * out_stride + dbase + i] = barrett128(h0, l0, P);
-        out1[op * out_stride + dbase + i] = barrett128(h1, l1, P);
+      if (i < n) {  // NP <= 4 products: below 2^(shift + 64) for every prime below 2^61
+        out0[op * out_stride + dbase + i] = barrett_sum(h0, l0, P);
+        out1[op * out_stride + dbase + i] = barrett_sum(h1, l1, P);
       }
     }
   }
