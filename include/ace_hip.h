@@ -268,7 +268,9 @@ int ace_encode_scaled(ace_ctx* ctx, int64_t* res, const double* values, size_t n
 int ace_extend(ace_ctx* ctx, int64_t* res, const int64_t* src, size_t level);
 /* Dot_prod / Fast_dot_prod (:502-529): digits = n_parts x (level+num_p) limbs;
  * key = n_parts polynomials, key_stride words apart, each laid out as all num_q
- * Q limbs followed by num_p P limbs and viewed at `level` (Derive_poly :701-707). */
+ * Q limbs followed by num_p P limbs and viewed at `level` (Derive_poly :701-707).
+ * Digits and key words must be residues (below the prime of their limb), as everything the library writes is: the
+ * products are summed in 128 bits and reduced once, which relies on that bound. */
 int ace_dot_prod(ace_ctx* ctx, int64_t* res, const int64_t* digits, const int64_t* key,
                  size_t key_stride, size_t n_parts, size_t level);
 /* Fast_rotate_ext without its Mod_down (evaluator.c:503-566, as Rotate_iteration of bootstrap.c:1233-1373 uses it):
