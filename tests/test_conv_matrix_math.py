@@ -1,0 +1,117 @@
+"""The arithmetic behind the base conversion on the matrix cores (ace-compiler_amd/csrc/ace_poly.hip,
+baseconv_mx_kernel; the conversion itself is Fast_basis_conversion, rns_poly_impl.c:324-336), restated with numpy
+integers of the kernel's widths and checked against Python's big integers at the extremes the bounds are tight for:
+
+  * signed bytes of a word: (x + 0x80..80) xor 0x80..80, read as int8, sum to x again;
+  * the int32 byte sums of up to 16 source limbs stay below 2^21 in size, two of them packed into an int32 do not wrap;
+  * V = sum_p 2^(8p) S_p is congruent to sum_k x_k hat_kj and below 2^14 m in size;
+  * the FP64 estimate of V / m is within 1/2 + 2^-30 of it, so V - Q m, taken in wrapping 64-bit arithmetic, lies
+    within m of zero and one conditional addition gives the canonical residue.
+No GPU and no oracle: this pins the mathematics, the parity tests pin the kernel."""
+import numpy as np
+import pytest
+
+BIAS = 0x8080808080808080
+M64 = (1 << 64) - 1
+
+
+def signed_bytes(x):
+    """the eight int8 digits d_a of x (x = sum d_a 2^(8a)), as the kernel forms them"""
+    y = ((x + BIAS) & M64) ^ BIAS
+    return [((y >> (8 * a)) & 0xFF) - (256 if (y >> (8 * a)) & 0x80 else 0) for a in range(8)]
+
+
+def kernel_residue(xs, hats, m):
+    """one output of the kernel: sources xs, cofactors hats (residues mod m), target modulus m"""
+    assert len(xs) == len(hats) <= 16
+    # table: signed bytes of hat * 2^(8a) mod m
+    S = np.zeros(8, np.int64)
+    for x, h in zip(xs, hats):
+        d = signed_bytes(x)
+        for a in range(8):
+            e = signed_bytes(h * pow(256, a, m) % m)
+            for p in range(8):
+                S[p] += d[a] * e[p]
+    assert np.all(np.abs(S) <= 1 << 21), "a byte sum leaves the int32 budget the packing assumes"
+    S32 = S.astype(np.int32)
+    with np.errstate(over="raise"):
+        u0 = np.int32(S32[0] + (S32[1] << np.int32(8)))
+        v0 = np.int32(S32[2] + (S32[3] << np.int32(8)))
+        u1 = np.int32(S32[4] + (S32[5] << np.int32(8)))
+        v1 = np.int32(S32[6] + (S32[7] << np.int32(8)))
+    for packed, lo, hi in ((u0, S[0], S[1]), (v0, S[2], S[3]), (u1, S[4], S[5]), (v1, S[6], S[7])):
+        assert int(packed) == int(lo) + (int(hi) << 8), "two byte sums do not fit an int32"
+    t0 = int(u0) + (int(v0) << 16)
+    t1 = int(u1) + (int(v1) << 16)
+    V = t0 + (t1 << 32)
+    v_lo = V & M64
+    d0 = np.float64(int(v0)) * np.float64(65536.0) + np.float64(int(u0))
+    d1 = np.float64(int(v1)) * np.float64(65536.0) + np.float64(int(u1))
+    assert int(d0) == t0 and int(d1) == t1, "the halves are not exact in FP64"
+    vd = np.float64(d1) * np.float64(4294967296.0) + np.float64(d0)  # one rounding, as the FMA gives
+    minv = np.float64(1.0) / np.float64(m)
+    quot = int(np.rint(vd * minv))
+    r = (v_lo - quot * m) & M64
+    r = r - (1 << 64) if r >> 63 else r  # as a signed 64-bit word
+    want = sum(x * h for x, h in zip(xs, hats))
+    assert (V - want) % m == 0, "V is not congruent to the sum"
+    assert abs(V) < (m << 14), "V leaves the bound the quotient estimate relies on"
+    assert abs(quot) < 1 << 15
+    assert -m < r < m, "V - Q m is not within m of zero"
+    r = r + m if r < 0 else r
+    return r, want % m
+
+
+PRIMES = [(1 << 61) - 1, 2305843009213317121, 1152921504606830593, 72057594037338113, 1125899877875713, 1099510824961,
+          786433]
+
+
+def patterns(m):
+    vals = [0, 1, m - 1, (m + 1) // 2, m // 2]
+    for b in (0x80, 0x7F, 0xFF, 0x81, 0x01):
+        vals.append(int.from_bytes(bytes([b] * 8), "little") % m)
+    vals.append(0x0080008000800080 % m)
+    vals.append(0x7F807F807F807F80 % m)
+    return vals
+
+
+@pytest.mark.parametrize("m", PRIMES)
+def test_extreme_words(m):
+    pats = patterns(m)
+    for n_src in (1, 3, 8, 12, 16):
+        for x in pats:
+            for h in pats:
+                got, want = kernel_residue([x] * n_src, [h] * n_src, m)
+                assert got == want, (m, n_src, hex(x), hex(h))
+
+
+def test_words_whose_products_have_extreme_signed_bytes():
+    """cofactors chosen so that hat * 2^(8a) mod m has bytes of one sign for several a: the byte sums then add up
+    instead of cancelling"""
+    m = (1 << 61) - 1
+    worst = 0
+    for target in (int.from_bytes(bytes([0x80] * 7 + [0x10]), "little"), int.from_bytes(bytes([0x7F] * 7 + [0x1F]), "little")):
+        for a in range(8):
+            h = target * pow(pow(256, a, m), -1, m) % m  # then hat * 2^(8a) mod m == target
+            for x in (int.from_bytes(bytes([0x80] * 7 + [0x0F]), "little") % m, int.from_bytes(bytes([0x7F] * 8), "little") % m):
+                got, want = kernel_residue([x] * 16, [h] * 16, m)
+                assert got == want
+                worst += 1
+    assert worst == 32
+
+
+def test_random_words():
+    rng = np.random.Generator(np.random.PCG64(2026))
+    for m in PRIMES:
+        for _ in range(40):
+            n_src = int(rng.integers(1, 17))
+            xs = [int(rng.integers(0, min(m, 1 << 62), dtype=np.uint64)) % (1 << 61) for _ in range(n_src)]
+            hs = [int(rng.integers(0, m, dtype=np.uint64)) for _ in range(n_src)]
+            got, want = kernel_residue(xs, hs, m)
+            assert got == want
+
+
+def test_signed_bytes_sum_to_the_word():
+    for x in [0, 1, 0x80, 0x7F, 0xFF, 0x8000, (1 << 61) - 1, 0x7F7F7F7F7F7F7F7F, 0x0080808080808080, 0x00FFFFFFFFFFFFFF]:
+        d = signed_bytes(x)
+        assert all(-128 <= v <= 127 for v in d) and sum(v << (8 * a) for a, v in enumerate(d)) == x
