@@ -115,3 +115,35 @@ def test_signed_bytes_sum_to_the_word():
     for x in [0, 1, 0x80, 0x7F, 0xFF, 0x8000, (1 << 61) - 1, 0x7F7F7F7F7F7F7F7F, 0x0080808080808080, 0x00FFFFFFFFFFFFFF]:
         d = signed_bytes(x)
         assert all(-128 <= v <= 127 for v in d) and sum(v << (8 * a) for a, v in enumerate(d)) == x
+
+
+def sum_terms(shift):
+    """products of residues a 128-bit sum may hold before the single-word reduction (ace_device.h, sum_terms)"""
+    return 4 if shift >= 60 else 8 if shift == 59 else 16
+
+
+@pytest.mark.parametrize("q", [(1 << 61) - 1, (1 << 60) + 33 * (1 << 17) + 1, 1152921504606830593, (1 << 59) + 1,
+                               576460752303439873, 72057594037338113, 1125899877875713, 1099510824961, 786433, 3])
+def test_single_word_barrett_of_a_sum_of_products(q):
+    """barrett_sum (ace_device.h): (hi:lo) mod q by the Barrett step of the 64-bit modular product (Mul_int64_mod_barret,
+    modular.h) for a value below 2^(shift + 64), which sum_terms products of residues are: quotient at most 2 too
+    small, so two conditional subtractions finish it.  Checked at the largest sums and at random ones."""
+    shift = q.bit_length() - 1
+    mu_sh = (1 << (shift + 64)) // q
+    assert mu_sh < 1 << 65
+    rng = np.random.Generator(np.random.PCG64(q % 1000))
+    n = sum_terms(shift)
+    cases = [n * (q - 1) * (q - 1), (n - 1) * (q - 1) * (q - 1) + (q - 1), 0, q - 1, q, (q - 1) * (q - 1)]
+    cases += [sum(int(rng.integers(0, q, dtype=np.uint64)) * int(rng.integers(0, q, dtype=np.uint64)) for _ in range(n))
+              for _ in range(200)]
+    for V in cases:
+        assert V < 1 << (shift + 64), "the sum leaves the range the reduction is valid for"
+        hi, lo = V >> 64, V & M64
+        x1 = ((hi << (64 - shift)) & M64) | (lo >> shift)
+        assert x1 == V >> shift, "the shifted value does not fit 64 bits"
+        quot = (x1 * (mu_sh & M64)) >> 64 if mu_sh <= M64 else x1  # mu_sh = 2^64 only for q = 2^shift, never a prime above 2
+        r = (lo - quot * q) & M64
+        assert r < 3 * q and r == V - quot * q
+        r = r - q if r >= q else r
+        r = r - q if r >= q else r
+        assert r == V % q
