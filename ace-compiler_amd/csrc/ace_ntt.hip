@@ -57,18 +57,23 @@ namespace ace {
 // (twiddles keep the default policy).  Measured on the 768-limb batch: loads and stores both hinted take 4 to 10 % off
 // the strided passes and up to 9 % off the forward chunk pass, depending on the machine; either alone changes nothing,
 // and hinted 16-byte loads of the inverse chunk pass (four per 64-byte line and lane) cost 20 %, so those stay cached.
-// ACE_NTT_NT bits: 1 strided stores, 2 strided loads, 4 chunk stores, 8 forward chunk loads.
+// The tails fused into the forward chunk pass (Mod_down, Rescale) read their operands and write their results once as
+// well: hinted, the key switch gains about 1 %; the gathered reads of the tail that carries an automorphism gain nothing
+// and stay cached.  The selector is a template argument: as a function argument of the inlined helpers it was folded
+// away at some call sites and not at others once there were more of them.
+// ACE_NTT_NT bits: 1 strided stores, 2 strided loads, 4 chunk stores, 8 forward chunk loads, 16 tail stores, 32 tail
+// loads, 64 gathered tail loads.
 #ifndef ACE_NTT_NT
-#define ACE_NTT_NT 15
+#define ACE_NTT_NT 63
 #endif
-template <class P>
-__device__ __forceinline__ P ldg(const P* p, int bit) {
-  if (ACE_NTT_NT & bit) return __builtin_nontemporal_load(p);
-  return *p;
+template <int BIT, class P>
+__device__ __forceinline__ P ldg(const P* p) {
+  if constexpr ((ACE_NTT_NT & BIT) != 0) return __builtin_nontemporal_load(p);
+  else return *p;
 }
-template <class P>
-__device__ __forceinline__ void stg(P* p, P v, int bit) {
-  if (ACE_NTT_NT & bit) __builtin_nontemporal_store(v, p);
+template <int BIT, class P>
+__device__ __forceinline__ void stg(P* p, P v) {
+  if constexpr ((ACE_NTT_NT & BIT) != 0) __builtin_nontemporal_store(v, p);
   else *p = v;
 }
 constexpr int kChunk = 4096;
@@ -308,7 +313,7 @@ __device__ __forceinline__ void fwd_strided_body(const DevCtx& c, const PolySeq&
   if (PRO == 0) {
     const u64* __restrict__ src = srcs.at(blockIdx.z) + off;
 #pragma unroll
-    for (int r = 0; r < R; ++r) v[r] = ar.in_canon(ldg(src + r * rs + col, 2));
+    for (int r = 0; r < R; ++r) v[r] = ar.in_canon(ldg<2>(src + r * rs + col));
   } else {
     const DevPrime P = c.primes[pi];
     const u32 lt = pos.prime[limb];
@@ -351,7 +356,7 @@ stages:
   // which then runs its first two rounds (six stages) without reducing
   reduce_all<A, R>(ar, v);
 #pragma unroll
-  for (int r = 0; r < R; ++r) stg(dst + r * rs + col, ar.out_mid(v[r]), 1);
+  for (int r = 0; r < R; ++r) stg<1>(dst + r * rs + col, ar.out_mid(v[r]));
 }
 // One launch covers limbs of both arithmetic back ends: the choice is uniform over a work-group.
 template <int LOGR, int PRO>
@@ -457,7 +462,7 @@ __device__ __forceinline__ void fwd_chunk_body(u64* lds_words, const DevCtx& c, 
   const u32 tw0 = (1u << logr) + chunk;
   u64 raw[8], nxt[8];
 #pragma unroll
-  for (int r = 0; r < 8; ++r) raw[r] = ldg(base + t + 512 * r, 8);
+  for (int r = 0; r < 8; ++r) raw[r] = ldg<8>(base + t + 512 * r);
   for (u32 it = 0; it < cnt; ++it) {
     base = datas.at(poly0 + it) + loff;
     if (it + 1 < cnt) {
@@ -512,7 +517,7 @@ __device__ __forceinline__ void fwd_chunk_body(u64* lds_words, const DevCtx& c, 
     const u32 wpos = cm.wv * 512 + ((u32)t & 63);  // first of this thread's words in the wave order
     if (EPI == 0) {
 #pragma unroll
-      for (int r = 0; r < 8; ++r) stg(base + wpos + 64 * r, ldsu[cm.wave + ChunkMap::wave_off(r)], 4);
+      for (int r = 0; r < 8; ++r) stg<4>(base + wpos + 64 * r, ldsu[cm.wave + ChunkMap::wave_off(r)]);
     } else {
       const u32 p = poly0 + it, lt = pos.prime[limb];
       const u64 q = c.primes[pi].q, w = f.cst[2 * lt], wp = f.cst[2 * lt + 1];
@@ -537,16 +542,16 @@ __device__ __forceinline__ void fwd_chunk_body(u64* lds_words, const DevCtx& c, 
 #pragma unroll
           for (int r = 0; r < 4; ++r) s[r] = (u32)order[512 * (r0 + r)] & (u32)(kChunk - 1);
 #pragma unroll
-          for (int r = 0; r < 4; ++r) sv[r] = src[s[r]];
+          for (int r = 0; r < 4; ++r) sv[r] = ldg<64>(src + s[r]);
           if (addend) {
 #pragma unroll
-            for (int r = 0; r < 4; ++r) av[r] = addend[s[r]];
+            for (int r = 0; r < 4; ++r) av[r] = ldg<64>(addend + s[r]);
           }
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             u64 v = shoup_mul(sub_mod(sv[r], ldsu[lds_pos((int)s[r])], q), w, wp, q);
             if (addend) v = add_mod(v, av[r], q);
-            out[512 * (r0 + r)] = v;
+            stg<16>(out + 512 * (r0 + r), v);
           }
         }
         if (kPolysPerBlock > 1) __syncthreads();  // the gathered LDS reads are not the words this thread writes next
@@ -560,10 +565,10 @@ __device__ __forceinline__ void fwd_chunk_body(u64* lds_words, const DevCtx& c, 
         for (int r0 = 0; r0 < 8; r0 += 4) {
           u64 sv[4], av[4];
 #pragma unroll
-          for (int r = 0; r < 4; ++r) sv[r] = src[64 * (r0 + r)];
+          for (int r = 0; r < 4; ++r) sv[r] = ldg<32>(src + 64 * (r0 + r));
           if (addend) {
 #pragma unroll
-            for (int r = 0; r < 4; ++r) av[r] = addend[64 * (r0 + r)];
+            for (int r = 0; r < 4; ++r) av[r] = ldg<32>(addend + 64 * (r0 + r));
           }
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
@@ -575,7 +580,7 @@ __device__ __forceinline__ void fwd_chunk_body(u64* lds_words, const DevCtx& c, 
             } else {
               v = add_mod(shoup_mul(sv[r], w, wp, q), y, q);
             }
-            out[64 * (r0 + r)] = v;
+            stg<16>(out + 64 * (r0 + r), v);
           }
         }
       }
@@ -696,7 +701,7 @@ __device__ __forceinline__ void inv_chunk_body(u64* lds_words, const DevCtx& c, 
     gs_stage<A, 8, 1>(ar, v, (mh >> 10) + (chunk << 1));
     if (!SKIP) gs_stage<A, 8, 2>(ar, v, (mh >> 11) + (chunk << 0));  // else the strided pass runs it as its first
 #pragma unroll
-    for (int r = 0; r < 8; ++r) stg(dst + off + t + 512 * r, ar.out_mid(v[r]), 4);
+    for (int r = 0; r < 8; ++r) stg<4>(dst + off + t + 512 * r, ar.out_mid(v[r]));
     if (kPolysPerBlock > 1) __syncthreads();  // the next polynomial's first round writes words other waves still read
 #pragma unroll
     for (int r = 0; r < 8; ++r) raw[r] = nxt[r];
@@ -727,10 +732,10 @@ __device__ __forceinline__ void inv_strided_body(const DevCtx& c, const PolySeq&
   ar.init(c, pi, true, scale, limb);
   typename A::T v[R];
 #pragma unroll
-  for (int r = 0; r < R; ++r) v[r] = ar.in_mid(ldg(data + r * rs + col, 2));
+  for (int r = 0; r < R; ++r) v[r] = ar.in_mid(ldg<2>(data + r * rs + col));
   inv_strided_stages<A, LOGR>(ar, v);
 #pragma unroll
-  for (int r = 0; r < R; ++r) stg(data + r * rs + col, ar.out_scaled(v[r]), 1);
+  for (int r = 0; r < R; ++r) stg<1>(data + r * rs + col, ar.out_scaled(v[r]));
 }
 // ONLY: 0 = limbs of both back ends (the choice is uniform over a work-group), 1 = integer limbs only, 2 = FP64
 // limbs only.  The two bodies in one function need 130 registers at LOGR = 4 where each alone needs 78 / 90, and
