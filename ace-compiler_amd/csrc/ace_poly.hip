@@ -10,6 +10,27 @@
 
 namespace ace {
 
+// Streams that a kernel reads or writes once go past the caches with the non-temporal hint where that was measured
+// to pay (loads and stores of a kernel together: either alone changes nothing).  ACE_POLY_NT bits, with what each
+// gave on one machine: 2 the inner product that shares a key, digits and results (key switch +2 %; its key, read
+// once per four operands, is better left cached: bit 16); 4 the inner product that shares the digits, keys and
+// results (rotations +3 %; its digits stay cached: bit 32); 64 the extended-basis rotation, 128 the grouped plaintext
+// sums, 256 the plain inner product (a bootstrap 21.45 -> 21.2 ms together).  Not set: 1 the tensor product (no
+// change), 8 the base conversion (1 % slower).
+#ifndef ACE_POLY_NT
+#define ACE_POLY_NT (2 | 4 | 64 | 128 | 256)
+#endif
+template <int BIT, class P>
+__device__ __forceinline__ P ldn(const P* p) {
+  if constexpr ((ACE_POLY_NT & BIT) != 0) return __builtin_nontemporal_load(p);
+  else return *p;
+}
+template <int BIT, class P>
+__device__ __forceinline__ void stn(P* p, P v) {
+  if constexpr ((ACE_POLY_NT & BIT) != 0) __builtin_nontemporal_store(v, p);
+  else *p = v;
+}
+
 constexpr int kThreads = 256;
 constexpr int kUnroll = 4;
 
@@ -105,11 +126,11 @@ __global__ __launch_bounds__(kThreads) void plain_mac_groups_kernel(DevCtx c, Ma
       h0[g] = h1[g] = 0;
     }
     for (u32 j = 0; j < ops.n_ops; ++j) {
-      const u64 x0 = ops.a0[j][base + i], x1 = ops.a1[j][base + i];
+      const u64 x0 = ldn<128>(ops.a0[j] + base + i), x1 = ldn<128>(ops.a1[j] + base + i);
 #pragma unroll
       for (int g = 0; g < kMacGroups; ++g) {
         if (g < (int)ops.n_groups && ops.p[g][j]) {
-          const u64 w = ops.p[g][j][pbase + i];
+          const u64 w = ldn<128>(ops.p[g][j] + pbase + i);
           mac128(h0[g], l0[g], x0, w);
           mac128(h1[g], l1[g], x1, w);
         }
@@ -118,8 +139,8 @@ __global__ __launch_bounds__(kThreads) void plain_mac_groups_kernel(DevCtx c, Ma
 #pragma unroll
     for (int g = 0; g < kMacGroups; ++g) {
       if (g < (int)ops.n_groups) {
-        ops.r0[g][base + i] = barrett128(h0[g], l0[g], P);
-        ops.r1[g][base + i] = barrett128(h1[g], l1[g], P);
+        stn<128>(ops.r0[g] + base + i, barrett128(h0[g], l0[g], P));
+        stn<128>(ops.r1[g] + base + i, barrett128(h1[g], l1[g], P));
       }
     }
   }
@@ -386,10 +407,10 @@ __global__ __launch_bounds__(kThreads) void tensor_kernel(DevCtx c, u64* __restr
   b0 += blockIdx.z * in_stride; b1 += blockIdx.z * in_stride;
 #pragma unroll
   ACE_EW_LOOP(i, n) {
-    u64 x0 = a0[base + i], x1 = a1[base + i], y0 = b0[base + i], y1 = b1[base + i];
-    d0[base + i] = mulmod(x0, y0, P);
-    d1[base + i] = add_mod(mulmod(x0, y1, P), mulmod(x1, y0, P), P.q);
-    d2[base + i] = mulmod(x1, y1, P);
+    u64 x0 = ldn<1>(a0 + base + i), x1 = ldn<1>(a1 + base + i), y0 = ldn<1>(b0 + base + i), y1 = ldn<1>(b1 + base + i);
+    stn<1>(d0 + base + i, mulmod(x0, y0, P));
+    stn<1>(d1 + base + i, add_mod(mulmod(x0, y1, P), mulmod(x1, y0, P), P.q));
+    stn<1>(d2 + base + i, mulmod(x1, y1, P));
   }
 }
 
@@ -584,7 +605,11 @@ __device__ __forceinline__ void conv_mx_quad(const uint4 (&row)[STEPS], const Co
       res[tile] = (u64)(r < 0 ? r + (i64)m : r);
     }
     if (FULL || first_target + w < nc)
-      *reinterpret_cast<ulonglong2*>(out + tg[w].out_off) = make_ulonglong2(res[0], res[1]);
+    {
+      typedef u64 u64x2 __attribute__((ext_vector_type(2)));
+      const u64x2 pr = {res[0], res[1]};
+      stn<8>(reinterpret_cast<u64x2*>(out + tg[w].out_off), pr);
+    }
   }
 }
 
@@ -615,7 +640,11 @@ __global__ __launch_bounds__(kMxThreads) void baseconv_mx_kernel(DevCtx c, u64* 
 #pragma unroll
       for (int w = 0; w < 2; ++w) {
         const u32 k = 4 * s + 2 * half + w;
-        v[s][w] = *reinterpret_cast<const ulonglong2*>(t + (u64)min(k, nd - 1) * n);
+        {
+          typedef u64 u64x2 __attribute__((ext_vector_type(2)));
+          const u64x2 pr = ldn<8>(reinterpret_cast<const u64x2*>(t + (u64)min(k, nd - 1) * n));
+          v[s][w] = make_ulonglong2(pr.x, pr.y);
+        }
       }
 #pragma unroll
     for (int s = 0; s < STEPS; ++s)
@@ -750,17 +779,17 @@ __global__ __launch_bounds__(kThreads) void dotprod_kernel(DevCtx c, u64* __rest
     u64 h0 = 0, l0 = 0, h1 = 0, l1 = 0;
     u32 terms = 0;
     for (u32 d = 0; d < n_parts; ++d) {
-      u64 x = digits[d * digit_stride + dbase + i];
-      mac128(h0, l0, x, key0[d * key_stride + kbase + i]);
-      if (TWO) mac128(h1, l1, x, key1[d * key_stride + kbase + i]);
+      u64 x = ldn<256>(digits + d * digit_stride + dbase + i);
+      mac128(h0, l0, x, ldn<256>(key0 + d * key_stride + kbase + i));
+      if (TWO) mac128(h1, l1, x, ldn<256>(key1 + d * key_stride + kbase + i));
       if (++terms == max_terms && d + 1 < n_parts) {  // the reduced sum counts as one term
         l0 = barrett_sum(h0, l0, P); h0 = 0;
         if (TWO) { l1 = barrett_sum(h1, l1, P); h1 = 0; }
         terms = 1;
       }
     }
-    out0[dbase + i] = barrett_sum(h0, l0, P);
-    if (TWO) out1[dbase + i] = barrett_sum(h1, l1, P);
+    stn<256>(out0 + dbase + i, barrett_sum(h0, l0, P));
+    if (TWO) stn<256>(out1 + dbase + i, barrett_sum(h1, l1, P));
   }
 }
 
@@ -786,8 +815,8 @@ __global__ __launch_bounds__(kThreads) void ext_rotate_kernel(DevCtx c, u64* __r
     u32 terms = 0;
     for (u32 d = 0; d < n_parts; ++d) {
       const u64 x = digits[d * digit_stride + dbase + j];
-      mac128(h0, l0, x, key0[d * key_stride + kbase + j]);
-      mac128(h1, l1, x, key1[d * key_stride + kbase + j]);
+      mac128(h0, l0, x, ldn<64>(key0 + d * key_stride + kbase + j));
+      mac128(h1, l1, x, ldn<64>(key1 + d * key_stride + kbase + j));
       if (++terms == max_terms && d + 1 < n_parts) {  // the reduced sum counts as one term
         l0 = barrett_sum(h0, l0, P); h0 = 0;
         l1 = barrett_sum(h1, l1, P); h1 = 0;
@@ -798,8 +827,8 @@ __global__ __launch_bounds__(kThreads) void ext_rotate_kernel(DevCtx c, u64* __r
     if (addend0) v0 = add_mod(v0, addend0[dbase + j], P.q);
     if (accumulate & 1) v0 = add_mod(v0, out0[dbase + i], P.q);
     if (accumulate & 2) v1 = add_mod(v1, out1[dbase + i], P.q);
-    out0[dbase + i] = v0;
-    out1[dbase + i] = v1;
+    stn<64>(out0 + dbase + i, v0);
+    stn<64>(out1 + dbase + i, v1);
   }
 }
 void launch_ext_rotate(hipStream_t st, const DevCtx& c, u64* out0, u64* out1, const u64* digits, u64 digit_stride,
@@ -832,8 +861,8 @@ __global__ __launch_bounds__(kThreads) void dotprod_shared_key_kernel(
     const u64 i = i0 + u * kThreads;
 #pragma unroll
     for (int d = 0; d < NP; ++d) {
-      k0[u][d] = i < n ? key0[d * key_stride + kbase + i] : 0;
-      k1[u][d] = i < n ? key1[d * key_stride + kbase + i] : 0;
+      k0[u][d] = i < n ? ldn<16>(key0 + d * key_stride + kbase + i) : 0;
+      k1[u][d] = i < n ? ldn<16>(key1 + d * key_stride + kbase + i) : 0;
     }
   }
   for (u32 op = blockIdx.z; op < n_ops; op += gridDim.z) {
@@ -843,7 +872,7 @@ __global__ __launch_bounds__(kThreads) void dotprod_shared_key_kernel(
     for (int u = 0; u < kUnroll; ++u) {
       const u64 i = i0 + u * kThreads;
 #pragma unroll
-      for (int d = 0; d < NP; ++d) x[u][d] = i < n ? dg[d * digit_stride + i] : 0;
+      for (int d = 0; d < NP; ++d) x[u][d] = i < n ? ldn<2>(dg + d * digit_stride + i) : 0;
     }
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
@@ -855,8 +884,8 @@ __global__ __launch_bounds__(kThreads) void dotprod_shared_key_kernel(
         mac128(h1, l1, x[u][d], k1[u][d]);
       }
       if (i < n) {  // NP <= 4 products: below 2^(shift + 64) for every prime below 2^61
-        out0[op * out_stride + dbase + i] = barrett_sum(h0, l0, P);
-        out1[op * out_stride + dbase + i] = barrett_sum(h1, l1, P);
+        stn<2>(out0 + op * out_stride + dbase + i, barrett_sum(h0, l0, P));
+        stn<2>(out1 + op * out_stride + dbase + i, barrett_sum(h1, l1, P));
       }
     }
   }
@@ -880,7 +909,7 @@ __global__ __launch_bounds__(kThreads) void dotprod_shared_digits_kernel(
   for (int u = 0; u < kUnroll; ++u) {
     const u64 i = i0 + u * kThreads;
 #pragma unroll
-    for (int d = 0; d < NP; ++d) x[u][d] = i < n ? digits[d * digit_stride + dbase + i] : 0;
+    for (int d = 0; d < NP; ++d) x[u][d] = i < n ? ldn<32>(digits + d * digit_stride + dbase + i) : 0;
   }
   for (u32 op = blockIdx.z; op < n_ops; op += gridDim.z) {
     const u64* __restrict__ key0 = keys.p[op] + kbase;
@@ -891,8 +920,8 @@ __global__ __launch_bounds__(kThreads) void dotprod_shared_digits_kernel(
       const u64 i = i0 + u * kThreads;
 #pragma unroll
       for (int d = 0; d < NP; ++d) {
-        k0[u][d] = i < n ? key0[d * key_stride + i] : 0;
-        k1[u][d] = i < n ? key1[d * key_stride + i] : 0;
+        k0[u][d] = i < n ? ldn<4>(key0 + d * key_stride + i) : 0;
+        k1[u][d] = i < n ? ldn<4>(key1 + d * key_stride + i) : 0;
       }
     }
 #pragma unroll
@@ -905,8 +934,8 @@ __global__ __launch_bounds__(kThreads) void dotprod_shared_digits_kernel(
         mac128(h1, l1, x[u][d], k1[u][d]);
       }
       if (i < n) {  // NP <= 4 products: below 2^(shift + 64) for every prime below 2^61
-        out0[op * out_stride + dbase + i] = barrett_sum(h0, l0, P);
-        out1[op * out_stride + dbase + i] = barrett_sum(h1, l1, P);
+        stn<4>(out0 + op * out_stride + dbase + i, barrett_sum(h0, l0, P));
+        stn<4>(out1 + op * out_stride + dbase + i, barrett_sum(h1, l1, P));
       }
     }
   }
