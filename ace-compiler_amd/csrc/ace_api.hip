@@ -912,14 +912,16 @@ void do_decomp_modup(ace_ctx* c, u64* res, const u64* digit, size_t level, size_
 // (num_decomp x (level+K) limbs).  One INTT over all limbs (each scaled by its
 // own digit's inverse cofactor), one base-conversion launch per 4 digits, one
 // NTT over every converted limb.
+// skip_own: the digits' own limbs are not copied into the raised polynomials (the caller's inner product reads them
+// from src: OwnLimbs)
 void do_precomp(ace_ctx* c, u64* res, u64 res_stride, const u64* src, u64 src_stride, size_t nb, size_t level,
-                bool is_ntt) {
+                bool is_ntt, bool skip_own = false) {
   const PrecompDev& pd = c->precomp_at(level);
   const size_t N = c->h.N, nd = c->h.num_decomp(level), T = level + c->h.K;
   size_t mark = c->ws_used;
   u64* t = c->take(nb * level * N);
   // the digits' own limbs pass through; the inverse transform of a large ring drops that copy as it reads them
-  const bool by_transform = is_ntt && c->d.logN > 12;
+  const bool by_transform = is_ntt && c->d.logN > 12 && !skip_own;
   if (is_ntt) {
     const CopyThrough through{seq_strided(res, res_stride), (u64)(T * N), (u32)c->h.part_size};
     if (!launch_ntt(c->stream, c->d, seq_strided(t, level * N), seq_strided(src, src_stride), c->q_lm, nullptr,
@@ -929,7 +931,7 @@ void do_precomp(ace_ctx* c, u64* res, u64 res_stride, const u64* src, u64 src_st
     for (size_t o = 0; o < nb; ++o)
       launch_mul_const(c->stream, c->d, t + o * level * N, src + o * src_stride, pd.scale_coef, c->q_lm, (u32)level);
   }
-  if (!by_transform)
+  if (!by_transform && !skip_own)
     launch_digit_copy(c->stream, c->d, res, src, (u32)level, (u32)c->h.part_size, (u32)nd, T * N, res_stride,
                       src_stride, (u32)nb);
   for (size_t j0 = 0; j0 < nd; j0 += kMaxConvJobs) {
@@ -1084,13 +1086,14 @@ LimbMap key_pos(const ace_ctx* c, size_t level) {
 // 2o and 2o+1 of `out`.  The addend, and with `orders` the automorphism of
 // operand o (table o), are fused into the Mod_down tail.
 void do_switch_key(ace_ctx* c, const PolySeq& out, const u64* digits, u64 digits_op_stride, const KeySet& keys,
-                   size_t nb, size_t level, const PolySeq* addend, int addend_mode, const OrderSet* orders = nullptr) {
+                   size_t nb, size_t level, const PolySeq* addend, int addend_mode, const OrderSet* orders = nullptr,
+                   const OwnLimbs* own = nullptr) {
   const size_t N = c->h.N, T = level + c->h.K, kpoly = (c->h.L + c->h.K) * N, nd = c->h.num_decomp(level);
   size_t mark = c->ws_used;
   u64* e = c->take(nb * 2 * T * N);  // [operand][b|a][T limbs]
   LimbMap lm = poly_lm(c, level, true), kp = key_pos(c, level);
   launch_dotprod(c->stream, c->d, e, e + T * N, 2 * T * N, digits, T * N, digits_op_stride, keys, kpoly, 2 * kpoly,
-                 (u32)nd, lm, kp, (u32)T, (u32)nb);
+                 (u32)nd, lm, kp, (u32)T, (u32)nb, own);
   do_mod_down(c, out, seq_strided(e, T * N), 2 * nb, level, true, addend, addend_mode, orders);
   c->ws_used = mark;
 }
@@ -1111,9 +1114,13 @@ void do_mul_relin_rescale(ace_ctx* c, u64* r0, u64* r1, u64 out_stride, const u6
   u64* digits = c->take(nb * nd * T * N);
   launch_tensor(c->stream, c->d, d01, d01 + level * N, d2, a0, a1, b0, b1, c->q_lm, (u32)level, (u32)nb,
                 2 * level * N, level * N, in_stride);
-  do_precomp(c, digits, nd * T * N, d2, level * N, nb, level, true);
+  // where the inner product can read the digits' own limbs from d2 itself, Mod_up does not copy them
+  const bool from_d2 = c->d.logN > 12 && dotprod_reads_own(1, (u32)nb, true, (u32)nd);
+  const OwnLimbs own{d2, (u64)(level * N), (u32)c->h.part_size, (u32)level};
+  do_precomp(c, digits, nd * T * N, d2, level * N, nb, level, true, from_d2);
   PolySeq ds = seq_strided(d01, level * N);
-  do_switch_key(c, ds, digits, nd * T * N, one_key(swk), nb, level, &ds, 1);  // relinearised ct replaces d0, d1
+  do_switch_key(c, ds, digits, nd * T * N, one_key(swk), nb, level, &ds, 1, nullptr,
+                from_d2 ? &own : nullptr);  // relinearised ct replaces d0, d1
   do_rescale(c, seq_pair(r0, r1, out_stride), ds, 2 * nb, level, true);
 }
 

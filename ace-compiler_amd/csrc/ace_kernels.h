@@ -147,9 +147,18 @@ void launch_digit_copy(hipStream_t st, const DevCtx& c, u64* res, const u64* src
                        u32 n_digits, u64 digit_stride, u64 res_stride, u64 src_stride, u32 n_ops);
 // inner product with a switch key for n_ops operands: out0/out1 (n_limbs limbs, out_stride apart) =
 // sum_d digits[op][d] * key[d][0/1]; key limb of launch limb t is key_limb[t]; out1 may be null.
+// Where the raised digits do not hold the digits' own limbs (the Q limbs of the polynomial that was decomposed,
+// which Mod_up only passes through): limb t < level of digit t / part_size is read from src + op * op_stride + t * N.
+struct OwnLimbs {
+  const u64* src;
+  u64 op_stride;
+  u32 part_size, level;
+};
+// whether launch_dotprod with these arguments reads own limbs from OwnLimbs (only the kernel that shares a key does)
+bool dotprod_reads_own(u32 n_keys, u32 n_ops, bool two_halves, u32 n_parts);
 void launch_dotprod(hipStream_t st, const DevCtx& c, u64* out0, u64* out1, u64 out_stride, const u64* digits,
                     u64 digit_stride, u64 digits_op_stride, const KeySet& keys, u64 key1_off, u64 key_stride,
-                    u32 n_parts, const LimbMap& lm, const LimbMap& key_limb, u32 n_limbs, u32 n_ops);
+                    u32 n_parts, const LimbMap& lm, const LimbMap& key_limb, u32 n_limbs, u32 n_ops, const OwnLimbs* own = nullptr);
 // out0[i] (+)= (sum_d digit_d * key0_d)[order[i]] (+ addend0[order[i]]), out1[i] (+)= (sum_d digit_d * key1_d)[order[i]];
 // accumulate bit 0 / 1: add to what out0 / out1 holds
 void launch_ext_rotate(hipStream_t st, const DevCtx& c, u64* out0, u64* out1, const u64* digits, u64 digit_stride,

@@ -847,11 +847,13 @@ template <int NP>
 __global__ __launch_bounds__(kThreads) void dotprod_shared_key_kernel(
     DevCtx c, u64* __restrict__ out0, u64* __restrict__ out1, u64 out_stride, const u64* __restrict__ digits,
     u64 digit_stride, u64 digits_op_stride, const u64* __restrict__ key0, u64 key1_off, u64 key_stride, LimbMap lm,
-    LimbMap key_limb, u32 n_ops) {
+    LimbMap key_limb, u32 n_ops, OwnLimbs own) {
   const u32 limb = blockIdx.y;
   const DevPrime P = c.primes[lm.prime[limb]];
   const u64 n = c.N, dbase = (u64)limb * n, kbase = (u64)key_limb.prime[limb] * n;
   const u64* __restrict__ key1 = key0 + key1_off;
+  // the digit this limb is an own limb of (NP: none, or the digits hold their own limbs)
+  const int own_d = (own.src && limb < own.level) ? min((int)(limb / own.part_size), NP - 1) : NP;
   // the thread's kUnroll coefficients are handled together so that every operand has
   // kUnroll * NP independent loads in flight
   const u64 i0 = (u64)blockIdx.x * (kThreads * kUnroll) + threadIdx.x;
@@ -872,7 +874,8 @@ __global__ __launch_bounds__(kThreads) void dotprod_shared_key_kernel(
     for (int u = 0; u < kUnroll; ++u) {
       const u64 i = i0 + u * kThreads;
 #pragma unroll
-      for (int d = 0; d < NP; ++d) x[u][d] = i < n ? ldn<2>(dg + d * digit_stride + i) : 0;
+      for (int d = 0; d < NP; ++d)
+        x[u][d] = i >= n ? 0 : d == own_d ? ldn<2>(own.src + op * own.op_stride + dbase + i) : ldn<2>(dg + d * digit_stride + i);
     }
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
@@ -941,18 +944,24 @@ __global__ __launch_bounds__(kThreads) void dotprod_shared_digits_kernel(
   }
 }
 
+bool dotprod_reads_own(u32 n_keys, u32 n_ops, bool two_halves, u32 n_parts) {
+  return n_keys == 1 && n_ops > 1 && two_halves && n_parts >= 1 && n_parts <= 4;
+}
+
 void launch_dotprod(hipStream_t st, const DevCtx& c, u64* out0, u64* out1, u64 out_stride, const u64* digits,
                     u64 digit_stride, u64 digits_op_stride, const KeySet& keys, u64 key1_off, u64 key_stride,
-                    u32 n_parts, const LimbMap& lm, const LimbMap& key_limb, u32 n_limbs, u32 n_ops) {
+                    u32 n_parts, const LimbMap& lm, const LimbMap& key_limb, u32 n_limbs, u32 n_ops,
+                    const OwnLimbs* own) {
   if (!n_limbs || !n_ops) return;
-  if (keys.n == 1 && n_ops > 1 && out1 && n_parts >= 1 && n_parts <= 4) {
+  if (dotprod_reads_own(keys.n, n_ops, out1 != nullptr, n_parts)) {
+    const OwnLimbs ol = own ? *own : OwnLimbs{nullptr, 0, 1, 0};
     // NP <= 4 products of residues below 2^61 fit 128 bits without an intermediate reduction
     dim3 g = ew_grid(c.N, n_limbs, n_ops < 4 ? n_ops : 4);
 #define ACE_DP_CASE(NP)                                                                                          \
   case NP:                                                                                                       \
     hipLaunchKernelGGL(dotprod_shared_key_kernel<NP>, g, dim3(kThreads), 0, st, c, out0, out1, out_stride,       \
                        digits, digit_stride, digits_op_stride, keys.p[0], key1_off, key_stride, lm, key_limb,    \
-                       n_ops);                                                                                   \
+                       n_ops, ol);                                                                               \
     break;
     switch (n_parts) { ACE_DP_CASE(1) ACE_DP_CASE(2) ACE_DP_CASE(3) ACE_DP_CASE(4) }
 #undef ACE_DP_CASE
