@@ -944,6 +944,11 @@ __global__ __launch_bounds__(kThreads) void dotprod_shared_digits_kernel(
   }
 }
 
+// How many blocks share the walk over the operands of a batch (blockIdx.z): the shared operand is fetched that many
+// times.  A key is 93 MiB, so the kernel that shares it splits the operands two ways only; the digits that
+// rotations share are a twentieth of one key, and sixteen blocks walking two keys each keep more of the machine's
+// memory channels busy than four walking eight (rotations +2 %).
+constexpr u32 kSharedKeySplit = 2, kSharedDigitsSplit = 16;
 bool dotprod_reads_own(u32 n_keys, u32 n_ops, bool two_halves, u32 n_parts) {
   return n_keys == 1 && n_ops > 1 && two_halves && n_parts >= 1 && n_parts <= 4;
 }
@@ -956,7 +961,7 @@ void launch_dotprod(hipStream_t st, const DevCtx& c, u64* out0, u64* out1, u64 o
   if (dotprod_reads_own(keys.n, n_ops, out1 != nullptr, n_parts)) {
     const OwnLimbs ol = own ? *own : OwnLimbs{nullptr, 0, 1, 0};
     // NP <= 4 products of residues below 2^61 fit 128 bits without an intermediate reduction
-    dim3 g = ew_grid(c.N, n_limbs, n_ops < 4 ? n_ops : 4);
+    dim3 g = ew_grid(c.N, n_limbs, n_ops < kSharedKeySplit ? n_ops : kSharedKeySplit);
 #define ACE_DP_CASE(NP)                                                                                          \
   case NP:                                                                                                       \
     hipLaunchKernelGGL(dotprod_shared_key_kernel<NP>, g, dim3(kThreads), 0, st, c, out0, out1, out_stride,       \
@@ -968,7 +973,7 @@ void launch_dotprod(hipStream_t st, const DevCtx& c, u64* out0, u64* out1, u64 o
     return;
   }
   if (keys.n == n_ops && n_ops > 1 && digits_op_stride == 0 && out1 && n_parts >= 1 && n_parts <= 4) {
-    dim3 g = ew_grid(c.N, n_limbs, n_ops < 4 ? n_ops : 4);
+    dim3 g = ew_grid(c.N, n_limbs, n_ops < kSharedDigitsSplit ? n_ops : kSharedDigitsSplit);
 #define ACE_DP_CASE(NP)                                                                                          \
   case NP:                                                                                                       \
     hipLaunchKernelGGL(dotprod_shared_digits_kernel<NP>, g, dim3(kThreads), 0, st, c, out0, out1, out_stride,    \
