@@ -297,31 +297,22 @@ __device__ __forceinline__ void inv_strided_stages(const A& ar, typename A::T* v
   }
 }
 
-// forward, strided pass: stages 0..LOGR-1.  grid = (N/R/256, n_limbs, n_polys)
-// PRO = 1: the input is not read from src but formed from the last limb of a
-// rescale (FwdFuse::pro).
-template <class A, int LOGR, int PRO>
-__device__ __forceinline__ void fwd_strided_body(const DevCtx& c, const PolySeq& dsts, const PolySeq& srcs,
-                                                 const LimbMap& pos, const FwdFuse& f, u32 limb, u32 pi) {
-  constexpr int R = 1 << LOGR;
-  const u32 col = blockIdx.x * 256 + threadIdx.x;
-  const u64 rs = c.N >> LOGR;  // row stride
-  // uniform row base + per-thread 32-bit column: rows are addressed off scalar registers
-  const u64 off = (u64)pos.prime[limb] * c.N;
-  u64* __restrict__ dst = dsts.at(blockIdx.z) + off;
-  A ar;
-  ar.init(c, pi, false, nullptr, 0);
-  typename A::T v[R];
+// What a thread of a forward strided pass starts from: R words of its column, `step` words apart from `first` on.
+// PRO = 0: read from src.  PRO = 1: formed from the last limb of a rescale (FwdFuse::pro).
+template <class A, int R, int PRO>
+__device__ __forceinline__ void fwd_strided_input(const A& ar, const DevCtx& c, const PolySeq& srcs, const LimbMap& pos,
+                                                  const FwdFuse& f, u32 limb, u32 pi, u32 col, u64 first, u64 step,
+                                                  typename A::T* v) {
   if (PRO == 0) {
-    const u64* __restrict__ src = srcs.at(blockIdx.z) + off;
+    const u64* __restrict__ src = srcs.at(blockIdx.z) + (u64)pos.prime[limb] * c.N + first;
 #pragma unroll
-    for (int r = 0; r < R; ++r) v[r] = ar.in_canon(ldg<2>(src + r * rs + col));
+    for (int r = 0; r < R; ++r) v[r] = ar.in_canon(ldg<2>(src + r * step + col));
   } else {
     const DevPrime P = c.primes[pi];
     const u32 lt = pos.prime[limb];
     const u64 ql = c.primes[f.last_prime].q, half = ql >> 1;
     const u64 K = f.sw[3 * lt], Kp = f.sw[3 * lt + 1], diff = f.sw[3 * lt + 2];
-    const u64* __restrict__ last = f.last + blockIdx.z * f.last_stride + col;
+    const u64* __restrict__ last = f.last + blockIdx.z * f.last_stride + first + col;
     if constexpr (A::kFp) {
       // Both primes small enough for FP64: the centred value of the last limb's word (|x| <= ql/2 <= q) times the
       // centred constant is one exact FP64 product, about a fifth of the integer path's instructions; its result
@@ -333,26 +324,47 @@ __device__ __forceinline__ void fwd_strided_body(const DevCtx& c, const PolySeq&
         const double kci = kc * ar.qinv;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-          double x = ar.in_canon(last[r * rs]);
+          double x = ar.in_canon(last[r * step]);
           x = x > halfd ? x - qld : x;
           v[r] = ar.mulmod(x, kc, kci);
         }
-        goto stages;
+        return;
       }
+    }
+    // All words are requested before the first is used, and the three cases below are uniform over the launch's
+    // limb: a per-word branch would make every load wait for the one before it.
+    u64 xs[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) xs[r] = last[r * step];
+    if (P.q > ql) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) xs[r] += xs[r] > half ? P.q - ql : 0;
+    } else if (ql < 2 * P.q) {
+      // diff = 2 q - ql here, so a shifted word stays below 2 q
+#pragma unroll
+      for (int r = 0; r < R; ++r) xs[r] = csub(xs[r] + (xs[r] > half ? diff : 0), P.q);
+    } else {
+#pragma unroll
+      for (int r = 0; r < R; ++r) xs[r] = barrett128(0, xs[r] + (xs[r] > half ? diff : 0), P);
     }
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      u64 x = last[r * rs];
-      if (P.q > ql) {
-        if (x > half) x += P.q - ql;
-      } else {
-        if (x > half) x += diff;
-        if (x >= P.q) x = barrett128(0, x, P);
-      }
-      v[r] = ar.in_canon(shoup_mul(x, K, Kp, P.q));
-    }
+    for (int r = 0; r < R; ++r) v[r] = ar.in_canon(shoup_mul(xs[r], K, Kp, P.q));
   }
-stages:
+}
+
+// forward, strided pass: stages 0..LOGR-1.  grid = (N/R/256, n_limbs, n_polys)
+template <class A, int LOGR, int PRO>
+__device__ __forceinline__ void fwd_strided_body(const DevCtx& c, const PolySeq& dsts, const PolySeq& srcs,
+                                                 const LimbMap& pos, const FwdFuse& f, u32 limb, u32 pi) {
+  constexpr int R = 1 << LOGR;
+  const u32 col = blockIdx.x * 256 + threadIdx.x;
+  const u64 rs = c.N >> LOGR;  // row stride
+  // uniform row base + per-thread 32-bit column: rows are addressed off scalar registers
+  u64* __restrict__ dst = dsts.at(blockIdx.z) + (u64)pos.prime[limb] * c.N;
+  A ar;
+  ar.init(c, pi, false, nullptr, 0);
+  typename A::T v[R];
+  fwd_strided_input<A, R, PRO>(ar, c, srcs, pos, f, limb, pi, col, 0, rs, v);
   fwd_strided_stages<A, LOGR>(ar, v);
   // this pass is bound by HBM and has instruction slots to spare: it hands centred values to the chunk pass,
   // which then runs its first two rounds (six stages) without reducing
@@ -751,6 +763,88 @@ __global__ __launch_bounds__(256) void ntt_inv_strided(DevCtx c, PolySeq datas, 
 }
 
 // ---------------------------------------------------------------------------
+// The strided passes of N = 2^16 for launches too small to fill the machine.  A column's sixteen words are spread
+// over the four waves of a work-group, four words each: two stages, one exchange through LDS, two more stages.
+// Such a launch is four times the waves of the plain pass, each with a quarter of a column's 32 butterflies, where
+// the plain pass would leave most SIMDs with a single wave that works through a whole column on its own.
+// grid = (N/16/64, n_limbs, n_polys), 256 threads; results are those of the plain pass.
+constexpr int kSplitCols = 64;
+template <class A, int PRO>
+__device__ __forceinline__ void fwd_strided_split_body(u64* lds_words, const DevCtx& c, const PolySeq& dsts,
+                                                       const PolySeq& srcs, const LimbMap& pos, const FwdFuse& f,
+                                                       u32 limb, u32 pi) {
+  typedef typename A::T T;
+  const u32 j = (u32)__builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const u32 col = blockIdx.x * kSplitCols + lane;
+  const u64 rs = c.N >> 4;
+  u64* __restrict__ dst = dsts.at(blockIdx.z) + (u64)pos.prime[limb] * c.N;
+  A ar;
+  ar.init(c, pi, false, nullptr, 0);
+  T v[4];
+  // rows j, j+4, j+8, j+12: the pairs of the stages of span 8 and 4
+  fwd_strided_input<A, 4, PRO>(ar, c, srcs, pos, f, limb, pi, col, j * rs, 4 * rs, v);
+  ct_stage<A, 4, 0>(ar, v, 1);
+  ct_stage<A, 4, 1>(ar, v, 2);
+  T* x = reinterpret_cast<T*>(lds_words);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) x[(j + 4 * k) * kSplitCols + lane] = v[k];
+  __syncthreads();
+  // rows 4j .. 4j+3: group j of the stage of span 2, groups 2j and 2j+1 of the last one
+#pragma unroll
+  for (int k = 0; k < 4; ++k) v[k] = x[(4 * j + k) * kSplitCols + lane];
+  ct_stage<A, 4, 0>(ar, v, 4 + j);
+  ct_stage<A, 4, 1>(ar, v, 8 + 2 * j);
+  reduce_all<A, 4>(ar, v);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) stg<1>(dst + (4 * j + k) * rs + col, ar.out_mid(v[k]));
+}
+template <int PRO>
+__global__ __launch_bounds__(256) void ntt_fwd_strided_split(DevCtx c, PolySeq dsts, PolySeq srcs, LimbMap lm,
+                                                             LimbMap pos, FwdFuse f) {
+  __shared__ u64 lds[16 * kSplitCols];
+  const u32 limb = gridDim.y - 1 - blockIdx.y, pi = lm.prime[limb];
+  if (c.fp_ok[pi]) fwd_strided_split_body<ArithFp, PRO>(lds, c, dsts, srcs, pos, f, limb, pi);
+  else fwd_strided_split_body<ArithInt, PRO>(lds, c, dsts, srcs, pos, f, limb, pi);
+}
+template <class A>
+__device__ __forceinline__ void inv_strided_split_body(u64* lds_words, const DevCtx& c, const PolySeq& datas,
+                                                       const LimbMap& pos, const u64* __restrict__ scale, u32 limb,
+                                                       u32 pi) {
+  typedef typename A::T T;
+  const u32 j = (u32)__builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const u32 col = blockIdx.x * kSplitCols + lane;
+  const u64 rs = c.N >> 4;
+  u64* __restrict__ data = datas.at(blockIdx.z) + (u64)pos.prime[limb] * c.N;
+  A ar;
+  ar.init(c, pi, true, scale, limb);
+  T v[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) v[k] = ar.in_mid(ldg<2>(data + (4 * j + k) * rs + col));
+  // the reductions stand where inv_strided_stages has them: before the first and the fourth stage
+  reduce_all<A, 4>(ar, v);
+  gs_stage<A, 4, 0>(ar, v, 8 + 2 * j);
+  gs_stage<A, 4, 1>(ar, v, 4 + j);
+  T* x = reinterpret_cast<T*>(lds_words);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) x[(4 * j + k) * kSplitCols + lane] = v[k];
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < 4; ++k) v[k] = x[(j + 4 * k) * kSplitCols + lane];
+  gs_stage<A, 4, 0>(ar, v, 2);
+  reduce_all<A, 4>(ar, v);
+  gs_stage<A, 4, 1>(ar, v, 1);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) stg<1>(data + (j + 4 * k) * rs + col, ar.out_scaled(v[k]));
+}
+__global__ __launch_bounds__(256) void ntt_inv_strided_split(DevCtx c, PolySeq datas, LimbMap lm, LimbMap pos,
+                                                             const u64* __restrict__ scale) {
+  __shared__ u64 lds[16 * kSplitCols];
+  const u32 limb = gridDim.y - 1 - blockIdx.y, pi = lm.prime[limb];
+  if (c.fp_ok[pi]) inv_strided_split_body<ArithFp>(lds, c, datas, pos, scale, limb, pi);
+  else inv_strided_split_body<ArithInt>(lds, c, datas, pos, scale, limb, pi);
+}
+
+// ---------------------------------------------------------------------------
 // N <= 4096: one workgroup per limb, the limb in LDS, one butterfly per
 // thread per step (integer back end).  grid = (1, n_limbs, n_polys)
 __global__ __launch_bounds__(256) void ntt_small(DevCtx c, PolySeq dsts, PolySeq srcs, LimbMap lm, LimbMap pos,
@@ -797,6 +891,18 @@ __global__ __launch_bounds__(256) void ntt_small(DevCtx c, PolySeq dsts, PolySeq
 // a column), and the chunk pass skips it.  Measured on 768 limbs at N = 2^16: the chunk passes gain 2 %, the inverse
 // strided pass stays where it was and the forward one, which then needs 122 registers, loses 6 %: the inverse
 // transform shifts (SI), the forward one does not (SF).
+// Launches of fewer limbs than this take the split strided passes (N = 2^16) if any of their limbs is on the integer
+// back end: an FP64 column is a fifth of the instructions, and a launch of those gains nothing from the split.
+static bool split_strided(const DevCtx& c, const LimbMap& lm, u32 n_limbs, u32 n_polys) {
+  static const long below = [] {
+    const char* e = getenv("ACE_NTT_SPLIT_BELOW");
+    return e ? atol(e) : 96L;
+  }();
+  if ((long)n_limbs * (long)n_polys >= below) return false;
+  for (u32 t = 0; t < n_limbs; ++t)
+    if (!c.fp_ok[lm.prime[t]]) return true;
+  return false;
+}
 template <int LOGR, int SF, int SI>
 static void run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolySeq& src, const LimbMap& lm,
                       const LimbMap& pos, u32 n_limbs, u32 n_polys, bool inverse, const u64* scale, int passes,
@@ -805,7 +911,13 @@ static void run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst, const
   if (!inverse) {
     constexpr int LS = LOGR + SF, SHIFT = SF;
     dim3 gs((c.N >> LS) / 256, n_limbs, n_polys);
-    if (passes & 1) {
+    if ((passes & 1) && LS == 4 && split_strided(c, lm, n_limbs, n_polys)) {
+      dim3 gq((c.N >> 4) / kSplitCols, n_limbs, n_polys);
+      if (f.pro == 0)
+        hipLaunchKernelGGL((ntt_fwd_strided_split<0>), gq, dim3(256), 0, st, c, dst, src, lm, pos, f);
+      else
+        hipLaunchKernelGGL((ntt_fwd_strided_split<1>), gq, dim3(256), 0, st, c, dst, src, lm, pos, f);
+    } else if (passes & 1) {
       if (f.pro == 0)
         hipLaunchKernelGGL((ntt_fwd_strided<LS, 0>), gs, dim3(256), 0, st, c, dst, src, lm, pos, f);
       else
@@ -834,7 +946,10 @@ static void run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst, const
         hipLaunchKernelGGL((ntt_inv_chunk<SHIFT, 0>), gc, dim3(kChunkThreads), 0, st, c, dst, src, copies, lm, pos,
                            n_limbs, n_polys);
     }
-    if (passes & 2) {
+    if ((passes & 2) && LS == 4 && split_strided(c, lm, n_limbs, n_polys)) {
+      dim3 gq((c.N >> 4) / kSplitCols, n_limbs, n_polys);
+      hipLaunchKernelGGL(ntt_inv_strided_split, gq, dim3(256), 0, st, c, dst, lm, pos, scale);
+    } else if (passes & 2) {
       u32 n_fp = 0;
       for (u32 t = 0; t < n_limbs; ++t) n_fp += c.fp_ok[lm.prime[t]] ? 1 : 0;
       if (n_fp == 0)

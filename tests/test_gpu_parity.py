@@ -282,6 +282,48 @@ def test_ntt_batched_polys(pair):
     eq(d, buf, "batched round trip")
 
 
+def test_strided_passes_of_small_and_large_launches_on_integer_limbs():
+    """At N = 65536 a transform of a few limbs on the integer back end spreads each column of its strided pass over
+    four waves; a launch of many limbs keeps a column in one thread.  Both must give the oracle's words: a single
+    polynomial (forward, inverse, and the Rescale whose strided pass forms its input from the dropped limb), then 40
+    copies of it in one launch, every one of which must come out like the single polynomial."""
+    cfg = (65536, 4, 60, 56, 2)
+    g, o = acefhe.Context(*cfg), Oracle(*cfg)
+    try:
+        N, L = g.N, g.L
+        idx = list(range(L + g.K))
+        pr = [g.primes[i] for i in idx]
+        nl = len(idx)
+        x = seeded.uniform_poly(91, pr, N)
+        d = g.upload(x)
+        g.ntt(d, d, idx)
+        fwd = o.ntt(x, idx)
+        eq(d, fwd, "forward, one polynomial")
+        g.intt(d, d, idx)
+        eq(d, x, "round trip, one polynomial")
+        d.free()
+        copies = 40
+        many = np.tile(x, copies)
+        d = g.upload(many)
+        g.ntt(d, d, idx, n_polys=copies, poly_stride_limbs=nl)
+        eq(d, np.tile(fwd, copies), "forward, 40 polynomials")
+        g.intt(d, d, idx, n_polys=copies, poly_stride_limbs=nl)
+        eq(d, many, "round trip, 40 polynomials")
+        d.free()
+        for level in range(2, L + 1):
+            c = seeded.uniform_poly(95 + level, g.primes[:level], N)
+            dc = g.upload(c)
+            for is_ntt in (True, False):
+                dr = g.alloc((level - 1) * N)
+                g.rescale(dr, dc, level, is_ntt)
+                eq(dr, o.rescale(c, level, is_ntt), "rescale l=%d ntt=%d" % (level, is_ntt))
+                dr.free()
+            dc.free()
+    finally:
+        g.close()
+        o.close()
+
+
 def test_hw_ops(pair):
     g, o = pair.g, pair.o
     N = g.N
