@@ -65,6 +65,15 @@ struct RescaleDev {
   u64* tail = nullptr;  // [level-1][2]: q_l^-1, Shoup
 };
 
+// Constants of a Mod_down and a Rescale that share one forward transform (do_switch_key_rescale)
+struct ModDownRescaleDev {
+  u64* inv_scale = nullptr;  // [1 + K][2]: (1/N * P^-1 mod q_last) for the dropped limb, then the P limbs' Mod_down scales
+  u64* ycst = nullptr;       // [level-1][2]: -(P q_last)^-1 mod q_t
+  u64* tail = nullptr;       // [level-1][2]: (P q_last)^-1 mod q_t
+  LimbMap inv_lm{};          // the dropped limb, then the P limbs
+  u64 pinv_last = 0, pinv_last_p = 0;
+};
+
 // Scratch of ace_mod_down_noalloc: the intermediates of one Mod_down (the scaled inverse transform of the P limbs
 // and their conversion to the Q basis), held in a device array that exists from the moment the library is loaded.
 // Each GPU has its own copy at its own address; host code reaches it only through the pointer that
@@ -187,6 +196,7 @@ struct ace_ctx {
   std::map<std::pair<size_t, size_t>, ModUpDev> modup;
   std::map<size_t, RescaleDev> rescale;
   std::map<size_t, PrecompDev> precomp;
+  std::map<size_t, ModDownRescaleDev> moddown_rescale;
   // Mod_down / Extend constants
   u64* phat = nullptr;        // [K][L]
   u64* pscale_ntt = nullptr;  // [K][2]
@@ -267,6 +277,9 @@ struct ace_ctx {
   // FP64 tables of a base conversion (ConvJob::fw / fq) for the targets below kFpConvTargetLimit
   bool conv_fp = true;
   bool conv_matrix = true;  // base conversions on the matrix cores (ACE_CONV_MATRIX=0 in the environment: off)
+  // Mod_down followed by Rescale through one forward transform where an entry point knows both
+  // (ACE_SHARE_TRANSFORM=0 in the environment: the two one after the other; same words)
+  bool share_transform = true;
   void conv_fp_tables(ConvJob& j, const std::vector<size_t>& src, const std::vector<size_t>& tgt, const u64* hat,
                       size_t hat_stride) {
     j.fw = j.fq = nullptr;
@@ -451,6 +464,37 @@ struct ace_ctx {
     return rescale.emplace(level, r).first->second;
   }
 
+  const ModDownRescaleDev& moddown_rescale_at(size_t level) {
+    auto it = moddown_rescale.find(level);
+    if (it != moddown_rescale.end()) return it->second;
+    std::vector<u64> qi, nqi;
+    h.rescale_table(level, qi, nqi);
+    const size_t last = level - 1;
+    const u64 ql = h.primes[last].q;
+    ModDownRescaleDev m;
+    std::vector<u64> sc(2 * (1 + h.K)), yc(2 * last), tl(2 * last);
+    const u64 a = mul_mod(h.primes[last].ninv, h.pinv_modq[last], ql);
+    sc[0] = a; sc[1] = shoup(a, ql);
+    m.inv_lm.prime[0] = (uint8_t)last;
+    for (size_t j = 0; j < h.K; ++j) {
+      const u64 q = h.primes[h.L + j].q, b = mul_mod(h.primes[h.L + j].ninv, h.phat_inv[j], q);
+      sc[2 * (1 + j)] = b; sc[2 * (1 + j) + 1] = shoup(b, q);
+      m.inv_lm.prime[1 + j] = (uint8_t)(h.L + j);
+    }
+    for (size_t i = 0; i < last; ++i) {
+      const u64 q = h.primes[i].q;
+      const u64 y = mul_mod(h.pinv_modq[i], nqi[i], q), t = mul_mod(h.pinv_modq[i], qi[i], q);
+      yc[2 * i] = y; yc[2 * i + 1] = shoup(y, q);
+      tl[2 * i] = t; tl[2 * i + 1] = shoup(t, q);
+    }
+    m.inv_scale = upload_vec(sc);
+    m.ycst = upload_vec(yc);
+    m.tail = upload_vec(tl);
+    m.pinv_last = h.pinv_modq[last];
+    m.pinv_last_p = shoup(m.pinv_last, ql);
+    return moddown_rescale.emplace(level, m).first->second;
+  }
+
   void init_device() {
     static_scratch = static_scratch_of_current_device();
     HIP_OK(hipStreamCreateWithFlags(&stream, hipStreamNonBlocking));
@@ -475,6 +519,8 @@ struct ace_ctx {
       conv_fp = !(force_int && force_int[0] == '1');
       const char* no_matrix = std::getenv("ACE_CONV_MATRIX");
       conv_matrix = !(no_matrix && no_matrix[0] == '0');
+      const char* no_share = std::getenv("ACE_SHARE_TRANSFORM");
+      share_transform = !(no_share && no_share[0] == '0');
       bool use_fp = conv_fp && h.logN > 12;
       std::vector<double> w(T * h.N, 0.0), iw(T * h.N, 0.0);
       for (size_t i = 0; i < T; ++i) {
@@ -1098,6 +1144,63 @@ void do_switch_key(ace_ctx* c, const PolySeq& out, const u64* digits, u64 digits
   c->ws_used = mark;
 }
 
+KeySet one_key(const u64* swk);
+// Fast_switch_key with the addend, followed by Rescale_ciphertext (evaluator.c:411-462, 342-362), for nb operands on
+// a ring of more than 4096 coefficients: results 2o and 2o+1 of `out` (level - 1 limbs) are
+// Rescale(Mod_down(inner product of operand o) + addend.at(2o), .at(2o+1)).  Mod_down ends and Rescale begins with a
+// forward transform over the same limbs; the transform is linear modulo each prime, so one transform of
+// w = -(conv * (P q_l)^-1 + Switch_modulus(last) * q_l^-1) serves both: out_t = e'_t * (P q_l)^-1 + NTT(w)_t with
+// e' = inner product + P * addend (the inner product kernel adds the lifted addend) and conv the P part of e'
+// converted to the Q basis.  The dropped limb's coefficient form, which Rescale switches to the other primes, is
+// INTT(e'_last) * P^-1 - conv_last: the inverse transform that serves the P limbs takes that limb along.
+// Every step is exact modulo its prime and Switch_modulus sees the same canonical word, so the results are the words
+// of do_switch_key followed by do_rescale.
+void do_switch_key_rescale(ace_ctx* c, const PolySeq& out, const u64* digits, u64 digits_op_stride, const u64* swk,
+                           size_t nb, size_t level, const PolySeq& addend, const OwnLimbs* own) {
+  const size_t N = c->h.N, K = c->h.K, T = level + K, kpoly = (c->h.L + K) * N, nd = c->h.num_decomp(level);
+  const size_t np = 2 * nb;
+  const ModDownRescaleDev& m = c->moddown_rescale_at(level);
+  const RescaleDev& r = c->rescale_at(level);
+  size_t mark = c->ws_used;
+  u64* e = c->take(np * T * N);        // [operand][b|a][T limbs], the addend lifted in
+  u64* t = c->take(np * (K + 1) * N);  // per polynomial: the dropped limb's z, then the scaled P limbs
+  u64* y = c->take(np * level * N);
+  LimbMap lm = poly_lm(c, level, true), kp = key_pos(c, level);
+  const Lift lift{addend, c->pmodq, (u32)level};
+  launch_dotprod(c->stream, c->d, e, e + T * N, 2 * T * N, digits, T * N, digits_op_stride, one_key(swk), kpoly,
+                 2 * kpoly, (u32)nd, lm, kp, (u32)T, (u32)nb, own, &lift);
+  launch_ntt(c->stream, c->d, seq_strided(t, (K + 1) * N), seq_strided(e + (level - 1) * N, T * N), m.inv_lm, nullptr,
+             (u32)(K + 1), (u32)np, true, m.inv_scale);
+  ConvBatch b{};
+  b.matrix = c->conv_matrix;
+  b.n_jobs = 1;
+  b.job[0] = c->p2q_job;
+  b.job[0].nc = (u32)level;
+  b.t_stride = (K + 1) * N;
+  b.out_stride = level * N;
+  launch_baseconv(c->stream, c->d, y, t + N, b, (u32)np);
+  FwdFuse f{};
+  f.pro = 2;
+  f.last_prime = (u32)(level - 1);
+  f.sw = r.sw;
+  f.z = t;
+  f.z_stride = (K + 1) * N;
+  f.ylast = y + (level - 1) * N;
+  f.ylast_stride = level * N;
+  f.pinv_last = m.pinv_last;
+  f.pinv_last_p = m.pinv_last_p;
+  f.ycst = m.ycst;
+  f.epi = 2;
+  f.out = out;
+  f.src = seq_strided(e, T * N);
+  f.addend = out;
+  f.cst = m.tail;
+  PolySeq ys = seq_strided(y, level * N);
+  if (!launch_ntt(c->stream, c->d, ys, ys, c->q_lm, nullptr, (u32)(level - 1), (u32)np, false, nullptr, 3, &f))
+    throw std::runtime_error("internal: fused Mod_down + Rescale transform rejected");
+  c->ws_used = mark;
+}
+
 KeySet one_key(const u64* swk) {
   KeySet k{};
   k.n = 1;
@@ -1119,6 +1222,11 @@ void do_mul_relin_rescale(ace_ctx* c, u64* r0, u64* r1, u64 out_stride, const u6
   const OwnLimbs own{d2, (u64)(level * N), (u32)c->h.part_size, (u32)level};
   do_precomp(c, digits, nd * T * N, d2, level * N, nb, level, true, from_d2);
   PolySeq ds = seq_strided(d01, level * N);
+  if (c->d.logN > 12 && level >= 2 && c->share_transform) {
+    do_switch_key_rescale(c, seq_pair(r0, r1, out_stride), digits, nd * T * N, swk, nb, level, ds,
+                          from_d2 ? &own : nullptr);
+    return;
+  }
   do_switch_key(c, ds, digits, nd * T * N, one_key(swk), nb, level, &ds, 1, nullptr,
                 from_d2 ? &own : nullptr);  // relinearised ct replaces d0, d1
   do_rescale(c, seq_pair(r0, r1, out_stride), ds, 2 * nb, level, true);

@@ -154,11 +154,20 @@ struct OwnLimbs {
   u64 op_stride;
   u32 part_size, level;
 };
+// An addend lifted to the extended basis on the way out (what Extend, rns_poly.c:483-500, would add before a
+// Mod_down): limb t < level of operand op's results gains addend.at(2 op) [t] * cst[2t] and addend.at(2 op + 1) [t] *
+// cst[2t] (cst: P mod q_t and its Shoup companion).  The Mod_down of such a sum is Mod_down(sum) + addend.
+struct Lift {
+  PolySeq addend;
+  const u64* cst;
+  u32 level;
+};
 // whether launch_dotprod with these arguments reads own limbs from OwnLimbs (only the kernel that shares a key does)
 bool dotprod_reads_own(u32 n_keys, u32 n_ops, bool two_halves, u32 n_parts);
 void launch_dotprod(hipStream_t st, const DevCtx& c, u64* out0, u64* out1, u64 out_stride, const u64* digits,
                     u64 digit_stride, u64 digits_op_stride, const KeySet& keys, u64 key1_off, u64 key_stride,
-                    u32 n_parts, const LimbMap& lm, const LimbMap& key_limb, u32 n_limbs, u32 n_ops, const OwnLimbs* own = nullptr);
+                    u32 n_parts, const LimbMap& lm, const LimbMap& key_limb, u32 n_limbs, u32 n_ops, const OwnLimbs* own = nullptr,
+                    const Lift* lift = nullptr);  // lift: only with both halves (out1 != null) and keys.n == 1 or n_ops == 1
 // out0[i] (+)= (sum_d digit_d * key0_d)[order[i]] (+ addend0[order[i]]), out1[i] (+)= (sum_d digit_d * key1_d)[order[i]];
 // accumulate bit 0 / 1: add to what out0 / out1 holds
 void launch_ext_rotate(hipStream_t st, const DevCtx& c, u64* out0, u64* out1, const u64* digits, u64 digit_stride,

@@ -298,7 +298,9 @@ __device__ __forceinline__ void inv_strided_stages(const A& ar, typename A::T* v
 }
 
 // What a thread of a forward strided pass starts from: R words of its column, `step` words apart from `first` on.
-// PRO = 0: read from src.  PRO = 1: formed from the last limb of a rescale (FwdFuse::pro).
+// PRO = 0: read from src.  PRO = 1: formed from the last limb of a rescale (FwdFuse::pro).  PRO = 2: the same plus
+// the source word times a constant, the last limb's word being formed from two operands on the way (a Mod_down and
+// a Rescale that share this transform).
 template <class A, int R, int PRO>
 __device__ __forceinline__ void fwd_strided_input(const A& ar, const DevCtx& c, const PolySeq& srcs, const LimbMap& pos,
                                                   const FwdFuse& f, u32 limb, u32 pi, u32 col, u64 first, u64 step,
@@ -312,30 +314,49 @@ __device__ __forceinline__ void fwd_strided_input(const A& ar, const DevCtx& c, 
     const u32 lt = pos.prime[limb];
     const u64 ql = c.primes[f.last_prime].q, half = ql >> 1;
     const u64 K = f.sw[3 * lt], Kp = f.sw[3 * lt + 1], diff = f.sw[3 * lt + 2];
-    const u64* __restrict__ last = f.last + blockIdx.z * f.last_stride + first + col;
+    // All words are requested before the first is used, and the cases below are uniform over the launch's
+    // limb: a per-word branch would make every load wait for the one before it.
+    u64 xs[R], ys[R];
+    if (PRO == 1) {
+      const u64* __restrict__ last = f.last + blockIdx.z * f.last_stride + first + col;
+#pragma unroll
+      for (int r = 0; r < R; ++r) xs[r] = last[r * step];
+    } else {
+      const u64* __restrict__ z = f.z + blockIdx.z * f.z_stride + first + col;
+      const u64* __restrict__ yl = f.ylast + blockIdx.z * f.ylast_stride + first + col;
+      const u64* __restrict__ src = srcs.at(blockIdx.z) + (u64)lt * c.N + first + col;
+      u64 zs[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r) { zs[r] = z[r * step]; xs[r] = yl[r * step]; ys[r] = ldg<2>(src + r * step); }
+#pragma unroll
+      for (int r = 0; r < R; ++r) xs[r] = sub_mod(zs[r], shoup_mul(xs[r], f.pinv_last, f.pinv_last_p, ql), ql);
+    }
+    const u64 Ay = PRO == 2 ? f.ycst[2 * lt] : 0, Ayp = PRO == 2 ? f.ycst[2 * lt + 1] : 0;
     if constexpr (A::kFp) {
       // Both primes small enough for FP64: the centred value of the last limb's word (|x| <= ql/2 <= q) times the
       // centred constant is one exact FP64 product, about a fifth of the integer path's instructions; its result
-      // (below 0.72 q) is what the stages take.
+      // (below 0.72 q) is what the stages take.  With the second product (below 0.93 q) the sum is reduced once.
       if (ql < ((u64)1 << 52) && ql <= 2 * P.q) {
         const double qld = (double)ql, halfd = (double)half;
         double kc = ar.in_canon(K);
         if (K > (P.q >> 1)) kc -= ar.q;
         const double kci = kc * ar.qinv;
+        double ac = ar.in_canon(Ay);
+        if (Ay > (P.q >> 1)) ac -= ar.q;
+        const double aci = ac * ar.qinv;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-          double x = ar.in_canon(last[r * step]);
+          double x = ar.in_canon(xs[r]);
           x = x > halfd ? x - qld : x;
           v[r] = ar.mulmod(x, kc, kci);
+          if (PRO == 2) {
+            v[r] += ar.mulmod(ar.in_canon(ys[r]), ac, aci);
+            ar.reduce(v[r]);
+          }
         }
         return;
       }
     }
-    // All words are requested before the first is used, and the three cases below are uniform over the launch's
-    // limb: a per-word branch would make every load wait for the one before it.
-    u64 xs[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) xs[r] = last[r * step];
     if (P.q > ql) {
 #pragma unroll
       for (int r = 0; r < R; ++r) xs[r] += xs[r] > half ? P.q - ql : 0;
@@ -348,7 +369,11 @@ __device__ __forceinline__ void fwd_strided_input(const A& ar, const DevCtx& c, 
       for (int r = 0; r < R; ++r) xs[r] = barrett128(0, xs[r] + (xs[r] > half ? diff : 0), P);
     }
 #pragma unroll
-    for (int r = 0; r < R; ++r) v[r] = ar.in_canon(shoup_mul(xs[r], K, Kp, P.q));
+    for (int r = 0; r < R; ++r) {
+      u64 w = shoup_mul(xs[r], K, Kp, P.q);
+      if (PRO == 2) w = add_mod(w, shoup_mul(ys[r], Ay, Ayp, P.q), P.q);
+      v[r] = ar.in_canon(w);
+    }
   }
 }
 
@@ -915,13 +940,17 @@ static void run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst, const
       dim3 gq((c.N >> 4) / kSplitCols, n_limbs, n_polys);
       if (f.pro == 0)
         hipLaunchKernelGGL((ntt_fwd_strided_split<0>), gq, dim3(256), 0, st, c, dst, src, lm, pos, f);
-      else
+      else if (f.pro == 1)
         hipLaunchKernelGGL((ntt_fwd_strided_split<1>), gq, dim3(256), 0, st, c, dst, src, lm, pos, f);
+      else
+        hipLaunchKernelGGL((ntt_fwd_strided_split<2>), gq, dim3(256), 0, st, c, dst, src, lm, pos, f);
     } else if (passes & 1) {
       if (f.pro == 0)
         hipLaunchKernelGGL((ntt_fwd_strided<LS, 0>), gs, dim3(256), 0, st, c, dst, src, lm, pos, f);
-      else
+      else if (f.pro == 1)
         hipLaunchKernelGGL((ntt_fwd_strided<LS, 1>), gs, dim3(256), 0, st, c, dst, src, lm, pos, f);
+      else
+        hipLaunchKernelGGL((ntt_fwd_strided<LS, 2>), gs, dim3(256), 0, st, c, dst, src, lm, pos, f);
     }
     if (passes & 2) {
       const u32 lr = LOGR;

@@ -764,8 +764,12 @@ __global__ __launch_bounds__(kThreads) void dotprod_kernel(DevCtx c, u64* __rest
                                                            u64 out_stride, const u64* __restrict__ digits,
                                                            u64 digit_stride, u64 digits_op_stride, KeySet keys,
                                                            u64 key1_off, u64 key_stride, u32 n_parts, LimbMap lm,
-                                                           LimbMap key_limb) {
+                                                           LimbMap key_limb, Lift lift) {
   const u32 limb = blockIdx.y, op = blockIdx.z;
+  const bool lifted = TWO && lift.cst && limb < lift.level;
+  const u64 lw = lifted ? lift.cst[2 * limb] : 0, lwp = lifted ? lift.cst[2 * limb + 1] : 0;
+  const u64* __restrict__ add0 = lifted ? lift.addend.at(2 * op) + (u64)limb * c.N : nullptr;
+  const u64* __restrict__ add1 = lifted ? lift.addend.at(2 * op + 1) + (u64)limb * c.N : nullptr;
   const DevPrime P = c.primes[lm.prime[limb]];
   const u64 n = c.N, dbase = (u64)limb * n, kbase = (u64)key_limb.prime[limb] * n;
   const u64* __restrict__ key0 = keys.p[keys.n == 1 ? 0 : op];
@@ -788,8 +792,13 @@ __global__ __launch_bounds__(kThreads) void dotprod_kernel(DevCtx c, u64* __rest
         terms = 1;
       }
     }
-    stn<256>(out0 + dbase + i, barrett_sum(h0, l0, P));
-    if (TWO) stn<256>(out1 + dbase + i, barrett_sum(h1, l1, P));
+    u64 v0 = barrett_sum(h0, l0, P), v1 = TWO ? barrett_sum(h1, l1, P) : 0;
+    if (lifted) {
+      v0 = add_mod(v0, shoup_mul(ldn<256>(add0 + i), lw, lwp, P.q), P.q);
+      v1 = add_mod(v1, shoup_mul(ldn<256>(add1 + i), lw, lwp, P.q), P.q);
+    }
+    stn<256>(out0 + dbase + i, v0);
+    if (TWO) stn<256>(out1 + dbase + i, v1);
   }
 }
 
@@ -847,9 +856,11 @@ template <int NP>
 __global__ __launch_bounds__(kThreads) void dotprod_shared_key_kernel(
     DevCtx c, u64* __restrict__ out0, u64* __restrict__ out1, u64 out_stride, const u64* __restrict__ digits,
     u64 digit_stride, u64 digits_op_stride, const u64* __restrict__ key0, u64 key1_off, u64 key_stride, LimbMap lm,
-    LimbMap key_limb, u32 n_ops, OwnLimbs own) {
+    LimbMap key_limb, u32 n_ops, OwnLimbs own, Lift lift) {
   const u32 limb = blockIdx.y;
   const DevPrime P = c.primes[lm.prime[limb]];
+  const bool lifted = lift.cst && limb < lift.level;
+  const u64 lw = lifted ? lift.cst[2 * limb] : 0, lwp = lifted ? lift.cst[2 * limb + 1] : 0;
   const u64 n = c.N, dbase = (u64)limb * n, kbase = (u64)key_limb.prime[limb] * n;
   const u64* __restrict__ key1 = key0 + key1_off;
   // the digit this limb is an own limb of (NP: none, or the digits hold their own limbs)
@@ -887,8 +898,13 @@ __global__ __launch_bounds__(kThreads) void dotprod_shared_key_kernel(
         mac128(h1, l1, x[u][d], k1[u][d]);
       }
       if (i < n) {  // NP <= 4 products: below 2^(shift + 64) for every prime below 2^61
-        stn<2>(out0 + op * out_stride + dbase + i, barrett_sum(h0, l0, P));
-        stn<2>(out1 + op * out_stride + dbase + i, barrett_sum(h1, l1, P));
+        u64 v0 = barrett_sum(h0, l0, P), v1 = barrett_sum(h1, l1, P);
+        if (lifted) {
+          v0 = add_mod(v0, shoup_mul(ldn<2>(lift.addend.at(2 * op) + dbase + i), lw, lwp, P.q), P.q);
+          v1 = add_mod(v1, shoup_mul(ldn<2>(lift.addend.at(2 * op + 1) + dbase + i), lw, lwp, P.q), P.q);
+        }
+        stn<2>(out0 + op * out_stride + dbase + i, v0);
+        stn<2>(out1 + op * out_stride + dbase + i, v1);
       }
     }
   }
@@ -956,8 +972,9 @@ bool dotprod_reads_own(u32 n_keys, u32 n_ops, bool two_halves, u32 n_parts) {
 void launch_dotprod(hipStream_t st, const DevCtx& c, u64* out0, u64* out1, u64 out_stride, const u64* digits,
                     u64 digit_stride, u64 digits_op_stride, const KeySet& keys, u64 key1_off, u64 key_stride,
                     u32 n_parts, const LimbMap& lm, const LimbMap& key_limb, u32 n_limbs, u32 n_ops,
-                    const OwnLimbs* own) {
+                    const OwnLimbs* own, const Lift* lift) {
   if (!n_limbs || !n_ops) return;
+  const Lift lf = lift ? *lift : Lift{PolySeq{{nullptr, nullptr}, 0}, nullptr, 0};
   if (dotprod_reads_own(keys.n, n_ops, out1 != nullptr, n_parts)) {
     const OwnLimbs ol = own ? *own : OwnLimbs{nullptr, 0, 1, 0};
     // NP <= 4 products of residues below 2^61 fit 128 bits without an intermediate reduction
@@ -966,13 +983,13 @@ void launch_dotprod(hipStream_t st, const DevCtx& c, u64* out0, u64* out1, u64 o
   case NP:                                                                                                       \
     hipLaunchKernelGGL(dotprod_shared_key_kernel<NP>, g, dim3(kThreads), 0, st, c, out0, out1, out_stride,       \
                        digits, digit_stride, digits_op_stride, keys.p[0], key1_off, key_stride, lm, key_limb,    \
-                       n_ops, ol);                                                                               \
+                       n_ops, ol, lf);                                                                           \
     break;
     switch (n_parts) { ACE_DP_CASE(1) ACE_DP_CASE(2) ACE_DP_CASE(3) ACE_DP_CASE(4) }
 #undef ACE_DP_CASE
     return;
   }
-  if (keys.n == n_ops && n_ops > 1 && digits_op_stride == 0 && out1 && n_parts >= 1 && n_parts <= 4) {
+  if (!lift && keys.n == n_ops && n_ops > 1 && digits_op_stride == 0 && out1 && n_parts >= 1 && n_parts <= 4) {
     dim3 g = ew_grid(c.N, n_limbs, n_ops < kSharedDigitsSplit ? n_ops : kSharedDigitsSplit);
 #define ACE_DP_CASE(NP)                                                                                          \
   case NP:                                                                                                       \
@@ -986,10 +1003,10 @@ void launch_dotprod(hipStream_t st, const DevCtx& c, u64* out0, u64* out1, u64 o
   dim3 g = ew_grid(c.N, n_limbs, n_ops);
   if (out1)
     hipLaunchKernelGGL(dotprod_kernel<true>, g, dim3(kThreads), 0, st, c, out0, out1, out_stride, digits,
-                       digit_stride, digits_op_stride, keys, key1_off, key_stride, n_parts, lm, key_limb);
+                       digit_stride, digits_op_stride, keys, key1_off, key_stride, n_parts, lm, key_limb, lf);
   else
     hipLaunchKernelGGL(dotprod_kernel<false>, g, dim3(kThreads), 0, st, c, out0, out1, out_stride, digits,
-                       digit_stride, digits_op_stride, keys, key1_off, key_stride, n_parts, lm, key_limb);
+                       digit_stride, digits_op_stride, keys, key1_off, key_stride, n_parts, lm, key_limb, lf);
 }
 
 // ---- Mod_down tail (rns_poly.c:292-303): (src - y) * P^-1 [+ addend] --------
