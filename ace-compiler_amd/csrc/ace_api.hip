@@ -68,10 +68,11 @@ struct RescaleDev {
 // Constants of a Mod_down and a Rescale that share one forward transform (do_switch_key_rescale)
 struct ModDownRescaleDev {
   u64* inv_scale = nullptr;  // [1 + K][2]: (1/N * P^-1 mod q_last) for the dropped limb, then the P limbs' Mod_down scales
-  u64* ycst = nullptr;       // [level-1][2]: -(P q_last)^-1 mod q_t
   u64* tail = nullptr;       // [level-1][2]: (P q_last)^-1 mod q_t
   LimbMap inv_lm{};          // the dropped limb, then the P limbs
-  u64 pinv_last = 0, pinv_last_p = 0;
+  // P -> Q conversion onto the level's limbs with a constant folded into each target's column of the matrix:
+  // -(P q_last)^-1 mod q_t for t < level - 1, P^-1 mod q_last for the dropped limb
+  ConvJob job{};
 };
 
 // Scratch of ace_mod_down_noalloc: the intermediates of one Mod_down (the scaled inverse transform of the P limbs
@@ -472,7 +473,7 @@ struct ace_ctx {
     const size_t last = level - 1;
     const u64 ql = h.primes[last].q;
     ModDownRescaleDev m;
-    std::vector<u64> sc(2 * (1 + h.K)), yc(2 * last), tl(2 * last);
+    std::vector<u64> sc(2 * (1 + h.K)), tl(2 * last), colc(level);
     const u64 a = mul_mod(h.primes[last].ninv, h.pinv_modq[last], ql);
     sc[0] = a; sc[1] = shoup(a, ql);
     m.inv_lm.prime[0] = (uint8_t)last;
@@ -483,15 +484,33 @@ struct ace_ctx {
     }
     for (size_t i = 0; i < last; ++i) {
       const u64 q = h.primes[i].q;
-      const u64 y = mul_mod(h.pinv_modq[i], nqi[i], q), t = mul_mod(h.pinv_modq[i], qi[i], q);
-      yc[2 * i] = y; yc[2 * i + 1] = shoup(y, q);
+      const u64 t = mul_mod(h.pinv_modq[i], qi[i], q);
+      colc[i] = mul_mod(h.pinv_modq[i], nqi[i], q);
       tl[2 * i] = t; tl[2 * i + 1] = shoup(t, q);
     }
+    colc[last] = h.pinv_modq[last];
     m.inv_scale = upload_vec(sc);
-    m.ycst = upload_vec(yc);
     m.tail = upload_vec(tl);
-    m.pinv_last = h.pinv_modq[last];
-    m.pinv_last_p = shoup(m.pinv_last, ql);
+    {
+      std::vector<u64> ph(h.K * level);
+      std::vector<size_t> src, tgt;
+      for (size_t j = 0; j < h.K; ++j) {
+        src.push_back(h.L + j);
+        for (size_t i = 0; i < level; ++i)
+          ph[j * level + i] = mul_mod(h.phat_modq[i * h.K + j], colc[i], h.primes[i].q);
+      }
+      for (size_t i = 0; i < level; ++i) {
+        tgt.push_back(i);
+        m.job.map.prime[i] = (uint8_t)i;
+        m.job.map.out_limb[i] = (uint8_t)i;
+      }
+      m.job.hat = upload_vec(ph);
+      m.job.hat_stride = (u32)level;
+      m.job.nd = (u32)h.K;
+      m.job.nc = (u32)level;
+      conv_fp_tables(m.job, src, tgt, ph.data(), level);
+      conv_matrix_tables(m.job, tgt, ph.data(), level, h.K);
+    }
     return moddown_rescale.emplace(level, m).first->second;
   }
 
@@ -1151,8 +1170,9 @@ KeySet one_key(const u64* swk);
 // forward transform over the same limbs; the transform is linear modulo each prime, so one transform of
 // w = -(conv * (P q_l)^-1 + Switch_modulus(last) * q_l^-1) serves both: out_t = e'_t * (P q_l)^-1 + NTT(w)_t with
 // e' = inner product + P * addend (the inner product kernel adds the lifted addend) and conv the P part of e'
-// converted to the Q basis.  The dropped limb's coefficient form, which Rescale switches to the other primes, is
-// INTT(e'_last) * P^-1 - conv_last: the inverse transform that serves the P limbs takes that limb along.
+// converted to the Q basis (the factor -(P q_l)^-1 is folded into the conversion's matrix).  The dropped limb's
+// coefficient form, which Rescale switches to the other primes, is INTT(e'_last) * P^-1 - conv_last * P^-1: the
+// inverse transform that serves the P limbs takes that limb along.
 // Every step is exact modulo its prime and Switch_modulus sees the same canonical word, so the results are the words
 // of do_switch_key followed by do_rescale.
 void do_switch_key_rescale(ace_ctx* c, const PolySeq& out, const u64* digits, u64 digits_op_stride, const u64* swk,
@@ -1174,8 +1194,7 @@ void do_switch_key_rescale(ace_ctx* c, const PolySeq& out, const u64* digits, u6
   ConvBatch b{};
   b.matrix = c->conv_matrix;
   b.n_jobs = 1;
-  b.job[0] = c->p2q_job;
-  b.job[0].nc = (u32)level;
+  b.job[0] = m.job;
   b.t_stride = (K + 1) * N;
   b.out_stride = level * N;
   launch_baseconv(c->stream, c->d, y, t + N, b, (u32)np);
@@ -1187,9 +1206,6 @@ void do_switch_key_rescale(ace_ctx* c, const PolySeq& out, const u64* digits, u6
   f.z_stride = (K + 1) * N;
   f.ylast = y + (level - 1) * N;
   f.ylast_stride = level * N;
-  f.pinv_last = m.pinv_last;
-  f.pinv_last_p = m.pinv_last_p;
-  f.ycst = m.ycst;
   f.epi = 2;
   f.out = out;
   f.src = seq_strided(e, T * N);

@@ -186,10 +186,11 @@ struct OrderSet {  // one automorphism table per rotation, or one shared (n == 1
 //          Switch_modulus(last[p*last_stride + i], q_last -> q_t) * sw[3t] (Shoup sw[3t+1], sw[3t+2] = q_t - q_last mod q_t)
 //   pro 2  Mod_down and Rescale sharing one forward transform (the transform is linear, so the two that
 //          Mod_down and Rescale would run one after the other on the same limbs are one transform of a sum): with
-//          y = the P part converted to the Q basis (the transform's source, limb t) and z = the inverse transform of
-//          the dropped limb of (polynomial + P * addend) scaled by P^-1,
-//            last[i]   = z[p*z_stride + i] - ylast[p*ylast_stride + i] * pinv_last            (mod q_last)
-//            input[i]  = Switch_modulus(last[i], q_last -> q_t) * sw[3t] + y_t[i] * ycst[2t]  (mod q_t)
+//          y_t = -(P q_last)^-1 times the P part converted to prime t (the transform's source; the constant is part
+//          of the conversion's matrix), ylast = P^-1 times the P part converted to the dropped prime, and z = the
+//          inverse transform of the dropped limb of (polynomial + P * addend) scaled by P^-1,
+//            last[i]   = z[p*z_stride + i] - ylast[p*ylast_stride + i]                (mod q_last)
+//            input[i]  = Switch_modulus(last[i], q_last -> q_t) * sw[3t] + y_t[i]     (mod q_t)
 //          `last` is the word Rescale's inverse transform of the Mod_down result's last limb would hold.
 //   epi 1  Mod_down tail (rns_poly.c:292-303): out = (src - ntt) * cst[2t] (+ addend).  With index tables
 //          (orders.n != 0; polynomials 2r and 2r+1 use table r) the automorphism that ends a rotation is applied
@@ -207,8 +208,6 @@ struct FwdFuse {
   const u64* sw;
   const u64 *z, *ylast;  // pro 2
   u64 z_stride, ylast_stride;
-  u64 pinv_last, pinv_last_p;
-  const u64* ycst;
   PolySeq out, src, addend;
   int addend_mode;
   const u64* cst;

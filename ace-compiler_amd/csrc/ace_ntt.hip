@@ -299,8 +299,8 @@ __device__ __forceinline__ void inv_strided_stages(const A& ar, typename A::T* v
 
 // What a thread of a forward strided pass starts from: R words of its column, `step` words apart from `first` on.
 // PRO = 0: read from src.  PRO = 1: formed from the last limb of a rescale (FwdFuse::pro).  PRO = 2: the same plus
-// the source word times a constant, the last limb's word being formed from two operands on the way (a Mod_down and
-// a Rescale that share this transform).
+// the source word, the last limb's word being the difference of two operands (a Mod_down and a Rescale that share
+// this transform).
 template <class A, int R, int PRO>
 __device__ __forceinline__ void fwd_strided_input(const A& ar, const DevCtx& c, const PolySeq& srcs, const LimbMap& pos,
                                                   const FwdFuse& f, u32 limb, u32 pi, u32 col, u64 first, u64 step,
@@ -329,28 +329,24 @@ __device__ __forceinline__ void fwd_strided_input(const A& ar, const DevCtx& c, 
 #pragma unroll
       for (int r = 0; r < R; ++r) { zs[r] = z[r * step]; xs[r] = yl[r * step]; ys[r] = ldg<2>(src + r * step); }
 #pragma unroll
-      for (int r = 0; r < R; ++r) xs[r] = sub_mod(zs[r], shoup_mul(xs[r], f.pinv_last, f.pinv_last_p, ql), ql);
+      for (int r = 0; r < R; ++r) xs[r] = sub_mod(zs[r], xs[r], ql);
     }
-    const u64 Ay = PRO == 2 ? f.ycst[2 * lt] : 0, Ayp = PRO == 2 ? f.ycst[2 * lt + 1] : 0;
     if constexpr (A::kFp) {
       // Both primes small enough for FP64: the centred value of the last limb's word (|x| <= ql/2 <= q) times the
       // centred constant is one exact FP64 product, about a fifth of the integer path's instructions; its result
-      // (below 0.72 q) is what the stages take.  With the second product (below 0.93 q) the sum is reduced once.
+      // (below 0.93 q) is what the stages take.  With the source word added (PRO = 2) the sum is reduced once.
       if (ql < ((u64)1 << 52) && ql <= 2 * P.q) {
         const double qld = (double)ql, halfd = (double)half;
         double kc = ar.in_canon(K);
         if (K > (P.q >> 1)) kc -= ar.q;
         const double kci = kc * ar.qinv;
-        double ac = ar.in_canon(Ay);
-        if (Ay > (P.q >> 1)) ac -= ar.q;
-        const double aci = ac * ar.qinv;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
           double x = ar.in_canon(xs[r]);
           x = x > halfd ? x - qld : x;
           v[r] = ar.mulmod(x, kc, kci);
           if (PRO == 2) {
-            v[r] += ar.mulmod(ar.in_canon(ys[r]), ac, aci);
+            v[r] += ar.in_canon(ys[r]);
             ar.reduce(v[r]);
           }
         }
@@ -371,7 +367,7 @@ __device__ __forceinline__ void fwd_strided_input(const A& ar, const DevCtx& c, 
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       u64 w = shoup_mul(xs[r], K, Kp, P.q);
-      if (PRO == 2) w = add_mod(w, shoup_mul(ys[r], Ay, Ayp, P.q), P.q);
+      if (PRO == 2) w = add_mod(w, ys[r], P.q);
       v[r] = ar.in_canon(w);
     }
   }
@@ -778,11 +774,13 @@ __device__ __forceinline__ void inv_strided_body(const DevCtx& c, const PolySeq&
 }
 // ONLY: 0 = limbs of both back ends (the choice is uniform over a work-group), 1 = integer limbs only, 2 = FP64
 // limbs only.  The two bodies in one function need 130 registers at LOGR = 4 where each alone needs 78 / 90, and
-// most launches are of one kind (the special primes of a Mod_down, the digit of a Mod_up).
+// most launches are of one kind (the special primes of a Mod_down, the digit of a Mod_up).  A launch covers the limbs
+// limb0 .. limb0 + gridDim.y - 1 of the transform, so that a transform whose limbs change kind once or twice along
+// the list is served by one launch of the fitting kind per stretch.
 template <int LOGR, int ONLY>
 __global__ __launch_bounds__(256) void ntt_inv_strided(DevCtx c, PolySeq datas, LimbMap lm, LimbMap pos,
-                                                       const u64* __restrict__ scale) {
-  const u32 limb = gridDim.y - 1 - blockIdx.y, pi = lm.prime[limb];
+                                                       const u64* __restrict__ scale, u32 limb0) {
+  const u32 limb = limb0 + gridDim.y - 1 - blockIdx.y, pi = lm.prime[limb];
   if (ONLY == 2 || (ONLY == 0 && c.fp_ok[pi])) inv_strided_body<ArithFp, LOGR>(c, datas, pos, scale, limb, pi);
   else inv_strided_body<ArithInt, LOGR>(c, datas, pos, scale, limb, pi);
 }
@@ -979,14 +977,25 @@ static void run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst, const
       dim3 gq((c.N >> 4) / kSplitCols, n_limbs, n_polys);
       hipLaunchKernelGGL(ntt_inv_strided_split, gq, dim3(256), 0, st, c, dst, lm, pos, scale);
     } else if (passes & 2) {
-      u32 n_fp = 0;
-      for (u32 t = 0; t < n_limbs; ++t) n_fp += c.fp_ok[lm.prime[t]] ? 1 : 0;
-      if (n_fp == 0)
-        hipLaunchKernelGGL((ntt_inv_strided<LS, 1>), gs, dim3(256), 0, st, c, dst, lm, pos, scale);
-      else if (n_fp == n_limbs)
-        hipLaunchKernelGGL((ntt_inv_strided<LS, 2>), gs, dim3(256), 0, st, c, dst, lm, pos, scale);
-      else
-        hipLaunchKernelGGL((ntt_inv_strided<LS, 0>), gs, dim3(256), 0, st, c, dst, lm, pos, scale);
+      // stretches of limbs of one kind
+      u32 starts[4], n_runs = 0;
+      for (u32 t = 0; t < n_limbs; ++t)
+        if (t == 0 || c.fp_ok[lm.prime[t]] != c.fp_ok[lm.prime[t - 1]]) {
+          if (n_runs < 4) starts[n_runs] = t;
+          ++n_runs;
+        }
+      if (n_runs <= 3) {
+        for (u32 k = 0; k < n_runs; ++k) {
+          const u32 a = starts[k], b = k + 1 < n_runs ? starts[k + 1] : n_limbs;
+          dim3 gr(gs.x, b - a, n_polys);
+          if (c.fp_ok[lm.prime[a]])
+            hipLaunchKernelGGL((ntt_inv_strided<LS, 2>), gr, dim3(256), 0, st, c, dst, lm, pos, scale, a);
+          else
+            hipLaunchKernelGGL((ntt_inv_strided<LS, 1>), gr, dim3(256), 0, st, c, dst, lm, pos, scale, a);
+        }
+      } else {
+        hipLaunchKernelGGL((ntt_inv_strided<LS, 0>), gs, dim3(256), 0, st, c, dst, lm, pos, scale, 0u);
+      }
     }
   }
 }
