@@ -1176,7 +1176,7 @@ KeySet one_key(const u64* swk);
 // Every step is exact modulo its prime and Switch_modulus sees the same canonical word, so the results are the words
 // of do_switch_key followed by do_rescale.
 void do_switch_key_rescale(ace_ctx* c, const PolySeq& out, const u64* digits, u64 digits_op_stride, const u64* swk,
-                           size_t nb, size_t level, const PolySeq& addend, const OwnLimbs* own) {
+                           size_t nb, size_t level, const Lift& lift, const OwnLimbs* own) {
   const size_t N = c->h.N, K = c->h.K, T = level + K, kpoly = (c->h.L + K) * N, nd = c->h.num_decomp(level);
   const size_t np = 2 * nb;
   const ModDownRescaleDev& m = c->moddown_rescale_at(level);
@@ -1186,7 +1186,6 @@ void do_switch_key_rescale(ace_ctx* c, const PolySeq& out, const u64* digits, u6
   u64* t = c->take(np * (K + 1) * N);  // per polynomial: the dropped limb's z, then the scaled P limbs
   u64* y = c->take(np * level * N);
   LimbMap lm = poly_lm(c, level, true), kp = key_pos(c, level);
-  const Lift lift{addend, c->pmodq, (u32)level};
   launch_dotprod(c->stream, c->d, e, e + T * N, 2 * T * N, digits, T * N, digits_op_stride, one_key(swk), kpoly,
                  2 * kpoly, (u32)nd, lm, kp, (u32)T, (u32)nb, own, &lift);
   launch_ntt(c->stream, c->d, seq_strided(t, (K + 1) * N), seq_strided(e + (level - 1) * N, T * N), m.inv_lm, nullptr,
@@ -1228,18 +1227,24 @@ KeySet one_key(const u64* swk) {
 void do_mul_relin_rescale(ace_ctx* c, u64* r0, u64* r1, u64 out_stride, const u64* a0, const u64* a1, const u64* b0,
                           const u64* b1, u64 in_stride, const u64* swk, size_t nb, size_t level) {
   const size_t N = c->h.N, nd = c->h.num_decomp(level), T = level + c->h.K;
-  u64* d01 = c->take(nb * 2 * level * N);  // [operand][c0|c1][level limbs]
-  u64* d2 = c->take(nb * level * N);
-  u64* digits = c->take(nb * nd * T * N);
-  launch_tensor(c->stream, c->d, d01, d01 + level * N, d2, a0, a1, b0, b1, c->q_lm, (u32)level, (u32)nb,
-                2 * level * N, level * N, in_stride);
   // where the inner product can read the digits' own limbs from d2 itself, Mod_up does not copy them
   const bool from_d2 = c->d.logN > 12 && dotprod_reads_own(1, (u32)nb, true, (u32)nd);
+  const bool shared = c->d.logN > 12 && level >= 2 && c->share_transform;
+  // the same kernel can form the first two terms of the tensor product where it adds them, lifted, to its sums:
+  // they are then neither written nor read back
+  const bool on_the_way = shared && from_d2;
+  u64* d01 = on_the_way ? nullptr : c->take(nb * 2 * level * N);  // [operand][c0|c1][level limbs]
+  u64* d2 = c->take(nb * level * N);
+  u64* digits = c->take(nb * nd * T * N);
+  launch_tensor(c->stream, c->d, d01, d01 ? d01 + level * N : nullptr, d2, a0, a1, b0, b1, c->q_lm, (u32)level,
+                (u32)nb, 2 * level * N, level * N, in_stride);
   const OwnLimbs own{d2, (u64)(level * N), (u32)c->h.part_size, (u32)level};
   do_precomp(c, digits, nd * T * N, d2, level * N, nb, level, true, from_d2);
-  PolySeq ds = seq_strided(d01, level * N);
-  if (c->d.logN > 12 && level >= 2 && c->share_transform) {
-    do_switch_key_rescale(c, seq_pair(r0, r1, out_stride), digits, nd * T * N, swk, nb, level, ds,
+  PolySeq ds = seq_strided(d01 ? d01 : d2, level * N);  // (never read when the terms are formed on the way)
+  if (shared) {
+    Lift lift{ds, c->pmodq, (u32)level, nullptr, nullptr, nullptr, nullptr, 0};
+    if (on_the_way) lift.a0 = a0, lift.a1 = a1, lift.b0 = b0, lift.b1 = b1, lift.in_stride = in_stride;
+    do_switch_key_rescale(c, seq_pair(r0, r1, out_stride), digits, nd * T * N, swk, nb, level, lift,
                           from_d2 ? &own : nullptr);
     return;
   }

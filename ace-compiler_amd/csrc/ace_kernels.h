@@ -136,7 +136,7 @@ void launch_gather(hipStream_t st, const DevCtx& c, u64* r, const u64* a, const 
 // n_rot rotations: rotation z gathers (a0,a1) + z*a_stride into (r0,r1) + z*r_stride with table orders.p[z]
 void launch_gather2(hipStream_t st, const DevCtx& c, u64* r0, u64* r1, u64 r_stride, const u64* a0, const u64* a1,
                     u64 a_stride, const OrderSet& orders, const LimbMap& lm, u32 n_limbs, u32 n_rot);
-// tensor product of n_ops ciphertext pairs: d0 = a0*b0, d1 = a0*b1 + a1*b0, d2 = a1*b1
+// tensor product of n_ops ciphertext pairs: d0 = a0*b0, d1 = a0*b1 + a1*b0, d2 = a1*b1; d0 == null: d2 only
 void launch_tensor(hipStream_t st, const DevCtx& c, u64* d0, u64* d1, u64* d2, const u64* a0, const u64* a1,
                    const u64* b0, const u64* b1, const LimbMap& lm, u32 n_limbs, u32 n_ops, u64 d01_stride,
                    u64 d2_stride, u64 in_stride);
@@ -157,10 +157,14 @@ struct OwnLimbs {
 // An addend lifted to the extended basis on the way out (what Extend, rns_poly.c:483-500, would add before a
 // Mod_down): limb t < level of operand op's results gains addend.at(2 op) [t] * cst[2t] and addend.at(2 op + 1) [t] *
 // cst[2t] (cst: P mod q_t and its Shoup companion).  The Mod_down of such a sum is Mod_down(sum) + addend.
+// With a0 set the addend is the tensor product of operand op's ciphertexts, formed on the way instead of being read:
+// (a0 b0, a0 b1 + a1 b0) at a0 + op * in_stride etc. (only the kernel that shares one key among the operands).
 struct Lift {
   PolySeq addend;
   const u64* cst;
   u32 level;
+  const u64 *a0, *a1, *b0, *b1;
+  u64 in_stride;
 };
 // whether launch_dotprod with these arguments reads own limbs from OwnLimbs (only the kernel that shares a key does)
 bool dotprod_reads_own(u32 n_keys, u32 n_ops, bool two_halves, u32 n_parts);

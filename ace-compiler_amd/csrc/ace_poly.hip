@@ -414,10 +414,29 @@ __global__ __launch_bounds__(kThreads) void tensor_kernel(DevCtx c, u64* __restr
   }
 }
 
+// the last term alone, for callers that form the other two where they are consumed (Lift)
+__global__ __launch_bounds__(kThreads) void tensor_d2_kernel(DevCtx c, u64* __restrict__ d2, const u64* __restrict__ a1,
+                                                             const u64* __restrict__ b1, LimbMap lm, u64 d2_stride,
+                                                             u64 in_stride) {
+  const u32 limb = blockIdx.y;
+  const DevPrime P = c.primes[lm.prime[limb]];
+  const u64 n = c.N, base = (u64)limb * n;
+  d2 += blockIdx.z * d2_stride;
+  a1 += blockIdx.z * in_stride;
+  b1 += blockIdx.z * in_stride;
+#pragma unroll
+  ACE_EW_LOOP(i, n) stn<1>(d2 + base + i, mulmod(ldn<1>(a1 + base + i), ldn<1>(b1 + base + i), P));
+}
+
 void launch_tensor(hipStream_t st, const DevCtx& c, u64* d0, u64* d1, u64* d2, const u64* a0, const u64* a1,
                    const u64* b0, const u64* b1, const LimbMap& lm, u32 n_limbs, u32 n_ops, u64 d01_stride,
                    u64 d2_stride, u64 in_stride) {
   if (!n_limbs || !n_ops) return;
+  if (!d0) {
+    hipLaunchKernelGGL(tensor_d2_kernel, ew_grid(c.N, n_limbs, n_ops), dim3(kThreads), 0, st, c, d2, a1, b1, lm,
+                       d2_stride, in_stride);
+    return;
+  }
   hipLaunchKernelGGL(tensor_kernel, ew_grid(c.N, n_limbs, n_ops), dim3(kThreads), 0, st, c, d0, d1, d2, a0, a1, b0,
                      b1, lm, d01_stride, d2_stride, in_stride);
 }
@@ -899,7 +918,15 @@ __global__ __launch_bounds__(kThreads) void dotprod_shared_key_kernel(
       }
       if (i < n) {  // NP <= 4 products: below 2^(shift + 64) for every prime below 2^61
         u64 v0 = barrett_sum(h0, l0, P), v1 = barrett_sum(h1, l1, P);
-        if (lifted) {
+        if (lifted && lift.a0) {
+          const u64 o = op * lift.in_stride + dbase + i;
+          const u64 x0 = ldn<2>(lift.a0 + o), x1 = ldn<2>(lift.a1 + o), y0 = ldn<2>(lift.b0 + o), y1 = ldn<2>(lift.b1 + o);
+          u64 h = 0, l = 0;  // two products of residues stay below 2^(shift + 64)
+          mac128(h, l, x0, y1);
+          mac128(h, l, x1, y0);
+          v0 = add_mod(v0, shoup_mul(mulmod(x0, y0, P), lw, lwp, P.q), P.q);
+          v1 = add_mod(v1, shoup_mul(barrett_sum(h, l, P), lw, lwp, P.q), P.q);
+        } else if (lifted) {
           v0 = add_mod(v0, shoup_mul(ldn<2>(lift.addend.at(2 * op) + dbase + i), lw, lwp, P.q), P.q);
           v1 = add_mod(v1, shoup_mul(ldn<2>(lift.addend.at(2 * op + 1) + dbase + i), lw, lwp, P.q), P.q);
         }
@@ -974,7 +1001,7 @@ void launch_dotprod(hipStream_t st, const DevCtx& c, u64* out0, u64* out1, u64 o
                     u32 n_parts, const LimbMap& lm, const LimbMap& key_limb, u32 n_limbs, u32 n_ops,
                     const OwnLimbs* own, const Lift* lift) {
   if (!n_limbs || !n_ops) return;
-  const Lift lf = lift ? *lift : Lift{PolySeq{{nullptr, nullptr}, 0}, nullptr, 0};
+  const Lift lf = lift ? *lift : Lift{PolySeq{{nullptr, nullptr}, 0}, nullptr, 0, nullptr, nullptr, nullptr, nullptr, 0};
   if (dotprod_reads_own(keys.n, n_ops, out1 != nullptr, n_parts)) {
     const OwnLimbs ol = own ? *own : OwnLimbs{nullptr, 0, 1, 0};
     // NP <= 4 products of residues below 2^61 fit 128 bits without an intermediate reduction
