@@ -55,6 +55,7 @@ def _sig(lib):
     f("ace_copy", C.c_int, _vp, _vp, _vp, _sz)
     f("ace_zero", C.c_int, _vp, _vp, _sz)
     f("ace_sync", C.c_int, _vp)
+    f("ace_memory_stats", None, _vp, C.POINTER(C.c_size_t))
     f("ace_timer_start", C.c_int, _vp)
     f("ace_timer_stop_ms", C.c_float, _vp)
     f("ace_ntt", C.c_int, _vp, _vp, _vp, _i32p, _sz, _sz, _sz)
@@ -117,7 +118,7 @@ EXPORTS = [
     "ace_degree", "ace_num_q", "ace_num_p", "ace_num_parts", "ace_part_size", "ace_num_decomp", "ace_prime",
     "ace_root", "ace_modulus", "ace_host_twiddles", "ace_host_tbl_modup", "ace_host_tbl_moddown",
     "ace_host_tbl_rescale", "ace_host_automorphism_order", "ace_alloc", "ace_free", "ace_upload", "ace_download",
-    "ace_copy", "ace_zero", "ace_sync", "ace_timer_start", "ace_timer_stop_ms", "ace_ntt", "ace_intt", "ace_ntt_pass",
+    "ace_copy", "ace_zero", "ace_sync", "ace_memory_stats", "ace_timer_start", "ace_timer_stop_ms", "ace_ntt", "ace_intt", "ace_ntt_pass",
     "ace_hw_modadd", "ace_hw_modsub", "ace_hw_modmul", "ace_hw_modmuladd", "ace_hw_modadd_scalar",
     "ace_hw_modsub_scalar", "ace_hw_modmul_scalar", "ace_hw_modmuladd_scalar", "ace_hw_rotate",
     "ace_find_automorphism_index", "ace_automorphism_order", "ace_poly_add", "ace_poly_sub", "ace_poly_mul",
@@ -277,6 +278,12 @@ class Context:
 
     def sync(self):
         self._chk(self.lib.ace_sync(self.h))
+
+    def memory_stats(self):
+        """(arena words, pooled words, live buffers, pooled buffers) of the context right now."""
+        out = (C.c_size_t * 4)()
+        self.lib.ace_memory_stats(self.h, out)
+        return tuple(int(v) for v in out)
 
     def timer_start(self):
         self._chk(self.lib.ace_timer_start(self.h))

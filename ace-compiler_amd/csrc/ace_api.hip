@@ -224,6 +224,43 @@ struct ace_ctx {
           "scale_mod_size or decrease scale of msg");
     }
   }
+  // Index tables of rotations seen so far -> whether the forward chunk pass may apply them on the way out (every
+  // 4096-word block of the table draws on one block of the source, and the blocks' sources are a permutation:
+  // true of Precompute_automorphism_order's NTT-form tables, number_theory.c:211-222).  Tables made by
+  // ace_automorphism_order are entered as they are made, a caller's own table is examined on the device when a
+  // rotation first uses it; writing to a table through this library (upload, copy, zero, free) forgets the verdict.
+  std::unordered_map<const void*, bool> order_fits;
+  u32* order_report = nullptr;  // [1 + N / 4096] on the device
+  void forget_orders(const void* dst, size_t words) {
+    if (order_fits.empty()) return;
+    const uintptr_t lo = (uintptr_t)dst, hi = lo + words * sizeof(u64);
+    for (auto it = order_fits.begin(); it != order_fits.end();) {
+      const uintptr_t a = (uintptr_t)it->first, b = a + (size_t)h.N * sizeof(i64);
+      if (a < hi && lo < b) it = order_fits.erase(it);
+      else ++it;
+    }
+  }
+  bool order_fits_chunks(const i64* order) {
+    auto it = order_fits.find(order);
+    if (it != order_fits.end()) return it->second;
+    bool ok = false;
+    if (d.logN > 12) {
+      const u32 nb = h.N >> 12;
+      std::vector<u32> rep(1 + nb, 0);
+      HIP_OK(hipMemsetAsync(order_report, 0, rep.size() * sizeof(u32), stream));
+      launch_order_check(stream, d, order, order_report);
+      HIP_OK(hipMemcpyAsync(rep.data(), order_report, rep.size() * sizeof(u32), hipMemcpyDeviceToHost, stream));
+      HIP_OK(hipStreamSynchronize(stream));
+      ok = rep[0] == 0;
+      std::vector<char> seen(nb, 0);
+      for (u32 b = 0; ok && b < nb; ++b) {
+        if (rep[1 + b] >= nb || seen[rep[1 + b]]) ok = false;
+        else seen[rep[1 + b]] = 1;
+      }
+    }
+    order_fits[order] = ok;
+    return ok;
+  }
   LimbMap q_lm{}, p_lm{};     // identity maps: limb t -> prime t / prime L+t
   // ace_alloc / ace_free: sizes of the buffers handed out, and freed buffers kept for reuse
   static constexpr size_t kPoolLimitWords = (size_t)4 << 30;  // 32 GiB
@@ -601,6 +638,10 @@ struct ace_ctx {
       p2q_job.nc = (u32)h.L;
       conv_fp_tables(p2q_job, src, tgt, ph.data(), h.L);
       conv_matrix_tables(p2q_job, tgt, ph.data(), h.L, h.K);
+    }
+    {
+      std::vector<u32> rep(1 + (h.N >> 12) + 1, 0);
+      order_report = upload_vec(rep);
     }
     pscale_ntt = upload_vec(sn);
     pscale_coef = upload_vec(scf);
@@ -1049,7 +1090,10 @@ void do_mod_down(ace_ctx* c, const PolySeq& res, const PolySeq& src, size_t np, 
   launch_baseconv(c->stream, c->d, y, t, b, (u32)np);
   if (is_ntt) {
     PolySeq ys = seq_strided(y, level * N);
-    if (c->d.logN > 12) {  // the tail, and with `orders` the automorphism, ride on the transform's last kernel
+    bool fits = true;  // index tables of another make go through the separate tail, which takes any table
+    if (orders && c->d.logN > 12)
+      for (u32 k = 0; k < orders->n; ++k) fits = fits && c->order_fits_chunks(orders->p[k]);
+    if (c->d.logN > 12 && fits) {  // the tail, and with `orders` the automorphism, ride on the transform's last kernel
       FwdFuse f{};
       f.epi = 1;
       if (orders) f.orders = *orders;
@@ -1459,6 +1503,7 @@ void ace_free(ace_ctx* c, int64_t* p) {
   auto it = c->live.find(p);
   if (it == c->live.end()) return;  // not from ace_alloc of this context (a view, or freed twice)
   const size_t words = it->second;
+  c->forget_orders(p, words);
   try {  // recorded calls may still name this buffer; a zero fill of it that nothing has looked at is moot
     c->flush_pending_declared({ace_ctx::span(p, words)}, {});
   } catch (const std::exception& e) {
@@ -1478,6 +1523,7 @@ void ace_free(ace_ctx* c, int64_t* p) {
 static constexpr size_t kRecordedWords = (size_t)1 << 20;
 int ace_upload(ace_ctx* c, int64_t* dst, const int64_t* src, size_t n) {
   ACE_TRY
+  c->forget_orders(dst, n);
   HIP_OK(hipMemcpyAsync(dst, src, n * sizeof(u64), hipMemcpyHostToDevice, c->stream));
   HIP_OK(hipStreamSynchronize(c->stream));
   ACE_CATCH_INT
@@ -1492,6 +1538,7 @@ int ace_copy(ace_ctx* c, int64_t* dst, const int64_t* src, size_t n) {
   ACE_TRY_KEEP_RUN
   if (!dst || !src) return fail("ace_copy: null argument");
   if (dst == src || n == 0) return 0;
+  c->forget_orders(dst, n);
   if (c->batching && n <= kRecordedWords) {  // a copy is an elementwise entry like any other
     // whole limbs go in limb by limb, so that they join the limb-sized calls around them in one run
     const size_t N = c->h.N, pieces = (n % N == 0 && n / N <= 16) ? n / N : 1, each = n / pieces;
@@ -1507,6 +1554,7 @@ int ace_zero(ace_ctx* c, int64_t* dst, size_t n) {
   ACE_TRY_KEEP_RUN
   if (!dst) return fail("ace_zero: null argument");
   if (n == 0) return 0;
+  c->forget_orders(dst, n);
   if (c->batching && n <= kRecordedWords) {
     const size_t N = c->h.N, pieces = (n % N == 0 && n / N <= 16) ? n / N : 1, each = n / pieces;
     for (size_t t = 0; t < pieces; ++t)
@@ -1558,6 +1606,12 @@ int ace_join(ace_ctx* c) {
   ACE_CATCH_INT
 }
 
+void ace_memory_stats(const ace_ctx* c, size_t out[4]) {
+  out[0] = c->ws_words;
+  out[1] = c->pooled_words;
+  out[2] = c->live.size();
+  out[3] = c->pool.size();
+}
 int ace_timer_start(ace_ctx* c) {
   ACE_TRY
   HIP_OK(hipEventRecord(c->ev0, c->stream));
@@ -1733,6 +1787,8 @@ int ace_automorphism_order(ace_ctx* c, int64_t* dev_order, uint32_t k, int is_nt
   automorphism_order(ord.data(), k, c->h.N, is_ntt != 0);
   c->h2d(dev_order, ord.data(), ord.size() * sizeof(i64));
   HIP_OK(hipStreamSynchronize(c->stream));
+  c->forget_orders(dev_order, c->h.N);
+  if (is_ntt) c->order_fits[dev_order] = true;
   ACE_CATCH_INT
 }
 
@@ -1983,6 +2039,8 @@ int ace_mod_down_noalloc(ace_ctx* c, int64_t* res, const int64_t* src, size_t le
   ACE_TRY_BARE
   if (!res || !src) return fail("ace_mod_down_noalloc: null argument");
   if (!level_ok(c, level)) return fail("ace_mod_down_noalloc: level out of range");
+  if (c->fork_state)  // both lanes would use the one static array
+    return fail("ace_mod_down_noalloc: not between ace_fork and ace_join (the static scratch serves one stream)");
   const size_t need = (level + c->h.K) * (size_t)c->h.N;
   if (need > kStaticScratchWords)
     return fail("ace_mod_down_noalloc: (level + num_p) * degree = " + std::to_string(need) + " words exceeds the static "
@@ -2162,7 +2220,10 @@ static int encode_impl(ace_ctx* c, int64_t* res, const void* values, int kind, s
   if (p_cnt != 0 && p_cnt != K) return fail("ace_encode: p_cnt must be 0 or the number of special primes");
   const bool by_scale = explicit_scale > 0.0;
   if (by_scale) {
-    if ((uint32_t)std::log2(explicit_scale) >= c->q0_bits + (level - 1) * c->sf_bits) return fail("invalid scale for encode");
+    // (encoder.c:355-357 casts log2(scale) to uint32_t and derives the scale degree the same way; below 1 both
+    // conversions are out of range and what the reference then does depends on the compiler: refused here)
+    if (explicit_scale < 1.0 || std::log2(explicit_scale) >= (double)(c->q0_bits + (level - 1) * c->sf_bits))
+      return fail("invalid scale for encode");
     sf_degree = 1;
   } else if (sf_degree < 1 || c->sf_bits * sf_degree >= c->q0_bits + (level - 1) * c->sf_bits) {
     return fail("invalid scaling factor for encode");
@@ -2355,6 +2416,11 @@ int ace_mul_relin_rescale_batch(ace_ctx* c, int64_t* r0, int64_t* r1, size_t out
   ACE_CATCH_INT
 }
 
+static bool ranges_overlap(const void* a, size_t a_words, const void* b, size_t b_words) {
+  const uintptr_t x = (uintptr_t)a, y = (uintptr_t)b;
+  return x < y + b_words * sizeof(u64) && y < x + a_words * sizeof(u64);
+}
+
 // Fast_rotate for nr <= kMaxBatchPtrs rotations of one ciphertext sharing the digits:
 // switch key, add c0 to the first polynomial, permute -- the last two inside the Mod_down tail
 static void do_fast_rotate(ace_ctx* c, u64* r0, u64* r1, u64 r_stride, const u64* c0, const u64* digits,
@@ -2368,7 +2434,12 @@ int ace_fast_rotate(ace_ctx* c, int64_t* r0, int64_t* r1, const int64_t* c0, con
   ACE_TRY
   if (!r0 || !r1 || !c0 || !digits || !swk || !order) return fail("ace_fast_rotate: null argument");
   if (!level_ok(c, level)) return fail("ace_fast_rotate: level out of range");
-  if (r0 == c0 || r1 == c0) return fail("ace_fast_rotate: the result must not overwrite c0 (it is permuted on the way out)");
+  {
+    const size_t pw = level * (size_t)c->h.N, dw = c->h.num_decomp(level) * (level + c->h.K) * (size_t)c->h.N;
+    if (ranges_overlap(r0, pw, c0, pw) || ranges_overlap(r1, pw, c0, pw) || ranges_overlap(r0, pw, digits, dw) ||
+        ranges_overlap(r1, pw, digits, dw) || ranges_overlap(r0, pw, r1, pw))
+      return fail("ace_fast_rotate: the results must not overlap c0, the digits or each other (they are permuted on the way out)");
+  }
   c->ensure_ws(c->std_ws(level));
   c->ws_used = 0;
   OrderSet os{};
@@ -2384,7 +2455,11 @@ int ace_rotate_batch(ace_ctx* c, int64_t* r0s, int64_t* r1s, const int64_t* c0, 
   if (count == 0) return 0;
   if (!r0s || !r1s || !c0 || !c1 || !swks || !orders) return fail("ace_rotate_batch: null argument");
   if (!level_ok(c, level)) return fail("ace_rotate_batch: level out of range");
-  if (r0s == c0 || r1s == c0) return fail("ace_rotate_batch: the results must not overwrite c0 (it is permuted on the way out)");
+  {
+    const size_t pw = level * (size_t)c->h.N, rw = count * pw;
+    if (ranges_overlap(r0s, rw, c0, pw) || ranges_overlap(r1s, rw, c0, pw) || ranges_overlap(r0s, rw, r1s, rw))
+      return fail("ace_rotate_batch: the results must not overlap c0 or each other (they are permuted on the way out)");
+  }
   for (size_t i = 0; i < count; ++i)
     if (!swks[i] || !orders[i]) return fail("ace_rotate_batch: null key or order table");
   const size_t N = c->h.N, nd = c->h.num_decomp(level), T = level + c->h.K;

@@ -201,6 +201,10 @@ void launch_from_level0(hipStream_t st, const DevCtx& c, u64* out, const u64* sr
 void launch_mul_const(hipStream_t st, const DevCtx& c, u64* out, const u64* src, const u64* cst, const LimbMap& lm,
                       u32 n_limbs);
 void launch_fill_zero(hipStream_t st, u64* p, u64 n);
+// What the forward chunk pass needs of an index table before it can apply it on the way out (FwdFuse, epi 1):
+// report[0] = 1 if an entry lies outside [0, N) or a 4096-word block of the table draws on more than one block of
+// the source; report[1 + b] = the source block of block b.  report: 1 + N / 4096 words, zeroed by the kernel's caller.
+void launch_order_check(hipStream_t st, const DevCtx& c, const i64* order, u32* report);
 // Embedding_inv (util/src/ntt.c:631-675) over len complex values: out = result, r = input (overwritten)
 void launch_embedding_inv(hipStream_t st, const DevCtx& c, double2* out, double2* r, const double2* rou,
                           const u32* rot, u32 len);

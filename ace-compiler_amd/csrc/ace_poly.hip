@@ -774,6 +774,18 @@ void launch_digit_copy(hipStream_t st, const DevCtx& c, u64* res, const u64* src
                      part_size, n_digits, digit_stride, res_stride, src_stride);
 }
 
+__global__ __launch_bounds__(kThreads) void order_check_kernel(const i64* __restrict__ order, u32 n, u32* report) {
+  const u32 i = blockIdx.x * kThreads + threadIdx.x;
+  if (i >= n) return;
+  const i64 v = order[i], first = order[i & ~4095u];
+  if (v < 0 || v >= (i64)n || first < 0 || (v >> 12) != (first >> 12)) report[0] = 1;
+  if ((i & 4095u) == 0) report[1 + (i >> 12)] = (u32)((u64)v >> 12);
+}
+void launch_order_check(hipStream_t st, const DevCtx& c, const i64* order, u32* report) {
+  hipLaunchKernelGGL(order_check_kernel, dim3((c.N + kThreads - 1) / kThreads), dim3(kThreads), 0, st, order, c.N,
+                     report);
+}
+
 // ---- Dot_prod (rns_poly.c:502-529, rns_poly_impl.c:102-162) ----------------
 // Both key halves in one pass so the digits are read once.  Products of residues are accumulated in 128 bits
 // (the reference's Fast_dotprod_poly) and reduced by one single-word Barrett step while the sum stays below

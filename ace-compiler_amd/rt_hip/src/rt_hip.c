@@ -776,8 +776,9 @@ void Rotate_batch_ciph(CIPHER res_arr, CIPHER c, const int32_t* rot_idx, uint32_
   free(where);
 }
 
+/* res may be c: the rotated polynomials are formed apart and copied over the operand afterwards, as Fast_rotate
+ * assigns its result last (evaluator.c:503-522) */
 CIPHER Rotate_ciph(CIPHER res, CIPHER c, int32_t rot_idx) {
-  FMT_ASSERT(res != c, "Rotate_ciph: in-place rotation is not supported");
   Rotate_batch_ciph(res, c, &rot_idx, 1);
   return res;
 }

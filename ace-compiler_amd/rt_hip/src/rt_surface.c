@@ -5,6 +5,7 @@
  */
 #include <complex.h>
 #include <math.h>
+#include <sys/random.h>
 
 #include "rt_internal.h"
 
@@ -102,11 +103,8 @@ void Sample_uniform_poly(POLY p) {
   FMT_ASSERT(Num_p(p) == 0 || Num_alloc(p) == Poly_level(p) + G.K, "Sample_uniform_poly: allocate the polynomial at its level");
   const char* env  = getenv("RT_HIP_SEED");
   uint64_t    seed = env ? strtoull(env, NULL, 0) : 0;
-  if (!seed) {
-    struct timespec ts;
-    clock_gettime(CLOCK_REALTIME, &ts);
-    seed = (uint64_t)ts.tv_nsec ^ ((uint64_t)ts.tv_sec << 20) ^ 0x9E3779B97F4A7C15ull;
-  }
+  if (!seed) /* from the operating system, like the keys: a caller may use the polynomial as a mask */
+    FMT_ASSERT(getrandom(&seed, sizeof(seed), 0) == (ssize_t)sizeof(seed), "Sample_uniform_poly: getrandom failed");
   ACE_OK(ace_sample_uniform(G.ctx, p->_data, Poly_level(p), Num_p(p) != 0, seed, ++Sample_stream));
 }
 void Sample_ternary_poly(POLY p, size_t hamming_weight) {

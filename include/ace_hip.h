@@ -105,6 +105,11 @@ int      ace_sync(ace_ctx* ctx);
 int      ace_fork(ace_ctx* ctx);
 int      ace_fork_switch(ace_ctx* ctx);
 int      ace_join(ace_ctx* ctx);
+/* Device memory the context holds right now, in 64-bit words and buffers (no counterpart in the reference; for
+ * tests that check that a call allocates nothing): out[0] = scratch arena of the current lane, out[1] = freed
+ * buffers kept for reuse (words), out[2] = buffers handed out by ace_alloc and not yet freed, out[3] = freed buffers
+ * kept for reuse (count). */
+void     ace_memory_stats(const ace_ctx* ctx, size_t out[4]);
 /* HIP-event stopwatch on the context's stream (for benchmarks) */
 int      ace_timer_start(ace_ctx* ctx);
 float    ace_timer_stop_ms(ace_ctx* ctx); /* synchronises; <0 on error */
@@ -124,7 +129,11 @@ int ace_intt(ace_ctx* ctx, int64_t* dst, const int64_t* src, const int32_t* prim
 
 /* One of the two kernels a transform consists of when degree > 4096 (pass 1 then
  * pass 2 equals ace_ntt / ace_intt).  For profiling each kernel on its own; the
- * intermediate buffer holds lazily reduced values. */
+ * intermediate buffer holds lazily reduced values.  Both passes of a transform must be
+ * called with the same n_limbs and n_polys: how the stages are divided between the two
+ * kernels depends on the size of the launch (n_limbs * n_polys >= 192 moves one stage
+ * of the inverse transform from pass 1 to pass 2), so passes issued with different
+ * shapes run that stage twice or not at all. */
 int ace_ntt_pass(ace_ctx* ctx, int64_t* dst, const int64_t* src, const int32_t* prime_idx,
                  size_t n_limbs, size_t n_polys, size_t poly_stride_limbs, int inverse, int pass);
 
@@ -206,14 +215,15 @@ int ace_precomp_batch(ace_ctx* ctx, int64_t* res, size_t res_stride, const int64
                       size_t count, size_t level, int is_ntt);
 int ace_mod_down_batch(ace_ctx* ctx, int64_t* res, size_t res_stride, const int64_t* src, size_t src_stride,
                        size_t count, size_t level, int is_ntt);
-/* Mod_down for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
- * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same operands and result as ace_mod_down;
+/* Mod_down for callers that cannot allocate device memory (tight serving loops, harnesses that forbid hipMalloc,
+ * code that prepares a HIP graph -- capture itself is not exercised by this library's tests).  No counterpart in the reference.  Same operands and result as ace_mod_down;
  * the intermediates live in a 16 MiB device array that is part of the library image (one copy per GPU, held until
  * the process ends), so the call performs no hipMalloc / hipFree and takes nothing from the context's arena.
  * Rejected when (level + num_p) * degree exceeds 2^21 words, and while more than 96 recorded ace_hw_* calls or a
  * paired Mod_down / Rescale are pending (their launch may allocate: ace_sync first; up to 96 recorded calls are
  * launched first, as kernel arguments).  Every call on one GPU shares that array: calls that overlap in time on one GPU (two
- * contexts, two streams) race; calls on one context are ordered by its stream.  Nothing in the array needs to
+ * contexts, two streams) race; calls on one context are ordered by its stream, and the call is rejected between
+ * ace_fork and ace_join, when the context issues on two streams.  Nothing in the array needs to
  * start at zero: each call writes every word it later reads. */
 int ace_mod_down_noalloc(ace_ctx* ctx, int64_t* res, const int64_t* src, size_t level, int is_ntt);
 /* Rescale (:310-404): src level limbs -> res level-1 limbs */
@@ -306,11 +316,19 @@ int ace_mul_relin_rescale(ace_ctx* ctx, int64_t* r0, int64_t* r1, const int64_t*
 int ace_mul_relin_rescale_batch(ace_ctx* ctx, int64_t* r0, int64_t* r1, size_t out_stride, const int64_t* a0,
                                 const int64_t* a1, const int64_t* b0, const int64_t* b1, size_t in_stride,
                                 const int64_t* swk, size_t level, size_t count);
-/* Fast_rotate (evaluator.c:503-522) with the digits of c1 hoisted (Alloc_precomp) */
+/* Fast_rotate (evaluator.c:503-522) with the digits of c1 hoisted (Alloc_precomp).
+ * order: a device table of `degree` entries, result[i] = value at order[i] (what Auto_order hands out; made by
+ * ace_automorphism_order or uploaded by the caller).  Tables of Precompute_automorphism_order's NTT form
+ * (number_theory.c:211-222) are applied inside the last kernel of the Mod_down transform; any other table
+ * (examined on the device the first time a rotation uses it, one stream synchronisation) goes through a separate
+ * pass and gives the same words more slowly.  A table must not be rewritten other than through ace_upload,
+ * ace_copy, ace_zero, ace_free or ace_automorphism_order while the context is alive.
+ * r0 and r1 must not overlap c0, the digits or each other: the result is permuted on the way out. */
 int ace_fast_rotate(ace_ctx* ctx, int64_t* r0, int64_t* r1, const int64_t* c0, const int64_t* digits,
                     const int64_t* swk, const int64_t* order, size_t level);
 /* Rotate_batch_ciph (cipher.c:459-479): one ModUp of c1, then `count` rotations.
- * r0s/r1s: count x level limbs; swks/orders: host arrays of `count` device pointers. */
+ * r0s/r1s: count x level limbs; swks/orders: host arrays of `count` device pointers (tables as for
+ * ace_fast_rotate).  The result slabs must not overlap c0 or each other (c1 is consumed before they are written). */
 int ace_rotate_batch(ace_ctx* ctx, int64_t* r0s, int64_t* r1s, const int64_t* c0, const int64_t* c1,
                      const int64_t* const* swks, const int64_t* const* orders, size_t count, size_t level);
 

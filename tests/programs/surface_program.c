@@ -281,6 +281,39 @@ int main(int argc, char** argv) {
     CHECK(Same(&v1, &v2), "Set_ciph_data");
     Free_ciph_poly(&low, 1), Free_ciph_poly(&work, 1);
   }
+  /* rotations and the conjugation written over their operand (Fast_rotate builds its result in a temporary and
+   * assigns it last, evaluator.c:503-522, so Rotate_ciph(&x, &x, k) is valid there): the words of the out-of-place
+   * call */
+  {
+    CIPHERTEXT apart, inplace, many[3];
+    memset(&apart, 0, sizeof(apart)), memset(&inplace, 0, sizeof(inplace)), memset(many, 0, sizeof(many));
+    Rotate_ciph(&apart, &ct, 3);
+    Copy_ciph(&inplace, &ct);
+    Rotate_ciph(&inplace, &inplace, 3);
+    CHECK(Same(&apart._c0_poly, &inplace._c0_poly) && Same(&apart._c1_poly, &inplace._c1_poly), "Rotate_ciph in place");
+    double* want = (double*)malloc(slots * sizeof(double));
+    for (uint32_t i = 0; i < slots; ++i) want[i] = x[(i + 3) % slots];
+    CHECK(Max_err(&inplace, want, slots) < 1e-4, "Rotate_ciph in place, message: %g", Max_err(&inplace, want, slots));
+    extern void* Rt_find_rot(int32_t rot_idx); /* the runtime's key registry; a deep chain has the key already */
+    if (!Rt_find_rot((int32_t)(2 * N - 1))) Rt_generate_rotation_key((int32_t)(2 * N - 1));
+    Conjugate_ciph(&apart, &ct);
+    Copy_ciph(&inplace, &ct);
+    Conjugate_ciph(&inplace, &inplace);
+    CHECK(Same(&apart._c0_poly, &inplace._c0_poly) && Same(&apart._c1_poly, &inplace._c1_poly), "Conjugate_ciph in place");
+    CHECK(Max_err(&inplace, x, slots) < 1e-4, "conjugate of a real message");
+    /* a batch whose first result is the operand itself */
+    int32_t idx[3] = {1, -1, 3};
+    Copy_ciph(&many[0], &ct);
+    Rotate_batch_ciph(many, &many[0], idx, 3);
+    for (int k = 0; k < 3; ++k) {
+      Rotate_ciph(&apart, &ct, idx[k]);
+      CHECK(Same(&apart._c0_poly, &many[k]._c0_poly) && Same(&apart._c1_poly, &many[k]._c1_poly),
+            "Rotate_batch_ciph over its operand, rotation %d", idx[k]);
+    }
+    free(want);
+    Free_ciph_poly(&apart, 1), Free_ciph_poly(&inplace, 1);
+    for (int k = 0; k < 3; ++k) Free_ciph_poly(&many[k], 1);
+  }
   printf("ok ciph\n");
 
   /* Raise_mod from level 1: the message survives modulo q0 (values are small against q0 / scale) */

@@ -664,6 +664,9 @@ def test_encode(pair):
                 if np.log2(scale) + 3 < q0_bits + (level - 1) * sf_bits:
                     g.encode_scaled(dr, vals, slots, level, scale, pc)
                     eq(dr, o.encode_scaled(vals, slots, level, scale, pc), "encode_scaled slots=%d level=%d p=%d" % (slots, level, pc))
+                for bad_scale in (0.75, 0.25, 2.0 ** (q0_bits + (level - 1) * sf_bits)):  # below 1, or too large for the level
+                    with pytest.raises(acefhe.AceError, match="invalid scale"):
+                        g.encode_scaled(dr, vals, slots, level, bad_scale, pc)
     # real-valued messages (doubles, floats) are widened on the device: same residues as the complex form, with
     # calls recorded and issued one by one
     for side in (True, False):
@@ -896,6 +899,37 @@ def test_rotation(pair):
     g.fast_rotate(r0, r1, dc0, dd, dswk[0], dord[0], level)
     eq(r0, got0[:n], "fast_rotate == batch[0]")
     eq(r1, got1[:n], "fast_rotate == batch[0] c1")
+    # index tables the caller uploads itself: one of the automorphism's make (on large rings applied inside the
+    # transform's last kernel, once the library has examined it), and a permutation that is no automorphism and
+    # scatters every block of the result over the whole source (the separate pass): result[i] = value at table[i]
+    k = len(rots) - 1
+    mine = g.upload(np.asarray(orders[k], dtype=np.int64))
+    g.fast_rotate(r0, r1, dc0, dd, dswk[k], mine, level)
+    eq(r0, got0[k * n:(k + 1) * n], "caller's copy of an automorphism table")
+    eq(r1, got1[k * n:(k + 1) * n], "caller's copy of an automorphism table, c1")
+    scatter = (np.arange(N, dtype=np.int64) * 5 + 3) % N
+    w0, w1 = o.fast_rotate(c0, digits, swks[0], scatter, level)
+    other = g.upload(scatter)
+    for _ in range(2):  # the second call finds the verdict on the table cached
+        g.fast_rotate(r0, r1, dc0, dd, dswk[0], other, level)
+        eq(r0, w0, "a table that is no automorphism")
+        eq(r1, w1, "a table that is no automorphism, c1")
+    # the same buffer rewritten through the library: the verdict on the old contents must not survive
+    other.set(np.asarray(orders[0], dtype=np.int64))
+    g.fast_rotate(r0, r1, dc0, dd, dswk[0], other, level)
+    eq(r0, got0[:n], "table buffer rewritten")
+    mine.set(scatter)
+    g.fast_rotate(r0, r1, dc0, dd, dswk[0], mine, level)
+    eq(r0, w0, "table buffer rewritten with a table that is no automorphism")
+    # results that overlap c0 or the digits would be read after they are written
+    with pytest.raises(acefhe.AceError, match="overlap"):
+        g.fast_rotate(dc0.view(0, n), r1, dc0, dd, dswk[0], dord[0], level)
+    with pytest.raises(acefhe.AceError, match="overlap"):
+        g.fast_rotate(r0, dd.view(N, n), dc0, dd, dswk[0], dord[0], level)
+    if len(rots) > 1:
+        inside = g.alloc(len(rots) * n)
+        with pytest.raises(acefhe.AceError, match="overlap"):
+            g.rotate_batch(inside, r1s, inside.view(n, n), dc1, dswk, dord, level)
 
 
 def test_rejected_calls(pair):

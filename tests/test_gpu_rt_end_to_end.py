@@ -38,8 +38,6 @@ def test_gemm_square_program(degree, dim):
     assert "max_err" in r.stdout
 
 
-# eg_fhertlib_mul_const_rtv builds and links too, but cannot pass anywhere: it multiplies the message 20 at scale 2^30
-# by a plaintext at scale 2^30 under a 63-bit modulus (20 * 2^60 > Q) and validates the wrapped value.
 @pytest.mark.parametrize("name", EXAMPLES)
 def test_reference_example(name):
     exe = os.path.join(EXAMPLES_DIR, "eg_fhertlib_" + name)
@@ -47,6 +45,19 @@ def test_reference_example(name):
         pytest.skip("built only where the reference tree is present")
     r = run([exe], 77)
     assert r.returncode == 0 and "SUCESS" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
+
+
+def test_reference_example_that_expects_its_validation_to_fail():
+    """eg_fhertlib_mul_const_rtv.c:62-68 is the reference's negative test of the run-time validation: the generated
+    code calls Validate() on a value that cannot match (20 * 2^60 wraps under its 63-bit modulus), the harness
+    compares the output with data that must not match either, prints EXPECTED FAILED! and returns 0."""
+    exe = os.path.join(EXAMPLES_DIR, "eg_fhertlib_mul_const_rtv")
+    if not os.path.exists(exe):
+        pytest.skip("built only where the reference tree is present")
+    r = run([exe], 77)
+    assert r.returncode == 0 and "EXPECTED FAILED!" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
+    assert "NOT EXPECTED" not in r.stdout
+    assert "ERROR: validation failed" in r.stderr, r.stderr[-2000:]
 
 
 def test_reference_generated_sine_program():

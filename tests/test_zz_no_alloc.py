@@ -17,7 +17,9 @@ def both(g, e, level, is_ntt):
     want, got = g.alloc(level * N), g.alloc(level * N)
     g.mod_down(want, de, level, is_ntt)
     w = want.get()
+    before = g.memory_stats()
     g.mod_down_noalloc(got, de, level, is_ntt)
+    assert g.memory_stats() == before, "the call changed the context's arena, pool or live buffers"
     r = got.get()
     assert (de.get() == e).all(), "operand changed"
     for b in (de, want, got):
@@ -71,6 +73,13 @@ def test_mod_down_noalloc_equals_mod_down(cfg):
         g.mod_down_noalloc(dr, de, L, True)
         assert (dr.get() == want.get()).all()
         assert int(a.get()[0]) == 100
+        # between ace_fork and ace_join the context issues on two streams, which would share the one array: refused
+        g.fork()
+        with pytest.raises(acefhe.AceError, match="ace_fork"):
+            g.mod_down_noalloc(dr, de, L, True)
+        g.join()
+        g.mod_down_noalloc(dr, de, L, True)
+        assert (dr.get() == want.get()).all()
     finally:
         g.close()
 
