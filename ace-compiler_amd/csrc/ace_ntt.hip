@@ -411,9 +411,10 @@ __global__ __launch_bounds__(256, 4) void ntt_fwd_strided(DevCtx c, PolySeq dsts
 // batch at N=2^16, 24 primes: 12 MiB of twiddle fetches with this map, 230 MiB
 // with groups varying fastest, where 4.6 MB of streaming data passes through the
 // L2 between two uses of the same twiddles.)
+template <int LOGC = kLogChunk>
 __device__ __forceinline__ bool chunk_block(const DevCtx& c, u32 n_limbs, u32 slots_per_group, u32& chunk,
                                             u32& limb, u32& slot_in_group) {
-  const u32 n_chunks = c.N >> kLogChunk, n_groups = n_limbs * n_chunks;
+  const u32 n_chunks = c.N >> LOGC, n_groups = n_limbs * n_chunks;
   const u32 id = blockIdx.x, xcd = id & 7, slot = id >> 3;
   const u32 grp = (slot / slots_per_group) * 8 + xcd;
   slot_in_group = slot % slots_per_group;
@@ -424,8 +425,8 @@ __device__ __forceinline__ bool chunk_block(const DevCtx& c, u32 n_limbs, u32 sl
   limb = n_limbs - 1 - grp / n_chunks;
   return true;
 }
-static inline unsigned chunk_grid(const DevCtx& c, u32 n_limbs, u32 slots_per_group) {
-  u32 n_groups = n_limbs * (c.N >> kLogChunk);
+static inline unsigned chunk_grid(const DevCtx& c, u32 n_limbs, u32 slots_per_group, int logc = kLogChunk) {
+  u32 n_groups = n_limbs * (c.N >> logc);
   return ((n_groups + 7) / 8) * 8 * slots_per_group;
 }
 
@@ -753,6 +754,96 @@ __global__ __launch_bounds__(kChunkThreads, kChunkWaves) void ntt_inv_chunk(DevC
   else inv_chunk_body<ArithInt, SKIP, COPY>(lds, c, dsts, srcs, copies, pos, n_polys, chunk, limb, pblk, pi);
 }
 
+// The inverse chunk pass of a transform whose strided pass takes the span of 2048 (SKIP): its eleven stages never
+// pair words of different halves of a 4096-word chunk, so a half is a work-group's whole job: 2048 words, 256
+// threads, and the one work-group barrier is among four waves, one on each SIMD, instead of eight.  Rounds as in
+// inv_chunk_body; the last has two stages (spans 512 and 1024) on the words t + 256 r of a thread, register r holding
+// the word at t + 256 (r >> 2 & 1) + 512 (r & 1) + 1024 (r >> 1 & 1) so that the two stages pair neighbouring registers
+// and registers two apart.
+constexpr int kLogHalf = 11, kHalf = 1 << kLogHalf, kHalfThreads = 256;
+template <class A>
+__device__ __forceinline__ void inv_half_body(u64* lds_words, const DevCtx& c, const PolySeq& dsts,
+                                              const PolySeq& srcs, const LimbMap& pos, u32 half, u32 limb, u32 poly,
+                                              u32 pi) {
+  typedef typename A::T T;
+  T* lds = reinterpret_cast<T*>(lds_words);
+  const int t = threadIdx.x;
+  const u64 off = (u64)pos.prime[limb] * c.N + (u64)half * kHalf;
+  A ar;
+  ar.init(c, pi, true, nullptr, 0);
+  const ChunkMap cm(t);
+  const u32 mh = c.N >> 1;  // groups at span 1
+  u64 raw[8];
+  {
+    const ulonglong2* src2 = reinterpret_cast<const ulonglong2*>(srcs.at(poly) + off + 8 * t);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const ulonglong2 x = src2[k];
+      raw[2 * k] = x.x;
+      raw[2 * k + 1] = x.y;
+    }
+  }
+  u64* dst = dsts.at(poly);
+  T v[8];
+#pragma unroll
+  for (int r = 0; r < 8; ++r) v[r] = ar.in_canon(raw[r]);
+  // spans 1, 2, 4
+  gs_stage<A, 8, 0>(ar, v, (mh >> 0) + (half << 10) + ((u32)t << 2));
+  gs_stage<A, 8, 1>(ar, v, (mh >> 1) + (half << 9) + ((u32)t << 1));
+  ar.recentre_sum_of_four(v[0]);
+  ar.recentre_sum_of_four(v[4]);
+  gs_stage<A, 8, 2>(ar, v, (mh >> 2) + (half << 8) + ((u32)t << 0));
+#pragma unroll
+  for (int r = 0; r < 8; ++r) lds[cm.narrow + ChunkMap::narrow_off(r)] = v[r];
+  wave_sync();  // the words read next were written by this wave
+  // spans 8, 16, 32
+#pragma unroll
+  for (int r = 0; r < 8; ++r) v[r] = lds[cm.octet + ChunkMap::octet_off(r)];
+  reduce_all<A, 8>(ar, v);
+  gs_stage<A, 8, 0>(ar, v, (mh >> 3) + (half << 7) + (cm.h << 2));
+  gs_stage<A, 8, 1>(ar, v, (mh >> 4) + (half << 6) + (cm.h << 1));
+  gs_stage<A, 8, 2>(ar, v, (mh >> 5) + (half << 5) + (cm.h << 0));
+#pragma unroll
+  for (int r = 0; r < 8; ++r) lds[cm.octet + ChunkMap::octet_off(r)] = v[r];
+  wave_sync();  // the words read next were written by this wave
+  // spans 64, 128, 256
+#pragma unroll
+  for (int r = 0; r < 8; ++r) v[r] = lds[cm.wave + ChunkMap::wave_off(r)];
+  reduce_all<A, 8>(ar, v);
+  gs_stage<A, 8, 0>(ar, v, (mh >> 6) + (half << 4) + (cm.wv << 2));
+  gs_stage<A, 8, 1>(ar, v, (mh >> 7) + (half << 3) + (cm.wv << 1));
+  gs_stage<A, 8, 2>(ar, v, (mh >> 8) + (half << 2) + (cm.wv << 0));
+#pragma unroll
+  for (int r = 0; r < 8; ++r) lds[cm.wave + ChunkMap::wave_off(r)] = v[r];
+  __syncthreads();
+  // spans 512 and 1024; twiddles are uniform over the work-group
+  constexpr auto word = [](int r) constexpr { return 256 * ((r >> 2) & 1) + 512 * (r & 1) + 1024 * ((r >> 1) & 1); };
+#pragma unroll
+  for (int r = 0; r < 8; ++r) v[r] = lds[cm.wide + word(r) + word(r) / 16];
+  reduce_all<A, 8>(ar, v);
+  {
+    typename A::TWL two[2], tw[4];
+    ar.template load_tw<2>((mh >> 9) + (half << 1), two);
+    tw[0] = tw[2] = two[0];
+    tw[1] = tw[3] = two[1];
+    gs_stage_pre<A, 8, 0>(ar, v, tw);
+    ar.template load_tw<1>((mh >> 10) + half, two);
+    two[1] = two[0];
+    gs_stage_pre<A, 8, 1>(ar, v, two);
+  }
+#pragma unroll
+  for (int r = 0; r < 8; ++r) stg<512>(dst + off + t + word(r), ar.out_mid(v[r]));
+}
+__global__ __launch_bounds__(kHalfThreads, kChunkWaves) void ntt_inv_half(DevCtx c, PolySeq dsts, PolySeq srcs, LimbMap lm,
+                                                                       LimbMap pos, u32 n_limbs, u32 n_polys) {
+  __shared__ u64 lds[kHalf + kHalf / 16];
+  u32 half, limb, poly;
+  if (!chunk_block<kLogHalf>(c, n_limbs, n_polys, half, limb, poly)) return;
+  const u32 pi = lm.prime[limb];
+  if (c.fp_ok[pi]) inv_half_body<ArithFp>(lds, c, dsts, srcs, pos, half, limb, poly, pi);
+  else inv_half_body<ArithInt>(lds, c, dsts, srcs, pos, half, limb, poly, pi);
+}
+
 // inverse, strided pass: spans 4096..N/2, then scale every word by the limb's
 // constant (default 1/N) and store canonical residues.  In place.
 // scale: nullptr, or (constant, Shoup companion) pairs indexed by the limb's place in the launch.
@@ -966,9 +1057,16 @@ static void run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst, const
     constexpr int LS = LOGR + SI, SHIFT = SI;
     dim3 gs((c.N >> LS) / 256, n_limbs, n_polys);
     if (passes & 1) {
+      static const bool halves = [] {
+        const char* e = getenv("ACE_NTT_INV_HALF");
+        return !e || e[0] != '0';
+      }();
       if (copies.seq.b[0])
         hipLaunchKernelGGL((ntt_inv_chunk<SHIFT, 1>), gc, dim3(kChunkThreads), 0, st, c, dst, src, copies, lm, pos,
                            n_limbs, n_polys);
+      else if (SHIFT == 1 && halves)
+        hipLaunchKernelGGL(ntt_inv_half, dim3(chunk_grid(c, n_limbs, n_polys, kLogHalf)), dim3(kHalfThreads), 0, st, c,
+                           dst, src, lm, pos, n_limbs, n_polys);
       else
         hipLaunchKernelGGL((ntt_inv_chunk<SHIFT, 0>), gc, dim3(kChunkThreads), 0, st, c, dst, src, copies, lm, pos,
                            n_limbs, n_polys);
