@@ -56,6 +56,8 @@ def _sig(lib):
     f("ace_zero", C.c_int, _vp, _vp, _sz)
     f("ace_sync", C.c_int, _vp)
     f("ace_memory_stats", None, _vp, C.POINTER(C.c_size_t))
+    f("ace_ctx_share", _vp, _vp)
+    f("ace_fork_release", C.c_int, _vp)
     f("ace_timer_start", C.c_int, _vp)
     f("ace_timer_stop_ms", C.c_float, _vp)
     f("ace_ntt", C.c_int, _vp, _vp, _vp, _i32p, _sz, _sz, _sz)
@@ -118,7 +120,7 @@ EXPORTS = [
     "ace_degree", "ace_num_q", "ace_num_p", "ace_num_parts", "ace_part_size", "ace_num_decomp", "ace_prime",
     "ace_root", "ace_modulus", "ace_host_twiddles", "ace_host_tbl_modup", "ace_host_tbl_moddown",
     "ace_host_tbl_rescale", "ace_host_automorphism_order", "ace_alloc", "ace_free", "ace_upload", "ace_download",
-    "ace_copy", "ace_zero", "ace_sync", "ace_memory_stats", "ace_timer_start", "ace_timer_stop_ms", "ace_ntt", "ace_intt", "ace_ntt_pass",
+    "ace_copy", "ace_zero", "ace_sync", "ace_memory_stats", "ace_ctx_share", "ace_fork_release", "ace_timer_start", "ace_timer_stop_ms", "ace_ntt", "ace_intt", "ace_ntt_pass",
     "ace_hw_modadd", "ace_hw_modsub", "ace_hw_modmul", "ace_hw_modmuladd", "ace_hw_modadd_scalar",
     "ace_hw_modsub_scalar", "ace_hw_modmul_scalar", "ace_hw_modmuladd_scalar", "ace_hw_rotate",
     "ace_find_automorphism_index", "ace_automorphism_order", "ace_poly_add", "ace_poly_sub", "ace_poly_mul",
@@ -175,9 +177,11 @@ class DevBuf:
 class Context:
     """One CRT context (primes, tables in HBM, one HIP stream)."""
 
-    def __init__(self, degree, num_q, q0_bits=0, sf_bits=0, parts=1, primes=None):
+    def __init__(self, degree, num_q, q0_bits=0, sf_bits=0, parts=1, primes=None, share=None):
         self.lib = lib()
-        if primes is None:
+        if share is not None:  # a further context over `share`'s tables, for another host thread
+            h = self.lib.ace_ctx_share(share.h)
+        elif primes is None:
             h = self.lib.ace_ctx_create(degree, num_q, q0_bits, sf_bits, parts)
         else:
             p = np.ascontiguousarray(primes, dtype=np.int64)
@@ -193,6 +197,10 @@ class Context:
         self.primes = [self.lib.ace_prime(self.h, i) for i in range(self.L + self.K)]
         self.roots = [self.lib.ace_root(self.h, i) for i in range(self.L + self.K)]
         self.has_device = bool(self.lib.ace_has_device(self.h))
+
+    def share(self):
+        """A context over the same tables with its own stream, arena and pool (close it before this one)."""
+        return Context(0, 0, share=self)
 
     def err(self):
         return (self.lib.ace_last_error() or b"").decode()
@@ -275,6 +283,9 @@ class Context:
 
     def join(self):
         self._chk(self.lib.ace_join(self.h))
+
+    def fork_release(self):
+        self._chk(self.lib.ace_fork_release(self.h))
 
     def sync(self):
         self._chk(self.lib.ace_sync(self.h))

@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
@@ -13,6 +14,7 @@
 #include <set>
 #include <unordered_set>
 #include <memory>
+#include <mutex>
 #include <stdexcept>
 #include <string>
 #include <unordered_map>
@@ -109,8 +111,30 @@ struct PendingRun {
   std::unordered_set<uintptr_t> rot_res, rot_src;  // results / sources (and index tables) of rotates
 };
 
-struct ace_ctx {
+// What the contexts of one family share (a context made by ace_ctx_create and those made from it by ace_ctx_share):
+// the host tables, and the record of the buffers ace_alloc has handed out, so that a buffer may be freed through
+// another context of the family than the one that made it.
+struct Family {
   HostContext h;
+  std::mutex mu;  // guards `live` and `order_fits`
+  std::unordered_map<void*, size_t> live;
+  std::atomic<size_t> pooled_words{0};  // freed buffers kept for reuse by all contexts of the family together
+  size_t pool_limit_words = (size_t)4 << 30;  // at most this much of it: a third of the GPU's memory, or ACE_POOL_LIMIT_GB (set by the root)
+  // Index tables of rotations seen so far -> whether the forward chunk pass may apply them on the way out (every
+  // 4096-word block of the table draws on one block of the source, and the blocks' sources are a permutation:
+  // true of Precompute_automorphism_order's NTT-form tables, number_theory.c:211-222).  Tables made by
+  // ace_automorphism_order are entered as they are made, a caller's own table is examined on the device when a
+  // rotation first uses it; writing to a table through this library (upload, copy, zero, free) forgets the verdict.
+  std::unordered_map<const void*, bool> order_fits;
+};
+
+struct ace_ctx {
+  std::shared_ptr<Family> family;
+  HostContext& h;
+  std::unordered_map<void*, size_t>& live;  // sizes of the buffers handed out (guarded by family->mu)
+  ace_ctx* parent = nullptr;  // the context whose device tables this one uses (null: its own)
+  ace_ctx() : family(std::make_shared<Family>()), h(family->h), live(family->live) {}
+  explicit ace_ctx(ace_ctx* from) : family(from->family), h(family->h), live(family->live), parent(from) {}
   bool device_ok = false;  // false: host tables only (no GPU present), every compute call is rejected
   hipStream_t stream = nullptr;
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
@@ -224,25 +248,28 @@ struct ace_ctx {
           "scale_mod_size or decrease scale of msg");
     }
   }
-  // Index tables of rotations seen so far -> whether the forward chunk pass may apply them on the way out (every
-  // 4096-word block of the table draws on one block of the source, and the blocks' sources are a permutation:
-  // true of Precompute_automorphism_order's NTT-form tables, number_theory.c:211-222).  Tables made by
-  // ace_automorphism_order are entered as they are made, a caller's own table is examined on the device when a
-  // rotation first uses it; writing to a table through this library (upload, copy, zero, free) forgets the verdict.
-  std::unordered_map<const void*, bool> order_fits;
-  u32* order_report = nullptr;  // [1 + N / 4096] on the device
+  u32* order_report = nullptr;  // [1 + N / 4096] on the device: what order_check_kernel found (see Family::order_fits)
   void forget_orders(const void* dst, size_t words) {
-    if (order_fits.empty()) return;
+    std::lock_guard<std::mutex> lock(family->mu);
+    auto& fits = family->order_fits;
+    if (fits.empty()) return;
     const uintptr_t lo = (uintptr_t)dst, hi = lo + words * sizeof(u64);
-    for (auto it = order_fits.begin(); it != order_fits.end();) {
+    for (auto it = fits.begin(); it != fits.end();) {
       const uintptr_t a = (uintptr_t)it->first, b = a + (size_t)h.N * sizeof(i64);
-      if (a < hi && lo < b) it = order_fits.erase(it);
+      if (a < hi && lo < b) it = fits.erase(it);
       else ++it;
     }
   }
+  void note_order(const void* order, bool ok) {
+    std::lock_guard<std::mutex> lock(family->mu);
+    family->order_fits[order] = ok;
+  }
   bool order_fits_chunks(const i64* order) {
-    auto it = order_fits.find(order);
-    if (it != order_fits.end()) return it->second;
+    {
+      std::lock_guard<std::mutex> lock(family->mu);
+      auto it = family->order_fits.find(order);
+      if (it != family->order_fits.end()) return it->second;
+    }
     bool ok = false;
     if (d.logN > 12) {
       const u32 nb = h.N >> 12;
@@ -258,19 +285,18 @@ struct ace_ctx {
         else seen[rep[1 + b]] = 1;
       }
     }
-    order_fits[order] = ok;
+    note_order(order, ok);
     return ok;
   }
   LimbMap q_lm{}, p_lm{};     // identity maps: limb t -> prime t / prime L+t
   // ace_alloc / ace_free: sizes of the buffers handed out, and freed buffers kept for reuse
-  static constexpr size_t kPoolLimitWords = (size_t)4 << 30;  // 32 GiB
-  std::unordered_map<void*, size_t> live;
   std::multimap<size_t, void*> pool;
   size_t pooled_words = 0;
   void drop_pool() {
     if (stream) (void)hipStreamSynchronize(stream);
     for (auto& kv : pool) (void)hipFree(kv.second);
     pool.clear();
+    family->pooled_words -= pooled_words;
     pooled_words = 0;
   }
   // scratch arena
@@ -551,8 +577,45 @@ struct ace_ctx {
     return moddown_rescale.emplace(level, m).first->second;
   }
 
+  // A context that shares `from`'s device tables (twiddles, per-prime constants, P -> Q conversion, encoder tables)
+  // and has its own stream, scratch arena, buffer pool, recorded run and lazily built per-level tables.
+  void init_shared(const ace_ctx& from) {
+    static_scratch = static_scratch_of_current_device();
+    HIP_OK(hipStreamCreateWithFlags(&stream, hipStreamNonBlocking));
+    HIP_OK(hipEventCreate(&ev0));
+    HIP_OK(hipEventCreate(&ev1));
+    d = from.d;
+    conv_fp = from.conv_fp;
+    conv_matrix = from.conv_matrix;
+    share_transform = from.share_transform;
+    q_lm = from.q_lm;
+    p_lm = from.p_lm;
+    phat = from.phat;
+    p2q_job = from.p2q_job;
+    pscale_ntt = from.pscale_ntt;
+    pscale_coef = from.pscale_coef;
+    pinv = from.pinv;
+    pmodq = from.pmodq;
+    fft_rou = from.fft_rou;
+    rot_group = from.rot_group;
+    q0_bits = from.q0_bits;
+    sf_bits = from.sf_bits;
+    batching = from.batching;
+    std::vector<int> z(1, 0);
+    d_err = upload_vec(z);
+    std::vector<u32> rep(1 + (h.N >> 12) + 1, 0);
+    order_report = upload_vec(rep);
+  }
+
   void init_device() {
     static_scratch = static_scratch_of_current_device();
+    {
+      // A ResNet-20 image leaves about 10 GiB of freed polynomials behind for the next one, per thread that runs
+      // images; beyond the limit a freed buffer goes back to the driver, which waits for the stream each time.
+      size_t free_b = 0, total_b = 0;
+      if (hipMemGetInfo(&free_b, &total_b) == hipSuccess && total_b) family->pool_limit_words = total_b / 3 / sizeof(u64);
+      if (const char* gb = std::getenv("ACE_POOL_LIMIT_GB")) family->pool_limit_words = (size_t)(atof(gb) * (double)(1 << 27));
+    }
     HIP_OK(hipStreamCreateWithFlags(&stream, hipStreamNonBlocking));
     HIP_OK(hipEventCreate(&ev0));
     HIP_OK(hipEventCreate(&ev1));
@@ -654,6 +717,10 @@ struct ace_ctx {
       flush_pending();
     } catch (...) {
     }
+    if (std::getenv("ACE_HIP_PROFILE"))
+      std::fprintf(stderr, "[ace_hip] context %p: arena %.2f GiB, %zu freed buffers kept (%.2f GiB), second lane %.2f GiB\n",
+                   (void*)this, (double)ws_words / (double)(1 << 27), pool.size(), (double)pooled_words / (double)(1 << 27),
+                   (double)(idle.ws_words + idle.pooled_words) / (double)(1 << 27));
     if (stream) (void)hipStreamSynchronize(stream);
     for (Stage& st : stages) {
       if (st.host) (void)hipHostFree(st.host);
@@ -664,6 +731,7 @@ struct ace_ctx {
     for (void* p : owned) (void)hipFree(p);
     drop_pool();
     for (auto& kv : idle.pool) (void)hipFree(kv.second);
+    family->pooled_words -= idle.pooled_words;
     if (idle.ws) (void)hipFree(idle.ws);
     if (idle.stream) (void)hipStreamDestroy(idle.stream);
     if (fork_ev) (void)hipEventDestroy(fork_ev);
@@ -1370,6 +1438,8 @@ struct ScopedProf {
     if (!g_prof.on) return;
     timespec t1;
     clock_gettime(CLOCK_MONOTONIC, &t1);
+    static std::mutex mu;  // contexts of a family run on several threads
+    std::lock_guard<std::mutex> lock(mu);
     auto& e = g_prof.t[name];
     e.first += 1;
     e.second += (double)(t1.tv_sec - t0.tv_sec) + 1e-9 * (double)(t1.tv_nsec - t0.tv_nsec);
@@ -1438,6 +1508,21 @@ ace_ctx* ace_ctx_create_with_primes(uint32_t degree, size_t num_q, const int64_t
   return make_ctx(degree, std::vector<i64>(q_primes, q_primes + num_q), num_parts);
 }
 
+ace_ctx* ace_ctx_share(ace_ctx* from) {
+  try {
+    if (!from) throw std::runtime_error("ace_ctx_share: null context");
+    if (!from->device_ok) throw std::runtime_error("ace_ctx_share: the context holds host tables only (no HIP device)");
+    ace_ctx* root = from->parent ? from->parent : from;
+    std::unique_ptr<ace_ctx> c(new ace_ctx(root));
+    c->init_shared(*root);
+    c->device_ok = true;
+    return c.release();
+  } catch (const std::exception& e) {
+    g_err = e.what();
+    return nullptr;
+  }
+}
+
 void ace_ctx_destroy(ace_ctx* ctx) { delete ctx; }
 
 uint32_t ace_degree(const ace_ctx* c) { return c->h.N; }
@@ -1473,6 +1558,7 @@ static int64_t* alloc_words(ace_ctx* c, size_t n_words, bool zero) {
       p = static_cast<u64*>(it->second);
       c->pool.erase(it);
       c->pooled_words -= words;
+      c->family->pooled_words -= words;
     } else {
       hipError_t e = hipMalloc((void**)&p, words * sizeof(u64));
       if (e != hipSuccess && c->pooled_words) {  // give the cached buffers back and try once more
@@ -1482,7 +1568,10 @@ static int64_t* alloc_words(ace_ctx* c, size_t n_words, bool zero) {
       }
       HIP_OK(e);
     }
-    c->live[p] = words;
+    {
+      std::lock_guard<std::mutex> lock(c->family->mu);
+      c->live[p] = words;
+    }
     if (zero) {
       const size_t N = c->h.N;
       if (c->batching && n_words % N == 0 && n_words / N <= 64) {  // as entries of one limb each, next to the calls that follow
@@ -1500,19 +1589,27 @@ static int64_t* alloc_words(ace_ctx* c, size_t n_words, bool zero) {
 void ace_free(ace_ctx* c, int64_t* p) {
   ScopedProf prof_scope_("ace_free");
   if (!p || !c || !c->device_ok) return;
-  auto it = c->live.find(p);
-  if (it == c->live.end()) return;  // not from ace_alloc of this context (a view, or freed twice)
-  const size_t words = it->second;
+  size_t words = 0;
+  {
+    std::lock_guard<std::mutex> lock(c->family->mu);
+    auto it = c->live.find(p);
+    if (it == c->live.end()) return;  // not from ace_alloc of this family (a view, or freed twice)
+    words = it->second;
+  }
   c->forget_orders(p, words);
   try {  // recorded calls may still name this buffer; a zero fill of it that nothing has looked at is moot
     c->flush_pending_declared({ace_ctx::span(p, words)}, {});
   } catch (const std::exception& e) {
     (void)fail(e.what());
   }
-  c->live.erase(it);
-  if (c->pooled_words + words <= ace_ctx::kPoolLimitWords) {
+  {
+    std::lock_guard<std::mutex> lock(c->family->mu);
+    c->live.erase(p);
+  }
+  if (c->family->pooled_words.load() + words <= c->family->pool_limit_words) {
     c->pool.emplace(words, p);
     c->pooled_words += words;
+    c->family->pooled_words += words;
     return;
   }
   (void)hipStreamSynchronize(c->stream);
@@ -1606,10 +1703,35 @@ int ace_join(ace_ctx* c) {
   ACE_CATCH_INT
 }
 
+int ace_fork_release(ace_ctx* c) {
+  ACE_TRY
+  if (c->fork_state) return fail("ace_fork_release: the context is forked");
+  if (c->idle.stream) {
+    HIP_OK(hipStreamSynchronize(c->idle.stream));
+    for (auto& kv : c->idle.pool) (void)hipFree(kv.second);
+    c->idle.pool.clear();
+    c->family->pooled_words -= c->idle.pooled_words;
+    c->idle.pooled_words = 0;
+    if (c->idle.ws) (void)hipFree(c->idle.ws);
+    c->idle.ws = nullptr;
+    c->idle.ws_words = c->idle.ws_used = 0;
+    HIP_OK(hipStreamDestroy(c->idle.stream));
+    c->idle.stream = nullptr;
+    HIP_OK(hipEventDestroy(c->fork_ev));
+    HIP_OK(hipEventDestroy(c->join_ev));
+    c->fork_ev = c->join_ev = nullptr;
+    // (the second lane's image of recorded runs, if any, stays with the context's other allocations)
+  }
+  ACE_CATCH_INT
+}
+
 void ace_memory_stats(const ace_ctx* c, size_t out[4]) {
   out[0] = c->ws_words;
   out[1] = c->pooled_words;
-  out[2] = c->live.size();
+  {
+    std::lock_guard<std::mutex> lock(c->family->mu);
+    out[2] = c->live.size();
+  }
   out[3] = c->pool.size();
 }
 int ace_timer_start(ace_ctx* c) {
@@ -1788,7 +1910,7 @@ int ace_automorphism_order(ace_ctx* c, int64_t* dev_order, uint32_t k, int is_nt
   c->h2d(dev_order, ord.data(), ord.size() * sizeof(i64));
   HIP_OK(hipStreamSynchronize(c->stream));
   c->forget_orders(dev_order, c->h.N);
-  if (is_ntt) c->order_fits[dev_order] = true;
+  if (is_ntt) c->note_order(dev_order, true);
   ACE_CATCH_INT
 }
 

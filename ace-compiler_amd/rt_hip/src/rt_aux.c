@@ -238,8 +238,8 @@ bool Is_trace_on(void) { return Trace_on; }
  * and the harness entry points work on the same store ------------------------------------------------------- */
 void Io_init(void) {}
 void Io_fini(void) {
-  IO_SLOT** tab[2] = {&G.in, &G.out};
-  size_t*   cnt[2] = {&G.n_in, &G.n_out};
+  IO_SLOT** tab[2] = {&LANE.in, &LANE.out};
+  size_t*   cnt[2] = {&LANE.n_in, &LANE.n_out};
   for (int k = 0; k < 2; ++k) {
     for (size_t i = 0; i < *cnt[k]; ++i) free((*tab[k])[i].name);
     free(*tab[k]);
@@ -253,17 +253,17 @@ static void* slot_get(IO_SLOT* s, size_t n, const char* name, size_t idx) {
   return f->ct;
 }
 void Io_set_input(const char* name, size_t idx, void* ct) {
-  IO_SLOT* s = Rt_find_slot(G.in, G.n_in, name, idx);
-  if (!s) s = Rt_add_slot(&G.in, &G.n_in, name, idx);
+  IO_SLOT* s = Rt_find_slot(LANE.in, LANE.n_in, name, idx);
+  if (!s) s = Rt_add_slot(&LANE.in, &LANE.n_in, name, idx);
   s->ct = (CIPHERTEXT*)ct;
 }
-void* Io_get_input(const char* name, size_t idx) { return slot_get(G.in, G.n_in, name, idx); }
+void* Io_get_input(const char* name, size_t idx) { return slot_get(LANE.in, LANE.n_in, name, idx); }
 void  Io_set_output(const char* name, size_t idx, void* ct) {
-  IO_SLOT* s = Rt_find_slot(G.out, G.n_out, name, idx);
-  if (!s) s = Rt_add_slot(&G.out, &G.n_out, name, idx);
+  IO_SLOT* s = Rt_find_slot(LANE.out, LANE.n_out, name, idx);
+  if (!s) s = Rt_add_slot(&LANE.out, &LANE.n_out, name, idx);
   s->ct = (CIPHERTEXT*)ct;
 }
-void* Io_get_output(const char* name, size_t idx) { return slot_get(G.out, G.n_out, name, idx); }
+void* Io_get_output(const char* name, size_t idx) { return slot_get(LANE.out, LANE.n_out, name, idx); }
 
 /* ---- time per event (rtlib_timing.c:18-126) -------------------------------------------------------------------
  * Events are numbered as the compiler numbers them: its core, NN and FHE lists (air/base/rt_timing.h:20,
@@ -280,8 +280,10 @@ static const struct {
 #undef X
 };
 #define RTM_COUNT (sizeof(Rtm_events) / sizeof(Rtm_events[0]))
-static uint64_t       Rtm_nsec[RTM_COUNT], Rtm_sub_nsec[RTM_COUNT], Rtm_calls[RTM_COUNT];
-struct RTM_INFO_STACK Rtm_stack = {{{0, 0, 0, 0, 0}}, 0, RTLIB_TIMING_MAX_LEVEL};
+/* per thread, as in the reference's OpenMP build (include/common/rtlib_timing.h:123-126): the table that
+ * Report_rtlib_timing prints is the calling thread's */
+static __thread uint64_t       Rtm_nsec[RTM_COUNT], Rtm_sub_nsec[RTM_COUNT], Rtm_calls[RTM_COUNT];
+__thread struct RTM_INFO_STACK Rtm_stack = {{{0, 0, 0, 0, 0}}, 0, RTLIB_TIMING_MAX_LEVEL};
 static int            Rtm_enabled = -1;
 
 static bool rtm_on(void) {
@@ -305,7 +307,7 @@ void Append_rtlib_timing(uint32_t event, uint32_t id, uint64_t nsec, uint64_t su
 void Mark_rtm_start(uint32_t event, uint32_t id) {
   if (!rtm_on()) return;
   IS_TRUE(Rtm_stack._size < Rtm_stack._max_size, "FATAL: RTM stack overflow");
-  if (G.ctx) (void)ace_sync(G.ctx);
+  if (G.root) (void)ace_sync(RT_CTX);
   struct RTM_INFO* info = &Rtm_stack._info[Rtm_stack._size++];
   struct timespec  ts;
   clock_gettime(CLOCK_REALTIME, &ts);
@@ -313,7 +315,7 @@ void Mark_rtm_start(uint32_t event, uint32_t id) {
 }
 void Mark_rtm_end(uint32_t event, uint64_t id) {
   if (!rtm_on()) return;
-  if (G.ctx) (void)ace_sync(G.ctx);
+  if (G.root) (void)ace_sync(RT_CTX);
   struct timespec ts;
   clock_gettime(CLOCK_REALTIME, &ts);
   IS_TRUE(Rtm_stack._size > 0, "FATAL: RTM stack underflow");

@@ -48,9 +48,18 @@ static void fill_sin_poly(SIN_POLY* p, size_t hamming_weight, bool even) {
   }
 }
 static const SIN_POLY* sin_poly(void) {
-  if (Sin_poly.n_coeff) return &Sin_poly;
-  const char* env = getenv("RTLIB_BTS_EVEN_POLY");
-  fill_sin_poly(&Sin_poly, Get_context_params()->_hamming_weight, env && atoi(env) != 0);
+  if (__atomic_load_n(&Sin_poly.n_coeff, __ATOMIC_ACQUIRE)) return &Sin_poly;
+  Rt_shared_lock();
+  if (!Sin_poly.n_coeff) {
+    SIN_POLY    p;
+    const char* env = getenv("RTLIB_BTS_EVEN_POLY");
+    fill_sin_poly(&p, Get_context_params()->_hamming_weight, env && atoi(env) != 0);
+    uint32_t n = p.n_coeff;
+    p.n_coeff  = 0;
+    Sin_poly   = p;
+    __atomic_store_n(&Sin_poly.n_coeff, n, __ATOMIC_RELEASE); /* the count makes the rest visible */
+  }
+  Rt_shared_unlock();
   return &Sin_poly;
 }
 /* for inspection without a context: the series of a Hamming weight; returns the number of coefficients */
@@ -303,7 +312,7 @@ static void encode_levels(BTS_PRECOM* pre, bool encoding, const DCMPLX* ksi, con
         pt->_scaling_factor = G.sc;
         pt->_sf_degree      = 1;
         pt->_slots          = len;
-        ACE_OK(ace_encode(G.ctx, pt->_poly._data, (const double*)rot, len, len, level, 1, G.K));
+        ACE_OK(ace_encode(RT_CTX, pt->_poly._data, (const double*)rot, len, len, level, 1, G.K));
       }
   }
   free(rot);
@@ -312,7 +321,7 @@ static void encode_levels(BTS_PRECOM* pre, bool encoding, const DCMPLX* ksi, con
 }
 
 static BTS_PRECOM* find_precom(uint32_t slots) {
-  for (BTS_PRECOM* p = Precoms; p; p = p->next)
+  for (BTS_PRECOM* p = __atomic_load_n(&Precoms, __ATOMIC_ACQUIRE); p; p = p->next)
     if (p->slots == slots) return p;
   return NULL;
 }
@@ -323,7 +332,16 @@ static uint32_t bootstrap_depth(const BTS_PRECOM* pre) {
 
 /* Bootstrap_setup with the level budgets {3, 3} of Bootstrap_precom (bootstrap.c:1061-1197,
  * ckks_context.c:239-262) */
+static BTS_PRECOM* setup_locked(uint32_t slots);
 static BTS_PRECOM* setup(uint32_t slots) {
+  BTS_PRECOM* pre = find_precom(slots); /* the list only grows, at its head, by whole entries */
+  if (pre) return pre;
+  Rt_shared_lock();
+  pre = setup_locked(slots);
+  Rt_shared_unlock();
+  return pre;
+}
+static BTS_PRECOM* setup_locked(uint32_t slots) {
   BTS_PRECOM* pre = find_precom(slots);
   if (pre) return pre;
   FMT_ASSERT(slots >= 2 && (slots & (slots - 1)) == 0 && slots <= G.N / 2, "bootstrap: invalid slot count %u", slots);
@@ -354,19 +372,25 @@ static BTS_PRECOM* setup(uint32_t slots) {
   encode_levels(pre, false, ksi, rot_group, 1.0 / ratio, 1.0, (uint32_t)(G.L - approx_mod_depth() - (uint32_t)pre->enc.budget));
   free(ksi);
   free(rot_group);
+  Rt_shared_publish(); /* the diagonals are encoded on this thread's stream and read on every thread's */
   pre->next = Precoms;
-  Precoms   = pre;
+  __atomic_store_n(&Precoms, pre, __ATOMIC_RELEASE);
   return pre;
 }
 
 /* rotation keys of every step of both transforms, the sparse-packing sums, and conjugation
  * (bootstrap.c:211-285,1199-1231) */
 static void need_rot_key(int32_t rot) {
-  if (rot == 0 || (uint32_t)rot == G.N / 2 || Rt_find_rot(rot)) return;
-  Rt_generate_rotation_key(rot);
+  if (rot == 0 || (uint32_t)rot == G.N / 2) return;
+  ROT_KEY* r = Rt_find_rot(rot);
+  if (r && __atomic_load_n(&r->swk._public_keys, __ATOMIC_ACQUIRE)) return;
+  Rt_shared_lock(); /* another thread may be making this key */
+  r = Rt_find_rot(rot);
+  if (!r || !r->swk._public_keys) Rt_generate_rotation_key(rot);
+  Rt_shared_unlock();
 }
 static void keygen(BTS_PRECOM* pre) {
-  if (pre->keys) return;
+  if (__atomic_load_n(&pre->keys, __ATOMIC_ACQUIRE)) return;
   for (int enc = 1; enc >= 0; --enc) {
     const FFT_PLAN* p = enc ? &pre->enc : &pre->dec;
     int32_t         s_of[32], n;
@@ -380,7 +404,7 @@ static void keygen(BTS_PRECOM* pre) {
   }
   for (uint32_t j = 1; j < G.N / (2 * pre->slots); j <<= 1) need_rot_key((int32_t)(j * pre->slots));
   need_rot_key((int32_t)(2 * G.N - 1));
-  pre->keys = true;
+  __atomic_store_n(&pre->keys, true, __ATOMIC_RELEASE);
 }
 
 /* Bootstrap_precom (context/src/ckks_context.c:239-262): when the chain is deep enough to bootstrap at all, the
@@ -421,7 +445,7 @@ static void add_const(CIPHER c, double value) { /* Add_const, in place */
   int64_t w[128];
   size_t  l = Level(c);
   Rt_encode_val_words(w, value, (uint32_t)l, c->_scaling_factor);
-  ACE_OK(ace_poly_add_scalars(G.ctx, c->_c0_poly._data, c->_c0_poly._data, w, l));
+  ACE_OK(ace_poly_add_scalars(RT_CTX, c->_c0_poly._data, c->_c0_poly._data, w, l));
 }
 static void scale_words(CIPHER res, CIPHER c, const int64_t* w, double sf, uint32_t deg) {
   size_t l = Level(c);
@@ -431,8 +455,8 @@ static void scale_words(CIPHER res, CIPHER c, const int64_t* w, double sf, uint3
     res->_slots = c->_slots;
   }
   res->_c0_poly._is_ntt = res->_c1_poly._is_ntt = true;
-  ACE_OK(ace_poly_mul_scalars(G.ctx, res->_c0_poly._data, c->_c0_poly._data, w, l));
-  ACE_OK(ace_poly_mul_scalars(G.ctx, res->_c1_poly._data, c->_c1_poly._data, w, l));
+  ACE_OK(ace_poly_mul_scalars(RT_CTX, res->_c0_poly._data, c->_c0_poly._data, w, l));
+  ACE_OK(ace_poly_mul_scalars(RT_CTX, res->_c1_poly._data, c->_c1_poly._data, w, l));
   res->_scaling_factor = sf;
   res->_sf_degree      = deg;
 }
@@ -455,22 +479,18 @@ static void set_level(CIPHER c, size_t level) {
 /* The monomial X^power over all Q limbs in NTT form, kept on the device once built: a bootstrap multiplies by the
  * same two monomials every time, and building one means a host buffer of a whole polynomial, an upload (which waits
  * for the GPU to finish everything issued so far) and a transform. */
-#define MONO_SLOTS 8
+#define MONO_SLOTS 16
 static struct {
   uint32_t power;
   int64_t* dev;
 } Mono[MONO_SLOTS];
-static size_t Mono_n;
+static size_t Mono_n; /* entries below it are complete, on the device too, and stay until the context ends */
 static void   mono_clear(void) {
   for (size_t i = 0; i < Mono_n; ++i) Rt_dev_free(Mono[i].dev);
   Mono_n = 0;
 }
-static int64_t* monomial(uint32_t power) {
-  size_t n = G.N, l = G.L;
-  power %= (uint32_t)(2 * n);
-  for (size_t i = 0; i < Mono_n; ++i)
-    if (Mono[i].power == power) return Mono[i].dev;
-  if (Mono_n == MONO_SLOTS) mono_clear();
+static int64_t* build_monomial(uint32_t power) {
+  size_t   n = G.N, l = G.L;
   int64_t* host = (int64_t*)calloc(l * n, sizeof(int64_t));
   int64_t* mono = Rt_dev_alloc(l * n);
   int32_t  idx[128];
@@ -478,17 +498,40 @@ static int64_t* monomial(uint32_t power) {
     host[t * n + power % n] = power < n ? 1 : G.q[t]._val - 1;
     idx[t]                  = (int32_t)t;
   }
-  ACE_OK(ace_upload(G.ctx, mono, host, l * n));
-  ACE_OK(ace_ntt(G.ctx, mono, mono, idx, l, 1, 0));
+  ACE_OK(ace_upload(RT_CTX, mono, host, l * n));
+  ACE_OK(ace_ntt(RT_CTX, mono, mono, idx, l, 1, 0));
   free(host);
-  Mono[Mono_n].power = power;
-  Mono[Mono_n].dev   = mono;
-  Mono_n++;
+  return mono;
+}
+/* *temporary: the table is full and the caller frees the polynomial after use */
+static int64_t* monomial(uint32_t power, bool* temporary) {
+  power %= (uint32_t)(2 * G.N);
+  *temporary = false;
+  size_t seen = __atomic_load_n(&Mono_n, __ATOMIC_ACQUIRE);
+  for (size_t i = 0; i < seen; ++i)
+    if (Mono[i].power == power) return Mono[i].dev;
+  Rt_shared_lock();
+  int64_t* mono = NULL;
+  for (size_t i = 0; i < Mono_n && !mono; ++i)
+    if (Mono[i].power == power) mono = Mono[i].dev;
+  if (!mono) {
+    mono = build_monomial(power);
+    if (Mono_n < MONO_SLOTS) {
+      Rt_shared_publish(); /* built on this thread's stream, read on every thread's */
+      Mono[Mono_n].power = power;
+      Mono[Mono_n].dev   = mono;
+      __atomic_store_n(&Mono_n, Mono_n + 1, __ATOMIC_RELEASE);
+    } else {
+      *temporary = true;
+    }
+  }
+  Rt_shared_unlock();
   return mono;
 }
 CIPHER Mul_mono_ciph(CIPHER res, CIPHER c, uint32_t power) { /* Mul_by_monomial (evaluator.c:260-286) */
   size_t   l    = Level(c);
-  int64_t* mono = monomial(power); /* limb t of a polynomial at any level is limb t of the chain */
+  bool     temporary;
+  int64_t* mono = monomial(power, &temporary); /* limb t of a polynomial at any level is limb t of the chain */
   if (res != c) {
     Init_poly(&res->_c0_poly, &c->_c0_poly);
     Init_poly(&res->_c1_poly, &c->_c1_poly);
@@ -496,8 +539,9 @@ CIPHER Mul_mono_ciph(CIPHER res, CIPHER c, uint32_t power) { /* Mul_by_monomial 
     res->_sf_degree      = c->_sf_degree;
     res->_slots          = c->_slots;
   }
-  ACE_OK(ace_poly_mul(G.ctx, res->_c0_poly._data, c->_c0_poly._data, mono, l, 0));
-  ACE_OK(ace_poly_mul(G.ctx, res->_c1_poly._data, c->_c1_poly._data, mono, l, 0));
+  ACE_OK(ace_poly_mul(RT_CTX, res->_c0_poly._data, c->_c0_poly._data, mono, l, 0));
+  ACE_OK(ace_poly_mul(RT_CTX, res->_c1_poly._data, c->_c1_poly._data, mono, l, 0));
+  if (temporary) Rt_dev_free(mono);
   res->_c0_poly._is_ntt = res->_c1_poly._is_ntt = true;
   return res;
 }
@@ -527,7 +571,7 @@ static void ext_rotate(EXT_CT* out, const int64_t* digits, size_t n_digits, cons
   ROT_KEY* key = Rt_find_rot(rot);
   FMT_ASSERT(key, "cannot find auto key of rotation %d", rot);
   size_t half = (G.L + G.K) * G.N;
-  ACE_OK(ace_ext_rotate(G.ctx, out->c0, out->c1, digits, key->swk._public_keys->dev, half, 2 * half, n_digits, c0_ext,
+  ACE_OK(ace_ext_rotate(RT_CTX, out->c0, out->c1, digits, key->swk._public_keys->dev, half, 2 * half, n_digits, c0_ext,
                         key->order, level, accumulate));
 }
 static void rotate_iteration(CIPHER ct, BTS_PRECOM* pre, bool encoding, int32_t s, bool is_rem, bool first_step) {
@@ -535,12 +579,12 @@ static void rotate_iteration(CIPHER ct, BTS_PRECOM* pre, bool encoding, int32_t 
   PLAINTEXT*      plains = (encoding ? pre->enc_plain : pre->dec_plain)[s];
   LEVEL_ROTS      r      = level_rots(p, s, encoding, is_rem, pre->slots);
   if (!first_step) rescale(ct);
-  size_t level = Level(ct), T = level + G.K, n = G.N, nd = ace_num_decomp(G.ctx, level);
+  size_t level = Level(ct), T = level + G.K, n = G.N, nd = ace_num_decomp(RT_CTX, level);
 
   int64_t* digits = Rt_dev_alloc_raw(nd * T * n);
-  ACE_OK(ace_precomp(G.ctx, digits, ct->_c1_poly._data, level, 1));
+  ACE_OK(ace_precomp(RT_CTX, digits, ct->_c1_poly._data, level, 1));
   int64_t* c0_ext = Rt_dev_alloc_raw(T * n);
-  ACE_OK(ace_extend(G.ctx, c0_ext, ct->_c0_poly._data, level));
+  ACE_OK(ace_extend(RT_CTX, c0_ext, ct->_c0_poly._data, level));
   EXT_CT  outer = ext_alloc(level);
   EXT_CT* rots = (EXT_CT*)calloc((size_t)r.giant, sizeof(EXT_CT));
   for (int32_t j = 0; j < r.giant; ++j) {
@@ -549,7 +593,7 @@ static void rotate_iteration(CIPHER ct, BTS_PRECOM* pre, bool encoding, int32_t 
       ext_rotate(&rots[j], digits, nd, c0_ext, r.in[j], level, 0);
     } else { /* Switch_key_ext: the ciphertext itself, lifted */
       Rt_dev_copy(rots[j].c0, c0_ext, T * n);
-      ACE_OK(ace_extend(G.ctx, rots[j].c1, ct->_c1_poly._data, level));
+      ACE_OK(ace_extend(RT_CTX, rots[j].c1, ct->_c1_poly._data, level));
     }
   }
   /* the inner sums of all baby-step groups first: the groups share the rotated ciphertexts, which are read once
@@ -581,7 +625,7 @@ static void rotate_iteration(CIPHER ct, BTS_PRECOM* pre, bool encoding, int32_t 
       inp[i * r.giant + j] = plains[d]._poly._data;
     }
   }
-  ACE_OK(ace_ext_plain_mac_groups(G.ctx, in_r0, in_r1, (size_t)r.baby, in0, in1, (size_t)r.giant, inp, level, plain_level));
+  ACE_OK(ace_ext_plain_mac_groups(RT_CTX, in_r0, in_r1, (size_t)r.baby, in0, in1, (size_t)r.giant, inp, level, plain_level));
   /* The result is sum_i rotation_i(inner sum i).  Group 0 is not rotated: its two halves start the running sums
    * `first` (c0 parts that need no key switch) and `sum1`.  A rotated group's c1 part is brought down, raised again
    * and rotated with its key; its c0 part rides along as the addend; both land in (outer.c0, sum1). */
@@ -592,16 +636,16 @@ static void rotate_iteration(CIPHER ct, BTS_PRECOM* pre, bool encoding, int32_t 
   for (int32_t i = 1; i < r.baby;) {
     EXT_CT* in = &inners[i];
     if (r.out[i] == 0) {
-      ACE_OK(ace_poly_add(G.ctx, first, first, in->c0, level, 1));
-      ACE_OK(ace_poly_add(G.ctx, sum1, sum1, in->c1, level, 1));
+      ACE_OK(ace_poly_add(RT_CTX, first, first, in->c0, level, 1));
+      ACE_OK(ace_poly_add(RT_CTX, sum1, sum1, in->c1, level, 1));
       ++i;
       continue;
     }
     int32_t end = i;
     while (end < r.baby && r.out[end] != 0) ++end;
     size_t cnt = (size_t)(end - i);
-    ACE_OK(ace_mod_down_batch(G.ctx, low, level * n, in->c1, 2 * T * n, cnt, level, 1));
-    ACE_OK(ace_precomp_batch(G.ctx, low_digits, nd * T * n, low, level * n, cnt, level, 1));
+    ACE_OK(ace_mod_down_batch(RT_CTX, low, level * n, in->c1, 2 * T * n, cnt, level, 1));
+    ACE_OK(ace_precomp_batch(RT_CTX, low_digits, nd * T * n, low, level * n, cnt, level, 1));
     for (int32_t g = i; g < end; ++g) {
       EXT_CT into = {outer.c0, sum1};
       ext_rotate(&into, low_digits + (size_t)(g - i) * nd * T * n, nd, inners[g].c0, r.out[g], level,
@@ -610,13 +654,13 @@ static void rotate_iteration(CIPHER ct, BTS_PRECOM* pre, bool encoding, int32_t 
     }
     i = end;
   }
-  if (outer0_set) ACE_OK(ace_poly_add(G.ctx, first, first, outer.c0, level, 1));
+  if (outer0_set) ACE_OK(ace_poly_add(RT_CTX, first, first, outer.c0, level, 1));
   free(inners);
   free(in_r0);
   free(in_r1);
   free((void*)inp);
-  ACE_OK(ace_mod_down(G.ctx, ct->_c0_poly._data, first, level, 1));
-  ACE_OK(ace_mod_down(G.ctx, ct->_c1_poly._data, sum1, level, 1));
+  ACE_OK(ace_mod_down(RT_CTX, ct->_c0_poly._data, first, level, 1));
+  ACE_OK(ace_mod_down(RT_CTX, ct->_c1_poly._data, sum1, level, 1));
   ct->_scaling_factor *= G.sc;
   ct->_sf_degree += 1;
 
@@ -751,7 +795,7 @@ static void weighted_sum(CIPHER out, CHEB_BASIS* b, const double* w, uint32_t co
   out->_slots          = like->_slots;
   out->_scaling_factor = like->_scaling_factor * G.sc;
   out->_sf_degree      = like->_sf_degree + 1;
-  ACE_OK(ace_ciph_wsum(G.ctx, out->_c0_poly._data, out->_c1_poly._data, in0, in1, words, terms, level));
+  ACE_OK(ace_ciph_wsum(RT_CTX, out->_c0_poly._data, out->_c1_poly._data, in0, in1, words, terms, level));
   free(words);
   rescale(out);
 }
@@ -898,20 +942,27 @@ static void eval_chebyshev(CIPHER ct, const double* coeff, uint32_t n_coeff, boo
 static void eval_approx_mod(CIPHER ct);
 /* The real and the imaginary half of a fully packed ciphertext go through the same series independently: the second
  * is issued on the library's second lane, so that its kernels (one polynomial each, too small for the machine)
- * overlap with the first's.  RT_HIP_ONE_LANE=1 issues them one after the other. */
+ * overlap with the first's.  RT_HIP_ONE_LANE=1 issues them one after the other, and so does a program that runs
+ * on several host threads (a second thread has called into the runtime): their streams fill the machine already,
+ * and twice as many streams as threads share the hardware's few queues (three threads: 0.66 s per ResNet-20 image
+ * with the second lanes, 0.55 s without).  A second stream that was used before the other threads came still costs
+ * them -- the driver then serves two of the threads' streams through one queue (0.69 s) -- so a program that will
+ * run images on several threads lets every thread call in once (Rt_sync() will do) before the first bootstrap; the
+ * reference's driver, whose first image is already inside its parallel loop, does so by itself. */
 static void eval_approx_mod_pair(CIPHER a, CIPHER b) {
   static int one_lane = -1;
   if (one_lane < 0) one_lane = getenv("RT_HIP_ONE_LANE") && atoi(getenv("RT_HIP_ONE_LANE")) != 0;
-  if (one_lane) {
+  if (one_lane || Rt_lane_count() > 1) {
+    if (!one_lane) ACE_OK(ace_fork_release(RT_CTX)); /* a second stream from before the other threads came */
     eval_approx_mod(a);
     eval_approx_mod(b);
     return;
   }
-  ACE_OK(ace_fork(G.ctx));
+  ACE_OK(ace_fork(RT_CTX));
   eval_approx_mod(b);
-  ACE_OK(ace_fork_switch(G.ctx));
+  ACE_OK(ace_fork_switch(RT_CTX));
   eval_approx_mod(a);
-  ACE_OK(ace_join(G.ctx));
+  ACE_OK(ace_join(RT_CTX));
 }
 static void eval_approx_mod(CIPHER ct) {
   const SIN_POLY* p = sin_poly();
@@ -1033,7 +1084,7 @@ CIPHER Eval_bootstrap_ciph(CIPHER res, CIPHER ct, uint32_t level_after_bts, uint
 /* ---- the stages on their own (cipher.c:585-767) ------------------------------------------------------
  * The same pieces as above, cut where the compiler's staged operators cut them.  The imaginary half of a fully
  * packed input lives here between the first two calls. */
-static struct {
+static __thread struct {
   bool       active, full;
   uint32_t   slots;
   CIPHERTEXT sub;

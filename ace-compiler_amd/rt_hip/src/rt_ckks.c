@@ -10,8 +10,13 @@
 
 #include "rt_internal.h"
 
-/* ---- random numbers: xoshiro256** seeded through splitmix64 --------------------------------- */
-static uint64_t Rng[4];
+/* ---- random numbers: xoshiro256** seeded through splitmix64 ---------------------------------
+ * One generator per host thread, as in the reference's OpenMP build (util/src/prng.c:13-16).  The thread that
+ * generates the keys seeds its own; any other thread's is seeded the first time it draws: from the keys' seed and
+ * the thread's ordinal when that seed was given (reproducible runs), else from the operating system. */
+static __thread uint64_t Rng[4];
+static __thread bool     Rng_ready;
+static uint64_t          Master_seed; /* the seed given to Rt_generate_keys, 0: none */
 static uint64_t splitmix(uint64_t* s) {
   uint64_t z = (*s += 0x9E3779B97F4A7C15ull);
   z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
@@ -22,7 +27,20 @@ static void rng_seed(uint64_t seed) {
   for (int i = 0; i < 4; ++i) Rng[i] = splitmix(&seed);
 }
 static inline uint64_t rotl(uint64_t x, int k) { return (x << k) | (x >> (64 - k)); }
+static void rng_first_use(void) {
+  const char* env  = getenv("RT_HIP_SEED");
+  uint64_t    seed = Master_seed ? Master_seed : env ? strtoull(env, NULL, 0) : 0;
+  if (seed) {
+    seed += 0xD1342543DE82EF95ull * Rt_this_lane()->ordinal;
+    rng_seed(seed);
+  } else {
+    FMT_ASSERT(getrandom(Rng, sizeof(Rng), 0) == (ssize_t)sizeof(Rng) && (Rng[0] | Rng[1] | Rng[2] | Rng[3]),
+               "no entropy source");
+  }
+  Rng_ready = true;
+}
 static uint64_t rng_next(void) {
+  if (!Rng_ready) rng_first_use();
   uint64_t r = rotl(Rng[1] * 5, 7) * 9, t = Rng[1] << 17;
   Rng[2] ^= Rng[0];
   Rng[3] ^= Rng[1];
@@ -70,18 +88,7 @@ static void sample_ternary(int64_t* v, size_t n, size_t weight) {
   }
 }
 
-static bool Rng_ready;
-void Rt_sample_ternary(int64_t* v, size_t n, size_t hamming_weight) {
-  if (!Rng_ready) { /* no key generation has seeded the stream yet: seed it as Rt_generate_keys(0) would */
-    const char* env  = getenv("RT_HIP_SEED");
-    uint64_t    seed = env ? strtoull(env, NULL, 0) : 0;
-    if (seed) rng_seed(seed);
-    else FMT_ASSERT(getrandom(Rng, sizeof(Rng), 0) == (ssize_t)sizeof(Rng) && (Rng[0] | Rng[1] | Rng[2] | Rng[3]),
-                    "no entropy source");
-    Rng_ready = true;
-  }
-  sample_ternary(v, n, hamming_weight);
-}
+void Rt_sample_ternary(int64_t* v, size_t n, size_t hamming_weight) { sample_ternary(v, n, hamming_weight); }
 
 /* ---- small helpers over the device ------------------------------------------------------------ */
 static uint64_t Seed, Stream; /* of the device-side uniform sampler: one stream per polynomial */
@@ -91,19 +98,19 @@ static void small_to_dev(int64_t* dev, const int64_t* v, size_t level, bool with
   size_t  T = level + (with_p ? G.K : 0);
   int32_t idx[128];
   for (size_t t = 0; t < T; ++t) idx[t] = (int32_t)(t < level ? t : G.L + (t - level));
-  ACE_OK(ace_expand_small(G.ctx, dev, v, level, with_p));
-  ACE_OK(ace_ntt(G.ctx, dev, dev, idx, T, 1, 0));
+  ACE_OK(ace_expand_small(RT_CTX, dev, v, level, with_p));
+  ACE_OK(ace_ntt(RT_CTX, dev, dev, idx, T, 1, 0));
 }
 /* uniform residues, drawn on the device: a uniform polynomial is uniform in NTT form too */
 static void uniform_to_dev(int64_t* dev, size_t level, bool with_p) {
-  ACE_OK(ace_sample_uniform(G.ctx, dev, level, with_p, Seed, Stream++));
+  ACE_OK(ace_sample_uniform(RT_CTX, dev, level, with_p, Seed, __atomic_fetch_add(&Stream, 1, __ATOMIC_RELAXED)));
 }
 
 /* ---- keys (ckks/src/key_gen.c:127-262) ----------------------------------------------------------- */
 /* a switch key taking a polynomial that multiplies s_src to a pair that decrypts under s_res (both: device,
  * L+k limbs, NTT), built in place in HBM: per digit b = -a*s_res + e + P*s_src on the digit's limbs */
 static void make_switch_key(SWITCH_KEY* key, const int64_t* s_res, const int64_t* s_src) {
-  size_t   n = G.N, T = G.L + G.K, ps = ace_part_size(G.ctx);
+  size_t   n = G.N, T = G.L + G.K, ps = ace_part_size(RT_CTX);
   int64_t* dev = Rt_dev_alloc_raw(2 * G.parts * T * n);
   int64_t *e = Rt_dev_alloc_raw(T * n), *t = Rt_dev_alloc_raw(n);
   int64_t* small = (int64_t*)malloc(n * sizeof(int64_t));
@@ -112,13 +119,13 @@ static void make_switch_key(SWITCH_KEY* key, const int64_t* s_res, const int64_t
     uniform_to_dev(a, G.L, true);
     sample_triangle(small, n);
     small_to_dev(e, small, G.L, true);
-    ACE_OK(ace_poly_mul(G.ctx, b, a, s_res, G.L, 1));
-    ACE_OK(ace_poly_sub(G.ctx, b, e, b, G.L, 1));
+    ACE_OK(ace_poly_mul(RT_CTX, b, a, s_res, G.L, 1));
+    ACE_OK(ace_poly_sub(RT_CTX, b, e, b, G.L, 1));
     for (size_t i = d * ps; i < (d + 1) * ps && i < G.L; ++i) {
       uint64_t q = (uint64_t)G.q[i]._val, pm = 1; /* P mod q_i */
       for (size_t j = 0; j < G.K; ++j) pm = (uint64_t)((unsigned __int128)pm * ((uint64_t)G.p[j]._val % q) % q);
-      ACE_OK(ace_hw_modmul_scalar(G.ctx, t, s_src + i * n, (int64_t)pm, i, n));
-      ACE_OK(ace_hw_modadd(G.ctx, b + i * n, b + i * n, t, i, n));
+      ACE_OK(ace_hw_modmul_scalar(RT_CTX, t, s_src + i * n, (int64_t)pm, i, n));
+      ACE_OK(ace_hw_modadd(RT_CTX, b + i * n, b + i * n, t, i, n));
     }
   }
   free(small);
@@ -143,6 +150,7 @@ static uint64_t inv_mod_pow2(uint64_t k, uint64_t m) { /* k odd, m a power of tw
 
 void Rt_generate_rotation_key(int32_t rot_idx) {
   FMT_ASSERT(G.secret_ntt, "Rt_generate_keys() has not run");
+  Rt_shared_lock(); /* one key at a time; the key is whole on the device before another thread can find it */
   size_t   n = G.N, T = G.L + G.K;
   ROT_KEY* entry = Rt_rot_entry(rot_idx);
   uint32_t k = entry->auto_idx;
@@ -155,6 +163,7 @@ void Rt_generate_rotation_key(int32_t rot_idx) {
   make_switch_key(&Rt_find_rot(rot_idx)->swk, s_res, G.secret_ntt);
   free(rs);
   Rt_dev_free(s_res);
+  Rt_shared_unlock();
 }
 
 void Rt_generate_keys(uint64_t seed) {
@@ -163,6 +172,7 @@ void Rt_generate_keys(uint64_t seed) {
     const char* env = getenv("RT_HIP_SEED");
     seed = env ? strtoull(env, NULL, 0) : 0;
   }
+  Master_seed = seed;
   if (seed) {
     rng_seed(seed); /* a fixed seed: reproducible runs for tests and benchmarks only */
   } else {
@@ -194,13 +204,13 @@ void Rt_generate_keys(uint64_t seed) {
   uniform_to_dev(G.pk1, G.L, false);
   sample_triangle(small, n);
   small_to_dev(e, small, G.L, false);
-  ACE_OK(ace_poly_mul(G.ctx, G.pk0, G.pk1, G.secret_ntt, G.L, 0));
-  ACE_OK(ace_poly_sub(G.ctx, G.pk0, e, G.pk0, G.L, 0));
+  ACE_OK(ace_poly_mul(RT_CTX, G.pk0, G.pk1, G.secret_ntt, G.L, 0));
+  ACE_OK(ace_poly_sub(RT_CTX, G.pk0, e, G.pk0, G.L, 0));
   Rt_dev_free(e);
   free(small);
   /* relinearisation key: from s^2 to s */
   int64_t* s2 = Rt_dev_alloc_raw(T * n);
-  ACE_OK(ace_poly_mul(G.ctx, s2, G.secret_ntt, G.secret_ntt, G.L, 1));
+  ACE_OK(ace_poly_mul(RT_CTX, s2, G.secret_ntt, G.secret_ntt, G.L, 1));
   make_switch_key(&G.relin, G.secret_ntt, s2);
   Rt_dev_free(s2);
   for (size_t i = 0; i < prm->_num_rot_idx; ++i)
@@ -214,8 +224,8 @@ void Rt_get_secret(int64_t* host_small) {
 }
 void Rt_get_public_key(int64_t* host_pk0, int64_t* host_pk1) {
   FMT_ASSERT(G.pk0, "Rt_generate_keys() has not run");
-  ACE_OK(ace_download(G.ctx, host_pk0, G.pk0, G.L * G.N));
-  ACE_OK(ace_download(G.ctx, host_pk1, G.pk1, G.L * G.N));
+  ACE_OK(ace_download(RT_CTX, host_pk0, G.pk0, G.L * G.N));
+  ACE_OK(ace_download(RT_CTX, host_pk1, G.pk1, G.L * G.N));
 }
 
 void Rt_ckks_finalize(void) {
@@ -291,8 +301,8 @@ static void encode_value(PLAIN plain, double value, uint32_t sc_degree, uint32_t
   Rt_encode_val_words(words, value, level, scale);
   for (uint32_t t = 0; t < level; ++t) {
     int64_t* limb = plain->_poly._data + (size_t)t * G.N;
-    ACE_OK(ace_zero(G.ctx, limb, G.N));
-    ACE_OK(ace_hw_modadd_scalar(G.ctx, limb, limb, words[t], t, G.N));
+    ACE_OK(ace_zero(RT_CTX, limb, G.N));
+    ACE_OK(ace_hw_modadd_scalar(RT_CTX, limb, limb, words[t], t, G.N));
   }
 }
 
@@ -300,7 +310,7 @@ static void encode_vector(PLAIN plain, const double* re_im, size_t len, uint32_t
   if (level == 0) level = (uint32_t)G.L;
   FMT_ASSERT(level <= G.L, "level should not be larger than mul_depth + 1");
   init_plain(plain, level, pow(G.sc, sc_degree), sc_degree, G.N / 2);
-  ACE_OK(ace_encode(G.ctx, plain->_poly._data, re_im, len, 0, level, sc_degree, 0));
+  ACE_OK(ace_encode(RT_CTX, plain->_poly._data, re_im, len, 0, level, sc_degree, 0));
 }
 /* a plaintext of `level` limbs at scale degree sc_degree whose polynomial the caller fills in (NTT form) */
 int64_t* Rt_plain_prepare(PLAIN plain, uint32_t sc_degree, uint32_t level) {
@@ -314,7 +324,7 @@ void Rt_encode_real(PLAIN plain, const void* values, int is_f32, size_t len, uin
   if (level == 0) level = (uint32_t)G.L;
   FMT_ASSERT(level <= G.L, "level should not be larger than mul_depth + 1");
   init_plain(plain, level, pow(G.sc, sc_degree), sc_degree, G.N / 2);
-  ACE_OK(ace_encode_real(G.ctx, plain->_poly._data, values, is_f32, len, 0, level, sc_degree, 0));
+  ACE_OK(ace_encode_real(RT_CTX, plain->_poly._data, values, is_f32, len, 0, level, sc_degree, 0));
 }
 
 /* n_vec real-valued vectors into the polynomials dev_base + v * stride (level limbs each, NTT form) */
@@ -322,7 +332,7 @@ void Rt_encode_real_batch(int64_t* dev_base, size_t stride, const void* const* v
                           size_t n_vec, uint32_t sc_degree, uint32_t level) {
   if (level == 0) level = (uint32_t)G.L;
   FMT_ASSERT(level <= G.L, "level should not be larger than mul_depth + 1");
-  ACE_OK(ace_encode_real_batch(G.ctx, dev_base, stride, values, is_f32, len, n_vec, 0, level, sc_degree, 0));
+  ACE_OK(ace_encode_real_batch(RT_CTX, dev_base, stride, values, is_f32, len, n_vec, 0, level, sc_degree, 0));
 }
 
 void Encode_double(PLAIN plain, double* input, size_t len, uint32_t sc_degree, uint32_t level) {
@@ -362,7 +372,7 @@ void Encode_dcmplx_ext(PLAIN plain, DCMPLX* input, size_t len, uint32_t level, u
   plain->_sf_degree      = 1;
   plain->_slots          = G.N / 2;
   p->_is_ntt             = true;
-  ACE_OK(ace_encode(G.ctx, p->_data, (const double*)input, len, 0, level, 1, p_cnt));
+  ACE_OK(ace_encode(RT_CTX, p->_data, (const double*)input, len, 0, level, 1, p_cnt));
 }
 /* Encode_float_with_scale (ckks/src/plain.c:104-123): the scale is given, the degree recorded is the least
  * power of the scaling factor that reaches it (Get_approx_sf_degree, encoder.c:328-335) */
@@ -379,14 +389,14 @@ void Encode_float_with_scale(PLAIN plain, float* input, size_t len, double scale
     Rt_encode_val_words(words, (double)*input, level, scale);
     for (uint32_t t = 0; t < level; ++t) {
       int64_t* limb = plain->_poly._data + (size_t)t * G.N;
-      ACE_OK(ace_zero(G.ctx, limb, G.N));
-      ACE_OK(ace_hw_modadd_scalar(G.ctx, limb, limb, words[t], t, G.N));
+      ACE_OK(ace_zero(RT_CTX, limb, G.N));
+      ACE_OK(ace_hw_modadd_scalar(RT_CTX, limb, limb, words[t], t, G.N));
     }
     return;
   }
   double* v = (double*)calloc(2 * len, sizeof(double));
   for (size_t i = 0; i < len; ++i) v[2 * i] = (double)input[i];
-  ACE_OK(ace_encode_scaled(G.ctx, plain->_poly._data, v, len, 0, level, scale, 0));
+  ACE_OK(ace_encode_scaled(RT_CTX, plain->_poly._data, v, len, 0, level, scale, 0));
   free(v);
 }
 /* Encode_single_double (ckks/src/plain.c:139-147): `level` host words */
@@ -425,15 +435,15 @@ CIPHER Add_plain(CIPHER res, CIPHER c, PLAIN plain) {
   FMT_ASSERT(c->_scaling_factor == plain->_scaling_factor, "Scaling factors are not equal.");
   Init_ciph_same_scale_plain(res, c, plain);
   size_t level = Level(res), n = G.N;
-  ACE_OK(ace_poly_add(G.ctx, res->_c0_poly._data, c->_c0_poly._data, plain->_poly._data, level, 0));
+  ACE_OK(ace_poly_add(RT_CTX, res->_c0_poly._data, c->_c0_poly._data, plain->_poly._data, level, 0));
   Rt_dev_copy(res->_c1_poly._data, c->_c1_poly._data, level * n);
   return res;
 }
 CIPHER Mul_plain(CIPHER res, CIPHER c, PLAIN plain) {
   Init_ciph_up_scale_plain(res, c, plain);
   size_t level = Level(res);
-  ACE_OK(ace_poly_mul(G.ctx, res->_c0_poly._data, c->_c0_poly._data, plain->_poly._data, level, 0));
-  ACE_OK(ace_poly_mul(G.ctx, res->_c1_poly._data, c->_c1_poly._data, plain->_poly._data, level, 0));
+  ACE_OK(ace_poly_mul(RT_CTX, res->_c0_poly._data, c->_c0_poly._data, plain->_poly._data, level, 0));
+  ACE_OK(ace_poly_mul(RT_CTX, res->_c1_poly._data, c->_c1_poly._data, plain->_poly._data, level, 0));
   return res;
 }
 
@@ -456,13 +466,13 @@ CIPHER Encrypt(CIPHER res, PLAIN plain) {
   /* c0 = pk0 u + e1 + m ; c1 = pk1 u + e2 */
   sample_triangle(small, n);
   small_to_dev(e, small, level, false);
-  ACE_OK(ace_poly_mul(G.ctx, res->_c0_poly._data, G.pk0, u, level, 0));
-  ACE_OK(ace_poly_add(G.ctx, res->_c0_poly._data, res->_c0_poly._data, e, level, 0));
-  ACE_OK(ace_poly_add(G.ctx, res->_c0_poly._data, res->_c0_poly._data, pt->_data, level, 0));
+  ACE_OK(ace_poly_mul(RT_CTX, res->_c0_poly._data, G.pk0, u, level, 0));
+  ACE_OK(ace_poly_add(RT_CTX, res->_c0_poly._data, res->_c0_poly._data, e, level, 0));
+  ACE_OK(ace_poly_add(RT_CTX, res->_c0_poly._data, res->_c0_poly._data, pt->_data, level, 0));
   sample_triangle(small, n);
   small_to_dev(e, small, level, false);
-  ACE_OK(ace_poly_mul(G.ctx, res->_c1_poly._data, G.pk1, u, level, 0));
-  ACE_OK(ace_poly_add(G.ctx, res->_c1_poly._data, res->_c1_poly._data, e, level, 0));
+  ACE_OK(ace_poly_mul(RT_CTX, res->_c1_poly._data, G.pk1, u, level, 0));
+  ACE_OK(ace_poly_add(RT_CTX, res->_c1_poly._data, res->_c1_poly._data, e, level, 0));
   res->_c0_poly._is_ntt = res->_c1_poly._is_ntt = true;
   free(small);
   Rt_dev_free(u);
@@ -474,8 +484,8 @@ void Rt_decrypt(PLAIN res, CIPHER c) {
   FMT_ASSERT(G.secret_ntt, "Rt_generate_keys() has not run");
   size_t level = Level(c);
   init_plain(res, level, c->_scaling_factor, c->_sf_degree, c->_slots);
-  ACE_OK(ace_poly_mul(G.ctx, res->_poly._data, c->_c1_poly._data, G.secret_ntt, level, 0));
-  ACE_OK(ace_poly_add(G.ctx, res->_poly._data, res->_poly._data, c->_c0_poly._data, level, 0));
+  ACE_OK(ace_poly_mul(RT_CTX, res->_poly._data, c->_c1_poly._data, G.secret_ntt, level, 0));
+  ACE_OK(ace_poly_add(RT_CTX, res->_poly._data, res->_poly._data, c->_c0_poly._data, level, 0));
 }
 
 /* ---- decoding (ckks/src/encoder.c:657-704): Reconstruct, the conversion to double and the embedding run on the
@@ -484,7 +494,7 @@ void Rt_decode(DCMPLX* res, PLAIN plain) {
   POLY     p     = &plain->_poly;
   uint32_t slots = plain->_slots ? plain->_slots : (uint32_t)(G.N / 2);
   FMT_ASSERT(p->_num_primes_p == 0, "decoding an extended plaintext is not supported");
-  ACE_OK(ace_decode(G.ctx, (double*)res, p->_data, p->_num_primes, p->_is_ntt, slots, plain->_scaling_factor));
+  ACE_OK(ace_decode(RT_CTX, (double*)res, p->_data, p->_num_primes, p->_is_ntt, slots, plain->_scaling_factor));
 }
 
 DCMPLX* Get_dcmplx_msg_from_plain(PLAIN plain) {
@@ -583,7 +593,7 @@ bool Within_value_range(CIPHER c, double* msg, uint32_t len) {
   double*      in  = (double*)calloc(2 * (size_t)n, sizeof(double));
   double*      out = (double*)calloc(2 * (size_t)n, sizeof(double));
   for (uint32_t i = 0; i < len; ++i) in[2 * i] = msg[i];
-  ACE_OK(ace_embedding_inv(G.ctx, out, in, n));
+  ACE_OK(ace_embedding_inv(RT_CTX, out, in, n));
   double biggest = 0; /* Transform_msg_within_range, encoder.c:217-231 */
   for (size_t i = 0; i < 2 * (size_t)n; ++i) {
     double up = fabs(out[i] * c->_scaling_factor);
@@ -605,7 +615,7 @@ CIPHER Real_relu(CIPHER c) {
   PLAINTEXT pt;
   memset(&pt, 0, sizeof(pt));
   init_plain(&pt, Level(c), pow(G.sc, c->_sf_degree), c->_sf_degree, n);
-  ACE_OK(ace_encode(G.ctx, pt._poly._data, (const double*)m, n, n, Level(c), c->_sf_degree, 0));
+  ACE_OK(ace_encode(RT_CTX, pt._poly._data, (const double*)m, n, n, Level(c), c->_sf_degree, 0));
   CIPHER res = (CIPHER)calloc(1, sizeof(CIPHERTEXT));
   Encrypt(res, &pt);
   Free_plain_poly(&pt);
@@ -673,7 +683,7 @@ static void prepare_input(TENSOR* input, const char* name, bool dup) {
     PLAINTEXT pt;
     memset(&pt, 0, sizeof(pt));
     encode_vector(&pt, v, len, 1, (uint32_t)level);
-    IO_SLOT*    s  = Rt_add_slot(&G.in, &G.n_in, name, (size_t)i);
+    IO_SLOT*    s  = Rt_add_slot(&LANE.in, &LANE.n_in, name, (size_t)i);
     CIPHERTEXT* ct = (CIPHERTEXT*)calloc(1, sizeof(CIPHERTEXT));
     Encrypt(ct, &pt);
     s->ct = ct;
@@ -693,7 +703,7 @@ double* Handle_output(const char* name) {
   if (len == 0) len = G.N / 2;
   double* ret = (double*)calloc(len, sizeof(double));
   for (int i = 0; i < sch->_count; ++i) {
-    IO_SLOT* s = Rt_find_slot(G.out, G.n_out, name, (size_t)i);
+    IO_SLOT* s = Rt_find_slot(LANE.out, LANE.n_out, name, (size_t)i);
     FMT_ASSERT(s && s->ct, "not find data");
     PLAINTEXT pt;
     memset(&pt, 0, sizeof(pt));

@@ -291,7 +291,19 @@ static bool encode_ahead(void* pt, uint32_t index, size_t ofst, size_t len, uint
   return true;
 }
 
+/* The kept plaintexts and the synthetic entries are shared by the program's threads: one thread at a time looks
+ * them up or adds to them, and a thread that has added polynomials waits for its stream before it lets go, because
+ * the next thread copies them on a stream of its own. */
+static void* from_msg_locked(void* pt, uint32_t index, size_t ofst, size_t len, uint32_t scale, uint32_t level, bool* added);
 void* Pt_from_msg_ofst(void* pt, uint32_t index, size_t ofst, size_t len, uint32_t scale, uint32_t level) {
+  bool added = false;
+  Rt_shared_lock();
+  from_msg_locked(pt, index, ofst, len, scale, level, &added);
+  if (added) Rt_shared_publish();
+  Rt_shared_unlock();
+  return pt;
+}
+static void* from_msg_locked(void* pt, uint32_t index, size_t ofst, size_t len, uint32_t scale, uint32_t level, bool* added) {
   const size_t   words = (size_t)(level ? level : Get_q_cnt()) * Degree();
   const uint64_t k1    = cache_key1(index, scale, level);
   const uint64_t k2    = ((uint64_t)ofst << 32) | (uint64_t)len;
@@ -304,7 +316,10 @@ void* Pt_from_msg_ofst(void* pt, uint32_t index, size_t ofst, size_t len, uint32
       return pt;
     }
     if (Cache.words + words > Cache.limit_words) cell = NULL;
-    if (cell && encode_ahead(pt, index, ofst, len, scale, level, words)) return pt;
+    if (cell && encode_ahead(pt, index, ofst, len, scale, level, words)) {
+      *added = true;
+      return pt;
+    }
     if (cell) cell = cache_find(k1, k2); /* the table may have grown */
   }
   Pt_encode_entry(pt, index, ofst, len, scale, level);
@@ -314,6 +329,7 @@ void* Pt_from_msg_ofst(void* pt, uint32_t index, size_t ofst, size_t len, uint32
     cell->k2 = k2;
     ++Cache.count;
     Cache.words += words;
+    *added = true;
   }
   return pt;
 }
@@ -332,7 +348,9 @@ void* Pt_from_msg(void* pt, uint32_t index, size_t len, uint32_t scale, uint32_t
   return Pt_from_msg_ofst(pt, index, 0, len, scale, level);
 }
 void Pt_from_msg_ofst_validate(void* pt, float* buf, uint32_t index, size_t ofst, size_t len, uint32_t scale, uint32_t level) {
+  Rt_shared_lock();
   double* v = entry_values(index, ofst, len);
+  Rt_shared_unlock();
   for (size_t i = 0; i < len; ++i)
     FMT_ASSERT(fabs((double)buf[i] - v[i]) < 0.000001, "Pt_from_msg_validate failed. index=%u, i=%zu: %f != %f.", index, i,
                (double)buf[i], v[i]);
@@ -372,22 +390,29 @@ static PLAINTEXT* load_plain_entry(uint32_t index) {
              "plaintext %u does not fit this context (degree %u, %zu + %zu primes)", index, poly->_ring_degree,
              poly->_num_primes, poly->_num_primes_p);
   poly->_data = Rt_dev_alloc_raw(words);
-  ACE_OK(ace_upload(G.ctx, poly->_data, (const int64_t*)(raw + 16 + sizeof(PLAINTEXT)), words)); /* waits for the copy */
+  ACE_OK(ace_upload(RT_CTX, poly->_data, (const int64_t*)(raw + 16 + sizeof(PLAINTEXT)), words)); /* waits for the copy */
   free(raw);
   return Data.pt[index] = pt;
 }
 void* Pt_get(uint32_t index, size_t len, uint32_t scale, uint32_t level) {
   (void)len, (void)scale, (void)level; /* the entry carries its own shape, as in the reference */
-  return load_plain_entry(index);
+  Rt_shared_lock(); /* the upload waits for the copy, so the entry is whole when the lock is released */
+  PLAINTEXT* pt = load_plain_entry(index);
+  Rt_shared_unlock();
+  return pt;
 }
 void Pt_prefetch(uint32_t index) {
+  Rt_shared_lock();
   if (plaintext_file() && index < Data.hdr.ent_count) (void)load_plain_entry(index);
+  Rt_shared_unlock();
 }
 void Pt_free(uint32_t index) {
+  Rt_shared_lock();
   FMT_ASSERT(plaintext_file() && index < Data.hdr.ent_count && Data.pt[index], "BLOCK_INFO state is not ready");
   Free_poly_data(&Data.pt[index]->_poly);
   free(Data.pt[index]);
   Data.pt[index] = NULL;
+  Rt_shared_unlock();
 }
 void* Pt_get_validate(float* buf, uint32_t index, size_t len, uint32_t scale, uint32_t level) {
   (void)buf, (void)len, (void)scale, (void)level;

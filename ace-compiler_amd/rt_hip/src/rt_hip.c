@@ -5,6 +5,7 @@
 #include "rt_hip.h"
 
 #include <math.h>
+#include <pthread.h>
 #include <stdarg.h>
 #include <time.h>
 
@@ -12,6 +13,52 @@
 #include "rt_internal.h"
 
 struct rt_state G;
+
+/* ---- one lane per host thread ---------------------------------------------------------- */
+__thread struct rt_lane* Rt_lane;
+static pthread_mutex_t   Lanes_lock = PTHREAD_MUTEX_INITIALIZER;
+static struct rt_lane**  Lanes; /* every lane made since Prepare_context, [0] = that thread's */
+static size_t            N_lanes, Cap_lanes;
+
+static struct rt_lane* new_lane(ace_ctx* ctx) {
+  struct rt_lane* l = (struct rt_lane*)calloc(1, sizeof(*l));
+  l->ctx            = ctx;
+  l->generation     = G.generation;
+  pthread_mutex_lock(&Lanes_lock);
+  if (N_lanes == Cap_lanes) {
+    Cap_lanes = Cap_lanes ? 2 * Cap_lanes : 8;
+    Lanes     = (struct rt_lane**)realloc(Lanes, Cap_lanes * sizeof(*Lanes));
+  }
+  l->ordinal     = (unsigned)N_lanes;
+  Lanes[N_lanes] = l;
+  __atomic_store_n(&N_lanes, N_lanes + 1, __ATOMIC_RELAXED);
+  pthread_mutex_unlock(&Lanes_lock);
+  clock_gettime(CLOCK_MONOTONIC, &l->t0);
+  return Rt_lane = l;
+}
+size_t Rt_lane_count(void) { return __atomic_load_n(&N_lanes, __ATOMIC_RELAXED); }
+/* the calling thread has no lane of the current context yet */
+struct rt_lane* Rt_lane_slow(void) {
+  if (!G.root) Rt_fatal(__FILE__, __LINE__, "Prepare_context() has not run");
+  ace_ctx* ctx = ace_ctx_share(G.root);
+  if (!ctx) Rt_fatal(__FILE__, __LINE__, "no context for this thread: %s", ace_last_error());
+  return new_lane(ctx);
+}
+
+static pthread_mutex_t Shared_lock;
+static pthread_once_t  Shared_once = PTHREAD_ONCE_INIT;
+static void            shared_init(void) {
+  pthread_mutexattr_t a;
+  pthread_mutexattr_init(&a);
+  pthread_mutexattr_settype(&a, PTHREAD_MUTEX_RECURSIVE); /* key generation runs inside the bootstrap's set-up */
+  pthread_mutex_init(&Shared_lock, &a);
+}
+void Rt_shared_lock(void) {
+  pthread_once(&Shared_once, shared_init);
+  pthread_mutex_lock(&Shared_lock);
+}
+void Rt_shared_unlock(void) { pthread_mutex_unlock(&Shared_lock); }
+void Rt_shared_publish(void) { ACE_OK(ace_sync(RT_CTX)); }
 
 void Rt_fatal(const char* file, int line, const char* fmt, ...) {
   va_list ap;
@@ -26,37 +73,38 @@ void Rt_fatal(const char* file, int line, const char* fmt, ...) {
 
 /* ---- lifecycle ----------------------------------------------------------------- */
 void Prepare_context(void) {
-  FMT_ASSERT(!G.ctx, "Prepare_context() called twice");
+  FMT_ASSERT(!G.root, "Prepare_context() called twice");
   FMT_ASSERT(Get_context_params, "the program does not define Get_context_params()");
   CKKS_PARAMS* prm = Get_context_params();
   /* Get_default_num_q_parts (util/src/std_param.c:356-363) */
   size_t parts = prm->_num_q_parts ? prm->_num_q_parts : prm->_mul_depth > 3 ? 3 : prm->_mul_depth == 0 ? 1 : 2;
-  G.ctx = ace_ctx_create(prm->_poly_degree, prm->_mul_depth + 1, prm->_first_mod_size, prm->_scaling_mod_size, parts);
-  if (!G.ctx) Rt_fatal(__FILE__, __LINE__, "%s", ace_last_error());
-  if (!ace_has_device(G.ctx)) Rt_fatal(__FILE__, __LINE__, "no HIP device: this runtime has no CPU path");
-  G.N     = ace_degree(G.ctx);
-  G.L     = ace_num_q(G.ctx);
-  G.K     = ace_num_p(G.ctx);
-  G.parts = ace_num_parts(G.ctx);
+  G.root = ace_ctx_create(prm->_poly_degree, prm->_mul_depth + 1, prm->_first_mod_size, prm->_scaling_mod_size, parts);
+  if (!G.root) Rt_fatal(__FILE__, __LINE__, "%s", ace_last_error());
+  if (!ace_has_device(G.root)) Rt_fatal(__FILE__, __LINE__, "no HIP device: this runtime has no CPU path");
+  ++G.generation;
+  new_lane(G.root); /* this thread issues on the root context itself */
+  G.N     = ace_degree(RT_CTX);
+  G.L     = ace_num_q(RT_CTX);
+  G.K     = ace_num_p(RT_CTX);
+  G.parts = ace_num_parts(RT_CTX);
   G.input_level = prm->_input_level;
   G.sc    = ldexp(1.0, (int)prm->_scaling_mod_size);
   G.q     = (MODULUS*)aligned_alloc(16, sizeof(MODULUS) * (G.L + G.K));
   G.p     = G.q + G.L;
   for (size_t i = 0; i < G.L + G.K; ++i) {
     uint64_t f[5];
-    ace_modulus(G.ctx, i, f);
+    ace_modulus(RT_CTX, i, f);
     G.q[i]._val     = (int64_t)f[0];
     G.q[i]._br_k    = (int64_t)f[1];
     G.q[i]._br_m    = (int64_t)f[2];
     G.q[i]._prec128 = ((unsigned __int128)f[4] << 64) | f[3];
   }
   if (Get_rt_data_info && Get_rt_data_info()) Pt_mgr_init(Get_rt_data_info()->_file_name);
-  clock_gettime(CLOCK_MONOTONIC, &G.t0);
 }
 
 static void free_key(SWITCH_KEY* k) {
   if (!k->_public_keys) return;
-  ace_free(G.ctx, k->_public_keys->dev);
+  ace_free(RT_CTX, k->_public_keys->dev);
   free(k->_public_keys);
   k->_public_keys = NULL;
 }
@@ -73,21 +121,36 @@ static void free_slots(IO_SLOT* s, size_t n) {
 }
 
 void Finalize_context(void) {
-  if (!G.ctx) return;
+  if (!G.root) return;
   Pt_mgr_fini(); /* always: the kept plaintexts are device buffers of this context */
   Rt_bootstrap_finalize();
   Rt_ckks_finalize();
   free_key(&G.relin);
   for (size_t i = 0; i < G.n_rot; ++i) {
-    free_key(&G.rot[i].swk);
-    ace_free(G.ctx, G.rot[i].order);
+    free_key(&G.rot[i]->swk);
+    ace_free(RT_CTX, G.rot[i]->order);
   }
+  for (size_t i = 0; i < G.n_rot; ++i) free(G.rot[i]);
   free(G.rot);
-  free_slots(G.in, G.n_in);
-  free_slots(G.out, G.n_out);
+  /* the other threads' lanes first: their contexts use the root's tables */
+  for (size_t i = N_lanes; i-- > 0;) {
+    struct rt_lane* l = Lanes[i];
+    Rt_lane           = l; /* the slots' polynomials go back through the lane that holds them */
+    free_slots(l->in, l->n_in);
+    free_slots(l->out, l->n_out);
+    if (l->ctx != G.root) ace_ctx_destroy(l->ctx);
+    if (i) free(l);
+  }
+  Rt_lane = NULL;
+  if (N_lanes) free(Lanes[0]);
+  free(Lanes);
+  Lanes   = NULL;
+  N_lanes = Cap_lanes = 0;
   free(G.q);
-  ace_ctx_destroy(G.ctx);
+  ace_ctx_destroy(G.root);
+  uint64_t generation = G.generation;
   memset(&G, 0, sizeof(G));
+  G.generation = generation;
   Report_rtlib_timing(); /* ckks_context.c:207-210: the table of times, if the environment asks for one */
   Close_trace_file();
 }
@@ -105,15 +168,15 @@ uint32_t Degree(void) { return G.N; }
 size_t   Get_q_cnt(void) { return G.L; }
 size_t   Get_p_cnt(void) { return G.K; }
 size_t   Get_q_parts(void) { return G.parts; }
-CRT_CONTEXT* Get_crt_context(void) { return G.ctx; }
-NTT_CONTEXT* Get_ntt_ctx(void) { return G.ctx; }
-size_t       Get_part_size(void) { return G.ctx ? ace_part_size(G.ctx) : 0; }
+CRT_CONTEXT* Get_crt_context(void) { return G.root; }
+NTT_CONTEXT* Get_ntt_ctx(void) { return G.root; }
+size_t       Get_part_size(void) { return G.root ? ace_part_size(G.root) : 0; }
 MODULUS* Q_modulus(void) { return G.q; }
 MODULUS* P_modulus(void) { return G.p; }
 double   Get_default_sc(void) { return G.sc; }
 size_t   Rt_num_decomp(size_t level) {
   NEED_CTX();
-  return ace_num_decomp(G.ctx, level);
+  return ace_num_decomp(RT_CTX, level);
 }
 
 /* prime index of a MODULUS the program took from Q_modulus() / P_modulus() */
@@ -125,39 +188,39 @@ static size_t prime_of(const MODULUS* m) {
 /* ---- device memory --------------------------------------------------------------- */
 int64_t* Rt_dev_alloc(size_t n_words) {
   NEED_CTX();
-  int64_t* p = ace_alloc(G.ctx, n_words);
+  int64_t* p = ace_alloc(RT_CTX, n_words);
   if (!p) Rt_fatal(__FILE__, __LINE__, "device allocation of %zu words failed: %s", n_words, ace_last_error());
   return p;
 }
 void Rt_sync(void) {
   NEED_CTX();
-  ACE_OK(ace_sync(G.ctx));
+  ACE_OK(ace_sync(RT_CTX));
 }
 int64_t* Rt_dev_alloc_raw(size_t n_words) { /* not zero-filled: for buffers written before they are read */
   NEED_CTX();
-  int64_t* p = ace_alloc_uninit(G.ctx, n_words);
+  int64_t* p = ace_alloc_uninit(RT_CTX, n_words);
   if (!p) Rt_fatal(__FILE__, __LINE__, "device allocation of %zu words failed: %s", n_words, ace_last_error());
   return p;
 }
-void Rt_copy_words(int64_t* dst, const int64_t* src, size_t n_words) { ACE_OK(ace_copy(G.ctx, dst, src, n_words)); }
+void Rt_copy_words(int64_t* dst, const int64_t* src, size_t n_words) { ACE_OK(ace_copy(RT_CTX, dst, src, n_words)); }
 void Rt_dev_free(int64_t* p) {
-  if (p && G.ctx) ace_free(G.ctx, p);
+  if (p && G.root) ace_free(RT_CTX, p);
 }
-void Rt_dev_copy(int64_t* dst, const int64_t* src, size_t n_words) { ACE_OK(ace_copy(G.ctx, dst, src, n_words)); }
+void Rt_dev_copy(int64_t* dst, const int64_t* src, size_t n_words) { ACE_OK(ace_copy(RT_CTX, dst, src, n_words)); }
 
 size_t Rt_p_offset(POLY p) { return (p->_num_alloc_primes - p->_num_primes_p) * (size_t)p->_ring_degree; }
 
 void Rt_upload_poly(POLY dst, const int64_t* host) {
   size_t n = dst->_ring_degree;
-  ACE_OK(ace_upload(G.ctx, dst->_data, host, dst->_num_primes * n));
+  ACE_OK(ace_upload(RT_CTX, dst->_data, host, dst->_num_primes * n));
   if (dst->_num_primes_p)
-    ACE_OK(ace_upload(G.ctx, dst->_data + Rt_p_offset(dst), host + dst->_num_primes * n, dst->_num_primes_p * n));
+    ACE_OK(ace_upload(RT_CTX, dst->_data + Rt_p_offset(dst), host + dst->_num_primes * n, dst->_num_primes_p * n));
 }
 void Rt_download_poly(int64_t* host, POLY src) {
   size_t n = src->_ring_degree;
-  ACE_OK(ace_download(G.ctx, host, src->_data, src->_num_primes * n));
+  ACE_OK(ace_download(RT_CTX, host, src->_data, src->_num_primes * n));
   if (src->_num_primes_p)
-    ACE_OK(ace_download(G.ctx, host + src->_num_primes * n, src->_data + Rt_p_offset(src), src->_num_primes_p * n));
+    ACE_OK(ace_download(RT_CTX, host + src->_num_primes * n, src->_data + Rt_p_offset(src), src->_num_primes_p * n));
 }
 
 /* ---- polynomial containers --------------------------------------------------------- */
@@ -200,7 +263,7 @@ void Init_poly(POLY res, POLY like) {
   if (!res->_data) {
     Alloc_poly_data(res, n, nq, np);
   } else {
-    ACE_OK(ace_zero(G.ctx, res->_data, Get_poly_alloc_len(res)));
+    ACE_OK(ace_zero(RT_CTX, res->_data, Get_poly_alloc_len(res)));
     res->_num_primes   = nq;
     res->_num_primes_p = np;
   }
@@ -241,13 +304,13 @@ static void need_packed_ext(POLY p, const char* who) {
 
 /* ---- key switching pieces ------------------------------------------------------------ */
 static size_t digit_len(size_t level, uint32_t part) {
-  size_t ps = ace_part_size(G.ctx), nd = ace_num_decomp(G.ctx, level);
+  size_t ps = ace_part_size(RT_CTX), nd = ace_num_decomp(RT_CTX, level);
   FMT_ASSERT(part < nd, "digit index %u out of range (%zu digits at level %zu)", part, nd, level);
   return part == nd - 1 ? level - ps * part : ps;
 }
 
 POLY Decomp(POLY res, POLY poly, uint32_t part) {
-  size_t   level = poly->_num_primes, len = digit_len(level, part), start = ace_part_size(G.ctx) * part;
+  size_t   level = poly->_num_primes, len = digit_len(level, part), start = ace_part_size(RT_CTX) * part;
   uint32_t n = poly->_ring_degree;
   if (res->_num_alloc_primes < len) {
     Free_poly_data(res);
@@ -266,7 +329,7 @@ POLY Mod_up(POLY res, POLY digit, uint32_t part) {
   size_t level = res->_num_primes;
   FMT_ASSERT(digit->_ring_degree == res->_ring_degree && digit->_num_primes == digit_len(level, part),
              "Mod_up: digit size does not match part %u at level %zu", part, level);
-  ACE_OK(ace_mod_up(G.ctx, res->_data, digit->_data, level, part, digit->_is_ntt));
+  ACE_OK(ace_mod_up(RT_CTX, res->_data, digit->_data, level, part, digit->_is_ntt));
   res->_is_ntt = digit->_is_ntt;
   return res;
 }
@@ -275,7 +338,7 @@ POLY Decomp_modup(POLY res, POLY poly, uint32_t part) {
   need_packed_ext(res, "Decomp_modup");
   FMT_ASSERT(res->_num_primes == poly->_num_primes && res->_ring_degree == poly->_ring_degree,
              "Decomp_modup: result size not match");
-  ACE_OK(ace_decomp_modup(G.ctx, res->_data, poly->_data, poly->_num_primes, part, poly->_is_ntt));
+  ACE_OK(ace_decomp_modup(RT_CTX, res->_data, poly->_data, poly->_num_primes, part, poly->_is_ntt));
   res->_is_ntt = poly->_is_ntt;
   return res;
 }
@@ -285,7 +348,7 @@ POLY Mod_down(POLY res, POLY poly) {
   need_packed_ext(poly, "Mod_down");
   FMT_ASSERT(res->_ring_degree == poly->_ring_degree && res->_num_primes == poly->_num_primes,
              "Mod_down: result size not match");
-  ACE_OK(ace_mod_down(G.ctx, res->_data, poly->_data, poly->_num_primes, poly->_is_ntt));
+  ACE_OK(ace_mod_down(RT_CTX, res->_data, poly->_data, poly->_num_primes, poly->_is_ntt));
   res->_is_ntt = poly->_is_ntt;
   return res;
 }
@@ -302,7 +365,7 @@ POLY Rescale(POLY res, POLY poly) {
   size_t level = poly->_num_primes;
   FMT_ASSERT(level >= 2, "Level of rescale opnd is too small");
   FMT_ASSERT(res->_num_primes == level && res->_ring_degree == poly->_ring_degree, "Rescale: primes not match");
-  ACE_OK(ace_rescale(G.ctx, res->_data, poly->_data, level, poly->_is_ntt));
+  ACE_OK(ace_rescale(RT_CTX, res->_data, poly->_data, level, poly->_is_ntt));
   res->_is_ntt = poly->_is_ntt;
   Set_poly_level(res, level - 1); /* the dropped limb stays allocated, as in the reference */
   return res;
@@ -313,7 +376,7 @@ POLY Mod_down_rescale(POLY res, POLY poly) {
   size_t level = poly->_num_primes;
   FMT_ASSERT(res->_ring_degree == poly->_ring_degree && res->_num_primes == level && level > 1 && res->_num_primes_p == 0,
              "Reduce_and_rescale_rns: size not match");
-  ACE_OK(ace_mod_down_rescale(G.ctx, res->_data, poly->_data, level, poly->_is_ntt));
+  ACE_OK(ace_mod_down_rescale(RT_CTX, res->_data, poly->_data, level, poly->_is_ntt));
   poly->_is_ntt = false;
   Set_poly_level(res, level - 1);
   res->_is_ntt = true;
@@ -323,12 +386,12 @@ POLY Mod_down_rescale(POLY res, POLY poly) {
 void Transform_values_from_level0(POLY res, POLY poly) {
   FMT_ASSERT(res->_ring_degree == poly->_ring_degree, "unmatched ring degree");
   FMT_ASSERT(Get_poly_alloc_len(res) >= Get_poly_len(poly) && res->_num_alloc_primes <= G.L, "not enough memory");
-  ACE_OK(ace_transform_from_level0(G.ctx, res->_data, poly->_data, res->_num_primes));
+  ACE_OK(ace_transform_from_level0(RT_CTX, res->_data, poly->_data, res->_num_primes));
 }
 
 POLY_ARR Precomp(POLY_ARR res, size_t size, POLY input) {
   size_t level = input->_num_primes, T = level + G.K;
-  FMT_ASSERT(size == ace_num_decomp(G.ctx, level), "length of precompute not match");
+  FMT_ASSERT(size == ace_num_decomp(RT_CTX, level), "length of precompute not match");
   bool slab = true;
   for (size_t d = 0; d < size; ++d) {
     need_packed_ext(&res[d], "Precomp");
@@ -336,10 +399,10 @@ POLY_ARR Precomp(POLY_ARR res, size_t size, POLY input) {
     if (res[d]._data != res[0]._data + d * T * (size_t)G.N) slab = false;
   }
   if (slab) {
-    ACE_OK(ace_precomp(G.ctx, res[0]._data, input->_data, level, input->_is_ntt));
+    ACE_OK(ace_precomp(RT_CTX, res[0]._data, input->_data, level, input->_is_ntt));
   } else {
     for (size_t d = 0; d < size; ++d)
-      ACE_OK(ace_decomp_modup(G.ctx, res[d]._data, input->_data, level, d, input->_is_ntt));
+      ACE_OK(ace_decomp_modup(RT_CTX, res[d]._data, input->_data, level, d, input->_is_ntt));
   }
   for (size_t d = 0; d < size; ++d) res[d]._is_ntt = input->_is_ntt;
   return res;
@@ -367,13 +430,13 @@ POLY Dot_prod(POLY res, POLY_ARR digits, POLY_ARR key, uint32_t size) {
   }
   if (slab) {
     size_t stride = size > 1 ? (size_t)(key[1]._data - key[0]._data) : 0;
-    ACE_OK(ace_dot_prod(G.ctx, res->_data, digits[0]._data, key[0]._data, stride, size, level));
+    ACE_OK(ace_dot_prod(RT_CTX, res->_data, digits[0]._data, key[0]._data, stride, size, level));
   } else { /* operands scattered: accumulate digit by digit, limb by limb */
-    ACE_OK(ace_zero(G.ctx, res->_data, T * n));
+    ACE_OK(ace_zero(RT_CTX, res->_data, T * n));
     for (uint32_t d = 0; d < size; ++d) {
       for (size_t t = 0; t < T; ++t) {
         size_t kl = t < level ? t : G.L + (t - level), pi = kl; /* key limb == prime index */
-        ACE_OK(ace_hw_modmuladd(G.ctx, res->_data + t * n, digits[d]._data + t * n, key[d]._data + kl * n, pi, n));
+        ACE_OK(ace_hw_modmuladd(RT_CTX, res->_data + t * n, digits[d]._data + t * n, key[d]._data + kl * n, pi, n));
       }
     }
   }
@@ -384,7 +447,7 @@ POLY Dot_prod(POLY res, POLY_ARR digits, POLY_ARR key, uint32_t size) {
 POLY Extend(POLY res, POLY poly) {
   FMT_ASSERT(res->_ring_degree == poly->_ring_degree && res->_num_primes == poly->_num_primes, "Extend: size not match");
   FMT_ASSERT(res->_num_alloc_primes == poly->_num_primes + G.K, "Extend: alloc_size not match");
-  ACE_OK(ace_extend(G.ctx, res->_data, poly->_data, poly->_num_primes));
+  ACE_OK(ace_extend(RT_CTX, res->_data, poly->_data, poly->_num_primes));
   res->_num_primes_p = G.K;
   res->_is_ntt       = poly->_is_ntt;
   return res;
@@ -396,16 +459,16 @@ static void transform_inplace(POLY poly, bool inverse) {
   FMT_ASSERT(l + k <= 128, "too many limbs");
   for (size_t i = 0; i < l; ++i) idx[i] = (int32_t)i;
   if (inverse)
-    ACE_OK(ace_intt(G.ctx, poly->_data, poly->_data, idx, l, 1, 0));
+    ACE_OK(ace_intt(RT_CTX, poly->_data, poly->_data, idx, l, 1, 0));
   else
-    ACE_OK(ace_ntt(G.ctx, poly->_data, poly->_data, idx, l, 1, 0));
+    ACE_OK(ace_ntt(RT_CTX, poly->_data, poly->_data, idx, l, 1, 0));
   if (k) {
     for (size_t j = 0; j < k; ++j) idx[j] = (int32_t)(G.L + j);
     int64_t* p = poly->_data + Rt_p_offset(poly);
     if (inverse)
-      ACE_OK(ace_intt(G.ctx, p, p, idx, k, 1, 0));
+      ACE_OK(ace_intt(RT_CTX, p, p, idx, k, 1, 0));
     else
-      ACE_OK(ace_ntt(G.ctx, p, p, idx, k, 1, 0));
+      ACE_OK(ace_ntt(RT_CTX, p, p, idx, k, 1, 0));
   }
   (void)n;
   poly->_is_ntt = !inverse;
@@ -425,14 +488,14 @@ static POLY poly_ew(poly_ew_fn fn, const char* who, POLY res, POLY a, POLY b) {
              "%s: size not match", who);
   FMT_ASSERT(a->_is_ntt == b->_is_ntt, "%s: operands in different forms", who);
   size_t level = a->_num_primes, n = a->_ring_degree, k = a->_num_primes_p < b->_num_primes_p ? a->_num_primes_p : b->_num_primes_p;
-  ACE_OK(fn(G.ctx, res->_data, a->_data, b->_data, level, 0));
+  ACE_OK(fn(RT_CTX, res->_data, a->_data, b->_data, level, 0));
   if (k) { /* P limbs of each operand sit at its own offset */
     FMT_ASSERT(k == G.K && res->_num_primes_p == G.K, "%s: p primes not match", who);
     for (size_t j = 0; j < k; ++j) {
       int64_t *r = res->_data + Rt_p_offset(res) + j * n, *x = a->_data + Rt_p_offset(a) + j * n, *y = b->_data + Rt_p_offset(b) + j * n;
-      if (fn == ace_poly_add) ACE_OK(ace_hw_modadd(G.ctx, r, x, y, G.L + j, n));
-      else if (fn == ace_poly_sub) ACE_OK(ace_hw_modsub(G.ctx, r, x, y, G.L + j, n));
-      else ACE_OK(ace_hw_modmul(G.ctx, r, x, y, G.L + j, n));
+      if (fn == ace_poly_add) ACE_OK(ace_hw_modadd(RT_CTX, r, x, y, G.L + j, n));
+      else if (fn == ace_poly_sub) ACE_OK(ace_hw_modsub(RT_CTX, r, x, y, G.L + j, n));
+      else ACE_OK(ace_hw_modmul(RT_CTX, r, x, y, G.L + j, n));
     }
   }
   res->_is_ntt = a->_is_ntt;
@@ -450,7 +513,7 @@ POLY Mul_poly(POLY res, POLY a, POLY b) {
 /* ---- HAL ------------------------------------------------------------------------------- */
 #define HW2(NAME, FN)                                                                       \
   int64_t* NAME(int64_t* res, int64_t* a, int64_t* b, MODULUS* m, uint32_t degree) {        \
-    ACE_OK(FN(G.ctx, res, a, b, prime_of(m), degree));                                      \
+    ACE_OK(FN(RT_CTX, res, a, b, prime_of(m), degree));                                      \
     return res + degree;                                                                    \
   }
 #define HW1(NAME, FN)                                                                       \
@@ -458,7 +521,7 @@ POLY Mul_poly(POLY res, POLY a, POLY b) {
     int64_t q = m->_val;                                                                    \
     s %= q;                                                                                 \
     if (s < 0) s += q;                                                                      \
-    ACE_OK(FN(G.ctx, res, a, s, prime_of(m), degree));                                      \
+    ACE_OK(FN(RT_CTX, res, a, s, prime_of(m), degree));                                      \
     return res + degree;                                                                    \
   }
 HW2(Hw_modadd, ace_hw_modadd)
@@ -471,18 +534,18 @@ HW1(Hw_modmul_scalar, ace_hw_modmul_scalar)
 HW1(Hw_modmuladd_scalar, ace_hw_modmuladd_scalar)
 
 int64_t* Hw_rotate(int64_t* res, int64_t* a, int64_t* order, MODULUS* m, uint32_t degree) {
-  ACE_OK(ace_hw_rotate(G.ctx, res, a, order, prime_of(m), degree));
+  ACE_OK(ace_hw_rotate(RT_CTX, res, a, order, prime_of(m), degree));
   return res + degree;
 }
 void Hw_ntt(int64_t* res, int64_t* a, size_t prime_idx, uint32_t degree) {
   int32_t idx = (int32_t)prime_idx;
   FMT_ASSERT(degree == G.N, "Hw_ntt: degree not match");
-  ACE_OK(ace_ntt(G.ctx, res, a, &idx, 1, 1, 0));
+  ACE_OK(ace_ntt(RT_CTX, res, a, &idx, 1, 1, 0));
 }
 void Hw_intt(int64_t* res, int64_t* a, size_t prime_idx, uint32_t degree) {
   int32_t idx = (int32_t)prime_idx;
   FMT_ASSERT(degree == G.N, "Hw_intt: degree not match");
-  ACE_OK(ace_intt(G.ctx, res, a, &idx, 1, 1, 0));
+  ACE_OK(ace_intt(RT_CTX, res, a, &idx, 1, 1, 0));
 }
 
 /* ---- keys --------------------------------------------------------------------------------- */
@@ -499,18 +562,23 @@ void Rt_install_key_dev(SWITCH_KEY* k, int64_t* dev) {
     v._data += T * n;
     kp->pk[d]._p1 = v;
   }
-  k->_public_keys = kp;
+  Rt_shared_publish(); /* other threads read the key on their own streams as soon as they can see it */
+  __atomic_store_n(&k->_public_keys, kp, __ATOMIC_RELEASE);
 }
 void Rt_install_key(SWITCH_KEY* k, const int64_t* host) {
   size_t   words = 2 * G.parts * (G.L + G.K) * G.N;
   int64_t* dev   = Rt_dev_alloc_raw(words);
-  ACE_OK(ace_upload(G.ctx, dev, host, words));
+  ACE_OK(ace_upload(RT_CTX, dev, host, words));
   Rt_install_key_dev(k, dev);
 }
 
+/* Entries are made one at a time (under the shared lock where threads may race for a key) and never move: the
+ * table of pointers has a fixed size, an entry is complete before the count that makes it visible goes up. */
+#define RT_MAX_ROT_KEYS 8192
 ROT_KEY* Rt_find_rot(int32_t rot_idx) {
-  for (size_t i = 0; i < G.n_rot; ++i)
-    if (G.rot[i].rot_idx == rot_idx) return &G.rot[i];
+  size_t n = __atomic_load_n(&G.n_rot, __ATOMIC_ACQUIRE);
+  for (size_t i = 0; i < n; ++i)
+    if (G.rot[i]->rot_idx == rot_idx) return G.rot[i];
   return NULL;
 }
 
@@ -518,16 +586,20 @@ ROT_KEY* Rt_find_rot(int32_t rot_idx) {
 ROT_KEY* Rt_rot_entry(int32_t rot_idx) {
   ROT_KEY* r = Rt_find_rot(rot_idx);
   if (r) return r;
-  if (G.n_rot == G.cap_rot) {
-    G.cap_rot = G.cap_rot ? 2 * G.cap_rot : 16;
-    G.rot     = (ROT_KEY*)realloc(G.rot, G.cap_rot * sizeof(ROT_KEY));
+  Rt_shared_lock();
+  r = Rt_find_rot(rot_idx);
+  if (!r) {
+    if (!G.rot) G.rot = (ROT_KEY**)calloc(RT_MAX_ROT_KEYS, sizeof(ROT_KEY*));
+    FMT_ASSERT(G.n_rot < RT_MAX_ROT_KEYS, "more than %d rotation keys", RT_MAX_ROT_KEYS);
+    r           = (ROT_KEY*)calloc(1, sizeof(*r));
+    r->rot_idx  = rot_idx;
+    r->auto_idx = (uint32_t)rot_idx == 2 * G.N - 1 ? 2 * G.N - 1 : ace_find_automorphism_index(RT_CTX, rot_idx);
+    r->order    = Rt_dev_alloc(G.N);
+    ACE_OK(ace_automorphism_order(RT_CTX, r->order, r->auto_idx, 1)); /* waits for the upload */
+    G.rot[G.n_rot] = r;
+    __atomic_store_n(&G.n_rot, G.n_rot + 1, __ATOMIC_RELEASE);
   }
-  r = &G.rot[G.n_rot++];
-  memset(r, 0, sizeof(*r));
-  r->rot_idx  = rot_idx;
-  r->auto_idx = (uint32_t)rot_idx == 2 * G.N - 1 ? 2 * G.N - 1 : ace_find_automorphism_index(G.ctx, rot_idx);
-  r->order    = Rt_dev_alloc(G.N);
-  ACE_OK(ace_automorphism_order(G.ctx, r->order, r->auto_idx, 1));
+  Rt_shared_unlock();
   return r;
 }
 
@@ -704,7 +776,7 @@ CIPHER3 Mul_ciph3(CIPHER3 res, CIPHER a, CIPHER b) {
   Init_ciph3_up_scale(res, a, b);
   size_t l = res->_c0_poly._num_primes;
   FMT_ASSERT(a->_c0_poly._is_ntt && b->_c0_poly._is_ntt, "Mul_ciph3: operands must be in NTT form");
-  ACE_OK(ace_mul_ciph3(G.ctx, res->_c0_poly._data, res->_c1_poly._data, res->_c2_poly._data, a->_c0_poly._data,
+  ACE_OK(ace_mul_ciph3(RT_CTX, res->_c0_poly._data, res->_c1_poly._data, res->_c2_poly._data, a->_c0_poly._data,
                        a->_c1_poly._data, b->_c0_poly._data, b->_c1_poly._data, l));
   return res;
 }
@@ -712,7 +784,7 @@ CIPHER3 Mul_ciph3(CIPHER3 res, CIPHER a, CIPHER b) {
 CIPHER Relin(CIPHER res, CIPHER3 c) {
   FMT_ASSERT(G.relin._public_keys, "no relinearisation key loaded");
   Init_ciph_same_scale_ciph3(res, c);
-  ACE_OK(ace_relin(G.ctx, res->_c0_poly._data, res->_c1_poly._data, c->_c0_poly._data, c->_c1_poly._data,
+  ACE_OK(ace_relin(RT_CTX, res->_c0_poly._data, res->_c1_poly._data, c->_c0_poly._data, c->_c1_poly._data,
                    c->_c2_poly._data, G.relin._public_keys->dev, c->_c0_poly._num_primes));
   return res;
 }
@@ -734,7 +806,7 @@ CIPHER Rescale_ciph(CIPHER res, CIPHER c) {
   double   sf  = c->_scaling_factor / G.sc;
   uint32_t deg = c->_sf_degree - 1;
   Rt_shape_ciph(res, c, sf, deg);
-  ACE_OK(ace_rescale_ciph(G.ctx, res->_c0_poly._data, res->_c1_poly._data, c->_c0_poly._data, c->_c1_poly._data, level));
+  ACE_OK(ace_rescale_ciph(RT_CTX, res->_c0_poly._data, res->_c1_poly._data, c->_c0_poly._data, c->_c1_poly._data, level));
   Set_poly_level(&res->_c0_poly, level - 1);
   Set_poly_level(&res->_c1_poly, level - 1);
   return res;
@@ -761,7 +833,7 @@ void Rotate_batch_ciph(CIPHER res_arr, CIPHER c, const int32_t* rot_idx, uint32_
   }
   if (m) {
     int64_t *s0 = Rt_dev_alloc(m * level * n), *s1 = Rt_dev_alloc(m * level * n);
-    ACE_OK(ace_rotate_batch(G.ctx, s0, s1, c->_c0_poly._data, c->_c1_poly._data, keys, orders, m, level));
+    ACE_OK(ace_rotate_batch(RT_CTX, s0, s1, c->_c0_poly._data, c->_c1_poly._data, keys, orders, m, level));
     for (uint32_t j = 0; j < m; ++j) {
       CIPHER out = &res_arr[where[j]];
       Rt_shape_ciph(out, c, c->_scaling_factor, c->_sf_degree);
@@ -812,7 +884,7 @@ void Rt_set_input(const char* name, size_t idx, const int64_t* c0, const int64_t
                   uint32_t sf_degree, uint32_t slots) {
   NEED_CTX();
   FMT_ASSERT(level >= 1 && level <= G.L, "Rt_set_input: level out of range");
-  IO_SLOT*    s  = Rt_add_slot(&G.in, &G.n_in, name, idx);
+  IO_SLOT*    s  = Rt_add_slot(&LANE.in, &LANE.n_in, name, idx);
   CIPHERTEXT* ct = (CIPHERTEXT*)calloc(1, sizeof(CIPHERTEXT));
   Alloc_poly_data(&ct->_c0_poly, G.N, level, 0);
   Alloc_poly_data(&ct->_c1_poly, G.N, level, 0);
@@ -826,7 +898,7 @@ void Rt_set_input(const char* name, size_t idx, const int64_t* c0, const int64_t
 }
 
 CIPHERTEXT Get_input_data(const char* name, size_t idx) {
-  IO_SLOT* s = Rt_find_slot(G.in, G.n_in, name, idx);
+  IO_SLOT* s = Rt_find_slot(LANE.in, LANE.n_in, name, idx);
   FMT_ASSERT(s && s->ct, "not find data: input \"%s\"[%zu]", name, idx);
   CIPHERTEXT ret = *s->ct; /* ownership of the polynomials moves to the program */
   free(s->ct);
@@ -835,7 +907,7 @@ CIPHERTEXT Get_input_data(const char* name, size_t idx) {
 }
 
 void Set_output_data(const char* name, size_t idx, CIPHER data) {
-  IO_SLOT*    s  = Rt_add_slot(&G.out, &G.n_out, name, idx);
+  IO_SLOT*    s  = Rt_add_slot(&LANE.out, &LANE.n_out, name, idx);
   CIPHERTEXT* ct = (CIPHERTEXT*)calloc(1, sizeof(CIPHERTEXT));
   Copy_ciph(ct, data);
   Free_ciph_poly(data, 1);
@@ -843,7 +915,7 @@ void Set_output_data(const char* name, size_t idx, CIPHER data) {
 }
 
 size_t Rt_get_output(const char* name, size_t idx, int64_t* c0, int64_t* c1, CIPHERTEXT* meta) {
-  IO_SLOT* s = Rt_find_slot(G.out, G.n_out, name, idx);
+  IO_SLOT* s = Rt_find_slot(LANE.out, LANE.n_out, name, idx);
   if (!s || !s->ct) return 0;
   if (c0) Rt_download_poly(c0, &s->ct->_c0_poly);
   if (c1) Rt_download_poly(c1, &s->ct->_c1_poly);
@@ -858,13 +930,13 @@ size_t Rt_get_output(const char* name, size_t idx, int64_t* c0, int64_t* c1, CIP
 static double since_start(void) {
   struct timespec t;
   clock_gettime(CLOCK_MONOTONIC, &t);
-  return (double)(t.tv_sec - G.t0.tv_sec) + 1e-9 * (double)(t.tv_nsec - G.t0.tv_nsec);
+  return (double)(t.tv_sec - LANE.t0.tv_sec) + 1e-9 * (double)(t.tv_nsec - LANE.t0.tv_nsec);
 }
 void Tm_start(const char* msg) {
-  clock_gettime(CLOCK_MONOTONIC, &G.t0);
+  clock_gettime(CLOCK_MONOTONIC, &LANE.t0);
   if (msg) printf("[RT_STAT] %s: timer started\n", msg);
 }
 void Tm_taken(const char* msg) {
-  if (G.ctx) (void)ace_sync(G.ctx); /* the stream is asynchronous: wait, so the figure covers the work */
+  if (G.root) (void)ace_sync(RT_CTX); /* the stream is asynchronous: wait, so the figure covers the work */
   printf("[RT_STAT] %s: %.6f s\n", msg ? msg : "", since_start());
 }

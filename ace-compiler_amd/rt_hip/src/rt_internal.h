@@ -26,18 +26,17 @@ typedef struct {
   CIPHERTEXT* ct;
 } IO_SLOT;
 
+/* What the threads of a program share: the root context (tables in HBM), the parameters and the keys. */
 struct rt_state {
-  ace_ctx* ctx;
+  ace_ctx* root; /* made by Prepare_context; the thread that called it issues on it */
+  uint64_t generation; /* counts Prepare_context calls: a thread's lane of an earlier context is stale */
   uint32_t N;
   size_t   L, K, parts, input_level;
   MODULUS *q, *p;
   double   sc;
   SWITCH_KEY relin;
-  ROT_KEY*   rot;
-  size_t     n_rot, cap_rot;
-  IO_SLOT *in, *out;
-  size_t   n_in, n_out;
-  struct timespec t0;
+  ROT_KEY**  rot; /* entries never move once made (Rt_find_rot is read by every thread) */
+  size_t     n_rot;
   /* key material of Rt_generate_keys (rt_ckks.c); absent when the harness loads keys itself */
   int64_t* secret_small; /* host: N signed coefficients */
   int64_t* secret_ntt;   /* device: (L+k) limbs */
@@ -45,11 +44,40 @@ struct rt_state {
 };
 extern struct rt_state G;
 
+/* What every host thread has for itself, as the reference's OpenMP build keeps its I/O tables, timers and
+ * generator per thread (common/src/io_lib.c:24-27, include/common/rtlib_timing.h:123-126, util/src/prng.c:13-16):
+ * a context of the root's family (its own HIP stream, scratch arena, buffer pool and recorded calls), the named
+ * input and output ciphertexts, the stopwatch of Tm_start.  A thread other than Prepare_context's gets its lane
+ * the first time it calls into the runtime; Finalize_context destroys them all. */
+struct rt_lane {
+  ace_ctx* ctx;
+  uint64_t generation;
+  unsigned ordinal; /* 0: the thread of Prepare_context */
+  IO_SLOT *in, *out;
+  size_t   n_in, n_out;
+  struct timespec t0;
+};
+extern __thread struct rt_lane* Rt_lane;
+struct rt_lane* Rt_lane_slow(void);
+size_t          Rt_lane_count(void); /* threads that have called into the runtime since Prepare_context */
+static inline struct rt_lane* Rt_this_lane(void) {
+  struct rt_lane* l = Rt_lane;
+  return (l && l->generation == G.generation) ? l : Rt_lane_slow();
+}
+#define RT_CTX (Rt_this_lane()->ctx)
+#define LANE (*Rt_this_lane())
+/* setting up what all threads share after the first use (rotation keys made on demand, the bootstrap's plaintext
+ * diagonals and monomials, kept weight plaintexts): one thread at a time, and what it built is complete on the
+ * device (Rt_shared_publish) before the lock is released, because the other threads read it on their own streams */
+void Rt_shared_lock(void);
+void Rt_shared_unlock(void);
+void Rt_shared_publish(void); /* waits for the calling thread's stream */
+
 #define ACE_OK(call)                                                       \
   do {                                                                     \
     if ((call) != 0) Rt_fatal(__FILE__, __LINE__, "%s", ace_last_error()); \
   } while (0)
-#define NEED_CTX() FMT_ASSERT(G.ctx, "Prepare_context() has not run")
+#define NEED_CTX() FMT_ASSERT(G.root, "Prepare_context() has not run")
 
 size_t   Rt_p_offset(POLY p);
 int64_t* Rt_dev_alloc_raw(size_t n_words);

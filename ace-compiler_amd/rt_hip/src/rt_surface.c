@@ -61,7 +61,7 @@ POLY Init_poly_by_opnd(POLY res, POLY opnd1, POLY opnd2, bool is_ext) {
 void Set_coeff_at(POLY p, int64_t val, uint32_t idx) {
   FMT_ASSERT(p, "null poly");
   FMT_ASSERT(idx < Get_poly_alloc_len(p), "idx outof bound");
-  ACE_OK(ace_upload(G.ctx, p->_data + idx, &val, 1));
+  ACE_OK(ace_upload(RT_CTX, p->_data + idx, &val, 1));
 }
 
 static int64_t* download_whole(POLY p) {
@@ -105,7 +105,7 @@ void Sample_uniform_poly(POLY p) {
   uint64_t    seed = env ? strtoull(env, NULL, 0) : 0;
   if (!seed) /* from the operating system, like the keys: a caller may use the polynomial as a mask */
     FMT_ASSERT(getrandom(&seed, sizeof(seed), 0) == (ssize_t)sizeof(seed), "Sample_uniform_poly: getrandom failed");
-  ACE_OK(ace_sample_uniform(G.ctx, p->_data, Poly_level(p), Num_p(p) != 0, seed, ++Sample_stream));
+  ACE_OK(ace_sample_uniform(RT_CTX, p->_data, Poly_level(p), Num_p(p) != 0, seed, __atomic_add_fetch(&Sample_stream, 1, __ATOMIC_RELAXED)));
 }
 void Sample_ternary_poly(POLY p, size_t hamming_weight) {
   NEED_CTX();
@@ -114,7 +114,7 @@ void Sample_ternary_poly(POLY p, size_t hamming_weight) {
   size_t   n = p->_ring_degree;
   int64_t* v = (int64_t*)calloc(n, sizeof(int64_t));
   Rt_sample_ternary(v, n, hamming_weight);
-  ACE_OK(ace_expand_small(G.ctx, p->_data, v, Poly_level(p), Num_p(p) != 0));
+  ACE_OK(ace_expand_small(RT_CTX, p->_data, v, Poly_level(p), Num_p(p) != 0));
   free(v);
 }
 
@@ -195,7 +195,7 @@ POLY Scalar_integer_multiply_poly(POLY res, POLY poly, int64_t scalar) {
 }
 POLY Scalars_integer_multiply_poly_qpart(POLY res, POLY poly, VALUE_LIST* scalars, size_t part_idx) {
   const int64_t* w  = list_words(scalars, res, false);
-  size_t         ps = ace_part_size(G.ctx), first = ps * part_idx, last = first + ps;
+  size_t         ps = ace_part_size(RT_CTX), first = ps * part_idx, last = first + ps;
   if (last > Poly_level(res)) last = Poly_level(res);
   return per_limb_scalars(Hw_modmul_scalar, res, poly, w, NULL, 0, first, last); /* the other limbs stay as they are */
 }
@@ -206,7 +206,7 @@ POLY Automorphism_transform(POLY res, POLY poly, VALUE_LIST* precomp) {
   FMT_ASSERT(precomp && LIST_LEN(precomp) == n, "invalid index table length");
   FMT_ASSERT(res->_data != poly->_data, "Automorphism_transform: res must not be the operand");
   int64_t* order = Rt_dev_alloc_raw(n);
-  ACE_OK(ace_upload(G.ctx, order, Get_i64_values(precomp), n));
+  ACE_OK(ace_upload(RT_CTX, order, Get_i64_values(precomp), n));
   for (size_t t = 0; t < Poly_level(res); ++t) Hw_rotate(Coeffs(res, t, n), Coeffs(poly, t, n), order, &G.q[t], n);
   for (size_t t = 0; t < Num_p(res); ++t)
     Hw_rotate(Get_p_coeffs(res) + t * (size_t)n, Get_p_coeffs(poly) + t * (size_t)n, order, &G.p[t], n);
@@ -235,7 +235,7 @@ void Set_poly_data(POLY poly, L_POLY lpoly, size_t idx) {
   FMT_ASSERT(idx < Get_num_pq(poly), "Set_poly_data_from_lpoly: idx overflow");
   Set_coeffs(poly, (uint32_t)idx, Get_rdgree(poly), Get_lpoly_coeffs(&lpoly));
 }
-void Zero_lpoly(LPOLY p) { ACE_OK(ace_zero(G.ctx, p->_data, p->_ring_degree)); }
+void Zero_lpoly(LPOLY p) { ACE_OK(ace_zero(RT_CTX, p->_data, p->_ring_degree)); }
 void Copy_lpoly(LPOLY res, L_POLY poly) {
   Rt_dev_copy(res->_data, poly._data, res->_ring_degree);
   res->_is_ntt = poly._is_ntt;
@@ -243,7 +243,7 @@ void Copy_lpoly(LPOLY res, L_POLY poly) {
 void Print_lpoly(FILE* fp, LPOLY p) {
   FMT_ASSERT(p, "null lpoly");
   int64_t* h = (int64_t*)malloc(p->_ring_degree * sizeof(int64_t));
-  ACE_OK(ace_download(G.ctx, h, p->_data, p->_ring_degree));
+  ACE_OK(ace_download(RT_CTX, h, p->_data, p->_ring_degree));
   fprintf(fp, "is_ntt: %s, raw data: \n", p->_is_ntt ? "Y" : "N");
   for (uint32_t j = 0; j < p->_ring_degree; ++j) fprintf(fp, "%ld ", (long)h[j]);
   fprintf(fp, "\n");

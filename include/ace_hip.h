@@ -40,6 +40,15 @@ ace_ctx* ace_ctx_create_with_primes(uint32_t degree, size_t num_q,
  * the context still holds every host-side table (primes, roots, cofactors) and
  * answers the getters below, but each call that would touch the GPU is
  * rejected with an error: there is no CPU fallback. */
+/* A further context over the same tables, for another host thread (the reference runs the images of a batch under
+ * `#pragma omp parallel for` with the CRT context shared and the I/O, timing and generator state per thread:
+ * dataset/resnet_cifar.main.inc:81-112, common/src/io_lib.c:24-27).  The new context shares the primes, twiddles and
+ * conversion tables of `ctx` in HBM and has its own HIP stream, scratch arena, buffer pool and recorded calls, so
+ * the two may be used from two threads at the same time; each context by itself is still used by one thread at a
+ * time.  Buffers are plain device pointers: any context of the family may read and write them (the caller orders
+ * uses on different contexts, e.g. with ace_sync) and ace_free accepts a buffer that a sibling's ace_alloc made.
+ * The contexts made this way must be destroyed before `ctx` is.  NULL without a HIP device. */
+ace_ctx*    ace_ctx_share(ace_ctx* ctx);
 void        ace_ctx_destroy(ace_ctx* ctx);
 int         ace_has_device(const ace_ctx* ctx);
 const char* ace_last_error(void);
@@ -105,6 +114,11 @@ int      ace_sync(ace_ctx* ctx);
 int      ace_fork(ace_ctx* ctx);
 int      ace_fork_switch(ace_ctx* ctx);
 int      ace_join(ace_ctx* ctx);
+/* Gives back the second stream with its scratch arena and kept buffers (made by the first ace_fork; the next
+ * ace_fork makes them again).  For a program that goes on with several contexts of a family on several threads:
+ * the hardware serves a process's streams through a few queues, and a stream that is no longer used still holds
+ * its place among them.  Rejected between ace_fork and ace_join. */
+int      ace_fork_release(ace_ctx* ctx);
 /* Device memory the context holds right now, in 64-bit words and buffers (no counterpart in the reference; for
  * tests that check that a call allocates nothing): out[0] = scratch arena of the current lane, out[1] = freed
  * buffers kept for reuse (words), out[2] = buffers handed out by ace_alloc and not yet freed, out[3] = freed buffers

@@ -846,6 +846,60 @@ def test_two_lanes_equal_one(pair):
     g.join()
 
 
+def test_contexts_of_a_family_on_two_threads(pair):
+    """ace_ctx_share: a second context over the same tables, used from another host thread at the same time as the
+    first: each thread's HMult + relinearise + rescale and rotation are the words of the same calls made alone, a
+    buffer that one context allocated is read by the other and freed through it."""
+    import threading
+
+    g, o = pair.g, pair.o
+    N, level = g.N, g.L
+    if level < 2:
+        pytest.skip("needs two limbs")
+    if N > 8192:
+        pytest.skip("covered at the smaller rings (N = 65536: the ResNet-20 program on three threads)")
+    pr = g.primes[:level]
+    swk = make_swk(g, 4100)
+    ops = [tuple(seeded.uniform_poly(4000 + 10 * t + i, pr, N) for i in range(4)) for t in range(2)]
+    want = [o.mul_relin_rescale(*ops[t], swk, level) for t in range(2)]
+    h = g.share()
+    try:
+        dswk = g.upload(swk)  # allocated by the first context, used by both
+        ctxs, got, errs = [g, h], [None, None], []
+
+        def work(t):
+            try:
+                c = ctxs[t]
+                d = [c.upload(v) for v in ops[t]]
+                r0, r1 = c.alloc((level - 1) * N), c.alloc((level - 1) * N)
+                for _ in range(8):  # long enough for the two threads' launches to interleave
+                    c.mul_relin_rescale(r0, r1, d[0], d[1], d[2], d[3], dswk, level)
+                got[t] = (r0.get(), r1.get())
+                for b in d + [r0, r1]:
+                    b.free()
+            except Exception as e:  # noqa: BLE001 -- reported by the main thread
+                errs.append(e)
+
+        th = [threading.Thread(target=work, args=(t,)) for t in range(2)]
+        for x in th:
+            x.start()
+        for x in th:
+            x.join()
+        assert not errs, errs
+        for t in range(2):
+            eq(got[t][0], want[t][0], "thread %d c0" % t)
+            eq(got[t][1], want[t][1], "thread %d c1" % t)
+        # a buffer of the first context freed through the second: accepted (the family keeps one record)
+        before = g.memory_stats()[2]
+        buf = g.alloc(N)
+        assert g.memory_stats()[2] == before + 1
+        h.lib.ace_free(h.h, buf.ptr)
+        buf.ptr = None
+        assert g.memory_stats()[2] == before
+    finally:
+        h.close()
+
+
 def test_rotation_many(pair):
     """More rotations than one batched launch holds (small rings only: the oracle does each one)."""
     g, o = pair.g, pair.o
