@@ -17,6 +17,7 @@
 #include <mutex>
 #include <stdexcept>
 #include <string>
+#include <tuple>
 #include <unordered_map>
 #include <vector>
 
@@ -1428,6 +1429,43 @@ struct HostProf {
   }
 };
 HostProf g_prof;
+
+// ACE_HIP_CENSUS=<file>: how often each entry point was called with which size, written when the process ends as
+// lines "<entry point> <a> <b> <calls>" (a: level or number of limbs, b: a second size such as the number of
+// operands; 0 where there is none).  For cost models of a whole program on other machines (bench.py's estimate of
+// the reference's CPU time): the counts, not this library's times, are what such a model needs.
+struct Census {
+  bool on = false;
+  std::string path;
+  std::mutex mu;
+  std::map<std::tuple<std::string, size_t, size_t>, unsigned long long> n;
+  Census() {
+    const char* e = std::getenv("ACE_HIP_CENSUS");
+    if (e && *e) on = true, path = e;
+  }
+  void add(const char* name, size_t a, size_t b) {
+    std::lock_guard<std::mutex> lock(mu);
+    ++n[std::make_tuple(std::string(name), a, b)];
+  }
+  void write(const std::string& to) {
+    if (FILE* f = std::fopen(to.c_str(), "w")) {
+      for (auto& kv : n)
+        std::fprintf(f, "%s %zu %zu %llu\n", std::get<0>(kv.first).c_str(), std::get<1>(kv.first), std::get<2>(kv.first), kv.second);
+      std::fclose(f);
+    }
+  }
+  ~Census() {
+    if (!on) return;
+    if (FILE* f = std::fopen(path.c_str(), "w")) {
+      for (auto& kv : n)
+        std::fprintf(f, "%s %zu %zu %llu\n", std::get<0>(kv.first).c_str(), std::get<1>(kv.first), std::get<2>(kv.first), kv.second);
+      std::fclose(f);
+    }
+  }
+};
+Census g_census;
+#define CENSUS_AS(name, a, b) do { if (g_census.on) g_census.add(name, (size_t)(a), (size_t)(b)); } while (0)
+#define CENSUS(a, b) CENSUS_AS(__func__, a, b)
 struct ScopedProf {
   const char* name;
   timespec t0;
@@ -1633,6 +1671,7 @@ int ace_download(ace_ctx* c, int64_t* dst, const int64_t* src, size_t n) {
 }
 int ace_copy(ace_ctx* c, int64_t* dst, const int64_t* src, size_t n) {
   ACE_TRY_KEEP_RUN
+  CENSUS(n, 0);
   if (!dst || !src) return fail("ace_copy: null argument");
   if (dst == src || n == 0) return 0;
   c->forget_orders(dst, n);
@@ -1649,6 +1688,7 @@ int ace_copy(ace_ctx* c, int64_t* dst, const int64_t* src, size_t n) {
 }
 int ace_zero(ace_ctx* c, int64_t* dst, size_t n) {
   ACE_TRY_KEEP_RUN
+  CENSUS(n, 0);
   if (!dst) return fail("ace_zero: null argument");
   if (n == 0) return 0;
   c->forget_orders(dst, n);
@@ -1725,6 +1765,13 @@ int ace_fork_release(ace_ctx* c) {
   ACE_CATCH_INT
 }
 
+void ace_census_mark(const char* label) {
+  if (!g_census.on || !label) return;
+  std::lock_guard<std::mutex> lock(g_census.mu);
+  g_census.write(g_census.path + "." + label);
+  g_census.n.clear();
+}
+
 void ace_memory_stats(const ace_ctx* c, size_t out[4]) {
   out[0] = c->ws_words;
   out[1] = c->pooled_words;
@@ -1758,6 +1805,7 @@ float ace_timer_stop_ms(ace_ctx* c) {
 static int ntt_common(ace_ctx* c, int64_t* dst, const int64_t* src, const int32_t* prime_idx, size_t n_limbs,
                       size_t n_polys, size_t stride_limbs, bool inverse, int passes = 3) {
   ACE_TRY
+  CENSUS_AS(inverse ? "ace_intt" : "ace_ntt", n_limbs * n_polys, 0);
   if (n_limbs == 0 || n_polys == 0) return 0;
   if (!dst || !src || !prime_idx) return fail("ace_ntt: null argument");
   if (n_limbs > (size_t)kMaxPrimes) return fail("ace_ntt: more than 96 limbs per polynomial");
@@ -1794,6 +1842,7 @@ int ace_ntt_pass(ace_ctx* c, int64_t* dst, const int64_t* src, const int32_t* pr
 static int hw_common(ace_ctx* c, EwOp op, int64_t* r, const int64_t* a, const int64_t* b, int64_t s, size_t pi,
                      size_t n) {
   ACE_TRY_KEEP_RUN
+  CENSUS_AS(op == EW_ADD || op == EW_SUB ? "hw_add" : op == EW_MUL ? "hw_mul" : op == EW_MULADD ? "hw_mac" : op == EW_ADD_S || op == EW_SUB_S ? "hw_add_scalar" : op == EW_MUL_S ? "hw_mul_scalar" : "hw_mac_scalar", n, 0);
   if (n == 0) return 0;
   if (!r || !a || (op < EW_ADD_S && !b)) return fail("ace_hw: null argument");
   if (pi >= c->h.L + c->h.K) return fail("ace_hw: prime index out of range");
@@ -1819,6 +1868,7 @@ int ace_hw_modmuladd_scalar(ace_ctx* c, int64_t* r, const int64_t* a, int64_t s,
 
 int ace_hw_rotate(ace_ctx* c, int64_t* r, const int64_t* a, const int64_t* order, size_t pi, size_t n) {
   ACE_TRY_KEEP_RUN
+  CENSUS(n, 0);
   if (n == 0) return 0;
   if (!r || !a || !order) return fail("ace_hw_rotate: null argument");
   if (r == a) return fail("ace_hw_rotate: in-place gather is not supported");
@@ -1917,6 +1967,7 @@ int ace_automorphism_order(ace_ctx* c, int64_t* dev_order, uint32_t k, int is_nt
 // ---- polynomial ops ---------------------------------------------------------------
 static int poly_ew(ace_ctx* c, EwOp op, int64_t* r, const int64_t* a, const int64_t* b, size_t level, int with_p) {
   ACE_TRY
+  CENSUS_AS(op == EW_MUL ? "poly_mul" : "poly_add", level + (with_p ? c->h.K : 0), 0);
   if (!r || !a || !b) return fail("ace_poly: null argument");
   if (!level_ok(c, level)) return fail("ace_poly: level out of range");
   LimbMap lm = poly_lm(c, level, with_p != 0);
@@ -1930,6 +1981,7 @@ int ace_poly_mul(ace_ctx* c, int64_t* r, const int64_t* a, const int64_t* b, siz
 int ace_ext_plain_mac(ace_ctx* c, int64_t* r0, int64_t* r1, const int64_t* const* a0, const int64_t* const* a1,
                       const int64_t* const* plain, size_t count, size_t level, size_t plain_level, int accumulate) {
   ACE_TRY
+  CENSUS(level, count);
   if (!r0 || !r1 || !a0 || !a1 || !plain) return fail("ace_ext_plain_mac: null argument");
   if (!level_ok(c, level) || !level_ok(c, plain_level) || plain_level < level)
     return fail("ace_ext_plain_mac: levels out of range (the plaintext may not sit below the ciphertext)");
@@ -1957,6 +2009,11 @@ int ace_ext_plain_mac_groups(ace_ctx* c, int64_t* const* r0, int64_t* const* r1,
                              const int64_t* const* a0, const int64_t* const* a1, size_t count,
                              const int64_t* const* plain, size_t level, size_t plain_level) {
   ACE_TRY
+  if (g_census.on && plain) {  // the products actually formed
+    size_t terms = 0;
+    for (size_t k = 0; k < n_groups * count; ++k) terms += plain[k] != nullptr;
+    CENSUS_AS("ace_ext_plain_mac", level, terms);
+  }
   if (!r0 || !r1 || !a0 || !a1 || !plain) return fail("ace_ext_plain_mac_groups: null argument");
   if (!level_ok(c, level) || !level_ok(c, plain_level) || plain_level < level)
     return fail("ace_ext_plain_mac_groups: levels out of range (the plaintext may not sit below the ciphertext)");
@@ -1996,6 +2053,7 @@ int ace_ext_plain_mac_groups(ace_ctx* c, int64_t* const* r0, int64_t* const* r1,
 
 static int poly_scalars(ace_ctx* c, bool mul, int64_t* r, const int64_t* a, const int64_t* scalars, size_t level) {
   ACE_TRY
+  CENSUS_AS(mul ? "poly_mul_scalars" : "poly_add_scalars", level, 0);
   if (!r || !a || !scalars) return fail("ace_poly_scalars: null argument");
   if (!level_ok(c, level)) return fail("ace_poly_scalars: level out of range");
   LimbScalars s{};
@@ -2035,6 +2093,7 @@ int ace_expand_small(ace_ctx* c, int64_t* res, const int64_t* small_host, size_t
 int ace_ciph_wsum(ace_ctx* c, int64_t* r0, int64_t* r1, const int64_t* const* a0, const int64_t* const* a1,
                   const int64_t* weights, size_t count, size_t level) {
   ACE_TRY
+  CENSUS(level, count);
   if (!r0 || !r1 || !a0 || !a1 || !weights) return fail("ace_ciph_wsum: null argument");
   if (!level_ok(c, level)) return fail("ace_ciph_wsum: level out of range");
   if (!count || count > kMaxMacOps) return fail("ace_ciph_wsum: between 1 and 32 terms");
@@ -2058,6 +2117,7 @@ int ace_ciph_wsum(ace_ctx* c, int64_t* r0, int64_t* r1, const int64_t* const* a0
 
 int ace_poly_automorphism(ace_ctx* c, int64_t* r, const int64_t* a, const int64_t* order, size_t level, int with_p) {
   ACE_TRY
+  CENSUS(level + (with_p ? c->h.K : 0), 0);
   if (!r || !a || !order) return fail("ace_poly_automorphism: null argument");
   if (r == a) return fail("ace_poly_automorphism: in-place gather is not supported");
   if (!level_ok(c, level)) return fail("ace_poly_automorphism: level out of range");
@@ -2068,6 +2128,7 @@ int ace_poly_automorphism(ace_ctx* c, int64_t* r, const int64_t* a, const int64_
 
 int ace_decomp_modup(ace_ctx* c, int64_t* res, const int64_t* src, size_t level, size_t part, int is_ntt) {
   ACE_TRY_BARE
+  CENSUS(level, part);
   if (!res || !src) return fail("ace_decomp_modup: null argument");
   if (!level_ok(c, level)) return fail("ace_decomp_modup: level out of range");
   if (part >= c->h.num_decomp(level)) return fail("ace_decomp_modup: digit index out of range");
@@ -2080,6 +2141,7 @@ int ace_decomp_modup(ace_ctx* c, int64_t* res, const int64_t* src, size_t level,
 
 int ace_mod_up(ace_ctx* c, int64_t* res, const int64_t* digit, size_t level, size_t part, int is_ntt) {
   ACE_TRY_BARE
+  CENSUS(level, part);
   if (!res || !digit) return fail("ace_mod_up: null argument");
   if (!level_ok(c, level)) return fail("ace_mod_up: level out of range");
   if (part >= c->h.num_decomp(level)) return fail("ace_mod_up: digit index out of range");
@@ -2092,6 +2154,7 @@ int ace_mod_up(ace_ctx* c, int64_t* res, const int64_t* digit, size_t level, siz
 
 int ace_precomp(ace_ctx* c, int64_t* res, const int64_t* src, size_t level, int is_ntt) {
   ACE_TRY_BARE
+  CENSUS(level, 1);
   if (!res || !src) return fail("ace_precomp: null argument");
   if (!level_ok(c, level)) return fail("ace_precomp: level out of range");
   c->flush_pending_overwriting(res, c->h.num_decomp(level) * (level + c->h.K) * (size_t)c->h.N, src,
@@ -2104,6 +2167,7 @@ int ace_precomp(ace_ctx* c, int64_t* res, const int64_t* src, size_t level, int 
 
 int ace_mod_down(ace_ctx* c, int64_t* res, const int64_t* src, size_t level, int is_ntt) {
   ACE_TRY_BARE
+  CENSUS(level, 1);
   if (!res || !src) return fail("ace_mod_down: null argument");
   if (!level_ok(c, level)) return fail("ace_mod_down: level out of range");
   c->flush_pending_overwriting(res, level * (size_t)c->h.N, src, (level + c->h.K) * (size_t)c->h.N, true);
@@ -2127,6 +2191,7 @@ static int batch_args_ok(const char* who, const void* res, size_t res_stride, si
 int ace_precomp_batch(ace_ctx* c, int64_t* res, size_t res_stride, const int64_t* src, size_t src_stride, size_t count,
                       size_t level, int is_ntt) {
   ACE_TRY_BARE
+  CENSUS_AS("ace_precomp", level, count);
   if (!level_ok(c, level)) return fail("ace_precomp_batch: level out of range");
   const size_t N = c->h.N, res_words = c->h.num_decomp(level) * (level + c->h.K) * N, src_words = level * N;
   if (int rc = batch_args_ok("ace_precomp_batch", res, res_stride, res_words, src, src_stride, src_words, count)) return rc;
@@ -2144,6 +2209,7 @@ int ace_precomp_batch(ace_ctx* c, int64_t* res, size_t res_stride, const int64_t
 int ace_mod_down_batch(ace_ctx* c, int64_t* res, size_t res_stride, const int64_t* src, size_t src_stride, size_t count,
                        size_t level, int is_ntt) {
   ACE_TRY_BARE
+  CENSUS_AS("ace_mod_down", level, count);
   if (!level_ok(c, level)) return fail("ace_mod_down_batch: level out of range");
   const size_t N = c->h.N, res_words = level * N, src_words = (level + c->h.K) * N;
   if (int rc = batch_args_ok("ace_mod_down_batch", res, res_stride, res_words, src, src_stride, src_words, count)) return rc;
@@ -2196,6 +2262,7 @@ int ace_mod_down_noalloc(ace_ctx* c, int64_t* res, const int64_t* src, size_t le
 
 int ace_rescale(ace_ctx* c, int64_t* res, const int64_t* src, size_t level, int is_ntt) {
   ACE_TRY_BARE
+  CENSUS(level, 1);
   if (!res || !src) return fail("ace_rescale: null argument");
   if (level < 2 || level > c->h.L) return fail("Level of rescale opnd is too small");
   c->flush_pending_overwriting(res, (level - 1) * (size_t)c->h.N, src, level * (size_t)c->h.N, true);
@@ -2205,6 +2272,7 @@ int ace_rescale(ace_ctx* c, int64_t* res, const int64_t* src, size_t level, int 
 
 int ace_mod_down_rescale(ace_ctx* c, int64_t* res, int64_t* poly, size_t level, int is_ntt) {
   ACE_TRY
+  CENSUS(level, 0);
   if (!res || !poly) return fail("ace_mod_down_rescale: null argument");
   if (level < 2 || level > c->h.L) return fail("ace_mod_down_rescale: level out of range");
   if (res == poly) return fail("ace_mod_down_rescale: the result must not overwrite the operand");
@@ -2219,6 +2287,7 @@ int ace_mod_down_rescale(ace_ctx* c, int64_t* res, int64_t* poly, size_t level, 
 
 int ace_reduce_rescale_modup(ace_ctx* c, int64_t* res, int64_t* raised, int64_t* poly, size_t level, int is_ntt) {
   ACE_TRY
+  CENSUS(level, 0);
   if (!res || !raised || !poly) return fail("ace_reduce_rescale_modup: null argument");
   if (level < 2 || level > c->h.L) return fail("ace_reduce_rescale_modup: level out of range");
   if (res == poly || raised == poly || raised == res) return fail("ace_reduce_rescale_modup: buffers must be distinct");
@@ -2237,6 +2306,7 @@ int ace_reduce_rescale_modup(ace_ctx* c, int64_t* res, int64_t* raised, int64_t*
 
 int ace_transform_from_level0(ace_ctx* c, int64_t* res, const int64_t* src, size_t level) {
   ACE_TRY
+  CENSUS(level, 0);
   if (!res || !src) return fail("ace_transform_from_level0: null argument");
   if (!level_ok(c, level)) return fail("ace_transform_from_level0: level out of range");
   if (res != src && res < src + c->h.N && src < res + level * (size_t)c->h.N)
@@ -2263,6 +2333,7 @@ int ace_embedding_inv(ace_ctx* c, double* host_out, const double* host_in, size_
 int ace_decode(ace_ctx* c, double* host_out, const int64_t* poly, size_t level, int is_ntt, uint32_t slots,
                double factor) {
   ACE_TRY
+  CENSUS(level, 0);
   if (!host_out || !poly) return fail("ace_decode: null argument");
   const size_t N = c->h.N, L = c->h.L;
   if (!slots) slots = (uint32_t)(N / 2);
@@ -2325,6 +2396,7 @@ static int encode_impl(ace_ctx* c, int64_t* res, const void* values, int kind, s
                        size_t level, uint32_t sf_degree, size_t p_cnt, double explicit_scale = 0.0,
                        const void* const* vecs = nullptr, size_t n_vec = 1, size_t res_stride = 0) {
   ACE_TRY
+  CENSUS_AS("ace_encode", level, n_vec);
   if (n_vec == 0) return 0;
   if (!vecs) vecs = &values;
   if (!res) return fail("ace_encode: null argument");
@@ -2417,6 +2489,7 @@ int ace_encode_scaled(ace_ctx* c, int64_t* res, const double* values, size_t n_v
 
 int ace_extend(ace_ctx* c, int64_t* res, const int64_t* src, size_t level) {
   ACE_TRY
+  CENSUS(level, 0);
   if (!res || !src) return fail("ace_extend: null argument");
   if (!level_ok(c, level)) return fail("ace_extend: level out of range");
   launch_mul_const(c->stream, c->d, U(res), U(src), c->pmodq, c->q_lm, (u32)level);
@@ -2427,6 +2500,7 @@ int ace_extend(ace_ctx* c, int64_t* res, const int64_t* src, size_t level) {
 int ace_dot_prod(ace_ctx* c, int64_t* res, const int64_t* digits, const int64_t* key, size_t key_stride,
                  size_t n_parts, size_t level) {
   ACE_TRY
+  CENSUS(level, 0);
   if (!res || !digits || !key) return fail("ace_dot_prod: null argument");
   if (!level_ok(c, level)) return fail("ace_dot_prod: level out of range");
   if (n_parts == 0 || n_parts > c->h.parts) return fail("ace_dot_prod: number of digits out of range");
@@ -2441,6 +2515,7 @@ int ace_ext_rotate(ace_ctx* c, int64_t* out0, int64_t* out1, const int64_t* digi
                    size_t key_half_words, size_t key_stride, size_t n_parts, const int64_t* addend0,
                    const int64_t* order, size_t level, int accumulate) {
   ACE_TRY
+  CENSUS(level, 0);
   if (!out0 || !out1 || !digits || !key || !order) return fail("ace_ext_rotate: null argument");
   if (!level_ok(c, level)) return fail("ace_ext_rotate: level out of range");
   if (n_parts == 0 || n_parts > c->h.parts) return fail("ace_ext_rotate: number of digits out of range");
@@ -2459,6 +2534,7 @@ int ace_ext_rotate(ace_ctx* c, int64_t* out0, int64_t* out1, const int64_t* digi
 int ace_mul_ciph3(ace_ctx* c, int64_t* d0, int64_t* d1, int64_t* d2, const int64_t* a0, const int64_t* a1,
                   const int64_t* b0, const int64_t* b1, size_t level) {
   ACE_TRY_BARE
+  CENSUS(level, 0);
   if (!d0 || !d1 || !d2 || !a0 || !a1 || !b0 || !b1) return fail("ace_mul_ciph3: null argument");
   if (!level_ok(c, level)) return fail("ace_mul_ciph3: level out of range");
   {
@@ -2473,6 +2549,7 @@ int ace_mul_ciph3(ace_ctx* c, int64_t* d0, int64_t* d1, int64_t* d2, const int64
 int ace_fast_switch_key(ace_ctx* c, int64_t* out0, int64_t* out1, const int64_t* digits, const int64_t* swk,
                         size_t level) {
   ACE_TRY
+  CENSUS(level, 0);
   if (!out0 || !out1 || !digits || !swk) return fail("ace_fast_switch_key: null argument");
   if (!level_ok(c, level)) return fail("ace_fast_switch_key: level out of range");
   c->ensure_ws(c->std_ws(level));
@@ -2484,6 +2561,7 @@ int ace_fast_switch_key(ace_ctx* c, int64_t* out0, int64_t* out1, const int64_t*
 int ace_relin(ace_ctx* c, int64_t* r0, int64_t* r1, const int64_t* d0, const int64_t* d1, const int64_t* d2,
               const int64_t* swk, size_t level) {
   ACE_TRY
+  CENSUS(level, 0);
   if (!r0 || !r1 || !d0 || !d1 || !d2 || !swk) return fail("ace_relin: null argument");
   if (!level_ok(c, level)) return fail("ace_relin: level out of range");
   c->ensure_ws(c->std_ws(level));
@@ -2498,6 +2576,7 @@ int ace_relin(ace_ctx* c, int64_t* r0, int64_t* r1, const int64_t* d0, const int
 
 int ace_rescale_ciph(ace_ctx* c, int64_t* r0, int64_t* r1, const int64_t* c0, const int64_t* c1, size_t level) {
   ACE_TRY
+  CENSUS(level, 0);
   if (!r0 || !r1 || !c0 || !c1) return fail("ace_rescale_ciph: null argument");
   if (level < 2 || level > c->h.L) return fail("Level of rescale opnd is too small");
   c->ensure_ws(c->std_ws(level));
@@ -2509,6 +2588,7 @@ int ace_rescale_ciph(ace_ctx* c, int64_t* r0, int64_t* r1, const int64_t* c0, co
 int ace_mul_relin_rescale(ace_ctx* c, int64_t* r0, int64_t* r1, const int64_t* a0, const int64_t* a1,
                           const int64_t* b0, const int64_t* b1, const int64_t* swk, size_t level) {
   ACE_TRY
+  CENSUS(level, 1);
   if (!r0 || !r1 || !a0 || !a1 || !b0 || !b1 || !swk) return fail("ace_mul_relin_rescale: null argument");
   if (level < 2 || level > c->h.L) return fail("ace_mul_relin_rescale: level out of range");
   c->ensure_ws(c->std_ws(level));
@@ -2521,6 +2601,7 @@ int ace_mul_relin_rescale_batch(ace_ctx* c, int64_t* r0, int64_t* r1, size_t out
                                 const int64_t* a1, const int64_t* b0, const int64_t* b1, size_t in_stride,
                                 const int64_t* swk, size_t level, size_t count) {
   ACE_TRY
+  CENSUS_AS("ace_mul_relin_rescale", level, count);
   if (count == 0) return 0;
   if (!r0 || !r1 || !a0 || !a1 || !b0 || !b1 || !swk) return fail("ace_mul_relin_rescale_batch: null argument");
   if (level < 2 || level > c->h.L) return fail("ace_mul_relin_rescale_batch: level out of range");
@@ -2554,6 +2635,7 @@ static void do_fast_rotate(ace_ctx* c, u64* r0, u64* r1, u64 r_stride, const u64
 int ace_fast_rotate(ace_ctx* c, int64_t* r0, int64_t* r1, const int64_t* c0, const int64_t* digits,
                     const int64_t* swk, const int64_t* order, size_t level) {
   ACE_TRY
+  CENSUS(level, 0);
   if (!r0 || !r1 || !c0 || !digits || !swk || !order) return fail("ace_fast_rotate: null argument");
   if (!level_ok(c, level)) return fail("ace_fast_rotate: level out of range");
   {
@@ -2574,6 +2656,7 @@ int ace_fast_rotate(ace_ctx* c, int64_t* r0, int64_t* r1, const int64_t* c0, con
 int ace_rotate_batch(ace_ctx* c, int64_t* r0s, int64_t* r1s, const int64_t* c0, const int64_t* c1,
                      const int64_t* const* swks, const int64_t* const* orders, size_t count, size_t level) {
   ACE_TRY
+  CENSUS(level, count);
   if (count == 0) return 0;
   if (!r0s || !r1s || !c0 || !c1 || !swks || !orders) return fail("ace_rotate_batch: null argument");
   if (!level_ok(c, level)) return fail("ace_rotate_batch: level out of range");

@@ -19,6 +19,7 @@ import argparse
 import json
 import os
 import subprocess
+import tempfile
 import sys
 import time
 
@@ -187,9 +188,20 @@ def bootstrap_leg():
         f = r.stdout.split()
         vals = dict(zip(f[0::2], f[1::2]))
         ms = float(vals["ms"])
+        # the margin against 1e-3 over the keys and messages (there is no bit-level counterpart to compare with):
+        # four more seeds, the last of them with a census of the bootstrap's calls for the CPU estimate
+        errs = [float(vals["max_err"])]
+        census = os.path.join(tempfile.mkdtemp(prefix="ace_census_"), "census.txt")
+        for seed in (2, 3, 4, 5):
+            rs = subprocess.run([exe, "65536", "33", "60", "56", "192", "32768", "15", str(seed)], capture_output=True,
+                                text=True, timeout=240, env=dict(os.environ, ACE_HIP_CENSUS=census) if seed == 5 else None)
+            fs = rs.stdout.split()
+            errs.append(float(fs[fs.index("max_err") + 1]))
+        est = reference_cpu_estimate(census + ".bootstrap", (65536, 34, 60, 56, 3))
         return {"bootstrap": {"workload": "one bootstrap, N=65536, 34 limbs (60/56 bits), 32768 slots, to level 15",
                               "ms": ms, "first_call_ms": float(vals["first_ms"]),
-                              "max_err": float(vals["max_err"]), "exit_status": r.returncode,
+                              "max_err": float(vals["max_err"]), "max_err_over_5_seeds": max(errs),
+                              "cpu_estimate": est, "exit_status": r.returncode,
                               "published_cpu_ms": round(784.03e3 / 19, 1),
                               "published_cpu_note": "the reference's published run, same chain, one CPU thread of "
                                                     "other hardware: not a same-run baseline"}}
@@ -242,6 +254,13 @@ def resnet20_leg():
                                     "s_per_image": float(w[7]),
                                     "note": "images 2-10 on three host threads of one process sharing one set of keys "
                                             "(30 GB) and the kept weight plaintexts; wall time of the batch / images"}
+        # what the same calls would cost in the reference's C code on this host (an estimate: see the function)
+        census = os.path.join(tempfile.mkdtemp(prefix="ace_census_"), "census.txt")
+        rc = subprocess.run([exe, "3", "32", "32", "10", "1"], capture_output=True, text=True, timeout=400,
+                            env=dict(env, ACE_HIP_CENSUS=census, RT_HIP_PLAINTEXT_CACHE_GB="0"))
+        est = reference_cpu_estimate(census, (65536, 34, 60, 56, 3)) if rc.returncode == 0 else None
+        if est:
+            out["cpu_estimate"] = est
         env["MODEL_KEY_SEED"] = "22"
         r2 = subprocess.run([exe, "3", "32", "32", "10", "1"], capture_output=True, text=True, timeout=400, env=env)
         again = [float(v) for v in [l for l in r2.stdout.splitlines() if l.startswith("output:")][0].split()[1:]]
@@ -250,6 +269,83 @@ def resnet20_leg():
         return {"resnet20": out}
     except Exception as e:
         return {"resnet20": {"error": repr(e)[:200]}}
+
+
+def reference_cpu_estimate(census_path, chain, seconds_cap=40.0):
+    """What a program's calls would take in the reference's own C code on this host, one thread: the counts of a
+    census of the library's entry points (ACE_HIP_CENSUS: entry point, level, second size, calls) times the
+    reference functions each entry point stands for, those timed by the compiled reference (oracle/_ref/ref_driver:
+    Hw_modadd / Hw_modmul / Hw_modmuladd / Hw_modmul_scalar / Hw_rotate / Ftt_fwd / Ftt_inv per limb, Decomp_modup,
+    Mod_down, Rescale, Dot_prod, Encode_at_level_with_sf) at nine levels of the same chain and interpolated between
+    them.  An estimate, labelled so: the reference's CKKS layer cannot be built here, so its bootstrap and ciphertext
+    operations enter as the sums of the polynomial functions they are made of (evaluator.c, bootstrap.c)."""
+    import numpy as np
+    import refdrv
+
+    if not refdrv.available() or not os.path.exists(census_path):
+        return None
+    N, L, q0, sf, parts = chain
+    s = refdrv.RefSession(*chain)
+    levels = sorted({3, 6, 10, 14, 18, 22, 26, 30, L} & set(range(3, L + 1)))
+    ks = [s.add(refdrv.OP_TIME_PRIMITIVES, lv, 7) for lv in levels]
+    info, res = s.run()
+    K, part_size = info["K"], info["part_size"]
+    tab = np.array([[float(v) * 1e-9 for v in res[k]] for k in ks])  # [level sample][primitive] seconds
+    names = ["add", "mul", "mac", "mul_scalar", "rot", "ntt", "intt", "decomp_modup", "mod_down", "rescale", "dot", "encode"]
+    per_limb = {n: float(np.median(tab[:, i])) for i, n in enumerate(names[:7])}
+
+    def t(name, level):
+        return float(np.interp(level, levels, tab[:, names.index(name)]))
+
+    nd = lambda lv: -(-lv // part_size)
+    a_, m_, c_, ms_, r_ = (per_limb[k] for k in ("add", "mul", "mac", "mul_scalar", "rot"))
+    switch = lambda lv: 2 * t("dot", lv) + 2 * t("mod_down", lv)
+    precomp = lambda lv: nd(lv) * t("decomp_modup", lv)
+    cost = {
+        "hw_add": lambda lv, b: a_, "hw_mul": lambda lv, b: m_, "hw_mac": lambda lv, b: c_,
+        "hw_add_scalar": lambda lv, b: a_, "hw_mul_scalar": lambda lv, b: ms_, "hw_mac_scalar": lambda lv, b: ms_ + a_,
+        "ace_hw_rotate": lambda lv, b: r_,
+        "ace_zero": lambda words, b: words * 8 / 5e9, "ace_copy": lambda words, b: words * 16 / 5e9,
+        "ace_encode": lambda lv, b: max(b, 1) * t("encode", lv),
+        "ace_mod_down": lambda lv, b: max(b, 1) * t("mod_down", lv),
+        "ace_rescale": lambda lv, b: t("rescale", lv),
+        "ace_decomp_modup": lambda lv, b: t("decomp_modup", lv), "ace_mod_up": lambda lv, b: t("decomp_modup", lv),
+        "ace_precomp": lambda lv, b: max(b, 1) * precomp(lv),
+        "poly_add": lambda limbs, b: limbs * a_, "poly_mul": lambda limbs, b: limbs * m_,
+        "poly_add_scalars": lambda lv, b: lv * a_, "poly_mul_scalars": lambda lv, b: lv * ms_,
+        "ace_ext_rotate": lambda lv, b: 2 * t("dot", lv) + (lv + K) * (2 * r_ + a_),
+        "ace_ext_plain_mac": lambda lv, b: b * 2 * (lv + K) * (m_ + a_),
+        "ace_ciph_wsum": lambda lv, b: b * 2 * lv * (ms_ + a_),
+        "ace_mul_ciph3": lambda lv, b: lv * (4 * m_ + a_),
+        "ace_relin": lambda lv, b: precomp(lv) + switch(lv) + 2 * lv * a_,
+        "ace_rescale_ciph": lambda lv, b: 2 * t("rescale", lv),
+        "ace_mul_relin_rescale": lambda lv, b: max(b, 1) * (lv * (4 * m_ + a_) + precomp(lv) + switch(lv) + 2 * lv * a_ + 2 * t("rescale", lv)),
+        "ace_rotate_batch": lambda lv, b: precomp(lv) + b * (switch(lv) + lv * (a_ + 2 * r_)),
+        "ace_fast_rotate": lambda lv, b: switch(lv) + lv * (a_ + 2 * r_),
+        "ace_fast_switch_key": lambda lv, b: switch(lv), "ace_dot_prod": lambda lv, b: t("dot", lv),
+        "ace_extend": lambda lv, b: lv * ms_,
+        "ace_ntt": lambda limbs, b: limbs * per_limb["ntt"], "ace_intt": lambda limbs, b: limbs * per_limb["intt"],
+        "ace_transform_from_level0": lambda lv, b: lv * a_,
+        "ace_mod_down_rescale": lambda lv, b: t("mod_down", lv) + t("rescale", lv),
+        "ace_reduce_rescale_modup": lambda lv, b: t("mod_down", lv) + t("rescale", lv) + t("decomp_modup", lv),
+        "ace_poly_automorphism": lambda limbs, b: limbs * r_,
+    }
+    total, by_entry, unknown = 0.0, {}, set()
+    for line in open(census_path):
+        name, a, b, n = line.split()
+        f = cost.get(name)
+        if not f:
+            unknown.add(name)
+            continue
+        sec = int(n) * f(int(a), int(b))
+        total += sec
+        by_entry[name] = by_entry.get(name, 0.0) + sec
+    top = dict(sorted(((k, round(v, 1)) for k, v in by_entry.items()), key=lambda kv: -kv[1])[:8])
+    return {"cpu_estimate_s": round(total, 1), "cores": 1, "kind": "estimate from the reference's own functions",
+            "largest_parts_s": top, "not_counted": sorted(unknown),
+            "method": "calls of one image by entry point and level (ACE_HIP_CENSUS, weight plaintexts encoded every "
+                      "time as the reference does) x the reference's Hw_* / Ftt / Decomp_modup / Mod_down / Rescale / "
+                      "Dot_prod / Encode timed on this host at %d levels of the chain, gcc -O3, one thread" % len(levels)}
 
 
 def keyswitch_cpu_reference(level):

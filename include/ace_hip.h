@@ -124,6 +124,12 @@ int      ace_fork_release(ace_ctx* ctx);
  * buffers kept for reuse (words), out[2] = buffers handed out by ace_alloc and not yet freed, out[3] = freed buffers
  * kept for reuse (count). */
 void     ace_memory_stats(const ace_ctx* ctx, size_t out[4]);
+/* With ACE_HIP_CENSUS=<file> in the environment the library counts the calls of its entry points by size and writes
+ * "<entry point> <level or limbs> <second size> <calls>" lines to <file> when the process ends (no counterpart in
+ * the reference; the counts feed cost models of a whole program, such as the benchmark's estimate of the
+ * reference's CPU time).  ace_census_mark writes the counts so far to <file>.<label> and starts again from zero, so
+ * that a program's phases (key generation, images) can be told apart.  Without the variable: nothing. */
+void     ace_census_mark(const char* label);
 /* HIP-event stopwatch on the context's stream (for benchmarks) */
 int      ace_timer_start(ace_ctx* ctx);
 float    ace_timer_stop_ms(ace_ctx* ctx); /* synchronises; <0 on error */

@@ -41,7 +41,7 @@ enum {
   OP_NTT = 1, OP_INTT, OP_HW, OP_DECOMP_MODUP, OP_PRECOMP, OP_MOD_DOWN,
   OP_RESCALE, OP_DOT_PROD, OP_AUTO_ORDER, OP_AUTO_INDEX, OP_AUTOMORPHISM,
   OP_EXTEND, OP_TBL_MODUP, OP_TBL_MODDOWN, OP_TBL_RESCALE, OP_POLY, OP_TWIDDLES,
-  OP_MOD_UP, OP_MOD_DOWN_RESCALE, OP_REDUCE_RESCALE_MODUP, OP_FROM_LEVEL0, OP_ENCODE, OP_DECODE, OP_EMBEDDING, OP_TIME_NTT, OP_ENCODE_SCALED, OP_TIME_KEYSWITCH
+  OP_MOD_UP, OP_MOD_DOWN_RESCALE, OP_REDUCE_RESCALE_MODUP, OP_FROM_LEVEL0, OP_ENCODE, OP_DECODE, OP_EMBEDDING, OP_TIME_NTT, OP_ENCODE_SCALED, OP_TIME_KEYSWITCH, OP_TIME_PRIMITIVES
 };
 
 static int64_t* in_buf;
@@ -146,6 +146,115 @@ int main(int argc, char** argv) {
         wr1(trips);
         wr1(ns);
         wr(data, nl * N);
+        break;
+      }
+      case OP_TIME_PRIMITIVES: { /* a1 = level, a2 = seed; no input.  The functions a compiled program and the
+                                    bootstrap are made of, each run once at `level` on uniform residues and timed on
+                                    its own.  out = nanoseconds of: Hw_modadd, Hw_modmul, Hw_modmuladd,
+                                    Hw_modmul_scalar, Hw_rotate, Hw_ntt, Hw_intt (each per limb: the mean over the
+                                    level's limbs), Decomp_modup of digit 0, Mod_down, Rescale (level >= 3, else 0),
+                                    one Dot_prod over all digits, Encode_at_level_with_sf of N/2 values */
+        size_t lv = (size_t)a1, nd = Get_num_decomp(Get_crt_context(), lv), T = lv + K;
+        uint64_t st = (uint64_t)a2 * 0x9E3779B97F4A7C15ull + 1;
+        int64_t *x = (int64_t*)malloc(T * N * sizeof(int64_t)), *y = (int64_t*)malloc(T * N * sizeof(int64_t));
+        int64_t* r = (int64_t*)malloc(T * N * sizeof(int64_t));
+        for (size_t t = 0; t < T; t++) {
+          uint64_t q = (uint64_t)Get_modulus_val(prime_at(t < lv ? t : L + (t - lv)));
+          for (size_t i = 0; i < N; i++) {
+            st = st * 6364136223846793005ull + 1442695040888963407ull;
+            x[t * N + i] = (int64_t)((st >> 3) % q);
+            st = st * 6364136223846793005ull + 1442695040888963407ull;
+            y[t * N + i] = (int64_t)((st >> 3) % q);
+          }
+        }
+        struct timespec t0, t1;
+        int64_t ns[12] = {0};
+#define P_TICK() clock_gettime(CLOCK_MONOTONIC, &t0)
+#define P_TOCK(k, div) (clock_gettime(CLOCK_MONOTONIC, &t1), ns[k] = ((int64_t)(t1.tv_sec - t0.tv_sec) * 1000000000 + (t1.tv_nsec - t0.tv_nsec)) / (int64_t)(div))
+        VALUE_LIST* order = Alloc_value_list(I64_TYPE, N);
+        Precompute_automorphism_order(order, 5, (uint32_t)N, true);
+        memset(r, 0, T * N * sizeof(int64_t)); /* the pages of the result are there before the first timed loop */
+        P_TICK();
+        for (size_t t = 0; t < lv; t++) Hw_modadd(r + t * N, x + t * N, y + t * N, Get_modulus(prime_at(t)), N);
+        P_TOCK(0, lv);
+        P_TICK();
+        for (size_t t = 0; t < lv; t++) Hw_modmul(r + t * N, x + t * N, y + t * N, Get_modulus(prime_at(t)), N);
+        P_TOCK(1, lv);
+        P_TICK();
+        for (size_t t = 0; t < lv; t++) Hw_modmuladd(r + t * N, x + t * N, y + t * N, Get_modulus(prime_at(t)), N);
+        P_TOCK(2, lv);
+        P_TICK();
+        for (size_t t = 0; t < lv; t++) Hw_modmul_scalar(r + t * N, x + t * N, 12345, Get_modulus(prime_at(t)), N);
+        P_TOCK(3, lv);
+        P_TICK();
+        for (size_t t = 0; t < lv; t++) Hw_rotate(r + t * N, x + t * N, Get_i64_values(order), Get_modulus(prime_at(t)), N);
+        P_TOCK(4, lv);
+        P_TICK();
+        for (size_t t = 0; t < lv; t++) {
+          VALUE_LIST vl;
+          Init_i64_value_list_no_copy(&vl, N, r + t * N);
+          Ftt_fwd(&vl, Get_ntt(prime_at(t)), &vl);
+        }
+        P_TOCK(5, lv);
+        P_TICK();
+        for (size_t t = 0; t < lv; t++) {
+          VALUE_LIST vl;
+          Init_i64_value_list_no_copy(&vl, N, r + t * N);
+          Ftt_inv(&vl, Get_ntt(prime_at(t)), &vl);
+        }
+        P_TOCK(6, lv);
+        POLYNOMIAL src, ext, down, low, kb[16], dg[16], acc;
+        wrap_poly(&src, x, lv, 0, true);
+        wrap_poly(&ext, r, lv, K, true);
+        P_TICK();
+        Decomp_modup(&ext, &src, 0);
+        P_TOCK(7, 1);
+        memset(&down, 0, sizeof(down)), memset(&low, 0, sizeof(low)), memset(&acc, 0, sizeof(acc));
+        Alloc_poly_data(&down, (uint32_t)N, lv, 0);
+        Set_is_ntt(&down, true);
+        wrap_poly(&ext, y, lv, K, true);
+        P_TICK();
+        Mod_down(&down, &ext);
+        P_TOCK(8, 1);
+        if (lv >= 3) { /* (the reference's Rescale drops the limb through Modswitch, which wants two limbs left) */
+          Alloc_poly_data(&low, (uint32_t)N, lv - 1, 0);
+          Set_is_ntt(&low, true);
+          P_TICK();
+          Rescale(&low, &down);
+          P_TOCK(9, 1);
+          Free_poly_data(&low);
+        }
+        /* the digits and the key halves of one inner product: the same limbs seen nd times (what is timed is the
+         * arithmetic; a key is viewed at `level`, as Derive_poly does) */
+        for (size_t d = 0; d < nd && d < 16; d++) {
+          wrap_poly(&dg[d], x, lv, K, true);
+          wrap_poly(&kb[d], y, lv, K, true);
+        }
+        P_TICK();
+        Dot_prod(&acc, dg, kb, (uint32_t)nd);
+        P_TOCK(10, 1);
+        Free_poly_data(&acc);
+        Free_poly_data(&down);
+        {
+          CKKS_ENCODER* enc = (CKKS_ENCODER*)Context->_encoder;
+          size_t        nv  = N / 2;
+          VALUE_LIST*   vals = Alloc_value_list(DCMPLX_TYPE, nv);
+          for (size_t i = 0; i < nv; i++) {
+            st = st * 6364136223846793005ull + 1442695040888963407ull;
+            DCMPLX_VALUE_AT(vals, i) = (double)(int64_t)(st >> 11) / (double)(1ull << 52) - 1.0;
+          }
+          PLAINTEXT pt;
+          memset(&pt, 0, sizeof(pt));
+          P_TICK();
+          Encode_at_level_with_sf(&pt, enc, vals, (uint32_t)lv, (uint32_t)nv, 1);
+          P_TOCK(11, 1);
+          Free_poly_data(Get_plain_poly(&pt));
+          Free_value_list(vals);
+        }
+        Free_value_list(order);
+        free(x), free(y), free(r);
+        wr1(12);
+        wr(ns, 12);
         break;
       }
       case OP_TIME_KEYSWITCH: { /* a1 = level, a2 = seed; no input.  The pieces of one key switch at `level`, each run

@@ -9,6 +9,7 @@
 #include <math.h>
 #include <time.h>
 
+#include "ace_hip.h"
 #include "rt_ant/rt_ant.h"
 
 static CKKS_PARAMS Params = {._provider = LIB_ANT};
@@ -70,9 +71,11 @@ int main(int argc, char** argv) {
   Rt_sync();
   /* BOOTSTRAP_REPEAT=n times the call n times over (for profiles in which the steady state should dominate) */
   int    repeat = getenv("BOOTSTRAP_REPEAT") ? atoi(getenv("BOOTSTRAP_REPEAT")) : 1;
+  ace_census_mark("setup"); /* with ACE_HIP_CENSUS: the calls of the timed bootstraps alone go to <file>.bootstrap */
   double t0     = Now_ms();
   for (int k = 0; k < (repeat < 1 ? 1 : repeat); ++k) Eval_bootstrap_ciph(&fresh, &ct, level_after, slots);
   Rt_sync();
+  ace_census_mark("bootstrap");
   double t1 = t0 + (Now_ms() - t0) / (repeat < 1 ? 1 : repeat);
   Rt_decrypt(&back, &fresh);
   double* y = Get_msg_from_plain(&back);

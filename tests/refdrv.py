@@ -11,7 +11,8 @@ DRIVER = os.path.join(ROOT, "oracle", "_ref", "ref_driver")
 (OP_NTT, OP_INTT, OP_HW, OP_DECOMP_MODUP, OP_PRECOMP, OP_MOD_DOWN, OP_RESCALE, OP_DOT_PROD,
  OP_AUTO_ORDER, OP_AUTO_INDEX, OP_AUTOMORPHISM, OP_EXTEND, OP_TBL_MODUP, OP_TBL_MODDOWN,
  OP_TBL_RESCALE, OP_POLY, OP_TWIDDLES, OP_MOD_UP, OP_MOD_DOWN_RESCALE, OP_REDUCE_RESCALE_MODUP,
- OP_FROM_LEVEL0, OP_ENCODE, OP_DECODE, OP_EMBEDDING, OP_TIME_NTT, OP_ENCODE_SCALED, OP_TIME_KEYSWITCH) = range(1, 28)
+ OP_FROM_LEVEL0, OP_ENCODE, OP_DECODE, OP_EMBEDDING, OP_TIME_NTT, OP_ENCODE_SCALED, OP_TIME_KEYSWITCH,
+ OP_TIME_PRIMITIVES) = range(1, 29)
 
 HW_OPS = {"modadd": 0, "modsub": 1, "modmul": 2, "modmuladd": 3, "modadd_scalar": 4,
           "modsub_scalar": 5, "modmul_scalar": 6, "modmuladd_scalar": 7, "rotate": 8}

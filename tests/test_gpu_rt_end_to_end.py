@@ -216,6 +216,27 @@ def resnet20_run(chain, key_seed, images=1, threads=1, amplitude=AMPLITUDE):
     return [[float(v) for v in row] for row in rows]
 
 
+def test_bootstrap_precision_over_seeds_and_slot_counts():
+    """The bootstrap has no bit-level counterpart here, so its margin against the 1e-3 bound is shown over the keys
+    and messages rather than on one draw: five seeds at the full slot count of the model ring on the published
+    chain (60 / 56 bits, refreshed to level 15 as the ResNet programs ask), and the sparse slot counts a packed
+    model uses (a sparsely packed message is raised, summed over its copies and refreshed through the shorter
+    transforms)."""
+    assert os.path.exists(BOOTSTRAP), "tests/programs/bootstrap_program is not built"
+    worst = 0.0
+    for seed in (1, 2, 3, 4, 5):
+        err, rc = bootstrap_error("65536 33 60 56 192 32768 15 %d" % seed)
+        print("seed", seed, "max_err %.3g" % err, flush=True)
+        assert rc == 0 and err < 1e-3, (seed, err)
+        worst = max(worst, err)
+    for slots in (16384, 8192, 4096):
+        err, rc = bootstrap_error("65536 33 60 56 192 %d 15 1" % slots)
+        print("slots", slots, "max_err %.3g" % err, flush=True)
+        assert rc == 0 and err < 1e-3, (slots, err)
+        worst = max(worst, err)
+    print("worst max_err %.3g" % worst, flush=True)
+
+
 def resnet20_logits(chain, key_seed, amplitude=AMPLITUDE):
     return resnet20_run(chain, key_seed, amplitude=amplitude)[0]
 
