@@ -276,6 +276,29 @@ def test_reference_resnet20_program_on_three_threads():
         assert d < 1e-3 and d < 0.01 * max(abs(v) for v in a), (i, d)
 
 
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_operator_block_at_the_model_ring(seed, tmp_path):
+    """One block of a compiled model at the size the whole models run at (N=65536, 34 limbs, 60/56 bits), with weights
+    the test program knows (tests/programs/operator_program.c): a 3x3 convolution over four channels laid out as the
+    compiler lays out ResNet-20's first one, its plaintexts read by Pt_from_msg from a side-file the program writes,
+    then Bootstrap to level 15 and the compiler's own App_relu / Rotate / Relinearize from the included ResNet-20
+    program.  Expected values are the validation mode's float models (Conv_impl, Relu_impl), which are pinned to the
+    reference's rt_validate.c.  Bounds: the convolution 1e-5 (measured 8e-10), the bootstrapped values 1e-3 (5e-4),
+    the ReLU 1e-3 where |x| >= 0.1 as in the reference's relu example (4e-4) and 1e-2 everywhere (3e-3: the
+    polynomial's fit is loosest around zero)."""
+    exe = os.path.join(rt_program.ROOT, "oracle", "_ref", "models", "operator_block")
+    if not os.path.exists(exe):
+        pytest.skip("built only where the reference tree is present")
+    print("running", exe, seed, flush=True)
+    r = subprocess.run([exe, str(tmp_path / "block.msg"), str(seed)], capture_output=True, text=True, timeout=200)
+    print(r.stdout, flush=True)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    f = r.stdout.split()
+    v = {f[i]: float(f[i + 1]) for i in range(0, 12, 2)}
+    assert v["conv_err"] < 1e-5 and v["bootstrap_err"] < 1e-3 and v["relu_err_away_from_zero"] < 1e-3
+    assert v["relu_err"] < 1e-2 and v["level"] == 15
+
+
 def test_reference_resnet20_program_runs_on_its_compiled_in_chain():
     """The same program with the parameters it carries (51 / 46 bits): runs to the end.  Its bootstraps are far
     outside their precision on this chain (test_bootstrap_precision_at_the_model_ring), in the reference's arithmetic
