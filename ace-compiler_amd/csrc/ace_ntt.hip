@@ -92,6 +92,13 @@ __device__ __forceinline__ void wave_sync() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// A 16-byte load per lane that writes LDS directly (no registers held while it is on its way).
+__device__ __forceinline__ void stage_request(const u64* src, u64* lds_block) {
+  // lane L's 16 bytes go to lds_block + 16 L; m0 carries the block's LDS address
+  const u32 at = (u32)__builtin_amdgcn_readfirstlane((int)(u32)(size_t)(__attribute__((address_space(3))) void*)lds_block);
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(at) : "memory", "m0");
+}
+
 // ---------------------------------------------------------------------------
 struct ArithInt {
   typedef u64 T;
@@ -639,6 +646,107 @@ __global__ __launch_bounds__(kChunkThreads, kChunkWaves) void ntt_fwd_chunk(DevC
   else fwd_chunk_body<ArithInt, EPI, SKIP>(lds, c, datas, pos, logr, n_polys, f, chunk, limb, pblk, pi);
 }
 
+// The forward chunk pass for launches of many polynomials whose limbs are all on the FP64 back end, in runs of
+// `run` polynomials per work-group with the next polynomial's words on their way into LDS meanwhile (see
+// ntt_inv_half_run below for the scheme and its reasons).  A wave stages the 512 words its first round works on
+// (lane + 512 r of the chunk's 64-word column group): staging load j brings the 16-byte pairs of r = 2j (lanes 0-31)
+// and r = 2j + 1 (lanes 32-63), which land as [r][lane] in the wave's 4 KiB.  66 KiB of LDS per work-group: two
+// work-groups, 16 waves, per CU.
+__global__ __launch_bounds__(kChunkThreads, 4) void ntt_fwd_chunk_run(DevCtx c, PolySeq datas, LimbMap lm, LimbMap pos,
+                                                                    u32 logr, u32 n_limbs, u32 n_polys, u32 run) {
+  typedef ArithFp A;
+  __shared__ double lds[kChunk + kChunk / 16];
+  __shared__ __attribute__((aligned(16))) u64 stage[kChunk];
+  u32 chunk, limb, pblk;
+  if (!chunk_block(c, n_limbs, (n_polys + run - 1) / run, chunk, limb, pblk)) return;
+  const u32 pi = lm.prime[limb];
+  const int t = threadIdx.x;
+  const u32 poly0 = pblk * run;
+  const u32 cnt = min(run, n_polys - poly0);
+  const u64 loff = (u64)pos.prime[limb] * c.N + (u64)chunk * kChunk;
+  A ar;
+  ar.init(c, pi, false, nullptr, 0);
+  const ChunkMap cm(t);
+  const u32 lane = (u32)t & 63;
+  u64* mine = stage + cm.wv * 512;
+  auto request = [&](u32 poly) {
+    const u64* src = datas.at(poly) + loff + cm.wv * 64 + 2 * (lane & 31) + 512 * (lane >> 5);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) stage_request(src + 1024 * j, mine + 128 * j);
+  };
+  // twiddle index of local stage ls, local group g of this chunk: (m0 << ls) + (chunk << ls) + g
+  const u32 tw0 = (1u << logr) + chunk;
+  A::TWL a0[1], a1[2], a2[4], b0[1], b1[2], b2[4], c0[1], c1[2], c2[4], d0[1], d1[2], d2[4];
+  ar.load_tw<1>(tw0 << 0, a0);
+  ar.load_tw<2>(tw0 << 1, a1);
+  ar.load_tw<4>(tw0 << 2, a2);
+  ar.load_tw<1>((tw0 << 3) + (cm.wv << 0), b0);
+  ar.load_tw<2>((tw0 << 4) + (cm.wv << 1), b1);
+  ar.load_tw<4>((tw0 << 5) + (cm.wv << 2), b2);
+  ar.load_tw<1>((tw0 << 6) + (cm.h << 0), c0);
+  ar.load_tw<2>((tw0 << 7) + (cm.h << 1), c1);
+  ar.load_tw<4>((tw0 << 8) + (cm.h << 2), c2);
+  ar.load_tw<1>((tw0 << 9) + ((u32)t << 0), d0);
+  ar.load_tw<2>((tw0 << 10) + ((u32)t << 1), d1);
+  ar.load_tw<4>((tw0 << 11) + ((u32)t << 2), d2);
+  {  // the compiler waits for the per-lane ones here, so that its count of pending loads is zero afterwards
+    auto use = [](double& x) { asm volatile("" : "+v"(x)); };
+    use(c0[0]);
+    for (auto& x : c1) use(x);
+    for (auto& x : c2) use(x);
+    use(d0[0]);
+    for (auto& x : d1) use(x);
+    for (auto& x : d2) use(x);
+  }
+  request(poly0);
+  u64* ldsu = reinterpret_cast<u64*>(lds);
+  for (u32 it = 0; it < cnt; ++it) {
+    // this polynomial's words are in LDS: its four loads are older than the eight stores of the previous one
+    if (it == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    double v[8];
+#pragma unroll
+    for (int r = 0; r < 8; ++r) v[r] = ar.in_mid(mine[64 * r + lane]);  // centred by the strided pass
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // in registers before the next ones overwrite them
+    if (it + 1 < cnt) request(poly0 + it + 1);
+    ct_stage_pre<A, 8, 0>(ar, v, a0);
+    ct_stage_pre<A, 8, 1>(ar, v, a1);
+    ct_stage_pre<A, 8, 2>(ar, v, a2);
+#pragma unroll
+    for (int r = 0; r < 8; ++r) lds[cm.wide + ChunkMap::wide_off(r)] = v[r];
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < 8; ++r) v[r] = lds[cm.wave + ChunkMap::wave_off(r)];
+    ct_stage_pre<A, 8, 0>(ar, v, b0);
+    ct_stage_pre<A, 8, 1>(ar, v, b1);
+    ct_stage_pre<A, 8, 2>(ar, v, b2);
+#pragma unroll
+    for (int r = 0; r < 8; ++r) lds[cm.wave + ChunkMap::wave_off(r)] = v[r];
+    wave_sync();  // the words read next were written by this wave
+#pragma unroll
+    for (int r = 0; r < 8; ++r) v[r] = lds[cm.octet + ChunkMap::octet_off(r)];
+    reduce_all<A, 8>(ar, v);
+    ct_stage_pre<A, 8, 0>(ar, v, c0);
+    ct_stage_pre<A, 8, 1>(ar, v, c1);
+    ct_stage_pre<A, 8, 2>(ar, v, c2);
+#pragma unroll
+    for (int r = 0; r < 8; ++r) lds[cm.octet + ChunkMap::octet_off(r)] = v[r];
+    wave_sync();  // the words read next were written by this wave
+#pragma unroll
+    for (int r = 0; r < 8; ++r) v[r] = lds[cm.narrow + ChunkMap::narrow_off(r)];
+    ct_stage_pre<A, 8, 0>(ar, v, d0);
+    ct_stage_pre<A, 8, 1>(ar, v, d1);
+    ct_stage_pre<A, 8, 2>(ar, v, d2);
+#pragma unroll
+    for (int r = 0; r < 8; ++r) ldsu[cm.narrow + ChunkMap::narrow_off(r)] = ar.out_canon(v[r]);
+    wave_sync();  // the result leaves in the wave order: every word a wave stores was written by that wave
+    u64* out = datas.at(poly0 + it) + loff + cm.wv * 512 + lane;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) stg<4>(out + 64 * r, ldsu[cm.wave + ChunkMap::wave_off(r)]);
+    __syncthreads();  // the next polynomial's first round writes words that other waves may still be reading
+  }
+}
+
 // ---------------------------------------------------------------------------
 // inverse, chunk pass: spans 1..2048 on 4096 contiguous words; src -> dst.
 // Nothing is scaled here: 1/N (times an optional per-limb constant) is applied
@@ -761,18 +869,124 @@ __global__ __launch_bounds__(kChunkThreads, kChunkWaves) void ntt_inv_chunk(DevC
 // the word at t + 256 (r >> 2 & 1) + 512 (r & 1) + 1024 (r >> 1 & 1) so that the two stages pair neighbouring registers
 // and registers two apart.
 constexpr int kLogHalf = 11, kHalf = 1 << kLogHalf, kHalfThreads = 256;
+// the twiddles of a thread for the eleven stages of a half; they depend on the limb, the half and the thread only
+template <class A>
+struct HalfTw {
+  typename A::TWL a0[4], a1[2], a2[1], b0[4], b1[2], b2[1], c0[4], c1[2], c2[1], d0[2], d1[1];
+  __device__ __forceinline__ void load(const A& ar, const ChunkMap& cm, u32 mh, u32 half, u32 t) {
+    ar.template load_tw<4>((mh >> 0) + (half << 10) + (t << 2), a0);
+    ar.template load_tw<2>((mh >> 1) + (half << 9) + (t << 1), a1);
+    ar.template load_tw<1>((mh >> 2) + (half << 8) + (t << 0), a2);
+    ar.template load_tw<4>((mh >> 3) + (half << 7) + (cm.h << 2), b0);
+    ar.template load_tw<2>((mh >> 4) + (half << 6) + (cm.h << 1), b1);
+    ar.template load_tw<1>((mh >> 5) + (half << 5) + (cm.h << 0), b2);
+    ar.template load_tw<4>((mh >> 6) + (half << 4) + (cm.wv << 2), c0);
+    ar.template load_tw<2>((mh >> 7) + (half << 3) + (cm.wv << 1), c1);
+    ar.template load_tw<1>((mh >> 8) + (half << 2) + (cm.wv << 0), c2);
+    ar.template load_tw<2>((mh >> 9) + (half << 1), d0);
+    ar.template load_tw<1>((mh >> 10) + half, d1);
+  }
+  // makes the compiler wait for the loads above here, so that its count of pending loads is zero afterwards
+  __device__ __forceinline__ void settle() {
+    auto use = [](typename A::TWL& x) { asm volatile("" : "+v"(x)); };
+    for (auto& x : a0) use(x);
+    for (auto& x : a1) use(x);
+    use(a2[0]);
+    for (auto& x : b0) use(x);
+    for (auto& x : b1) use(x);
+    use(b2[0]);
+  }
+};
+// the eleven stages of a half from the words a thread loaded (raw[r] = word 8 t + r of the half) to the words it
+// stores (word(r) of its column t); twiddles loaded stage by stage, or handed in (pre)
+__device__ __forceinline__ constexpr int half_word(int r) { return 256 * ((r >> 2) & 1) + 512 * (r & 1) + 1024 * ((r >> 1) & 1); }
+template <class A, bool PRE>
+__device__ __forceinline__ void inv_half_rounds(typename A::T* lds, const A& ar, const ChunkMap& cm, u32 mh, u32 half,
+                                                const u64* raw, u64* out, const HalfTw<A>* pre) {
+  typedef typename A::T T;
+  const int t = threadIdx.x;
+  T v[8];
+#pragma unroll
+  for (int r = 0; r < 8; ++r) v[r] = ar.in_canon(raw[r]);
+  // spans 1, 2, 4
+  if constexpr (PRE) {
+    gs_stage_pre<A, 8, 0>(ar, v, pre->a0);
+    gs_stage_pre<A, 8, 1>(ar, v, pre->a1);
+  } else {
+    gs_stage<A, 8, 0>(ar, v, (mh >> 0) + (half << 10) + ((u32)t << 2));
+    gs_stage<A, 8, 1>(ar, v, (mh >> 1) + (half << 9) + ((u32)t << 1));
+  }
+  ar.recentre_sum_of_four(v[0]);
+  ar.recentre_sum_of_four(v[4]);
+  if constexpr (PRE) gs_stage_pre<A, 8, 2>(ar, v, pre->a2);
+  else gs_stage<A, 8, 2>(ar, v, (mh >> 2) + (half << 8) + ((u32)t << 0));
+#pragma unroll
+  for (int r = 0; r < 8; ++r) lds[cm.narrow + ChunkMap::narrow_off(r)] = v[r];
+  wave_sync();  // the words read next were written by this wave
+  // spans 8, 16, 32
+#pragma unroll
+  for (int r = 0; r < 8; ++r) v[r] = lds[cm.octet + ChunkMap::octet_off(r)];
+  reduce_all<A, 8>(ar, v);
+  if constexpr (PRE) {
+    gs_stage_pre<A, 8, 0>(ar, v, pre->b0);
+    gs_stage_pre<A, 8, 1>(ar, v, pre->b1);
+    gs_stage_pre<A, 8, 2>(ar, v, pre->b2);
+  } else {
+    gs_stage<A, 8, 0>(ar, v, (mh >> 3) + (half << 7) + (cm.h << 2));
+    gs_stage<A, 8, 1>(ar, v, (mh >> 4) + (half << 6) + (cm.h << 1));
+    gs_stage<A, 8, 2>(ar, v, (mh >> 5) + (half << 5) + (cm.h << 0));
+  }
+#pragma unroll
+  for (int r = 0; r < 8; ++r) lds[cm.octet + ChunkMap::octet_off(r)] = v[r];
+  wave_sync();  // the words read next were written by this wave
+  // spans 64, 128, 256
+#pragma unroll
+  for (int r = 0; r < 8; ++r) v[r] = lds[cm.wave + ChunkMap::wave_off(r)];
+  reduce_all<A, 8>(ar, v);
+  if constexpr (PRE) {
+    gs_stage_pre<A, 8, 0>(ar, v, pre->c0);
+    gs_stage_pre<A, 8, 1>(ar, v, pre->c1);
+    gs_stage_pre<A, 8, 2>(ar, v, pre->c2);
+  } else {
+    gs_stage<A, 8, 0>(ar, v, (mh >> 6) + (half << 4) + (cm.wv << 2));
+    gs_stage<A, 8, 1>(ar, v, (mh >> 7) + (half << 3) + (cm.wv << 1));
+    gs_stage<A, 8, 2>(ar, v, (mh >> 8) + (half << 2) + (cm.wv << 0));
+  }
+#pragma unroll
+  for (int r = 0; r < 8; ++r) lds[cm.wave + ChunkMap::wave_off(r)] = v[r];
+  __syncthreads();
+  // spans 512 and 1024; twiddles are uniform over the work-group
+#pragma unroll
+  for (int r = 0; r < 8; ++r) v[r] = lds[cm.wide + half_word(r) + half_word(r) / 16];
+  reduce_all<A, 8>(ar, v);
+  {
+    typename A::TWL two[2], tw[4];
+    if constexpr (PRE) {
+      two[0] = pre->d0[0];
+      two[1] = pre->d0[1];
+    } else {
+      ar.template load_tw<2>((mh >> 9) + (half << 1), two);
+    }
+    tw[0] = tw[2] = two[0];
+    tw[1] = tw[3] = two[1];
+    gs_stage_pre<A, 8, 0>(ar, v, tw);
+    if constexpr (PRE) two[0] = pre->d1[0];
+    else ar.template load_tw<1>((mh >> 10) + half, two);
+    two[1] = two[0];
+    gs_stage_pre<A, 8, 1>(ar, v, two);
+  }
+#pragma unroll
+  for (int r = 0; r < 8; ++r) out[r] = ar.out_mid(v[r]);
+}
 template <class A>
 __device__ __forceinline__ void inv_half_body(u64* lds_words, const DevCtx& c, const PolySeq& dsts,
                                               const PolySeq& srcs, const LimbMap& pos, u32 half, u32 limb, u32 poly,
                                               u32 pi) {
-  typedef typename A::T T;
-  T* lds = reinterpret_cast<T*>(lds_words);
   const int t = threadIdx.x;
   const u64 off = (u64)pos.prime[limb] * c.N + (u64)half * kHalf;
   A ar;
   ar.init(c, pi, true, nullptr, 0);
   const ChunkMap cm(t);
-  const u32 mh = c.N >> 1;  // groups at span 1
   u64 raw[8];
   {
     const ulonglong2* src2 = reinterpret_cast<const ulonglong2*>(srcs.at(poly) + off + 8 * t);
@@ -783,56 +997,11 @@ __device__ __forceinline__ void inv_half_body(u64* lds_words, const DevCtx& c, c
       raw[2 * k + 1] = x.y;
     }
   }
-  u64* dst = dsts.at(poly);
-  T v[8];
+  u64 out[8];
+  inv_half_rounds<A, false>(reinterpret_cast<typename A::T*>(lds_words), ar, cm, c.N >> 1, half, raw, out, nullptr);
+  u64* dst = dsts.at(poly) + off + t;
 #pragma unroll
-  for (int r = 0; r < 8; ++r) v[r] = ar.in_canon(raw[r]);
-  // spans 1, 2, 4
-  gs_stage<A, 8, 0>(ar, v, (mh >> 0) + (half << 10) + ((u32)t << 2));
-  gs_stage<A, 8, 1>(ar, v, (mh >> 1) + (half << 9) + ((u32)t << 1));
-  ar.recentre_sum_of_four(v[0]);
-  ar.recentre_sum_of_four(v[4]);
-  gs_stage<A, 8, 2>(ar, v, (mh >> 2) + (half << 8) + ((u32)t << 0));
-#pragma unroll
-  for (int r = 0; r < 8; ++r) lds[cm.narrow + ChunkMap::narrow_off(r)] = v[r];
-  wave_sync();  // the words read next were written by this wave
-  // spans 8, 16, 32
-#pragma unroll
-  for (int r = 0; r < 8; ++r) v[r] = lds[cm.octet + ChunkMap::octet_off(r)];
-  reduce_all<A, 8>(ar, v);
-  gs_stage<A, 8, 0>(ar, v, (mh >> 3) + (half << 7) + (cm.h << 2));
-  gs_stage<A, 8, 1>(ar, v, (mh >> 4) + (half << 6) + (cm.h << 1));
-  gs_stage<A, 8, 2>(ar, v, (mh >> 5) + (half << 5) + (cm.h << 0));
-#pragma unroll
-  for (int r = 0; r < 8; ++r) lds[cm.octet + ChunkMap::octet_off(r)] = v[r];
-  wave_sync();  // the words read next were written by this wave
-  // spans 64, 128, 256
-#pragma unroll
-  for (int r = 0; r < 8; ++r) v[r] = lds[cm.wave + ChunkMap::wave_off(r)];
-  reduce_all<A, 8>(ar, v);
-  gs_stage<A, 8, 0>(ar, v, (mh >> 6) + (half << 4) + (cm.wv << 2));
-  gs_stage<A, 8, 1>(ar, v, (mh >> 7) + (half << 3) + (cm.wv << 1));
-  gs_stage<A, 8, 2>(ar, v, (mh >> 8) + (half << 2) + (cm.wv << 0));
-#pragma unroll
-  for (int r = 0; r < 8; ++r) lds[cm.wave + ChunkMap::wave_off(r)] = v[r];
-  __syncthreads();
-  // spans 512 and 1024; twiddles are uniform over the work-group
-  constexpr auto word = [](int r) constexpr { return 256 * ((r >> 2) & 1) + 512 * (r & 1) + 1024 * ((r >> 1) & 1); };
-#pragma unroll
-  for (int r = 0; r < 8; ++r) v[r] = lds[cm.wide + word(r) + word(r) / 16];
-  reduce_all<A, 8>(ar, v);
-  {
-    typename A::TWL two[2], tw[4];
-    ar.template load_tw<2>((mh >> 9) + (half << 1), two);
-    tw[0] = tw[2] = two[0];
-    tw[1] = tw[3] = two[1];
-    gs_stage_pre<A, 8, 0>(ar, v, tw);
-    ar.template load_tw<1>((mh >> 10) + half, two);
-    two[1] = two[0];
-    gs_stage_pre<A, 8, 1>(ar, v, two);
-  }
-#pragma unroll
-  for (int r = 0; r < 8; ++r) stg<512>(dst + off + t + word(r), ar.out_mid(v[r]));
+  for (int r = 0; r < 8; ++r) stg<512>(dst + half_word(r), out[r]);
 }
 __global__ __launch_bounds__(kHalfThreads, kChunkWaves) void ntt_inv_half(DevCtx c, PolySeq dsts, PolySeq srcs, LimbMap lm,
                                                                        LimbMap pos, u32 n_limbs, u32 n_polys) {
@@ -842,6 +1011,72 @@ __global__ __launch_bounds__(kHalfThreads, kChunkWaves) void ntt_inv_half(DevCtx
   const u32 pi = lm.prime[limb];
   if (c.fp_ok[pi]) inv_half_body<ArithFp>(lds, c, dsts, srcs, pos, half, limb, poly, pi);
   else inv_half_body<ArithInt>(lds, c, dsts, srcs, pos, half, limb, poly, pi);
+}
+
+// The same pass for launches of many polynomials whose limbs are all on the FP64 back end: a work-group takes the same
+// half of the same limb of `run` polynomials one after the other, and the words of the next one are on their way
+// into LDS (16-byte loads that write LDS directly, no registers held) while the current one is transformed.  A wave's
+// loads fill its own 4 KiB of the staging array, 1 KiB per instruction: instruction j brings the j-th 16 bytes of every
+// lane's 64, so that a lane finds its eight words with four 16-byte LDS reads that are contiguous over the lanes.  Only
+// the wave itself reads what its loads wrote, so no barrier guards the staging array.
+// Vector memory operations complete in the order of issue, so any load issued after the staging loads would wait for
+// them: the thread's 24 twiddles are therefore loaded once, ahead of the loop (they are the same for every
+// polynomial), and the one wait of an iteration lets the eight stores issued after the staging loads stay outstanding
+// (`vmcnt(8)`: at most the eight youngest operations pending, hence the four loads done).  The staging loads are issued from inline
+// assembly: issued through the compiler's builtin, every LDS access after them (the exchanges through the other array
+// included) is made to wait for them.  The compiler does not count these loads; its own counts are then too low, which
+// makes its waits longer than needed, never shorter, and inside the loop it has no load of its own to wait for.
+// 33 KiB of LDS per work-group: four work-groups, 16 waves, per CU, each with 16 KiB on the way for most of its time.
+__device__ __forceinline__ void inv_half_run_body(double* lds, u64* stage, const DevCtx& c, const PolySeq& dsts,
+                                                  const PolySeq& srcs, const LimbMap& pos, u32 n_polys, u32 run,
+                                                  u32 half, u32 limb, u32 pblk, u32 pi) {
+  typedef ArithFp A;
+  const int t = threadIdx.x;
+  const u32 poly0 = pblk * run;
+  const u32 cnt = min(run, n_polys - poly0);
+  const u64 off = (u64)pos.prime[limb] * c.N + (u64)half * kHalf;
+  A ar;
+  ar.init(c, pi, true, nullptr, 0);
+  const ChunkMap cm(t);
+  u64* mine = stage + cm.wv * 512;  // this wave's four blocks of 128 words
+  auto request = [&](u32 poly) {
+    const u64* src = srcs.at(poly) + off + 8 * t;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) stage_request(src + 2 * j, mine + 128 * j);
+  };
+  HalfTw<A> tw;
+  tw.load(ar, cm, c.N >> 1, half, (u32)t);
+  tw.settle();
+  request(poly0);
+  for (u32 it = 0; it < cnt; ++it) {
+    // this polynomial's words are in LDS: its four loads are older than the eight stores of the previous one, and
+    // before the first polynomial nothing was issued after them
+    if (it == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    u64 raw[8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const ulonglong2 x = *reinterpret_cast<const ulonglong2*>(mine + 128 * j + 2 * (t & 63));
+      raw[2 * j] = x.x;
+      raw[2 * j + 1] = x.y;
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // ... and in registers, before the next ones overwrite them
+    if (it + 1 < cnt) request(poly0 + it + 1);
+    u64 out[8];
+    inv_half_rounds<A, true>(lds, ar, cm, c.N >> 1, half, raw, out, &tw);
+    u64* dst = dsts.at(poly0 + it) + off + t;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) stg<512>(dst + half_word(r), out[r]);
+    __syncthreads();  // the next polynomial's first round writes words other waves still read
+  }
+}
+__global__ __launch_bounds__(kHalfThreads, 4) void ntt_inv_half_run(DevCtx c, PolySeq dsts, PolySeq srcs, LimbMap lm,
+                                                                  LimbMap pos, u32 n_limbs, u32 n_polys, u32 run) {
+  __shared__ double lds[kHalf + kHalf / 16];
+  __shared__ __attribute__((aligned(16))) u64 stage[kHalf];
+  u32 half, limb, pblk;
+  if (!chunk_block<kLogHalf>(c, n_limbs, (n_polys + run - 1) / run, half, limb, pblk)) return;
+  inv_half_run_body(lds, stage, c, dsts, srcs, pos, n_polys, run, half, limb, pblk, lm.prime[limb]);
 }
 
 // inverse, strided pass: spans 4096..N/2, then scale every word by the limb's
@@ -1017,6 +1252,37 @@ static bool split_strided(const DevCtx& c, const LimbMap& lm, u32 n_limbs, u32 n
     if (!c.fp_ok[lm.prime[t]]) return true;
   return false;
 }
+// How many polynomials a work-group of a run kernel takes one after the other: eight, or four where eight would leave
+// fewer than two rounds of work-groups for the `resident` that fit the machine at once; 0 = too few polynomials for runs.
+constexpr u32 kCUs = 256;  // MI355X
+static u32 run_length(u32 groups, u32 n_polys, u32 resident) {
+  for (u32 run : {8u, 4u})
+    if (n_polys >= 2 * run && (u64)groups * ((n_polys + run - 1) / run) >= 2ull * resident) return run;
+  return 0;
+}
+static bool all_fp(const DevCtx& c, const LimbMap& lm, u32 n_limbs) {
+  for (u32 t = 0; t < n_limbs; ++t)
+    if (!c.fp_ok[lm.prime[t]]) return false;
+  return true;
+}
+// Whether a work-group may ask for its next polynomial's words before it has stored the current one's: in place (a
+// polynomial's words are read before any of them is written, and polynomials of a sequence do not overlap), or source
+// and destination apart altogether.
+static bool in_place_or_apart(const DevCtx& c, const PolySeq& dst, const PolySeq& src, const LimbMap& pos, u32 n_limbs,
+                              u32 n_polys) {
+  if (dst.b[0] == src.b[0] && dst.b[1] == src.b[1] && dst.pair_stride == src.pair_stride) return true;
+  u64 top = 0;
+  for (u32 t = 0; t < n_limbs; ++t) top = std::max<u64>(top, pos.prime[t]);
+  const u64 words = (top + 1) * c.N;
+  auto span = [&](const PolySeq& q, const u64*& lo, const u64*& hi) {
+    lo = std::min(q.b[0], q.b[1]);
+    hi = std::max(q.b[0], q.b[1]) + (u64)((n_polys - 1) >> 1) * q.pair_stride + words;
+  };
+  const u64 *dl, *dh, *sl, *sh;
+  span(dst, dl, dh);
+  span(src, sl, sh);
+  return dh <= sl || sh <= dl;
+}
 template <int LOGR, int SF, int SI>
 static void run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolySeq& src, const LimbMap& lm,
                       const LimbMap& pos, u32 n_limbs, u32 n_polys, bool inverse, const u64* scale, int passes,
@@ -1043,7 +1309,17 @@ static void run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst, const
     }
     if (passes & 2) {
       const u32 lr = LOGR;
-      if (f.epi == 0)
+      static const bool runs = [] {
+        const char* e = getenv("ACE_NTT_FWD_RUN");
+        return !e || e[0] != '0';
+      }();
+      // (the chunk pass works in place on dst, which the strided pass has filled)
+      const u32 run = runs && f.epi == 0 && SHIFT == 0 && all_fp(c, lm, n_limbs)
+                          ? run_length(n_limbs * (c.N >> kLogChunk), n_polys, 2 * kCUs) : 0;
+      if (run)
+        hipLaunchKernelGGL(ntt_fwd_chunk_run, dim3(chunk_grid(c, n_limbs, (n_polys + run - 1) / run)),
+                           dim3(kChunkThreads), 0, st, c, dst, lm, pos, lr, n_limbs, n_polys, run);
+      else if (f.epi == 0)
         hipLaunchKernelGGL((ntt_fwd_chunk<0, SHIFT>), gc, dim3(kChunkThreads), 0, st, c, dst, lm, pos, lr, n_limbs,
                            n_polys, f);
       else if (f.epi == 1)
@@ -1061,9 +1337,19 @@ static void run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst, const
         const char* e = getenv("ACE_NTT_INV_HALF");
         return !e || e[0] != '0';
       }();
+      static const bool runs = [] {
+        const char* e = getenv("ACE_NTT_INV_RUN");
+        return !e || e[0] != '0';
+      }();
+      const u32 run = SHIFT == 1 && halves && runs && !copies.seq.b[0] && all_fp(c, lm, n_limbs) &&
+                              in_place_or_apart(c, dst, src, pos, n_limbs, n_polys)
+                          ? run_length(n_limbs * (c.N >> kLogHalf), n_polys, 4 * kCUs) : 0;
       if (copies.seq.b[0])
         hipLaunchKernelGGL((ntt_inv_chunk<SHIFT, 1>), gc, dim3(kChunkThreads), 0, st, c, dst, src, copies, lm, pos,
                            n_limbs, n_polys);
+      else if (run)
+        hipLaunchKernelGGL(ntt_inv_half_run, dim3(chunk_grid(c, n_limbs, (n_polys + run - 1) / run, kLogHalf)),
+                           dim3(kHalfThreads), 0, st, c, dst, src, lm, pos, n_limbs, n_polys, run);
       else if (SHIFT == 1 && halves)
         hipLaunchKernelGGL(ntt_inv_half, dim3(chunk_grid(c, n_limbs, n_polys, kLogHalf)), dim3(kHalfThreads), 0, st, c,
                            dst, src, lm, pos, n_limbs, n_polys);

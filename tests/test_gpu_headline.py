@@ -128,3 +128,51 @@ def test_ntt_batch_of_32_polynomials(big):
     for p in check:
         eq(x.view(p * per_poly, per_poly), hosts[p], "round trip, polynomial %d" % p)
     x.free()
+
+
+@pytest.mark.parametrize("polys,limbs,stride", [(16, 24, 24), (19, 24, 24), (17, 24, 25), (33, 3, 3)])
+def test_transforms_of_many_polynomials_equal_single_transforms(big, polys, limbs, stride):
+    """Launches large enough to fill the machine twice over, with all limbs below 2^50.2, take the chunk passes that
+    work through runs of eight or four polynomials with the next one's words on their way into LDS (ace_ntt.hip:
+    ntt_fwd_chunk_run, ntt_inv_half_run, run_length); smaller ones (the last case) take the one-polynomial kernels.
+    Every polynomial of the batch must come out as it does alone: in place and into another buffer, counts that the
+    run length does not divide, a gap limb between the polynomials that must survive, and two of them against the
+    oracle."""
+    g, o, _, _ = big
+    import seeded
+    N = g.N
+    idx = list(range(limbs))
+    per, gap = stride * N, (stride - limbs) * N
+    host = np.zeros(polys * per, np.int64)
+    marker = np.arange(N, dtype=np.int64) * 3 + 1
+    for p in range(polys):
+        host[p * per:p * per + limbs * N] = seeded.uniform_poly(3000 + p, g.primes[:limbs], N)
+        if gap:
+            host[p * per + limbs * N:(p + 1) * per] = marker
+    x, y, one = g.upload(host), g.upload(np.zeros(polys * per, np.int64)), g.alloc(limbs * N)
+    g.ntt(y, x, idx, n_polys=polys, poly_stride_limbs=stride)      # into another buffer
+    g.ntt(x, x, idx, n_polys=polys, poly_stride_limbs=stride)      # in place
+    fwd = x.get()
+    for p in range(polys):
+        s = slice(p * per, p * per + limbs * N)
+        one.set(host[s])
+        g.ntt(one, one, idx)
+        eq(fwd[s], one.get(), "forward in place, polynomial %d" % p)
+        eq(y.view(p * per, limbs * N), fwd[s], "forward into another buffer, polynomial %d" % p)
+        if gap:
+            eq(fwd[p * per + limbs * N:(p + 1) * per], marker, "gap limb after polynomial %d" % p)
+    for p in (0, polys - 1):
+        s = slice(p * per, p * per + limbs * N)
+        eq(fwd[s], o.ntt(host[s], idx), "forward against the oracle, polynomial %d" % p)
+    y.set(np.zeros(polys * per, np.int64))
+    g.intt(y, x, idx, n_polys=polys, poly_stride_limbs=stride)     # into another buffer
+    g.intt(x, x, idx, n_polys=polys, poly_stride_limbs=stride)     # in place
+    back = x.get()
+    for p in range(polys):
+        s = slice(p * per, p * per + limbs * N)
+        eq(back[s], host[s], "round trip in place, polynomial %d" % p)
+        eq(y.view(p * per, limbs * N), host[s], "inverse into another buffer, polynomial %d" % p)
+        if gap:
+            eq(back[p * per + limbs * N:(p + 1) * per], marker, "gap limb after the inverse, polynomial %d" % p)
+    for b in (x, y, one):
+        b.free()
