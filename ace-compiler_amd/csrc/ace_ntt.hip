@@ -412,41 +412,47 @@ __global__ __launch_bounds__(256, 4) void ntt_fwd_strided(DevCtx c, PolySeq dsts
 // Work-group -> (chunk, limb, polynomial slot) for the chunk passes.  The grid
 // is one-dimensional.  Hardware hands consecutive work-groups to the 8 XCDs in
 // turn and each XCD has its own 4 MiB L2.  The map below gives every XCD whole
-// (limb, chunk) groups and runs the polynomials of a group back to back on that
-// XCD, so the group's 32 KiB of twiddles is fetched from HBM once per launch
-// instead of once per polynomial.  (Measured with FETCH_SIZE on a 32-polynomial
-// batch at N=2^16, 24 primes: 12 MiB of twiddle fetches with this map, 230 MiB
-// with groups varying fastest, where 4.6 MB of streaming data passes through the
-// L2 between two uses of the same twiddles.)
-// SLOT_MAJOR (the run kernels, whose work-groups load their twiddles once for a run of polynomials): the groups of
-// an XCD run back to back for the first slot, then for the second, ...  Work-groups that run at the same time then
-// touch different limbs and chunks of a few polynomials instead of the same chunk of many polynomials, whose addresses
-// differ by multiples of the polynomial stride and crowd the same memory channels (chunk passes of the 768-limb batch:
-// 0.149 -> 0.141 ms forward, 0.159 -> 0.148 ms inverse; the twiddles are fetched once per slot instead of once).
+// (limb, chunk) groups, so that the polynomials of a group find the group's
+// 32 KiB of twiddles in that L2.  (Measured with FETCH_SIZE on a 32-polynomial
+// batch at N=2^16, 24 primes: 12 MiB of twiddle fetches with all polynomials of
+// a group back to back, 230 MiB with groups varying fastest over all XCDs, where
+// 4.6 MB of streaming data passes through the L2 between two uses of the same
+// twiddles.)
+// Within an XCD the slots of a group (its polynomials, or runs of them) are not all run back to back: work-groups
+// that run at the same time would then touch the same chunk of many polynomials, whose addresses differ by multiples
+// of the polynomial stride and crowd the same memory channels (chunk passes of the 768-limb batch in runs: 0.149 ->
+// 0.141 ms forward, 0.159 -> 0.148 ms inverse).  The groups of an XCD are visited `visit` slots at a time: all groups
+// for the first `visit` slots, then all groups for the next ones.  One slot per visit for the run kernels (SLOT_MAJOR),
+// whose work-groups keep their twiddles in registers over a run; ACE_NTT_VISIT (4) for the others where a group has
+// at least twice as many slots, so that a group's twiddles are in the L2 for the few work-groups that share them at a
+// time and come from the memory-side cache on later visits; all slots (the plain limb-major order) otherwise.
+#ifndef ACE_NTT_VISIT
+#define ACE_NTT_VISIT 4
+#endif
+template <bool SLOT_MAJOR>
+__host__ __device__ __forceinline__ u32 chunk_visit(u32 slots_per_group) {
+  if (SLOT_MAJOR) return 1;
+  return slots_per_group >= 2 * ACE_NTT_VISIT ? ACE_NTT_VISIT : slots_per_group;
+}
 template <int LOGC = kLogChunk, bool SLOT_MAJOR = false>
 __device__ __forceinline__ bool chunk_block(const DevCtx& c, u32 n_limbs, u32 slots_per_group, u32& chunk,
                                             u32& limb, u32& slot_in_group) {
   const u32 n_chunks = c.N >> LOGC, n_groups = n_limbs * n_chunks;
   const u32 id = blockIdx.x, xcd = id & 7, slot = id >> 3;
-  u32 grp;
-  if (SLOT_MAJOR) {
-    const u32 per_xcd = (n_groups + 7) / 8;
-    grp = (slot % per_xcd) * 8 + xcd;
-    slot_in_group = slot / per_xcd;
-  } else {
-    grp = (slot / slots_per_group) * 8 + xcd;
-    slot_in_group = slot % slots_per_group;
-  }
-  if (grp >= n_groups) return false;
+  const u32 visit = chunk_visit<SLOT_MAJOR>(slots_per_group), per_xcd = (n_groups + 7) / 8;
+  const u32 grp = ((slot / visit) % per_xcd) * 8 + xcd;
+  slot_in_group = (slot / (visit * per_xcd)) * visit + slot % visit;
+  if (grp >= n_groups || slot_in_group >= slots_per_group) return false;
   chunk = grp % n_chunks;
   // last limbs first: where a launch mixes back ends, the special primes (integer back end, 2.5x the work) sit at
   // the end of the limb list and should not be the tail of the launch
   limb = n_limbs - 1 - grp / n_chunks;
   return true;
 }
+template <bool SLOT_MAJOR = false>
 static inline unsigned chunk_grid(const DevCtx& c, u32 n_limbs, u32 slots_per_group, int logc = kLogChunk) {
-  u32 n_groups = n_limbs * (c.N >> logc);
-  return ((n_groups + 7) / 8) * 8 * slots_per_group;
+  const u32 n_groups = n_limbs * (c.N >> logc), visit = chunk_visit<SLOT_MAJOR>(slots_per_group);
+  return ((n_groups + 7) / 8) * 8 * ((slots_per_group + visit - 1) / visit) * visit;
 }
 
 // Polynomials handled by one work-group of a chunk pass.  They share the
@@ -1342,7 +1348,7 @@ static void run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst, const
       const u32 run = runs && f.epi == 0 && SHIFT == 0 && all_fp(c, lm, n_limbs)
                           ? run_length(n_limbs * (c.N >> kLogChunk), n_polys, 2 * kCUs) : 0;
       if (run)
-        hipLaunchKernelGGL(ntt_fwd_chunk_run, dim3(chunk_grid(c, n_limbs, (n_polys + run - 1) / run)),
+        hipLaunchKernelGGL(ntt_fwd_chunk_run, dim3(chunk_grid<true>(c, n_limbs, (n_polys + run - 1) / run)),
                            dim3(kChunkThreads), 0, st, c, dst, lm, pos, lr, n_limbs, n_polys, run);
       else if (f.epi == 0)
         hipLaunchKernelGGL((ntt_fwd_chunk<0, SHIFT>), gc, dim3(kChunkThreads), 0, st, c, dst, lm, pos, lr, n_limbs,
@@ -1373,7 +1379,7 @@ static void run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst, const
         hipLaunchKernelGGL((ntt_inv_chunk<SHIFT, 1>), gc, dim3(kChunkThreads), 0, st, c, dst, src, copies, lm, pos,
                            n_limbs, n_polys);
       else if (run)
-        hipLaunchKernelGGL(ntt_inv_half_run, dim3(chunk_grid(c, n_limbs, (n_polys + run - 1) / run, kLogHalf)),
+        hipLaunchKernelGGL(ntt_inv_half_run, dim3(chunk_grid<true>(c, n_limbs, (n_polys + run - 1) / run, kLogHalf)),
                            dim3(kHalfThreads), 0, st, c, dst, src, lm, pos, n_limbs, n_polys, run);
       else if (SHIFT == 1 && halves)
         hipLaunchKernelGGL(ntt_inv_half, dim3(chunk_grid(c, n_limbs, n_polys, kLogHalf)), dim3(kHalfThreads), 0, st, c,

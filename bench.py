@@ -31,7 +31,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 # HBM bytes per launch of each NTT kernel on this workload, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs of this script, calibrated against the plain copy of the same buffer
 # (profiles/ntt_batch_N65536_L24.md).  Algorithmic bytes per launch are 805306368.
-TRAFFIC_BYTES = {'ntt_fwd_strided': 805492216, 'ntt_fwd_chunk': 818298120, 'ntt_inv_chunk': 818245899, 'ntt_inv_strided': 805688097}
+TRAFFIC_BYTES = {'ntt_fwd_strided': 805524267, 'ntt_fwd_chunk_run': 818408808, 'ntt_inv_half_run': 853094267, 'ntt_inv_strided': 805770728}
 N, LIMBS, POLYS = 65536, 24, 32
 CFG = (N, LIMBS, 50, 50, 3)
 
@@ -470,7 +470,8 @@ def main():
     # FETCH_SIZE / WRITE_SIZE counters of a profiling run are calibrated
     g.copy(scratch, x)
     g.sync()
-    for name, inv, which in (("ntt_fwd_strided", 0, 1), ("ntt_fwd_chunk", 0, 2), ("ntt_inv_chunk", 1, 1),
+    # (the names are those of the kernels these four passes launch on this workload)
+    for name, inv, which in (("ntt_fwd_strided", 0, 1), ("ntt_fwd_chunk_run", 0, 2), ("ntt_inv_half_run", 1, 1),
                              ("ntt_inv_strided", 1, 2)):
         src = x if which == 1 else scratch
         f = lambda: g.ntt_pass(scratch, src, idx, POLYS, LIMBS, inv, which)
