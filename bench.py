@@ -266,6 +266,14 @@ def resnet20_leg():
         again = [float(v) for v in [l for l in r2.stdout.splitlines() if l.startswith("output:")][0].split()[1:]]
         out["logits_first_image"] = logits
         out["logit_spread_under_other_keys"] = max(abs(x - y) for x, y in zip(logits, again))
+        # the same generated program over the plain-float stand-in runtime, on the host: what the logits must be
+        shadow = exe + "_shadow"
+        if os.path.exists(shadow):
+            rs = subprocess.run([shadow, "3", "32", "32", "10", "1"], capture_output=True, text=True, timeout=200, env=env)
+            if rs.returncode == 0:
+                want = [float(v) for v in [l for l in rs.stdout.splitlines() if l.startswith("output:")][0].split()[1:]]
+                out["logits_plain_float_run"] = want
+                out["max_difference_from_plain_float_run"] = round(max(abs(x - y) for x, y in zip(logits, want)), 6)
         return {"resnet20": out}
     except Exception as e:
         return {"resnet20": {"error": repr(e)[:200]}}

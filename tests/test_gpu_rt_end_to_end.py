@@ -259,6 +259,44 @@ def test_reference_resnet20_program_is_stable_under_the_keys():
     assert spread < 1e-3 and spread < 0.01 * max(abs(v) for v in a), spread
 
 
+MODELS_DIR = os.path.join(rt_program.ROOT, "oracle", "_ref", "models")
+
+
+def model_logits(exe, images, env):
+    print("running", exe, "images", images, flush=True)
+    r = subprocess.run([exe, "3", "32", "32", "10", "1", str(images)], capture_output=True, text=True, timeout=140, env=env)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    rows = [[float(v) for v in l.split("output:")[1].split()] for l in r.stdout.splitlines() if l.startswith("output:")]
+    assert len(rows) == images and all(len(row) == 10 for row in rows), r.stdout[-2000:]
+    return rows
+
+
+@pytest.mark.parametrize("model,images", [("resnet20_cifar10_pre.onnx", 2), ("resnet32_cifar10_pre.onnx", 1),
+                                          ("resnet32_cifar100_pre.onnx", 1), ("resnet44_cifar10_pre.onnx", 1),
+                                          ("resnet56_cifar10_pre.onnx", 1), ("resnet110_cifar10_pre.onnx", 1)])
+def test_reference_models_decrypt_to_their_plain_float_run(model, images):
+    """The value-level check of the whole models.  The reference's weight files and expected logits are not in its
+    tree, so the expected output is made here: the same generated program (unchanged) is compiled a second time
+    over a plain-float stand-in for the runtime (tests/programs/shadow/rt_ant/rt_ant.h: a ciphertext is its message,
+    Hw_* act slot by slot, rotations permute slots, Rescale and Bootstrap copy) and run on the host with the same
+    image and the same pseudo-random weights.  The encrypted run on the GPU -- 34 limbs at N = 65536, 197 to 268
+    rotation keys, 19 to 109 bootstraps, the compiler's polynomial ReLUs -- must decrypt to the same ten logits within
+    1e-3, the bound of the reference's own drivers (measured 2e-4 on logits of 0.1 to 1.8).  A rotation by a wrong
+    amount, a plaintext at a wrong level or scale, a lost limb or a wrong key anywhere in the 7 000 to 25 000 lines
+    fails this; so does a bootstrap outside its precision."""
+    gpu, host = os.path.join(MODELS_DIR, model), os.path.join(MODELS_DIR, model + "_shadow")
+    if not (os.path.exists(gpu) and os.path.exists(host)):
+        pytest.skip("built only where the reference tree is present")
+    env = dict(os.environ, RT_HIP_SYNTHETIC_WEIGHTS=AMPLITUDE, MODEL_Q0_BITS="60", MODEL_SF_BITS="56", MODEL_KEY_SEED="11")
+    want = model_logits(host, images, env)
+    got = model_logits(gpu, images, env)
+    for i, (g, w) in enumerate(zip(got, want)):
+        d = max(abs(x - y) for x, y in zip(g, w))
+        print("image", i + 1, "plain float", w, "encrypted", g, "difference %.3g" % d, flush=True)
+        assert max(abs(v) for v in w) > 0.05, "the logits carry no signal"
+        assert d < 1e-3, (i, d)
+
+
 def test_reference_resnet20_program_on_three_threads():
     """Images of a batch on several host threads at once, as the reference's driver runs them
     (dataset/resnet_cifar.main.inc:81-112: `#pragma omp parallel for`, input and output sections critical): one set
