@@ -8,8 +8,8 @@
  * bootstraps' error.  Semantics restated from the reference's program-facing API: include/poly/rns_poly.h:140-468,
  * include/hal/hal.h:24-111 (Hw_* element-wise on one limb), ckks/include/cipher.h, ckks/src/plain.c:29-63 (an encoded
  * vector fills the first `len` slots, the others are zero; a single value fills every slot), porting/pt_mgr.c:188-243
- * (Pt_from_msg: `len` values of entry `index`), common/src/rt_data... io (Prepare_input with the NORMAL scheme: the
- * tensor's values in order).  Weight entries are the reproducible pseudo-random values the runtime substitutes for a
+ * (Pt_from_msg: `len` values of entry `index`); an input tensor under the NORMAL data scheme is its values in order
+ * (the harness fills it in).  Weight entries are the reproducible pseudo-random values the runtime substitutes for a
  * missing weight file (RT_HIP_SYNTHETIC_WEIGHTS=<amplitude>), restated below. */
 #ifndef SHADOW_RT_ANT_H
 #define SHADOW_RT_ANT_H
