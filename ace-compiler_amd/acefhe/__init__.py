@@ -55,6 +55,7 @@ def _sig(lib):
     f("ace_copy", C.c_int, _vp, _vp, _vp, _sz)
     f("ace_zero", C.c_int, _vp, _vp, _sz)
     f("ace_sync", C.c_int, _vp)
+    f("ace_sync_device", C.c_int, _vp)
     f("ace_memory_stats", None, _vp, C.POINTER(C.c_size_t))
     f("ace_ctx_share", _vp, _vp)
     f("ace_fork_release", C.c_int, _vp)
@@ -121,7 +122,7 @@ EXPORTS = [
     "ace_degree", "ace_num_q", "ace_num_p", "ace_num_parts", "ace_part_size", "ace_num_decomp", "ace_prime",
     "ace_root", "ace_modulus", "ace_host_twiddles", "ace_host_tbl_modup", "ace_host_tbl_moddown",
     "ace_host_tbl_rescale", "ace_host_automorphism_order", "ace_alloc", "ace_free", "ace_upload", "ace_download",
-    "ace_copy", "ace_zero", "ace_sync", "ace_memory_stats", "ace_ctx_share", "ace_fork_release", "ace_census_mark", "ace_timer_start", "ace_timer_stop_ms", "ace_ntt", "ace_intt", "ace_ntt_pass",
+    "ace_copy", "ace_zero", "ace_sync", "ace_sync_device", "ace_memory_stats", "ace_ctx_share", "ace_fork_release", "ace_census_mark", "ace_timer_start", "ace_timer_stop_ms", "ace_ntt", "ace_intt", "ace_ntt_pass",
     "ace_hw_modadd", "ace_hw_modsub", "ace_hw_modmul", "ace_hw_modmuladd", "ace_hw_modadd_scalar",
     "ace_hw_modsub_scalar", "ace_hw_modmul_scalar", "ace_hw_modmuladd_scalar", "ace_hw_rotate",
     "ace_find_automorphism_index", "ace_automorphism_order", "ace_poly_add", "ace_poly_sub", "ace_poly_mul",

@@ -1707,6 +1707,11 @@ int ace_sync(ace_ctx* c) {
   c->check_deferred();
   ACE_CATCH_INT
 }
+int ace_sync_device(ace_ctx* c) {
+  ACE_TRY_BARE
+  HIP_OK(hipDeviceSynchronize());
+  ACE_CATCH_INT
+}
 // ---- two lanes ------------------------------------------------------------------
 int ace_fork(ace_ctx* c) {
   ACE_TRY

@@ -958,6 +958,7 @@ static void eval_approx_mod_pair(CIPHER a, CIPHER b) {
     eval_approx_mod(b);
     return;
   }
+  Rt_plaintexts_settle(); /* the second stream may be encoding weight plaintexts ahead of the program */
   ACE_OK(ace_fork(RT_CTX));
   eval_approx_mod(b);
   ACE_OK(ace_fork_switch(RT_CTX));

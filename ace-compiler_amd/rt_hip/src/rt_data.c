@@ -111,6 +111,7 @@ static void cache_clear(void) {
   memset(&Cache, 0, sizeof(Cache));
 }
 
+static void flight_land(void);
 bool Pt_mgr_init(const char* fname) {
   const char* gb    = getenv("RT_HIP_PLAINTEXT_CACHE_GB");
   cache_clear();
@@ -155,6 +156,7 @@ bool Pt_mgr_init(const char* fname) {
 }
 
 void Pt_mgr_fini(void) {
+  flight_land();
   cache_clear();
   if (Data.pt)
     for (uint64_t i = 0; i < Data.hdr.ent_count; ++i)
@@ -199,29 +201,43 @@ static double* entry_values(uint32_t index, size_t first, size_t len) {
 }
 
 /* the entry's values where they lie (floats or doubles of the file, possibly unaligned: only ever copied) */
+/* room in the table of synthetic entries for the indices below `count` (one thread at a time) */
+static void synthetic_reserve(size_t count) {
+  if (count <= Data.syn_count) return;
+  size_t n     = count + 64;
+  Data.syn     = (double**)realloc(Data.syn, n * sizeof(double*));
+  Data.syn_len = (size_t*)realloc(Data.syn_len, n * sizeof(size_t));
+  for (size_t i = Data.syn_count; i < n; ++i) {
+    Data.syn[i]     = NULL;
+    Data.syn_len[i] = 0;
+  }
+  Data.syn_count = n;
+}
+/* the values of one entry up to `upto`; entries are independent of each other */
+static void synthetic_fill(uint32_t index, size_t upto) {
+  if (Data.syn_len[index] >= upto) return;
+  Data.syn[index] = (double*)realloc(Data.syn[index], upto * sizeof(double));
+  for (size_t i = Data.syn_len[index]; i < upto; ++i) {
+    uint64_t z = ((uint64_t)index << 32 | (uint64_t)i) + 0x9E3779B97F4A7C15ull;
+    z          = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z          = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z ^= z >> 31;
+    Data.syn[index][i] = Data.amplitude * ((double)(int64_t)(z >> 11) / (double)(1ull << 52) - 1.0);
+  }
+  Data.syn_len[index] = upto;
+}
 static const double* synthetic_entry(uint32_t index, size_t upto) {
-  if (index >= Data.syn_count) {
-    size_t n     = (size_t)index + 64;
-    Data.syn     = (double**)realloc(Data.syn, n * sizeof(double*));
-    Data.syn_len = (size_t*)realloc(Data.syn_len, n * sizeof(size_t));
-    for (size_t i = Data.syn_count; i < n; ++i) {
-      Data.syn[i]     = NULL;
-      Data.syn_len[i] = 0;
-    }
-    Data.syn_count = n;
-  }
-  if (Data.syn_len[index] < upto) {
-    Data.syn[index] = (double*)realloc(Data.syn[index], upto * sizeof(double));
-    for (size_t i = Data.syn_len[index]; i < upto; ++i) {
-      uint64_t z = ((uint64_t)index << 32 | (uint64_t)i) + 0x9E3779B97F4A7C15ull;
-      z          = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
-      z          = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
-      z ^= z >> 31;
-      Data.syn[index][i] = Data.amplitude * ((double)(int64_t)(z >> 11) / (double)(1ull << 52) - 1.0);
-    }
-    Data.syn_len[index] = upto;
-  }
+  synthetic_reserve((size_t)index + 1);
+  synthetic_fill(index, upto);
   return Data.syn[index];
+}
+/* The entries index .. index + count - 1 made by several host threads: a weight file's entries are there to be
+ * copied, and the values that stand in for them (a hash per value, 100 million of them for ResNet-20) should not
+ * cost a run more than reading the file would. */
+static void synthetic_entries(uint32_t index, size_t count, size_t upto) {
+  synthetic_reserve((size_t)index + count);
+#pragma omp parallel for schedule(static, 1) num_threads(8) if (count > 1)
+  for (size_t n = 0; n < count; ++n) synthetic_fill(index + (uint32_t)n, upto);
 }
 
 static const void* entry_bytes(uint32_t index, size_t first, size_t len, int* is_f32) {
@@ -255,7 +271,7 @@ static bool entry_has(uint32_t index, size_t first, size_t len) {
 static uint64_t cache_key1(uint32_t index, uint32_t scale, uint32_t level) {
   return ((uint64_t)index << 32) | ((uint64_t)(scale & 0xFFFF) << 16) | (level ? level : Get_q_cnt());
 }
-static bool encode_ahead(void* pt, uint32_t index, size_t ofst, size_t len, uint32_t scale, uint32_t level, size_t words) {
+static size_t ahead_count(void) {
   static size_t ahead;
   if (!ahead) {
     const char* env = getenv("RT_HIP_PLAINTEXT_AHEAD");
@@ -263,21 +279,28 @@ static bool encode_ahead(void* pt, uint32_t index, size_t ofst, size_t len, uint
     if (ahead < 1) ahead = 1;
     if (ahead > PT_AHEAD_MAX) ahead = PT_AHEAD_MAX;
   }
-  if (ahead < 2) return false;
-  const uint64_t k2 = ((uint64_t)ofst << 32) | (uint64_t)len;
+  return ahead;
+}
+/* Encodes the entries index, index + 1, ... (up to the first one kept already, at most `ahead_count()`, at least
+ * `at_least`) in one set of launches on the current stream, straight into the kept plaintexts; returns how many. */
+static size_t encode_run(uint32_t index, size_t ofst, size_t len, uint32_t scale, uint32_t level, size_t words,
+                         size_t at_least, int64_t** first) {
+  const size_t   ahead = ahead_count();
+  const uint64_t k2    = ((uint64_t)ofst << 32) | (uint64_t)len;
   const void*    vals[PT_AHEAD_MAX];
   int            is_f32 = 0;
   size_t         n      = 0;
   while (4 * (Cache.count + ahead + 1) > 3 * Cache.cap) cache_grow();
+  if (Data.synthetic && (uint64_t)index + ahead < (1ull << 32)) synthetic_entries(index, ahead, ofst + len);
   for (; n < ahead && (uint64_t)index + n < (1ull << 32); ++n) {
     uint32_t idx = index + (uint32_t)n;
     if (Cache.words + (n + 1) * words > Cache.limit_words || !entry_has(idx, ofst, len)) break;
     if (cache_find(cache_key1(idx, scale, level), k2)->k1) break; /* kept already: the run ends here */
     vals[n] = entry_bytes(idx, ofst, len, &is_f32);
   }
-  if (n < 2) return false;
+  if (n < at_least) return 0;
   int64_t* base = cache_room_run(words, n);
-  if (!base) return false;
+  if (!base) return 0;
   Rt_encode_real_batch(base, words, vals, is_f32, len, n, scale, level);
   for (size_t i = 0; i < n; ++i) {
     PT_CELL* c = cache_find(cache_key1(index + (uint32_t)i, scale, level), k2);
@@ -287,7 +310,64 @@ static bool encode_ahead(void* pt, uint32_t index, size_t ofst, size_t len, uint
     ++Cache.count;
     Cache.words += words;
   }
+  if (first) *first = base;
+  return n;
+}
+
+/* While the program works through one run of entries, the next run is encoded on the library's second stream
+ * (ace_fork / ace_fork_switch): a polynomial's encoding is a dozen launches too small for the machine, like the
+ * products that consume the one before it, and the two overlap.  One run is in flight at a time; the first request
+ * for one of its entries makes the program's stream wait for it (ace_join) and sends off the run after it.  Only
+ * while a single host thread uses the runtime (several threads fill the machine by themselves, and their streams
+ * already share the hardware's queues); RT_HIP_PLAINTEXT_ASYNC=0 keeps every encoding on the program's stream. */
+static struct {
+  bool     active;
+  ace_ctx* ctx; /* the context (of the one thread there was) whose second stream carries the run */
+  uint32_t first, count, scale, level;
+  uint64_t k2;
+} Flight;
+static bool async_encodes(void) {
+  static int off = -1;
+  if (off < 0) off = getenv("RT_HIP_PLAINTEXT_ASYNC") && atoi(getenv("RT_HIP_PLAINTEXT_ASYNC")) == 0;
+  return !off && ahead_count() >= 2 && Rt_lane_count() == 1;
+}
+static void flight_land(void) {
+  if (!Flight.active) return;
+  if (Flight.ctx != RT_CTX) { /* another thread has come since: it cannot join that context's streams, it waits */
+    ACE_OK(ace_sync_device(RT_CTX));
+    return;
+  }
+  ACE_OK(ace_join(RT_CTX));
+  Flight.active = false;
+}
+static void flight_start(uint32_t index, size_t ofst, size_t len, uint32_t scale, uint32_t level, size_t words) {
+  if (Flight.active || !async_encodes()) return;
+  ACE_OK(ace_fork(RT_CTX));
+  size_t n = encode_run(index, ofst, len, scale, level, words, 1, NULL);
+  ACE_OK(ace_fork_switch(RT_CTX));
+  if (!n) {
+    ACE_OK(ace_join(RT_CTX));
+    return;
+  }
+  Flight.active = true;
+  Flight.ctx    = RT_CTX;
+  Flight.first = index, Flight.count = (uint32_t)n, Flight.scale = scale, Flight.level = level;
+  Flight.k2 = ((uint64_t)ofst << 32) | (uint64_t)len;
+}
+/* before anything else uses the second stream, and before the kept plaintexts go away */
+void Rt_plaintexts_settle(void) {
+  Rt_shared_lock();
+  flight_land();
+  Rt_shared_unlock();
+}
+
+static bool encode_ahead(void* pt, uint32_t index, size_t ofst, size_t len, uint32_t scale, uint32_t level, size_t words) {
+  if (ahead_count() < 2) return false;
+  int64_t* base = NULL;
+  size_t   n    = encode_run(index, ofst, len, scale, level, words, 2, &base);
+  if (!n) return false;
   Rt_copy_words(Rt_plain_prepare((PLAIN)pt, scale, level), base, words);
+  flight_start(index + (uint32_t)n, ofst, len, scale, level, words);
   return true;
 }
 
@@ -312,6 +392,16 @@ static void* from_msg_locked(void* pt, uint32_t index, size_t ofst, size_t len, 
     if (4 * (Cache.count + 1) > 3 * Cache.cap) cache_grow();
     cell = cache_find(k1, k2);
     if (cell->k1) { /* encoded before: the polynomial is copied */
+      if (Flight.active && Flight.scale == scale && Flight.level == level && Flight.k2 == k2 && index >= Flight.first &&
+          index - Flight.first < Flight.count) { /* ... once the run it belongs to has landed; the next run goes off */
+        const uint32_t next = Flight.first + Flight.count;
+        int64_t* const dev  = cell->dev;
+        flight_land();
+        flight_start(next, ofst, len, scale, level, words);
+        *added = true;
+        Rt_copy_words(Rt_plain_prepare((PLAIN)pt, scale, level), dev, words);
+        return pt;
+      }
       Rt_copy_words(Rt_plain_prepare((PLAIN)pt, scale, level), cell->dev, words);
       return pt;
     }

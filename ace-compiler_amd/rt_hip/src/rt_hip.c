@@ -42,7 +42,11 @@ struct rt_lane* Rt_lane_slow(void) {
   if (!G.root) Rt_fatal(__FILE__, __LINE__, "Prepare_context() has not run");
   ace_ctx* ctx = ace_ctx_share(G.root);
   if (!ctx) Rt_fatal(__FILE__, __LINE__, "no context for this thread: %s", ace_last_error());
-  return new_lane(ctx);
+  struct rt_lane* lane = new_lane(ctx);
+  /* From here on Rt_shared_publish() waits (the count of lanes is above one); what the first thread built while it
+   * was alone may still be on its way: wait for everything once. */
+  ACE_OK(ace_sync_device(ctx));
+  return lane;
 }
 
 static pthread_mutex_t Shared_lock;
@@ -58,7 +62,11 @@ void Rt_shared_lock(void) {
   pthread_mutex_lock(&Shared_lock);
 }
 void Rt_shared_unlock(void) { pthread_mutex_unlock(&Shared_lock); }
-void Rt_shared_publish(void) { ACE_OK(ace_sync(RT_CTX)); }
+/* What a thread has built for all of them (keys, plaintexts, tables) on its own stream is complete before another
+ * thread, on another stream, can find it; while there is only one thread there is nobody to wait for. */
+void Rt_shared_publish(void) {
+  if (Rt_lane_count() > 1) ACE_OK(ace_sync(RT_CTX));
+}
 
 void Rt_fatal(const char* file, int line, const char* fmt, ...) {
   va_list ap;

@@ -100,6 +100,9 @@ int      ace_download(ace_ctx* ctx, int64_t* host_dst, const int64_t* dev_src, s
 int      ace_copy(ace_ctx* ctx, int64_t* dev_dst, const int64_t* dev_src, size_t n_words);
 int      ace_zero(ace_ctx* ctx, int64_t* dev_dst, size_t n_words);
 int      ace_sync(ace_ctx* ctx);
+/* Waits for every stream of the process on the context's GPU (the contexts of a family and their second lanes): for a
+ * thread that is about to read what another thread's context may still be writing.  Touches no state of `ctx`. */
+int      ace_sync_device(ace_ctx* ctx);
 /* Two lanes.  No counterpart in the reference, whose runtime is synchronous: calls enqueue on one stream per context
  * and therefore run one after another on the GPU, although a single polynomial's kernels do not fill the machine.
  * Where a program has two independent pieces of work (the two sine evaluations of a fully packed bootstrap):
