@@ -144,7 +144,8 @@ float    ace_timer_stop_ms(ace_ctx* ctx); /* synchronises; <0 on error */
  * Polynomial p (0..n_polys-1) limb t (0..n_limbs-1) lives at
  * base + (p*poly_stride_limbs + t)*degree and uses prime prime_idx[t].
  * Forward: natural order in, bit-reversed out.  Inverse: the opposite, 1/N
- * included.  dst may equal src. */
+ * included.  dst may equal src; otherwise the two must not overlap (polynomials of a batch are transformed in any
+ * order, several at a time). */
 int ace_ntt(ace_ctx* ctx, int64_t* dst, const int64_t* src, const int32_t* prime_idx,
             size_t n_limbs, size_t n_polys, size_t poly_stride_limbs);
 int ace_intt(ace_ctx* ctx, int64_t* dst, const int64_t* src, const int32_t* prime_idx,
