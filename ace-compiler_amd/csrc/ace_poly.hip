@@ -928,9 +928,22 @@ __global__ __launch_bounds__(kThreads) void dotprod_shared_key_kernel(
         mac128(h0, l0, x[u][d], k0[u][d]);
         mac128(h1, l1, x[u][d], k1[u][d]);
       }
+      // The lifted tensor terms P a0 b0 and P (a0 b1 + a1 b0) join the sums before their one reduction where the sums
+      // have room for two more products: P a0 and P a1 are reduced (two Shoup products), the three products with
+      // b0 / b1 are not.  The residue of the whole sum is the same word as the sum of the residues.
+      const bool fold = lifted && lift.a0 && sum_terms(P) >= NP + 2;
+      if (fold && i < n) {
+        const u64 o = op * lift.in_stride + dbase + i;
+        const u64 x0 = ldn<2>(lift.a0 + o), x1 = ldn<2>(lift.a1 + o), y0 = ldn<2>(lift.b0 + o), y1 = ldn<2>(lift.b1 + o);
+        const u64 px0 = shoup_mul(x0, lw, lwp, P.q), px1 = shoup_mul(x1, lw, lwp, P.q);
+        mac128(h0, l0, px0, y0);
+        mac128(h1, l1, px0, y1);
+        mac128(h1, l1, px1, y0);
+      }
       if (i < n) {  // NP <= 4 products: below 2^(shift + 64) for every prime below 2^61
         u64 v0 = barrett_sum(h0, l0, P), v1 = barrett_sum(h1, l1, P);
-        if (lifted && lift.a0) {
+        if (fold) {
+        } else if (lifted && lift.a0) {
           const u64 o = op * lift.in_stride + dbase + i;
           const u64 x0 = ldn<2>(lift.a0 + o), x1 = ldn<2>(lift.a1 + o), y0 = ldn<2>(lift.b0 + o), y1 = ldn<2>(lift.b1 + o);
           u64 h = 0, l = 0;  // two products of residues stay below 2^(shift + 64)
