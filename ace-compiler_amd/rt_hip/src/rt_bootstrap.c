@@ -952,13 +952,13 @@ static void eval_approx_mod(CIPHER ct);
 static void eval_approx_mod_pair(CIPHER a, CIPHER b) {
   static int one_lane = -1;
   if (one_lane < 0) one_lane = getenv("RT_HIP_ONE_LANE") && atoi(getenv("RT_HIP_ONE_LANE")) != 0;
+  Rt_plaintexts_settle(); /* the second stream may be encoding weight plaintexts ahead of the program */
   if (one_lane || Rt_lane_count() > 1) {
     if (!one_lane) ACE_OK(ace_fork_release(RT_CTX)); /* a second stream from before the other threads came */
     eval_approx_mod(a);
     eval_approx_mod(b);
     return;
   }
-  Rt_plaintexts_settle(); /* the second stream may be encoding weight plaintexts ahead of the program */
   ACE_OK(ace_fork(RT_CTX));
   eval_approx_mod(b);
   ACE_OK(ace_fork_switch(RT_CTX));
