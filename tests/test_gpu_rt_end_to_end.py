@@ -201,10 +201,12 @@ def test_bootstrap_precision_at_the_model_ring():
 AMPLITUDE = "0.33"
 
 
-def resnet20_run(chain, key_seed, images=1, threads=1, amplitude=AMPLITUDE):
+def resnet20_run(chain, key_seed, images=1, threads=1, amplitude=AMPLITUDE, late_threads=False):
     """logits of each image, in the order of the images"""
     env = dict(os.environ, RT_HIP_SYNTHETIC_WEIGHTS=amplitude, MODEL_Q0_BITS=str(chain[0]), MODEL_SF_BITS=str(chain[1]),
                MODEL_KEY_SEED=str(key_seed), MODEL_THREADS=str(threads))
+    if late_threads:
+        env["MODEL_LATE_THREADS"] = "1"
     print("running", RESNET20, "chain", chain, "key seed", key_seed, "images", images, "threads", threads, flush=True)
     r = subprocess.run([RESNET20, "3", "32", "32", "10", "1", str(images)], capture_output=True, text=True, timeout=230,
                        env=env)
@@ -307,11 +309,14 @@ def test_reference_resnet20_program_on_three_threads():
     if not os.path.exists(RESNET20):
         pytest.skip("built only where the reference tree is present")
     one = resnet20_run((60, 56), 11, images=4)
-    three = resnet20_run((60, 56), 11, images=4, threads=3)
-    for i, (a, b) in enumerate(zip(one, three)):
-        d = max(abs(x - y) for x, y in zip(a, b))
-        print("image", i + 1, "one thread", a, "difference on three threads", d, flush=True)
-        assert d < 1e-3 and d < 0.01 * max(abs(v) for v in a), (i, d)
+    # the second run's other threads first call in after the first image: they meet a runtime that has worked alone
+    # (no waiting after publishing, weight plaintexts of the next run still on their way on its second stream)
+    for late in (False, True):
+        three = resnet20_run((60, 56), 11, images=4, threads=3, late_threads=late)
+        for i, (a, b) in enumerate(zip(one, three)):
+            d = max(abs(x - y) for x, y in zip(a, b))
+            print("image", i + 1, "one thread", a, "difference on three threads", d, "late" if late else "", flush=True)
+            assert d < 1e-3 and d < 0.01 * max(abs(v) for v in a), (i, d, late)
 
 
 @pytest.mark.parametrize("seed", [1, 2, 3])
