@@ -1109,6 +1109,9 @@ void do_precomp(ace_ctx* c, u64* res, u64 res_stride, const u64* src, u64 src_st
   if (!by_transform && !skip_own)
     launch_digit_copy(c->stream, c->d, res, src, (u32)level, (u32)c->h.part_size, (u32)nd, T * N, res_stride,
                       src_stride, (u32)nb);
+  // (large launches of N = 2^16 whose digits fit one conversion launch: conversion and strided pass of the transform
+  // in one kernel)
+  bool strided_done = false;
   for (size_t j0 = 0; j0 < nd; j0 += kMaxConvJobs) {
     ConvBatch b{};
     b.matrix = c->conv_matrix;
@@ -1116,12 +1119,15 @@ void do_precomp(ace_ctx* c, u64* res, u64 res_stride, const u64* src, u64 src_st
     for (u32 k = 0; k < b.n_jobs; ++k) b.job[k] = pd.jobs[j0 + k];
     b.t_stride = level * N;
     b.out_stride = res_stride;
-    launch_baseconv(c->stream, c->d, res, t, b, (u32)nb);
+    if (is_ntt && pd.one_ntt_launch && nd <= (size_t)kMaxConvJobs)
+      strided_done = launch_baseconv_fwd_strided(c->stream, c->d, res, t, b, (u32)nb);
+    if (!strided_done) launch_baseconv(c->stream, c->d, res, t, b, (u32)nb);
   }
   if (is_ntt) {
     PolySeq rs = seq_strided(res, res_stride);
     if (pd.one_ntt_launch) {
-      launch_ntt(c->stream, c->d, rs, rs, pd.tgt_lm, &pd.tgt_pos, pd.n_tgt, (u32)nb, false, nullptr);
+      launch_ntt(c->stream, c->d, rs, rs, pd.tgt_lm, &pd.tgt_pos, pd.n_tgt, (u32)nb, false, nullptr,
+                 strided_done ? 2 : 3);
     } else {
       for (size_t d = 0; d < nd; ++d) {
         const ModUpDev& m = c->modup_at(level, d);
@@ -1156,7 +1162,9 @@ void do_mod_down(ace_ctx* c, const PolySeq& res, const PolySeq& src, size_t np, 
   b.job[0].nc = (u32)level;
   b.t_stride = K * N;
   b.out_stride = level * N;
-  launch_baseconv(c->stream, c->d, y, t, b, (u32)np);
+  // (large launches of N = 2^16: conversion and strided pass of the transform in one kernel)
+  const bool strided_done = is_ntt && launch_baseconv_fwd_strided(c->stream, c->d, y, t, b, (u32)np);
+  if (!strided_done) launch_baseconv(c->stream, c->d, y, t, b, (u32)np);
   if (is_ntt) {
     PolySeq ys = seq_strided(y, level * N);
     bool fits = true;  // index tables of another make go through the separate tail, which takes any table
@@ -1171,12 +1179,13 @@ void do_mod_down(ace_ctx* c, const PolySeq& res, const PolySeq& src, size_t np, 
       f.addend = addend_mode ? *addend : res;
       f.addend_mode = addend_mode;
       f.cst = c->pinv;
-      if (!launch_ntt(c->stream, c->d, ys, ys, c->q_lm, nullptr, (u32)level, (u32)np, false, nullptr, 3, &f))
+      if (!launch_ntt(c->stream, c->d, ys, ys, c->q_lm, nullptr, (u32)level, (u32)np, false, nullptr,
+                      strided_done ? 2 : 3, &f))
         throw std::runtime_error("internal: fused Mod_down transform rejected");
       c->ws_used = mark;
       return;
     }
-    launch_ntt(c->stream, c->d, ys, ys, c->q_lm, nullptr, (u32)level, (u32)np, false, nullptr);
+    launch_ntt(c->stream, c->d, ys, ys, c->q_lm, nullptr, (u32)level, (u32)np, false, nullptr, strided_done ? 2 : 3);
   }
   launch_moddown_tail(c->stream, c->d, res, src, y, level * N, addend_mode ? addend : nullptr, addend_mode, c->pinv,
                       c->q_lm, (u32)level, (u32)np, orders);

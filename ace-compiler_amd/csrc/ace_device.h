@@ -173,6 +173,32 @@ __device__ __forceinline__ u64 sub_mod(u64 a, u64 b, u64 q) {
 }
 
 
+// ---- pieces of the base conversion on the matrix cores shared by its kernels (see baseconv_mx_kernel) ----
+typedef int conv_v16i __attribute__((ext_vector_type(16)));
+typedef int conv_v4i __attribute__((ext_vector_type(4)));
+constexpr u64 kSignedBytes = 0x8080808080808080ull;
+// a source word as the MFMA's B operand takes it: its eight signed bytes (the carries moved up), low half first
+__device__ __forceinline__ void conv_mx_signed(u64 word, bool live, int& lo, int& hi) {
+  const u64 e = live ? (word + kSignedBytes) ^ kSignedBytes : 0;
+  lo = (int)(u32)e;
+  hi = (int)(u32)(e >> 32);
+}
+// the canonical residue mod m of V = sum_p 2^(8p) S[8w + p], the eight byte sums of target w of a lane's pair
+__device__ __forceinline__ u64 conv_mx_residue(const conv_v16i& S, int w, u64 m, double minv) {
+  // byte sums are below 2^21 in size: two of them, one shifted by a byte, fit a 32-bit word
+  const int u0 = S[8 * w + 0] + (S[8 * w + 1] << 8), v0 = S[8 * w + 2] + (S[8 * w + 3] << 8);
+  const int u1 = S[8 * w + 4] + (S[8 * w + 5] << 8), v1 = S[8 * w + 6] + (S[8 * w + 7] << 8);
+  const i64 t0 = (i64)u0 + ((i64)v0 << 16), t1 = (i64)u1 + ((i64)v1 << 16);
+  const u64 v_lo = (u64)t0 + ((u64)t1 << 32);  // V mod 2^64
+  const double d0 = __builtin_fma((double)v0, 65536.0, (double)u0);  // exact
+  const double d1 = __builtin_fma((double)v1, 65536.0, (double)u1);
+  const double vd = __builtin_fma(d1, 4294967296.0, d0);  // V to 53 bits
+  // |V / m| < 2^14 and the estimate is off by far less than 1/2: V - Q m lies within (1/2 + 2^-30) m of zero
+  const int quot = (int)__builtin_rint(vd * minv);
+  const i64 r = (i64)(v_lo - (u64)(i64)quot * m);
+  return (u64)(r < 0 ? r + (i64)m : r);
+}
+
 constexpr int kMaxBatchPtrs = 32;  // keys / index tables per batched launch
 struct OrderSet {  // one automorphism table per rotation, or one shared (n == 1)
   const i64* p[kMaxBatchPtrs];

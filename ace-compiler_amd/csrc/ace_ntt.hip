@@ -409,6 +409,138 @@ __global__ __launch_bounds__(256, 4) void ntt_fwd_strided(DevCtx c, PolySeq dsts
   else fwd_strided_body<ArithInt, LOGR, PRO>(c, dsts, srcs, pos, f, limb, pi);
 }
 
+// ---------------------------------------------------------------------------
+// Base conversion and the forward strided pass of the converted limbs in one kernel (N = 2^16, at most eight source
+// limbs): the conversion's result never goes to memory in coefficient form.  A work-group takes 64 columns of all
+// sixteen rows of one operand (polynomial x digit).  Its four waves hold the source words of four rows each as the
+// matrix product's operands (see baseconv_mx_kernel: a wave converts 64 coefficients of a row as two tiles of 32);
+// the targets are taken four at a time: every wave converts its rows to the quad's targets into LDS
+// ([target][row][column], 32 KiB), then wave w runs the four strided stages of target w of the quad, a column per
+// lane, and stores what ntt_fwd_strided would have stored (centred values for the chunk pass).
+// grid = (N/16/64, operands), 256 threads.
+constexpr int kCfsCols = 64;
+template <class A>
+__device__ __forceinline__ void conv_strided_column(const DevCtx& c, u32 pi, const u64* lds_target, u32 lane,
+                                                    u64* __restrict__ dst, u64 rs) {
+  A ar;
+  ar.init(c, pi, false, nullptr, 0);
+  typename A::T v[16];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) v[r] = ar.in_canon(lds_target[r * kCfsCols + lane]);
+  fwd_strided_stages<A, 4>(ar, v);
+  reduce_all<A, 16>(ar, v);
+#pragma unroll
+  for (int r = 0; r < 16; ++r) stg<1>(dst + r * rs + lane, ar.out_mid(v[r]));
+}
+template <int STEPS>
+__global__ __launch_bounds__(256, 4) void conv_fwd_strided_kernel(DevCtx c, u64* __restrict__ out_base,
+                                                               const u64* __restrict__ t_base, ConvBatch b) {
+  __shared__ __attribute__((aligned(16))) u64 lds[4 * 16 * kCfsCols];
+  const u64 n = c.N, rs = n >> 4;
+  const u32 lane = threadIdx.x & 63, half = lane >> 5;
+  const u32 wv = (u32)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const u32 col0 = blockIdx.x * kCfsCols;
+  const u32 jobi = blockIdx.y % b.n_jobs, op = blockIdx.y / b.n_jobs;
+  const ConvJob& J = b.job[jobi];
+  const u32 nd = J.nd, nc = J.nc;
+  const u64* __restrict__ t = t_base + op * b.t_stride + J.t_off + col0 + 2 * (lane & 31);
+  u64* __restrict__ out = out_base + op * b.out_stride + J.out_off + col0;
+  conv_v4i x[4][2][STEPS];
+  {
+    typedef u64 u64x2 __attribute__((ext_vector_type(2)));
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr) {
+      u64x2 v[STEPS][2];
+#pragma unroll
+      for (int s = 0; s < STEPS; ++s)
+#pragma unroll
+        for (int w = 0; w < 2; ++w) {
+          const u32 k = 4 * s + 2 * half + w;
+          v[s][w] = ldg<2>(reinterpret_cast<const u64x2*>(t + (u64)min(k, nd - 1) * n + (u64)(4 * wv + rr) * rs));
+        }
+#pragma unroll
+      for (int s = 0; s < STEPS; ++s)
+#pragma unroll
+        for (int w = 0; w < 2; ++w) {
+          const bool live = 4 * s + 2 * half + w < nd;
+          int lo, hi;
+          conv_mx_signed(v[s][w].x, live, lo, hi);
+          x[rr][0][s][2 * w] = lo;
+          x[rr][0][s][2 * w + 1] = hi;
+          conv_mx_signed(v[s][w].y, live, lo, hi);
+          x[rr][1][s][2 * w] = lo;
+          x[rr][1][s][2 * w + 1] = hi;
+        }
+    }
+  }
+  const uint4* __restrict__ mx = J.mx + lane;
+  const ConvTarget* __restrict__ mt = J.mt;
+  const u32 quads = (nc + 3) / 4;
+  uint4 row[STEPS];
+#pragma unroll
+  for (int s = 0; s < STEPS; ++s) row[s] = mx[s * 64];
+  for (u32 quad = 0; quad < quads; ++quad) {
+    // the tables end with a spare quad: the next quad's rows are asked for before this one's are used
+    uint4 row_next[STEPS];
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) row_next[s] = mx[((u64)(quad + 1) * kMxSteps + s) * 64];
+    const ConvTarget tg[2] = {mt[quad * 4 + 2 * half], mt[quad * 4 + 2 * half + 1]};
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr) {
+      conv_v16i acc[2];
+#pragma unroll
+      for (u32 tile = 0; tile < 2; ++tile) {
+        acc[tile] = conv_v16i{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) {
+          const conv_v4i a = {(int)row[s].x, (int)row[s].y, (int)row[s].z, (int)row[s].w};
+          acc[tile] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, x[rr][tile][s], acc[tile], 0, 0, 0);
+        }
+      }
+#pragma unroll
+      for (int w = 0; w < 2; ++w) {
+        typedef u64 u64x2 __attribute__((ext_vector_type(2)));
+        const u64x2 pr = {conv_mx_residue(acc[0], w, tg[w].m, tg[w].minv), conv_mx_residue(acc[1], w, tg[w].m, tg[w].minv)};
+        *reinterpret_cast<u64x2*>(lds + ((2 * half + w) * 16 + 4 * wv + rr) * kCfsCols + 2 * (lane & 31)) = pr;
+      }
+    }
+    __syncthreads();
+    const u32 j = quad * 4 + wv;
+    if (j < nc) {  // uniform over the wave
+      const u32 pi = J.map.prime[j];
+      u64* __restrict__ dst = out + (u64)J.map.out_limb[j] * n;
+      if (c.fp_ok[pi]) conv_strided_column<ArithFp>(c, pi, lds + wv * 16 * kCfsCols, lane, dst, rs);
+      else conv_strided_column<ArithInt>(c, pi, lds + wv * 16 * kCfsCols, lane, dst, rs);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) row[s] = row_next[s];
+  }
+}
+
+bool launch_baseconv_fwd_strided(hipStream_t st, const DevCtx& c, u64* out, const u64* t, const ConvBatch& b, u32 n_ops) {
+  static const bool on = [] {
+    const char* e = getenv("ACE_CONV_STRIDED");
+    return !e || e[0] != '0';
+  }();
+  if (!on || !b.matrix || !b.n_jobs || !n_ops || c.logN != 16) return false;
+  u32 max_nd = 0;
+  u64 limbs = 0;
+  for (u32 k = 0; k < b.n_jobs; ++k) {
+    if (!b.job[k].mx || !b.job[k].nc) return false;
+    max_nd = b.job[k].nd > max_nd ? b.job[k].nd : max_nd;
+    limbs += b.job[k].nc;
+  }
+  // launches too small for the machine are better served by the two kernels (the strided pass spread over four waves
+  // a column); more than eight source limbs would not fit the registers
+  if (max_nd > 8 || limbs * n_ops < 192) return false;
+  if ((((uintptr_t)out | (uintptr_t)t) & 15) || ((b.out_stride | b.t_stride) & 1)) return false;
+  dim3 g((u32)(c.N >> 4) / kCfsCols, b.n_jobs * n_ops);
+  if (max_nd <= 4) hipLaunchKernelGGL((conv_fwd_strided_kernel<1>), g, dim3(256), 0, st, c, out, t, b);
+  else hipLaunchKernelGGL((conv_fwd_strided_kernel<2>), g, dim3(256), 0, st, c, out, t, b);
+  return true;
+}
+
 // Work-group -> (chunk, limb, polynomial slot) for the chunk passes.  The grid
 // is one-dimensional.  Hardware hands consecutive work-groups to the 8 XCDs in
 // turn and each XCD has its own 4 MiB L2.  The map below gives every XCD whole
@@ -1427,7 +1559,9 @@ bool launch_ntt(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolyS
   }
   FwdFuse f{};
   if (fuse) {
-    if (inverse || c.logN <= kLogChunk || passes != 3) return false;  // only whole forward transforms of N > 4096
+    // only forward transforms of N > 4096: whole ones, or the chunk pass alone with an epilogue, for a caller whose own
+    // kernel has run the strided pass (launch_baseconv_fwd_strided)
+    if (inverse || c.logN <= kLogChunk || !(passes == 3 || (passes == 2 && fuse->pro == 0))) return false;
     f = *fuse;
   }
   LimbMap pos{};

@@ -582,9 +582,6 @@ __global__ __launch_bounds__(kThreads) void baseconv_kernel(DevCtx c, u64* __res
 // that registers 0-7 of a lane are the eight byte sums of target 2 (l / 32) of the quad, registers 8-15 those of target
 // 2 (l / 32) + 1.
 // Source words must be below 2^63 - 2^56 (residues of primes below 2^61 are).
-typedef int conv_v16i __attribute__((ext_vector_type(16)));
-typedef int conv_v4i __attribute__((ext_vector_type(4)));
-constexpr u64 kSignedBytes = 0x8080808080808080ull;
 constexpr u32 kMxThreads = 256, kMxCoefPerBlock = 64 * (kMxThreads / 64);
 
 // one quad of targets for the wave's two tiles; FULL: all four targets exist (no lane is left out, so the stores
@@ -608,21 +605,7 @@ __device__ __forceinline__ void conv_mx_quad(const uint4 (&row)[STEPS], const Co
     const u64 m = tg[w].m;
     u64 res[2];
 #pragma unroll
-    for (u32 tile = 0; tile < 2; ++tile) {
-      const conv_v16i& S = acc[tile];
-      // byte sums are below 2^21 in size: two of them, one shifted by a byte, fit a 32-bit word
-      const int u0 = S[8 * w + 0] + (S[8 * w + 1] << 8), v0 = S[8 * w + 2] + (S[8 * w + 3] << 8);
-      const int u1 = S[8 * w + 4] + (S[8 * w + 5] << 8), v1 = S[8 * w + 6] + (S[8 * w + 7] << 8);
-      const i64 t0 = (i64)u0 + ((i64)v0 << 16), t1 = (i64)u1 + ((i64)v1 << 16);
-      const u64 v_lo = (u64)t0 + ((u64)t1 << 32);  // V mod 2^64
-      const double d0 = __builtin_fma((double)v0, 65536.0, (double)u0);  // exact
-      const double d1 = __builtin_fma((double)v1, 65536.0, (double)u1);
-      const double vd = __builtin_fma(d1, 4294967296.0, d0);  // V to 53 bits
-      // |V / m| < 2^14 and the estimate is off by far less than 1/2: V - Q m lies within (1/2 + 2^-30) m of zero
-      const int quot = (int)__builtin_rint(vd * tg[w].minv);
-      const i64 r = (i64)(v_lo - (u64)(i64)quot * m);
-      res[tile] = (u64)(r < 0 ? r + (i64)m : r);
-    }
+    for (u32 tile = 0; tile < 2; ++tile) res[tile] = conv_mx_residue(acc[tile], w, m, tg[w].minv);
     if (FULL || first_target + w < nc)
     {
       typedef u64 u64x2 __attribute__((ext_vector_type(2)));
@@ -670,12 +653,13 @@ __global__ __launch_bounds__(kMxThreads) void baseconv_mx_kernel(DevCtx c, u64* 
 #pragma unroll
       for (int w = 0; w < 2; ++w) {
         const bool live = 4 * s + 2 * half + w < nd;
-        const u64 e0 = live ? (v[s][w].x + kSignedBytes) ^ kSignedBytes : 0;
-        const u64 e1 = live ? (v[s][w].y + kSignedBytes) ^ kSignedBytes : 0;
-        x[0][s][2 * w] = (int)(u32)e0;
-        x[0][s][2 * w + 1] = (int)(u32)(e0 >> 32);
-        x[1][s][2 * w] = (int)(u32)e1;
-        x[1][s][2 * w + 1] = (int)(u32)(e1 >> 32);
+        int lo, hi;
+        conv_mx_signed(v[s][w].x, live, lo, hi);
+        x[0][s][2 * w] = lo;
+        x[0][s][2 * w + 1] = hi;
+        conv_mx_signed(v[s][w].y, live, lo, hi);
+        x[1][s][2 * w] = lo;
+        x[1][s][2 * w + 1] = hi;
       }
   }
   const uint4* __restrict__ mx = J.mx + (u64)quad0 * kMxSteps * 64 + lane;
