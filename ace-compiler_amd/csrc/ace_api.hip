@@ -1318,7 +1318,6 @@ void do_switch_key_rescale(ace_ctx* c, const PolySeq& out, const u64* digits, u6
   b.job[0] = m.job;
   b.t_stride = (K + 1) * N;
   b.out_stride = level * N;
-  launch_baseconv(c->stream, c->d, y, t + N, b, (u32)np);
   FwdFuse f{};
   f.pro = 2;
   f.last_prime = (u32)(level - 1);
@@ -1333,7 +1332,11 @@ void do_switch_key_rescale(ace_ctx* c, const PolySeq& out, const u64* digits, u6
   f.addend = out;
   f.cst = m.tail;
   PolySeq ys = seq_strided(y, level * N);
-  if (!launch_ntt(c->stream, c->d, ys, ys, c->q_lm, nullptr, (u32)(level - 1), (u32)np, false, nullptr, 3, &f))
+  // (large launches of N = 2^16: conversion, prologue and strided pass of the transform in one kernel)
+  const bool strided_done = launch_baseconv_fwd_strided(c->stream, c->d, y, t + N, b, (u32)np, &f);
+  if (!strided_done) launch_baseconv(c->stream, c->d, y, t + N, b, (u32)np);
+  if (!launch_ntt(c->stream, c->d, ys, ys, c->q_lm, nullptr, (u32)(level - 1), (u32)np, false, nullptr,
+                  strided_done ? 2 : 3, &f))
     throw std::runtime_error("internal: fused Mod_down + Rescale transform rejected");
   c->ws_used = mark;
 }

@@ -146,7 +146,10 @@ void launch_baseconv(hipStream_t st, const DevCtx& c, u64* out, const u64* t, co
 // limb (in place where the conversion would have put it): the caller then runs launch_ntt with passes = 2.  Returns
 // false, having launched nothing, where the two kernels serve better or the shape is not covered (N != 2^16, more
 // than eight source limbs, a job without matrix tables, a launch too small to fill the machine).
-bool launch_baseconv_fwd_strided(hipStream_t st, const DevCtx& c, u64* out, const u64* t, const ConvBatch& b, u32 n_ops);
+// rescale: the FwdFuse of a transform whose prologue is pro 2 (a Mod_down and a Rescale sharing it): the prologue is
+// then carried out here as well, on the conversion's last target (`ylast`, which stays out of the transform).
+bool launch_baseconv_fwd_strided(hipStream_t st, const DevCtx& c, u64* out, const u64* t, const ConvBatch& b, u32 n_ops,
+                                 const FwdFuse* rescale = nullptr);
 // digit limbs of src copied into the raised polynomials (see digit_copy_kernel)
 void launch_digit_copy(hipStream_t st, const DevCtx& c, u64* res, const u64* src, u32 level, u32 part_size,
                        u32 n_digits, u64 digit_stride, u64 res_stride, u64 src_stride, u32 n_ops);

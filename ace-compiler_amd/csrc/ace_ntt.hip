@@ -419,23 +419,85 @@ __global__ __launch_bounds__(256, 4) void ntt_fwd_strided(DevCtx c, PolySeq dsts
 // lane, and stores what ntt_fwd_strided would have stored (centred values for the chunk pass).
 // grid = (N/16/64, operands), 256 threads.
 constexpr int kCfsCols = 64;
+// The input word of FwdFuse::pro 2 from the dropped limb's word `last` (canonical mod q_last) and the converted word y
+// (canonical mod q_t), one word at a time: the arithmetic of fwd_strided_input, whose cases are uniform over a limb.
 template <class A>
+struct SwitchIn {
+  DevPrime P;
+  u64 ql, half, K, Kp, diff;
+  double qld, halfd, kc, kci;
+  int mode;  // 0 FP64 product, 1 q > ql, 2 ql < 2 q, 3 Barrett
+  __device__ __forceinline__ void init(const A& ar, const DevCtx& c, u32 pi, u32 last_prime, const u64* sw, u32 lt) {
+    P = c.primes[pi];
+    ql = c.primes[last_prime].q;
+    half = ql >> 1;
+    K = sw[3 * lt], Kp = sw[3 * lt + 1], diff = sw[3 * lt + 2];
+    mode = P.q > ql ? 1 : ql < 2 * P.q ? 2 : 3;
+    if constexpr (A::kFp) {
+      if (ql < ((u64)1 << 52) && ql <= 2 * P.q) {
+        mode = 0;
+        qld = (double)ql, halfd = (double)half;
+        kc = ar.in_canon(K);
+        if (K > (P.q >> 1)) kc -= ar.q;
+        kci = kc * ar.qinv;
+      }
+    }
+  }
+  __device__ __forceinline__ typename A::T one(const A& ar, u64 last, u64 y) const {
+    if constexpr (A::kFp) {
+      if (mode == 0) {
+        double x = ar.in_canon(last);
+        x = x > halfd ? x - qld : x;
+        typename A::T v = ar.mulmod(x, kc, kci);
+        v += ar.in_canon(y);
+        ar.reduce(v);
+        return v;
+      }
+    }
+    u64 x = last;
+    if (mode == 1) x += x > half ? P.q - ql : 0;
+    else if (mode == 2) x = csub(x + (x > half ? diff : 0), P.q);
+    else x = barrett128(0, x + (x > half ? diff : 0), P);
+    return ar.in_canon(add_mod(shoup_mul(x, K, Kp, P.q), y, P.q));
+  }
+};
+// the Rescale half of a transform that a Mod_down and a Rescale share (FwdFuse::pro 2), for the kernel below
+struct ConvRescale {
+  const u64* z;  // null: a plain conversion
+  u64 z_stride;
+  const u64* sw;
+  u32 last_prime;
+};
+template <class A, bool SWITCH>
 __device__ __forceinline__ void conv_strided_column(const DevCtx& c, u32 pi, const u64* lds_target, u32 lane,
-                                                    u64* __restrict__ dst, u64 rs) {
+                                                    u64* __restrict__ dst, u64 rs, const ConvRescale& rz,
+                                                    const u64* lds_last, u32 lt) {
   A ar;
   ar.init(c, pi, false, nullptr, 0);
   typename A::T v[16];
+  if constexpr (SWITCH) {
+    SwitchIn<A> in;
+    in.init(ar, c, pi, rz.last_prime, rz.sw, lt);
 #pragma unroll
-  for (int r = 0; r < 16; ++r) v[r] = ar.in_canon(lds_target[r * kCfsCols + lane]);
+    for (int r = 0; r < 16; ++r) v[r] = in.one(ar, lds_last[r * kCfsCols + lane], lds_target[r * kCfsCols + lane]);
+  } else {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) v[r] = ar.in_canon(lds_target[r * kCfsCols + lane]);
+  }
   fwd_strided_stages<A, 4>(ar, v);
   reduce_all<A, 16>(ar, v);
 #pragma unroll
   for (int r = 0; r < 16; ++r) stg<1>(dst + r * rs + lane, ar.out_mid(v[r]));
 }
-template <int STEPS>
+// SWITCH: the conversion's last target is not transformed; it is the `ylast` of FwdFuse::pro 2, and every other
+// target's transform starts from Switch_modulus(z - ylast) * sw + (converted word), as ntt_fwd_strided<., 2> forms it.
+// The quad that holds the last target goes first, and z - ylast stays in LDS (8 KiB more) for the other quads.
+template <int STEPS, bool SWITCH>
 __global__ __launch_bounds__(256, 4) void conv_fwd_strided_kernel(DevCtx c, u64* __restrict__ out_base,
-                                                               const u64* __restrict__ t_base, ConvBatch b) {
+                                                               const u64* __restrict__ t_base, ConvBatch b,
+                                                               ConvRescale rz) {
   __shared__ __attribute__((aligned(16))) u64 lds[4 * 16 * kCfsCols];
+  __shared__ u64 lds_last[SWITCH ? 16 * kCfsCols : 1];
   const u64 n = c.N, rs = n >> 4;
   const u32 lane = threadIdx.x & 63, half = lane >> 5;
   const u32 wv = (u32)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
@@ -476,14 +538,19 @@ __global__ __launch_bounds__(256, 4) void conv_fwd_strided_kernel(DevCtx c, u64*
   const uint4* __restrict__ mx = J.mx + lane;
   const ConvTarget* __restrict__ mt = J.mt;
   const u32 quads = (nc + 3) / 4;
+  // the order of the quads: as they lie, or, SWITCH, the last one first
+  auto quad_at = [&](u32 k) { return !SWITCH ? k : k == 0 ? quads - 1 : k - 1; };
   uint4 row[STEPS];
 #pragma unroll
-  for (int s = 0; s < STEPS; ++s) row[s] = mx[s * 64];
-  for (u32 quad = 0; quad < quads; ++quad) {
-    // the tables end with a spare quad: the next quad's rows are asked for before this one's are used
+  for (int s = 0; s < STEPS; ++s) row[s] = mx[((u64)quad_at(0) * kMxSteps + s) * 64];
+  for (u32 k = 0; k < quads; ++k) {
+    const u32 quad = quad_at(k);
+    // the next quad's rows are asked for before this one's are used (the tables end with a spare quad, which the
+    // last round reads)
+    const u32 quad_next = k + 1 < quads ? quad_at(k + 1) : quads;
     uint4 row_next[STEPS];
 #pragma unroll
-    for (int s = 0; s < STEPS; ++s) row_next[s] = mx[((u64)(quad + 1) * kMxSteps + s) * 64];
+    for (int s = 0; s < STEPS; ++s) row_next[s] = mx[((u64)quad_next * kMxSteps + s) * 64];
     const ConvTarget tg[2] = {mt[quad * 4 + 2 * half], mt[quad * 4 + 2 * half + 1]};
 #pragma unroll
     for (int rr = 0; rr < 4; ++rr) {
@@ -505,12 +572,23 @@ __global__ __launch_bounds__(256, 4) void conv_fwd_strided_kernel(DevCtx c, u64*
       }
     }
     __syncthreads();
+    if (SWITCH && k == 0) {
+      const u64 ql = c.primes[rz.last_prime].q;
+      const u64* __restrict__ z = rz.z + op * rz.z_stride + col0;
+      const u64* ylast = lds + ((nc - 1) & 3) * 16 * kCfsCols;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const u32 p = threadIdx.x + 256 * i;  // row p / 64, column p % 64
+        lds_last[p] = sub_mod(z[(u64)(p >> 6) * rs + (p & 63)], ylast[p], ql);
+      }
+      __syncthreads();
+    }
     const u32 j = quad * 4 + wv;
-    if (j < nc) {  // uniform over the wave
-      const u32 pi = J.map.prime[j];
-      u64* __restrict__ dst = out + (u64)J.map.out_limb[j] * n;
-      if (c.fp_ok[pi]) conv_strided_column<ArithFp>(c, pi, lds + wv * 16 * kCfsCols, lane, dst, rs);
-      else conv_strided_column<ArithInt>(c, pi, lds + wv * 16 * kCfsCols, lane, dst, rs);
+    if (j < (SWITCH ? nc - 1 : nc)) {  // uniform over the wave
+      const u32 pi = J.map.prime[j], lt = J.map.out_limb[j];
+      u64* __restrict__ dst = out + (u64)lt * n;
+      if (c.fp_ok[pi]) conv_strided_column<ArithFp, SWITCH>(c, pi, lds + wv * 16 * kCfsCols, lane, dst, rs, rz, lds_last, lt);
+      else conv_strided_column<ArithInt, SWITCH>(c, pi, lds + wv * 16 * kCfsCols, lane, dst, rs, rz, lds_last, lt);
     }
     __syncthreads();
 #pragma unroll
@@ -518,7 +596,8 @@ __global__ __launch_bounds__(256, 4) void conv_fwd_strided_kernel(DevCtx c, u64*
   }
 }
 
-bool launch_baseconv_fwd_strided(hipStream_t st, const DevCtx& c, u64* out, const u64* t, const ConvBatch& b, u32 n_ops) {
+bool launch_baseconv_fwd_strided(hipStream_t st, const DevCtx& c, u64* out, const u64* t, const ConvBatch& b, u32 n_ops,
+                                 const FwdFuse* rescale) {
   static const bool on = [] {
     const char* e = getenv("ACE_CONV_STRIDED");
     return !e || e[0] != '0';
@@ -536,8 +615,21 @@ bool launch_baseconv_fwd_strided(hipStream_t st, const DevCtx& c, u64* out, cons
   if (max_nd > 8 || limbs * n_ops < 192) return false;
   if ((((uintptr_t)out | (uintptr_t)t) & 15) || ((b.out_stride | b.t_stride) & 1)) return false;
   dim3 g((u32)(c.N >> 4) / kCfsCols, b.n_jobs * n_ops);
-  if (max_nd <= 4) hipLaunchKernelGGL((conv_fwd_strided_kernel<1>), g, dim3(256), 0, st, c, out, t, b);
-  else hipLaunchKernelGGL((conv_fwd_strided_kernel<2>), g, dim3(256), 0, st, c, out, t, b);
+  ConvRescale rz{};
+  if (rescale) {
+    // the prologue that a Mod_down and a Rescale share: one job whose last target is the dropped limb's `ylast`,
+    // written where the conversion puts it but read from LDS here
+    const ConvJob& J = b.job[0];
+    if (rescale->pro != 2 || b.n_jobs != 1 || J.nc < 2 || J.map.out_limb[J.nc - 1] != J.nc - 1 ||
+        rescale->ylast != out + J.out_off + (u64)(J.nc - 1) * c.N || rescale->ylast_stride != b.out_stride)
+      return false;
+    rz = ConvRescale{rescale->z, rescale->z_stride, rescale->sw, rescale->last_prime};
+    if (max_nd <= 4) hipLaunchKernelGGL((conv_fwd_strided_kernel<1, true>), g, dim3(256), 0, st, c, out, t, b, rz);
+    else hipLaunchKernelGGL((conv_fwd_strided_kernel<2, true>), g, dim3(256), 0, st, c, out, t, b, rz);
+    return true;
+  }
+  if (max_nd <= 4) hipLaunchKernelGGL((conv_fwd_strided_kernel<1, false>), g, dim3(256), 0, st, c, out, t, b, rz);
+  else hipLaunchKernelGGL((conv_fwd_strided_kernel<2, false>), g, dim3(256), 0, st, c, out, t, b, rz);
   return true;
 }
 
@@ -1559,9 +1651,9 @@ bool launch_ntt(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolyS
   }
   FwdFuse f{};
   if (fuse) {
-    // only forward transforms of N > 4096: whole ones, or the chunk pass alone with an epilogue, for a caller whose own
-    // kernel has run the strided pass (launch_baseconv_fwd_strided)
-    if (inverse || c.logN <= kLogChunk || !(passes == 3 || (passes == 2 && fuse->pro == 0))) return false;
+    // only forward transforms of N > 4096: whole ones, or the chunk pass alone with its epilogue, for a caller whose own
+    // kernel has run the strided pass and the prologue (launch_baseconv_fwd_strided)
+    if (inverse || c.logN <= kLogChunk || !(passes == 3 || passes == 2)) return false;
     f = *fuse;
   }
   LimbMap pos{};
