@@ -493,7 +493,7 @@ __device__ __forceinline__ void conv_strided_column(const DevCtx& c, u32 pi, con
 // target's transform starts from Switch_modulus(z - ylast) * sw + (converted word), as ntt_fwd_strided<., 2> forms it.
 // The quad that holds the last target goes first, and z - ylast stays in LDS (8 KiB more) for the other quads.
 template <int STEPS, bool SWITCH>
-__global__ __launch_bounds__(256, 4) void conv_fwd_strided_kernel(DevCtx c, u64* __restrict__ out_base,
+__global__ __launch_bounds__(256, SWITCH ? 3 : 4) void conv_fwd_strided_kernel(DevCtx c, u64* __restrict__ out_base,
                                                                const u64* __restrict__ t_base, ConvBatch b,
                                                                ConvRescale rz) {
   __shared__ __attribute__((aligned(16))) u64 lds[4 * 16 * kCfsCols];

@@ -260,6 +260,72 @@ def test_precomp_and_mod_down_batches_equal_single_calls(pair):
         g.mod_down_batch(a, g.L * N, a, (g.L + K) * N, 2, g.L)  # results over operands
 
 
+def test_conversion_with_strided_pass_equals_the_two_kernels(pair):
+    """Launches of at least 192 converted limbs at N = 65536 run the base conversion and the strided pass of the
+    transform that follows it in one kernel (Mod_down and Precomp of many polynomials, and, with the shared
+    transform's prologue, HMult + relinearise + rescale of many pairs); single calls stay below that size and take
+    the two kernels, which the other tests pin against the oracle.  Same words either way."""
+    g = pair.g
+    N, K, level = g.N, g.K, g.L
+    if N != 65536:
+        pytest.skip("the kernel serves N = 65536")
+    T, nd = level + K, g.num_decomp(level)
+    count, distinct = 40, 4
+    assert count * level >= 192
+    ext = [draw_poly(g, 8800 + k, level, True)[1] for k in range(distinct)]
+    slab = g.alloc(count * T * N)
+    for k in range(count):
+        g.copy(slab.view(k * T * N, T * N), ext[k % distinct])
+    low = g.alloc(count * level * N)
+    g.mod_down_batch(low, level * N, slab, T * N, count, level, True)
+    one = g.alloc(level * N)
+    singles = []
+    for k in range(distinct):
+        g.mod_down(one, ext[k], level, True)
+        singles.append(one.get())
+    got = low.get().reshape(count, level * N)
+    for k in range(count):
+        eq(got[k], singles[k % distinct], "Mod_down of polynomial %d of %d" % (k, count))
+    dig = g.alloc(count * nd * T * N)
+    g.precomp_batch(dig, nd * T * N, low, level * N, count, level, True)
+    one_dig = g.alloc(nd * T * N)
+    want = []
+    for k in range(distinct):
+        g.precomp(one_dig, low.view(k * level * N, level * N), level, True)
+        want.append(one_dig.get())
+    got = dig.get().reshape(count, nd * T * N)
+    for k in range(count):
+        eq(got[k], want[k % distinct], "Precomp of polynomial %d of %d" % (k, count))
+    for b in (slab, low, one, dig, one_dig):
+        b.free()
+    # pairs of ciphertexts: 2 * nb polynomials of `level` targets each through the shared Mod_down + Rescale transform
+    nb = 20
+    assert 2 * nb * level >= 192
+    dk = g.alloc(2 * g.parts * (g.L + K) * N)
+    for i in range(2 * g.parts):
+        g.sample_uniform(dk.view(i * (g.L + K) * N, (g.L + K) * N), g.L, True, 0xACE, 8900 + i)
+    ops = [[draw_poly(g, 8910 + 4 * b + i, level, False)[1] for i in range(4)] for b in range(distinct)]
+    stride = level * N
+    dev = [g.alloc(nb * stride) for _ in range(4)]
+    for b in range(nb):
+        for i in range(4):
+            g.copy(dev[i].view(b * stride, stride), ops[b % distinct][i])
+    r0, r1 = g.alloc(nb * stride), g.alloc(nb * stride)
+    g.mul_relin_rescale_batch(r0, r1, stride, dev[0], dev[1], dev[2], dev[3], stride, dk, level, nb)
+    s0, s1 = g.alloc(stride), g.alloc(stride)
+    n = (level - 1) * N
+    want = []
+    for b in range(distinct):
+        g.mul_relin_rescale(s0, s1, *ops[b], dk, level)
+        want.append((s0.get()[:n], s1.get()[:n]))
+    got0, got1 = r0.get().reshape(nb, stride), r1.get().reshape(nb, stride)
+    for b in range(nb):
+        eq(got0[b][:n], want[b % distinct][0], "pair %d of %d, c0" % (b, nb))
+        eq(got1[b][:n], want[b % distinct][1], "pair %d of %d, c1" % (b, nb))
+    for b in [dk, r0, r1, s0, s1] + dev + ext + [x for o4 in ops for x in o4]:
+        b.free()
+
+
 def test_ntt_batched_polys(pair):
     g, o = pair.g, pair.o
     N = g.N
