@@ -795,10 +795,8 @@ __device__ __forceinline__ void fwd_chunk_body(u64* lds_words, const DevCtx& c, 
     for (int r = 0; r < 8; ++r) ldsu[cm.narrow + ChunkMap::narrow_off(r)] = ar.out_canon(v[r]);
     // The result leaves in the wave order (lane + 64 r inside the 512 words a wave owns): 512 contiguous bytes
     // per store instruction, and every word a wave stores was written by that wave, so no work-group barrier is
-    // needed.  Only the automorphism gathers from the whole chunk.
-    const bool gathers = EPI == 1 && f.orders.n != 0;
-    if (gathers) __syncthreads();
-    else wave_sync();
+    // needed.  Only the automorphism gathers from the whole chunk (after a barrier of its own).
+    wave_sync();
     const u32 wpos = cm.wv * 512 + ((u32)t & 63);  // first of this thread's words in the wave order
     if (EPI == 0) {
 #pragma unroll
@@ -809,36 +807,43 @@ __device__ __forceinline__ void fwd_chunk_body(u64* lds_words, const DevCtx& c, 
       const u64* addend =
           (EPI == 1 && (f.addend_mode == 1 || (f.addend_mode == 2 && !(p & 1)))) ? f.addend.at(p) + (u64)lt * c.N : nullptr;
       if (EPI == 1 && f.orders.n) {
-        // the automorphism on the way out: this chunk of the transform is the source of one chunk of the result
+        // The automorphism on the way out: this chunk of the transform is the source of one chunk of the result.
+        // The tail is formed at the source positions, operands read in the wave order like the plain tail's, and put
+        // back into LDS in place of the transform's words; the result chunk is then gathered from LDS, so that no
+        // global access is scattered.
         const i64* __restrict__ order = f.orders.p[f.orders.n == 1 ? 0 : (p >> 1)];
         const u32 n_chunks = c.N >> kLogChunk;
         u32 dc = chunk;
         for (u32 cc = 0; cc < n_chunks; ++cc)
           if ((u32)((u64)order[(u64)cc * kChunk] >> kLogChunk) == chunk) dc = cc;
         order += (u64)dc * kChunk + t;
-        const u64 so = (u64)lt * c.N + (u64)chunk * kChunk;  // where this chunk's operands lie
+        const u64 so = (u64)lt * c.N + (u64)chunk * kChunk + wpos;  // where this thread's operands lie
         u64* __restrict__ out = f.out.at(p) + (u64)lt * c.N + (u64)dc * kChunk + t;  // never an operand (checked by the callers)
         const u64* __restrict__ src = f.src.at(p) + so;
-        if (addend) addend += (u64)chunk * kChunk;
+        if (addend) addend += (u64)chunk * kChunk + wpos;
+        u32 s8[8];
+#pragma unroll
+        for (int r = 0; r < 8; ++r) s8[r] = (u32)order[512 * r] & (u32)(kChunk - 1);
 #pragma unroll
         for (int r0 = 0; r0 < 8; r0 += 4) {
-          u32 s[4];
           u64 sv[4], av[4];
 #pragma unroll
-          for (int r = 0; r < 4; ++r) s[r] = (u32)order[512 * (r0 + r)] & (u32)(kChunk - 1);
-#pragma unroll
-          for (int r = 0; r < 4; ++r) sv[r] = ldg<64>(src + s[r]);
+          for (int r = 0; r < 4; ++r) sv[r] = ldg<32>(src + 64 * (r0 + r));
           if (addend) {
 #pragma unroll
-            for (int r = 0; r < 4; ++r) av[r] = ldg<64>(addend + s[r]);
+            for (int r = 0; r < 4; ++r) av[r] = ldg<32>(addend + 64 * (r0 + r));
           }
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            u64 v = shoup_mul(sub_mod(sv[r], ldsu[lds_pos((int)s[r])], q), w, wp, q);
+            const int at = cm.wave + ChunkMap::wave_off(r0 + r);
+            u64 v = shoup_mul(sub_mod(sv[r], ldsu[at], q), w, wp, q);
             if (addend) v = add_mod(v, av[r], q);
-            stg<16>(out + 512 * (r0 + r), v);
+            ldsu[at] = v;
           }
         }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < 8; ++r) stg<16>(out + 512 * r, ldsu[lds_pos((int)s8[r])]);
         if (kPolysPerBlock > 1) __syncthreads();  // the gathered LDS reads are not the words this thread writes next
       } else {
         const u64 o = (u64)lt * c.N + (u64)chunk * kChunk + wpos;
