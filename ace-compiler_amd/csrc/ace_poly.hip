@@ -867,6 +867,9 @@ void launch_ext_rotate(hipStream_t st, const DevCtx& c, u64* out0, u64* out1, co
 // words in registers and walks the operands blockIdx.z, blockIdx.z + gridDim.z, ...
 // so the key, the largest stream of a key switch, is fetched gridDim.z times
 // instead of once per operand.
+// coefficients per thread of the kernel below: one (60-106 registers, four to eight waves per SIMD) serves the batched
+// key switch best: 377 us against 396 with two and 431 with four, whose 170 registers leave two waves per SIMD
+constexpr int kKeyUnroll = 1;
 template <int NP>
 __global__ __launch_bounds__(kThreads) void dotprod_shared_key_kernel(
     DevCtx c, u64* __restrict__ out0, u64* __restrict__ out1, u64 out_stride, const u64* __restrict__ digits,
@@ -880,12 +883,12 @@ __global__ __launch_bounds__(kThreads) void dotprod_shared_key_kernel(
   const u64* __restrict__ key1 = key0 + key1_off;
   // the digit this limb is an own limb of (NP: none, or the digits hold their own limbs)
   const int own_d = (own.src && limb < own.level) ? min((int)(limb / own.part_size), NP - 1) : NP;
-  // the thread's kUnroll coefficients are handled together so that every operand has
-  // kUnroll * NP independent loads in flight
-  const u64 i0 = (u64)blockIdx.x * (kThreads * kUnroll) + threadIdx.x;
-  u64 k0[kUnroll][NP], k1[kUnroll][NP];
+  // the thread's kKeyUnroll coefficients are handled together so that every operand has
+  // kKeyUnroll * NP independent loads in flight
+  const u64 i0 = (u64)blockIdx.x * (kThreads * kKeyUnroll) + threadIdx.x;
+  u64 k0[kKeyUnroll][NP], k1[kKeyUnroll][NP];
 #pragma unroll
-  for (int u = 0; u < kUnroll; ++u) {
+  for (int u = 0; u < kKeyUnroll; ++u) {
     const u64 i = i0 + u * kThreads;
 #pragma unroll
     for (int d = 0; d < NP; ++d) {
@@ -895,16 +898,16 @@ __global__ __launch_bounds__(kThreads) void dotprod_shared_key_kernel(
   }
   for (u32 op = blockIdx.z; op < n_ops; op += gridDim.z) {
     const u64* __restrict__ dg = digits + op * digits_op_stride + dbase;
-    u64 x[kUnroll][NP];
+    u64 x[kKeyUnroll][NP];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
+    for (int u = 0; u < kKeyUnroll; ++u) {
       const u64 i = i0 + u * kThreads;
 #pragma unroll
       for (int d = 0; d < NP; ++d)
         x[u][d] = i >= n ? 0 : d == own_d ? ldn<2>(own.src + op * own.op_stride + dbase + i) : ldn<2>(dg + d * digit_stride + i);
     }
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
+    for (int u = 0; u < kKeyUnroll; ++u) {
       const u64 i = i0 + u * kThreads;
       u64 h0 = 0, l0 = 0, h1 = 0, l1 = 0;
 #pragma unroll
@@ -951,6 +954,7 @@ __global__ __launch_bounds__(kThreads) void dotprod_shared_key_kernel(
 // thread walks the operands, so the digits are fetched gridDim.z times instead
 // of once per rotation (they do not survive in L2 between rotations: each
 // rotation streams a whole key through it).
+constexpr int kDigitsUnroll = kUnroll;  // coefficients per thread of the kernel below (two: 16 070 rotations/s against 17 000)
 template <int NP>
 __global__ __launch_bounds__(kThreads) void dotprod_shared_digits_kernel(
     DevCtx c, u64* __restrict__ out0, u64* __restrict__ out1, u64 out_stride, const u64* __restrict__ digits,
@@ -958,10 +962,10 @@ __global__ __launch_bounds__(kThreads) void dotprod_shared_digits_kernel(
   const u32 limb = blockIdx.y;
   const DevPrime P = c.primes[lm.prime[limb]];
   const u64 n = c.N, dbase = (u64)limb * n, kbase = (u64)key_limb.prime[limb] * n;
-  const u64 i0 = (u64)blockIdx.x * (kThreads * kUnroll) + threadIdx.x;
-  u64 x[kUnroll][NP];
+  const u64 i0 = (u64)blockIdx.x * (kThreads * kDigitsUnroll) + threadIdx.x;
+  u64 x[kDigitsUnroll][NP];
 #pragma unroll
-  for (int u = 0; u < kUnroll; ++u) {
+  for (int u = 0; u < kDigitsUnroll; ++u) {
     const u64 i = i0 + u * kThreads;
 #pragma unroll
     for (int d = 0; d < NP; ++d) x[u][d] = i < n ? ldn<32>(digits + d * digit_stride + dbase + i) : 0;
@@ -969,9 +973,9 @@ __global__ __launch_bounds__(kThreads) void dotprod_shared_digits_kernel(
   for (u32 op = blockIdx.z; op < n_ops; op += gridDim.z) {
     const u64* __restrict__ key0 = keys.p[op] + kbase;
     const u64* __restrict__ key1 = key0 + key1_off;
-    u64 k0[kUnroll][NP], k1[kUnroll][NP];
+    u64 k0[kDigitsUnroll][NP], k1[kDigitsUnroll][NP];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
+    for (int u = 0; u < kDigitsUnroll; ++u) {
       const u64 i = i0 + u * kThreads;
 #pragma unroll
       for (int d = 0; d < NP; ++d) {
@@ -980,7 +984,7 @@ __global__ __launch_bounds__(kThreads) void dotprod_shared_digits_kernel(
       }
     }
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
+    for (int u = 0; u < kDigitsUnroll; ++u) {
       const u64 i = i0 + u * kThreads;
       u64 h0 = 0, l0 = 0, h1 = 0, l1 = 0;
 #pragma unroll
@@ -1014,7 +1018,8 @@ void launch_dotprod(hipStream_t st, const DevCtx& c, u64* out0, u64* out1, u64 o
   if (dotprod_reads_own(keys.n, n_ops, out1 != nullptr, n_parts)) {
     const OwnLimbs ol = own ? *own : OwnLimbs{nullptr, 0, 1, 0};
     // NP <= 4 products of residues below 2^61 fit 128 bits without an intermediate reduction
-    dim3 g = ew_grid(c.N, n_limbs, n_ops < kSharedKeySplit ? n_ops : kSharedKeySplit);
+    dim3 g((unsigned)((c.N + kThreads * kKeyUnroll - 1) / (kThreads * kKeyUnroll)), n_limbs,
+           n_ops < kSharedKeySplit ? n_ops : kSharedKeySplit);
 #define ACE_DP_CASE(NP)                                                                                          \
   case NP:                                                                                                       \
     hipLaunchKernelGGL(dotprod_shared_key_kernel<NP>, g, dim3(kThreads), 0, st, c, out0, out1, out_stride,       \
@@ -1026,7 +1031,8 @@ void launch_dotprod(hipStream_t st, const DevCtx& c, u64* out0, u64* out1, u64 o
     return;
   }
   if (!lift && keys.n == n_ops && n_ops > 1 && digits_op_stride == 0 && out1 && n_parts >= 1 && n_parts <= 4) {
-    dim3 g = ew_grid(c.N, n_limbs, n_ops < kSharedDigitsSplit ? n_ops : kSharedDigitsSplit);
+    dim3 g((unsigned)((c.N + kThreads * kDigitsUnroll - 1) / (kThreads * kDigitsUnroll)), n_limbs,
+           n_ops < kSharedDigitsSplit ? n_ops : kSharedDigitsSplit);
 #define ACE_DP_CASE(NP)                                                                                          \
   case NP:                                                                                                       \
     hipLaunchKernelGGL(dotprod_shared_digits_kernel<NP>, g, dim3(kThreads), 0, st, c, out0, out1, out_stride,    \
