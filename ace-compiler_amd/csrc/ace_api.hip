@@ -345,6 +345,9 @@ struct ace_ctx {
   // Mod_down followed by Rescale through one forward transform where an entry point knows both
   // (ACE_SHARE_TRANSFORM=0 in the environment: the two one after the other; same words)
   bool share_transform = true;
+  // an HMult's d2 formed as the inverse transform of Mod_up reads its factors (ACE_PRODUCT_ON_LOAD=0: as a kernel of
+  // its own; same words)
+  bool product_on_load = true;
   void conv_fp_tables(ConvJob& j, const std::vector<size_t>& src, const std::vector<size_t>& tgt, const u64* hat,
                       size_t hat_stride) {
     j.fw = j.fq = nullptr;
@@ -589,6 +592,7 @@ struct ace_ctx {
     conv_fp = from.conv_fp;
     conv_matrix = from.conv_matrix;
     share_transform = from.share_transform;
+    product_on_load = from.product_on_load;
     q_lm = from.q_lm;
     p_lm = from.p_lm;
     phat = from.phat;
@@ -641,6 +645,8 @@ struct ace_ctx {
       conv_matrix = !(no_matrix && no_matrix[0] == '0');
       const char* no_share = std::getenv("ACE_SHARE_TRANSFORM");
       share_transform = !(no_share && no_share[0] == '0');
+      const char* no_product = std::getenv("ACE_PRODUCT_ON_LOAD");
+      product_on_load = !(no_product && no_product[0] == '0');
       bool use_fp = conv_fp && h.logN > 12;
       std::vector<double> w(T * h.N, 0.0), iw(T * h.N, 0.0);
       for (size_t i = 0; i < T; ++i) {
@@ -1089,15 +1095,25 @@ void do_decomp_modup(ace_ctx* c, u64* res, const u64* digit, size_t level, size_
 // NTT over every converted limb.
 // skip_own: the digits' own limbs are not copied into the raised polynomials (the caller's inner product reads them
 // from src: OwnLimbs)
-void do_precomp(ace_ctx* c, u64* res, u64 res_stride, const u64* src, u64 src_stride, size_t nb, size_t level,
-                bool is_ntt, bool skip_own = false) {
+// times (with skip_own, NTT form): the polynomial raised is the limb-wise product of src and times (same stride), formed
+// as the inverse transform reads them; false, with nothing launched, where that transform cannot do so.
+bool do_precomp(ace_ctx* c, u64* res, u64 res_stride, const u64* src, u64 src_stride, size_t nb, size_t level,
+                bool is_ntt, bool skip_own = false, const u64* times = nullptr) {
   const PrecompDev& pd = c->precomp_at(level);
   const size_t N = c->h.N, nd = c->h.num_decomp(level), T = level + c->h.K;
   size_t mark = c->ws_used;
   u64* t = c->take(nb * level * N);
   // the digits' own limbs pass through; the inverse transform of a large ring drops that copy as it reads them
   const bool by_transform = is_ntt && c->d.logN > 12 && !skip_own;
-  if (is_ntt) {
+  if (times) {
+    const PolySeq ts = seq_strided(times, src_stride);
+    if (!is_ntt || !skip_own ||
+        !launch_ntt(c->stream, c->d, seq_strided(t, level * N), seq_strided(src, src_stride), c->q_lm, nullptr,
+                    (u32)level, (u32)nb, true, pd.scale_ntt, 3, nullptr, nullptr, &ts)) {
+      c->ws_used = mark;
+      return false;
+    }
+  } else if (is_ntt) {
     const CopyThrough through{seq_strided(res, res_stride), (u64)(T * N), (u32)c->h.part_size};
     if (!launch_ntt(c->stream, c->d, seq_strided(t, level * N), seq_strided(src, src_stride), c->q_lm, nullptr,
                     (u32)level, (u32)nb, true, pd.scale_ntt, 3, nullptr, by_transform ? &through : nullptr))
@@ -1138,6 +1154,7 @@ void do_precomp(ace_ctx* c, u64* res, u64 res_stride, const u64* src, u64 src_st
     }
   }
   c->ws_used = mark;
+  return true;
 }
 
 // Mod_down (rns_poly.c:260-308) of np polynomials; addend_mode: 0 none,
@@ -1361,10 +1378,22 @@ void do_mul_relin_rescale(ace_ctx* c, u64* r0, u64* r1, u64 out_stride, const u6
   u64* d01 = on_the_way ? nullptr : c->take(nb * 2 * level * N);  // [operand][c0|c1][level limbs]
   u64* d2 = c->take(nb * level * N);
   u64* digits = c->take(nb * nd * T * N);
-  launch_tensor(c->stream, c->d, d01, d01 ? d01 + level * N : nullptr, d2, a0, a1, b0, b1, c->q_lm, (u32)level,
-                (u32)nb, 2 * level * N, level * N, in_stride);
-  const OwnLimbs own{d2, (u64)(level * N), (u32)c->h.part_size, (u32)level};
-  do_precomp(c, digits, nd * T * N, d2, level * N, nb, level, true, from_d2);
+  // With the terms formed on the way, d2 = a1 b1 need not exist in NTT form either where every limb's sums have room
+  // for the lifted terms (the inner product then has a1 and b1 at hand for the digits' own limbs) and the inverse
+  // transform that starts Mod_up can multiply as it reads (large launches of FP64-capable limbs).
+  bool product_on_load = on_the_way && c->product_on_load;
+  for (size_t t = 0; t < level && product_on_load; ++t) {
+    const uint32_t shift = c->h.primes[t].shift;
+    product_on_load = (shift >= 60 ? 4u : shift == 59 ? 8u : 16u) >= nd + 2;  // sum_terms of the kernel
+  }
+  if (product_on_load) product_on_load = do_precomp(c, digits, nd * T * N, a1, in_stride, nb, level, true, true, b1);
+  if (!product_on_load) {
+    launch_tensor(c->stream, c->d, d01, d01 ? d01 + level * N : nullptr, d2, a0, a1, b0, b1, c->q_lm, (u32)level,
+                  (u32)nb, 2 * level * N, level * N, in_stride);
+    do_precomp(c, digits, nd * T * N, d2, level * N, nb, level, true, from_d2);
+  }
+  const OwnLimbs own = product_on_load ? OwnLimbs{nullptr, 0, (u32)c->h.part_size, (u32)level, 1}
+                                       : OwnLimbs{d2, (u64)(level * N), (u32)c->h.part_size, (u32)level, 0};
   PolySeq ds = seq_strided(d01 ? d01 : d2, level * N);  // (never read when the terms are formed on the way)
   if (shared) {
     Lift lift{ds, c->pmodq, (u32)level, nullptr, nullptr, nullptr, nullptr, 0};

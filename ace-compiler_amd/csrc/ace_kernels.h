@@ -57,9 +57,13 @@ struct KeySet {   // one switch key per operand, or one shared by all (n == 1)
 // (both by default; single passes exist so a benchmark can time each kernel).
 // fuse: optional prologue / epilogue of a whole forward transform of N > 4096 (FwdFuse); with an epilogue dst
 // only holds the intermediate between the two kernels.  Returns false when the request cannot be served.
+// times: the inverse transform of the limb-wise product src * times (canonical words, modulo each limb's prime)
+// instead of src; served only by the kernel for large launches of FP64-capable limbs at N > 4096 -- false, and
+// nothing launched, otherwise (the caller then forms the product itself).
 bool launch_ntt(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolySeq& src, const LimbMap& lm,
                 const LimbMap* pos, u32 n_limbs, u32 n_polys, bool inverse, const u64* scale, int passes = 3,
-                const FwdFuse* fuse = nullptr, const CopyThrough* copy_src_to = nullptr);
+                const FwdFuse* fuse = nullptr, const CopyThrough* copy_src_to = nullptr,
+                const PolySeq* times = nullptr);
 
 constexpr u32 kMaxMacOps = 32;
 struct MacSet { // operands of one multiply-accumulate launch
@@ -158,9 +162,10 @@ void launch_digit_copy(hipStream_t st, const DevCtx& c, u64* res, const u64* src
 // Where the raised digits do not hold the digits' own limbs (the Q limbs of the polynomial that was decomposed,
 // which Mod_up only passes through): limb t < level of digit t / part_size is read from src + op * op_stride + t * N.
 struct OwnLimbs {
-  const u64* src;
+  const u64* src;  // null with `product`: the own limbs are Lift's a1 * b1, formed where they are used
   u64 op_stride;
   u32 part_size, level;
+  u32 product;
 };
 // An addend lifted to the extended basis on the way out (what Extend, rns_poly.c:483-500, would add before a
 // Mod_down): limb t < level of operand op's results gains addend.at(2 op) [t] * cst[2t] and addend.at(2 op + 1) [t] *

@@ -1150,14 +1150,17 @@ struct HalfTw {
 // the eleven stages of a half from the words a thread loaded (raw[r] = word 8 t + r of the half) to the words it
 // stores (word(r) of its column t); twiddles loaded stage by stage, or handed in (pre)
 __device__ __forceinline__ constexpr int half_word(int r) { return 256 * ((r >> 2) & 1) + 512 * (r & 1) + 1024 * ((r >> 1) & 1); }
-template <class A, bool PRE>
+// CENTRED: the eight values come as `vin`, each of magnitude at most q/2, instead of canonical words (`raw`); the
+// sums of four then stay within 2q without the shift that canonical words need.
+template <class A, bool PRE, bool CENTRED = false>
 __device__ __forceinline__ void inv_half_rounds(typename A::T* lds, const A& ar, const ChunkMap& cm, u32 mh, u32 half,
-                                                const u64* raw, u64* out, const HalfTw<A>* pre) {
+                                                const u64* raw, u64* out, const HalfTw<A>* pre,
+                                                const typename A::T* vin = nullptr) {
   typedef typename A::T T;
   const int t = threadIdx.x;
   T v[8];
 #pragma unroll
-  for (int r = 0; r < 8; ++r) v[r] = ar.in_canon(raw[r]);
+  for (int r = 0; r < 8; ++r) v[r] = CENTRED ? vin[r] : ar.in_canon(raw[r]);
   // spans 1, 2, 4
   if constexpr (PRE) {
     gs_stage_pre<A, 8, 0>(ar, v, pre->a0);
@@ -1166,8 +1169,10 @@ __device__ __forceinline__ void inv_half_rounds(typename A::T* lds, const A& ar,
     gs_stage<A, 8, 0>(ar, v, (mh >> 0) + (half << 10) + ((u32)t << 2));
     gs_stage<A, 8, 1>(ar, v, (mh >> 1) + (half << 9) + ((u32)t << 1));
   }
-  ar.recentre_sum_of_four(v[0]);
-  ar.recentre_sum_of_four(v[4]);
+  if constexpr (!CENTRED) {
+    ar.recentre_sum_of_four(v[0]);
+    ar.recentre_sum_of_four(v[4]);
+  }
   if constexpr (PRE) gs_stage_pre<A, 8, 2>(ar, v, pre->a2);
   else gs_stage<A, 8, 2>(ar, v, (mh >> 2) + (half << 8) + ((u32)t << 0));
   // in a run: the previous polynomial's last round, on other waves, has read the words written next
@@ -1283,8 +1288,13 @@ __global__ __launch_bounds__(kHalfThreads, kChunkWaves) void ntt_inv_half(DevCtx
 // What the scheme buys is not the overlap alone (the same loop without any arithmetic is only 5 % faster): 15 % fewer
 // vector instructions (no twiddle loads or addresses in the loop), the non-temporal hint on loads that fetch every
 // byte once, and the order of the work-groups (chunk_block, SLOT_MAJOR).
-__device__ __forceinline__ void inv_half_run_body(double* lds, u64* stage, const DevCtx& c, const PolySeq& dsts,
-                                                  const PolySeq& srcs, const LimbMap& pos, u32 n_polys, u32 run,
+// PRODUCT: the polynomial transformed is the limb-wise product of srcs and srcs2 (both staged; 49 KiB of LDS, three
+// work-groups per CU): the product of a word of each, exact in FP64 and brought to magnitude q/2, enters the first
+// round in place of a canonical word -- an HMult's d2 = a1 b1 is then never written in NTT form.
+template <bool PRODUCT>
+__device__ __forceinline__ void inv_half_run_body(double* lds, u64* stage, u64* stage2, const DevCtx& c,
+                                                  const PolySeq& dsts, const PolySeq& srcs, const PolySeq& srcs2,
+                                                  const LimbMap& pos, u32 n_polys, u32 run,
                                                   u32 half, u32 limb, u32 pblk, u32 pi) {
   typedef ArithFp A;
   const int t = threadIdx.x;
@@ -1295,31 +1305,53 @@ __device__ __forceinline__ void inv_half_run_body(double* lds, u64* stage, const
   ar.init(c, pi, true, nullptr, 0);
   const ChunkMap cm(t);
   u64* mine = stage + cm.wv * 512;  // this wave's four blocks of 128 words
+  u64* mine2 = PRODUCT ? stage2 + cm.wv * 512 : nullptr;
   auto request = [&](u32 poly) {  // 1 KiB of consecutive words per instruction
     const u64* src = srcs.at(poly) + off + cm.wv * 512 + 2 * (t & 63);
 #pragma unroll
     for (int j = 0; j < 4; ++j) stage_request(src + 128 * j, mine + 128 * j);
+    if constexpr (PRODUCT) {
+      const u64* src2 = srcs2.at(poly) + off + cm.wv * 512 + 2 * (t & 63);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) stage_request(src2 + 128 * j, mine2 + 128 * j);
+    }
   };
   HalfTw<A> tw;
   tw.load(ar, cm, c.N >> 1, half, (u32)t);
   tw.settle();
   request(poly0);
   for (u32 it = 0; it < cnt; ++it) {
-    // this polynomial's words are in LDS: its four loads are older than the eight stores of the previous one, and
-    // before the first polynomial nothing was issued after them
+    // this polynomial's words are in LDS: its four (eight) loads are older than the eight stores of the previous one,
+    // and before the first polynomial nothing was issued after them
     if (it == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-    u64 raw[8];
+    u64 raw[8], raw2[PRODUCT ? 8 : 1];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const ulonglong2 x = *reinterpret_cast<const ulonglong2*>(mine + 8 * (t & 63) + 2 * j);
       raw[2 * j] = x.x;
       raw[2 * j + 1] = x.y;
+      if constexpr (PRODUCT) {
+        const ulonglong2 y = *reinterpret_cast<const ulonglong2*>(mine2 + 8 * (t & 63) + 2 * j);
+        raw2[2 * j] = y.x;
+        raw2[2 * j + 1] = y.y;
+      }
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // ... and in registers, before the next ones overwrite them
     if (it + 1 < cnt) request(poly0 + it + 1);
     u64 out[8];
-    inv_half_rounds<A, true>(lds, ar, cm, c.N >> 1, half, raw, out, &tw);
+    if constexpr (PRODUCT) {
+      double v[8];
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        const double y = ar.in_canon(raw2[r]);
+        v[r] = ar.mulmod(ar.in_canon(raw[r]), y, y * ar.qinv);  // both in [0, q): magnitude below 1.4 q
+        ar.reduce(v[r]);
+      }
+      inv_half_rounds<A, true, true>(lds, ar, cm, c.N >> 1, half, raw, out, &tw, v);
+    } else {
+      inv_half_rounds<A, true>(lds, ar, cm, c.N >> 1, half, raw, out, &tw);
+    }
     u64* dst = dsts.at(poly0 + it) + off + t;
 #pragma unroll
     // cached, like the other inverse chunk passes: the strided pass that follows finds part of them in the caches
@@ -1327,13 +1359,16 @@ __device__ __forceinline__ void inv_half_run_body(double* lds, u64* stage, const
     for (int r = 0; r < 8; ++r) stg<512>(dst + half_word(r), out[r]);
   }
 }
-__global__ __launch_bounds__(kHalfThreads, 4) void ntt_inv_half_run(DevCtx c, PolySeq dsts, PolySeq srcs, LimbMap lm,
-                                                                  LimbMap pos, u32 n_limbs, u32 n_polys, u32 run) {
+template <bool PRODUCT>
+__global__ __launch_bounds__(kHalfThreads, PRODUCT ? 3 : 4) void ntt_inv_half_run(DevCtx c, PolySeq dsts, PolySeq srcs,
+                                                                                PolySeq srcs2, LimbMap lm, LimbMap pos,
+                                                                                u32 n_limbs, u32 n_polys, u32 run) {
   __shared__ double lds[kHalf + kHalf / 16];
   __shared__ __attribute__((aligned(16))) u64 stage[kHalf];
+  __shared__ __attribute__((aligned(16))) u64 stage2[PRODUCT ? kHalf : 2];
   u32 half, limb, pblk;
   if (!chunk_block<kLogHalf, true>(c, n_limbs, (n_polys + run - 1) / run, half, limb, pblk)) return;
-  inv_half_run_body(lds, stage, c, dsts, srcs, pos, n_polys, run, half, limb, pblk, lm.prime[limb]);
+  inv_half_run_body<PRODUCT>(lds, stage, stage2, c, dsts, srcs, srcs2, pos, n_polys, run, half, limb, pblk, lm.prime[limb]);
 }
 
 // inverse, strided pass: spans 4096..N/2, then scale every word by the limb's
@@ -1544,10 +1579,11 @@ static bool in_place_or_apart(const DevCtx& c, const PolySeq& dst, const PolySeq
   return dh <= sl || sh <= dl;
 }
 template <int LOGR, int SF, int SI>
-static void run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolySeq& src, const LimbMap& lm,
+static bool run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolySeq& src, const LimbMap& lm,
                       const LimbMap& pos, u32 n_limbs, u32 n_polys, bool inverse, const u64* scale, int passes,
-                      const FwdFuse& f, const CopyThrough& copies) {
+                      const FwdFuse& f, const CopyThrough& copies, const PolySeq* times) {
   dim3 gc(chunk_grid(c, n_limbs, (n_polys + kPolysPerBlock - 1) / kPolysPerBlock));
+  if (times && (!inverse || !(passes & 1))) return false;
   if (!inverse) {
     constexpr int LS = LOGR + SF, SHIFT = SF;
     dim3 gs((c.N >> LS) / 256, n_limbs, n_polys);
@@ -1602,14 +1638,19 @@ static void run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst, const
         return !e || e[0] != '0';
       }();
       const u32 run = SHIFT == 1 && halves && runs && !copies.seq.b[0] && all_fp(c, lm, n_limbs) &&
-                              in_place_or_apart(c, dst, src, pos, n_limbs, n_polys)
+                              in_place_or_apart(c, dst, src, pos, n_limbs, n_polys) &&
+                              (!times || in_place_or_apart(c, dst, *times, pos, n_limbs, n_polys))
                           ? run_length(n_limbs * (c.N >> kLogHalf), n_polys, 4 * kCUs) : 0;
-      if (copies.seq.b[0])
+      if (times) {  // only the run kernel multiplies on the way in
+        if (!run) return false;
+        hipLaunchKernelGGL(ntt_inv_half_run<true>, dim3(chunk_grid<true>(c, n_limbs, (n_polys + run - 1) / run, kLogHalf)),
+                           dim3(kHalfThreads), 0, st, c, dst, src, *times, lm, pos, n_limbs, n_polys, run);
+      } else if (copies.seq.b[0])
         hipLaunchKernelGGL((ntt_inv_chunk<SHIFT, 1>), gc, dim3(kChunkThreads), 0, st, c, dst, src, copies, lm, pos,
                            n_limbs, n_polys);
       else if (run)
-        hipLaunchKernelGGL(ntt_inv_half_run, dim3(chunk_grid<true>(c, n_limbs, (n_polys + run - 1) / run, kLogHalf)),
-                           dim3(kHalfThreads), 0, st, c, dst, src, lm, pos, n_limbs, n_polys, run);
+        hipLaunchKernelGGL(ntt_inv_half_run<false>, dim3(chunk_grid<true>(c, n_limbs, (n_polys + run - 1) / run, kLogHalf)),
+                           dim3(kHalfThreads), 0, st, c, dst, src, src, lm, pos, n_limbs, n_polys, run);
       else if (SHIFT == 1 && halves)
         hipLaunchKernelGGL(ntt_inv_half, dim3(chunk_grid(c, n_limbs, n_polys, kLogHalf)), dim3(kHalfThreads), 0, st, c,
                            dst, src, lm, pos, n_limbs, n_polys);
@@ -1642,12 +1683,14 @@ static void run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst, const
       }
     }
   }
+  return true;
 }
 
 bool launch_ntt(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolySeq& src, const LimbMap& lm,
                 const LimbMap* pos_in, u32 n_limbs, u32 n_polys, bool inverse, const u64* scale, int passes,
-                const FwdFuse* fuse, const CopyThrough* copy_src_to) {
+                const FwdFuse* fuse, const CopyThrough* copy_src_to, const PolySeq* times) {
   if (n_limbs == 0 || n_polys == 0) return true;
+  if (times && (!inverse || c.logN <= kLogChunk || copy_src_to || !(passes & 1))) return false;
   CopyThrough copies{};
   if (copy_src_to) {  // only the inverse chunk pass can drop a copy of what it reads
     if (!inverse || c.logN <= kLogChunk || !(passes & 1)) return false;
@@ -1671,7 +1714,7 @@ bool launch_ntt(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolyS
     auto aligned = [](const PolySeq& q) {
       return (((uintptr_t)q.b[0] | (uintptr_t)q.b[1]) & 15) == 0 && (q.pair_stride & 1) == 0;
     };
-    if (!aligned(dst) || !aligned(src)) return false;
+    if (!aligned(dst) || !aligned(src) || (times && !aligned(*times))) return false;
     if (f.epi && (!aligned(f.out) || !aligned(f.src) || (f.addend_mode && !aligned(f.addend)))) return false;
     if (copies.seq.b[0] && (!aligned(copies.seq) || (copies.digit_stride & 1))) return false;
   }
@@ -1687,9 +1730,10 @@ bool launch_ntt(hipStream_t st, const DevCtx& c, const PolySeq& dst, const PolyS
   switch (c.logN - kLogChunk) {
 #define ACE_NTT_CASE(LR, SH)                                                                       \
   case LR:                                                                                         \
-    if (SH && big) run_large<LR, 0, SH>(st, c, dst, src, lm, pos, n_limbs, n_polys, inverse, scale, passes, f, copies); \
-    else run_large<LR, 0, 0>(st, c, dst, src, lm, pos, n_limbs, n_polys, inverse, scale, passes, f, copies);          \
-    return true;
+    if (SH && big)                                                                                   \
+      return run_large<LR, 0, SH>(st, c, dst, src, lm, pos, n_limbs, n_polys, inverse, scale, passes, f, copies, times); \
+    if (times) return false;                                                                         \
+    return run_large<LR, 0, 0>(st, c, dst, src, lm, pos, n_limbs, n_polys, inverse, scale, passes, f, copies, times);
     ACE_NTT_CASE(1, ACE_NTT_SHIFT)
     ACE_NTT_CASE(2, ACE_NTT_SHIFT)
     ACE_NTT_CASE(3, ACE_NTT_SHIFT)

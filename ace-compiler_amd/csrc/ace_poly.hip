@@ -882,7 +882,9 @@ __global__ __launch_bounds__(kThreads) void dotprod_shared_key_kernel(
   const u64 n = c.N, dbase = (u64)limb * n, kbase = (u64)key_limb.prime[limb] * n;
   const u64* __restrict__ key1 = key0 + key1_off;
   // the digit this limb is an own limb of (NP: none, or the digits hold their own limbs)
-  const int own_d = (own.src && limb < own.level) ? min((int)(limb / own.part_size), NP - 1) : NP;
+  const int own_d = ((own.src || own.product) && limb < own.level) ? min((int)(limb / own.part_size), NP - 1) : NP;
+  // ... whose words are the product a1 b1 of the operands the lifted terms are formed from (never stored)
+  const bool own_product = own.product && own_d < NP;
   // the thread's kKeyUnroll coefficients are handled together so that every operand has
   // kKeyUnroll * NP independent loads in flight
   const u64 i0 = (u64)blockIdx.x * (kThreads * kKeyUnroll) + threadIdx.x;
@@ -904,24 +906,30 @@ __global__ __launch_bounds__(kThreads) void dotprod_shared_key_kernel(
       const u64 i = i0 + u * kThreads;
 #pragma unroll
       for (int d = 0; d < NP; ++d)
-        x[u][d] = i >= n ? 0 : d == own_d ? ldn<2>(own.src + op * own.op_stride + dbase + i) : ldn<2>(dg + d * digit_stride + i);
+        x[u][d] = (i >= n || (d == own_d && own_product)) ? 0
+                  : d == own_d ? ldn<2>(own.src + op * own.op_stride + dbase + i) : ldn<2>(dg + d * digit_stride + i);
     }
 #pragma unroll
     for (int u = 0; u < kKeyUnroll; ++u) {
       const u64 i = i0 + u * kThreads;
       u64 h0 = 0, l0 = 0, h1 = 0, l1 = 0;
-#pragma unroll
-      for (int d = 0; d < NP; ++d) {
-        mac128(h0, l0, x[u][d], k0[u][d]);
-        mac128(h1, l1, x[u][d], k1[u][d]);
-      }
       // The lifted tensor terms P a0 b0 and P (a0 b1 + a1 b0) join the sums before their one reduction where the sums
       // have room for two more products: P a0 and P a1 are reduced (two Shoup products), the three products with
       // b0 / b1 are not.  The residue of the whole sum is the same word as the sum of the residues.
       const bool fold = lifted && lift.a0 && sum_terms(P) >= NP + 2;
+      u64 x0 = 0, x1 = 0, y0 = 0, y1 = 0;
       if (fold && i < n) {
         const u64 o = op * lift.in_stride + dbase + i;
-        const u64 x0 = ldn<2>(lift.a0 + o), x1 = ldn<2>(lift.a1 + o), y0 = ldn<2>(lift.b0 + o), y1 = ldn<2>(lift.b1 + o);
+        x0 = ldn<2>(lift.a0 + o), x1 = ldn<2>(lift.a1 + o), y0 = ldn<2>(lift.b0 + o), y1 = ldn<2>(lift.b1 + o);
+      }
+      const u64 own_word = own_product ? mulmod(x1, y1, P) : 0;  // (the host asks for it only where every limb folds)
+#pragma unroll
+      for (int d = 0; d < NP; ++d) {
+        const u64 xd = (own_product && d == own_d) ? own_word : x[u][d];
+        mac128(h0, l0, xd, k0[u][d]);
+        mac128(h1, l1, xd, k1[u][d]);
+      }
+      if (fold && i < n) {
         const u64 px0 = shoup_mul(x0, lw, lwp, P.q), px1 = shoup_mul(x1, lw, lwp, P.q);
         mac128(h0, l0, px0, y0);
         mac128(h1, l1, px0, y1);
@@ -1016,7 +1024,7 @@ void launch_dotprod(hipStream_t st, const DevCtx& c, u64* out0, u64* out1, u64 o
   if (!n_limbs || !n_ops) return;
   const Lift lf = lift ? *lift : Lift{PolySeq{{nullptr, nullptr}, 0}, nullptr, 0, nullptr, nullptr, nullptr, nullptr, 0};
   if (dotprod_reads_own(keys.n, n_ops, out1 != nullptr, n_parts)) {
-    const OwnLimbs ol = own ? *own : OwnLimbs{nullptr, 0, 1, 0};
+    const OwnLimbs ol = own ? *own : OwnLimbs{nullptr, 0, 1, 0, 0};
     // NP <= 4 products of residues below 2^61 fit 128 bits without an intermediate reduction
     dim3 g((unsigned)((c.N + kThreads * kKeyUnroll - 1) / (kThreads * kKeyUnroll)), n_limbs,
            n_ops < kSharedKeySplit ? n_ops : kSharedKeySplit);
