@@ -962,15 +962,22 @@ __global__ __launch_bounds__(kThreads) void dotprod_shared_key_kernel(
 // thread walks the operands, so the digits are fetched gridDim.z times instead
 // of once per rotation (they do not survive in L2 between rotations: each
 // rotation streams a whole key through it).
-constexpr int kDigitsUnroll = kUnroll;  // coefficients per thread of the kernel below (two: 16 070 rotations/s against 17 000)
+constexpr int kDigitsUnroll = kUnroll;  // coefficients per thread of the kernel below (two: 754 us against 732)
 template <int NP>
 __global__ __launch_bounds__(kThreads) void dotprod_shared_digits_kernel(
     DevCtx c, u64* __restrict__ out0, u64* __restrict__ out1, u64 out_stride, const u64* __restrict__ digits,
-    u64 digit_stride, KeySet keys, u64 key1_off, u64 key_stride, LimbMap lm, LimbMap key_limb, u32 n_ops) {
-  const u32 limb = blockIdx.y;
+    u64 digit_stride, KeySet keys, u64 key1_off, u64 key_stride, LimbMap lm, LimbMap key_limb, u32 n_ops,
+    u32 blocks_x, u32 n_limbs, u32 split) {
+  // The grid is one-dimensional.  Hardware hands consecutive work-groups to the 8 XCDs in turn, each with its own L2:
+  // the `split` work-groups that share a tile of the digits (same coefficients, same limb, different keys) are
+  // consecutive work-groups of one XCD, so the tile comes from memory once and from that L2 for the others.
+  const u32 xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+  const u32 tile = (local / split) * 8 + xcd, first_op = local % split;
+  if (tile >= blocks_x * n_limbs) return;
+  const u32 limb = tile / blocks_x, bx = tile % blocks_x;
   const DevPrime P = c.primes[lm.prime[limb]];
   const u64 n = c.N, dbase = (u64)limb * n, kbase = (u64)key_limb.prime[limb] * n;
-  const u64 i0 = (u64)blockIdx.x * (kThreads * kDigitsUnroll) + threadIdx.x;
+  const u64 i0 = (u64)bx * (kThreads * kDigitsUnroll) + threadIdx.x;
   u64 x[kDigitsUnroll][NP];
 #pragma unroll
   for (int u = 0; u < kDigitsUnroll; ++u) {
@@ -978,7 +985,7 @@ __global__ __launch_bounds__(kThreads) void dotprod_shared_digits_kernel(
 #pragma unroll
     for (int d = 0; d < NP; ++d) x[u][d] = i < n ? ldn<32>(digits + d * digit_stride + dbase + i) : 0;
   }
-  for (u32 op = blockIdx.z; op < n_ops; op += gridDim.z) {
+  for (u32 op = first_op; op < n_ops; op += split) {
     const u64* __restrict__ key0 = keys.p[op] + kbase;
     const u64* __restrict__ key1 = key0 + key1_off;
     u64 k0[kDigitsUnroll][NP], k1[kDigitsUnroll][NP];
@@ -1011,7 +1018,8 @@ __global__ __launch_bounds__(kThreads) void dotprod_shared_digits_kernel(
 // How many blocks share the walk over the operands of a batch (blockIdx.z): the shared operand is fetched that many
 // times.  A key is 93 MiB, so the kernel that shares it splits the operands two ways only; the digits that
 // rotations share are a twentieth of one key, and sixteen blocks walking two keys each keep more of the machine's
-// memory channels busy than four walking eight (rotations +2 %).
+// memory channels busy than four walking eight (rotations +2 %; eight walking four and thirty-two walking one are
+// slower again: 773 and 754 us against 732 for the 32-rotation batch).
 constexpr u32 kSharedKeySplit = 2, kSharedDigitsSplit = 16;
 bool dotprod_reads_own(u32 n_keys, u32 n_ops, bool two_halves, u32 n_parts) {
   return n_keys == 1 && n_ops > 1 && two_halves && n_parts >= 1 && n_parts <= 4;
@@ -1039,12 +1047,14 @@ void launch_dotprod(hipStream_t st, const DevCtx& c, u64* out0, u64* out1, u64 o
     return;
   }
   if (!lift && keys.n == n_ops && n_ops > 1 && digits_op_stride == 0 && out1 && n_parts >= 1 && n_parts <= 4) {
-    dim3 g((unsigned)((c.N + kThreads * kDigitsUnroll - 1) / (kThreads * kDigitsUnroll)), n_limbs,
-           n_ops < kSharedDigitsSplit ? n_ops : kSharedDigitsSplit);
+    const u32 blocks_x = (u32)((c.N + kThreads * kDigitsUnroll - 1) / (kThreads * kDigitsUnroll));
+    const u32 split = n_ops < kSharedDigitsSplit ? n_ops : kSharedDigitsSplit;
+    dim3 g(((blocks_x * n_limbs + 7) / 8) * 8 * split);
 #define ACE_DP_CASE(NP)                                                                                          \
   case NP:                                                                                                       \
     hipLaunchKernelGGL(dotprod_shared_digits_kernel<NP>, g, dim3(kThreads), 0, st, c, out0, out1, out_stride,    \
-                       digits, digit_stride, keys, key1_off, key_stride, lm, key_limb, n_ops);                   \
+                       digits, digit_stride, keys, key1_off, key_stride, lm, key_limb, n_ops, blocks_x, n_limbs, \
+                       split);                                                                                   \
     break;
     switch (n_parts) { ACE_DP_CASE(1) ACE_DP_CASE(2) ACE_DP_CASE(3) ACE_DP_CASE(4) }
 #undef ACE_DP_CASE
