@@ -874,8 +874,13 @@ template <int NP>
 __global__ __launch_bounds__(kThreads) void dotprod_shared_key_kernel(
     DevCtx c, u64* __restrict__ out0, u64* __restrict__ out1, u64 out_stride, const u64* __restrict__ digits,
     u64 digit_stride, u64 digits_op_stride, const u64* __restrict__ key0, u64 key1_off, u64 key_stride, LimbMap lm,
-    LimbMap key_limb, u32 n_ops, OwnLimbs own, Lift lift) {
-  const u32 limb = blockIdx.y;
+    LimbMap key_limb, u32 n_ops, OwnLimbs own, Lift lift, u32 blocks_x, u32 n_limbs, u32 split) {
+  // one-dimensional grid: the `split` work-groups that share a tile of the key are neighbours on one XCD (see
+  // dotprod_shared_digits_kernel)
+  const u32 xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+  const u32 tile = (local / split) * 8 + xcd, first_op = local % split;
+  if (tile >= blocks_x * n_limbs) return;
+  const u32 limb = tile / blocks_x, bx = tile % blocks_x;
   const DevPrime P = c.primes[lm.prime[limb]];
   const bool lifted = lift.cst && limb < lift.level;
   const u64 lw = lifted ? lift.cst[2 * limb] : 0, lwp = lifted ? lift.cst[2 * limb + 1] : 0;
@@ -887,7 +892,7 @@ __global__ __launch_bounds__(kThreads) void dotprod_shared_key_kernel(
   const bool own_product = own.product && own_d < NP;
   // the thread's kKeyUnroll coefficients are handled together so that every operand has
   // kKeyUnroll * NP independent loads in flight
-  const u64 i0 = (u64)blockIdx.x * (kThreads * kKeyUnroll) + threadIdx.x;
+  const u64 i0 = (u64)bx * (kThreads * kKeyUnroll) + threadIdx.x;
   u64 k0[kKeyUnroll][NP], k1[kKeyUnroll][NP];
 #pragma unroll
   for (int u = 0; u < kKeyUnroll; ++u) {
@@ -898,7 +903,7 @@ __global__ __launch_bounds__(kThreads) void dotprod_shared_key_kernel(
       k1[u][d] = i < n ? ldn<16>(key1 + d * key_stride + kbase + i) : 0;
     }
   }
-  for (u32 op = blockIdx.z; op < n_ops; op += gridDim.z) {
+  for (u32 op = first_op; op < n_ops; op += split) {
     const u64* __restrict__ dg = digits + op * digits_op_stride + dbase;
     u64 x[kKeyUnroll][NP];
 #pragma unroll
@@ -1034,13 +1039,14 @@ void launch_dotprod(hipStream_t st, const DevCtx& c, u64* out0, u64* out1, u64 o
   if (dotprod_reads_own(keys.n, n_ops, out1 != nullptr, n_parts)) {
     const OwnLimbs ol = own ? *own : OwnLimbs{nullptr, 0, 1, 0, 0};
     // NP <= 4 products of residues below 2^61 fit 128 bits without an intermediate reduction
-    dim3 g((unsigned)((c.N + kThreads * kKeyUnroll - 1) / (kThreads * kKeyUnroll)), n_limbs,
-           n_ops < kSharedKeySplit ? n_ops : kSharedKeySplit);
+    const u32 blocks_x = (u32)((c.N + kThreads * kKeyUnroll - 1) / (kThreads * kKeyUnroll));
+    const u32 split = n_ops < kSharedKeySplit ? n_ops : kSharedKeySplit;
+    dim3 g(((blocks_x * n_limbs + 7) / 8) * 8 * split);
 #define ACE_DP_CASE(NP)                                                                                          \
   case NP:                                                                                                       \
     hipLaunchKernelGGL(dotprod_shared_key_kernel<NP>, g, dim3(kThreads), 0, st, c, out0, out1, out_stride,       \
                        digits, digit_stride, digits_op_stride, keys.p[0], key1_off, key_stride, lm, key_limb,    \
-                       n_ops, ol, lf);                                                                           \
+                       n_ops, ol, lf, blocks_x, n_limbs, split);                                                 \
     break;
     switch (n_parts) { ACE_DP_CASE(1) ACE_DP_CASE(2) ACE_DP_CASE(3) ACE_DP_CASE(4) }
 #undef ACE_DP_CASE
