@@ -723,6 +723,86 @@ struct ChunkMap {
   static __device__ __forceinline__ constexpr int narrow_off(int r) { return r; }
 };
 
+// What a forward chunk pass with an epilogue (FwdFuse::epi) does with the chunk it has transformed, in place of storing
+// it: the words lie in LDS in canonical form (`ldsu`, wave order: a wave reads the words it wrote); p is the
+// polynomial, lt its limb's place, pi the prime.  barrier_after_gather: the caller writes the LDS again without a
+// work-group barrier of its own.
+template <int EPI>
+__device__ __forceinline__ void fwd_chunk_tail(const DevCtx& c, const FwdFuse& f, u64* ldsu, const ChunkMap& cm, int t,
+                                               u32 wpos, u32 p, u32 lt, u32 pi, u32 chunk, bool barrier_after_gather) {
+  const u64 q = c.primes[pi].q, w = f.cst[2 * lt], wp = f.cst[2 * lt + 1];
+  const u64* addend =
+      (EPI == 1 && (f.addend_mode == 1 || (f.addend_mode == 2 && !(p & 1)))) ? f.addend.at(p) + (u64)lt * c.N : nullptr;
+  if (EPI == 1 && f.orders.n) {
+    // The automorphism on the way out: this chunk of the transform is the source of one chunk of the result.
+    // The tail is formed at the source positions, operands read in the wave order like the plain tail's, and put
+    // back into LDS in place of the transform's words; the result chunk is then gathered from LDS, so that no
+    // global access is scattered.
+    const i64* __restrict__ order = f.orders.p[f.orders.n == 1 ? 0 : (p >> 1)];
+    const u32 n_chunks = c.N >> kLogChunk;
+    u32 dc = chunk;
+    for (u32 cc = 0; cc < n_chunks; ++cc)
+      if ((u32)((u64)order[(u64)cc * kChunk] >> kLogChunk) == chunk) dc = cc;
+    order += (u64)dc * kChunk + t;
+    const u64 so = (u64)lt * c.N + (u64)chunk * kChunk + wpos;  // where this thread's operands lie
+    u64* __restrict__ out = f.out.at(p) + (u64)lt * c.N + (u64)dc * kChunk + t;  // never an operand (checked by the callers)
+    const u64* __restrict__ src = f.src.at(p) + so;
+    if (addend) addend += (u64)chunk * kChunk + wpos;
+    u32 s8[8];
+#pragma unroll
+    for (int r = 0; r < 8; ++r) s8[r] = (u32)order[512 * r] & (u32)(kChunk - 1);
+#pragma unroll
+    for (int r0 = 0; r0 < 8; r0 += 4) {
+      u64 sv[4], av[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) sv[r] = ldg<32>(src + 64 * (r0 + r));
+      if (addend) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) av[r] = ldg<32>(addend + 64 * (r0 + r));
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int at = cm.wave + ChunkMap::wave_off(r0 + r);
+        u64 v = shoup_mul(sub_mod(sv[r], ldsu[at], q), w, wp, q);
+        if (addend) v = add_mod(v, av[r], q);
+        ldsu[at] = v;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < 8; ++r) stg<16>(out + 512 * r, ldsu[lds_pos((int)s8[r])]);
+    if (barrier_after_gather) __syncthreads();  // the gathered LDS reads are not the words this thread writes next
+  } else {
+    const u64 o = (u64)lt * c.N + (u64)chunk * kChunk + wpos;
+    u64* out = f.out.at(p) + o;  // may alias the addend (in-place relinearisation)
+    const u64* __restrict__ src = f.src.at(p) + o;
+    if (addend) addend += (u64)chunk * kChunk + wpos;
+    // four words at a time: the operands of all eight would not fit beside the 64 registers of a thread
+#pragma unroll
+    for (int r0 = 0; r0 < 8; r0 += 4) {
+      u64 sv[4], av[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) sv[r] = ldg<32>(src + 64 * (r0 + r));
+      if (addend) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) av[r] = ldg<32>(addend + 64 * (r0 + r));
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const u64 y = ldsu[cm.wave + ChunkMap::wave_off(r0 + r)];
+        u64 v;
+        if (EPI == 1) {
+          v = shoup_mul(sub_mod(sv[r], y, q), w, wp, q);
+          if (addend) v = add_mod(v, av[r], q);
+        } else {
+          v = add_mod(shoup_mul(sv[r], w, wp, q), y, q);
+        }
+        stg<16>(out + 64 * (r0 + r), v);
+      }
+    }
+  }
+}
+
 // forward, chunk pass: stages logr..logN-1 on 4096 contiguous words, in place.
 // grid = chunk_grid(n_limbs, ceil(n_polys / kPolysPerBlock)), 512 threads: four
 // rounds of three stages with the chunk passing through LDS between them, and
@@ -802,78 +882,7 @@ __device__ __forceinline__ void fwd_chunk_body(u64* lds_words, const DevCtx& c, 
 #pragma unroll
       for (int r = 0; r < 8; ++r) stg<4>(base + wpos + 64 * r, ldsu[cm.wave + ChunkMap::wave_off(r)]);
     } else {
-      const u32 p = poly0 + it, lt = pos.prime[limb];
-      const u64 q = c.primes[pi].q, w = f.cst[2 * lt], wp = f.cst[2 * lt + 1];
-      const u64* addend =
-          (EPI == 1 && (f.addend_mode == 1 || (f.addend_mode == 2 && !(p & 1)))) ? f.addend.at(p) + (u64)lt * c.N : nullptr;
-      if (EPI == 1 && f.orders.n) {
-        // The automorphism on the way out: this chunk of the transform is the source of one chunk of the result.
-        // The tail is formed at the source positions, operands read in the wave order like the plain tail's, and put
-        // back into LDS in place of the transform's words; the result chunk is then gathered from LDS, so that no
-        // global access is scattered.
-        const i64* __restrict__ order = f.orders.p[f.orders.n == 1 ? 0 : (p >> 1)];
-        const u32 n_chunks = c.N >> kLogChunk;
-        u32 dc = chunk;
-        for (u32 cc = 0; cc < n_chunks; ++cc)
-          if ((u32)((u64)order[(u64)cc * kChunk] >> kLogChunk) == chunk) dc = cc;
-        order += (u64)dc * kChunk + t;
-        const u64 so = (u64)lt * c.N + (u64)chunk * kChunk + wpos;  // where this thread's operands lie
-        u64* __restrict__ out = f.out.at(p) + (u64)lt * c.N + (u64)dc * kChunk + t;  // never an operand (checked by the callers)
-        const u64* __restrict__ src = f.src.at(p) + so;
-        if (addend) addend += (u64)chunk * kChunk + wpos;
-        u32 s8[8];
-#pragma unroll
-        for (int r = 0; r < 8; ++r) s8[r] = (u32)order[512 * r] & (u32)(kChunk - 1);
-#pragma unroll
-        for (int r0 = 0; r0 < 8; r0 += 4) {
-          u64 sv[4], av[4];
-#pragma unroll
-          for (int r = 0; r < 4; ++r) sv[r] = ldg<32>(src + 64 * (r0 + r));
-          if (addend) {
-#pragma unroll
-            for (int r = 0; r < 4; ++r) av[r] = ldg<32>(addend + 64 * (r0 + r));
-          }
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int at = cm.wave + ChunkMap::wave_off(r0 + r);
-            u64 v = shoup_mul(sub_mod(sv[r], ldsu[at], q), w, wp, q);
-            if (addend) v = add_mod(v, av[r], q);
-            ldsu[at] = v;
-          }
-        }
-        __syncthreads();
-#pragma unroll
-        for (int r = 0; r < 8; ++r) stg<16>(out + 512 * r, ldsu[lds_pos((int)s8[r])]);
-        if (kPolysPerBlock > 1) __syncthreads();  // the gathered LDS reads are not the words this thread writes next
-      } else {
-        const u64 o = (u64)lt * c.N + (u64)chunk * kChunk + wpos;
-        u64* out = f.out.at(p) + o;  // may alias the addend (in-place relinearisation)
-        const u64* __restrict__ src = f.src.at(p) + o;
-        if (addend) addend += (u64)chunk * kChunk + wpos;
-        // four words at a time: the operands of all eight would not fit beside the 64 registers of a thread
-#pragma unroll
-        for (int r0 = 0; r0 < 8; r0 += 4) {
-          u64 sv[4], av[4];
-#pragma unroll
-          for (int r = 0; r < 4; ++r) sv[r] = ldg<32>(src + 64 * (r0 + r));
-          if (addend) {
-#pragma unroll
-            for (int r = 0; r < 4; ++r) av[r] = ldg<32>(addend + 64 * (r0 + r));
-          }
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const u64 y = ldsu[cm.wave + ChunkMap::wave_off(r0 + r)];
-            u64 v;
-            if (EPI == 1) {
-              v = shoup_mul(sub_mod(sv[r], y, q), w, wp, q);
-              if (addend) v = add_mod(v, av[r], q);
-            } else {
-              v = add_mod(shoup_mul(sv[r], w, wp, q), y, q);
-            }
-            stg<16>(out + 64 * (r0 + r), v);
-          }
-        }
-      }
+      fwd_chunk_tail<EPI>(c, f, ldsu, cm, t, wpos, poly0 + it, pos.prime[limb], pi, chunk, kPolysPerBlock > 1);
     }
     // the next polynomial's first round writes words that other waves may still be reading
     if (kPolysPerBlock > 1) __syncthreads();
@@ -1609,7 +1618,9 @@ static bool run_large(hipStream_t st, const DevCtx& c, const PolySeq& dst, const
         const char* e = getenv("ACE_NTT_FWD_RUN");
         return !e || e[0] != '0';
       }();
-      // (the chunk pass works in place on dst, which the strided pass has filled)
+      // (the chunk pass works in place on dst, which the strided pass has filled; with an epilogue the run kernel is
+      // slower than the plain one, whose eight waves per SIMD hide the tail's loads: 32 rotations 16 060 against
+      // 17 200 per second)
       const u32 run = runs && f.epi == 0 && SHIFT == 0 && all_fp(c, lm, n_limbs)
                           ? run_length(n_limbs * (c.N >> kLogChunk), n_polys, 2 * kCUs) : 0;
       if (run)
