@@ -1110,8 +1110,10 @@ __device__ __forceinline__ void inv_chunk_body(u64* lds_words, const DevCtx& c, 
     for (int r = 0; r < 8; ++r) raw[r] = nxt[r];
   }
 }
+// (compiled for six waves per SIMD: at eight, 64 registers, the integer body spills; the launches this kernel serves
+// are those of whole programs, far too small to fill eight)
 template <int SKIP, int COPY>
-__global__ __launch_bounds__(kChunkThreads, kChunkWaves) void ntt_inv_chunk(DevCtx c, PolySeq dsts, PolySeq srcs, CopyThrough copies,
+__global__ __launch_bounds__(kChunkThreads, 6) void ntt_inv_chunk(DevCtx c, PolySeq dsts, PolySeq srcs, CopyThrough copies,
                                                                   LimbMap lm, LimbMap pos, u32 n_limbs, u32 n_polys) {
   __shared__ u64 lds[kChunk + kChunk / 16];
   u32 chunk, limb, pblk;
