@@ -545,12 +545,6 @@ __global__ __launch_bounds__(256, SWITCH ? 3 : 4) void conv_fwd_strided_kernel(D
   for (int s = 0; s < STEPS; ++s) row[s] = mx[((u64)quad_at(0) * kMxSteps + s) * 64];
   for (u32 k = 0; k < quads; ++k) {
     const u32 quad = quad_at(k);
-    // the next quad's rows are asked for before this one's are used (the tables end with a spare quad, which the
-    // last round reads)
-    const u32 quad_next = k + 1 < quads ? quad_at(k + 1) : quads;
-    uint4 row_next[STEPS];
-#pragma unroll
-    for (int s = 0; s < STEPS; ++s) row_next[s] = mx[((u64)quad_next * kMxSteps + s) * 64];
     const ConvTarget tg[2] = {mt[quad * 4 + 2 * half], mt[quad * 4 + 2 * half + 1]};
 #pragma unroll
     for (int rr = 0; rr < 4; ++rr) {
@@ -572,6 +566,13 @@ __global__ __launch_bounds__(256, SWITCH ? 3 : 4) void conv_fwd_strided_kernel(D
       }
     }
     __syncthreads();
+    {
+      // the next quad's rows are asked for now and arrive while the columns are transformed (the tables end with a
+      // spare quad, which the last round reads)
+      const u32 quad_next = k + 1 < quads ? quad_at(k + 1) : quads;
+#pragma unroll
+      for (int s = 0; s < STEPS; ++s) row[s] = mx[((u64)quad_next * kMxSteps + s) * 64];
+    }
     if (SWITCH && k == 0) {
       const u64 ql = c.primes[rz.last_prime].q;
       const u64* __restrict__ z = rz.z + op * rz.z_stride + col0;
@@ -591,8 +592,6 @@ __global__ __launch_bounds__(256, SWITCH ? 3 : 4) void conv_fwd_strided_kernel(D
       else conv_strided_column<ArithInt, SWITCH>(c, pi, lds + wv * 16 * kCfsCols, lane, dst, rs, rz, lds_last, lt);
     }
     __syncthreads();
-#pragma unroll
-    for (int s = 0; s < STEPS; ++s) row[s] = row_next[s];
   }
 }
 
