@@ -1315,7 +1315,7 @@ KeySet one_key(const u64* swk);
 // Every step is exact modulo its prime and Switch_modulus sees the same canonical word, so the results are the words
 // of do_switch_key followed by do_rescale.
 void do_switch_key_rescale(ace_ctx* c, const PolySeq& out, const u64* digits, u64 digits_op_stride, const u64* swk,
-                           size_t nb, size_t level, const Lift& lift, const OwnLimbs* own) {
+                           size_t nb, size_t level, const Lift& lift, const OwnLimbs* own, bool twice = false) {
   const size_t N = c->h.N, K = c->h.K, T = level + K, kpoly = (c->h.L + K) * N, nd = c->h.num_decomp(level);
   const size_t np = 2 * nb;
   const ModDownRescaleDev& m = c->moddown_rescale_at(level);
@@ -1348,6 +1348,7 @@ void do_switch_key_rescale(ace_ctx* c, const PolySeq& out, const u64* digits, u6
   f.src = seq_strided(e, T * N);
   f.addend = out;
   f.cst = m.tail;
+  f.twice = twice ? 1u : 0u;  // Rescale(2 (Mod_down(e) + d)): see FwdFuse
   PolySeq ys = seq_strided(y, level * N);
   // (large launches of N = 2^16: conversion, prologue and strided pass of the transform in one kernel)
   const bool strided_done = launch_baseconv_fwd_strided(c->stream, c->d, y, t + N, b, (u32)np, &f);
@@ -1366,8 +1367,9 @@ KeySet one_key(const u64* swk) {
 }
 
 // Mul_ciphertext + Rescale_ciphertext for nb ciphertext pairs (evaluator.c:142-190, 342-362)
+// twice: the relinearised product is added to itself before the Rescale (Add_ciph between the two)
 void do_mul_relin_rescale(ace_ctx* c, u64* r0, u64* r1, u64 out_stride, const u64* a0, const u64* a1, const u64* b0,
-                          const u64* b1, u64 in_stride, const u64* swk, size_t nb, size_t level) {
+                          const u64* b1, u64 in_stride, const u64* swk, size_t nb, size_t level, bool twice = false) {
   const size_t N = c->h.N, nd = c->h.num_decomp(level), T = level + c->h.K;
   // where the inner product can read the digits' own limbs from d2 itself, Mod_up does not copy them
   const bool from_d2 = c->d.logN > 12 && dotprod_reads_own(1, (u32)nb, true, (u32)nd);
@@ -1399,11 +1401,15 @@ void do_mul_relin_rescale(ace_ctx* c, u64* r0, u64* r1, u64 out_stride, const u6
     Lift lift{ds, c->pmodq, (u32)level, nullptr, nullptr, nullptr, nullptr, 0};
     if (on_the_way) lift.a0 = a0, lift.a1 = a1, lift.b0 = b0, lift.b1 = b1, lift.in_stride = in_stride;
     do_switch_key_rescale(c, seq_pair(r0, r1, out_stride), digits, nd * T * N, swk, nb, level, lift,
-                          from_d2 ? &own : nullptr);
+                          from_d2 ? &own : nullptr, twice);
     return;
   }
   do_switch_key(c, ds, digits, nd * T * N, one_key(swk), nb, level, &ds, 1, nullptr,
                 from_d2 ? &own : nullptr);  // relinearised ct replaces d0, d1
+  if (twice)
+    for (size_t p = 0; p < 2 * nb; ++p)
+      launch_ew(c->stream, c->d, EW_ADD, d01 + p * level * N, d01 + p * level * N, d01 + p * level * N, 0, c->q_lm,
+                (u32)level, N);
   do_rescale(c, seq_pair(r0, r1, out_stride), ds, 2 * nb, level, true);
 }
 
@@ -2640,6 +2646,18 @@ int ace_mul_relin_rescale(ace_ctx* c, int64_t* r0, int64_t* r1, const int64_t* a
   c->ensure_ws(c->std_ws(level));
   c->ws_used = 0;
   do_mul_relin_rescale(c, U(r0), U(r1), 0, U(a0), U(a1), U(b0), U(b1), 0, U(swk), 1, level);
+  ACE_CATCH_INT
+}
+
+int ace_mul_relin_double_rescale(ace_ctx* c, int64_t* r0, int64_t* r1, const int64_t* a0, const int64_t* a1,
+                                 const int64_t* b0, const int64_t* b1, const int64_t* swk, size_t level) {
+  ACE_TRY
+  CENSUS(level, 1);
+  if (!r0 || !r1 || !a0 || !a1 || !b0 || !b1 || !swk) return fail("ace_mul_relin_double_rescale: null argument");
+  if (level < 2 || level > c->h.L) return fail("ace_mul_relin_double_rescale: level out of range");
+  c->ensure_ws(c->std_ws(level));
+  c->ws_used = 0;
+  do_mul_relin_rescale(c, U(r0), U(r1), 0, U(a0), U(a1), U(b0), U(b1), 0, U(swk), 1, level, true);
   ACE_CATCH_INT
 }
 

@@ -238,6 +238,9 @@ struct FwdFuse {
   int addend_mode;
   const u64* cst;
   OrderSet orders;
+  // pro 2 with epi 2 only: the Mod_down's result is doubled before the Rescale (Add_ciph of a product with itself
+  // between Relinearize and Rescale_ciph): z - ylast, the converted words and the tail's product count twice
+  u32 twice;
 };
 
 }  // namespace ace

@@ -337,6 +337,13 @@ __device__ __forceinline__ void fwd_strided_input(const A& ar, const DevCtx& c, 
       for (int r = 0; r < R; ++r) { zs[r] = z[r * step]; xs[r] = yl[r * step]; ys[r] = ldg<2>(src + r * step); }
 #pragma unroll
       for (int r = 0; r < R; ++r) xs[r] = sub_mod(zs[r], xs[r], ql);
+      if (f.twice) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          xs[r] = add_mod(xs[r], xs[r], ql);
+          ys[r] = add_mod(ys[r], ys[r], P.q);
+        }
+      }
     }
     if constexpr (A::kFp) {
       // Both primes small enough for FP64: the centred value of the last limb's word (|x| <= ql/2 <= q) times the
@@ -467,6 +474,7 @@ struct ConvRescale {
   u64 z_stride;
   const u64* sw;
   u32 last_prime;
+  u32 twice;  // FwdFuse::twice
 };
 template <class A, bool SWITCH>
 __device__ __forceinline__ void conv_strided_column(const DevCtx& c, u32 pi, const u64* lds_target, u32 lane,
@@ -479,7 +487,11 @@ __device__ __forceinline__ void conv_strided_column(const DevCtx& c, u32 pi, con
     SwitchIn<A> in;
     in.init(ar, c, pi, rz.last_prime, rz.sw, lt);
 #pragma unroll
-    for (int r = 0; r < 16; ++r) v[r] = in.one(ar, lds_last[r * kCfsCols + lane], lds_target[r * kCfsCols + lane]);
+    for (int r = 0; r < 16; ++r) {
+      u64 y = lds_target[r * kCfsCols + lane];
+      if (rz.twice) y = add_mod(y, y, in.P.q);
+      v[r] = in.one(ar, lds_last[r * kCfsCols + lane], y);
+    }
   } else {
 #pragma unroll
     for (int r = 0; r < 16; ++r) v[r] = ar.in_canon(lds_target[r * kCfsCols + lane]);
@@ -580,7 +592,9 @@ __global__ __launch_bounds__(256, SWITCH ? 3 : 4) void conv_fwd_strided_kernel(D
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const u32 p = threadIdx.x + 256 * i;  // row p / 64, column p % 64
-        lds_last[p] = sub_mod(z[(u64)(p >> 6) * rs + (p & 63)], ylast[p], ql);
+        u64 last = sub_mod(z[(u64)(p >> 6) * rs + (p & 63)], ylast[p], ql);
+        if (rz.twice) last = add_mod(last, last, ql);
+        lds_last[p] = last;
       }
       __syncthreads();
     }
@@ -622,7 +636,7 @@ bool launch_baseconv_fwd_strided(hipStream_t st, const DevCtx& c, u64* out, cons
     if (rescale->pro != 2 || b.n_jobs != 1 || J.nc < 2 || J.map.out_limb[J.nc - 1] != J.nc - 1 ||
         rescale->ylast != out + J.out_off + (u64)(J.nc - 1) * c.N || rescale->ylast_stride != b.out_stride)
       return false;
-    rz = ConvRescale{rescale->z, rescale->z_stride, rescale->sw, rescale->last_prime};
+    rz = ConvRescale{rescale->z, rescale->z_stride, rescale->sw, rescale->last_prime, rescale->twice};
     if (max_nd <= 4) hipLaunchKernelGGL((conv_fwd_strided_kernel<1, true>), g, dim3(256), 0, st, c, out, t, b, rz);
     else hipLaunchKernelGGL((conv_fwd_strided_kernel<2, true>), g, dim3(256), 0, st, c, out, t, b, rz);
     return true;
@@ -794,7 +808,9 @@ __device__ __forceinline__ void fwd_chunk_tail(const DevCtx& c, const FwdFuse& f
           v = shoup_mul(sub_mod(sv[r], y, q), w, wp, q);
           if (addend) v = add_mod(v, av[r], q);
         } else {
-          v = add_mod(shoup_mul(sv[r], w, wp, q), y, q);
+          u64 scaled = shoup_mul(sv[r], w, wp, q);
+          if (f.twice) scaled = add_mod(scaled, scaled, q);
+          v = add_mod(scaled, y, q);
         }
         stg<16>(out + 64 * (r0 + r), v);
       }

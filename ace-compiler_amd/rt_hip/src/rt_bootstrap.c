@@ -868,8 +868,7 @@ static void eval_ps(CIPHER out, CHEB_BASIS* b, const SERIES* f, uint32_t m) {
     Copy_ciph(out, t2);
     add_const(out, c.v[0] / 2);
   }
-  Mul_ciph(out, out, &qu);
-  rescale(out);
+  Rt_mul_rescale_ciph(out, out, &qu, false); /* Mul_ciph, then Rescale_ciph */
   Add_ciph(out, out, &su);
 
   Free_ciph_poly(&cu, 1);
@@ -882,9 +881,7 @@ static void eval_ps(CIPHER out, CHEB_BASIS* b, const SERIES* f, uint32_t m) {
 static void cheb_product(CIPHER res, CIPHER a, CIPHER b, CIPHER sub) {
   CIPHERTEXT prod;
   new_ciph(&prod);
-  Mul_ciph(&prod, a, b);
-  Add_ciph(&prod, &prod, &prod);
-  rescale(&prod);
+  Rt_mul_rescale_ciph(&prod, a, b, true); /* Mul_ciph, Add_ciph(prod, prod), Rescale_ciph */
   if (sub)
     Sub_ciph(&prod, &prod, sub);
   else

@@ -808,6 +808,31 @@ CIPHER Mul_ciph(CIPHER res, CIPHER a, CIPHER b) {
   return res;
 }
 
+/* Mul_ciph followed by Rescale_ciph on its result, in one set of launches: the key switch's Mod_down and the Rescale
+ * share a forward transform there.  The words and the scale are those of the two calls one after the other
+ * (evaluator.c:142-190, 288-306, 342-362).  twice: with Add_ciph of the product with itself between the two
+ * (chebyshev_impl.c:563-565).  res may be one of the operands. */
+CIPHER Rt_mul_rescale_ciph(CIPHER res, CIPHER a, CIPHER b, bool twice) {
+  FMT_ASSERT(G.relin._public_keys, "no relinearisation key loaded");
+  CIPHER pick  = lower_of(a, b);
+  size_t level = Level(pick);
+  FMT_ASSERT(level > 1, "rescale: multiply level is not big enought for more operation");
+  FMT_ASSERT(a->_c0_poly._is_ntt && b->_c0_poly._is_ntt, "Mul_ciph3: operands must be in NTT form");
+  FMT_ASSERT(a->_sf_degree + b->_sf_degree >= 2, "Scale degree of result dec to zero");
+  CIPHERTEXT t;
+  memset(&t, 0, sizeof(t));
+  Rt_shape_ciph(&t, pick, a->_scaling_factor * b->_scaling_factor / G.sc, a->_sf_degree + b->_sf_degree - 1);
+  ACE_OK((twice ? ace_mul_relin_double_rescale : ace_mul_relin_rescale)(
+      RT_CTX, t._c0_poly._data, t._c1_poly._data, a->_c0_poly._data, a->_c1_poly._data, b->_c0_poly._data,
+      b->_c1_poly._data, G.relin._public_keys->dev, level));
+  Set_poly_level(&t._c0_poly, level - 1);
+  Set_poly_level(&t._c1_poly, level - 1);
+  Free_poly_data(&res->_c0_poly);
+  Free_poly_data(&res->_c1_poly);
+  *res = t;
+  return res;
+}
+
 CIPHER Rescale_ciph(CIPHER res, CIPHER c) {
   size_t level = Level(c);
   FMT_ASSERT(level > 1, "rescale: multiply level is not big enought for more operation");

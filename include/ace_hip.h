@@ -334,7 +334,12 @@ int ace_rescale_ciph(ace_ctx* ctx, int64_t* r0, int64_t* r1, const int64_t* c0, 
 /* Mul_ciphertext + Rescale_ciphertext (evaluator.c:177-190, 342-362): r0/r1 level-1 limbs */
 int ace_mul_relin_rescale(ace_ctx* ctx, int64_t* r0, int64_t* r1, const int64_t* a0, const int64_t* a1,
                           const int64_t* b0, const int64_t* b1, const int64_t* swk, size_t level);
-/* The same for `count` independent ciphertext pairs that share the relinearisation key: pair i reads
+/* Mul_ciphertext, Add_ciphertext of the product with itself, Rescale_ciphertext (evaluator.c:177-190, 47-76, 342-362):
+ * 2ab one level down, the step of the Chebyshev product rule as Eval_chebyshev_ps issues it
+ * (chebyshev_impl.c:563-565, 581-583, 597-599).  The words of the three calls one after the other. */
+int ace_mul_relin_double_rescale(ace_ctx* ctx, int64_t* r0, int64_t* r1, const int64_t* a0, const int64_t* a1,
+                                 const int64_t* b0, const int64_t* b1, const int64_t* swk, size_t level);
+/* ace_mul_relin_rescale for `count` independent ciphertext pairs that share the relinearisation key: pair i reads
  * a0 + i*in_stride (likewise a1, b0, b1) and writes r0 + i*out_stride, r1 + i*out_stride (strides in
  * words).  Equivalent to `count` calls of ace_mul_relin_rescale; every kernel launch covers the batch. */
 int ace_mul_relin_rescale_batch(ace_ctx* ctx, int64_t* r0, int64_t* r1, size_t out_stride, const int64_t* a0,

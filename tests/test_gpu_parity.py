@@ -861,6 +861,38 @@ def test_mul_relin_rescale_batch(pair):
         g.mul_relin_rescale_batch(r0, r1, n - 1, dev[0], dev[1], dev[2], dev[3], in_stride, dk, level, 2)  # overlap
 
 
+def test_mul_relin_double_rescale_equals_its_three_calls(pair):
+    """2ab one level down in one call (Mul_ciphertext, the product added to itself, Rescale_ciphertext): the words of
+    ace_mul_ciph3, ace_relin, an elementwise sum and ace_rescale_ciph issued one after the other, each of which the
+    oracle pins; likewise ace_mul_relin_rescale without the sum."""
+    g = pair.g
+    N = g.N
+    if g.L < 2:
+        pytest.skip("needs two levels")
+    big_ring_skip(N)
+    swk = g.alloc(2 * g.parts * (g.L + g.K) * N)
+    for i in range(2 * g.parts):
+        g.sample_uniform(swk.view(i * (g.L + g.K) * N, (g.L + g.K) * N), g.L, True, 7, 990 + i)
+    for level in sorted({g.L, max(2, g.L - 1), 2}):
+        a = [draw_poly(g, 1000 + 4 * level + i, level, False)[1] for i in range(4)]
+        d = [g.alloc(level * N) for _ in range(3)]
+        r0, r1, s0, s1 = (g.alloc(level * N) for _ in range(4))
+        n = (level - 1) * N
+        for twice in (False, True):
+            g.mul_ciph3(d[0], d[1], d[2], a[0], a[1], a[2], a[3], level)
+            g.relin(r0, r1, d[0], d[1], d[2], swk, level)
+            if twice:
+                g.poly("add", r0, r0, r0, level)
+                g.poly("add", r1, r1, r1, level)
+            g.rescale_ciph(r0, r1, r0, r1, level)
+            (g.mul_relin_double_rescale if twice else g.mul_relin_rescale)(s0, s1, a[0], a[1], a[2], a[3], swk, level)
+            eq(s0.get()[:n], r0.get()[:n], "level %d twice=%d c0" % (level, twice))
+            eq(s1.get()[:n], r1.get()[:n], "level %d twice=%d c1" % (level, twice))
+        for b in a + d + [r0, r1, s0, s1]:
+            b.free()
+    swk.free()
+
+
 def test_two_lanes_equal_one(pair):
     """ace_fork / ace_fork_switch / ace_join: two independent sequences of calls (HMult + relinearise + rescale, a
     transform there and back, recorded elementwise calls, buffers allocated and freed on the way) issued on the two
