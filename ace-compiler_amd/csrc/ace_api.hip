@@ -2018,12 +2018,19 @@ int ace_automorphism_order(ace_ctx* c, int64_t* dev_order, uint32_t k, int is_nt
 
 // ---- polynomial ops ---------------------------------------------------------------
 static int poly_ew(ace_ctx* c, EwOp op, int64_t* r, const int64_t* a, const int64_t* b, size_t level, int with_p) {
-  ACE_TRY
+  ACE_TRY_KEEP_RUN
   CENSUS_AS(op == EW_MUL ? "poly_mul" : "poly_add", level + (with_p ? c->h.K : 0), 0);
   if (!r || !a || !b) return fail("ace_poly: null argument");
   if (!level_ok(c, level)) return fail("ace_poly: level out of range");
   LimbMap lm = poly_lm(c, level, with_p != 0);
-  launch_ew(c->stream, c->d, op, U(r), U(a), U(b), 0, lm, (u32)(level + (with_p ? c->h.K : 0)), c->h.N);
+  const size_t n_limbs = level + (with_p ? c->h.K : 0), N = c->h.N;
+  if (c->batching) {  // limb by limb into the recorded run: the sums and differences between two larger calls leave
+                      // as one launch (a ciphertext sum is two of these calls, often with a constant added next)
+    for (size_t t = 0; t < n_limbs; ++t)
+      c->run_append(BatchOp{U(r) + t * N, U(a) + t * N, U(b) + t * N, 0, (u32)op, (u32)lm.prime[t]}, N);
+    return 0;
+  }
+  launch_ew(c->stream, c->d, op, U(r), U(a), U(b), 0, lm, (u32)n_limbs, N);
   ACE_CATCH_INT
 }
 int ace_poly_add(ace_ctx* c, int64_t* r, const int64_t* a, const int64_t* b, size_t level, int with_p) { return poly_ew(c, EW_ADD, r, a, b, level, with_p); }
@@ -2104,7 +2111,7 @@ int ace_ext_plain_mac_groups(ace_ctx* c, int64_t* const* r0, int64_t* const* r1,
 }
 
 static int poly_scalars(ace_ctx* c, bool mul, int64_t* r, const int64_t* a, const int64_t* scalars, size_t level) {
-  ACE_TRY
+  ACE_TRY_KEEP_RUN
   CENSUS_AS(mul ? "poly_mul_scalars" : "poly_add_scalars", level, 0);
   if (!r || !a || !scalars) return fail("ace_poly_scalars: null argument");
   if (!level_ok(c, level)) return fail("ace_poly_scalars: level out of range");
@@ -2112,6 +2119,12 @@ static int poly_scalars(ace_ctx* c, bool mul, int64_t* r, const int64_t* a, cons
   for (size_t t = 0; t < level; ++t) {
     if (scalars[t] < 0 || (u64)scalars[t] >= c->h.primes[t].q) return fail("ace_poly_scalars: scalar is not a residue");
     s.v[t] = (u64)scalars[t];
+  }
+  if (c->batching) {  // (recorded like the sums above)
+    const size_t N = c->h.N;
+    for (size_t t = 0; t < level; ++t)
+      c->run_append(BatchOp{U(r) + t * N, U(a) + t * N, nullptr, s.v[t], (u32)(mul ? EW_MUL_S : EW_ADD_S), (u32)t}, N);
+    return 0;
   }
   launch_limb_scalars(c->stream, c->d, mul, U(r), U(a), s, poly_lm(c, level, false), (u32)level, c->h.N);
   ACE_CATCH_INT
