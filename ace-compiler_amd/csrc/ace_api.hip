@@ -1702,7 +1702,7 @@ void ace_free(ace_ctx* c, int64_t* p) {
 }
 // copies and fills longer than this go to the copy engine's / the fill kernel's own launch: a recorded entry moves
 // one word per thread, which is right for a limb and slow for a whole batch
-static constexpr size_t kRecordedWords = (size_t)1 << 20;
+static constexpr size_t kRecordedWords = (size_t)1 << 22;
 int ace_upload(ace_ctx* c, int64_t* dst, const int64_t* src, size_t n) {
   ACE_TRY
   c->forget_orders(dst, n);
@@ -1724,7 +1724,7 @@ int ace_copy(ace_ctx* c, int64_t* dst, const int64_t* src, size_t n) {
   c->forget_orders(dst, n);
   if (c->batching && n <= kRecordedWords) {  // a copy is an elementwise entry like any other
     // whole limbs go in limb by limb, so that they join the limb-sized calls around them in one run
-    const size_t N = c->h.N, pieces = (n % N == 0 && n / N <= 16) ? n / N : 1, each = n / pieces;
+    const size_t N = c->h.N, pieces = (n % N == 0 && n / N <= 64) ? n / N : 1, each = n / pieces;
     for (size_t t = 0; t < pieces; ++t)
       c->run_append(BatchOp{U(dst) + t * each, U(src) + t * each, nullptr, 0, (u32)BATCH_COPY, 0}, each);
     return 0;
@@ -1740,7 +1740,7 @@ int ace_zero(ace_ctx* c, int64_t* dst, size_t n) {
   if (n == 0) return 0;
   c->forget_orders(dst, n);
   if (c->batching && n <= kRecordedWords) {
-    const size_t N = c->h.N, pieces = (n % N == 0 && n / N <= 16) ? n / N : 1, each = n / pieces;
+    const size_t N = c->h.N, pieces = (n % N == 0 && n / N <= 64) ? n / N : 1, each = n / pieces;
     for (size_t t = 0; t < pieces; ++t)
       c->run_append(BatchOp{U(dst) + t * each, nullptr, nullptr, 0, (u32)BATCH_ZERO, 0}, each);
     return 0;
