@@ -1314,20 +1314,16 @@ KeySet one_key(const u64* swk);
 // inverse transform that serves the P limbs takes that limb along.
 // Every step is exact modulo its prime and Switch_modulus sees the same canonical word, so the results are the words
 // of do_switch_key followed by do_rescale.
-void do_switch_key_rescale(ace_ctx* c, const PolySeq& out, const u64* digits, u64 digits_op_stride, const u64* swk,
-                           size_t nb, size_t level, const Lift& lift, const OwnLimbs* own, bool twice = false) {
-  const size_t N = c->h.N, K = c->h.K, T = level + K, kpoly = (c->h.L + K) * N, nd = c->h.num_decomp(level);
-  const size_t np = 2 * nb;
+// Rescale(Mod_down(e_p)) for np polynomials of the extended basis (es.at(p): level + K limbs, NTT form) through the one
+// forward transform described above; twice: Rescale(2 Mod_down(e_p)).  Scratch from the arena.
+void do_moddown_rescale_shared(ace_ctx* c, const PolySeq& out, const PolySeq& es, size_t np, size_t level, bool twice) {
+  const size_t N = c->h.N, K = c->h.K;
   const ModDownRescaleDev& m = c->moddown_rescale_at(level);
   const RescaleDev& r = c->rescale_at(level);
   size_t mark = c->ws_used;
-  u64* e = c->take(np * T * N);        // [operand][b|a][T limbs], the addend lifted in
   u64* t = c->take(np * (K + 1) * N);  // per polynomial: the dropped limb's z, then the scaled P limbs
   u64* y = c->take(np * level * N);
-  LimbMap lm = poly_lm(c, level, true), kp = key_pos(c, level);
-  launch_dotprod(c->stream, c->d, e, e + T * N, 2 * T * N, digits, T * N, digits_op_stride, one_key(swk), kpoly,
-                 2 * kpoly, (u32)nd, lm, kp, (u32)T, (u32)nb, own, &lift);
-  launch_ntt(c->stream, c->d, seq_strided(t, (K + 1) * N), seq_strided(e + (level - 1) * N, T * N), m.inv_lm, nullptr,
+  launch_ntt(c->stream, c->d, seq_strided(t, (K + 1) * N), shifted(es, (level - 1) * N), m.inv_lm, nullptr,
              (u32)(K + 1), (u32)np, true, m.inv_scale);
   ConvBatch b{};
   b.matrix = c->conv_matrix;
@@ -1345,7 +1341,7 @@ void do_switch_key_rescale(ace_ctx* c, const PolySeq& out, const u64* digits, u6
   f.ylast_stride = level * N;
   f.epi = 2;
   f.out = out;
-  f.src = seq_strided(e, T * N);
+  f.src = es;
   f.addend = out;
   f.cst = m.tail;
   f.twice = twice ? 1u : 0u;  // Rescale(2 (Mod_down(e) + d)): see FwdFuse
@@ -1356,6 +1352,19 @@ void do_switch_key_rescale(ace_ctx* c, const PolySeq& out, const u64* digits, u6
   if (!launch_ntt(c->stream, c->d, ys, ys, c->q_lm, nullptr, (u32)(level - 1), (u32)np, false, nullptr,
                   strided_done ? 2 : 3, &f))
     throw std::runtime_error("internal: fused Mod_down + Rescale transform rejected");
+  c->ws_used = mark;
+}
+
+void do_switch_key_rescale(ace_ctx* c, const PolySeq& out, const u64* digits, u64 digits_op_stride, const u64* swk,
+                           size_t nb, size_t level, const Lift& lift, const OwnLimbs* own, bool twice = false) {
+  const size_t N = c->h.N, K = c->h.K, T = level + K, kpoly = (c->h.L + K) * N, nd = c->h.num_decomp(level);
+  const size_t np = 2 * nb;
+  size_t mark = c->ws_used;
+  u64* e = c->take(np * T * N);  // [operand][b|a][T limbs], the addend lifted in
+  LimbMap lm = poly_lm(c, level, true), kp = key_pos(c, level);
+  launch_dotprod(c->stream, c->d, e, e + T * N, 2 * T * N, digits, T * N, digits_op_stride, one_key(swk), kpoly,
+                 2 * kpoly, (u32)nd, lm, kp, (u32)T, (u32)nb, own, &lift);
+  do_moddown_rescale_shared(c, out, seq_strided(e, T * N), np, level, twice);
   c->ws_used = mark;
 }
 
@@ -2671,6 +2680,31 @@ int ace_mul_relin_double_rescale(ace_ctx* c, int64_t* r0, int64_t* r1, const int
   c->ensure_ws(c->std_ws(level));
   c->ws_used = 0;
   do_mul_relin_rescale(c, U(r0), U(r1), 0, U(a0), U(a1), U(b0), U(b1), 0, U(swk), 1, level, true);
+  ACE_CATCH_INT
+}
+
+static bool ranges_overlap(const void* a, size_t a_words, const void* b, size_t b_words);
+int ace_mod_down_pair_rescale(ace_ctx* c, int64_t* r0, int64_t* r1, const int64_t* e0, const int64_t* e1, size_t level) {
+  ACE_TRY
+  CENSUS(level, 2);
+  if (!r0 || !r1 || !e0 || !e1) return fail("ace_mod_down_pair_rescale: null argument");
+  if (level < 2 || level > c->h.L) return fail("ace_mod_down_pair_rescale: level out of range");
+  {
+    const size_t rw = (level - 1) * (size_t)c->h.N, ew = (level + c->h.K) * (size_t)c->h.N;
+    if (ranges_overlap(r0, rw, r1, rw) || ranges_overlap(r0, rw, e0, ew) || ranges_overlap(r0, rw, e1, ew) ||
+        ranges_overlap(r1, rw, e0, ew) || ranges_overlap(r1, rw, e1, ew))
+      return fail("ace_mod_down_pair_rescale: the results must not overlap the operands or each other");
+  }
+  c->ensure_ws(c->std_ws(level));
+  c->ws_used = 0;
+  const size_t N = c->h.N;
+  if (c->d.logN > 12 && c->share_transform) {
+    do_moddown_rescale_shared(c, seq_pair(U(r0), U(r1), 0), seq_pair(U(e0), U(e1), 0), 2, level, false);
+  } else {
+    u64* x = c->take(2 * level * N);
+    do_mod_down(c, seq_strided(x, level * N), seq_pair(U(e0), U(e1), 0), 2, level, true, nullptr, 0);
+    do_rescale(c, seq_pair(U(r0), U(r1), 0), seq_strided(x, level * N), 2, level, true);
+  }
   ACE_CATCH_INT
 }
 

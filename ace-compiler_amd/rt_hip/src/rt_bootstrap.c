@@ -574,11 +574,14 @@ static void ext_rotate(EXT_CT* out, const int64_t* digits, size_t n_digits, cons
   ACE_OK(ace_ext_rotate(RT_CTX, out->c0, out->c1, digits, key->swk._public_keys->dev, half, 2 * half, n_digits, c0_ext,
                         key->order, level, accumulate));
 }
-static void rotate_iteration(CIPHER ct, BTS_PRECOM* pre, bool encoding, int32_t s, bool is_rem, bool first_step) {
+/* rescaled_already: the previous iteration ended with its Rescale_ciph (see the end of this function);
+ * then_rescale: another iteration follows, which begins with a Rescale_ciph of this one's result */
+static void rotate_iteration(CIPHER ct, BTS_PRECOM* pre, bool encoding, int32_t s, bool is_rem, bool first_step,
+                             bool rescaled_already, bool then_rescale) {
   const FFT_PLAN* p      = encoding ? &pre->enc : &pre->dec;
   PLAINTEXT*      plains = (encoding ? pre->enc_plain : pre->dec_plain)[s];
   LEVEL_ROTS      r      = level_rots(p, s, encoding, is_rem, pre->slots);
-  if (!first_step) rescale(ct);
+  if (!first_step && !rescaled_already) rescale(ct);
   size_t level = Level(ct), T = level + G.K, n = G.N, nd = ace_num_decomp(RT_CTX, level);
 
   int64_t* digits = Rt_dev_alloc_raw(nd * T * n);
@@ -659,10 +662,23 @@ static void rotate_iteration(CIPHER ct, BTS_PRECOM* pre, bool encoding, int32_t 
   free(in_r0);
   free(in_r1);
   free((void*)inp);
-  ACE_OK(ace_mod_down(RT_CTX, ct->_c0_poly._data, first, level, 1));
-  ACE_OK(ace_mod_down(RT_CTX, ct->_c1_poly._data, sum1, level, 1));
-  ct->_scaling_factor *= G.sc;
-  ct->_sf_degree += 1;
+  if (then_rescale && level > 1) {
+    /* Mod_down of both sums and the Rescale_ciph that the next iteration would start with, through one forward
+     * transform (the words of the calls one after the other); the results need buffers of their own */
+    CIPHERTEXT down;
+    new_ciph(&down);
+    Rt_shape_ciph(&down, ct, ct->_scaling_factor, ct->_sf_degree); /* (sf * sc / sc, degree + 1 - 1) */
+    ACE_OK(ace_mod_down_pair_rescale(RT_CTX, down._c0_poly._data, down._c1_poly._data, first, sum1, level));
+    Set_poly_level(&down._c0_poly, level - 1);
+    Set_poly_level(&down._c1_poly, level - 1);
+    Free_ciph_poly(ct, 1);
+    *ct = down;
+  } else {
+    ACE_OK(ace_mod_down(RT_CTX, ct->_c0_poly._data, first, level, 1));
+    ACE_OK(ace_mod_down(RT_CTX, ct->_c1_poly._data, sum1, level, 1));
+    ct->_scaling_factor *= G.sc;
+    ct->_sf_degree += 1;
+  }
 
   for (int32_t j = 0; j < r.giant; ++j) ext_free(&rots[j]);
   free(rots);
@@ -680,7 +696,7 @@ static void coeff_slots_transform(CIPHER ct, BTS_PRECOM* pre, bool encoding) {
   int32_t         s_of[32], n;
   bool            rem_of[32];
   level_order(p, encoding, s_of, rem_of, &n);
-  for (int32_t t = 0; t < n; ++t) rotate_iteration(ct, pre, encoding, s_of[t], rem_of[t], t == 0);
+  for (int32_t t = 0; t < n; ++t) rotate_iteration(ct, pre, encoding, s_of[t], rem_of[t], t == 0, t > 0, t + 1 < n);
 }
 
 /* ---- Chebyshev series by Paterson-Stockmeyer (chebyshev_impl.c) -------------------------------------

@@ -334,6 +334,11 @@ int ace_rescale_ciph(ace_ctx* ctx, int64_t* r0, int64_t* r1, const int64_t* c0, 
 /* Mul_ciphertext + Rescale_ciphertext (evaluator.c:177-190, 342-362): r0/r1 level-1 limbs */
 int ace_mul_relin_rescale(ace_ctx* ctx, int64_t* r0, int64_t* r1, const int64_t* a0, const int64_t* a1,
                           const int64_t* b0, const int64_t* b1, const int64_t* swk, size_t level);
+/* Mod_down (rns_poly.c:260-308) of two polynomials of the extended basis (level + num_p limbs, NTT form) followed by
+ * Rescale (rns_poly.c:310-404) of both: what ends a linear transform carried out in the extended basis when a
+ * Rescale_ciphertext follows.  r0/r1: level - 1 limbs, apart from the operands and from each other.  The words of
+ * ace_mod_down twice and ace_rescale_ciph. */
+int ace_mod_down_pair_rescale(ace_ctx* ctx, int64_t* r0, int64_t* r1, const int64_t* e0, const int64_t* e1, size_t level);
 /* Mul_ciphertext, Add_ciphertext of the product with itself, Rescale_ciphertext (evaluator.c:177-190, 47-76, 342-362):
  * 2ab one level down, the step of the Chebyshev product rule as Eval_chebyshev_ps issues it
  * (chebyshev_impl.c:563-565, 581-583, 597-599).  The words of the three calls one after the other. */

@@ -893,6 +893,41 @@ def test_mul_relin_double_rescale_equals_its_three_calls(pair):
     swk.free()
 
 
+def test_mod_down_pair_rescale_equals_its_calls(pair):
+    """Mod_down of the two extended halves of a ciphertext followed by Rescale_ciphertext, in one call: the words of
+    ace_mod_down twice and ace_rescale_ciph issued one after the other, each of which the oracle pins; at the top
+    level, one below, and the lowest that can be rescaled; overlapping operands are rejected."""
+    g = pair.g
+    N = g.N
+    if g.L < 2:
+        pytest.skip("needs two levels")
+    big_ring_skip(N)
+    for level in sorted({g.L, max(2, g.L - 1), 2}):
+        e = [draw_poly(g, 1100 + 2 * level + i, level, True)[1] for i in range(2)]
+        kept = [b.get() for b in e]
+        m0, m1, r0, r1, s0, s1 = (g.alloc(level * N) for _ in range(6))
+        g.mod_down(m0, e[0], level)
+        g.mod_down(m1, e[1], level)
+        g.rescale_ciph(r0, r1, m0, m1, level)
+        g.mod_down_pair_rescale(s0, s1, e[0], e[1], level)
+        n = (level - 1) * N
+        eq(s0.get()[:n], r0.get()[:n], "level %d c0" % level)
+        eq(s1.get()[:n], r1.get()[:n], "level %d c1" % level)
+        eq(e[0], kept[0], "operand 0 untouched")
+        eq(e[1], kept[1], "operand 1 untouched")
+        with pytest.raises(acefhe.AceError):
+            g.mod_down_pair_rescale(e[0], s1, e[0], e[1], level)
+        for b in e + [m0, m1, r0, r1, s0, s1]:
+            b.free()
+    with pytest.raises(acefhe.AceError):
+        e0, e1 = (g.alloc((1 + g.K) * N) for _ in range(2))
+        try:
+            g.mod_down_pair_rescale(e0, e1, e0, e1, 1)  # nothing to drop at level 1
+        finally:
+            e0.free()
+            e1.free()
+
+
 def test_two_lanes_equal_one(pair):
     """ace_fork / ace_fork_switch / ace_join: two independent sequences of calls (HMult + relinearise + rescale, a
     transform there and back, recorded elementwise calls, buffers allocated and freed on the way) issued on the two
