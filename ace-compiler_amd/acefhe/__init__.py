@@ -105,6 +105,7 @@ def _sig(lib):
     f("ace_mul_relin_rescale", C.c_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz)
     f("ace_mod_down_pair_rescale", C.c_int, _vp, _vp, _vp, _vp, _vp, _sz)
     f("ace_mul_relin_double_rescale", C.c_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz)
+    f("ace_mul_relin_double_add_rescale", C.c_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64p, _sz)
     f("ace_mul_relin_rescale_batch", C.c_int, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _sz, _vp, _sz, _sz)
     f("ace_fast_rotate", C.c_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz)
     f("ace_rotate_batch", C.c_int, _vp, _vp, _vp, _vp, _vp, C.POINTER(_vp), C.POINTER(_vp), _sz, _sz)
@@ -131,7 +132,7 @@ EXPORTS = [
     "ace_poly_automorphism", "ace_decomp_modup", "ace_mod_up", "ace_mod_down_rescale",
     "ace_reduce_rescale_modup", "ace_transform_from_level0", "ace_host_fft_tables", "ace_embedding_inv", "ace_decode", "ace_fork", "ace_fork_switch", "ace_join", "ace_encode", "ace_encode_scaled", "ace_encode_real", "ace_encode_real_batch", "ace_ext_rotate", "ace_ext_plain_mac_groups", "ace_precomp", "ace_mod_down", "ace_rescale", "ace_extend",
     "ace_dot_prod", "ace_mul_ciph3", "ace_fast_switch_key", "ace_relin", "ace_rescale_ciph",
-    "ace_mul_relin_rescale", "ace_mod_down_pair_rescale", "ace_mul_relin_double_rescale", "ace_mul_relin_rescale_batch", "ace_fast_rotate", "ace_rotate_batch",
+    "ace_mul_relin_rescale", "ace_mod_down_pair_rescale", "ace_mul_relin_double_rescale", "ace_mul_relin_double_add_rescale", "ace_mul_relin_rescale_batch", "ace_fast_rotate", "ace_rotate_batch",
 ]
 
 _lib = None
@@ -451,6 +452,12 @@ class Context:
     def mul_relin_double_rescale(self, r0, r1, a0, a1, b0, b1, swk, level):
         self._chk(self.lib.ace_mul_relin_double_rescale(self.h, r0.ptr, r1.ptr, a0.ptr, a1.ptr, b0.ptr, b1.ptr, swk.ptr,
                                                         level))
+
+    def mul_relin_double_add_rescale(self, r0, r1, a0, a1, b0, b1, swk, constant, level):
+        sc = np.ascontiguousarray(constant, dtype=np.int64)
+        assert sc.size >= level
+        self._chk(self.lib.ace_mul_relin_double_add_rescale(self.h, r0.ptr, r1.ptr, a0.ptr, a1.ptr, b0.ptr, b1.ptr,
+                                                            swk.ptr, sc.ctypes.data_as(_i64p), level))
 
     def mul_relin_rescale_batch(self, r0, r1, out_stride, a0, a1, b0, b1, in_stride, swk, level, count):
         self._chk(self.lib.ace_mul_relin_rescale_batch(self.h, r0.ptr, r1.ptr, out_stride, a0.ptr, a1.ptr, b0.ptr,

@@ -73,6 +73,7 @@ struct ModDownRescaleDev {
   u64* inv_scale = nullptr;  // [1 + K][2]: (1/N * P^-1 mod q_last) for the dropped limb, then the P limbs' Mod_down scales
   u64* tail = nullptr;       // [level-1][2]: (P q_last)^-1 mod q_t
   LimbMap inv_lm{};          // the dropped limb, then the P limbs
+  std::vector<u64> ql_inv;   // host copy: q_last^-1 mod q_t, t < level - 1
   // P -> Q conversion onto the level's limbs with a constant folded into each target's column of the matrix:
   // -(P q_last)^-1 mod q_t for t < level - 1, P^-1 mod q_last for the dropped limb
   ConvJob job{};
@@ -556,6 +557,7 @@ struct ace_ctx {
       tl[2 * i] = t; tl[2 * i + 1] = shoup(t, q);
     }
     colc[last] = h.pinv_modq[last];
+    m.ql_inv.assign(qi.begin(), qi.begin() + last);
     m.inv_scale = upload_vec(sc);
     m.tail = upload_vec(tl);
     {
@@ -1316,7 +1318,13 @@ KeySet one_key(const u64* swk);
 // of do_switch_key followed by do_rescale.
 // Rescale(Mod_down(e_p)) for np polynomials of the extended basis (es.at(p): level + K limbs, NTT form) through the one
 // forward transform described above; twice: Rescale(2 Mod_down(e_p)).  Scratch from the arena.
-void do_moddown_rescale_shared(ace_ctx* c, const PolySeq& out, const PolySeq& es, size_t np, size_t level, bool twice) {
+// constant: `level` residues of an integer C that is added to polynomial 0 as a constant polynomial before the Rescale
+// (Add_const between the Mod_down and the Rescale: every word of limb t in NTT form + C mod q_t), or null:
+// Rescale(Mod_down(e_0) [* 2] + C).  Only coefficient 0 of the sum's coefficient form differs, so the dropped limb's
+// coefficient 0 gets C mod q_l before it is switched to the other primes (half of it where the kernel doubles
+// afterwards: the primes are odd), and every word of limb t of the result gets (C mod q_t) * q_l^-1.
+void do_moddown_rescale_shared(ace_ctx* c, const PolySeq& out, const PolySeq& es, size_t np, size_t level, bool twice,
+                               const u64* constant = nullptr) {
   const size_t N = c->h.N, K = c->h.K;
   const ModDownRescaleDev& m = c->moddown_rescale_at(level);
   const RescaleDev& r = c->rescale_at(level);
@@ -1325,6 +1333,15 @@ void do_moddown_rescale_shared(ace_ctx* c, const PolySeq& out, const PolySeq& es
   u64* y = c->take(np * level * N);
   launch_ntt(c->stream, c->d, seq_strided(t, (K + 1) * N), shifted(es, (level - 1) * N), m.inv_lm, nullptr,
              (u32)(K + 1), (u32)np, true, m.inv_scale);
+  const u64 ql = c->h.primes[level - 1].q;
+  if (constant) {
+    LimbScalars s{};
+    LimbMap last{};
+    last.prime[0] = (u32)(level - 1);
+    const u64 cl = constant[level - 1];
+    s.v[0] = !twice ? cl : (cl & 1) ? (cl + ql) >> 1 : cl >> 1;  // C / 2 modulo the odd q_l (q_l < 2^63)
+    launch_limb_scalars(c->stream, c->d, false, t, t, s, last, 1, 1);  // one word: z[0] of polynomial 0
+  }
   ConvBatch b{};
   b.matrix = c->conv_matrix;
   b.n_jobs = 1;
@@ -1352,11 +1369,21 @@ void do_moddown_rescale_shared(ace_ctx* c, const PolySeq& out, const PolySeq& es
   if (!launch_ntt(c->stream, c->d, ys, ys, c->q_lm, nullptr, (u32)(level - 1), (u32)np, false, nullptr,
                   strided_done ? 2 : 3, &f))
     throw std::runtime_error("internal: fused Mod_down + Rescale transform rejected");
+  if (constant) {
+    LimbScalars s{};
+    for (size_t i = 0; i + 1 < level; ++i) {
+      const u64 q = c->h.primes[i].q;
+      s.v[i] = mul_mod(constant[i], m.ql_inv[i], q);
+    }
+    u64* o = const_cast<u64*>(out.at(0));
+    launch_limb_scalars(c->stream, c->d, false, o, o, s, poly_lm(c, level - 1, false), (u32)(level - 1), N);
+  }
   c->ws_used = mark;
 }
 
 void do_switch_key_rescale(ace_ctx* c, const PolySeq& out, const u64* digits, u64 digits_op_stride, const u64* swk,
-                           size_t nb, size_t level, const Lift& lift, const OwnLimbs* own, bool twice = false) {
+                           size_t nb, size_t level, const Lift& lift, const OwnLimbs* own, bool twice = false,
+                           const u64* constant = nullptr) {
   const size_t N = c->h.N, K = c->h.K, T = level + K, kpoly = (c->h.L + K) * N, nd = c->h.num_decomp(level);
   const size_t np = 2 * nb;
   size_t mark = c->ws_used;
@@ -1364,7 +1391,7 @@ void do_switch_key_rescale(ace_ctx* c, const PolySeq& out, const u64* digits, u6
   LimbMap lm = poly_lm(c, level, true), kp = key_pos(c, level);
   launch_dotprod(c->stream, c->d, e, e + T * N, 2 * T * N, digits, T * N, digits_op_stride, one_key(swk), kpoly,
                  2 * kpoly, (u32)nd, lm, kp, (u32)T, (u32)nb, own, &lift);
-  do_moddown_rescale_shared(c, out, seq_strided(e, T * N), np, level, twice);
+  do_moddown_rescale_shared(c, out, seq_strided(e, T * N), np, level, twice, constant);
   c->ws_used = mark;
 }
 
@@ -1377,8 +1404,10 @@ KeySet one_key(const u64* swk) {
 
 // Mul_ciphertext + Rescale_ciphertext for nb ciphertext pairs (evaluator.c:142-190, 342-362)
 // twice: the relinearised product is added to itself before the Rescale (Add_ciph between the two)
+// constant (nb == 1): `level` residues of an integer added to c0 as a constant polynomial after that (Add_const)
 void do_mul_relin_rescale(ace_ctx* c, u64* r0, u64* r1, u64 out_stride, const u64* a0, const u64* a1, const u64* b0,
-                          const u64* b1, u64 in_stride, const u64* swk, size_t nb, size_t level, bool twice = false) {
+                          const u64* b1, u64 in_stride, const u64* swk, size_t nb, size_t level, bool twice = false,
+                          const u64* constant = nullptr) {
   const size_t N = c->h.N, nd = c->h.num_decomp(level), T = level + c->h.K;
   // where the inner product can read the digits' own limbs from d2 itself, Mod_up does not copy them
   const bool from_d2 = c->d.logN > 12 && dotprod_reads_own(1, (u32)nb, true, (u32)nd);
@@ -1410,7 +1439,7 @@ void do_mul_relin_rescale(ace_ctx* c, u64* r0, u64* r1, u64 out_stride, const u6
     Lift lift{ds, c->pmodq, (u32)level, nullptr, nullptr, nullptr, nullptr, 0};
     if (on_the_way) lift.a0 = a0, lift.a1 = a1, lift.b0 = b0, lift.b1 = b1, lift.in_stride = in_stride;
     do_switch_key_rescale(c, seq_pair(r0, r1, out_stride), digits, nd * T * N, swk, nb, level, lift,
-                          from_d2 ? &own : nullptr, twice);
+                          from_d2 ? &own : nullptr, twice, constant);
     return;
   }
   do_switch_key(c, ds, digits, nd * T * N, one_key(swk), nb, level, &ds, 1, nullptr,
@@ -1419,6 +1448,11 @@ void do_mul_relin_rescale(ace_ctx* c, u64* r0, u64* r1, u64 out_stride, const u6
     for (size_t p = 0; p < 2 * nb; ++p)
       launch_ew(c->stream, c->d, EW_ADD, d01 + p * level * N, d01 + p * level * N, d01 + p * level * N, 0, c->q_lm,
                 (u32)level, N);
+  if (constant) {
+    LimbScalars sc{};
+    for (size_t t = 0; t < level; ++t) sc.v[t] = constant[t];
+    launch_limb_scalars(c->stream, c->d, false, d01, d01, sc, poly_lm(c, level, false), (u32)level, N);
+  }
   do_rescale(c, seq_pair(r0, r1, out_stride), ds, 2 * nb, level, true);
 }
 
@@ -2680,6 +2714,26 @@ int ace_mul_relin_double_rescale(ace_ctx* c, int64_t* r0, int64_t* r1, const int
   c->ensure_ws(c->std_ws(level));
   c->ws_used = 0;
   do_mul_relin_rescale(c, U(r0), U(r1), 0, U(a0), U(a1), U(b0), U(b1), 0, U(swk), 1, level, true);
+  ACE_CATCH_INT
+}
+
+int ace_mul_relin_double_add_rescale(ace_ctx* c, int64_t* r0, int64_t* r1, const int64_t* a0, const int64_t* a1,
+                                     const int64_t* b0, const int64_t* b1, const int64_t* swk, const int64_t* constant,
+                                     size_t level) {
+  ACE_TRY
+  CENSUS(level, 1);
+  if (!r0 || !r1 || !a0 || !a1 || !b0 || !b1 || !swk || !constant)
+    return fail("ace_mul_relin_double_add_rescale: null argument");
+  if (level < 2 || level > c->h.L) return fail("ace_mul_relin_double_add_rescale: level out of range");
+  u64 words[kMaxPrimes];
+  for (size_t t = 0; t < level; ++t) {
+    if (constant[t] < 0 || (u64)constant[t] >= c->h.primes[t].q)
+      return fail("ace_mul_relin_double_add_rescale: constant is not a residue");
+    words[t] = (u64)constant[t];
+  }
+  c->ensure_ws(c->std_ws(level));
+  c->ws_used = 0;
+  do_mul_relin_rescale(c, U(r0), U(r1), 0, U(a0), U(a1), U(b0), U(b1), 0, U(swk), 1, level, true, words);
   ACE_CATCH_INT
 }
 

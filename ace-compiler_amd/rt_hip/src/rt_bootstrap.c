@@ -884,7 +884,7 @@ static void eval_ps(CIPHER out, CHEB_BASIS* b, const SERIES* f, uint32_t m) {
     Copy_ciph(out, t2);
     add_const(out, c.v[0] / 2);
   }
-  Rt_mul_rescale_ciph(out, out, &qu, false); /* Mul_ciph, then Rescale_ciph */
+  Rt_mul_rescale_ciph(out, out, &qu, false, NULL); /* Mul_ciph, then Rescale_ciph */
   Add_ciph(out, out, &su);
 
   Free_ciph_poly(&cu, 1);
@@ -897,7 +897,7 @@ static void eval_ps(CIPHER out, CHEB_BASIS* b, const SERIES* f, uint32_t m) {
 static void cheb_product(CIPHER res, CIPHER a, CIPHER b, CIPHER sub) {
   CIPHERTEXT prod;
   new_ciph(&prod);
-  Rt_mul_rescale_ciph(&prod, a, b, true); /* Mul_ciph, Add_ciph(prod, prod), Rescale_ciph */
+  Rt_mul_rescale_ciph(&prod, a, b, true, NULL); /* Mul_ciph, Add_ciph(prod, prod), Rescale_ciph */
   if (sub)
     Sub_ciph(&prod, &prod, sub);
   else
@@ -983,11 +983,9 @@ static void eval_approx_mod(CIPHER ct) {
   if (p->even) add_const(ct, -1.0 / (4.0 * p->k_bound));
   eval_chebyshev(ct, p->coeff, p->n_coeff, p->even);
   int32_t r = (int32_t)p->double_angle;
-  for (int32_t j = 1; j <= r; ++j) {
-    Mul_ciph(ct, ct, ct);
-    Add_ciph(ct, ct, ct);
-    add_const(ct, -1.0 / pow(2.0 * M_PI, pow(2.0, j - r)));
-    rescale(ct);
+  for (int32_t j = 1; j <= r; ++j) { /* Mul_ciph, Add_ciph(ct, ct), Add_const, Rescale_ciph (bootstrap.c:1508-1515) */
+    const double scalar = -1.0 / pow(2.0 * M_PI, pow(2.0, j - r));
+    Rt_mul_rescale_ciph(ct, ct, ct, true, &scalar);
   }
 }
 

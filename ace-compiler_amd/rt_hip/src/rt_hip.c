@@ -812,7 +812,7 @@ CIPHER Mul_ciph(CIPHER res, CIPHER a, CIPHER b) {
  * share a forward transform there.  The words and the scale are those of the two calls one after the other
  * (evaluator.c:142-190, 288-306, 342-362).  twice: with Add_ciph of the product with itself between the two
  * (chebyshev_impl.c:563-565).  res may be one of the operands. */
-CIPHER Rt_mul_rescale_ciph(CIPHER res, CIPHER a, CIPHER b, bool twice) {
+CIPHER Rt_mul_rescale_ciph(CIPHER res, CIPHER a, CIPHER b, bool twice, const double* then_add) {
   FMT_ASSERT(G.relin._public_keys, "no relinearisation key loaded");
   CIPHER pick  = lower_of(a, b);
   size_t level = Level(pick);
@@ -822,9 +822,18 @@ CIPHER Rt_mul_rescale_ciph(CIPHER res, CIPHER a, CIPHER b, bool twice) {
   CIPHERTEXT t;
   memset(&t, 0, sizeof(t));
   Rt_shape_ciph(&t, pick, a->_scaling_factor * b->_scaling_factor / G.sc, a->_sf_degree + b->_sf_degree - 1);
-  ACE_OK((twice ? ace_mul_relin_double_rescale : ace_mul_relin_rescale)(
-      RT_CTX, t._c0_poly._data, t._c1_poly._data, a->_c0_poly._data, a->_c1_poly._data, b->_c0_poly._data,
-      b->_c1_poly._data, G.relin._public_keys->dev, level));
+  if (then_add) { /* Add_const of the doubled product, at the product's scale (evaluator.c:127-140) */
+    int64_t w[128];
+    FMT_ASSERT(twice && level <= 128, "Rt_mul_rescale_ciph: a constant goes with the doubled product");
+    Rt_encode_val_words(w, *then_add, (uint32_t)level, a->_scaling_factor * b->_scaling_factor);
+    ACE_OK(ace_mul_relin_double_add_rescale(RT_CTX, t._c0_poly._data, t._c1_poly._data, a->_c0_poly._data,
+                                            a->_c1_poly._data, b->_c0_poly._data, b->_c1_poly._data,
+                                            G.relin._public_keys->dev, w, level));
+  } else {
+    ACE_OK((twice ? ace_mul_relin_double_rescale : ace_mul_relin_rescale)(
+        RT_CTX, t._c0_poly._data, t._c1_poly._data, a->_c0_poly._data, a->_c1_poly._data, b->_c0_poly._data,
+        b->_c1_poly._data, G.relin._public_keys->dev, level));
+  }
   Set_poly_level(&t._c0_poly, level - 1);
   Set_poly_level(&t._c1_poly, level - 1);
   Free_poly_data(&res->_c0_poly);

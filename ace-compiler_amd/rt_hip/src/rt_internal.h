@@ -98,8 +98,9 @@ void     Rt_series_divide(double* q, size_t* n_q, double* r, size_t* n_r, const 
 /* Encode_val: `level` residues of trunc(value * scale), large products through the approximation factor */
 void     Rt_encode_val_words(int64_t* res, double value, uint32_t level, double scale);
 void     Rt_copy_words(int64_t* dst, const int64_t* src, size_t n_words);
-/* Mul_ciph (+ Add_ciph of the product with itself) + Rescale_ciph: the same words in fewer launches */
-CIPHER   Rt_mul_rescale_ciph(CIPHER res, CIPHER a, CIPHER b, bool twice);
+/* Mul_ciph (+ Add_ciph of the product with itself (+ Add_const of *then_add, if not NULL)) + Rescale_ciph: the same
+ * words in fewer launches */
+CIPHER   Rt_mul_rescale_ciph(CIPHER res, CIPHER a, CIPHER b, bool twice, const double* then_add);
 void     Rt_plaintexts_settle(void); /* the run of weight plaintexts being encoded on the second stream has landed */
 int64_t* Rt_plain_prepare(PLAIN plain, uint32_t sc_degree, uint32_t level);
 void     Rt_encode_real(PLAIN plain, const void* values, int is_f32, size_t len, uint32_t sc_degree, uint32_t level);

@@ -329,6 +329,7 @@ def reference_cpu_estimate(census_path, chain, seconds_cap=40.0):
         "ace_rescale_ciph": lambda lv, b: 2 * t("rescale", lv),
         "ace_mul_relin_rescale": lambda lv, b: max(b, 1) * (lv * (4 * m_ + a_) + precomp(lv) + switch(lv) + 2 * lv * a_ + 2 * t("rescale", lv)),
         "ace_mul_relin_double_rescale": lambda lv, b: lv * (4 * m_ + a_) + precomp(lv) + switch(lv) + 4 * lv * a_ + 2 * t("rescale", lv),
+        "ace_mul_relin_double_add_rescale": lambda lv, b: lv * (4 * m_ + a_) + precomp(lv) + switch(lv) + 5 * lv * a_ + 2 * t("rescale", lv),
         "ace_mod_down_pair_rescale": lambda lv, b: 2 * t("mod_down", lv) + 2 * t("rescale", lv),
         "ace_rotate_batch": lambda lv, b: precomp(lv) + b * (switch(lv) + lv * (a_ + 2 * r_)),
         "ace_fast_rotate": lambda lv, b: switch(lv) + lv * (a_ + 2 * r_),

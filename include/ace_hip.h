@@ -344,6 +344,14 @@ int ace_mod_down_pair_rescale(ace_ctx* ctx, int64_t* r0, int64_t* r1, const int6
  * (chebyshev_impl.c:563-565, 581-583, 597-599).  The words of the three calls one after the other. */
 int ace_mul_relin_double_rescale(ace_ctx* ctx, int64_t* r0, int64_t* r1, const int64_t* a0, const int64_t* a1,
                                  const int64_t* b0, const int64_t* b1, const int64_t* swk, size_t level);
+/* Mul_ciphertext, Add_ciphertext(prod, prod), Add_const and Rescale_ciphertext (evaluator.c:177-190, 47-76, 127-140
+ * with Add_scalars :113-124, 342-362): a double-angle step of the bootstrap's sine
+ * evaluation (bootstrap.c:1504-1516).  constant: host array of `level` residues, one per limb, of the integer that is
+ * added to every word of c0 (NTT form) between the sum and the Rescale.  r0/r1 level-1 limbs.  The words of
+ * ace_mul_ciph3, ace_relin, two elementwise sums, ace_poly_add_scalars and ace_rescale_ciph. */
+int ace_mul_relin_double_add_rescale(ace_ctx* ctx, int64_t* r0, int64_t* r1, const int64_t* a0, const int64_t* a1,
+                                     const int64_t* b0, const int64_t* b1, const int64_t* swk, const int64_t* constant,
+                                     size_t level);
 /* ace_mul_relin_rescale for `count` independent ciphertext pairs that share the relinearisation key: pair i reads
  * a0 + i*in_stride (likewise a1, b0, b1) and writes r0 + i*out_stride, r1 + i*out_stride (strides in
  * words).  Equivalent to `count` calls of ace_mul_relin_rescale; every kernel launch covers the batch. */

@@ -888,6 +888,22 @@ def test_mul_relin_double_rescale_equals_its_three_calls(pair):
             (g.mul_relin_double_rescale if twice else g.mul_relin_rescale)(s0, s1, a[0], a[1], a[2], a[3], swk, level)
             eq(s0.get()[:n], r0.get()[:n], "level %d twice=%d c0" % (level, twice))
             eq(s1.get()[:n], r1.get()[:n], "level %d twice=%d c1" % (level, twice))
+        # ... and with a constant between the sum and the Rescale (a double-angle step of the sine evaluation):
+        # residues of small and of large integers, of either parity in the dropped limb, and zero
+        q = [int(g.primes[t]) for t in range(level)]
+        for case, big in enumerate((12345678901234567, -3, (1 << 200) + 977, 0, -(1 << 131) - 2)):
+            cst = [big % qt for qt in q]
+            g.mul_ciph3(d[0], d[1], d[2], a[0], a[1], a[2], a[3], level)
+            g.relin(r0, r1, d[0], d[1], d[2], swk, level)
+            g.poly("add", r0, r0, r0, level)
+            g.poly("add", r1, r1, r1, level)
+            g.poly_scalars(False, r0, r0, cst, level)
+            g.rescale_ciph(r0, r1, r0, r1, level)
+            g.mul_relin_double_add_rescale(s0, s1, a[0], a[1], a[2], a[3], swk, cst, level)
+            eq(s0.get()[:n], r0.get()[:n], "level %d constant %d c0" % (level, case))
+            eq(s1.get()[:n], r1.get()[:n], "level %d constant %d c1" % (level, case))
+        with pytest.raises(acefhe.AceError):
+            g.mul_relin_double_add_rescale(s0, s1, a[0], a[1], a[2], a[3], swk, [q[0]] + [0] * (level - 1), level)
         for b in a + d + [r0, r1, s0, s1]:
             b.free()
     swk.free()
