@@ -127,7 +127,7 @@ struct Family {
   // true of Precompute_automorphism_order's NTT-form tables, number_theory.c:211-222).  Tables made by
   // ace_automorphism_order are entered as they are made, a caller's own table is examined on the device when a
   // rotation first uses it; writing to a table through this library (upload, copy, zero, free) forgets the verdict.
-  std::unordered_map<const void*, bool> order_fits;
+  std::map<uintptr_t, bool> order_fits;  // by address: forgetting the tables a write overlaps is a range query
 };
 
 struct ace_ctx {
@@ -220,6 +220,7 @@ struct ace_ctx {
   }
   bool run_accepts(const BatchOp& o, u64 n) const;
   void run_append(const BatchOp& o, u64 n);
+  void drop_untouched_fills(const void* p, size_t words);
   std::map<std::pair<size_t, size_t>, ModUpDev> modup;
   std::map<size_t, RescaleDev> rescale;
   std::map<size_t, PrecompDev> precomp;
@@ -255,21 +256,19 @@ struct ace_ctx {
     std::lock_guard<std::mutex> lock(family->mu);
     auto& fits = family->order_fits;
     if (fits.empty()) return;
-    const uintptr_t lo = (uintptr_t)dst, hi = lo + words * sizeof(u64);
-    for (auto it = fits.begin(); it != fits.end();) {
-      const uintptr_t a = (uintptr_t)it->first, b = a + (size_t)h.N * sizeof(i64);
-      if (a < hi && lo < b) it = fits.erase(it);
-      else ++it;
-    }
+    // a table at address a (N words) overlaps [lo, hi) when a < hi and lo < a + span
+    const uintptr_t lo = (uintptr_t)dst, hi = lo + words * sizeof(u64), span = (uintptr_t)h.N * sizeof(i64);
+    auto it = fits.lower_bound(lo >= span ? lo - span + 1 : 0);
+    while (it != fits.end() && it->first < hi) it = fits.erase(it);
   }
   void note_order(const void* order, bool ok) {
     std::lock_guard<std::mutex> lock(family->mu);
-    family->order_fits[order] = ok;
+    family->order_fits[(uintptr_t)order] = ok;
   }
   bool order_fits_chunks(const i64* order) {
     {
       std::lock_guard<std::mutex> lock(family->mu);
-      auto it = family->order_fits.find(order);
+      auto it = family->order_fits.find((uintptr_t)order);
       if (it != family->order_fits.end()) return it->second;
     }
     bool ok = false;
@@ -800,6 +799,33 @@ void ace_ctx::run_append(const BatchOp& o, u64 n) {
   } else {
     run.written.insert((uintptr_t)o.r);
   }
+}
+
+// Recorded zero fills inside [p, p + words) that no later entry of the run reads or writes are taken out (the
+// buffer is being released: nobody will see them).
+void ace_ctx::drop_untouched_fills(const void* p, size_t words) {
+  if (run.ops.empty()) return;
+  const uintptr_t lo = (uintptr_t)p, hi = lo + words * sizeof(u64);
+  auto in_span = [&](const void* x) { return (uintptr_t)x >= lo && (uintptr_t)x < hi; };
+  std::unordered_set<uintptr_t> later;  // ranges of the buffer that entries behind the current one touch
+  std::vector<uint8_t> gone(run.ops.size(), 0);
+  bool any = false;
+  for (size_t k = run.ops.size(); k-- > 0;) {
+    const BatchOp& o = run.ops[k];
+    if (o.op == BATCH_ZERO && in_span(o.r) && !later.count((uintptr_t)o.r)) {
+      gone[k] = 1;
+      any = true;
+      continue;
+    }
+    if (in_span(o.r)) later.insert((uintptr_t)o.r);
+    if (o.a && in_span(o.a)) later.insert((uintptr_t)o.a);
+    if (o.b && in_span(o.b)) later.insert((uintptr_t)o.b);
+  }
+  if (!any) return;
+  size_t w = 0;
+  for (size_t k = 0; k < run.ops.size(); ++k)
+    if (!gone[k]) run.ops[w++] = run.ops[k];
+  run.ops.resize(w);  // (the sets of touched ranges keep the fills' addresses: they only make the run more careful)
 }
 
 void ace_ctx::flush_run() {
@@ -1691,6 +1717,7 @@ static int64_t* alloc_words(ace_ctx* c, size_t n_words, bool zero) {
       hipError_t e = hipMalloc((void**)&p, words * sizeof(u64));
       if (e != hipSuccess && c->pooled_words) {  // give the cached buffers back and try once more
         (void)hipGetLastError();
+        c->flush_pending();  // recorded calls may name buffers of the pool
         c->drop_pool();
         e = hipMalloc((void**)&p, words * sizeof(u64));
       }
@@ -1725,8 +1752,16 @@ void ace_free(ace_ctx* c, int64_t* p) {
     words = it->second;
   }
   c->forget_orders(p, words);
-  try {  // recorded calls may still name this buffer; a zero fill of it that nothing has looked at is moot
-    c->flush_pending_declared({ace_ctx::span(p, words)}, {});
+  const bool keep = c->family->pooled_words.load() + words <= c->family->pool_limit_words;
+  try {
+    // A pending Mod_down / Rescale may read the buffer: it goes out now.  Recorded calls that name the buffer may
+    // stay recorded where the buffer stays mapped (in this lane's pool): whoever is handed it next is served on the
+    // same stream, and entries that are recorded for it later join the chain of those that name it now (the
+    // ranges are the same: the pool hands a buffer out for the size it was made for).  A zero fill of the buffer
+    // that nothing has looked at is moot.
+    c->flush_poly();
+    if (keep) c->drop_untouched_fills(p, words);
+    else c->flush_run();
   } catch (const std::exception& e) {
     (void)fail(e.what());
   }
@@ -1734,7 +1769,7 @@ void ace_free(ace_ctx* c, int64_t* p) {
     std::lock_guard<std::mutex> lock(c->family->mu);
     c->live.erase(p);
   }
-  if (c->family->pooled_words.load() + words <= c->family->pool_limit_words) {
+  if (keep) {
     c->pool.emplace(words, p);
     c->pooled_words += words;
     c->family->pooled_words += words;
