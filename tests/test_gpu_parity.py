@@ -1359,6 +1359,60 @@ def test_recorded_inner_product_through_a_scratch_limb(pair):
         eq(x, w, what)
 
 
+def test_recorded_products_summed_two_halves_at_a_time(pair):
+    """The shape generated code gives a convolution's sum of plaintext products: per limb, Hw_modmul of both halves
+    of a ciphertext into a temporary ciphertext, then Hw_modadd of both halves into the running sum, term after term,
+    the temporary freed and allocated again between terms (a released buffer that stays in the pool does not end the
+    recorded run: the entries for its next owner follow those that name it now).  Results, and what the temporaries
+    hold at the end, are those of one launch per call -- also where a term's product is read a second time and where
+    the sum goes elsewhere than onto itself."""
+    g = pair.g
+    N, L = g.N, g.L
+    big_ring_skip(N)
+    level = min(L, 3)
+    terms = 7
+    mk = lambda seed: np.concatenate([seeded.uniform_poly(seed + t, [g.primes[t]], N) for t in range(level)])
+    rots = [(mk(7700 + 10 * j), mk(7705 + 10 * j)) for j in range(terms)]
+    plains = [mk(7800 + 10 * j) for j in range(terms)]
+    start0, start1 = mk(7900), mk(7910)
+
+    def program(realloc):
+        limb = lambda buf, t: buf.view(t * N, N)
+        dr = [(g.upload(a), g.upload(b)) for a, b in rots]
+        dp = [g.upload(x) for x in plains]
+        s0, s1, side, other = g.upload(start0), g.upload(start1), g.upload(start0), g.alloc(level * N)
+        t0, t1 = g.alloc(level * N), g.alloc(level * N)
+        for j in range(terms):
+            if realloc and j:
+                t0.free()
+                t1.free()
+                t0, t1 = g.alloc(level * N), g.alloc(level * N)
+            for t in range(level):
+                g.hw("modmul", limb(t0, t), limb(dr[j][0], t), limb(dp[j], t), t)
+                g.hw("modmul", limb(t1, t), limb(dr[j][1], t), limb(dp[j], t), t)
+                g.hw("modadd", limb(s0, t), limb(s0, t), limb(t0, t), t)
+                if j == 2:  # the sum lands elsewhere: not a sum onto itself
+                    g.hw("modadd", limb(other, t), limb(s1, t), limb(t1, t), t)
+                else:
+                    g.hw("modadd", limb(s1, t), limb(t1, t), limb(s1, t), t)
+                if j == 4:  # a second reader of the product
+                    g.hw("modsub", limb(side, t), limb(side, t), limb(t0, t), t)
+        out = [s0.get(), s1.get(), side.get(), other.get(), t0.get(), t1.get()]
+        for b in [s0, s1, side, other, t0, t1] + dp + [x for pr in dr for x in pr]:
+            b.free()
+        return out
+
+    for realloc in (False, True):
+        g.set_batching(False)
+        want = program(realloc)
+        g.set_batching(True)
+        got = program(realloc)
+        names = ("first half", "second half", "second reader", "sum elsewhere", "temporary 0 afterwards",
+                 "temporary 1 afterwards")
+        for w, x, what in zip(want, got, names):
+            eq(x, w, "%s (temporaries allocated per term: %s)" % (what, realloc))
+
+
 def test_recorded_zero_fills_that_nothing_sees(pair):
     """Generated code zero-fills every polynomial it allocates and then overwrites or accumulates into it.  Recorded,
     a fill that is overwritten before it is read is dropped, a product or a sum added to fresh zeros becomes the
