@@ -153,6 +153,9 @@ struct ace_ctx {
   static constexpr int kStages = 256;
   Stage stages[kStages];
   int next_stage = 0;
+  static constexpr int kGatherStages = 8;
+  Stage gather_stages[kGatherStages];
+  int next_gather = 0;
   void h2d(void* dev_dst, const void* src, size_t bytes) {
     if (!bytes) return;
     Stage& st = stages[next_stage];
@@ -170,6 +173,29 @@ struct ace_ctx {
     if (!st.done) HIP_OK(hipEventCreateWithFlags(&st.done, hipEventDisableTiming));
     std::memcpy(st.host, src, bytes);
     HIP_OK(hipMemcpyAsync(dev_dst, st.host, bytes, hipMemcpyHostToDevice, stream));
+    HIP_OK(hipEventRecord(st.done, stream));
+    st.pending = true;
+  }
+  // n host arrays of `bytes` each to consecutive places of the device: one staging block, one copy
+  void h2d_gather(void* dev_dst, const void* const* srcs, size_t n, size_t bytes) {
+    if (!bytes || !n) return;
+    if (n == 1) return h2d(dev_dst, srcs[0], bytes);
+    // (blocks of their own: the ring above keeps many small blocks, and pinned memory is slow to allocate)
+    Stage& st = gather_stages[next_gather];
+    next_gather = (next_gather + 1) % kGatherStages;
+    if (st.pending) {
+      HIP_OK(hipEventSynchronize(st.done));
+      st.pending = false;
+    }
+    if (st.cap < n * bytes) {
+      if (st.host) HIP_OK(hipHostFree(st.host));
+      st.host = nullptr;
+      st.cap = std::max<size_t>(n * bytes, 64 * 1024);
+      HIP_OK(hipHostMalloc(&st.host, st.cap, hipHostMallocDefault));
+    }
+    if (!st.done) HIP_OK(hipEventCreateWithFlags(&st.done, hipEventDisableTiming));
+    for (size_t v = 0; v < n; ++v) std::memcpy(static_cast<char*>(st.host) + v * bytes, srcs[v], bytes);
+    HIP_OK(hipMemcpyAsync(dev_dst, st.host, n * bytes, hipMemcpyHostToDevice, stream));
     HIP_OK(hipEventRecord(st.done, stream));
     st.pending = true;
   }
@@ -736,6 +762,10 @@ struct ace_ctx {
     }
     if (fork_state == 1) swap_lanes();  // destroyed in the middle of a fork: back to the first lane
     if (idle.stream) (void)hipStreamSynchronize(idle.stream);
+    for (Stage& st : gather_stages) {
+      if (st.host) (void)hipHostFree(st.host);
+      if (st.done) (void)hipEventDestroy(st.done);
+    }
     for (void* p : owned) (void)hipFree(p);
     drop_pool();
     for (auto& kv : idle.pool) (void)hipFree(kv.second);
@@ -2581,8 +2611,7 @@ static int encode_impl(ace_ctx* c, int64_t* res, const void* values, int kind, s
         launch_fill_zero(st, reinterpret_cast<u64*>(z + n_values), 2 * (size_t)(slots - n_values));
       c->h2d(z, vecs[0], n_values * value_bytes);
     } else {
-      for (size_t v = 0; v < n_vec; ++v)
-        c->h2d(static_cast<char*>(raw) + v * n_values * value_bytes, vecs[v], n_values * value_bytes);
+      c->h2d_gather(raw, vecs, n_vec, n_values * value_bytes);
       launch_widen_real(st, z, raw, kind == 2, (u32)n_values, slots, (u32)n_vec);
     }
   };
