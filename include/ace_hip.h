@@ -88,9 +88,11 @@ int ace_host_automorphism_order(const ace_ctx* ctx, int64_t* host_order, uint32_
 
 /* ---- device memory -------------------------------------------------------
  * Replaces the malloc+memset of Alloc_poly_data (include/poly/rns_poly.h:109-119):
- * zero-filled HBM, n int64 words.  ace_free keeps the buffer (up to 32 GiB in
- * total) for the next ace_alloc of the same size, so alloc/free pairs inside a
- * program's loops cost a fill kernel, not a hipMalloc. */
+ * zero-filled HBM, n int64 words.  ace_free keeps the buffer (up to a third of
+ * the device's memory in total, or ACE_POOL_LIMIT_GB) for the next ace_alloc of
+ * the same size on the same context, so alloc/free pairs inside a program's
+ * loops cost a fill (recorded with the Hw_* calls around it, and dropped where
+ * nothing reads the zeros), not a hipMalloc. */
 int64_t* ace_alloc(ace_ctx* ctx, size_t n_words);
 /* the same without the zero fill, for buffers that are written before they are read */
 int64_t* ace_alloc_uninit(ace_ctx* ctx, size_t n_words);
